@@ -1,0 +1,995 @@
+#include "HipLowering.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <sstream>
+
+namespace akg {
+
+const char *kernelFamilyName(KernelFamily f) {
+  switch (f) {
+    case KernelFamily::Elementwise: return "elementwise";
+    case KernelFamily::RowReduce: return "row_reduce";
+    case KernelFamily::GemmEpilogue: return "gemm_epilogue";
+  }
+  return "?";
+}
+
+LoweringOptions LoweringOptions::fromEnvironment() {
+  LoweringOptions o;
+  auto readInt = [](const char *name) {
+    const char *v = std::getenv(name);
+    return (v && *v) ? std::atoi(v) : 0;
+  };
+  o.vec = readInt("AKG_HIP_VEC");
+  o.threadsPerRow = readInt("AKG_HIP_TPR");
+  o.chunks = readInt("AKG_HIP_CHUNKS");
+  o.block = readInt("AKG_HIP_BLOCK");
+  o.gemmVariant = readInt("AKG_HIP_GEMM_VARIANT");
+  return o;
+}
+
+namespace lowering {
+
+const char *dtypeTag(DType t) {
+  switch (t) {
+    case DType::Bool: return "akg::b1";
+    case DType::I8: return "akg::i8";
+    case DType::I16: return "akg::i16";
+    case DType::I32: return "akg::i32";
+    case DType::I64: return "akg::i64";
+    case DType::F16: return "akg::f16";
+    case DType::BF16: return "akg::bf16";
+    case DType::F32: return "akg::f32";
+    case DType::F64: return "akg::f64";
+  }
+  return "?";
+}
+
+const char *computeTypeName(DType t) {
+  switch (t) {
+    case DType::Bool: return "bool";
+    case DType::I8:
+    case DType::I16:
+    case DType::I32: return "int";
+    case DType::I64: return "long long";
+    case DType::F16:
+    case DType::BF16:
+    case DType::F32: return "float";
+    case DType::F64: return "double";
+  }
+  return "?";
+}
+
+static float roundToBf16(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, sizeof(u));
+  if ((u & 0x7fffffffu) > 0x7f800000u) return f;
+  u += 0x7fffu + ((u >> 16) & 1u);
+  u &= 0xffff0000u;
+  std::memcpy(&f, &u, sizeof(u));
+  return f;
+}
+
+static float roundToF16(float f) {
+  if (std::isnan(f) || std::isinf(f) || f == 0.0f) return f;
+  double a = std::fabs(static_cast<double>(f));
+  if (a >= 65520.0) return std::copysign(INFINITY, f);
+  int e = 0;
+  (void)std::frexp(a, &e);  // a = m * 2^e with m in [0.5, 1): leading bit has weight 2^(e-1)
+  int lead = e - 1;
+  double quantum = (lead < -14) ? std::ldexp(1.0, -24) : std::ldexp(1.0, lead - 10);
+  double r = std::nearbyint(a / quantum) * quantum;  // default rounding mode: to nearest even
+  return static_cast<float>(std::copysign(r, static_cast<double>(f)));
+}
+
+std::string literalFor(DType t, double value) {
+  char buf[96];
+  switch (t) {
+    case DType::Bool: return value != 0.0 ? "true" : "false";
+    case DType::I8:
+    case DType::I16:
+    case DType::I32: {
+      long long v = static_cast<long long>(value);
+      if (t == DType::I8) v = static_cast<signed char>(v);
+      if (t == DType::I16) v = static_cast<short>(v);
+      if (t == DType::I32) v = static_cast<int>(v);
+      if (v == -2147483648LL) return "(-2147483647 - 1)";
+      std::snprintf(buf, sizeof(buf), "(%lld)", v);
+      return buf;
+    }
+    case DType::I64: {
+      long long v = static_cast<long long>(value);
+      if (v == (-9223372036854775807LL - 1)) return "(-9223372036854775807LL - 1)";
+      std::snprintf(buf, sizeof(buf), "(%lldLL)", v);
+      return buf;
+    }
+    case DType::F64: {
+      if (std::isnan(value)) return "__builtin_nan(\"\")";
+      if (std::isinf(value)) return value > 0 ? "__builtin_inf()" : "(-__builtin_inf())";
+      std::snprintf(buf, sizeof(buf), "(%a)", value);
+      return buf;
+    }
+    case DType::F16:
+    case DType::BF16:
+    case DType::F32: {
+      float f = static_cast<float>(value);
+      if (t == DType::F16) f = roundToF16(f);
+      if (t == DType::BF16) f = roundToBf16(f);
+      if (std::isnan(f)) return "__builtin_nanf(\"\")";
+      if (std::isinf(f)) return f > 0 ? "__builtin_inff()" : "(-__builtin_inff())";
+      std::snprintf(buf, sizeof(buf), "(%af)", static_cast<double>(f));
+      return buf;
+    }
+  }
+  return "0";
+}
+
+uint64_t countAlgorithmicBytes(const OpGraph &g) {
+  uint64_t bytes = 0;
+  for (int id : g.inputs) bytes += static_cast<uint64_t>(g.tensor(id).numel()) * dtypeSize(g.tensor(id).dtype);
+  for (int id : g.outputs) bytes += static_cast<uint64_t>(g.tensor(id).numel()) * dtypeSize(g.tensor(id).dtype);
+  return bytes;
+}
+
+std::vector<std::vector<int64_t>> buildShapeArgs(const OpGraph &g) {
+  // One record per kernel argument: [offset, sizes..., strides...] (RecordStaticShapeArgs,
+  // KernelOutliningExt.cpp:384-423). All tensors are dense row-major with offset 0.
+  std::vector<std::vector<int64_t>> out;
+  auto add = [&](const TensorValue &t) {
+    std::vector<int64_t> rec;
+    rec.push_back(0);
+    for (int64_t d : t.shape) rec.push_back(d);
+    std::vector<int64_t> strides(t.shape.size(), 1);
+    for (int i = static_cast<int>(t.shape.size()) - 2; i >= 0; --i) {
+      strides[static_cast<size_t>(i)] = strides[static_cast<size_t>(i) + 1] * t.shape[static_cast<size_t>(i) + 1];
+    }
+    for (int64_t s : strides) rec.push_back(s);
+    out.push_back(rec);
+  };
+  for (int id : g.inputs) add(g.tensor(id));
+  for (int id : g.outputs) add(g.tensor(id));
+  return out;
+}
+
+bool isReduceKind(OpKind k) {
+  return k == OpKind::ReduceSum || k == OpKind::ReduceMax || k == OpKind::ReduceMin || k == OpKind::ReduceProd ||
+         k == OpKind::ReduceAll || k == OpKind::ReduceAny;
+}
+
+bool isElementwiseKind(OpKind k) {
+  switch (k) {
+    case OpKind::MatMul:
+    case OpKind::Unknown:
+    case OpKind::Unsupported:
+      return false;
+    default:
+      return !isReduceKind(k);
+  }
+}
+
+std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vector<std::string> &in) {
+  const DType od = g.tensor(op.outputs[0]).dtype;
+  const std::string tag = dtypeTag(od);
+  const std::string ct = computeTypeName(od);
+  auto inType = [&](size_t i) { return g.tensor(op.inputs[i]).dtype; };
+  auto need = [&](size_t n) {
+    if (in.size() != n) {
+      throw LoweringError("op " + op.name + ": expected " + std::to_string(n) + " operands, found " +
+                          std::to_string(in.size()));
+    }
+  };
+  auto conv = [&](size_t i) {
+    if (ct == computeTypeName(inType(i))) return in[i];
+    return "static_cast<" + ct + ">(" + in[i] + ")";
+  };
+  auto asBool = [&](size_t i) {
+    if (inType(i) == DType::Bool) return in[i];
+    return "(" + in[i] + " != 0)";
+  };
+  auto rnd = [&](const std::string &e) {
+    if (od == DType::F16 || od == DType::BF16 || od == DType::I8 || od == DType::I16) return tag + "::rnd(" + e + ")";
+    return e;
+  };
+  auto arith = [&]() {
+    if (od == DType::Bool) throw LoweringError("op " + op.name + ": arithmetic on bool tensors is not supported");
+  };
+  auto floatOnly = [&]() {
+    if (!isFloatType(od)) throw LoweringError("op " + op.name + ": only floating-point tensors are supported");
+  };
+  auto unaryMath = [&](const char *fn) {
+    need(1);
+    floatOnly();
+    return rnd(std::string("akg::") + fn + "(" + conv(0) + ")");
+  };
+  auto binary = [&](const char *fn) {
+    need(2);
+    arith();
+    return rnd(std::string("akg::") + fn + "(" + conv(0) + ", " + conv(1) + ")");
+  };
+  auto compare = [&](const char *sym) {
+    need(2);
+    std::string a = in[0], b = in[1];
+    if (std::string(computeTypeName(inType(0))) != computeTypeName(inType(1))) {
+      a = "static_cast<double>(" + a + ")";
+      b = "static_cast<double>(" + b + ")";
+    }
+    std::string e = "(" + a + " " + sym + " " + b + ")";
+    if (od == DType::Bool) return e;
+    return "static_cast<" + ct + ">(" + e + ")";
+  };
+  auto predicate = [&](const char *fn) {
+    need(1);
+    if (!isFloatType(inType(0))) throw LoweringError("op " + op.name + ": operand must be floating point");
+    std::string e = std::string("akg::") + fn + "(" + in[0] + ")";
+    if (od == DType::Bool) return e;
+    return "static_cast<" + ct + ">(" + e + ")";
+  };
+
+  switch (op.kind) {
+    case OpKind::Add: return binary("op_add");
+    case OpKind::Sub: return binary("op_sub");
+    case OpKind::Mul: return binary("op_mul");
+    case OpKind::Div: return binary("op_div");
+    case OpKind::Maximum: return binary("op_maximum");
+    case OpKind::Minimum: return binary("op_minimum");
+    case OpKind::Pow: floatOnly(); return binary("op_pow");
+    case OpKind::Atan2: floatOnly(); return binary("op_atan2");
+    case OpKind::Neg: need(1); arith(); return rnd("akg::op_neg(" + conv(0) + ")");
+    case OpKind::Abs: need(1); arith(); return rnd("akg::op_abs(" + conv(0) + ")");
+    case OpKind::Square: need(1); arith(); return rnd("akg::op_mul(" + conv(0) + ", " + conv(0) + ")");
+    case OpKind::Exp: return unaryMath("op_exp");
+    case OpKind::Log: return unaryMath("op_log");
+    case OpKind::Tanh: return unaryMath("op_tanh");
+    case OpKind::Rsqrt: return unaryMath("op_rsqrt");
+    case OpKind::Sqrt: return unaryMath("op_sqrt");
+    case OpKind::Reciprocal: return unaryMath("op_inv");
+    case OpKind::Floor: return unaryMath("op_floor");
+    case OpKind::Sin: return unaryMath("op_sin");
+    case OpKind::Cos: return unaryMath("op_cos");
+    case OpKind::Asin: return unaryMath("op_asin");
+    case OpKind::Acos: return unaryMath("op_acos");
+    case OpKind::Atan: return unaryMath("op_atan");
+    case OpKind::Asinh: return unaryMath("op_asinh");
+    case OpKind::Acosh: return unaryMath("op_acosh");
+    case OpKind::IsNan: return predicate("op_isnan");
+    case OpKind::IsInf: return predicate("op_isinf");
+    case OpKind::IsFinite: return predicate("op_isfinite");
+    case OpKind::Equal: return compare("==");
+    case OpKind::NotEqual: return compare("!=");
+    case OpKind::Greater: return compare(">");
+    case OpKind::GreaterEqual: return compare(">=");
+    case OpKind::Less: return compare("<");
+    case OpKind::LessEqual: return compare("<=");
+    case OpKind::LogicalNot: {
+      need(1);
+      std::string e = "(!" + asBool(0) + ")";
+      return od == DType::Bool ? e : "static_cast<" + ct + ">(" + e + ")";
+    }
+    case OpKind::LogicalAnd: {
+      need(2);
+      std::string e = "(" + asBool(0) + " && " + asBool(1) + ")";
+      return od == DType::Bool ? e : "static_cast<" + ct + ">(" + e + ")";
+    }
+    case OpKind::LogicalOr: {
+      need(2);
+      std::string e = "(" + asBool(0) + " || " + asBool(1) + ")";
+      return od == DType::Bool ? e : "static_cast<" + ct + ">(" + e + ")";
+    }
+    case OpKind::Select: {
+      need(3);
+      return "(" + asBool(0) + " ? " + conv(1) + " : " + conv(2) + ")";
+    }
+    case OpKind::Cast: {
+      need(1);
+      return std::string("akg::cast<") + tag + ", " + dtypeTag(inType(0)) + ">(" + in[0] + ")";
+    }
+    case OpKind::AddN: {
+      if (in.empty()) throw LoweringError("op AddN: no operands");
+      arith();
+      std::string e = conv(0);
+      for (size_t i = 1; i < in.size(); ++i) e = rnd("akg::op_add(" + e + ", " + conv(i) + ")");
+      return e;
+    }
+    case OpKind::Reshape:
+    case OpKind::BroadcastTo:
+      need(1);
+      return conv(0);
+    default:
+      break;
+  }
+  throw LoweringError("op " + op.name + " has no elementwise lowering");
+}
+
+}  // namespace lowering
+
+namespace {
+
+using lowering::computeTypeName;
+using lowering::dtypeTag;
+
+int64_t product(const std::vector<int64_t> &v, size_t from = 0, size_t to = static_cast<size_t>(-1)) {
+  int64_t p = 1;
+  if (to > v.size()) to = v.size();
+  for (size_t i = from; i < to; ++i) p *= v[i];
+  return p;
+}
+
+int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+int pow2AtLeast(int64_t x) {
+  int p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+// Right-aligns `shape` to `rank` dims (numpy broadcasting), dropping surplus leading 1s.
+std::vector<int64_t> padShape(const std::vector<int64_t> &shape, size_t rank, const std::string &what) {
+  std::vector<int64_t> s = shape;
+  while (s.size() > rank && s.front() == 1) s.erase(s.begin());
+  if (s.size() > rank) throw LoweringError(what + ": rank exceeds the kernel's iteration space");
+  std::vector<int64_t> out(rank - s.size(), 1);
+  out.insert(out.end(), s.begin(), s.end());
+  return out;
+}
+
+enum class ValRank { Const, Uniform, Tile };
+
+struct ValInfo {
+  bool defined = false;
+  ValRank rank = ValRank::Const;
+  std::string ident;         // variable name (Tile: array, Uniform: scalar); Const: literal text
+  bool rowvecNoKeep = false; // Uniform value whose tensor shape lacks the trailing 1 (reduce without keep_dims)
+};
+
+// How a kernel input is addressed relative to the iteration space [rows, cols].
+struct InputAccess {
+  bool lastDimFull = false;          // true: V consecutive elements per chunk; false: one element per row
+  std::vector<int64_t> foldedShape;  // shape aligned to the (possibly folded) iteration space
+};
+
+class TileEmitter {
+ public:
+  TileEmitter(const OpGraph &g, const LoweringOptions &o) : g_(g), opt_(o) {}
+
+  LoweredKernel run() {
+    analyse();
+    pickSchedule();
+    emit();
+    LoweredKernel k;
+    k.kernelName = g_.name + "_kernel";
+    k.source = src_.str();
+    k.family = rowMode_ ? KernelFamily::RowReduce : KernelFamily::Elementwise;
+    k.grid[0] = static_cast<unsigned>(grid_);
+    k.block[0] = static_cast<unsigned>(block_);
+    k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
+    k.shapeArgs = lowering::buildShapeArgs(g_);
+    std::ostringstream note;
+    note << kernelFamilyName(k.family) << " rows=" << rows_ << " cols=" << cols_ << " vec=" << vec_
+         << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
+         << " block=" << block_ << " grid=" << grid_;
+    k.scheduleNote = note.str();
+    return k;
+  }
+
+ private:
+  const OpGraph &g_;
+  LoweringOptions opt_;
+  std::ostringstream src_;
+
+  bool rowMode_ = false;
+  std::vector<int64_t> full_;     // iteration space (folded in elementwise mode)
+  int64_t rows_ = 1, cols_ = 1, numel_ = 1;
+  std::vector<InputAccess> access_;  // per graph input
+  std::vector<ValInfo> vals_;        // per tensor
+
+  int vec_ = 1, tpr_ = 1, chunks_ = 1, rowsPerBlock_ = 1, block_ = 256;
+  int64_t grid_ = 1;
+  bool raggedCols_ = false, raggedRows_ = false, raggedFlat_ = false;
+  int reduceCount_ = 0;
+
+  // ------------------------------------------------------------------ analysis
+  void analyse() {
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::Unknown) {
+        throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
+      }
+      if (op.kind == OpKind::Unsupported) {
+        throw LoweringError("op " + op.name + " has no gfx950 kernel family yet");
+      }
+      if (op.kind == OpKind::MatMul) throw LoweringError("internal: MatMul reached the tile emitter");
+      if (lowering::isReduceKind(op.kind)) rowMode_ = true;
+    }
+    if (rowMode_) {
+      analyseRowSpace();
+    } else {
+      analyseElementwiseSpace();
+    }
+  }
+
+  void analyseRowSpace() {
+    const OpNode *first = nullptr;
+    for (const OpNode &op : g_.ops) {
+      if (lowering::isReduceKind(op.kind)) {
+        first = &op;
+        break;
+      }
+    }
+    std::vector<int64_t> space = g_.tensor(first->inputs[0]).shape;
+    while (space.size() > 1 && space.front() == 1) space.erase(space.begin());
+    if (space.empty() || space.back() <= 1) {
+      throw LoweringError("reduction over an innermost axis of extent 1 is not supported");
+    }
+    const size_t r = space.size();
+    for (const OpNode &op : g_.ops) {
+      if (!lowering::isReduceKind(op.kind)) continue;
+      const TensorValue &in = g_.tensor(op.inputs[0]);
+      std::vector<int64_t> s = padShape(in.shape, r, "reduce operand " + in.name);
+      if (s != space) {
+        throw LoweringError("all reductions of one kernel must run over the same tensor shape");
+      }
+      // Real (extent > 1) reduced axes must be exactly the innermost axis: direction X.
+      std::vector<int64_t> real;
+      int64_t lead = static_cast<int64_t>(in.shape.size()) - static_cast<int64_t>(r);
+      for (int64_t a : op.axes) {
+        if (in.shape[static_cast<size_t>(a)] > 1) real.push_back(a - lead);
+      }
+      if (real.size() != 1 || real[0] != static_cast<int64_t>(r) - 1) {
+        throw LoweringError("op " + op.name +
+                            ": only reductions over the innermost axis (direction X) have a kernel family yet");
+      }
+    }
+    full_ = space;
+    cols_ = space.back();
+    rows_ = product(space, 0, r - 1);
+    numel_ = rows_ * cols_;
+    access_.resize(g_.inputs.size());
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      const TensorValue &t = g_.tensor(g_.inputs[i]);
+      std::vector<int64_t> s = padShape(t.shape, r, "input " + t.name);
+      for (size_t d = 0; d < r; ++d) {
+        if (s[d] != 1 && s[d] != space[d]) {
+          throw LoweringError("input " + t.name + " is not broadcast-compatible with the reduced tensor");
+        }
+      }
+      access_[i].foldedShape = s;
+      access_[i].lastDimFull = (s[r - 1] == cols_);
+    }
+  }
+
+  void analyseElementwiseSpace() {
+    std::vector<int64_t> space = g_.tensor(g_.outputs[0]).shape;
+    for (int id : g_.outputs) {
+      if (g_.tensor(id).shape != space) {
+        throw LoweringError("all outputs of an elementwise kernel must have the same shape");
+      }
+    }
+    const size_t r = space.size();
+    std::vector<std::vector<int64_t>> padded;
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      const TensorValue &t = g_.tensor(g_.inputs[i]);
+      std::vector<int64_t> s = padShape(t.shape, r, "input " + t.name);
+      for (size_t d = 0; d < r; ++d) {
+        if (s[d] != 1 && s[d] != space[d]) {
+          throw LoweringError("input " + t.name + " is not broadcast-compatible with the output shape");
+        }
+      }
+      padded.push_back(s);
+    }
+    // Dimension folding (the role FoldDimension plays in the reference): drop unit dims, then merge adjacent
+    // dims that every input either spans fully or broadcasts together.
+    std::vector<size_t> keep;
+    for (size_t d = 0; d < r; ++d) {
+      if (space[d] != 1) keep.push_back(d);
+    }
+    std::vector<int64_t> folded;
+    std::vector<std::vector<int64_t>> foldedIn(padded.size());
+    auto status = [&](size_t input, size_t d) { return padded[input][d] == space[d]; };
+    for (size_t k = 0; k < keep.size(); ++k) {
+      size_t d = keep[k];
+      bool merge = !folded.empty();
+      if (merge) {
+        size_t prev = keep[k - 1];
+        for (size_t i = 0; i < padded.size(); ++i) {
+          if (status(i, d) != status(i, prev)) {
+            merge = false;
+            break;
+          }
+        }
+      }
+      if (merge) {
+        folded.back() *= space[d];
+        for (size_t i = 0; i < padded.size(); ++i) foldedIn[i].back() *= padded[i][d];
+      } else {
+        folded.push_back(space[d]);
+        for (size_t i = 0; i < padded.size(); ++i) foldedIn[i].push_back(padded[i][d]);
+      }
+    }
+    if (folded.empty()) {
+      folded.push_back(1);
+      for (auto &f : foldedIn) f.push_back(1);
+    }
+    full_ = folded;
+    cols_ = folded.back();
+    rows_ = product(folded, 0, folded.size() - 1);
+    numel_ = rows_ * cols_;
+    access_.resize(g_.inputs.size());
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      access_[i].foldedShape = foldedIn[i];
+      access_[i].lastDimFull = (foldedIn[i].back() == cols_);
+    }
+  }
+
+  // ------------------------------------------------------------------ schedule
+  void pickSchedule() {
+    // Chunk width: 16 bytes of the narrowest element type that is moved chunk-wise, so the widest access of
+    // every tensor is at least one 128-bit instruction.
+    size_t minSize = 8;
+    bool any = false;
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      if (!access_[i].lastDimFull) continue;
+      minSize = std::min(minSize, dtypeSize(g_.tensor(g_.inputs[i]).dtype));
+      any = true;
+    }
+    for (int id : g_.outputs) {
+      if (rowMode_ && g_.tensor(id).numel() != numel_) continue;
+      minSize = std::min(minSize, dtypeSize(g_.tensor(id).dtype));
+      any = true;
+    }
+    if (!any) minSize = 4;
+    int v = opt_.vec > 0 ? opt_.vec : static_cast<int>(16 / minSize);
+    v = std::max(1, std::min(v, 16));
+    while (v > 1 && (cols_ % v) != 0) v >>= 1;
+    if ((v & (v - 1)) != 0) v = 1;
+    vec_ = v;
+
+    if (rowMode_) {
+      // One row per group of tpr threads, about 32 elements per thread so that a 4096..8192-wide row of a
+      // 2-byte type has 4 x 128-bit loads in flight per thread and the row stays in registers.
+      int targetPerThread = std::max(vec_, 32);
+      int tpr = opt_.threadsPerRow > 0 ? opt_.threadsPerRow : pow2AtLeast(ceilDiv(cols_, targetPerThread));
+      tpr = std::max(1, std::min(tpr, 1024));
+      if ((tpr & (tpr - 1)) != 0) tpr = pow2AtLeast(tpr);
+      // never more threads than chunks in a row
+      while (tpr > 1 && static_cast<int64_t>(tpr) * vec_ > cols_ * 2) tpr >>= 1;
+      tpr_ = tpr;
+      chunks_ = static_cast<int>(ceilDiv(cols_, static_cast<int64_t>(tpr_) * vec_));
+      if (static_cast<int64_t>(chunks_) * vec_ > 256) {
+        throw LoweringError("row of " + std::to_string(cols_) +
+                            " elements does not fit the register-resident row kernel (max 262144 per row)");
+      }
+      block_ = opt_.block > 0 ? opt_.block : 256;
+      block_ = std::max(block_, tpr_);
+      block_ = std::min(block_, 1024);
+      if (block_ % tpr_ != 0 || block_ % 64 != 0) block_ = std::max(tpr_, 64);
+      rowsPerBlock_ = block_ / tpr_;
+      grid_ = ceilDiv(rows_, rowsPerBlock_);
+      raggedCols_ = (static_cast<int64_t>(chunks_) * tpr_ * vec_ != cols_);
+      raggedRows_ = (rows_ % rowsPerBlock_) != 0;
+    } else {
+      block_ = opt_.block > 0 ? opt_.block : 256;
+      if (block_ % 64 != 0 || block_ > 1024) block_ = 256;
+      int chunks = opt_.chunks > 0 ? opt_.chunks : std::max(1, 16 / vec_);
+      // Small problems: fewer chunks per thread so the grid still covers the chip.
+      while (chunks > 1 && ceilDiv(numel_, static_cast<int64_t>(block_) * vec_ * chunks) < 1024) chunks >>= 1;
+      chunks_ = std::max(1, chunks);
+      tpr_ = block_;
+      rowsPerBlock_ = 1;
+      int64_t perBlock = static_cast<int64_t>(block_) * vec_ * chunks_;
+      grid_ = std::max<int64_t>(1, ceilDiv(numel_, perBlock));
+      raggedFlat_ = (numel_ % perBlock) != 0;
+    }
+    if (grid_ > 2147483647LL) throw LoweringError("grid too large");
+  }
+
+  // ------------------------------------------------------------------ emission helpers
+  std::string ctOf(int tensorId) const { return computeTypeName(g_.tensor(tensorId).dtype); }
+  std::string tagOf(int tensorId) const { return dtypeTag(g_.tensor(tensorId).dtype); }
+
+  std::string operandExpr(int tensorId) const {
+    const ValInfo &v = vals_[static_cast<size_t>(tensorId)];
+    if (!v.defined) throw LoweringError("internal: operand " + g_.tensor(tensorId).name + " used before definition");
+    if (v.rank == ValRank::Tile) return v.ident + "[j][e]";
+    return v.ident;
+  }
+
+  void line(const std::string &s) { src_ << s << "\n"; }
+
+  // Offset of the first element of `row` for an input, as an expression in `rowVar`.
+  std::string rowOffsetExpr(const InputAccess &a, const std::string &rowVar) const {
+    const std::vector<int64_t> &s = a.foldedShape;
+    const size_t r = full_.size();
+    bool allFull = true, allOne = true;
+    for (size_t d = 0; d + 1 < r; ++d) {
+      if (s[d] != full_[d]) allFull = false;
+      if (s[d] != 1) allOne = false;
+    }
+    if (r == 1 || allOne) return "0L";
+    if (allFull) return "(" + rowVar + " * " + std::to_string(s[r - 1]) + "L)";
+    // general leading-dim broadcast: decompose the row index over the leading dims
+    std::vector<int64_t> stride(r, 0);
+    int64_t acc = s[r - 1];
+    for (int d = static_cast<int>(r) - 2; d >= 0; --d) {
+      stride[static_cast<size_t>(d)] = (s[static_cast<size_t>(d)] == 1) ? 0 : acc;
+      acc *= s[static_cast<size_t>(d)];
+    }
+    // emitted as a sum of ((row / inner_extent) % extent) * stride terms
+    std::ostringstream e;
+    int64_t div = 1;
+    bool firstTerm = true;
+    for (int d = static_cast<int>(r) - 2; d >= 0; --d) {
+      int64_t extent = full_[static_cast<size_t>(d)];
+      if (stride[static_cast<size_t>(d)] != 0) {
+        if (!firstTerm) e << " + ";
+        e << "((" << rowVar << " / " << div << "L) % " << extent << "L) * " << stride[static_cast<size_t>(d)] << "L";
+        firstTerm = false;
+      }
+      div *= extent;
+    }
+    if (firstTerm) return "0L";
+    return "(" + e.str() + ")";
+  }
+
+  // ------------------------------------------------------------------ emission
+  void emit() {
+    vals_.assign(g_.tensors.size(), ValInfo());
+    const std::string kname = g_.name + "_kernel";
+
+    line("// Generated by the akg HIP lowering for gfx950. Op description: " + g_.name);
+    line("// family: " + std::string(rowMode_ ? "row_reduce" : "elementwise") + ", fusion class: " +
+         operatorTemplateName(g_.operatorTemplate));
+    line("#include \"akg_rt.hpp\"");
+    line("");
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << block_ << ") void " << kname << "(";
+    size_t argc = 0;
+    for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
+    }
+    line(") {");
+    src_ << "  constexpr int V = " << vec_ << ";\n";
+    src_ << "  constexpr int NCHUNK = " << chunks_ << ";\n";
+    src_ << "  constexpr int BLOCK = " << block_ << ";\n";
+    src_ << "  constexpr long COLS = " << cols_ << "L;\n";
+    src_ << "  constexpr long ROWS = " << rows_ << "L;\n";
+    line("  const int tid = static_cast<int>(threadIdx.x);");
+    if (rowMode_) {
+      src_ << "  constexpr int TPR = " << tpr_ << ";\n";
+      src_ << "  constexpr int RPB = " << rowsPerBlock_ << ";\n";
+      line("  const int tcol = tid % TPR;");
+      line("  const long akg_row_raw = static_cast<long>(blockIdx.x) * RPB + (tid / TPR);");
+      if (raggedRows_) {
+        line("  const bool akg_row_ok = akg_row_raw < ROWS;");
+        line("  const long akg_row = akg_row_ok ? akg_row_raw : (ROWS - 1);");
+      } else {
+        line("  const long akg_row = akg_row_raw;");
+      }
+      if (tpr_ > 64) {
+        line("  __shared__ double akg_scratch[2][BLOCK / 64];");
+      }
+      line("  long akg_rows[NCHUNK];");
+      line("  long akg_cols[NCHUNK];");
+      line("  bool akg_ok[NCHUNK];");
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      line("    akg_rows[j] = akg_row;");
+      line("    akg_cols[j] = (static_cast<long>(j) * TPR + tcol) * V;");
+      line(std::string("    akg_ok[j] = ") + (raggedCols_ ? "akg_cols[j] < COLS;" : "true;"));
+      line("  }");
+    } else {
+      line("  constexpr long NUMEL = ROWS * COLS;");
+      line("  const long akg_base = static_cast<long>(blockIdx.x) * (static_cast<long>(BLOCK) * V * NCHUNK);");
+      line("  long akg_rows[NCHUNK];");
+      line("  long akg_cols[NCHUNK];");
+      line("  long akg_flat[NCHUNK];");
+      line("  bool akg_ok[NCHUNK];");
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      line("    const long i = akg_base + (static_cast<long>(j) * BLOCK + tid) * V;");
+      line(std::string("    akg_ok[j] = ") + (raggedFlat_ ? "i < NUMEL;" : "true;"));
+      line("    const long ic = akg_ok[j] ? i : 0L;");
+      line("    akg_flat[j] = ic;");
+      if (rows_ == 1) {
+        line("    akg_rows[j] = 0L;");
+        line("    akg_cols[j] = ic;");
+      } else {
+        line("    akg_rows[j] = ic / COLS;");
+        line("    akg_cols[j] = ic % COLS;");
+      }
+      line("  }");
+    }
+    line("");
+
+    // loads of kernel inputs
+    for (size_t i = 0; i < g_.inputs.size(); ++i) emitInputLoad(i);
+    // constants
+    for (size_t t = 0; t < g_.tensors.size(); ++t) {
+      const TensorValue &tv = g_.tensors[t];
+      if (!tv.isConst) continue;
+      ValInfo &v = vals_[t];
+      v.defined = true;
+      v.rank = ValRank::Const;
+      v.ident = lowering::literalFor(tv.dtype, tv.constValue);
+    }
+    // ops in description order
+    for (const OpNode &op : g_.ops) {
+      if (lowering::isReduceKind(op.kind)) {
+        emitReduce(op);
+      } else {
+        emitElementwise(op);
+      }
+    }
+    // stores
+    for (size_t i = 0; i < g_.outputs.size(); ++i) emitOutputStore(i);
+    line("}");
+  }
+
+  void emitInputLoad(size_t i) {
+    const int id = g_.inputs[i];
+    const TensorValue &t = g_.tensor(id);
+    const InputAccess &a = access_[i];
+    ValInfo &v = vals_[static_cast<size_t>(id)];
+    v.defined = true;
+    const std::string tag = tagOf(id);
+    const std::string ct = ctOf(id);
+    std::ostringstream nm;
+    if (a.lastDimFull) {
+      v.rank = ValRank::Tile;
+      nm << "t_in" << i;
+      v.ident = nm.str();
+      src_ << "  " << ct << " " << v.ident << "[NCHUNK][V];\n";
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      src_ << "    if (akg_ok[j]) {\n";
+      src_ << "      akg::load_chunk<" << tag << ", V>(in" << i << " + " << rowOffsetExpr(a, "akg_rows[j]")
+           << " + akg_cols[j], " << v.ident << "[j]);\n";
+      src_ << "    } else {\n";
+      src_ << "      akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(" << tag
+           << "::storage()));\n";
+      src_ << "    }\n";
+      line("  }");
+    } else if (rowMode_) {
+      // one element per row (or a single element for the whole kernel)
+      v.rank = ValRank::Uniform;
+      nm << "u_in" << i;
+      v.ident = nm.str();
+      src_ << "  const " << ct << " " << v.ident << " = " << tag << "::load(in" << i << "["
+           << rowOffsetExpr(a, "akg_row") << "]);\n";
+      (void)t;
+    } else {
+      // elementwise mode: replicate the per-row element over the chunk
+      v.rank = ValRank::Tile;
+      nm << "t_in" << i;
+      v.ident = nm.str();
+      src_ << "  " << ct << " " << v.ident << "[NCHUNK][V];\n";
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      src_ << "    akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(in" << i << "["
+           << rowOffsetExpr(a, "akg_rows[j]") << "]));\n";
+      line("  }");
+    }
+  }
+
+  void emitElementwise(const OpNode &op) {
+    if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+    const int outId = op.outputs[0];
+    const TensorValue &outT = g_.tensor(outId);
+    ValRank rank = ValRank::Const;
+    bool anyNoKeep = false, anyTile = false;
+    for (int in : op.inputs) {
+      const ValInfo &vi = vals_[static_cast<size_t>(in)];
+      if (!vi.defined) throw LoweringError("op " + op.name + ": operand " + g_.tensor(in).name + " is undefined");
+      if (vi.rank == ValRank::Tile) {
+        rank = ValRank::Tile;
+        anyTile = true;
+      } else if (vi.rank == ValRank::Uniform && rank != ValRank::Tile) {
+        rank = ValRank::Uniform;
+      }
+      if (vi.rowvecNoKeep) anyNoKeep = true;
+    }
+    if (rank == ValRank::Const) rank = ValRank::Uniform;
+    if (anyTile && anyNoKeep) {
+      throw LoweringError("op " + op.name + ": a reduce result without keep_dims cannot be broadcast against the "
+                          "reduced tensor; reshape it to [...,1] first");
+    }
+    // shape sanity: a Tile result must span the innermost dim, a Uniform result must not
+    if (rowMode_) {
+      int64_t last = outT.shape.empty() ? 1 : outT.shape.back();
+      if (rank == ValRank::Tile && last != cols_) {
+        throw LoweringError("op " + op.name + ": result shape does not match its operands");
+      }
+    }
+
+    std::vector<std::string> operands;
+    for (int in : op.inputs) operands.push_back(operandExpr(in));
+    const std::string expr = lowering::elementwiseExpr(g_, op, operands);
+
+    ValInfo &v = vals_[static_cast<size_t>(outId)];
+    v.defined = true;
+    v.rank = rank;
+    std::ostringstream nm;
+    if (rank == ValRank::Tile) {
+      nm << "t" << outId;
+      v.ident = nm.str();
+      src_ << "  " << ctOf(outId) << " " << v.ident << "[NCHUNK][V];  // " << op.name << " -> " << outT.name << "\n";
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      line("#pragma unroll");
+      line("    for (int e = 0; e < V; ++e) {");
+      src_ << "      " << v.ident << "[j][e] = " << expr << ";\n";
+      line("    }");
+      line("  }");
+    } else {
+      nm << "u" << outId;
+      v.ident = nm.str();
+      src_ << "  const " << ctOf(outId) << " " << v.ident << " = " << expr << ";  // " << op.name << " -> " << outT.name
+           << "\n";
+      // A per-row value whose shape lacks the trailing 1 (reduce without keep_dims, or a reshape of one).
+      v.rowvecNoKeep = rowMode_ && outT.numel() != 1 && !outT.shape.empty() && outT.shape.back() != 1;
+    }
+  }
+
+  void emitReduce(const OpNode &op) {
+    const int inId = op.inputs[0];
+    const int outId = op.outputs[0];
+    const ValInfo &in = vals_[static_cast<size_t>(inId)];
+    if (!in.defined || in.rank != ValRank::Tile) {
+      throw LoweringError("op " + op.name + ": the reduced operand must span the innermost axis");
+    }
+    const DType od = g_.tensor(outId).dtype;
+    const std::string ct = computeTypeName(od);
+    const std::string tag = dtypeTag(od);
+    std::string red, init;
+    bool roundEachStep = (od == DType::F16 || od == DType::BF16 || od == DType::I8 || od == DType::I16);
+    auto largest = [&](bool negative) -> std::string {
+      // largest finite value of the result type (createFloatInitValue, MindSporeToLinalg.cpp:811-827)
+      double v = 0.0;
+      switch (od) {
+        case DType::F16: v = 65504.0; break;
+        case DType::BF16: v = 3.3895313892515355e38; break;
+        case DType::F32: v = 3.4028234663852886e38; break;
+        case DType::F64: v = 1.7976931348623157e308; break;
+        default: break;
+      }
+      return lowering::literalFor(od, negative ? -v : v);
+    };
+    auto intLimit = [&](bool minimum) -> std::string {
+      switch (od) {
+        case DType::I8: return minimum ? "(-128)" : "(127)";
+        case DType::I16: return minimum ? "(-32768)" : "(32767)";
+        case DType::I32: return minimum ? "(-2147483647 - 1)" : "(2147483647)";
+        case DType::I64: return minimum ? "(-9223372036854775807LL - 1)" : "(9223372036854775807LL)";
+        default: break;
+      }
+      throw LoweringError("op " + op.name + ": unsupported result type");
+    };
+    switch (op.kind) {
+      case OpKind::ReduceSum:
+        if (od == DType::Bool) throw LoweringError("ReduceSum on bool is not supported");
+        red = "akg::RedSum";
+        init = lowering::literalFor(od, 0.0);
+        break;
+      case OpKind::ReduceProd:
+        if (od == DType::Bool) throw LoweringError("ReducePrd on bool is not supported");
+        red = "akg::RedProd";
+        init = lowering::literalFor(od, 1.0);
+        break;
+      case OpKind::ReduceMax:
+        if (od == DType::Bool) throw LoweringError("ReduceMax on bool is not supported");
+        red = "akg::RedMax";
+        init = isFloatType(od) ? largest(true) : intLimit(true);
+        roundEachStep = false;
+        break;
+      case OpKind::ReduceMin:
+        if (od == DType::Bool) throw LoweringError("ReduceMin on bool is not supported");
+        red = "akg::RedMin";
+        init = isFloatType(od) ? largest(false) : intLimit(false);
+        roundEachStep = false;
+        break;
+      case OpKind::ReduceAll:
+        if (od != DType::Bool) throw LoweringError("ReduceAll needs a bool tensor");
+        red = "akg::RedAll";
+        init = "true";
+        roundEachStep = false;
+        break;
+      case OpKind::ReduceAny:
+        if (od != DType::Bool) throw LoweringError("ReduceAny needs a bool tensor");
+        red = "akg::RedAny";
+        init = "false";
+        roundEachStep = false;
+        break;
+      default:
+        throw LoweringError("internal: not a reduction");
+    }
+    if (std::string(computeTypeName(g_.tensor(inId).dtype)) != ct) {
+      throw LoweringError("op " + op.name + ": operand and result element types differ");
+    }
+    ValInfo &v = vals_[static_cast<size_t>(outId)];
+    std::ostringstream nm;
+    nm << "u" << outId;
+    const std::string acc = "acc" + std::to_string(outId);
+    src_ << "  " << ct << " " << acc << " = " << init << ";  // " << op.name << " -> " << g_.tensor(outId).name << "\n";
+    line("#pragma unroll");
+    line("  for (int j = 0; j < NCHUNK; ++j) {");
+    line("#pragma unroll");
+    line("    for (int e = 0; e < V; ++e) {");
+    std::string step = red + "::apply(" + acc + ", " + in.ident + "[j][e])";
+    if (roundEachStep) step = tag + "::rnd(" + step + ")";
+    if (raggedCols_) {
+      src_ << "      if (akg_ok[j]) " << acc << " = " << step << ";\n";
+    } else {
+      src_ << "      " << acc << " = " << step << ";\n";
+    }
+    line("    }");
+    line("  }");
+    std::string scratch = tpr_ > 64 ? "reinterpret_cast<" + ct + " *>(akg_scratch[" + std::to_string(reduceCount_ & 1) + "])"
+                                    : "static_cast<" + ct + " *>(nullptr)";
+    src_ << "  const " << ct << " " << nm.str() << " = " << (roundEachStep ? tag + "::rnd(" : "")
+         << "akg::group_reduce<" << red << ", TPR>(" << acc << ", " << scratch << ", tid)" << (roundEachStep ? ")" : "")
+         << ";\n";
+    ++reduceCount_;
+    v.defined = true;
+    v.rank = ValRank::Uniform;
+    v.ident = nm.str();
+    const TensorValue &outT = g_.tensor(outId);
+    v.rowvecNoKeep = outT.numel() != 1 && !outT.shape.empty() && outT.shape.back() != 1;
+  }
+
+  void emitOutputStore(size_t i) {
+    const int id = g_.outputs[i];
+    const TensorValue &t = g_.tensor(id);
+    const ValInfo &v = vals_[static_cast<size_t>(id)];
+    if (!v.defined) throw LoweringError("output " + t.name + " is never computed");
+    const std::string tag = tagOf(id);
+    const std::string ct = ctOf(id);
+    const bool fullSized = (t.numel() == numel_);
+    if (!rowMode_ || fullSized) {
+      if (!fullSized) throw LoweringError("output " + t.name + ": shape does not match the kernel's iteration space");
+      std::string src = v.ident;
+      if (v.rank != ValRank::Tile) {
+        // broadcast a uniform value over the chunk
+        src = "t_bcast" + std::to_string(i);
+        src_ << "  " << ct << " " << src << "[NCHUNK][V];\n";
+        line("#pragma unroll");
+        src_ << "  for (int j = 0; j < NCHUNK; ++j) akg::fill_chunk<" << tag << ", V>(" << src << "[j], " << v.ident
+             << ");\n";
+      }
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      std::string guard = "akg_ok[j]";
+      if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
+      std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
+      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V>(out" << i << " + " << offset << ", " << src
+           << "[j]);\n";
+      line("  }");
+    } else {
+      if (t.numel() != rows_) {
+        throw LoweringError("output " + t.name + ": shape is neither the reduced tensor's nor one value per row");
+      }
+      if (v.rank == ValRank::Tile) throw LoweringError("output " + t.name + ": internal rank mismatch");
+      std::string guard = "tcol == 0";
+      if (raggedRows_) guard += " && akg_row_ok";
+      src_ << "  if (" << guard << ") out" << i << "[akg_row] = " << tag << "::store(" << v.ident << ");\n";
+    }
+  }
+};
+
+}  // namespace
+
+LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options) {
+  if (graph.ops.empty()) throw LoweringError("op description has no ops");
+  bool hasMatMul = false;
+  for (const OpNode &op : graph.ops) {
+    if (op.kind == OpKind::MatMul) hasMatMul = true;
+  }
+  if (hasMatMul) return lowerGemmToHip(graph, options);
+  TileEmitter emitter(graph, options);
+  return emitter.run();
+}
+
+}  // namespace akg

@@ -1,0 +1,81 @@
+/**
+ * GPU lowering of an op graph for gfx950: picks a kernel family and a launch shape, and emits the HIP source
+ * of one kernel `<op>_kernel(inputs..., outputs...)`.
+ *
+ * Replaces the reference's generic GPU pipeline (akg-mlir/lib/Pipelines/GPUPipelines/GPUOpt.cpp:45-132:
+ * bufferize -> affine/scf loops -> AKGGPUMapping -> gpu.launch outlining -> NVVM). There a polyhedral
+ * scheduler maps one scalar element per thread per step; here each fusion class of the reference's own
+ * lattice (OperatorIdentify.cpp:51-93) has a hand-written skeleton for CDNA4 and the lowering only fills in
+ * the per-element chain:
+ *   Elementwise / Broadcast / Reshape  -> streaming kernel, 128-bit accesses, whole chain in registers
+ *   Reduction (direction X)            -> one row per thread group, row resident in registers across all
+ *                                         reductions of the fusion, wave64 butterfly + LDS reductions
+ *   Matmul (+ elementwise epilogue)    -> int8 MFMA tile kernel, epilogue applied to the int32 accumulators
+ * The kernel signature contract is the reference's: bare pointers, inputs then outputs
+ * (KernelOutliningExt.cpp:175-213, GPUCodegen.cpp:49-51).
+ */
+#ifndef AKG_HIP_HIPLOWERING_H_
+#define AKG_HIP_HIPLOWERING_H_
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "OpGraph.h"
+
+namespace akg {
+
+class LoweringError : public std::runtime_error {
+ public:
+  explicit LoweringError(const std::string &msg) : std::runtime_error(msg) {}
+};
+
+enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue };
+const char *kernelFamilyName(KernelFamily f);
+
+// Tuning knobs; 0 means "let the heuristic decide". They can be set through the environment
+// (AKG_HIP_VEC, AKG_HIP_TPR, AKG_HIP_CHUNKS, AKG_HIP_BLOCK) for sweeps.
+struct LoweringOptions {
+  int vec = 0;          // elements per chunk
+  int threadsPerRow = 0;
+  int chunks = 0;       // chunks per thread
+  int block = 0;        // threads per workgroup
+  int gemmVariant = 0;  // GEMM tile configuration selector
+  static LoweringOptions fromEnvironment();
+};
+
+struct LoweredKernel {
+  std::string kernelName;  // "<op>_kernel", as the reference names its outlined gpu.func
+  std::string source;      // HIP translation unit
+  KernelFamily family = KernelFamily::Elementwise;
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block[3] = {1, 1, 1};
+  uint64_t algorithmicBytes = 0;  // bytes of all kernel inputs and outputs, each counted once
+  uint64_t algorithmicOps = 0;    // 2*M*N*K for a contraction, 0 otherwise
+  std::string scheduleNote;       // human-readable schedule summary (vec, threads per row, ...)
+  // per kernel argument: [offset, sizes..., strides...] as in `<k>_shape_arg.txt`
+  std::vector<std::vector<int64_t>> shapeArgs;
+};
+
+LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options);
+
+// Family-specific entry used by lowerToHip (defined in HipLoweringGemm.cpp).
+LoweredKernel lowerGemmToHip(const OpGraph &graph, const LoweringOptions &options);
+
+// Shared helpers for the emitters.
+namespace lowering {
+const char *dtypeTag(DType t);          // "akg::f32", ...
+const char *computeTypeName(DType t);   // "float", "int", ...
+std::string literalFor(DType t, double value);  // constant of the compute type, already rounded to t
+uint64_t countAlgorithmicBytes(const OpGraph &g);
+std::vector<std::vector<int64_t>> buildShapeArgs(const OpGraph &g);
+// Expression of one elementwise op in terms of operand expressions (already in their compute types).
+std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vector<std::string> &operands);
+bool isElementwiseKind(OpKind k);
+bool isReduceKind(OpKind k);
+}  // namespace lowering
+
+}  // namespace akg
+
+#endif  // AKG_HIP_HIPLOWERING_H_

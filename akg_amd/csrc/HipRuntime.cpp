@@ -1,0 +1,549 @@
+/**
+ * C-ABI layer: compile (translate -> identify -> lower -> hiprtc -> artifacts) and the runtime launch shim.
+ *
+ * The launch shim replaces the CUDA driver-API program that the reference generates per kernel from a Python
+ * string template (akg-mlir/python/akg_mlir/utils/code_template.py:16-212, filled by gen_runtime_code.py:149-189).
+ * Differences that matter on MI355X: the code object is loaded once per handle, launches go to a caller's
+ * stream with device-resident buffers (akg_hip_launch), and the reference-style "host pointers in, host
+ * pointers out" call (akg_hip_run_host) is kept as a separate, explicitly slower entry point.
+ */
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+
+#include <cerrno>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <memory>
+#include <mutex>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "../../include/akg_hip.h"
+#include "HipLowering.h"
+#include "Json.h"
+#include "OpGraph.h"
+#include "Sha256.h"
+
+// Text of the device-side headers, generated at build time from kernels/*.hpp.
+#include "KernelLibEmbed.inc"
+
+#define AKG_HIP_VERSION_STRING "akg-hip 0.1 (gfx950)"
+
+struct akg_hip_kernel {
+  akg::OpGraph graph;
+  akg::LoweredKernel lowered;
+  std::vector<char> codeObject;
+  std::string codeSha256;
+  bool cacheHit = false;
+  std::mutex mu;
+  // loaded lazily on first launch, per device
+  struct Loaded {
+    int device = -1;
+    hipModule_t module = nullptr;
+    hipFunction_t function = nullptr;
+  };
+  std::vector<Loaded> loaded;
+};
+
+namespace {
+
+thread_local std::string g_lastError;
+
+int fail(int code, const std::string &msg) {
+  g_lastError = msg;
+  return code;
+}
+
+std::string hipErr(hipError_t e) { return std::string(hipGetErrorName(e)) + ": " + hipGetErrorString(e); }
+
+const std::vector<std::string> &compileFlags() {
+  // -ffp-contract=off: every op of the description is its own IEEE operation in the reference CPU pipeline;
+  //   fusing a*b+c into an fma would change results (and break the bit-exact int8 quantisation).
+  // packed-fp32-ops off: the compiler must not form v_pk_{add,mul,fma}_f32.
+  static const std::vector<std::string> flags = {
+    "--offload-arch=gfx950", "-O3",      "-std=c++17",     "-ffp-contract=off",
+    "-Xclang",               "-target-feature", "-Xclang", "-packed-fp32-ops",
+  };
+  return flags;
+}
+
+std::string sourceDigest(const std::string &source) {
+  akg::Sha256 h;
+  h.update(source.data(), source.size());
+  for (size_t i = 0; i < akg::kernel_lib::kNumHeaders; ++i) {
+    h.update(akg::kernel_lib::kHeaderNames[i], std::strlen(akg::kernel_lib::kHeaderNames[i]));
+    h.update(akg::kernel_lib::kHeaderTexts[i], std::strlen(akg::kernel_lib::kHeaderTexts[i]));
+  }
+  for (const auto &f : compileFlags()) h.update(f.data(), f.size());
+  return h.hexDigest();
+}
+
+bool readFile(const std::string &path, std::string *out) {
+  std::ifstream f(path, std::ios::binary);
+  if (!f) return false;
+  std::ostringstream ss;
+  ss << f.rdbuf();
+  *out = ss.str();
+  return true;
+}
+
+bool writeFile(const std::string &path, const void *data, size_t len) {
+  std::string tmp = path + ".tmp";
+  {
+    std::ofstream f(tmp, std::ios::binary | std::ios::trunc);
+    if (!f) return false;
+    f.write(static_cast<const char *>(data), static_cast<std::streamsize>(len));
+    if (!f) return false;
+  }
+  return std::rename(tmp.c_str(), path.c_str()) == 0;
+}
+
+bool makeDirs(const std::string &dir) {
+  if (dir.empty()) return false;
+  std::string cur;
+  for (size_t i = 0; i <= dir.size(); ++i) {
+    if (i == dir.size() || dir[i] == '/') {
+      if (!cur.empty() && cur != "/") {
+        if (mkdir(cur.c_str(), 0755) != 0 && errno != EEXIST) return false;
+      }
+    }
+    if (i < dir.size()) cur.push_back(dir[i]);
+  }
+  struct stat st;
+  return stat(dir.c_str(), &st) == 0 && S_ISDIR(st.st_mode);
+}
+
+int compileToCodeObject(const akg::LoweredKernel &k, std::vector<char> *code, std::string *log) {
+  hiprtcProgram prog = nullptr;
+  std::vector<const char *> headerTexts, headerNames;
+  for (size_t i = 0; i < akg::kernel_lib::kNumHeaders; ++i) {
+    headerTexts.push_back(akg::kernel_lib::kHeaderTexts[i]);
+    headerNames.push_back(akg::kernel_lib::kHeaderNames[i]);
+  }
+  std::string progName = k.kernelName + ".hip";
+  hiprtcResult r = hiprtcCreateProgram(&prog, k.source.c_str(), progName.c_str(), static_cast<int>(headerTexts.size()),
+                                       headerTexts.data(), headerNames.data());
+  if (r != HIPRTC_SUCCESS) {
+    *log = std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r);
+    return AKG_HIP_ERR_COMPILE;
+  }
+  std::vector<const char *> opts;
+  for (const auto &f : compileFlags()) opts.push_back(f.c_str());
+  r = hiprtcCompileProgram(prog, static_cast<int>(opts.size()), opts.data());
+  size_t logSize = 0;
+  if (hiprtcGetProgramLogSize(prog, &logSize) == HIPRTC_SUCCESS && logSize > 1) {
+    log->resize(logSize);
+    hiprtcGetProgramLog(prog, &(*log)[0]);
+  }
+  if (r != HIPRTC_SUCCESS) {
+    *log = std::string("hiprtcCompileProgram: ") + hiprtcGetErrorString(r) + "\n" + *log;
+    hiprtcDestroyProgram(&prog);
+    return AKG_HIP_ERR_COMPILE;
+  }
+  size_t size = 0;
+  r = hiprtcGetCodeSize(prog, &size);
+  if (r != HIPRTC_SUCCESS || size == 0) {
+    *log = "hiprtcGetCodeSize failed";
+    hiprtcDestroyProgram(&prog);
+    return AKG_HIP_ERR_COMPILE;
+  }
+  code->resize(size);
+  r = hiprtcGetCode(prog, code->data());
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS) {
+    *log = "hiprtcGetCode failed";
+    return AKG_HIP_ERR_COMPILE;
+  }
+  return AKG_HIP_OK;
+}
+
+std::string jsonEscape(const std::string &s) {
+  std::string o;
+  for (char c : s) {
+    if (c == '"' || c == '\\') {
+      o.push_back('\\');
+      o.push_back(c);
+    } else if (c == '\n') {
+      o += "\\n";
+    } else {
+      o.push_back(c);
+    }
+  }
+  return o;
+}
+
+// <op>.json: mapping result (GPUMapping.cpp:645-665) + kernelName / is_dynamic / sha256 (mlir_driver.py:807-815),
+// plus this backend's own bookkeeping keys.
+std::string metaJson(const akg_hip_kernel &k, const std::string &srcDigest) {
+  std::ostringstream os;
+  os << "{";
+  os << "\"blockIdx.x\": " << k.lowered.grid[0] << ", \"blockIdx.y\": " << k.lowered.grid[1]
+     << ", \"blockIdx.z\": " << k.lowered.grid[2] << ", ";
+  os << "\"threadIdx.x\": " << k.lowered.block[0] << ", \"threadIdx.y\": " << k.lowered.block[1]
+     << ", \"threadIdx.z\": " << k.lowered.block[2] << ", ";
+  os << "\"kernelName\": \"" << jsonEscape(k.lowered.kernelName) << "\", ";
+  os << "\"is_dynamic\": false, ";
+  os << "\"sha256\": \"" << k.codeSha256 << "\", ";
+  os << "\"target_info\": {\"arch\": \"gfx950\"}, ";
+  os << "\"family\": \"" << akg::kernelFamilyName(k.lowered.family) << "\", ";
+  os << "\"OperatorType\": \"" << akg::operatorTemplateName(k.graph.operatorTemplate) << "\", ";
+  os << "\"schedule\": \"" << jsonEscape(k.lowered.scheduleNote) << "\", ";
+  os << "\"algorithmic_bytes\": " << k.lowered.algorithmicBytes << ", ";
+  os << "\"algorithmic_ops\": " << k.lowered.algorithmicOps << ", ";
+  os << "\"source_sha256\": \"" << srcDigest << "\"";
+  os << "}";
+  return os.str();
+}
+
+std::string shapeArgText(const akg::LoweredKernel &k) {
+  std::ostringstream os;
+  os << "[";
+  for (size_t i = 0; i < k.shapeArgs.size(); ++i) {
+    os << (i ? "," : "") << "[";
+    for (size_t j = 0; j < k.shapeArgs[i].size(); ++j) os << (j ? "," : "") << k.shapeArgs[i][j];
+    os << "]";
+  }
+  os << "]";
+  return os.str();
+}
+
+int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel) {
+  if (outKernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "out_kernel is NULL");
+  *outKernel = nullptr;
+  std::unique_ptr<akg_hip_kernel> k(new akg_hip_kernel());
+  try {
+    k->graph = akg::translateJsonToOpGraph(jsonText);
+  } catch (const akg::json::ParseError &e) {
+    return fail(AKG_HIP_ERR_JSON, e.what());
+  } catch (const akg::TranslateError &e) {
+    return fail(AKG_HIP_ERR_TRANSLATE, e.what());
+  }
+  try {
+    k->lowered = akg::lowerToHip(k->graph, akg::LoweringOptions::fromEnvironment());
+  } catch (const akg::LoweringError &e) {
+    return fail(AKG_HIP_ERR_UNSUPPORTED, std::string("kernel ") + k->graph.name + ": " + e.what());
+  }
+  const std::string srcDigest = sourceDigest(k->lowered.source);
+
+  std::string dir = outDir ? std::string(outDir) : std::string();
+  std::string base;
+  if (!dir.empty()) {
+    if (!makeDirs(dir)) return fail(AKG_HIP_ERR_IO, "cannot create artifact directory " + dir);
+    base = dir + "/" + k->graph.name;
+    // cache probe
+    std::string meta, code;
+    if (readFile(base + ".json", &meta) && readFile(base + ".hsaco", &code) && !code.empty()) {
+      try {
+        akg::json::Value mv = akg::json::Value::parse(meta);
+        if (mv.contains("source_sha256") && mv.at("source_sha256").asString() == srcDigest &&
+            mv.contains("sha256") && mv.at("sha256").asString() == akg::Sha256::of(code)) {
+          k->codeObject.assign(code.begin(), code.end());
+          k->codeSha256 = mv.at("sha256").asString();
+          k->cacheHit = true;
+        }
+      } catch (const std::exception &) {
+        // unreadable meta: recompile
+      }
+    }
+  }
+  if (!k->cacheHit) {
+    std::string log;
+    int rc = compileToCodeObject(k->lowered, &k->codeObject, &log);
+    if (rc != AKG_HIP_OK) {
+      if (!base.empty()) (void)writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size());
+      return fail(rc, "device compilation of " + k->lowered.kernelName + " failed:\n" + log);
+    }
+    akg::Sha256 h;
+    h.update(k->codeObject.data(), k->codeObject.size());
+    k->codeSha256 = h.hexDigest();
+    if (!base.empty()) {
+      std::string meta = metaJson(*k, srcDigest);
+      std::string shapeArg = shapeArgText(k->lowered);
+      if (!writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size()) ||
+          !writeFile(base + ".hsaco", k->codeObject.data(), k->codeObject.size()) ||
+          !writeFile(base + "_shape_arg.txt", shapeArg.data(), shapeArg.size()) ||
+          !writeFile(base + ".json", meta.data(), meta.size())) {
+        return fail(AKG_HIP_ERR_IO, "cannot write artifacts under " + dir);
+      }
+    }
+  }
+  *outKernel = k.release();
+  g_lastError.clear();
+  return AKG_HIP_OK;
+}
+
+int ensureLoaded(akg_hip_kernel *k, hipFunction_t *fn) {
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipGetDevice: " + hipErr(e));
+  std::lock_guard<std::mutex> lock(k->mu);
+  for (const auto &l : k->loaded) {
+    if (l.device == device) {
+      *fn = l.function;
+      return AKG_HIP_OK;
+    }
+  }
+  akg_hip_kernel::Loaded l;
+  l.device = device;
+  e = hipModuleLoadData(&l.module, k->codeObject.data());
+  if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLoadData: " + hipErr(e));
+  e = hipModuleGetFunction(&l.function, l.module, k->lowered.kernelName.c_str());
+  if (e != hipSuccess) {
+    (void)hipModuleUnload(l.module);
+    return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + k->lowered.kernelName + "): " + hipErr(e));
+  }
+  k->loaded.push_back(l);
+  *fn = l.function;
+  return AKG_HIP_OK;
+}
+
+int numTensors(const akg_hip_kernel *k) { return static_cast<int>(k->graph.inputs.size() + k->graph.outputs.size()); }
+
+const akg::TensorValue &tensorAt(const akg_hip_kernel *k, int index) {
+  size_t nin = k->graph.inputs.size();
+  if (static_cast<size_t>(index) < nin) return k->graph.tensor(k->graph.inputs[static_cast<size_t>(index)]);
+  return k->graph.tensor(k->graph.outputs[static_cast<size_t>(index) - nin]);
+}
+
+int launchOn(akg_hip_kernel *k, hipFunction_t fn, void *const *devicePtrs, hipStream_t stream) {
+  int n = numTensors(k);
+  std::vector<void *> slots(static_cast<size_t>(n));
+  std::vector<void *> params(static_cast<size_t>(n));
+  for (int i = 0; i < n; ++i) {
+    slots[static_cast<size_t>(i)] = devicePtrs[i];
+    params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
+  }
+  hipError_t e = hipModuleLaunchKernel(fn, k->lowered.grid[0], k->lowered.grid[1], k->lowered.grid[2],
+                                       k->lowered.block[0], k->lowered.block[1], k->lowered.block[2], 0, stream,
+                                       params.data(), nullptr);
+  if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLaunchKernel: " + hipErr(e));
+  return AKG_HIP_OK;
+}
+
+int checkPtrs(const akg_hip_kernel *k, void *const *ptrs, int n) {
+  if (k == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel is NULL");
+  if (ptrs == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "pointer array is NULL");
+  if (n != numTensors(k)) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel " + k->graph.name + " takes " + std::to_string(numTensors(k)) +
+                                                " tensors, " + std::to_string(n) + " given");
+  }
+  for (int i = 0; i < n; ++i) {
+    if (ptrs[i] == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "tensor pointer " + std::to_string(i) + " is NULL");
+  }
+  return AKG_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int akg_hip_compile(const char *json_text, size_t json_len, const char *out_dir, akg_hip_kernel_t **out_kernel) {
+  if (json_text == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "json_text is NULL");
+  try {
+    return doCompile(std::string(json_text, json_len), out_dir, out_kernel);
+  } catch (const std::exception &e) {
+    return fail(AKG_HIP_ERR_INTERNAL, std::string("internal error: ") + e.what());
+  }
+}
+
+int akg_hip_compile_file(const char *info_path, const char *out_dir, akg_hip_kernel_t **out_kernel) {
+  if (info_path == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "info_path is NULL");
+  std::string path(info_path);
+  if (path.find("..") != std::string::npos) {
+    return fail(AKG_HIP_ERR_IO, "path " + path + " must not contain '..'");
+  }
+  std::string text;
+  if (!readFile(path, &text)) return fail(AKG_HIP_ERR_IO, "cannot read " + path);
+  try {
+    return doCompile(text, out_dir, out_kernel);
+  } catch (const std::exception &e) {
+    return fail(AKG_HIP_ERR_INTERNAL, std::string("internal error: ") + e.what());
+  }
+}
+
+int akg_hip_kernel_num_tensors(const akg_hip_kernel_t *kernel, int *n_tensors) {
+  if (kernel == nullptr || n_tensors == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  *n_tensors = numTensors(kernel);
+  return AKG_HIP_OK;
+}
+
+int akg_hip_kernel_tensor(const akg_hip_kernel_t *kernel, int index, akg_hip_tensor_desc *desc) {
+  if (kernel == nullptr || desc == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  if (index < 0 || index >= numTensors(kernel)) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "tensor index out of range");
+  const akg::TensorValue &t = tensorAt(kernel, index);
+  std::memset(desc, 0, sizeof(*desc));
+  desc->dtype = static_cast<int32_t>(t.dtype);
+  if (t.shape.size() > AKG_HIP_MAX_RANK) return fail(AKG_HIP_ERR_UNSUPPORTED, "tensor rank exceeds AKG_HIP_MAX_RANK");
+  desc->rank = static_cast<int32_t>(t.shape.size());
+  for (size_t i = 0; i < t.shape.size(); ++i) desc->shape[i] = t.shape[i];
+  desc->bytes = t.numel() * static_cast<int64_t>(akg::dtypeSize(t.dtype));
+  desc->is_output = static_cast<size_t>(index) >= kernel->graph.inputs.size() ? 1 : 0;
+  std::snprintf(desc->name, sizeof(desc->name), "%s", t.name.c_str());
+  return AKG_HIP_OK;
+}
+
+int akg_hip_kernel_get_info(const akg_hip_kernel_t *kernel, akg_hip_kernel_info *info) {
+  if (kernel == nullptr || info == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  std::memset(info, 0, sizeof(*info));
+  std::snprintf(info->kernel_name, sizeof(info->kernel_name), "%s", kernel->lowered.kernelName.c_str());
+  std::snprintf(info->family, sizeof(info->family), "%s", akg::kernelFamilyName(kernel->lowered.family));
+  std::snprintf(info->operator_type, sizeof(info->operator_type), "%s",
+                akg::operatorTemplateName(kernel->graph.operatorTemplate));
+  for (int i = 0; i < 3; ++i) {
+    info->grid[i] = kernel->lowered.grid[i];
+    info->block[i] = kernel->lowered.block[i];
+  }
+  info->algorithmic_bytes = kernel->lowered.algorithmicBytes;
+  info->algorithmic_ops = kernel->lowered.algorithmicOps;
+  info->cache_hit = kernel->cacheHit ? 1 : 0;
+  return AKG_HIP_OK;
+}
+
+int akg_hip_kernel_source(const akg_hip_kernel_t *kernel, const char **source) {
+  if (kernel == nullptr || source == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  *source = kernel->lowered.source.c_str();
+  return AKG_HIP_OK;
+}
+
+int akg_hip_launch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream) {
+  int rc = checkPtrs(kernel, device_ptrs, n_ptrs);
+  if (rc != AKG_HIP_OK) return rc;
+  hipFunction_t fn = nullptr;
+  rc = ensureLoaded(kernel, &fn);
+  if (rc != AKG_HIP_OK) return rc;
+  return launchOn(kernel, fn, device_ptrs, static_cast<hipStream_t>(stream));
+}
+
+int akg_hip_run_host(akg_hip_kernel_t *kernel, void *const *host_ptrs, int n_ptrs) {
+  int rc = checkPtrs(kernel, host_ptrs, n_ptrs);
+  if (rc != AKG_HIP_OK) return rc;
+  hipFunction_t fn = nullptr;
+  rc = ensureLoaded(kernel, &fn);
+  if (rc != AKG_HIP_OK) return rc;
+  const int n = numTensors(kernel);
+  std::vector<void *> dev(static_cast<size_t>(n), nullptr);
+  auto release = [&]() {
+    for (void *p : dev) {
+      if (p) (void)hipFree(p);
+    }
+  };
+  for (int i = 0; i < n; ++i) {
+    const akg::TensorValue &t = tensorAt(kernel, i);
+    size_t bytes = static_cast<size_t>(t.numel()) * akg::dtypeSize(t.dtype);
+    hipError_t e = hipMalloc(&dev[static_cast<size_t>(i)], bytes ? bytes : 1);
+    if (e != hipSuccess) {
+      release();
+      return fail(AKG_HIP_ERR_RUNTIME, "hipMalloc(" + std::to_string(bytes) + "): " + hipErr(e));
+    }
+    // Every tensor is copied in, outputs included: callers pre-fill outputs (with NaN in the reference
+    // harness) so that elements a kernel fails to write are detected.
+    e = hipMemcpy(dev[static_cast<size_t>(i)], host_ptrs[i], bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+      release();
+      return fail(AKG_HIP_ERR_RUNTIME, "hipMemcpy H2D: " + hipErr(e));
+    }
+  }
+  rc = launchOn(kernel, fn, dev.data(), nullptr);
+  if (rc == AKG_HIP_OK) {
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) rc = fail(AKG_HIP_ERR_RUNTIME, "kernel execution: " + hipErr(e));
+  }
+  if (rc == AKG_HIP_OK) {
+    const size_t nin = kernel->graph.inputs.size();
+    for (int i = static_cast<int>(nin); i < n; ++i) {
+      const akg::TensorValue &t = tensorAt(kernel, i);
+      size_t bytes = static_cast<size_t>(t.numel()) * akg::dtypeSize(t.dtype);
+      hipError_t e = hipMemcpy(host_ptrs[i], dev[static_cast<size_t>(i)], bytes, hipMemcpyDeviceToHost);
+      if (e != hipSuccess) {
+        rc = fail(AKG_HIP_ERR_RUNTIME, "hipMemcpy D2H: " + hipErr(e));
+        break;
+      }
+    }
+  }
+  release();
+  return rc;
+}
+
+int akg_hip_profile(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, int number, int repeat,
+                    double *avg_ms) {
+  int rc = checkPtrs(kernel, device_ptrs, n_ptrs);
+  if (rc != AKG_HIP_OK) return rc;
+  if (avg_ms == nullptr || number <= 0 || repeat <= 0) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "number and repeat must be positive and avg_ms non-NULL");
+  }
+  hipFunction_t fn = nullptr;
+  rc = ensureLoaded(kernel, &fn);
+  if (rc != AKG_HIP_OK) return rc;
+  hipStream_t stream = nullptr;
+  hipEvent_t start = nullptr, stop = nullptr;
+  hipError_t e = hipStreamCreate(&stream);
+  if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipStreamCreate: " + hipErr(e));
+  (void)hipEventCreate(&start);
+  (void)hipEventCreate(&stop);
+  auto cleanup = [&]() {
+    if (start) (void)hipEventDestroy(start);
+    if (stop) (void)hipEventDestroy(stop);
+    (void)hipStreamDestroy(stream);
+  };
+  // one untimed launch first, as the reference shim does
+  rc = launchOn(kernel, fn, device_ptrs, stream);
+  if (rc == AKG_HIP_OK && (e = hipStreamSynchronize(stream)) != hipSuccess) {
+    rc = fail(AKG_HIP_ERR_RUNTIME, "warm-up launch: " + hipErr(e));
+  }
+  double totalMs = 0.0;
+  for (int r = 0; r < repeat && rc == AKG_HIP_OK; ++r) {
+    (void)hipEventRecord(start, stream);
+    for (int i = 0; i < number && rc == AKG_HIP_OK; ++i) rc = launchOn(kernel, fn, device_ptrs, stream);
+    (void)hipEventRecord(stop, stream);
+    e = hipEventSynchronize(stop);
+    if (rc == AKG_HIP_OK && e != hipSuccess) rc = fail(AKG_HIP_ERR_RUNTIME, "timed launches: " + hipErr(e));
+    float ms = 0.0f;
+    if (rc == AKG_HIP_OK) {
+      (void)hipEventElapsedTime(&ms, start, stop);
+      totalMs += static_cast<double>(ms) / number;
+    }
+  }
+  cleanup();
+  if (rc == AKG_HIP_OK) *avg_ms = totalMs / repeat;
+  return rc;
+}
+
+void akg_hip_kernel_destroy(akg_hip_kernel_t *kernel) {
+  if (kernel == nullptr) return;
+  for (auto &l : kernel->loaded) {
+    if (l.module) (void)hipModuleUnload(l.module);
+  }
+  delete kernel;
+}
+
+const char *akg_hip_last_error(void) { return g_lastError.c_str(); }
+
+int akg_hip_translate(const char *json_text, size_t json_len, char **out_text) {
+  if (json_text == nullptr || out_text == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  *out_text = nullptr;
+  try {
+    akg::OpGraph g = akg::translateJsonToOpGraph(std::string(json_text, json_len));
+    std::string text = akg::printOpGraph(g);
+    char *buf = static_cast<char *>(std::malloc(text.size() + 1));
+    if (buf == nullptr) return fail(AKG_HIP_ERR_INTERNAL, "out of memory");
+    std::memcpy(buf, text.c_str(), text.size() + 1);
+    *out_text = buf;
+    return AKG_HIP_OK;
+  } catch (const akg::json::ParseError &e) {
+    return fail(AKG_HIP_ERR_JSON, e.what());
+  } catch (const akg::TranslateError &e) {
+    return fail(AKG_HIP_ERR_TRANSLATE, e.what());
+  } catch (const std::exception &e) {
+    return fail(AKG_HIP_ERR_INTERNAL, e.what());
+  }
+}
+
+void akg_hip_free_string(char *text) { std::free(text); }
+
+const char *akg_hip_version(void) { return AKG_HIP_VERSION_STRING; }
+
+}  // extern "C"

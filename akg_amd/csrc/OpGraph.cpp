@@ -1,0 +1,619 @@
+#include "OpGraph.h"
+
+#include <algorithm>
+#include <sstream>
+
+#include "Json.h"
+
+namespace akg {
+namespace {
+
+// Field names of the description format (TranslateToMindsporeDialect.cpp:55-75).
+constexpr auto kProcess = "process";
+constexpr auto kArch = "arch";
+constexpr auto kComputeCapability = "compute_capability";
+constexpr auto kTargetInfo = "target_info";
+constexpr auto kInputDesc = "input_desc";
+constexpr auto kOutputDesc = "output_desc";
+constexpr auto kTensorName = "tensor_name";
+constexpr auto kShape = "shape";
+constexpr auto kDataType = "data_type";
+constexpr auto kOpDesc = "op_desc";
+constexpr auto kName = "name";
+constexpr auto kAttr = "attr";
+constexpr auto kValue = "value";
+constexpr auto kPtrAddress = "ptr_address";
+constexpr auto kAxis = "axis";
+constexpr auto kTransposeA = "transpose_a";
+constexpr auto kTransposeB = "transpose_b";
+
+struct OpTableEntry {
+  const char *name;
+  OpKind kind;
+};
+
+// Op-name table: every name of MindBuilder::initMindOpFactory (:417-486). Names that this backend has no
+// kernel family for are kept in the table as Unsupported so that the error says so precisely.
+const OpTableEntry kOpTable[] = {
+  {"Abs", OpKind::Abs},
+  {"Neg", OpKind::Neg},
+  {"Exp", OpKind::Exp},
+  {"Log", OpKind::Log},
+  {"Tanh", OpKind::Tanh},
+  {"ACos", OpKind::Acos},
+  {"ASin", OpKind::Asin},
+  {"Sin", OpKind::Sin},
+  {"Cos", OpKind::Cos},
+  {"Asinh", OpKind::Asinh},
+  {"Acosh", OpKind::Acosh},
+  {"Atan", OpKind::Atan},
+  {"Rsqrt", OpKind::Rsqrt},
+  {"Floor", OpKind::Floor},
+  {"Square", OpKind::Square},
+  {"Sqrt", OpKind::Sqrt},
+  {"IsInf", OpKind::IsInf},
+  {"IsFinite", OpKind::IsFinite},
+  {"IsNan", OpKind::IsNan},
+  {"Reciprocal", OpKind::Reciprocal},
+  {"LogicalNot", OpKind::LogicalNot},
+  {"LogicalAnd", OpKind::LogicalAnd},
+  {"LogicalOr", OpKind::LogicalOr},
+  {"Pow", OpKind::Pow},
+  {"Add", OpKind::Add},
+  {"Sub", OpKind::Sub},
+  {"Maximum", OpKind::Maximum},
+  {"Minimum", OpKind::Minimum},
+  {"Mul", OpKind::Mul},
+  {"Div", OpKind::Div},
+  {"RealDiv", OpKind::Div},
+  {"Equal", OpKind::Equal},
+  {"GreaterEqual", OpKind::GreaterEqual},
+  {"Greater", OpKind::Greater},
+  {"LessEqual", OpKind::LessEqual},
+  {"Less", OpKind::Less},
+  {"NotEqual", OpKind::NotEqual},
+  {"Atan2", OpKind::Atan2},
+  {"Select", OpKind::Select},
+  {"ReduceMax", OpKind::ReduceMax},
+  {"ReduceMin", OpKind::ReduceMin},
+  {"ReduceSum", OpKind::ReduceSum},
+  {"ReducePrd", OpKind::ReduceProd},
+  {"ReduceAll", OpKind::ReduceAll},
+  {"ReduceAny", OpKind::ReduceAny},
+  {"ElemAny", OpKind::Unsupported},
+  {"ArgMax", OpKind::Unsupported},
+  {"BroadcastTo", OpKind::BroadcastTo},
+  {"Slice", OpKind::Unsupported},
+  {"Tile", OpKind::Unsupported},
+  {"Concat", OpKind::Unsupported},
+  {"Reshape", OpKind::Reshape},
+  {"Transpose", OpKind::Unsupported},
+  {"Split", OpKind::Unsupported},
+  {"Pad", OpKind::Unsupported},
+  {"Gather", OpKind::Unsupported},
+  {"InplaceAssign", OpKind::Unsupported},
+  {"Assign", OpKind::Unsupported},
+  {"UnsortedSegmentSum", OpKind::Unsupported},
+  {"StridedSlice", OpKind::Unsupported},
+  {"AddN", OpKind::AddN},
+  {"MatMul", OpKind::MatMul},
+  {"BatchMatMul", OpKind::Unsupported},
+  {"Cast", OpKind::Cast},
+};
+
+OpKind lookupOpKind(const std::string &name) {
+  for (const auto &e : kOpTable) {
+    if (name == e.name) return e.kind;
+  }
+  return OpKind::Unknown;
+}
+
+bool isReduceKind(OpKind k) {
+  return k == OpKind::ReduceSum || k == OpKind::ReduceMax || k == OpKind::ReduceMin || k == OpKind::ReduceProd ||
+         k == OpKind::ReduceAll || k == OpKind::ReduceAny;
+}
+
+// Ops whose second JSON input is an attribute in disguise (attrInputOpList, :123-125).
+bool isIndex1DAttrAsInput(const std::string &opName, size_t inputIdx) {
+  static const char *const kList[] = {"Reshape",   "BroadcastTo", "ReduceMax", "ReduceMin", "ReduceSum", "ReducePrd",
+                                      "ReduceAll", "ReduceAny",   "ArgMax",    "Transpose", "Tile"};
+  if (inputIdx != 1) return false;
+  for (const char *n : kList) {
+    if (opName == n) return true;
+  }
+  return false;
+}
+
+std::vector<int64_t> readShape(const json::Value &desc) {
+  // A missing shape means [1] (:322-325,393-395).
+  if (!desc.contains(kShape)) return {1};
+  std::vector<int64_t> shape = desc.at(kShape).asIntVector();
+  if (shape.empty()) return {1};
+  return shape;
+}
+
+const json::Value *findAttr(const json::Value &attrs, const std::string &name) {
+  for (size_t i = 0; i < attrs.size(); ++i) {
+    const json::Value &a = attrs[i];
+    if (a.contains(kName) && a.at(kName).isString() && a.at(kName).asString() == name) {
+      return &a.at(kValue);
+    }
+  }
+  return nullptr;
+}
+
+void checkAttrTypes(const json::Value &attrs, const std::string &opName) {
+  // Attribute records are {name, data_type in {bool,str,listInt,int,float}, value}; anything else is fatal in
+  // the reference (createMindsporeAttribute :504-531).
+  for (size_t i = 0; i < attrs.size(); ++i) {
+    const json::Value &a = attrs[i];
+    if (!a.contains(kDataType)) continue;
+    const std::string &t = a.at(kDataType).asString();
+    if (t != "bool" && t != "str" && t != "listInt" && t != "int" && t != "float") {
+      throw TranslateError("op " + opName + ": attribute type " + t + " is not supported");
+    }
+  }
+}
+
+class GraphBuilder {
+ public:
+  explicit GraphBuilder(const json::Value &root) : root_(root) {}
+
+  OpGraph build() {
+    if (!root_.isObject()) throw TranslateError("op description must be a JSON object");
+    graph_.name = root_.at("op").asString();
+    if (graph_.name.empty()) graph_.name = "main";
+    graph_.process = root_.at(kProcess).asString();
+    if (root_.contains(kTargetInfo) && root_.at(kTargetInfo).isObject()) {
+      const json::Value &ti = root_.at(kTargetInfo);
+      if (ti.contains(kComputeCapability) && ti.at(kComputeCapability).isString()) {
+        graph_.computeCapability = ti.at(kComputeCapability).asString();
+      }
+      if (ti.contains(kArch) && ti.at(kArch).isString()) graph_.arch = ti.at(kArch).asString();
+    }
+    parseInputs();
+    parseOps();
+    parseOutputs();
+    return std::move(graph_);
+  }
+
+ private:
+  const json::Value &root_;
+  OpGraph graph_;
+  std::map<std::string, int> operandList_;  // tensor_name -> tensor id (operandList, :110)
+
+  int addTensor(const std::string &name, DType dtype, const std::vector<int64_t> &shape) {
+    for (int64_t d : shape) {
+      if (d < 0) {
+        throw TranslateError("tensor " + name + ": dynamic dimensions (-1) are not supported by the HIP backend");
+      }
+    }
+    TensorValue t;
+    t.name = name;
+    t.dtype = dtype;
+    t.shape = shape;
+    graph_.tensors.push_back(t);
+    return static_cast<int>(graph_.tensors.size()) - 1;
+  }
+
+  void parseInputs() {
+    const json::Value &inputs = root_.at(kInputDesc);
+    for (size_t i = 0; i < inputs.size(); ++i) {
+      // input_desc is a list of single-element lists (:320).
+      const json::Value &desc = inputs[i][0];
+      std::string tensorName = desc.at(kTensorName).asString();
+      DType dtype = parseDType(desc.at(kDataType).asString());
+      int id = addTensor(tensorName, dtype, readShape(desc));
+      graph_.tensors[static_cast<size_t>(id)].inputIndex = static_cast<int>(i);
+      graph_.inputs.push_back(id);
+      operandList_[tensorName] = id;
+    }
+  }
+
+  int operandFor(const json::Value &desc, const std::string &opName) {
+    std::string tensorName = desc.at(kTensorName).asString();
+    auto it = operandList_.find(tensorName);
+    if (it != operandList_.end()) return it->second;
+    // Not yet defined: must be a constant carried in the JSON (handleDefaultOperand :793-808).
+    if (!desc.contains(kValue)) {
+      throw TranslateError("op " + opName + ": operand " + tensorName + " is undefined and carries no value");
+    }
+    const json::Value &val = desc.at(kValue);
+    std::vector<int64_t> shape = readShape(desc);
+    DType dtype = parseDType(desc.at(kDataType).asString());
+    double v = 0.0;
+    if (val.isNumber() || val.isBool()) {
+      v = val.asDouble();
+    } else if (val.isArray() && val.size() == 1 && (val[0].isNumber() || val[0].isBool())) {
+      v = val[0].asDouble();
+    } else if (val.isArray()) {
+      throw TranslateError("op " + opName + ": array-valued constant operand " + tensorName +
+                           " is not supported by the HIP backend");
+    } else {
+      throw TranslateError("Unexpected value from const input of op: " + opName);
+    }
+    int64_t n = 1;
+    for (int64_t d : shape) n *= d;
+    if (n != 1) {
+      throw TranslateError("op " + opName + ": constant operand " + tensorName + " must have one element");
+    }
+    int id = addTensor(tensorName, dtype, shape);
+    TensorValue &t = graph_.tensors[static_cast<size_t>(id)];
+    t.isConst = true;
+    // Integer constants are truncated toward zero as in buildDenseElementsAttr (:1390-1393).
+    t.constValue = isFloatType(dtype) ? v : static_cast<double>(static_cast<int64_t>(v));
+    operandList_[tensorName] = id;
+    return id;
+  }
+
+  void parseOps() {
+    const json::Value &ops = root_.at(kOpDesc);
+    for (size_t i = 0; i < ops.size(); ++i) {
+      const json::Value &opDesc = ops[i];
+      OpNode node;
+      node.name = opDesc.at(kName).asString();
+      node.kind = lookupOpKind(node.name);
+      static const json::Value kNoAttrs;
+      const json::Value &attrs = (opDesc.contains(kAttr) && opDesc.at(kAttr).isArray()) ? opDesc.at(kAttr) : kNoAttrs;
+      checkAttrTypes(attrs, node.name);
+      if (const json::Value *fake = findAttr(attrs, "fake_output")) {
+        if (fake->isBool() && fake->asBool()) {
+          throw TranslateError("op " + node.name + ": fake_output (in-place aliasing) is not supported");
+        }
+      }
+      if (opDesc.contains(kPtrAddress) && opDesc.at(kPtrAddress).isString()) {
+        node.ptrAddress = opDesc.at(kPtrAddress).asString();
+      }
+      const json::Value &inputDesc = opDesc.at(kInputDesc);
+      const json::Value &outputDesc = opDesc.at(kOutputDesc);
+      if (outputDesc.size() == 0) {
+        throw TranslateError("Error occurs when converting json: op name: " + node.name + " has empty outputDesc");
+      }
+
+      if (node.kind == OpKind::Unknown || node.kind == OpKind::Unsupported) {
+        // Keep the node (the translator itself accepts it); the scheduler rejects the kernel.
+        for (size_t j = 0; j < inputDesc.size(); ++j) {
+          const json::Value &d = inputDesc[j][0];
+          auto it = operandList_.find(d.at(kTensorName).asString());
+          if (it != operandList_.end()) node.inputs.push_back(it->second);
+        }
+      } else {
+        for (size_t j = 0; j < inputDesc.size(); ++j) {
+          if (isIndex1DAttrAsInput(node.name, j)) continue;
+          if (node.kind == OpKind::Cast && j > 0) continue;  // convertCastOp keeps the first operand only (:1351-1360)
+          node.inputs.push_back(operandFor(inputDesc[j][0], node.name));
+        }
+      }
+
+      if (isReduceKind(node.kind)) {
+        // Axis from the second input's value or from attr "axis" (:1280-1300); keep_dims defaults to false.
+        std::vector<int64_t> axes;
+        if (inputDesc.size() == 2) {
+          axes = inputDesc[1][0].at(kValue).asIntVector();
+        } else if (const json::Value *a = findAttr(attrs, kAxis)) {
+          axes = a->asIntVector();
+        } else {
+          throw TranslateError("op " + node.name + ": cannot find attribute axis");
+        }
+        int64_t rank = static_cast<int64_t>(readShape(inputDesc[0][0]).size());
+        if (axes.empty()) {
+          // An empty listInt becomes [1] in createMindsporeAttribute (:516-518).
+          axes.push_back(1);
+        }
+        for (auto &a : axes) {
+          if (a < 0) a += rank;
+          if (a < 0 || a >= rank) throw TranslateError("op " + node.name + ": reduce axis out of range");
+        }
+        std::sort(axes.begin(), axes.end());
+        axes.erase(std::unique(axes.begin(), axes.end()), axes.end());
+        node.axes = axes;
+        if (const json::Value *k = findAttr(attrs, "keep_dims")) node.keepDims = k->asBool();
+      }
+      if (node.kind == OpKind::MatMul) {
+        if (const json::Value *a = findAttr(attrs, kTransposeA)) node.transposeA = a->asBool();
+        if (const json::Value *b = findAttr(attrs, kTransposeB)) node.transposeB = b->asBool();
+      }
+
+      int opIndex = static_cast<int>(graph_.ops.size());
+      for (size_t j = 0; j < outputDesc.size(); ++j) {
+        const json::Value &d = outputDesc[j];
+        std::string tensorName = d.at(kTensorName).asString();
+        DType dtype = parseDType(d.at(kDataType).asString());
+        int id = addTensor(tensorName, dtype, readShape(d));
+        graph_.tensors[static_cast<size_t>(id)].producer = opIndex;
+        node.outputs.push_back(id);
+        operandList_[tensorName] = id;
+      }
+      graph_.ops.push_back(node);
+    }
+  }
+
+  void parseOutputs() {
+    const json::Value &outputs = root_.at(kOutputDesc);
+    for (size_t i = 0; i < outputs.size(); ++i) {
+      const json::Value &desc = outputs[i];
+      std::string tensorName = desc.at(kTensorName).asString();
+      auto it = operandList_.find(tensorName);
+      if (it == operandList_.end()) {
+        throw TranslateError("output " + tensorName + " is not produced by any op");
+      }
+      TensorValue &t = graph_.tensors[static_cast<size_t>(it->second)];
+      DType dtype = parseDType(desc.at(kDataType).asString());
+      if (dtype != t.dtype) {
+        throw TranslateError("output " + tensorName + ": data_type differs between output_desc and its producer");
+      }
+      std::vector<int64_t> shape = readShape(desc);
+      int64_t n = 1;
+      for (int64_t d : shape) n *= d;
+      if (n != t.numel()) {
+        throw TranslateError("output " + tensorName + ": shape differs between output_desc and its producer");
+      }
+      if (t.outputIndex >= 0) throw TranslateError("output " + tensorName + " is listed twice");
+      if (t.inputIndex >= 0) throw TranslateError("output " + tensorName + " aliases a kernel input");
+      t.outputIndex = static_cast<int>(i);
+      graph_.outputs.push_back(it->second);
+    }
+    if (graph_.outputs.empty()) throw TranslateError("op description has no outputs");
+  }
+};
+
+bool sameShape(const std::vector<int64_t> &a, const std::vector<int64_t> &b) { return a == b; }
+
+OperatorTemplate templateOfOp(const OpGraph &g, const OpNode &op) {
+  switch (op.kind) {
+    case OpKind::ReduceSum:
+    case OpKind::ReduceMax:
+    case OpKind::ReduceMin:
+    case OpKind::ReduceProd:
+    case OpKind::ReduceAll:
+    case OpKind::ReduceAny:
+      return OperatorTemplate::Reduction;
+    case OpKind::MatMul:
+      return OperatorTemplate::Matmul;
+    case OpKind::Reshape:
+      return OperatorTemplate::Reshape;
+    case OpKind::BroadcastTo:
+      return OperatorTemplate::Broadcast;
+    case OpKind::Unknown:
+    case OpKind::Unsupported:
+      return OperatorTemplate::Default;
+    default: {
+      // Elementwise when every operand has the result's shape, Broadcast otherwise (elementwiseMatch,
+      // OperatorIdentify.cpp:34-48).
+      const auto &resShape = g.tensor(op.outputs[0]).shape;
+      for (int in : op.inputs) {
+        if (!sameShape(g.tensor(in).shape, resShape)) return OperatorTemplate::Broadcast;
+      }
+      return OperatorTemplate::Elementwise;
+    }
+  }
+}
+
+}  // namespace
+
+int64_t TensorValue::numel() const {
+  int64_t n = 1;
+  for (int64_t d : shape) n *= d;
+  return n;
+}
+
+const char *dtypeName(DType t) {
+  switch (t) {
+    case DType::Bool: return "bool";
+    case DType::I8: return "int8";
+    case DType::I16: return "int16";
+    case DType::I32: return "int32";
+    case DType::I64: return "int64";
+    case DType::F16: return "float16";
+    case DType::BF16: return "bfloat16";
+    case DType::F32: return "float32";
+    case DType::F64: return "float64";
+  }
+  return "?";
+}
+
+size_t dtypeSize(DType t) {
+  switch (t) {
+    case DType::Bool:
+    case DType::I8: return 1;
+    case DType::I16:
+    case DType::F16:
+    case DType::BF16: return 2;
+    case DType::I32:
+    case DType::F32: return 4;
+    case DType::I64:
+    case DType::F64: return 8;
+  }
+  return 0;
+}
+
+bool isFloatType(DType t) { return t == DType::F16 || t == DType::BF16 || t == DType::F32 || t == DType::F64; }
+
+DType parseDType(const std::string &name) {
+  if (name == "bool" || name == "int1") return DType::Bool;
+  if (name == "int8" || name == "uint8" || name == "sint8") return DType::I8;
+  if (name == "int16") return DType::I16;
+  if (name == "int32") return DType::I32;
+  if (name == "int64") return DType::I64;
+  if (name == "float16") return DType::F16;
+  if (name == "bfloat16") return DType::BF16;
+  if (name == "float32") return DType::F32;
+  if (name == "float64") return DType::F64;
+  throw TranslateError("Error occurs when converting json: data type " + name + " is not supported");
+}
+
+const char *opKindName(OpKind k) {
+  switch (k) {
+    case OpKind::Abs: return "abs";
+    case OpKind::Neg: return "neg";
+    case OpKind::Exp: return "exp";
+    case OpKind::Log: return "log";
+    case OpKind::Tanh: return "tanh";
+    case OpKind::Rsqrt: return "rsqrt";
+    case OpKind::Sqrt: return "sqrt";
+    case OpKind::Reciprocal: return "inv";
+    case OpKind::Floor: return "floor";
+    case OpKind::Square: return "square";
+    case OpKind::Sin: return "sin";
+    case OpKind::Cos: return "cos";
+    case OpKind::Asin: return "asin";
+    case OpKind::Acos: return "acos";
+    case OpKind::Atan: return "atan";
+    case OpKind::Asinh: return "asinh";
+    case OpKind::Acosh: return "acosh";
+    case OpKind::IsInf: return "isinf";
+    case OpKind::IsFinite: return "isfinite";
+    case OpKind::IsNan: return "isnan";
+    case OpKind::LogicalNot: return "logical_not";
+    case OpKind::Cast: return "cast";
+    case OpKind::Add: return "add";
+    case OpKind::Sub: return "sub";
+    case OpKind::Mul: return "mul";
+    case OpKind::Div: return "div";
+    case OpKind::Maximum: return "maximum";
+    case OpKind::Minimum: return "minimum";
+    case OpKind::Pow: return "pow";
+    case OpKind::Atan2: return "atan2";
+    case OpKind::Equal: return "equal";
+    case OpKind::NotEqual: return "not_equal";
+    case OpKind::Greater: return "greater";
+    case OpKind::GreaterEqual: return "greater_equal";
+    case OpKind::Less: return "less";
+    case OpKind::LessEqual: return "less_equal";
+    case OpKind::LogicalAnd: return "logical_and";
+    case OpKind::LogicalOr: return "logical_or";
+    case OpKind::Select: return "select";
+    case OpKind::ReduceSum: return "reduce_sum";
+    case OpKind::ReduceMax: return "reduce_max";
+    case OpKind::ReduceMin: return "reduce_min";
+    case OpKind::ReduceProd: return "reduce_prod";
+    case OpKind::ReduceAll: return "reduce_all";
+    case OpKind::ReduceAny: return "reduce_any";
+    case OpKind::Reshape: return "reshape";
+    case OpKind::BroadcastTo: return "broadcast_to";
+    case OpKind::MatMul: return "matmul";
+    case OpKind::AddN: return "addn";
+    case OpKind::Unsupported: return "unsupported";
+    case OpKind::Unknown: return "unknown";
+  }
+  return "?";
+}
+
+const char *operatorTemplateName(OperatorTemplate t) {
+  switch (t) {
+    case OperatorTemplate::Default: return "Default";
+    case OperatorTemplate::Elementwise: return "Elementwise";
+    case OperatorTemplate::Broadcast: return "Broadcast";
+    case OperatorTemplate::Reshape: return "Reshape";
+    case OperatorTemplate::Transpose: return "Transpose";
+    case OperatorTemplate::Reduction: return "Reduction";
+    case OperatorTemplate::Matmul: return "Matmul";
+    case OperatorTemplate::Conv: return "Conv";
+  }
+  return "?";
+}
+
+OpGraph translateJsonToOpGraph(const std::string &jsonText) {
+  json::Value root = json::Value::parse(jsonText);
+  GraphBuilder builder(root);
+  OpGraph g = builder.build();
+  identifyOperator(&g);
+  return g;
+}
+
+void identifyOperator(OpGraph *graph) {
+  OperatorTemplate cur = OperatorTemplate::Default;
+  ReduceDirection dir = ReduceDirection::Unknown;
+  for (const OpNode &op : graph->ops) {
+    OperatorTemplate t = templateOfOp(*graph, op);
+    if (t > cur) cur = t;
+    if (t == OperatorTemplate::Reduction && !op.inputs.empty()) {
+      const auto &inShape = graph->tensor(op.inputs[0]).shape;
+      int64_t rank = static_cast<int64_t>(inShape.size());
+      // Count only axes that really reduce something (extent > 1), as size-1 axes are redundant reductions
+      // (akg-mlir/lib/Dialect/MindSpore/Transforms/RemoveRedundantReduce.cpp).
+      std::vector<int64_t> real;
+      int64_t nonUnit = 0;
+      for (int64_t d = 0; d < rank; ++d) {
+        if (inShape[static_cast<size_t>(d)] > 1) ++nonUnit;
+      }
+      for (int64_t a : op.axes) {
+        if (inShape[static_cast<size_t>(a)] > 1) real.push_back(a);
+      }
+      ReduceDirection d = ReduceDirection::Unknown;
+      if (static_cast<int64_t>(real.size()) == nonUnit) {
+        d = ReduceDirection::All;
+      } else if (!real.empty()) {
+        // X when the reduced axes are exactly the innermost non-unit ones.
+        bool innermost = true;
+        int64_t expect = rank - 1;
+        for (auto it = real.rbegin(); it != real.rend(); ++it) {
+          while (expect >= 0 && inShape[static_cast<size_t>(expect)] == 1) --expect;
+          if (*it != expect) {
+            innermost = false;
+            break;
+          }
+          --expect;
+        }
+        d = innermost ? ReduceDirection::X : ReduceDirection::Y;
+      }
+      if (dir == ReduceDirection::Unknown) {
+        dir = d;
+      } else if (dir != d && d != ReduceDirection::Unknown) {
+        dir = ReduceDirection::Y;  // mixed directions: treated as the general (non-X) case
+      }
+    }
+  }
+  graph->operatorTemplate = cur;
+  graph->reduceDirection = dir;
+}
+
+std::string printOpGraph(const OpGraph &g) {
+  std::ostringstream os;
+  auto typeStr = [&](const TensorValue &t) {
+    std::ostringstream s;
+    s << "tensor<";
+    for (int64_t d : t.shape) s << d << "x";
+    s << dtypeName(t.dtype) << ">";
+    return s.str();
+  };
+  os << "func.func @" << g.name << "(";
+  for (size_t i = 0; i < g.inputs.size(); ++i) {
+    const TensorValue &t = g.tensor(g.inputs[i]);
+    os << (i ? ", " : "") << "%" << t.name << ": " << typeStr(t);
+  }
+  os << ") -> (";
+  for (size_t i = 0; i < g.outputs.size(); ++i) os << (i ? ", " : "") << typeStr(g.tensor(g.outputs[i]));
+  os << ") attributes {mindspore_kernel, process = \"" << g.process << "\", compute_capability = \""
+     << g.computeCapability << "\", arch = \"" << g.arch << "\", OperatorType = \""
+     << operatorTemplateName(g.operatorTemplate) << "\"} {\n";
+  for (const TensorValue &t : g.tensors) {
+    if (t.isConst) {
+      os << "  %" << t.name << " = \"mindspore.const\"() {value = " << t.constValue << "} : " << typeStr(t) << "\n";
+    }
+  }
+  for (const OpNode &op : g.ops) {
+    os << "  ";
+    for (size_t i = 0; i < op.outputs.size(); ++i) os << (i ? ", " : "") << "%" << g.tensor(op.outputs[i]).name;
+    os << " = \"mindspore." << opKindName(op.kind) << "\"(";
+    for (size_t i = 0; i < op.inputs.size(); ++i) os << (i ? ", " : "") << "%" << g.tensor(op.inputs[i]).name;
+    os << ")";
+    if (!op.axes.empty()) {
+      os << " {axis = [";
+      for (size_t i = 0; i < op.axes.size(); ++i) os << (i ? ", " : "") << op.axes[i];
+      os << "], keepdims = " << (op.keepDims ? "true" : "false") << "}";
+    }
+    if (op.kind == OpKind::MatMul) {
+      os << " {transpose_a = " << (op.transposeA ? "true" : "false")
+         << ", transpose_b = " << (op.transposeB ? "true" : "false") << "}";
+    }
+    if (op.kind == OpKind::Unknown) os << " {ori_op = \"" << op.name << "\"}";
+    os << " : " << typeStr(g.tensor(op.outputs[0])) << "\n";
+  }
+  os << "  return";
+  for (size_t i = 0; i < g.outputs.size(); ++i) os << (i ? ", " : " ") << "%" << g.tensor(g.outputs[i]).name;
+  os << "\n}\n";
+  return os.str();
+}
+
+}  // namespace akg

@@ -1,0 +1,432 @@
+/**
+ * Device-side support library for the kernels the HIP lowering emits (gfx950 / CDNA4, wavefront 64).
+ *
+ * Everything here is written for one target only. The lowering emits one `extern "C" __global__` function
+ * per op description; that function is a thin, fully unrolled composition of the pieces below:
+ *   - dtype traits: how each element type of the op description is stored in memory, which register type
+ *     it is computed in, and how a result is rounded back to the declared type after every op (the CPU
+ *     pipeline of the reference computes each op in its declared result type),
+ *   - 128-bit vector global loads/stores,
+ *   - the per-op scalar semantics (tosa/linalg/libm lowering of the reference CPU pipeline),
+ *   - row-group reductions: xor butterfly inside a wavefront (DPP for the quad steps), LDS across wavefronts.
+ *
+ * Compiled by hiprtc, so it includes nothing.
+ */
+#pragma once
+
+namespace akg {
+
+typedef unsigned char u8;
+typedef signed char s8;
+typedef unsigned short u16;
+typedef unsigned int u32;
+typedef unsigned long long u64;
+typedef _Float16 half_t;
+typedef __bf16 bfloat_t;
+
+constexpr int kWaveSize = 64;
+
+#define AKG_DEV __device__ __forceinline__
+
+// ---------------------------------------------------------------------------------------------------------
+// dtype traits. `storage` is the in-memory element, `compute` the register type, `rnd` rounds a compute
+// value to the nearest representable value of the declared type (round-to-nearest-even, what arith.truncf
+// does in the reference CPU pipeline).
+// ---------------------------------------------------------------------------------------------------------
+struct f32 {
+  typedef float storage;
+  typedef float compute;
+  static AKG_DEV compute rnd(compute x) { return x; }
+  static AKG_DEV compute load(storage s) { return s; }
+  static AKG_DEV storage store(compute x) { return x; }
+};
+struct f64 {
+  typedef double storage;
+  typedef double compute;
+  static AKG_DEV compute rnd(compute x) { return x; }
+  static AKG_DEV compute load(storage s) { return s; }
+  static AKG_DEV storage store(compute x) { return x; }
+};
+struct f16 {
+  typedef half_t storage;
+  typedef float compute;
+  static AKG_DEV compute rnd(compute x) { return static_cast<float>(static_cast<half_t>(x)); }
+  static AKG_DEV compute load(storage s) { return static_cast<float>(s); }
+  static AKG_DEV storage store(compute x) { return static_cast<half_t>(x); }
+};
+struct bf16 {
+  typedef bfloat_t storage;
+  typedef float compute;
+  static AKG_DEV compute rnd(compute x) { return static_cast<float>(static_cast<bfloat_t>(x)); }
+  static AKG_DEV compute load(storage s) { return static_cast<float>(s); }
+  static AKG_DEV storage store(compute x) { return static_cast<bfloat_t>(x); }
+};
+struct i8 {
+  typedef s8 storage;
+  typedef int compute;
+  static AKG_DEV compute rnd(compute x) { return static_cast<int>(static_cast<s8>(x)); }
+  static AKG_DEV compute load(storage s) { return static_cast<int>(s); }
+  static AKG_DEV storage store(compute x) { return static_cast<s8>(x); }
+};
+struct i16 {
+  typedef short storage;
+  typedef int compute;
+  static AKG_DEV compute rnd(compute x) { return static_cast<int>(static_cast<short>(x)); }
+  static AKG_DEV compute load(storage s) { return static_cast<int>(s); }
+  static AKG_DEV storage store(compute x) { return static_cast<short>(x); }
+};
+struct i32 {
+  typedef int storage;
+  typedef int compute;
+  static AKG_DEV compute rnd(compute x) { return x; }
+  static AKG_DEV compute load(storage s) { return s; }
+  static AKG_DEV storage store(compute x) { return x; }
+};
+struct i64 {
+  typedef long long storage;
+  typedef long long compute;
+  static AKG_DEV compute rnd(compute x) { return x; }
+  static AKG_DEV compute load(storage s) { return s; }
+  static AKG_DEV storage store(compute x) { return x; }
+};
+// i1 tensors live in memory as one byte per element (0 or 1).
+struct b1 {
+  typedef u8 storage;
+  typedef bool compute;
+  static AKG_DEV compute rnd(compute x) { return x; }
+  static AKG_DEV compute load(storage s) { return s != 0; }
+  static AKG_DEV storage store(compute x) { return x ? 1 : 0; }
+};
+
+template <typename T>
+struct is_float_compute {
+  static constexpr bool value = false;
+};
+template <>
+struct is_float_compute<float> {
+  static constexpr bool value = true;
+};
+template <>
+struct is_float_compute<double> {
+  static constexpr bool value = true;
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// Vector memory access. A chunk of V consecutive elements is moved with the widest instructions the
+// alignment allows (the lowering only picks V such that every chunk start is V-element aligned).
+// ---------------------------------------------------------------------------------------------------------
+template <typename S, int V>
+struct alignas(sizeof(S) * V <= 16 ? sizeof(S) * V : 16) Pack {
+  S v[V];
+};
+
+template <typename DT, int V>
+AKG_DEV void load_chunk(const typename DT::storage *__restrict__ p, typename DT::compute (&dst)[V]) {
+  typedef Pack<typename DT::storage, V> P;
+  P raw = *reinterpret_cast<const P *>(p);
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(raw.v[e]);
+}
+
+template <typename DT, int V>
+AKG_DEV void store_chunk(typename DT::storage *__restrict__ p, const typename DT::compute (&src)[V]) {
+  typedef Pack<typename DT::storage, V> P;
+  P raw;
+#pragma unroll
+  for (int e = 0; e < V; ++e) raw.v[e] = DT::store(src[e]);
+  *reinterpret_cast<P *>(p) = raw;
+}
+
+template <typename DT, int V>
+AKG_DEV void fill_chunk(typename DT::compute (&dst)[V], typename DT::compute x) {
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = x;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Scalar op semantics. Overloaded on the compute type; names follow the op vocabulary.
+// Float ops are plain IEEE single operations (the build disables contraction), division and square root are
+// correctly rounded, transcendental functions are the device math library's.
+// ---------------------------------------------------------------------------------------------------------
+AKG_DEV float op_add(float a, float b) { return a + b; }
+AKG_DEV double op_add(double a, double b) { return a + b; }
+AKG_DEV int op_add(int a, int b) { return static_cast<int>(static_cast<u32>(a) + static_cast<u32>(b)); }
+AKG_DEV long long op_add(long long a, long long b) { return static_cast<long long>(static_cast<u64>(a) + static_cast<u64>(b)); }
+
+AKG_DEV float op_sub(float a, float b) { return a - b; }
+AKG_DEV double op_sub(double a, double b) { return a - b; }
+AKG_DEV int op_sub(int a, int b) { return static_cast<int>(static_cast<u32>(a) - static_cast<u32>(b)); }
+AKG_DEV long long op_sub(long long a, long long b) { return static_cast<long long>(static_cast<u64>(a) - static_cast<u64>(b)); }
+
+AKG_DEV float op_mul(float a, float b) { return a * b; }
+AKG_DEV double op_mul(double a, double b) { return a * b; }
+AKG_DEV int op_mul(int a, int b) { return static_cast<int>(static_cast<u32>(a) * static_cast<u32>(b)); }
+AKG_DEV long long op_mul(long long a, long long b) { return static_cast<long long>(static_cast<u64>(a) * static_cast<u64>(b)); }
+
+AKG_DEV float op_div(float a, float b) { return a / b; }
+AKG_DEV double op_div(double a, double b) { return a / b; }
+// arith.divsi; a zero divisor is undefined there and yields 0 here.
+AKG_DEV int op_div(int a, int b) { return b == 0 ? 0 : ((a == (-2147483647 - 1) && b == -1) ? a : a / b); }
+AKG_DEV long long op_div(long long a, long long b) { return b == 0 ? 0 : ((b == -1) ? static_cast<long long>(0ull - static_cast<u64>(a)) : a / b); }
+
+AKG_DEV float op_neg(float a) { return -a; }
+AKG_DEV double op_neg(double a) { return -a; }
+AKG_DEV int op_neg(int a) { return static_cast<int>(0u - static_cast<u32>(a)); }
+AKG_DEV long long op_neg(long long a) { return static_cast<long long>(0ull - static_cast<u64>(a)); }
+
+AKG_DEV float op_abs(float a) { return __builtin_fabsf(a); }
+AKG_DEV double op_abs(double a) { return __builtin_fabs(a); }
+AKG_DEV int op_abs(int a) { return a < 0 ? op_neg(a) : a; }
+AKG_DEV long long op_abs(long long a) { return a < 0 ? op_neg(a) : a; }
+
+// arith.maximumf / arith.minimumf: NaN-propagating.
+AKG_DEV float op_maximum(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmaxf(a, b)); }
+AKG_DEV double op_maximum(double a, double b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmax(a, b)); }
+AKG_DEV int op_maximum(int a, int b) { return a > b ? a : b; }
+AKG_DEV long long op_maximum(long long a, long long b) { return a > b ? a : b; }
+AKG_DEV float op_minimum(float a, float b) { return (a != a) ? a : ((b != b) ? b : __builtin_fminf(a, b)); }
+AKG_DEV double op_minimum(double a, double b) { return (a != a) ? a : ((b != b) ? b : __builtin_fmin(a, b)); }
+AKG_DEV int op_minimum(int a, int b) { return a < b ? a : b; }
+AKG_DEV long long op_minimum(long long a, long long b) { return a < b ? a : b; }
+
+AKG_DEV float op_exp(float a) { return expf(a); }
+AKG_DEV double op_exp(double a) { return exp(a); }
+AKG_DEV float op_log(float a) { return logf(a); }
+AKG_DEV double op_log(double a) { return log(a); }
+AKG_DEV float op_tanh(float a) { return tanhf(a); }
+AKG_DEV double op_tanh(double a) { return tanh(a); }
+AKG_DEV float op_sqrt(float a) { return __builtin_sqrtf(a); }
+AKG_DEV double op_sqrt(double a) { return __builtin_sqrt(a); }
+// math.rsqrt reaches the CPU as 1 / sqrt(x): two correctly rounded operations.
+AKG_DEV float op_rsqrt(float a) { return 1.0f / __builtin_sqrtf(a); }
+AKG_DEV double op_rsqrt(double a) { return 1.0 / __builtin_sqrt(a); }
+AKG_DEV float op_inv(float a) { return 1.0f / a; }
+AKG_DEV double op_inv(double a) { return 1.0 / a; }
+AKG_DEV float op_floor(float a) { return __builtin_floorf(a); }
+AKG_DEV double op_floor(double a) { return __builtin_floor(a); }
+AKG_DEV float op_sin(float a) { return sinf(a); }
+AKG_DEV double op_sin(double a) { return sin(a); }
+AKG_DEV float op_cos(float a) { return cosf(a); }
+AKG_DEV double op_cos(double a) { return cos(a); }
+AKG_DEV float op_asin(float a) { return asinf(a); }
+AKG_DEV double op_asin(double a) { return asin(a); }
+AKG_DEV float op_acos(float a) { return acosf(a); }
+AKG_DEV double op_acos(double a) { return acos(a); }
+AKG_DEV float op_atan(float a) { return atanf(a); }
+AKG_DEV double op_atan(double a) { return atan(a); }
+AKG_DEV float op_asinh(float a) { return asinhf(a); }
+AKG_DEV double op_asinh(double a) { return asinh(a); }
+AKG_DEV float op_acosh(float a) { return acoshf(a); }
+AKG_DEV double op_acosh(double a) { return acosh(a); }
+AKG_DEV float op_pow(float a, float b) { return powf(a, b); }
+AKG_DEV double op_pow(double a, double b) { return pow(a, b); }
+AKG_DEV float op_atan2(float a, float b) { return atan2f(a, b); }
+AKG_DEV double op_atan2(double a, double b) { return atan2(a, b); }
+
+AKG_DEV bool op_isnan(float a) { return a != a; }
+AKG_DEV bool op_isnan(double a) { return a != a; }
+AKG_DEV bool op_isinf(float a) { return __builtin_fabsf(a) == __builtin_inff(); }
+AKG_DEV bool op_isinf(double a) { return __builtin_fabs(a) == __builtin_inf(); }
+AKG_DEV bool op_isfinite(float a) { return __builtin_fabsf(a) < __builtin_inff(); }
+AKG_DEV bool op_isfinite(double a) { return __builtin_fabs(a) < __builtin_inf(); }
+
+// Reduction combiners (arith.addf / maxnumf / minnumf / mulf and their integer twins).
+struct RedSum {
+  template <typename T>
+  static AKG_DEV T apply(T a, T b) { return op_add(a, b); }
+};
+struct RedProd {
+  template <typename T>
+  static AKG_DEV T apply(T a, T b) { return op_mul(a, b); }
+};
+struct RedMax {
+  static AKG_DEV float apply(float a, float b) { return __builtin_fmaxf(a, b); }
+  static AKG_DEV double apply(double a, double b) { return __builtin_fmax(a, b); }
+  static AKG_DEV int apply(int a, int b) { return a > b ? a : b; }
+  static AKG_DEV long long apply(long long a, long long b) { return a > b ? a : b; }
+};
+struct RedMin {
+  static AKG_DEV float apply(float a, float b) { return __builtin_fminf(a, b); }
+  static AKG_DEV double apply(double a, double b) { return __builtin_fmin(a, b); }
+  static AKG_DEV int apply(int a, int b) { return a < b ? a : b; }
+  static AKG_DEV long long apply(long long a, long long b) { return a < b ? a : b; }
+};
+struct RedAll {
+  static AKG_DEV bool apply(bool a, bool b) { return a && b; }
+};
+struct RedAny {
+  static AKG_DEV bool apply(bool a, bool b) { return a || b; }
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// Cast (tosa.cast): float->float rounds to nearest even; float->int rounds to nearest even, saturates to the
+// destination range, then converts; float->bool is `!= 0`; int->float converts exactly or to nearest even;
+// int->narrower int saturates; int->bool is `!= 0`.
+// ---------------------------------------------------------------------------------------------------------
+template <typename DST>
+struct IntRange;
+template <>
+struct IntRange<i8> {
+  static constexpr long long lo = -128, hi = 127;
+};
+template <>
+struct IntRange<i16> {
+  static constexpr long long lo = -32768, hi = 32767;
+};
+template <>
+struct IntRange<i32> {
+  static constexpr long long lo = -2147483648LL, hi = 2147483647LL;
+};
+template <>
+struct IntRange<i64> {
+  static constexpr long long lo = (-9223372036854775807LL - 1), hi = 9223372036854775807LL;
+};
+
+template <typename DST, typename SRC>
+struct Caster {
+  // float -> float, int -> float (compute types are convertible; rnd applies the destination precision)
+  static AKG_DEV typename DST::compute run(typename SRC::compute x) {
+    return DST::rnd(static_cast<typename DST::compute>(x));
+  }
+};
+
+// math.roundeven
+AKG_DEV float round_even(float x) { return __builtin_rintf(x); }
+AKG_DEV double round_even(double x) { return __builtin_rint(x); }
+
+template <typename DST, typename SRCC, bool SrcIsFloat>
+struct ToInt;
+template <typename DST, typename SRCC>
+struct ToInt<DST, SRCC, true> {
+  static AKG_DEV typename DST::compute run(SRCC x) {
+    SRCC r = round_even(x);
+    const SRCC lo = static_cast<SRCC>(IntRange<DST>::lo);
+    const SRCC hi = static_cast<SRCC>(IntRange<DST>::hi);
+    if (r != r) return 0;
+    if (r <= lo) return static_cast<typename DST::compute>(IntRange<DST>::lo);
+    if (r >= hi) return static_cast<typename DST::compute>(IntRange<DST>::hi);
+    return static_cast<typename DST::compute>(r);
+  }
+};
+template <typename DST, typename SRCC>
+struct ToInt<DST, SRCC, false> {
+  static AKG_DEV typename DST::compute run(SRCC x) {
+    long long v = static_cast<long long>(x);
+    if (v < IntRange<DST>::lo) v = IntRange<DST>::lo;
+    if (v > IntRange<DST>::hi) v = IntRange<DST>::hi;
+    return static_cast<typename DST::compute>(v);
+  }
+};
+
+#define AKG_CAST_TO_INT(DSTT)                                                                              \
+  template <typename SRC>                                                                                  \
+  struct Caster<DSTT, SRC> {                                                                               \
+    static AKG_DEV typename DSTT::compute run(typename SRC::compute x) {                                   \
+      return ToInt<DSTT, typename SRC::compute, is_float_compute<typename SRC::compute>::value>::run(x);   \
+    }                                                                                                      \
+  };
+AKG_CAST_TO_INT(i8)
+AKG_CAST_TO_INT(i16)
+AKG_CAST_TO_INT(i32)
+AKG_CAST_TO_INT(i64)
+#undef AKG_CAST_TO_INT
+
+template <typename SRC>
+struct Caster<b1, SRC> {
+  static AKG_DEV bool run(typename SRC::compute x) { return x != static_cast<typename SRC::compute>(0); }
+};
+// bool sources: 0 / 1 (uitofp / zext)
+template <typename DST>
+struct FromBool {
+  static AKG_DEV typename DST::compute run(bool x) {
+    return x ? static_cast<typename DST::compute>(1) : static_cast<typename DST::compute>(0);
+  }
+};
+template <>
+struct Caster<f32, b1> : FromBool<f32> {};
+template <>
+struct Caster<f64, b1> : FromBool<f64> {};
+template <>
+struct Caster<f16, b1> : FromBool<f16> {};
+template <>
+struct Caster<bf16, b1> : FromBool<bf16> {};
+template <>
+struct Caster<i8, b1> : FromBool<i8> {};
+template <>
+struct Caster<i16, b1> : FromBool<i16> {};
+template <>
+struct Caster<i32, b1> : FromBool<i32> {};
+template <>
+struct Caster<i64, b1> : FromBool<i64> {};
+template <>
+struct Caster<b1, b1> {
+  static AKG_DEV bool run(bool x) { return x; }
+};
+
+template <typename DST, typename SRC>
+AKG_DEV typename DST::compute cast(typename SRC::compute x) {
+  return Caster<DST, SRC>::run(x);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Cross-lane reductions. A row is owned by a group of TPR threads (TPR a power of two). Up to one wavefront
+// the reduction is an xor butterfly: every lane ends with the same bits because each step combines the same
+// two partial results in both partners. The two innermost steps are DPP quad permutes; the rest go through
+// the LDS crossbar (ds_bpermute), which touches no LDS memory. Groups wider than a wavefront finish through
+// a small LDS array; every thread then folds the per-wavefront partials in the same fixed order.
+// ---------------------------------------------------------------------------------------------------------
+AKG_DEV int lane_xor_bits(int v, int mask) {
+  if (mask == 1) return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  if (mask == 2) return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  const int lane = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+  return __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, v);
+}
+
+AKG_DEV float lane_xor(float v, int mask) {
+  return __builtin_bit_cast(float, lane_xor_bits(__builtin_bit_cast(int, v), mask));
+}
+AKG_DEV int lane_xor(int v, int mask) { return lane_xor_bits(v, mask); }
+AKG_DEV bool lane_xor(bool v, int mask) { return lane_xor_bits(v ? 1 : 0, mask) != 0; }
+AKG_DEV double lane_xor(double v, int mask) {
+  u64 b = __builtin_bit_cast(u64, v);
+  u32 lo = static_cast<u32>(lane_xor_bits(static_cast<int>(b & 0xffffffffu), mask));
+  u32 hi = static_cast<u32>(lane_xor_bits(static_cast<int>(b >> 32), mask));
+  return __builtin_bit_cast(double, (static_cast<u64>(hi) << 32) | lo);
+}
+AKG_DEV long long lane_xor(long long v, int mask) {
+  u64 b = static_cast<u64>(v);
+  u32 lo = static_cast<u32>(lane_xor_bits(static_cast<int>(b & 0xffffffffu), mask));
+  u32 hi = static_cast<u32>(lane_xor_bits(static_cast<int>(b >> 32), mask));
+  return static_cast<long long>((static_cast<u64>(hi) << 32) | lo);
+}
+
+template <typename Red, int WIDTH, typename T>
+AKG_DEV T wave_group_reduce(T v) {
+  static_assert(WIDTH <= kWaveSize && (WIDTH & (WIDTH - 1)) == 0, "group width must be a power of two <= 64");
+#pragma unroll
+  for (int m = 1; m < WIDTH; m <<= 1) v = Red::apply(v, lane_xor(v, m));
+  return v;
+}
+
+// Reduction over a group of TPR threads. `scratch` points at this reduction's LDS slots (one per wavefront of
+// the block); it is only touched when TPR > 64. The caller alternates between two scratch arrays from one
+// reduction to the next, which makes a single barrier per reduction sufficient.
+template <typename Red, int TPR, typename T>
+AKG_DEV T group_reduce(T v, T *scratch, int tid) {
+  if constexpr (TPR <= kWaveSize) {
+    return wave_group_reduce<Red, TPR>(v);
+  } else {
+    constexpr int kWavesPerGroup = TPR / kWaveSize;
+    v = wave_group_reduce<Red, kWaveSize>(v);
+    const int wave = tid / kWaveSize;
+    if ((tid % kWaveSize) == 0) scratch[wave] = v;
+    __syncthreads();
+    const int first = (wave / kWavesPerGroup) * kWavesPerGroup;
+    T r = scratch[first];
+#pragma unroll
+    for (int w = 1; w < kWavesPerGroup; ++w) r = Red::apply(r, scratch[first + w]);
+    return r;
+  }
+}
+
+}  // namespace akg

@@ -1,0 +1,48 @@
+#!/usr/bin/env python3
+"""Regenerate the op descriptions (*.info) of this directory.
+
+`c1`..`c5` are the five fused-operator configurations the backend is measured on; the `small_*` files are the same
+patterns at sizes a scalar CPU run finishes instantly, plus ragged shapes that exercise tail handling.
+Run from the repository root: python akg_amd/fixtures/make_fixtures.py
+"""
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+from akg_amd import op_desc  # noqa: E402
+
+FIXTURES = {
+    # measured configurations
+    "c1_ew_tanh_add_mul_f32_1024x4096": lambda n: op_desc.elementwise_tanh_add_mul(1024, 4096, n),
+    "c2_softmax_f16_8192x4096": lambda n: op_desc.softmax_last_axis(8192, 4096, "float16", n),
+    "c3_layernorm_residual_bf16_16384x4096": lambda n: op_desc.layernorm_residual(16384, 4096, "bfloat16", 1e-5, n),
+    "c4_quant_int8_residual_bf16_32768x8192": lambda n: op_desc.quant_int8_residual(32768, 8192, "bfloat16", n),
+    "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": lambda n: op_desc.gemm_int8_dequant_bias_gelu(4096, 8192, 8192, "bfloat16", False, n),
+    # small parity cases
+    "small_ew_tanh_add_mul_f32_8x128": lambda n: op_desc.elementwise_tanh_add_mul(8, 128, n),
+    "small_ew_tanh_add_mul_f32_7x33": lambda n: op_desc.elementwise_tanh_add_mul(7, 33, n),
+    "small_softmax_f16_64x4096": lambda n: op_desc.softmax_last_axis(64, 4096, "float16", n),
+    "small_softmax_f16_33x1000": lambda n: op_desc.softmax_last_axis(33, 1000, "float16", n),
+    "small_softmax_f32_5x77": lambda n: op_desc.softmax_last_axis(5, 77, "float32", n),
+    "small_layernorm_residual_bf16_64x4096": lambda n: op_desc.layernorm_residual(64, 4096, "bfloat16", 1e-5, n),
+    "small_layernorm_residual_bf16_19x520": lambda n: op_desc.layernorm_residual(19, 520, "bfloat16", 1e-5, n),
+    "small_quant_int8_residual_bf16_64x8192": lambda n: op_desc.quant_int8_residual(64, 8192, "bfloat16", n),
+    "small_quant_int8_residual_bf16_37x1544": lambda n: op_desc.quant_int8_residual(37, 1544, "bfloat16", n),
+    "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),
+    "small_gemm_i8_dequant_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", True, n),
+}
+
+
+def main():
+    for name, make in FIXTURES.items():
+        path = os.path.join(HERE, name + ".info")
+        with open(path, "w", encoding="utf-8") as f:
+            f.write(make(name))
+            f.write("\n")
+        print("wrote", os.path.relpath(path))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,226 @@
+"""Author MindSpore graph-kernel op descriptions (`.info` JSON) programmatically.
+
+The document layout is the one the reference's translator reads
+(akg-mlir/lib/Target/MindsporeDialect/TranslateToMindsporeDialect.cpp:55-75,295-415): top-level `op`, `process`,
+`input_desc` (a list of single-element lists), `op_desc` (each with `name`, `attr`, `input_desc`, `output_desc`)
+and `output_desc`. Scalar constants are op inputs of shape [1] that carry a numeric `value` (:650-658).
+Only op names of the reference's op table (:417-486) are emitted.
+"""
+import json
+import re
+
+_IDENT = re.compile(r"^[A-Za-z_][A-Za-z0-9_]*$")
+
+
+class Tensor:
+    def __init__(self, name, shape, dtype, value=None):
+        self.name = name
+        self.shape = list(shape)
+        self.dtype = dtype
+        self.value = value
+
+    def desc(self, with_value=True):
+        d = {"data_type": self.dtype, "format": "DefaultFormat", "shape": list(self.shape), "tensor_name": self.name}
+        if with_value and self.value is not None:
+            d["value"] = self.value
+        return d
+
+
+class DescBuilder:
+    """Builds one fused-op description; tensors are created through `input`, `const` and the op methods."""
+
+    def __init__(self, name, process="hip", arch="gfx950"):
+        if not _IDENT.match(name):
+            raise ValueError("op name must be a C identifier: %r" % name)
+        self.name = name
+        self.process = process
+        self.arch = arch
+        self.inputs = []
+        self.ops = []
+        self._n_const = 0
+        self._n_out = 0
+
+    # -- tensors ---------------------------------------------------------------------------------------
+    def input(self, shape, dtype):
+        t = Tensor("input_%d" % len(self.inputs), shape, dtype)
+        self.inputs.append(t)
+        return t
+
+    def const(self, value, dtype):
+        self._n_const += 1
+        return Tensor("const_%d" % self._n_const, [1], dtype, value=value)
+
+    # -- generic op ------------------------------------------------------------------------------------
+    def op(self, name, inputs, shape, dtype, attrs=None):
+        out = Tensor("output_0_%d" % self._n_out, shape, dtype)
+        self._n_out += 1
+        self.ops.append({
+            "attr": attrs,
+            "impl_path": "",
+            "input_desc": [[t.desc()] for t in inputs],
+            "name": name,
+            "output_desc": [out.desc(with_value=False)],
+        })
+        return out
+
+    # -- shape helpers ---------------------------------------------------------------------------------
+    @staticmethod
+    def _broadcast(a, b):
+        ra, rb = list(a)[::-1], list(b)[::-1]
+        out = []
+        for i in range(max(len(ra), len(rb))):
+            da = ra[i] if i < len(ra) else 1
+            db = rb[i] if i < len(rb) else 1
+            if da != db and da != 1 and db != 1:
+                raise ValueError("shapes %s and %s do not broadcast" % (a, b))
+            out.append(max(da, db))
+        return out[::-1]
+
+    # -- op vocabulary used by the fused patterns ----------------------------------------------------------
+    def unary(self, name, x, dtype=None):
+        return self.op(name, [x], x.shape, dtype or x.dtype)
+
+    def binary(self, name, a, b, dtype=None):
+        return self.op(name, [a, b], self._broadcast(a.shape, b.shape), dtype or (a.dtype if a.value is None else b.dtype))
+
+    def add(self, a, b):
+        return self.binary("Add", a, b)
+
+    def sub(self, a, b):
+        return self.binary("Sub", a, b)
+
+    def mul(self, a, b):
+        return self.binary("Mul", a, b)
+
+    def div(self, a, b):
+        return self.binary("RealDiv", a, b)
+
+    def maximum(self, a, b):
+        return self.binary("Maximum", a, b)
+
+    def minimum(self, a, b):
+        return self.binary("Minimum", a, b)
+
+    def cast(self, x, dtype):
+        return self.op("Cast", [x], x.shape, dtype, attrs=[{"data_type": "str", "name": "dst_type", "value": dtype}])
+
+    def reduce(self, name, x, axis, keep_dims):
+        axes = [a % len(x.shape) for a in axis]
+        shape = [1 if i in axes else d for i, d in enumerate(x.shape)] if keep_dims else \
+                [d for i, d in enumerate(x.shape) if i not in axes]
+        if not shape:
+            shape = [1]
+        attrs = [{"data_type": "listInt", "name": "axis", "value": list(axis)},
+                 {"data_type": "bool", "name": "keep_dims", "value": bool(keep_dims)}]
+        return self.op(name, [x], shape, x.dtype, attrs=attrs)
+
+    def reshape(self, x, shape):
+        return self.op("Reshape", [x], shape, x.dtype, attrs=[{"data_type": "listInt", "name": "shape", "value": list(shape)}])
+
+    def matmul(self, a, b, dtype, transpose_b=False):
+        m, k = a.shape
+        n = b.shape[0] if transpose_b else b.shape[1]
+        attrs = [{"data_type": "bool", "name": "transpose_a", "value": False},
+                 {"data_type": "bool", "name": "transpose_b", "value": bool(transpose_b)}]
+        return self.op("MatMul", [a, b], [m, n], dtype, attrs=attrs)
+
+    # -- document --------------------------------------------------------------------------------------
+    def build(self, outputs):
+        return {
+            "composite": True,
+            "composite_graph": "akg_amd",
+            "id": 0,
+            "input_desc": [[t.desc()] for t in self.inputs],
+            "op": self.name,
+            "op_desc": self.ops,
+            "output_desc": [t.desc(with_value=False) for t in outputs],
+            "platform": "AKG",
+            "process": self.process,
+            "target_info": {"arch": self.arch},
+            "version": 2,
+        }
+
+    def dumps(self, outputs):
+        return json.dumps(self.build(outputs), indent=1, sort_keys=True)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# The five fused patterns, parameterised by shape.
+# ---------------------------------------------------------------------------------------------------------
+def elementwise_tanh_add_mul(rows, cols, name=None):
+    """out = tanh((a + b) * c), float32."""
+    b = DescBuilder(name or "Fused_Add_Mul_Tanh_f32_%dx%d" % (rows, cols))
+    x, y, z = (b.input([rows, cols], "float32") for _ in range(3))
+    out = b.unary("Tanh", b.mul(b.add(x, y), z))
+    return b.dumps([out])
+
+
+def softmax_last_axis(rows, cols, dtype="float16", name=None):
+    """Softmax over the last axis; internals in float32 behind explicit casts, as MindSpore emits them."""
+    b = DescBuilder(name or "Fused_Cast_ReduceMax_Sub_Exp_ReduceSum_RealDiv_Cast_softmax_%s_%dx%d" % (
+        {"float16": "f16", "bfloat16": "bf16", "float32": "f32"}[dtype], rows, cols))
+    x = b.input([rows, cols], dtype)
+    xf = b.cast(x, "float32") if dtype != "float32" else x
+    mx = b.reduce("ReduceMax", xf, [1], True)
+    e = b.unary("Exp", b.sub(xf, mx))
+    s = b.reduce("ReduceSum", e, [1], True)
+    p = b.div(e, s)
+    out = b.cast(p, dtype) if dtype != "float32" else p
+    return b.dumps([out])
+
+
+def layernorm_residual(rows, cols, dtype="bfloat16", eps=1e-5, name=None):
+    """out = LayerNorm(x) * gamma + beta + r over the last axis, float32 internals."""
+    b = DescBuilder(name or "Fused_LayerNorm_Residual_%s_%dx%d" % (
+        {"float16": "f16", "bfloat16": "bf16", "float32": "f32"}[dtype], rows, cols))
+    x = b.input([rows, cols], dtype)
+    gamma = b.input([cols], dtype)
+    beta = b.input([cols], dtype)
+    r = b.input([rows, cols], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    xf, gf, bf, rf = f(x), f(gamma), f(beta), f(r)
+    inv_n = b.const(1.0 / cols, "float32")
+    mean = b.mul(b.reduce("ReduceSum", xf, [1], True), inv_n)
+    xc = b.sub(xf, mean)
+    var = b.mul(b.reduce("ReduceSum", b.mul(xc, xc), [1], True), inv_n)
+    rstd = b.unary("Rsqrt", b.add(var, b.const(eps, "float32")))
+    y = b.add(b.add(b.mul(b.mul(xc, rstd), gf), bf), rf)
+    out = b.cast(y, dtype) if dtype != "float32" else y
+    return b.dumps([out])
+
+
+def quant_int8_residual(rows, cols, dtype="bfloat16", name=None):
+    """Per-token symmetric int8 quantisation of s = x + r: scale = absmax(s) / 127 per row,
+    q = cast_int8(clamp(s / scale, -127, 127)) with the cast rounding half to even. Outputs: q, scale."""
+    b = DescBuilder(name or "Fused_Add_Abs_ReduceMax_RealDiv_Cast_quant_%s_%dx%d" % (
+        {"float16": "f16", "bfloat16": "bf16", "float32": "f32"}[dtype], rows, cols))
+    x = b.input([rows, cols], dtype)
+    r = b.input([rows, cols], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    s = b.add(f(x), f(r))
+    amax = b.reduce("ReduceMax", b.unary("Abs", s), [1], False)
+    scale = b.div(amax, b.const(127.0, "float32"))
+    q = b.div(s, b.reshape(scale, [rows, 1]))
+    q = b.minimum(b.maximum(q, b.const(-127.0, "float32")), b.const(127.0, "float32"))
+    q8 = b.cast(q, "int8")
+    return b.dumps([q8, scale])
+
+
+def gemm_int8_dequant_bias_gelu(m, k, n, out_dtype="bfloat16", transpose_b=False, name=None):
+    """out = GELU_tanh(dequant(A @ B) + bias): int8 x int8 -> int32, times per-row and per-column float32 scales,
+    plus bias, GELU spelled with Mul/Add/Tanh (no Erf/Gelu in the op table)."""
+    b = DescBuilder(name or "Fused_MatMul_Cast_Mul_Mul_Add_GeluTanh_Cast_i8_%dx%dx%d%s" % (
+        m, k, n, "_tb" if transpose_b else ""))
+    a = b.input([m, k], "int8")
+    sa = b.input([m, 1], "float32")
+    w = b.input([n, k] if transpose_b else [k, n], "int8")
+    sb = b.input([n], "float32")
+    bias = b.input([n], out_dtype)
+    acc = b.matmul(a, w, "int32", transpose_b=transpose_b)
+    x = b.mul(b.mul(b.cast(acc, "float32"), sa), sb)
+    x = b.add(x, b.cast(bias, "float32") if out_dtype != "float32" else bias)
+    x3 = b.mul(b.mul(x, x), x)
+    inner = b.mul(b.add(x, b.mul(x3, b.const(0.044715, "float32"))), b.const(0.7978845608028654, "float32"))
+    g = b.mul(b.mul(x, b.add(b.unary("Tanh", inner), b.const(1.0, "float32"))), b.const(0.5, "float32"))
+    out = b.cast(g, out_dtype) if out_dtype != "float32" else g
+    return b.dumps([out])

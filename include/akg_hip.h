@@ -1,0 +1,144 @@
+/**
+ * akg_hip.h - C ABI of the MI355X (gfx950) backend for AKG-MLIR fused operators.
+ *
+ * Drop-in boundary: a MindSpore graph-kernel JSON op description goes in, a callable kernel with the same
+ * tensor signature (inputs in `input_desc` order, then outputs in `output_desc` order) comes out.
+ * Plain C types only; every function returns 0 on success or a negative akg_hip_status code and never
+ * terminates the process (the reference's tools exit non-zero and its launch shim calls exit(1),
+ * akg-mlir/python/akg_mlir/utils/code_template.py:47-56).
+ *
+ * Each entry point names the reference interface it replaces.
+ */
+#ifndef AKG_HIP_H_
+#define AKG_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum akg_hip_status {
+  AKG_HIP_OK = 0,
+  AKG_HIP_ERR_INVALID_ARGUMENT = -1,
+  AKG_HIP_ERR_JSON = -2,          /* malformed JSON text */
+  AKG_HIP_ERR_TRANSLATE = -3,     /* well-formed JSON that is not a valid op description */
+  AKG_HIP_ERR_UNSUPPORTED = -4,   /* valid description with no gfx950 kernel family (or an unknown op) */
+  AKG_HIP_ERR_COMPILE = -5,       /* device compilation failed */
+  AKG_HIP_ERR_IO = -6,            /* artifact directory / file access */
+  AKG_HIP_ERR_RUNTIME = -7,       /* HIP runtime error (no device, launch failure, out of memory) */
+  AKG_HIP_ERR_INTERNAL = -8
+} akg_hip_status;
+
+/* Element types of the op-description format (TranslateToMindsporeDialect.cpp:488-502). */
+typedef enum akg_hip_dtype {
+  AKG_HIP_BOOL = 0,
+  AKG_HIP_INT8 = 1,
+  AKG_HIP_INT16 = 2,
+  AKG_HIP_INT32 = 3,
+  AKG_HIP_INT64 = 4,
+  AKG_HIP_FLOAT16 = 5,
+  AKG_HIP_BFLOAT16 = 6,
+  AKG_HIP_FLOAT32 = 7,
+  AKG_HIP_FLOAT64 = 8
+} akg_hip_dtype;
+
+#define AKG_HIP_MAX_RANK 8
+
+typedef struct akg_hip_tensor_desc {
+  int32_t dtype;                      /* akg_hip_dtype */
+  int32_t rank;
+  int64_t shape[AKG_HIP_MAX_RANK];
+  int64_t bytes;                      /* dense row-major size */
+  int32_t is_output;                  /* 0: kernel input, 1: kernel output */
+  char name[64];                      /* tensor_name of the description */
+} akg_hip_tensor_desc;
+
+typedef struct akg_hip_kernel_info {
+  char kernel_name[256];              /* "<op>_kernel" (KernelOutliningExt.cpp:433) */
+  char family[32];                    /* "elementwise" | "row_reduce" | "gemm_epilogue" */
+  char operator_type[32];             /* fusion class, OperatorIdentify.cpp:51-93 */
+  uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json */
+  uint32_t block[3];                  /* threadIdx.x/y/z extents */
+  uint64_t algorithmic_bytes;         /* bytes of every input and output, each counted once */
+  uint64_t algorithmic_ops;           /* 2*M*N*K of the contraction, 0 for bandwidth-bound families */
+  int32_t cache_hit;                  /* 1 if the code object came from the artifact directory */
+} akg_hip_kernel_info;
+
+typedef struct akg_hip_kernel akg_hip_kernel_t;
+
+/**
+ * Compile one op description to a gfx950 code object and return a kernel handle. Needs no GPU.
+ * Replaces the compile half of MlirDriver.compile_gpu (akg-mlir/python/akg_mlir/mlir_driver.py:337-374):
+ * mindspore-translate -json-to-mindspore (TranslateToMindsporeDialect.cpp:1461) -> akg-opt --gpu-opt
+ * (GPUOpt.cpp:45-132) -> akg-opt --gpu-codegen (GPUCodegen.cpp:34-55) -> akg-translate -gen-ptx
+ * (TranslateToPTX.cpp:67-103).
+ * If out_dir is non-NULL the reference's artifact set is written there: <op>.hsaco (in place of <op>.ptx),
+ * <op>.json {blockIdx.*, threadIdx.*, kernelName, is_dynamic, sha256} (GPUMapping.cpp:645-665,
+ * mlir_driver.py:776-815), <op>_shape_arg.txt (KernelOutliningExt.cpp:384-423), <op>.hip (the emitted
+ * source, the counterpart of the <op>_gpu.mlir dump); a matching artifact found there is reused instead
+ * of compiling (the reference's KERNEL_META_DIR cache, mlir_driver.py:47-53).
+ */
+int akg_hip_compile(const char *json_text, size_t json_len, const char *out_dir, akg_hip_kernel_t **out_kernel);
+
+/** Same, reading the description from a file (the `-f x.info` of akg_benchmark, benchmark.py:249-328).
+ *  Paths containing ".." are rejected as in checkAndReadJson (akg/Utils/IOHelper.hpp:44-61). */
+int akg_hip_compile_file(const char *info_path, const char *out_dir, akg_hip_kernel_t **out_kernel);
+
+/** Number of kernel arguments (inputs + outputs). Replaces reading `input_desc`/`output_desc` on the Python
+ *  side (composite_op_helper.py:833-902). */
+int akg_hip_kernel_num_tensors(const akg_hip_kernel_t *kernel, int *n_tensors);
+
+/** Descriptor of argument `index` (inputs first, then outputs: BufferResultsToOutParams, GPUOpt.cpp:78). */
+int akg_hip_kernel_tensor(const akg_hip_kernel_t *kernel, int index, akg_hip_tensor_desc *desc);
+
+/** Launch shape, family, algorithmic work. Replaces get_gpu_setting_by_input (dynamic_utils.py:564-577). */
+int akg_hip_kernel_get_info(const akg_hip_kernel_t *kernel, akg_hip_kernel_info *info);
+
+/** Emitted HIP source of the kernel (NUL-terminated, owned by the handle). */
+int akg_hip_kernel_source(const akg_hip_kernel_t *kernel, const char **source);
+
+/**
+ * The hot call: enqueue the kernel on `stream` (a hipStream_t, NULL for the default stream) with one DEVICE
+ * pointer per argument, inputs then outputs. Asynchronous; allocates nothing. Replaces the cuLaunchKernel
+ * step of the generated shim (code_template.py:204) without its per-call context creation, module load,
+ * cuMemAlloc and copies.
+ */
+int akg_hip_launch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream);
+
+/**
+ * Reference-style execution with HOST pointers: allocate device buffers, copy every tensor in (outputs
+ * too, as the reference does, gen_runtime_code.py:95-97), launch, copy the outputs back, free. Replaces
+ * `extern "C" cuda_runtime_exec(T0* data_0, ...)` (code_template.py:160-211) called from MlirDriver.run_gpu
+ * (mlir_driver.py:426-447).
+ */
+int akg_hip_run_host(akg_hip_kernel_t *kernel, void *const *host_ptrs, int n_ptrs);
+
+/**
+ * Time `repeat` batches of `number` back-to-back launches on device-resident buffers with HIP events and
+ * return the mean milliseconds per launch. Replaces `cuda_runtime_profiling(..., number, repeat,
+ * min_repeat_ms)` (code_template.py:68-155), which timed with std::chrono around a stream synchronize.
+ */
+int akg_hip_profile(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, int number, int repeat,
+                    double *avg_ms);
+
+/** Release the handle (and its loaded module, if any). */
+void akg_hip_kernel_destroy(akg_hip_kernel_t *kernel);
+
+/** Message of the last failure on the calling thread ("" if none). */
+const char *akg_hip_last_error(void);
+
+/** Translate only: render the typed op graph (the `mindspore-translate -json-to-mindspore` output,
+ *  TranslateRegistration.cpp:42-50) into a malloc'ed string the caller frees with akg_hip_free_string. */
+int akg_hip_translate(const char *json_text, size_t json_len, char **out_text);
+void akg_hip_free_string(char *text);
+
+/** Library version string. */
+const char *akg_hip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* AKG_HIP_H_ */
