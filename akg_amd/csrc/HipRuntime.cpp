@@ -234,9 +234,10 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
   if (!dir.empty()) {
     if (!makeDirs(dir)) return fail(AKG_HIP_ERR_IO, "cannot create artifact directory " + dir);
     base = dir + "/" + k->graph.name;
-    // cache probe
+    // cache probe (AKG_HIP_NO_CACHE=1 forces a fresh device compilation)
+    const char *noCache = std::getenv("AKG_HIP_NO_CACHE");
     std::string meta, code;
-    if (readFile(base + ".json", &meta) && readFile(base + ".hsaco", &code) && !code.empty()) {
+    if (!(noCache && noCache[0] == '1') && readFile(base + ".json", &meta) && readFile(base + ".hsaco", &code) && !code.empty()) {
       try {
         akg::json::Value mv = akg::json::Value::parse(meta);
         if (mv.contains("source_sha256") && mv.at("source_sha256").asString() == srcDigest &&

@@ -1,0 +1,336 @@
+"""TEST INFRASTRUCTURE - CPU oracle, part 2: op-by-op numpy restatement of the same semantics.
+
+This is the checker, not the product: only tests, the smoke check and the CPU-baseline leg of the benchmark may import
+it. It evaluates a MindSpore graph-kernel JSON description one op at a time with numpy, every op in its declared
+result element type, and is deliberately written independently of oracle/gen_cpu.py (different language, no fusion,
+vectorised) so that the two can be checked against each other.
+
+Rules restated (reference file:line):
+  * op vocabulary and reading rules of the description: TranslateToMindsporeDialect.cpp:295-415,417-486,793-808,1273-1360
+  * elementwise ops in the result type; Cast = tosa.cast: MindSporeToTosa.cpp:475-504
+  * reductions: init value and combiner, accumulation in the result type, increasing index order:
+    MindSporeToLinalg.cpp:791-901,1333-1451
+  * MatMul accumulates in the output type from zero: MindSporeToLinalg.cpp:1453-1546
+  * numpy spelling of the expected values in the reference harness: python/akg_mlir/utils/op_dsl.py:126-168,295-327,747-809
+    (two of its rules are NOT followed because they contradict the compiled pipeline: `astype` truncation for
+    float->int casts, and int8 products without widening)
+
+bfloat16 tensors are numpy uint16 arrays holding the bit patterns; internally they are float32 arrays whose values are
+bfloat16-representable.
+"""
+import json
+
+import numpy as np
+
+FLOATS = ("float16", "bfloat16", "float32", "float64")
+NP_DTYPE = {"bool": np.bool_, "int8": np.int8, "int16": np.int16, "int32": np.int32, "int64": np.int64,
+            "float16": np.float16, "bfloat16": np.float32, "float32": np.float32, "float64": np.float64}
+ATTR_AS_INPUT = ("Reshape", "BroadcastTo", "ReduceMax", "ReduceMin", "ReduceSum", "ReducePrd", "ReduceAll", "ReduceAny",
+                 "ArgMax", "Transpose", "Tile")
+LARGEST = {"float16": 65504.0, "bfloat16": 3.3895313892515355e38, "float32": 3.4028234663852886e38,
+           "float64": 1.7976931348623157e308}
+
+
+# ---------------------------------------------------------------------------------------------------------
+# bfloat16 <-> float32 (round to nearest even, arith.truncf)
+# ---------------------------------------------------------------------------------------------------------
+def bf16_bits_to_f32(bits):
+    bits = np.asarray(bits, dtype=np.uint16)
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16_bits(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    u = x.view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    rounded = (u.astype(np.uint64) + 0x7FFF + ((u >> 16) & 1)) >> 16
+    out = rounded.astype(np.uint16)
+    if np.any(nan):
+        out = np.where(nan, ((u >> 16) | 0x40).astype(np.uint16), out)
+    return out
+
+
+def round_to_bf16(x):
+    return bf16_bits_to_f32(f32_to_bf16_bits(x))
+
+
+def canon_dtype(name):
+    if name in ("uint8", "sint8"):
+        return "int8"
+    if name == "int1":
+        return "bool"
+    if name not in NP_DTYPE:
+        raise ValueError("data type %s is not supported" % name)
+    return name
+
+
+def to_internal(arr, dtype):
+    """External array (bf16 as uint16 bits) -> internal array."""
+    if dtype == "bfloat16":
+        return bf16_bits_to_f32(arr)
+    return np.asarray(arr, dtype=NP_DTYPE[dtype])
+
+
+def to_external(arr, dtype):
+    if dtype == "bfloat16":
+        return f32_to_bf16_bits(arr)
+    return np.ascontiguousarray(arr, dtype=NP_DTYPE[dtype])
+
+
+def finish(x, dtype):
+    """Round a freshly computed array to the declared result type."""
+    if dtype == "bfloat16":
+        return round_to_bf16(np.asarray(x, dtype=np.float32))
+    return np.asarray(x).astype(NP_DTYPE[dtype], copy=False)
+
+
+def compute_view(x, dtype):
+    """Array to do arithmetic on: float16 computes in float32 and is rounded once per op."""
+    if dtype == "float16":
+        return x.astype(np.float32)
+    return x
+
+
+def cast(x, src, dst):
+    """tosa.cast."""
+    if dst == "bool":
+        return x != 0
+    if dst in FLOATS:
+        if src == "bool":
+            x = x.astype(np.float32)
+        if dst == "bfloat16":
+            return round_to_bf16(x.astype(np.float32))
+        return x.astype(NP_DTYPE[dst])
+    info = np.iinfo(NP_DTYPE[dst])
+    if src in FLOATS:
+        r = np.rint(x.astype(np.float64))            # round half to even
+        r = np.where(np.isnan(r), 0.0, r)
+        r = np.clip(r, float(info.min), float(info.max))
+        if dst == "int64":
+            r = np.where(r >= 9.223372036854775807e18, np.nextafter(9.223372036854775807e18, 0), r)
+        return r.astype(NP_DTYPE[dst])
+    if src == "bool":
+        return x.astype(NP_DTYPE[dst])
+    return np.clip(x.astype(np.int64), info.min, info.max).astype(NP_DTYPE[dst])   # saturating narrowing
+
+
+def maximum_nan(a, b):
+    return np.maximum(a, b)   # numpy's maximum propagates NaN, like arith.maximumf
+
+
+def minimum_nan(a, b):
+    return np.minimum(a, b)
+
+
+def serial_reduce(x, axes, combine, init, dtype, keep_dims):
+    """Reduce `axes` of x visiting the reduced indices in increasing order, rounding to `dtype` after every step."""
+    rank = x.ndim
+    kept = [d for d in range(rank) if d not in axes]
+    xt = np.transpose(x, kept + list(axes))
+    kept_shape = [x.shape[d] for d in kept]
+    xt = xt.reshape(kept_shape + [-1])
+    acc = np.full(kept_shape, init, dtype=xt.dtype)
+    for k in range(xt.shape[-1]):
+        acc = finish(combine(compute_view(acc, dtype), compute_view(xt[..., k], dtype)), dtype)
+    if keep_dims:
+        acc = acc.reshape([1 if d in axes else x.shape[d] for d in range(rank)])
+    return acc
+
+
+def matmul_exact_i32(a, b):
+    """int8 x int8 -> int32 with exact accumulation: float32 BLAS on K-blocks small enough that every partial sum
+    is an integer below 2**24 (127*127*1024 < 2**24), summed in int64 and wrapped to int32."""
+    m, k = a.shape
+    n = b.shape[1]
+    acc = np.zeros((m, n), dtype=np.int64)
+    step = 1024
+    for k0 in range(0, k, step):
+        pa = a[:, k0:k0 + step].astype(np.float32)
+        pb = b[k0:k0 + step, :].astype(np.float32)
+        acc += (pa @ pb).astype(np.int64)
+    return acc.astype(np.int32)   # two's complement wrap, as i32 accumulation would
+
+
+def evaluate(desc, inputs):
+    """Evaluate the description on `inputs` (list of external arrays in input_desc order); returns the list of
+    external output arrays in output_desc order."""
+    if isinstance(desc, str):
+        desc = json.loads(desc)
+    env = {}
+    dtypes = {}
+    shapes = {}
+    if len(inputs) != len(desc["input_desc"]):
+        raise ValueError("expected %d inputs" % len(desc["input_desc"]))
+    for entry, arr in zip(desc["input_desc"], inputs):
+        d = entry[0]
+        dt = canon_dtype(d["data_type"])
+        shape = d.get("shape", [1])
+        env[d["tensor_name"]] = to_internal(arr, dt).reshape(shape)
+        dtypes[d["tensor_name"]] = dt
+    for od in desc["op_desc"]:
+        name = od["name"]
+        attrs = {a["name"]: a["value"] for a in (od.get("attr") or [])}
+        ins, in_dt = [], []
+        for idx, entry in enumerate(od["input_desc"]):
+            if idx == 1 and name in ATTR_AS_INPUT:
+                continue
+            if name == "Cast" and idx > 0:
+                continue
+            d = entry[0]
+            tn = d["tensor_name"]
+            if tn not in env:
+                v = d["value"]
+                dt = canon_dtype(d["data_type"])
+                if isinstance(v, list):
+                    v = v[0]
+                if dt not in FLOATS and dt != "bool":
+                    v = int(v)
+                c = np.array([v]).astype(np.float32 if dt == "bfloat16" else NP_DTYPE[dt])
+                env[tn] = finish(c, dt) if dt in FLOATS else c
+                dtypes[tn] = dt
+            ins.append(env[tn])
+            in_dt.append(dtypes[tn])
+        o = od["output_desc"][0]
+        odt = canon_dtype(o["data_type"])
+        oshape = o.get("shape", [1])
+        cv = [compute_view(x, dt) for x, dt in zip(ins, in_dt)]
+
+        def same(x, dt=odt):
+            # operands of arithmetic ops are converted to the result's compute type if they differ
+            target = np.float32 if dt in ("float16", "bfloat16") else NP_DTYPE[dt]
+            return x.astype(target, copy=False)
+
+        with np.errstate(all="ignore"):
+            if name in ("Add", "Sub", "Mul"):
+                f = {"Add": np.add, "Sub": np.subtract, "Mul": np.multiply}[name]
+                res = f(same(cv[0]), same(cv[1]))
+            elif name in ("Div", "RealDiv"):
+                if odt in FLOATS:
+                    res = same(cv[0]) / same(cv[1])
+                else:
+                    a, b = same(cv[0]).astype(np.int64), same(cv[1]).astype(np.int64)
+                    q = np.where(b == 0, 0, np.trunc(a / np.where(b == 0, 1, b))).astype(np.int64)
+                    res = q
+            elif name == "Maximum":
+                res = maximum_nan(same(cv[0]), same(cv[1]))
+            elif name == "Minimum":
+                res = minimum_nan(same(cv[0]), same(cv[1]))
+            elif name == "Neg":
+                res = -same(cv[0])
+            elif name == "Abs":
+                res = np.abs(same(cv[0]))
+            elif name == "Square":
+                res = same(cv[0]) * same(cv[0])
+            elif name == "Exp":
+                res = np.exp(same(cv[0]))
+            elif name == "Log":
+                res = np.log(same(cv[0]))
+            elif name == "Tanh":
+                res = np.tanh(same(cv[0]))
+            elif name == "Sqrt":
+                res = np.sqrt(same(cv[0]))
+            elif name == "Rsqrt":
+                x = same(cv[0])
+                res = x.dtype.type(1) / np.sqrt(x)
+            elif name == "Reciprocal":
+                x = same(cv[0])
+                res = x.dtype.type(1) / x
+            elif name == "Floor":
+                res = np.floor(same(cv[0]))
+            elif name in ("Sin", "Cos", "ASin", "ACos", "Atan", "Asinh", "Acosh"):
+                f = {"Sin": np.sin, "Cos": np.cos, "ASin": np.arcsin, "ACos": np.arccos, "Atan": np.arctan,
+                     "Asinh": np.arcsinh, "Acosh": np.arccosh}[name]
+                res = f(same(cv[0]))
+            elif name == "Pow":
+                res = np.power(same(cv[0]), same(cv[1]))
+            elif name == "Atan2":
+                res = np.arctan2(same(cv[0]), same(cv[1]))
+            elif name in ("Equal", "NotEqual", "Greater", "GreaterEqual", "Less", "LessEqual"):
+                f = {"Equal": np.equal, "NotEqual": np.not_equal, "Greater": np.greater,
+                     "GreaterEqual": np.greater_equal, "Less": np.less, "LessEqual": np.less_equal}[name]
+                res = f(cv[0], cv[1])
+            elif name == "IsNan":
+                res = np.isnan(cv[0])
+            elif name == "IsInf":
+                res = np.isinf(cv[0])
+            elif name == "IsFinite":
+                res = np.isfinite(cv[0])
+            elif name == "LogicalNot":
+                res = np.logical_not(cv[0] != 0)
+            elif name == "LogicalAnd":
+                res = np.logical_and(cv[0] != 0, cv[1] != 0)
+            elif name == "LogicalOr":
+                res = np.logical_or(cv[0] != 0, cv[1] != 0)
+            elif name == "Select":
+                res = np.where(cv[0] != 0, same(cv[1]), same(cv[2]))
+            elif name == "AddN":
+                res = same(cv[0])
+                for x in cv[1:]:
+                    res = compute_view(finish(res + same(x), odt), odt)
+            elif name == "Cast":
+                res = cast(ins[0], in_dt[0], odt)
+            elif name == "Reshape":
+                res = ins[0].reshape(oshape)
+            elif name == "BroadcastTo":
+                res = np.broadcast_to(ins[0], oshape)
+            elif name in ("ReduceSum", "ReduceMax", "ReduceMin", "ReducePrd", "ReduceAll", "ReduceAny"):
+                if len(od["input_desc"]) == 2:
+                    axes = od["input_desc"][1][0]["value"]
+                else:
+                    axes = attrs["axis"]
+                if not isinstance(axes, list):
+                    axes = [axes]
+                if not axes:
+                    axes = [1]
+                rank = ins[0].ndim
+                axes = sorted(set(a + rank if a < 0 else a for a in axes))
+                keep = bool(attrs.get("keep_dims", False))
+                x = ins[0]
+                if name in ("ReduceSum", "ReducePrd"):
+                    comb = np.add if name == "ReduceSum" else np.multiply
+                    init = 0 if name == "ReduceSum" else 1
+                    res = serial_reduce(x, axes, comb, init, odt, keep)
+                elif name in ("ReduceMax", "ReduceMin"):
+                    # maxnumf / minnumf are associative and ignore NaN: order does not matter
+                    f = np.fmax if name == "ReduceMax" else np.fmin
+                    if odt in FLOATS:
+                        init = -LARGEST[odt] if name == "ReduceMax" else LARGEST[odt]
+                    else:
+                        info = np.iinfo(NP_DTYPE[odt])
+                        init = info.min if name == "ReduceMax" else info.max
+                    res = f.reduce(x, axis=tuple(axes), keepdims=keep)
+                    res = f(res, np.asarray(init, dtype=res.dtype))
+                else:
+                    f = np.logical_and if name == "ReduceAll" else np.logical_or
+                    res = f.reduce(x != 0, axis=tuple(axes), keepdims=keep)
+            elif name == "MatMul":
+                if attrs.get("transpose_a", False):
+                    raise ValueError("TransposeA is not supported")
+                a, b = ins[0], ins[1]
+                if attrs.get("transpose_b", False):
+                    b = b.T
+                if odt == "int32" and in_dt[0] == "int8" and in_dt[1] == "int8":
+                    res = matmul_exact_i32(a, b)
+                elif odt in ("float32", "float64"):
+                    # serial k order in the output type
+                    res = np.zeros((a.shape[0], b.shape[1]), dtype=NP_DTYPE[odt])
+                    for k in range(a.shape[1]):
+                        res = res + np.outer(a[:, k].astype(res.dtype), b[k, :].astype(res.dtype))
+                else:
+                    raise ValueError("MatMul %s x %s -> %s is not restated" % (in_dt[0], in_dt[1], odt))
+            else:
+                raise ValueError("op %s is not supported by the numpy restatement" % name)
+        res = finish(res, odt) if name not in ("Cast",) else res
+        res = np.asarray(res)
+        if res.size == int(np.prod(oshape)):
+            res = res.reshape(oshape)
+        else:
+            res = np.broadcast_to(res, oshape)
+        env[o["tensor_name"]] = res
+        dtypes[o["tensor_name"]] = odt
+        shapes[o["tensor_name"]] = oshape
+    outs = []
+    for d in desc["output_desc"]:
+        tn = d["tensor_name"]
+        outs.append(to_external(env[tn], dtypes[tn]).reshape(d.get("shape", [1])))
+    return outs
