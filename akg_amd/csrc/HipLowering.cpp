@@ -29,6 +29,7 @@ LoweringOptions LoweringOptions::fromEnvironment() {
   o.chunks = readInt("AKG_HIP_CHUNKS");
   o.block = readInt("AKG_HIP_BLOCK");
   o.gemmVariant = readInt("AKG_HIP_GEMM_VARIANT");
+  if (const char *nt = std::getenv("AKG_HIP_NT")) o.nonTemporal = (nt[0] != '0') ? 1 : 0;
   return o;
 }
 
@@ -171,8 +172,62 @@ bool isElementwiseKind(OpKind k) {
   }
 }
 
-std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vector<std::string> &in) {
+std::vector<bool> relaxedPrecisionTensors(const OpGraph &g) {
+  const size_t n = g.tensors.size();
+  std::vector<bool> relaxed(n, false);
+  if (const char *p = std::getenv("AKG_HIP_PRECISE")) {
+    if (p[0] == '1') return relaxed;
+  }
+  // demand[t]: 0 = no consumer seen yet, 1 = relaxed is enough, 2 = needs full precision
+  std::vector<int> demand(n, 0);
+  auto raise = [&](int t, int d) {
+    if (d > demand[static_cast<size_t>(t)]) demand[static_cast<size_t>(t)] = d;
+  };
+  for (int id : g.outputs) {
+    const DType dt = g.tensor(id).dtype;
+    raise(id, (dt == DType::F16 || dt == DType::BF16) ? 1 : 2);
+  }
+  for (size_t k = g.ops.size(); k-- > 0;) {
+    const OpNode &op = g.ops[k];
+    const int out = op.outputs[0];
+    const DType od = g.tensor(out).dtype;
+    int outDemand = demand[static_cast<size_t>(out)];
+    if (outDemand == 0) outDemand = 2;  // dead value: be conservative
+    int inDemand = outDemand;
+    switch (op.kind) {
+      case OpKind::Cast:
+        if (!isFloatType(od)) {
+          inDemand = 2;  // rounding to an integer / bool is discontinuous
+        } else if ((od == DType::F16 || od == DType::BF16) && outDemand == 1) {
+          inDemand = 1;
+        }
+        break;
+      case OpKind::Equal: case OpKind::NotEqual: case OpKind::Greater: case OpKind::GreaterEqual:
+      case OpKind::Less: case OpKind::LessEqual: case OpKind::Floor: case OpKind::IsNan: case OpKind::IsInf:
+      case OpKind::IsFinite: case OpKind::LogicalNot: case OpKind::LogicalAnd: case OpKind::LogicalOr:
+      case OpKind::MatMul:
+        inDemand = 2;
+        break;
+      default:
+        if (!isFloatType(od)) inDemand = 2;
+        break;
+    }
+    for (size_t i = 0; i < op.inputs.size(); ++i) {
+      int d = inDemand;
+      if (op.kind == OpKind::Select && i == 0) d = 2;
+      raise(op.inputs[i], d);
+    }
+  }
+  for (size_t t = 0; t < n; ++t) {
+    const DType dt = g.tensors[t].dtype;
+    relaxed[t] = demand[t] == 1 && (dt == DType::F32 || dt == DType::F16 || dt == DType::BF16);
+  }
+  return relaxed;
+}
+
+std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vector<std::string> &in, bool relaxed) {
   const DType od = g.tensor(op.outputs[0]).dtype;
+  if (od == DType::F64) relaxed = false;
   const std::string tag = dtypeTag(od);
   const std::string ct = computeTypeName(od);
   auto inType = [&](size_t i) { return g.tensor(op.inputs[i]).dtype; };
@@ -200,10 +255,10 @@ std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vecto
   auto floatOnly = [&]() {
     if (!isFloatType(od)) throw LoweringError("op " + op.name + ": only floating-point tensors are supported");
   };
-  auto unaryMath = [&](const char *fn) {
+  auto unaryMath = [&](const char *fn, const char *fastFn = nullptr) {
     need(1);
     floatOnly();
-    return rnd(std::string("akg::") + fn + "(" + conv(0) + ")");
+    return rnd(std::string("akg::") + ((relaxed && fastFn) ? fastFn : fn) + "(" + conv(0) + ")");
   };
   auto binary = [&](const char *fn) {
     need(2);
@@ -233,7 +288,7 @@ std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vecto
     case OpKind::Add: return binary("op_add");
     case OpKind::Sub: return binary("op_sub");
     case OpKind::Mul: return binary("op_mul");
-    case OpKind::Div: return binary("op_div");
+    case OpKind::Div: return (relaxed && isFloatType(od)) ? binary("fast_div") : binary("op_div");
     case OpKind::Maximum: return binary("op_maximum");
     case OpKind::Minimum: return binary("op_minimum");
     case OpKind::Pow: floatOnly(); return binary("op_pow");
@@ -241,12 +296,12 @@ std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vecto
     case OpKind::Neg: need(1); arith(); return rnd("akg::op_neg(" + conv(0) + ")");
     case OpKind::Abs: need(1); arith(); return rnd("akg::op_abs(" + conv(0) + ")");
     case OpKind::Square: need(1); arith(); return rnd("akg::op_mul(" + conv(0) + ", " + conv(0) + ")");
-    case OpKind::Exp: return unaryMath("op_exp");
-    case OpKind::Log: return unaryMath("op_log");
-    case OpKind::Tanh: return unaryMath("op_tanh");
-    case OpKind::Rsqrt: return unaryMath("op_rsqrt");
-    case OpKind::Sqrt: return unaryMath("op_sqrt");
-    case OpKind::Reciprocal: return unaryMath("op_inv");
+    case OpKind::Exp: return unaryMath("op_exp", "fast_exp");
+    case OpKind::Log: return unaryMath("op_log", "fast_log");
+    case OpKind::Tanh: return unaryMath("op_tanh", "fast_tanh");
+    case OpKind::Rsqrt: return unaryMath("op_rsqrt", "fast_rsqrt");
+    case OpKind::Sqrt: return unaryMath("op_sqrt", "fast_sqrt");
+    case OpKind::Reciprocal: return unaryMath("op_inv", "fast_rcp");
     case OpKind::Floor: return unaryMath("op_floor");
     case OpKind::Sin: return unaryMath("op_sin");
     case OpKind::Cos: return unaryMath("op_cos");
@@ -353,7 +408,7 @@ struct InputAccess {
 
 class TileEmitter {
  public:
-  TileEmitter(const OpGraph &g, const LoweringOptions &o) : g_(g), opt_(o) {}
+  TileEmitter(const OpGraph &g, const LoweringOptions &o) : g_(g), opt_(o) { nonTemporal_ = (o.nonTemporal != 0); }
 
   LoweredKernel run() {
     analyse();
@@ -390,6 +445,8 @@ class TileEmitter {
   int64_t grid_ = 1;
   bool raggedCols_ = false, raggedRows_ = false, raggedFlat_ = false;
   int reduceCount_ = 0;
+  bool nonTemporal_ = true;
+  std::vector<bool> relaxed_;
 
   // ------------------------------------------------------------------ analysis
   void analyse() {
@@ -525,18 +582,19 @@ class TileEmitter {
 
   // ------------------------------------------------------------------ schedule
   void pickSchedule() {
-    // Chunk width: 16 bytes of the narrowest element type that is moved chunk-wise, so the widest access of
-    // every tensor is at least one 128-bit instruction.
-    size_t minSize = 8;
+    // Chunk width: 16 bytes of the widest element type that is moved chunk-wise, so no tensor needs more than one
+    // 128-bit access per chunk (narrower tensors use 64- or 32-bit accesses, which still coalesce fully). Measured
+    // on MI355X: many small contiguous accesses per wave beat fewer, wider ones.
+    size_t minSize = 1;
     bool any = false;
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       if (!access_[i].lastDimFull) continue;
-      minSize = std::min(minSize, dtypeSize(g_.tensor(g_.inputs[i]).dtype));
+      minSize = std::max(minSize, dtypeSize(g_.tensor(g_.inputs[i]).dtype));
       any = true;
     }
     for (int id : g_.outputs) {
       if (rowMode_ && g_.tensor(id).numel() != numel_) continue;
-      minSize = std::min(minSize, dtypeSize(g_.tensor(id).dtype));
+      minSize = std::max(minSize, dtypeSize(g_.tensor(id).dtype));
       any = true;
     }
     if (!any) minSize = 4;
@@ -547,10 +605,12 @@ class TileEmitter {
     vec_ = v;
 
     if (rowMode_) {
-      // One row per group of tpr threads, about 32 elements per thread so that a 4096..8192-wide row of a
-      // 2-byte type has 4 x 128-bit loads in flight per thread and the row stays in registers.
-      int targetPerThread = std::max(vec_, 32);
-      int tpr = opt_.threadsPerRow > 0 ? opt_.threadsPerRow : pow2AtLeast(ceilDiv(cols_, targetPerThread));
+      // One row per group of tpr threads: about 16 elements per thread, at most 256 threads per row (wider rows
+      // get more chunks per thread instead; measured best on MI355X for 4096- and 8192-wide rows). The row stays
+      // in registers across all reductions of the fusion.
+      int targetPerThread = std::max(vec_, 16);
+      int tpr = opt_.threadsPerRow > 0 ? opt_.threadsPerRow
+                                       : std::min(256, pow2AtLeast(ceilDiv(cols_, targetPerThread)));
       tpr = std::max(1, std::min(tpr, 1024));
       if ((tpr & (tpr - 1)) != 0) tpr = pow2AtLeast(tpr);
       // never more threads than chunks in a row
@@ -636,6 +696,7 @@ class TileEmitter {
   // ------------------------------------------------------------------ emission
   void emit() {
     vals_.assign(g_.tensors.size(), ValInfo());
+    relaxed_ = lowering::relaxedPrecisionTensors(g_);
     const std::string kname = g_.name + "_kernel";
 
     line("// Generated by the akg HIP lowering for gfx950. Op description: " + g_.name);
@@ -746,7 +807,10 @@ class TileEmitter {
       line("#pragma unroll");
       line("  for (int j = 0; j < NCHUNK; ++j) {");
       src_ << "    if (akg_ok[j]) {\n";
-      src_ << "      akg::load_chunk<" << tag << ", V>(in" << i << " + " << rowOffsetExpr(a, "akg_rows[j]")
+      // a tensor as large as the iteration space is read exactly once: stream it
+      const bool streamed = nonTemporal_ && (t.numel() == numel_);
+      src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">(in" << i << " + "
+           << rowOffsetExpr(a, "akg_rows[j]")
            << " + akg_cols[j], " << v.ident << "[j]);\n";
       src_ << "    } else {\n";
       src_ << "      akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(" << tag
@@ -807,7 +871,29 @@ class TileEmitter {
 
     std::vector<std::string> operands;
     for (int in : op.inputs) operands.push_back(operandExpr(in));
-    const std::string expr = lowering::elementwiseExpr(g_, op, operands);
+    const bool relaxed = relaxed_[static_cast<size_t>(outId)];
+    std::string expr;
+    // float32 division of a tile by a per-row (or constant) divisor: hoist the reciprocal out of the element loop
+    const bool uniformDivisor = op.kind == OpKind::Div && rank == ValRank::Tile && op.inputs.size() == 2 &&
+                                vals_[static_cast<size_t>(op.inputs[1])].rank != ValRank::Tile &&
+                                std::string(computeTypeName(outT.dtype)) == "float" &&
+                                std::string(computeTypeName(g_.tensor(op.inputs[0]).dtype)) == "float" &&
+                                std::string(computeTypeName(g_.tensor(op.inputs[1]).dtype)) == "float";
+    if (uniformDivisor) {
+      const std::string hoisted = "d" + std::to_string(outId);
+      std::string q;
+      if (relaxed) {
+        src_ << "  const float " << hoisted << " = akg::fast_rcp(" << operands[1] << ");\n";
+        q = "(" + operands[0] + " * " + hoisted + ")";
+      } else {
+        src_ << "  const akg::UniformDivisor " << hoisted << " = akg::make_divisor(" << operands[1] << ");\n";
+        q = "akg::div_uniform(" + operands[0] + ", " + hoisted + ")";
+      }
+      const DType od = outT.dtype;
+      expr = (od == DType::F16 || od == DType::BF16) ? std::string(dtypeTag(od)) + "::rnd(" + q + ")" : q;
+    } else {
+      expr = lowering::elementwiseExpr(g_, op, operands, relaxed);
+    }
 
     ValInfo &v = vals_[static_cast<size_t>(outId)];
     v.defined = true;
@@ -964,7 +1050,8 @@ class TileEmitter {
       std::string guard = "akg_ok[j]";
       if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
       std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
-      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V>(out" << i << " + " << offset << ", " << src
+      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (nonTemporal_ ? "true" : "false") << ">(out"
+           << i << " + " << offset << ", " << src
            << "[j]);\n";
       line("  }");
     } else {

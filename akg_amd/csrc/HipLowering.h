@@ -42,6 +42,7 @@ struct LoweringOptions {
   int chunks = 0;       // chunks per thread
   int block = 0;        // threads per workgroup
   int gemmVariant = 0;  // GEMM tile configuration selector
+  int nonTemporal = 1;  // stream once-touched tensors with non-temporal accesses (AKG_HIP_NT=0 turns it off)
   static LoweringOptions fromEnvironment();
 };
 
@@ -71,7 +72,14 @@ std::string literalFor(DType t, double value);  // constant of the compute type,
 uint64_t countAlgorithmicBytes(const OpGraph &g);
 std::vector<std::vector<int64_t>> buildShapeArgs(const OpGraph &g);
 // Expression of one elementwise op in terms of operand expressions (already in their compute types).
-std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vector<std::string> &operands);
+// `relaxed` selects hardware-approximate transcendental / reciprocal sequences (see precisionDemand).
+std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vector<std::string> &operands,
+                            bool relaxed = false);
+// Backward precision-demand analysis. Returns, per tensor, true when every path from it to a kernel output
+// passes through a Cast to float16 / bfloat16 before anything that needs exact values (integer casts,
+// comparisons, Floor, float32 / float64 / integer outputs). Such values only need about 3 decimal digits, so
+// the lowering may compute them with ~1 ulp float32 hardware approximations (AKG_HIP_PRECISE=1 disables this).
+std::vector<bool> relaxedPrecisionTensors(const OpGraph &g);
 bool isElementwiseKind(OpKind k);
 bool isReduceKind(OpKind k);
 }  // namespace lowering

@@ -1,6 +1,6 @@
 /**
  * akg-hip: command-line driver over the C ABI. One tool where the reference has four
- * (mindspore-translate, akg-opt, akg-translate, akg-ptx-replace; akg-mlir/tools/*), because there is one
+ * (mindspore-translate, akg-opt, akg-translate, akg-ptx-replace; akg-mlir/tools), because there is one
  * step here: op description in, gfx950 code object + meta out.
  *
  *   akg-hip translate X.info            print the typed op graph (mindspore-translate -json-to-mindspore)

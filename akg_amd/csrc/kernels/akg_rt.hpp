@@ -115,26 +115,71 @@ struct is_float_compute<double> {
 // Vector memory access. A chunk of V consecutive elements is moved with the widest instructions the
 // alignment allows (the lowering only picks V such that every chunk start is V-element aligned).
 // ---------------------------------------------------------------------------------------------------------
-template <typename S, int V>
-struct alignas(sizeof(S) * V <= 16 ? sizeof(S) * V : 16) Pack {
-  S v[V];
+// Raw register image of a piece of a chunk: at most 16 bytes per memory instruction.
+template <int BYTES>
+struct Raw;
+template <>
+struct Raw<16> {
+  typedef u32 __attribute__((ext_vector_type(4))) type;
+};
+template <>
+struct Raw<8> {
+  typedef u32 __attribute__((ext_vector_type(2))) type;
+};
+template <>
+struct Raw<4> {
+  typedef u32 type;
+};
+template <>
+struct Raw<2> {
+  typedef u16 type;
+};
+template <>
+struct Raw<1> {
+  typedef u8 type;
 };
 
-template <typename DT, int V>
+// NT = true marks data that is touched exactly once by the whole grid (streamed tensors): the access is issued
+// as a non-temporal one so it does not displace reusable lines (broadcast vectors) from the caches. On MI355X a
+// streaming copy gains about 5 % of HBM bandwidth from this.
+template <typename DT, int V, bool NT = false>
 AKG_DEV void load_chunk(const typename DT::storage *__restrict__ p, typename DT::compute (&dst)[V]) {
-  typedef Pack<typename DT::storage, V> P;
-  P raw = *reinterpret_cast<const P *>(p);
+  typedef typename DT::storage S;
+  constexpr int kBytes = static_cast<int>(sizeof(S)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef typename Raw<kPiece>::type R;
+  R raw[kPieces];
+  const R *rp = reinterpret_cast<const R *>(p);
 #pragma unroll
-  for (int e = 0; e < V; ++e) dst[e] = DT::load(raw.v[e]);
+  for (int k = 0; k < kPieces; ++k) raw[k] = NT ? __builtin_nontemporal_load(rp + k) : rp[k];
+  S tmp[V];
+  __builtin_memcpy(tmp, raw, kBytes);
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(tmp[e]);
 }
 
-template <typename DT, int V>
+template <typename DT, int V, bool NT = false>
 AKG_DEV void store_chunk(typename DT::storage *__restrict__ p, const typename DT::compute (&src)[V]) {
-  typedef Pack<typename DT::storage, V> P;
-  P raw;
+  typedef typename DT::storage S;
+  constexpr int kBytes = static_cast<int>(sizeof(S)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef typename Raw<kPiece>::type R;
+  S tmp[V];
 #pragma unroll
-  for (int e = 0; e < V; ++e) raw.v[e] = DT::store(src[e]);
-  *reinterpret_cast<P *>(p) = raw;
+  for (int e = 0; e < V; ++e) tmp[e] = DT::store(src[e]);
+  R raw[kPieces];
+  __builtin_memcpy(raw, tmp, kBytes);
+  R *rp = reinterpret_cast<R *>(p);
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) {
+    if (NT) {
+      __builtin_nontemporal_store(raw[k], rp + k);
+    } else {
+      rp[k] = raw[k];
+    }
+  }
 }
 
 template <typename DT, int V>
@@ -230,6 +275,58 @@ AKG_DEV bool op_isinf(double a) { return __builtin_fabs(a) == __builtin_inf(); }
 AKG_DEV bool op_isfinite(float a) { return __builtin_fabsf(a) < __builtin_inff(); }
 AKG_DEV bool op_isfinite(double a) { return __builtin_fabs(a) < __builtin_inf(); }
 
+// ---------------------------------------------------------------------------------------------------------
+// Exact float32 division by a value that is the same for a whole row (softmax denominators, quantisation
+// scales). The correctly rounded reciprocal is computed once per row; per element the quotient is
+// q = a * rcp followed by one FMA residual correction, which yields the correctly rounded a / b (Markstein)
+// as long as nothing under- or overflows on the way. Operands outside a conservative exponent window, and
+// zero dividends (whose sign the correction would lose), take the ordinary IEEE division instead.
+// ---------------------------------------------------------------------------------------------------------
+struct UniformDivisor {
+  float b;
+  float rcp;
+  bool safe;
+};
+AKG_DEV UniformDivisor make_divisor(float b) {
+  UniformDivisor d;
+  d.b = b;
+  d.rcp = 1.0f / b;
+  const float ab = __builtin_fabsf(b);
+  d.safe = (ab >= 0x1p-60f) && (ab <= 0x1p+60f);
+  return d;
+}
+AKG_DEV float div_uniform(float a, const UniformDivisor &d) {
+  const float aa = __builtin_fabsf(a);
+  const bool fast = d.safe && (aa >= 0x1p-60f) && (aa <= 0x1p+60f);
+  const float q = a * d.rcp;
+  const float rem = __builtin_fmaf(-q, d.b, a);
+  float res = __builtin_fmaf(rem, d.rcp, q);
+  if (__builtin_expect(!fast, 0)) res = a / d.b;
+  return res;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Relaxed math, used only for values whose every path to a kernel output passes through a cast to a 16-bit
+// float (11 or 8 significant bits): hardware transcendental instructions (about 1 ulp of float32) instead of
+// the correctly rounded / libm-grade sequences. Never used on paths that reach a float32 or integer output.
+// ---------------------------------------------------------------------------------------------------------
+AKG_DEV float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+AKG_DEV float fast_div(float a, float b) { return a * __builtin_amdgcn_rcpf(b); }
+AKG_DEV float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 0x1.715476p+0f); }
+AKG_DEV float fast_log(float x) { return __builtin_amdgcn_logf(x) * 0x1.62e43p-1f; }
+AKG_DEV float fast_sqrt(float x) { return __builtin_amdgcn_sqrtf(x); }
+AKG_DEV float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+AKG_DEV float fast_tanh(float x) {
+  // tanh(|x|) = 1 - 2 / (exp(2|x|) + 1); for small |x| the odd Taylor polynomial avoids the cancellation.
+  const float ax = __builtin_fabsf(x);
+  const float x2 = x * x;
+  const float poly = ax * (1.0f + x2 * (-0x1.555556p-2f + x2 * (0x1.111112p-3f + x2 * (-0x1.ba1ba2p-5f + x2 * 0x1.664f48p-6f))));
+  const float t = __builtin_amdgcn_exp2f(ax * 0x1.715476p+1f);
+  const float big = 1.0f - 2.0f * __builtin_amdgcn_rcpf(t + 1.0f);
+  const float r = ax < 0.25f ? poly : big;
+  return __builtin_copysignf(r, x);
+}
+
 // Reduction combiners (arith.addf / maxnumf / minnumf / mulf and their integer twins).
 struct RedSum {
   template <typename T>
@@ -306,6 +403,22 @@ struct ToInt<DST, SRCC, true> {
     if (r <= lo) return static_cast<typename DST::compute>(IntRange<DST>::lo);
     if (r >= hi) return static_cast<typename DST::compute>(IntRange<DST>::hi);
     return static_cast<typename DST::compute>(r);
+  }
+};
+// float32 -> int8 / int16: both bounds are float32 values, so the clamp is one v_med3_f32 and the conversion is
+// always in range: v_rndne_f32, v_med3_f32, v_cvt_i32_f32 (+ the NaN -> 0 select).
+template <>
+struct ToInt<i8, float, true> {
+  static AKG_DEV int run(float x) {
+    float r = __builtin_amdgcn_fmed3f(__builtin_rintf(x), -128.0f, 127.0f);
+    return (x != x) ? 0 : static_cast<int>(r);
+  }
+};
+template <>
+struct ToInt<i16, float, true> {
+  static AKG_DEV int run(float x) {
+    float r = __builtin_amdgcn_fmed3f(__builtin_rintf(x), -32768.0f, 32767.0f);
+    return (x != x) ? 0 : static_cast<int>(r);
   }
 };
 template <typename DST, typename SRCC>
