@@ -20,6 +20,8 @@ FIXTURES = {
     "c3_layernorm_residual_bf16_16384x4096": lambda n: op_desc.layernorm_residual(16384, 4096, "bfloat16", 1e-5, n),
     "c4_quant_int8_residual_bf16_32768x8192": lambda n: op_desc.quant_int8_residual(32768, 8192, "bfloat16", n),
     "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": lambda n: op_desc.gemm_int8_dequant_bias_gelu(4096, 8192, 8192, "bfloat16", False, n),
+    # plain streaming kernel of known size, used to calibrate the HBM traffic counters
+    "calib_neg_f32_16384x4096": lambda n: _neg(16384, 4096, n),
     # small parity cases
     "small_ew_tanh_add_mul_f32_8x128": lambda n: op_desc.elementwise_tanh_add_mul(8, 128, n),
     "small_ew_tanh_add_mul_f32_7x33": lambda n: op_desc.elementwise_tanh_add_mul(7, 33, n),
@@ -33,6 +35,12 @@ FIXTURES = {
     "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", True, n),
 }
+
+
+def _neg(rows, cols, name):
+    b = op_desc.DescBuilder(name)
+    x = b.input([rows, cols], "float32")
+    return b.dumps([b.unary("Neg", x)])
 
 
 def main():
