@@ -1,11 +1,298 @@
+/**
+ * Lowering of the Matmul fusion class: one int8 MatMul followed by an elementwise epilogue over [M,N].
+ *
+ * The reference lowers MatMul to linalg.matmul and then through the same generic loop mapping as everything else
+ * (akg-mlir/lib/Conversion/MindSporeToLinalg/MindSporeToLinalg.cpp:1453-1546; no tensor-core path is wired into
+ * its GPU pipeline). Here the contraction runs on the MFMA units (kernels/akg_gemm_i8.hpp) and the ops that follow
+ * it in the description are emitted as an epilogue functor applied to the int32 accumulators in registers, so the
+ * [M,N] int32 / float32 intermediates never exist in memory.
+ *
+ * Epilogue operands are classified by how they vary over the output tile:
+ *   Full   [M,N]      4-element chunk per (row, 4 columns), loaded / computed per output chunk
+ *   Col    [N]/[1,N]  4 values per lane, loaded / computed once per lane (a lane owns 4 fixed columns)
+ *   Row    [M,1]      one value per output row
+ *   Scalar [1]        one value
+ */
+#include <sstream>
+
 #include "HipLowering.h"
 
 namespace akg {
+namespace {
+
+using lowering::computeTypeName;
+using lowering::dtypeTag;
+
+enum class EpiRank { Const = 0, Scalar = 1, Row = 2, Col = 3, Full = 4 };
+
+struct EpiVal {
+  bool defined = false;
+  EpiRank rank = EpiRank::Const;
+  std::string ident;
+};
+
+class GemmEmitter {
+ public:
+  GemmEmitter(const OpGraph &g, const LoweringOptions &o) : g_(g), opt_(o) {}
+
+  LoweredKernel run() {
+    analyse();
+    emit();
+    LoweredKernel k;
+    k.kernelName = g_.name + "_kernel";
+    k.source = src_.str();
+    k.family = KernelFamily::GemmEpilogue;
+    const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
+    k.grid[0] = static_cast<unsigned>(((tiles + 7) / 8) * 8);
+    k.block[0] = 256;
+    k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
+    k.algorithmicOps = 2ull * static_cast<uint64_t>(m_) * static_cast<uint64_t>(n_) * static_cast<uint64_t>(k_);
+    k.shapeArgs = lowering::buildShapeArgs(g_);
+    std::ostringstream note;
+    note << "gemm_epilogue M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
+         << " tile=256x256x64 mfma=i32_32x32x32_i8 waves=2x2 grid=" << k.grid[0];
+    k.scheduleNote = note.str();
+    return k;
+  }
+
+ private:
+  const OpGraph &g_;
+  LoweringOptions opt_;
+  std::ostringstream src_;
+  int64_t m_ = 0, n_ = 0, k_ = 0;
+  bool transB_ = false;
+  int matmulOp_ = -1;
+  int aId_ = -1, bId_ = -1, accId_ = -1;
+  std::vector<EpiVal> vals_;
+  std::vector<bool> relaxed_;
+  std::ostringstream members_, prepare_, apply_;
+
+  void analyse() {
+    for (size_t i = 0; i < g_.ops.size(); ++i) {
+      const OpNode &op = g_.ops[i];
+      if (op.kind == OpKind::MatMul) {
+        if (matmulOp_ >= 0) throw LoweringError("only one MatMul per kernel is supported");
+        matmulOp_ = static_cast<int>(i);
+      } else if (op.kind == OpKind::Unknown) {
+        throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
+      } else if (op.kind == OpKind::Unsupported || lowering::isReduceKind(op.kind)) {
+        throw LoweringError("op " + op.name + " cannot be fused into a MatMul epilogue yet");
+      }
+    }
+    const OpNode &mm = g_.ops[static_cast<size_t>(matmulOp_)];
+    if (mm.transposeA) throw LoweringError("MatMul: transpose_a is not supported (as in the reference)");
+    transB_ = mm.transposeB;
+    aId_ = mm.inputs[0];
+    bId_ = mm.inputs[1];
+    accId_ = mm.outputs[0];
+    const TensorValue &a = g_.tensor(aId_);
+    const TensorValue &b = g_.tensor(bId_);
+    const TensorValue &c = g_.tensor(accId_);
+    if (a.inputIndex < 0 || b.inputIndex < 0) {
+      throw LoweringError("MatMul operands must be kernel inputs (prologue fusion is not supported yet)");
+    }
+    if (a.dtype != DType::I8 || b.dtype != DType::I8 || c.dtype != DType::I32) {
+      throw LoweringError("MatMul: only int8 x int8 -> int32 has an MFMA kernel yet");
+    }
+    if (a.shape.size() != 2 || b.shape.size() != 2 || c.shape.size() != 2) {
+      throw LoweringError("MatMul: only rank-2 operands are supported");
+    }
+    m_ = a.shape[0];
+    k_ = a.shape[1];
+    n_ = transB_ ? b.shape[0] : b.shape[1];
+    const int64_t kb = transB_ ? b.shape[1] : b.shape[0];
+    if (kb != k_ || c.shape[0] != m_ || c.shape[1] != n_) throw LoweringError("MatMul: inconsistent shapes");
+    if (k_ % 16 != 0) throw LoweringError("MatMul: K must be a multiple of 16");
+    if (n_ % 4 != 0) throw LoweringError("MatMul: N must be a multiple of 4");
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::MatMul) continue;
+      for (int in : op.inputs) {
+        if (in == aId_ || in == bId_) throw LoweringError("MatMul operands cannot also feed the epilogue");
+      }
+    }
+    if (g_.tensor(accId_).outputIndex >= 0) {
+      // the raw int32 product as an output is fine: it is just another Full value
+    }
+  }
+
+  std::string ctOf(int id) const { return computeTypeName(g_.tensor(id).dtype); }
+  std::string tagOf(int id) const { return dtypeTag(g_.tensor(id).dtype); }
+
+  EpiRank classifyInput(const TensorValue &t) const {
+    if (t.numel() == 1) return EpiRank::Scalar;
+    std::vector<int64_t> s = t.shape;
+    while (s.size() > 2 && s.front() == 1) s.erase(s.begin());
+    if (s.size() == 1) s.insert(s.begin(), 1);
+    if (s.size() != 2) throw LoweringError("epilogue input " + t.name + ": rank exceeds the output's");
+    if (s[0] == m_ && s[1] == n_) return EpiRank::Full;
+    if (s[0] == 1 && s[1] == n_) return EpiRank::Col;
+    if (s[0] == m_ && s[1] == 1) return EpiRank::Row;
+    throw LoweringError("epilogue input " + t.name + " does not broadcast to the MatMul result");
+  }
+
+  std::string operand(int id) const {
+    const EpiVal &v = vals_[static_cast<size_t>(id)];
+    if (!v.defined) throw LoweringError("internal: epilogue operand " + g_.tensor(id).name + " undefined");
+    if (v.rank == EpiRank::Full || v.rank == EpiRank::Col) return v.ident + "[e]";
+    return v.ident;
+  }
+
+  void emit() {
+    vals_.assign(g_.tensors.size(), EpiVal());
+    relaxed_ = lowering::relaxedPrecisionTensors(g_);
+    const bool nt = opt_.nonTemporal != 0;
+
+    // accumulators
+    EpiVal &acc = vals_[static_cast<size_t>(accId_)];
+    acc.defined = true;
+    acc.rank = EpiRank::Full;
+    acc.ident = "acc";
+
+    // constants
+    for (size_t t = 0; t < g_.tensors.size(); ++t) {
+      if (!g_.tensors[t].isConst) continue;
+      vals_[t].defined = true;
+      vals_[t].rank = EpiRank::Const;
+      vals_[t].ident = lowering::literalFor(g_.tensors[t].dtype, g_.tensors[t].constValue);
+    }
+    // inputs
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      const int id = g_.inputs[i];
+      if (id == aId_ || id == bId_) continue;
+      const TensorValue &t = g_.tensor(id);
+      const EpiRank r = classifyInput(t);
+      EpiVal &v = vals_[static_cast<size_t>(id)];
+      v.defined = true;
+      v.rank = r;
+      const std::string tag = tagOf(id), ct = ctOf(id);
+      members_ << "  const " << tag << "::storage *__restrict__ in" << i << ";\n";
+      switch (r) {
+        case EpiRank::Scalar:
+          v.ident = "s_in" + std::to_string(i);
+          members_ << "  " << ct << " " << v.ident << ";\n";
+          prepare_ << "    " << v.ident << " = " << tag << "::load(in" << i << "[0]);\n";
+          break;
+        case EpiRank::Col:
+          v.ident = "c_in" + std::to_string(i);
+          members_ << "  " << ct << " " << v.ident << "[4];\n";
+          prepare_ << "    akg::load_chunk<" << tag << ", 4, false>(in" << i << " + col, " << v.ident << ");\n";
+          break;
+        case EpiRank::Row:
+          v.ident = "r_in" + std::to_string(i);
+          apply_ << "    const " << ct << " " << v.ident << " = " << tag << "::load(in" << i << "[row]);\n";
+          break;
+        case EpiRank::Full:
+          v.ident = "t_in" + std::to_string(i);
+          apply_ << "    " << ct << " " << v.ident << "[4];\n";
+          apply_ << "    akg::load_chunk<" << tag << ", 4, " << (nt ? "true" : "false") << ">(in" << i << " + row * " << n_
+                 << "L + col, " << v.ident << ");\n";
+          break;
+        default:
+          break;
+      }
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      members_ << "  " << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i << ";\n";
+    }
+    // ops
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::MatMul) continue;
+      if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+      const int outId = op.outputs[0];
+      bool hasRow = false, hasCol = false, hasFull = false, hasScalar = false;
+      for (int in : op.inputs) {
+        const EpiVal &vi = vals_[static_cast<size_t>(in)];
+        if (!vi.defined) throw LoweringError("op " + op.name + ": operand " + g_.tensor(in).name + " is undefined");
+        hasRow |= vi.rank == EpiRank::Row;
+        hasCol |= vi.rank == EpiRank::Col;
+        hasFull |= vi.rank == EpiRank::Full;
+        hasScalar |= vi.rank == EpiRank::Scalar;
+      }
+      EpiRank rank = EpiRank::Scalar;
+      if (hasFull || (hasRow && hasCol)) {
+        rank = EpiRank::Full;
+      } else if (hasCol) {
+        rank = EpiRank::Col;
+      } else if (hasRow) {
+        rank = EpiRank::Row;
+      }
+      (void)hasScalar;
+      std::vector<std::string> operands;
+      for (int in : op.inputs) operands.push_back(operand(in));
+      const std::string expr = lowering::elementwiseExpr(g_, op, operands, relaxed_[static_cast<size_t>(outId)]);
+      EpiVal &v = vals_[static_cast<size_t>(outId)];
+      v.defined = true;
+      v.rank = rank;
+      const std::string ct = ctOf(outId);
+      const std::string comment = "  // " + op.name + " -> " + g_.tensor(outId).name + "\n";
+      switch (rank) {
+        case EpiRank::Full:
+          v.ident = "t" + std::to_string(outId);
+          apply_ << "    " << ct << " " << v.ident << "[4];" << comment;
+          apply_ << "#pragma unroll\n    for (int e = 0; e < 4; ++e) " << v.ident << "[e] = " << expr << ";\n";
+          break;
+        case EpiRank::Col:
+          v.ident = "c" + std::to_string(outId);
+          members_ << "  " << ct << " " << v.ident << "[4];\n";
+          prepare_ << "#pragma unroll\n    for (int e = 0; e < 4; ++e) " << v.ident << "[e] = " << expr << ";" << comment;
+          break;
+        case EpiRank::Row:
+          v.ident = "r" + std::to_string(outId);
+          apply_ << "    const " << ct << " " << v.ident << " = " << expr << ";" << comment;
+          break;
+        default:
+          v.ident = "s" + std::to_string(outId);
+          members_ << "  " << ct << " " << v.ident << ";\n";
+          prepare_ << "    " << v.ident << " = " << expr << ";" << comment;
+          break;
+      }
+    }
+    // stores
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      const int id = g_.outputs[i];
+      const TensorValue &t = g_.tensor(id);
+      const EpiVal &v = vals_[static_cast<size_t>(id)];
+      if (!v.defined) throw LoweringError("output " + t.name + " is never computed");
+      if (t.numel() != m_ * n_ || v.rank != EpiRank::Full) {
+        throw LoweringError("output " + t.name + ": only [M,N] outputs of a MatMul fusion are supported");
+      }
+      apply_ << "    akg::store_chunk<" << tagOf(id) << ", 4, " << (nt ? "true" : "false") << ">(out" << i << " + row * "
+             << n_ << "L + col, " << v.ident << ");\n";
+    }
+
+    const std::string kname = g_.name + "_kernel";
+    src_ << "// Generated by the akg HIP lowering for gfx950. Op description: " << g_.name << "\n";
+    src_ << "// family: gemm_epilogue, fusion class: " << operatorTemplateName(g_.operatorTemplate) << "\n";
+    src_ << "#include \"akg_rt.hpp\"\n#include \"akg_gemm_i8.hpp\"\n\n";
+    src_ << "namespace {\nstruct Epilogue {\n" << members_.str();
+    src_ << "  AKG_DEV void prepare(long col) {\n    (void)col;\n" << prepare_.str() << "  }\n";
+    src_ << "  AKG_DEV void apply(const int (&acc)[4], long row, long col) {\n" << apply_.str() << "  }\n";
+    src_ << "};\n}  // namespace\n\n";
+    src_ << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(";
+    size_t argc = 0;
+    for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
+    }
+    src_ << ") {\n  Epilogue epi;\n";
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      const int id = g_.inputs[i];
+      if (id == aId_ || id == bId_) continue;
+      src_ << "  epi.in" << i << " = in" << i << ";\n";
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
+    src_ << "  akg::gemm_i8_256x256<" << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
+         << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
+  }
+};
+
+}  // namespace
 
 LoweredKernel lowerGemmToHip(const OpGraph &graph, const LoweringOptions &options) {
-  (void)graph;
-  (void)options;
-  throw LoweringError("MatMul fusions: kernel family not built yet");
+  GemmEmitter emitter(graph, options);
+  return emitter.run();
 }
 
 }  // namespace akg

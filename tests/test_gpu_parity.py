@@ -57,7 +57,7 @@ def check_fixture(name, seed, openmp):
         assert ok, "%s output %s: %s" % (name, d.name, msg)
 
 
-@pytest.mark.parametrize("name", [n for n in SMALL if "gemm" not in n])
+@pytest.mark.parametrize("name", SMALL)
 def test_small_fixture_matches_oracle(name):
     check_fixture(name, seed=harness.BASE_SEED + 100, openmp=False)
 
