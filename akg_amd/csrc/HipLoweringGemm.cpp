@@ -44,13 +44,13 @@ class GemmEmitter {
     k.family = KernelFamily::GemmEpilogue;
     const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
     k.grid[0] = static_cast<unsigned>(((tiles + 7) / 8) * 8);
-    k.block[0] = 256;
+    k.block[0] = static_cast<unsigned>(wavesM() * 2 * 64);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.algorithmicOps = 2ull * static_cast<uint64_t>(m_) * static_cast<uint64_t>(n_) * static_cast<uint64_t>(k_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
     note << "gemm_epilogue M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
-         << " tile=256x256x64 mfma=i32_32x32x32_i8 waves=2x2 grid=" << k.grid[0];
+         << " tile=256x256x64 mfma=i32_32x32x32_i8 waves=" << wavesM() << "x2 grid=" << k.grid[0];
     k.scheduleNote = note.str();
     return k;
   }
@@ -66,6 +66,9 @@ class GemmEmitter {
   std::vector<EpiVal> vals_;
   std::vector<bool> relaxed_;
   std::ostringstream members_, prepare_, apply_;
+
+  // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_GEMM_VARIANT=1.
+  int wavesM() const { return opt_.gemmVariant == 1 ? 2 : 4; }
 
   void analyse() {
     for (size_t i = 0; i < g_.ops.size(); ++i) {
@@ -268,7 +271,7 @@ class GemmEmitter {
     src_ << "  AKG_DEV void prepare(long col) {\n    (void)col;\n" << prepare_.str() << "  }\n";
     src_ << "  AKG_DEV void apply(const int (&acc)[4], long row, long col) {\n" << apply_.str() << "  }\n";
     src_ << "};\n}  // namespace\n\n";
-    src_ << "extern \"C\" __global__ __launch_bounds__(256) void " << kname << "(";
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << wavesM() * 128 << ") void " << kname << "(";
     size_t argc = 0;
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
@@ -284,7 +287,7 @@ class GemmEmitter {
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
     src_ << "  akg::gemm_i8_256x256<" << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
+         << ", " << wavesM() << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
   }
 };
 

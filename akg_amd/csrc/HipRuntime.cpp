@@ -64,10 +64,19 @@ const std::vector<std::string> &compileFlags() {
   // -ffp-contract=off: every op of the description is its own IEEE operation in the reference CPU pipeline;
   //   fusing a*b+c into an fma would change results (and break the bit-exact int8 quantisation).
   // packed-fp32-ops off: the compiler must not form v_pk_{add,mul,fma}_f32.
-  static const std::vector<std::string> flags = {
-    "--offload-arch=gfx950", "-O3",      "-std=c++17",     "-ffp-contract=off",
-    "-Xclang",               "-target-feature", "-Xclang", "-packed-fp32-ops",
-  };
+  static const std::vector<std::string> flags = [] {
+    std::vector<std::string> f = {
+      "--offload-arch=gfx950", "-O3",      "-std=c++17",     "-ffp-contract=off",
+      "-Xclang",               "-target-feature", "-Xclang", "-packed-fp32-ops",
+    };
+    // AKG_HIP_EXTRA_FLAGS: space-separated extra device-compiler flags (experiments; part of the cache key)
+    if (const char *extra = std::getenv("AKG_HIP_EXTRA_FLAGS")) {
+      std::istringstream is(extra);
+      std::string tok;
+      while (is >> tok) f.push_back(tok);
+    }
+    return f;
+  }();
   return flags;
 }
 
