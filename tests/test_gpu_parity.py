@@ -66,3 +66,90 @@ def test_small_fixture_matches_oracle(name):
 def test_full_size_config_matches_oracle(name):
     # full BASELINE sizes; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)
     check_fixture(name, seed=harness.BASE_SEED + 1 + FULL.index(name), openmp=True)
+
+
+REF_INFO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_info")
+REF_STATIC = sorted(f for f in os.listdir(REF_INFO)
+                    if f.endswith(".info") and ".dynamic." not in f and "13305325157517622155" not in f)
+
+
+@pytest.mark.parametrize("name", REF_STATIC)
+def test_reference_repository_descriptions_match_oracle(name):
+    """Op descriptions taken unchanged from the reference's own system-test data (static-shape ones)."""
+    path = os.path.join(REF_INFO, name)
+    print("case %s" % name, flush=True)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 200)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path)(inputs)
+    for d, g, e in zip(kernel.outputs, got, expect):
+        ok, msg = harness.compare(g, e, d.dtype)
+        print("  %s %s: %s" % (d.name, d.dtype, msg), flush=True)
+        assert ok, "%s output %s: %s" % (name, d.name, msg)
+
+
+def test_run_host_reference_style_call_and_driver():
+    """Host pointers in, outputs overwritten in place (the reference shim's calling convention), through HipDriver."""
+    path = os.path.join(FIXTURES, "small_layernorm_residual_bf16_19x520.info")
+    desc = harness.load_desc(path)
+    d = driver.HipDriver(input_file=path)
+    kernel = d.compile()
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 300)
+    outs = kernel.empty_outputs(fill_nan=True)
+    res = d.run(inputs + outs, output_indexes=[-1])
+    assert res[0] is outs[0]
+    expect = cpu_ref.CpuKernel(path)(inputs)
+    ok, msg = harness.compare(outs[0], expect[0], "bfloat16")
+    assert ok, msg
+    # wrong tensor count is an error, not a crash
+    with pytest.raises(ValueError):
+        kernel.run_host(inputs)
+
+
+def test_profile_entry_point_returns_a_plausible_time():
+    import torch
+    path = os.path.join(FIXTURES, "small_softmax_f16_64x4096.info")
+    kernel = driver.HipKernel.from_file(path)
+    bufs = [torch.zeros(t.nbytes, dtype=torch.uint8, device="cuda:0") for t in kernel.tensors]
+    ms = kernel.profile_ptrs([b.data_ptr() for b in bufs], number=5, repeat=3)
+    assert 0.0 < ms < 50.0
+
+
+def test_c5_full_size_gemm_fusion():
+    """Full configuration: 4096 x 8192 x 8192. The CPU oracle cannot run 2.7e11 MACs in a test, so:
+    (1) 96 sampled rows (all 8192 columns each, rows spread over every 256-row tile) against the oracle evaluated on
+        exactly those rows of A (exact int32 accumulation, same epilogue);
+    (2) every output against an independent computation of the same formula with torch on the GPU
+        (torch._int_mm for the exact int32 product), within the bfloat16 tolerance."""
+    import torch
+    from oracle import np_ref
+    from akg_amd import op_desc
+    name = "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192.info"
+    path = os.path.join(FIXTURES, name)
+    print("case %s" % name, flush=True)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 5)
+    got = run_on_gpu(kernel, inputs)[0]
+    a, sa, w, sb, bias = inputs
+    rng = np.random.default_rng(99)
+    rows = np.sort(np.concatenate([np.arange(16) * 256 + rng.integers(0, 256, 16), rng.integers(0, 4096, 80)]))
+    sub = json_loads(op_desc.gemm_int8_dequant_bias_gelu(len(rows), 8192, 8192, "bfloat16", False, "c5_rows"))
+    expect_rows = np_ref.evaluate(sub, [a[rows], sa[rows], w, sb, bias])[0]
+    ok, msg = harness.compare(got[rows], expect_rows, "bfloat16")
+    print("  sampled rows vs oracle: %s" % msg, flush=True)
+    assert ok, msg
+    dev = torch.device("cuda:0")
+    acc = torch._int_mm(torch.from_numpy(a).to(dev), torch.from_numpy(w).to(dev))
+    x = acc.float() * torch.from_numpy(sa).to(dev) * torch.from_numpy(sb).to(dev)
+    x = x + torch.from_numpy(harness.bf16_bits_to_f32(bias)).to(dev)
+    ref = torch.nn.functional.gelu(x, approximate="tanh").to(torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+    ok, msg = harness.compare(got, ref, "bfloat16")
+    print("  all outputs vs torch: %s" % msg, flush=True)
+    assert ok, msg
+
+
+def json_loads(text):
+    import json
+    return json.loads(text)

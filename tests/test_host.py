@@ -1,0 +1,297 @@
+"""Host-side logic, runnable without a GPU: the C-ABI library loads and exports every declared symbol, the JSON
+translator reads descriptions the way the reference's does (checked against Python's own JSON reader on the reference's
+own fixture files), error conventions, artifact formats, and the lowering decisions (family, schedule, math selection).
+No kernel is launched here.
+"""
+import ctypes
+import hashlib
+import json
+import os
+import re
+import subprocess
+
+import pytest
+
+from akg_amd import driver, harness, op_desc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FIXTURES = os.path.join(ROOT, "akg_amd", "fixtures")
+REF_INFO = os.path.join(ROOT, "tests", "golden", "ref_info")
+HEADER = os.path.join(ROOT, "include", "akg_hip.h")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# C ABI
+# ---------------------------------------------------------------------------------------------------------
+def declared_symbols():
+    with open(HEADER, "r", encoding="utf-8") as f:
+        text = f.read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(akg_hip_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_symbol_the_header_declares():
+    lib = driver.load_library()
+    names = declared_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), "libakg_hip.so does not export %s" % n
+    # and nothing in the signatures is a C++ / torch type: the header compiles as plain C
+    r = subprocess.run(["gcc", "-std=c99", "-fsyntax-only", "-x", "c", HEADER], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
+def test_version_and_last_error():
+    lib = driver.load_library()
+    assert b"gfx950" in lib.akg_hip_version()
+    h = ctypes.c_void_p()
+    rc = lib.akg_hip_compile(b"{", 1, None, ctypes.byref(h))
+    assert rc == -2 and not h.value
+    assert b"json" in lib.akg_hip_last_error()
+
+
+def test_null_arguments_are_rejected_not_crashed_on():
+    lib = driver.load_library()
+    h = ctypes.c_void_p()
+    assert lib.akg_hip_compile(None, 0, None, ctypes.byref(h)) == -1
+    assert lib.akg_hip_compile(b"{}", 2, None, None) == -1
+    n = ctypes.c_int()
+    assert lib.akg_hip_kernel_num_tensors(None, ctypes.byref(n)) == -1
+    assert lib.akg_hip_launch(None, None, 0, None) == -1
+    lib.akg_hip_kernel_destroy(None)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# translator vs an independent JSON reader, on the reference's own fixture files
+# ---------------------------------------------------------------------------------------------------------
+STATIC_REF = sorted(f for f in os.listdir(REF_INFO) if f.endswith(".info") and ".dynamic." not in f)
+
+
+@pytest.mark.parametrize("name", STATIC_REF)
+def test_signature_of_reference_fixture_matches_python_json(name):
+    path = os.path.join(REF_INFO, name)
+    desc = harness.load_desc(path)
+    text = driver.translate(open(path, "r", encoding="utf-8").read())
+    # function name and attributes
+    assert text.startswith("func.func @%s(" % desc["op"])
+    assert 'process = "%s"' % desc["process"] in text
+    arch = desc.get("target_info", {}).get("arch", "")
+    assert 'arch = "%s"' % arch in text
+    # inputs in input_desc order, outputs in output_desc order, uint8 read as int8
+    head = text.split("\n", 1)[0]
+    args = re.findall(r"%(\w+): tensor<([0-9x]*)(\w+)>", head)
+    assert [a[0] for a in args] == [e[0]["tensor_name"] for e in desc["input_desc"]]
+    for (nm, dims, dt), e in zip(args, desc["input_desc"]):
+        want_dt = "int8" if e[0]["data_type"] == "uint8" else e[0]["data_type"]
+        assert dt == want_dt
+        assert [int(d) for d in dims.split("x") if d] == e[0].get("shape", [1])
+    ret = re.search(r"return (.*)", text).group(1)
+    assert [r.strip().lstrip("%") for r in ret.split(",")] == [o["tensor_name"] for o in desc["output_desc"]]
+    # one mindspore op per op_desc entry, in order
+    ops = re.findall(r'= "mindspore\.(\w+)"', text)
+    ops = [o for o in ops if o != "const"]
+    assert len(ops) == len(desc["op_desc"])
+
+
+def test_scalar_constant_inputs_become_constants():
+    path = os.path.join(REF_INFO, "Fused_Mul_RealDiv_Exp_fusion_2550894545544229730.info")
+    text = driver.translate(open(path, "r", encoding="utf-8").read())
+    assert '"mindspore.const"() {value = -0.00599632' in text     # "value" on a shape-[1] operand, attr: null
+    assert text.count('"mindspore.mul"') == 1 and text.count('"mindspore.exp"') == 1
+
+
+def test_dynamic_shapes_are_a_translate_error():
+    path = os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.translate(open(path, "r", encoding="utf-8").read())
+    assert e.value.code == -3 and "dynamic" in str(e.value)
+
+
+def _desc(mutate):
+    d = json.loads(op_desc.elementwise_tanh_add_mul(4, 8, "t"))
+    mutate(d)
+    return json.dumps(d)
+
+
+def test_error_conventions():
+    # malformed JSON -> -2
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel('{"op": ', out_dir=None)
+    assert e.value.code == -2
+    # missing required key -> json error naming the key (the reference's .at() throws as well)
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(_desc(lambda d: d.pop("process")), out_dir=None)
+    assert "process" in str(e.value)
+    # dtype outside the type table -> translate error
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(_desc(lambda d: d["input_desc"][0][0].update(data_type="complex64")), out_dir=None)
+    assert e.value.code == -3
+    # op name outside the op table: translator accepts it (mindspore.unknown), lowering rejects it -> -4
+    unknown = _desc(lambda d: d["op_desc"][2].update(name="Erf"))
+    assert '"mindspore.unknown"' in driver.translate(unknown) and 'ori_op = "Erf"' in driver.translate(unknown)
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(unknown, out_dir=None)
+    assert e.value.code == -4 and "Erf" in str(e.value)
+    # attribute with an unsupported data_type is fatal
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(_desc(lambda d: d["op_desc"][0].update(attr=[{"name": "x", "data_type": "tensor", "value": 1}])),
+                         out_dir=None)
+    assert e.value.code == -3
+    # operand that is neither defined nor a constant
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(_desc(lambda d: d["op_desc"][0]["input_desc"][0][0].update(tensor_name="nowhere")), out_dir=None)
+    assert e.value.code == -3 and "nowhere" in str(e.value)
+    # reduce over a non-innermost axis: valid description, no kernel family yet
+    path = os.path.join(REF_INFO, "Fused_Mul_ReduceSum_split_13305325157517622155.info")
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel.from_file(path, out_dir=None)
+    assert e.value.code == -4
+    # path with '..' is refused (checkAndReadJson)
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel.from_file(os.path.join(FIXTURES, "..", "fixtures", "small_softmax_f32_5x77.info"), out_dir=None)
+    assert e.value.code == -6
+
+
+def test_uint8_is_read_as_int8_and_missing_shape_is_one():
+    def mut(d):
+        d["input_desc"][0][0]["data_type"] = "uint8"
+        d["op_desc"][0]["input_desc"][0][0]["data_type"] = "uint8"
+    text = driver.translate(_desc(mut))
+    assert "%input_0: tensor<4x8xint8>" in text
+
+    def drop(d):
+        d["input_desc"] = [[{"tensor_name": "input_0", "data_type": "float32"}]]
+        d["op_desc"] = [{"name": "Neg", "attr": None, "input_desc": [[{"tensor_name": "input_0", "data_type": "float32"}]],
+                         "output_desc": [{"tensor_name": "o", "data_type": "float32"}]}]
+        d["output_desc"] = [{"tensor_name": "o", "data_type": "float32"}]
+    text = driver.translate(_desc(drop))
+    assert "%input_0: tensor<1xfloat32>" in text
+
+
+def test_reduce_axis_from_second_input_and_negative_axis():
+    b = op_desc.DescBuilder("r")
+    x = b.input([4, 6], "float32")
+    out = b.reduce("ReduceSum", x, [-1], True)
+    d = b.build([out])
+    d["op_desc"][0]["attr"] = [{"name": "keep_dims", "data_type": "bool", "value": True}]
+    d["op_desc"][0]["input_desc"].append([{"tensor_name": "axis", "data_type": "int64", "shape": [1], "value": -1}])
+    text = driver.translate(json.dumps(d))
+    assert "axis = [1], keepdims = true" in text
+
+
+# ---------------------------------------------------------------------------------------------------------
+# lowering decisions and artifacts
+# ---------------------------------------------------------------------------------------------------------
+def test_fusion_class_and_family_per_configuration():
+    want = {
+        "c1_ew_tanh_add_mul_f32_1024x4096": ("Elementwise", "elementwise"),
+        "c2_softmax_f16_8192x4096": ("Reduction", "row_reduce"),
+        "c3_layernorm_residual_bf16_16384x4096": ("Reduction", "row_reduce"),
+        "c4_quant_int8_residual_bf16_32768x8192": ("Reduction", "row_reduce"),
+        "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": ("Matmul", "gemm_epilogue"),
+    }
+    bytes_want = {"c1_ew_tanh_add_mul_f32_1024x4096": 67108864, "c2_softmax_f16_8192x4096": 134217728,
+                  "c3_layernorm_residual_bf16_16384x4096": 402669568,
+                  "c4_quant_int8_residual_bf16_32768x8192": 1342308352,
+                  "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": 167837696}
+    for name, (cls, fam) in want.items():
+        k = driver.HipKernel.from_file(os.path.join(FIXTURES, name + ".info"))
+        assert (k.operator_type, k.family) == (cls, fam)
+        assert k.kernel_name == name + "_kernel"
+        assert k.algorithmic_bytes == bytes_want[name]
+        assert [t.is_output for t in k.tensors] == sorted(t.is_output for t in k.tensors)   # inputs first
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192.info"))
+    assert k.algorithmic_ops == 2 * 4096 * 8192 * 8192
+
+
+def test_artifacts_have_the_reference_layout(tmp_path):
+    info = os.path.join(FIXTURES, "small_quant_int8_residual_bf16_37x1544.info")
+    out = str(tmp_path / "meta")
+    k = driver.HipKernel.from_file(info, out_dir=out)
+    assert not k.cache_hit
+    name = "small_quant_int8_residual_bf16_37x1544"
+    for ext in (".hsaco", ".json", "_shape_arg.txt", ".hip"):
+        assert os.path.exists(os.path.join(out, name + ext))
+    meta = json.load(open(os.path.join(out, name + ".json")))
+    for key in ("blockIdx.x", "blockIdx.y", "blockIdx.z", "threadIdx.x", "threadIdx.y", "threadIdx.z"):
+        assert isinstance(meta[key], int)
+    assert meta["kernelName"] == name + "_kernel" and meta["is_dynamic"] is False
+    assert (meta["blockIdx.x"], meta["threadIdx.x"]) == (k.grid[0], k.block[0])
+    code = open(os.path.join(out, name + ".hsaco"), "rb").read()
+    assert code[:4] == b"\x7fELF"
+    assert meta["sha256"] == hashlib.sha256(code).hexdigest()          # hashlib as the independent digest
+    # [offset, sizes..., strides...] per kernel argument, inputs then outputs
+    shape_arg = json.load(open(os.path.join(out, name + "_shape_arg.txt")))
+    assert shape_arg == [[0, 37, 1544, 1544, 1], [0, 37, 1544, 1544, 1], [0, 37, 1544, 1544, 1], [0, 37, 1]]
+    # second compile reuses the artifact; a corrupted code object is detected and rebuilt
+    assert driver.HipKernel.from_file(info, out_dir=out).cache_hit
+    with open(os.path.join(out, name + ".hsaco"), "ab") as f:
+        f.write(b"x")
+    assert not driver.HipKernel.from_file(info, out_dir=out).cache_hit
+
+
+def test_math_selection_follows_the_precision_demand():
+    # float16 output: exp and the division by the row sum may use hardware approximations
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f16_33x1000.info")).source
+    assert "akg::fast_exp(" in src and "akg::fast_rcp(" in src and "akg::op_exp(" not in src
+    # float32 output: library-grade exp and exact division (hoisted reciprocal + FMA correction)
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f32_5x77.info")).source
+    assert "akg::op_exp(" in src and "akg::div_uniform(" in src and "fast_" not in src
+    # int8 output: the path into the integer cast is exact
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_quant_int8_residual_bf16_37x1544.info")).source
+    assert "akg::div_uniform(" in src and "fast_" not in src
+    # float32 elementwise chain: device-library tanh
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_ew_tanh_add_mul_f32_8x128.info")).source
+    assert "akg::op_tanh(" in src and "fast_" not in src
+    # AKG_HIP_PRECISE=1 switches every relaxation off
+    os.environ["AKG_HIP_PRECISE"] = "1"
+    try:
+        src = driver.HipKernel(open(os.path.join(FIXTURES, "small_softmax_f16_33x1000.info")).read(), out_dir=None).source
+        assert "fast_" not in src
+    finally:
+        del os.environ["AKG_HIP_PRECISE"]
+
+
+def test_streamed_tensors_use_non_temporal_accesses_broadcast_vectors_do_not():
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_layernorm_residual_bf16_19x520.info")).source
+    loads = re.findall(r"load_chunk<akg::bf16, V, (true|false)>\(in(\d)", src)
+    assert dict((i, nt) for nt, i in loads) == {"0": "true", "1": "false", "2": "false", "3": "true"}
+    assert "store_chunk<akg::bf16, V, true>" in src
+
+
+def test_ragged_shapes_get_guards_and_aligned_shapes_do_not():
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f32_5x77.info")).source
+    assert "akg_ok[j] = akg_cols[j] < COLS;" in src and "akg_row_ok" in src
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "c2_softmax_f16_8192x4096.info")).source
+    assert "akg_ok[j] = true;" in src and "akg_row_ok" not in src
+
+
+def test_elementwise_dimension_folding():
+    # all operands full-size: folded to one flat dimension; a broadcast operand keeps a [rows, cols] view
+    k = driver.HipKernel.from_file(os.path.join(REF_INFO, "fused_sub_add.info"), out_dir=None)
+    assert "constexpr long ROWS = 1L;" in k.source
+    k = driver.HipKernel.from_file(os.path.join(REF_INFO, "Fused_Cast_Mul_fusion_11325474031898152154.info"), out_dir=None)
+    assert k.operator_type == "Broadcast" and k.family == "elementwise"
+
+
+def test_hip_driver_mirrors_the_reference_driver_interface(tmp_path):
+    info = os.path.join(FIXTURES, "small_softmax_f32_5x77.info")
+    d = driver.HipDriver(input_file=info, output_dir=str(tmp_path))
+    assert d.kernel_name == "small_softmax_f32_5x77"
+    k = d.compile()
+    assert os.path.exists(os.path.join(str(tmp_path), "small_softmax_f32_5x77.json"))
+    assert [t.dtype for t in k.tensors] == ["float32", "float32"]
+    with pytest.raises(ValueError):
+        driver.HipDriver(input_file=info, backend="cuda")
+
+
+def test_cli_tool():
+    tool = os.path.join(ROOT, "akg_amd", "akg-hip")
+    info = os.path.join(FIXTURES, "small_softmax_f32_5x77.info")
+    r = subprocess.run([tool, "translate", info], capture_output=True, text=True)
+    assert r.returncode == 0 and "mindspore.reduce_max" in r.stdout
+    r = subprocess.run([tool, "info", info], capture_output=True, text=True)
+    assert r.returncode == 0 and "row_reduce" in r.stdout
+    r = subprocess.run([tool, "emit", os.path.join(REF_INFO, "Fused_Mul_ReduceSum_split_13305325157517622155.info")],
+                       capture_output=True, text=True)
+    assert r.returncode == 1 and "error -4" in r.stderr

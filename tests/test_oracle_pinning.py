@@ -1,0 +1,319 @@
+"""Pins the CPU oracle (oracle/gen_cpu.py C restatement and oracle/np_ref.py) WITHOUT restating its formulas:
+known-answer vectors for the rounding rules, closed forms and library routines for the fused patterns (scipy / torch in
+float64), brute force with exact rational arithmetic on tiny inputs, invariants, and the two independently written
+restatements against each other. The reference repository holds no numeric golden vectors for this path, so these are
+what the mathematics fixes; each check is chosen so that a plausible mistake (truncation instead of round-half-even, a
+dropped epsilon, a transposed operand, int8 products without widening, -inf instead of -FLT_MAX) fails it.
+"""
+import json
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from akg_amd import harness, op_desc
+from oracle import cpu_ref, gen_cpu, np_ref
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FIXTURES = os.path.join(ROOT, "akg_amd", "fixtures")
+
+
+def build_and_run(desc_text, inputs, tmp_path, name=None):
+    """Compile a description with the C restatement and run it; also evaluate the numpy restatement."""
+    desc = json.loads(desc_text)
+    path = os.path.join(str(tmp_path), (name or desc["op"]) + ".info")
+    with open(path, "w", encoding="utf-8") as f:
+        f.write(desc_text)
+    c_out = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    n_out = np_ref.evaluate(desc, inputs)
+    return desc, c_out, n_out
+
+
+# ---------------------------------------------------------------------------------------------------------
+# rounding rules: known-answer vectors
+# ---------------------------------------------------------------------------------------------------------
+BF16_KAT = [  # float32 bits -> bfloat16 bits under round-to-nearest-even
+    (0x3F800000, 0x3F80),  # 1.0
+    (0x3F808000, 0x3F80),  # tie, even mantissa below -> stays
+    (0x3F818000, 0x3F82),  # tie, odd mantissa below -> rounds up to even
+    (0x3F808001, 0x3F81),  # just above the tie
+    (0x3F807FFF, 0x3F80),  # just below the tie
+    (0x7F7FFFFF, 0x7F80),  # FLT_MAX rounds to +inf
+    (0xBF818000, 0xBF82),  # negative tie
+    (0x00000001, 0x0000),  # smallest subnormal -> 0
+    (0x7F800000, 0x7F80),  # inf
+]
+
+
+def test_bf16_round_to_nearest_even_known_answers():
+    bits = np.array([b for b, _ in BF16_KAT], dtype=np.uint32)
+    want = np.array([w for _, w in BF16_KAT], dtype=np.uint16)
+    got_np = np_ref.f32_to_bf16_bits(bits.view(np.float32))
+    got_h = harness.f32_to_bf16_bits(bits.view(np.float32))
+    assert np.array_equal(got_np, want)
+    assert np.array_equal(got_h, want)
+
+
+def test_bf16_cast_in_c_restatement_known_answers(tmp_path):
+    b = op_desc.DescBuilder("kat_cast_bf16")
+    x = b.input([len(BF16_KAT)], "float32")
+    text = b.dumps([b.cast(x, "bfloat16")])
+    bits = np.array([v for v, _ in BF16_KAT], dtype=np.uint32).view(np.float32)
+    _, c_out, n_out = build_and_run(text, [bits], tmp_path)
+    want = np.array([w for _, w in BF16_KAT], dtype=np.uint16)
+    assert np.array_equal(c_out[0], want)
+    assert np.array_equal(n_out[0], want)
+
+
+def test_f16_cast_matches_ieee_half_conversion(tmp_path):
+    # numpy's float32 -> float16 conversion is IEEE round-to-nearest-even; the C restatement converts in software.
+    rng = np.random.default_rng(7)
+    special = np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e6, -1e6, 5.9604645e-08, 2.9802322e-08, 2.98023224e-08 * 1.0000001,
+                        6.097555e-05, 6.1035156e-05, 1.0009765625, 1.00048828125, 1.00146484375, np.inf, -np.inf], dtype=np.float32)
+    x = np.concatenate([special, (rng.standard_normal(4000) * 10 ** rng.uniform(-9, 5, 4000)).astype(np.float32)])
+    b = op_desc.DescBuilder("kat_cast_f16")
+    t = b.input([x.size], "float32")
+    text = b.dumps([b.cast(t, "float16")])
+    _, c_out, n_out = build_and_run(text, [x], tmp_path)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16)
+    assert np.array_equal(c_out[0].view(np.uint16), want.view(np.uint16))
+    assert np.array_equal(n_out[0].view(np.uint16), want.view(np.uint16))
+
+
+def test_float_to_int8_cast_rounds_half_to_even_and_saturates(tmp_path):
+    x = np.array([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 126.5, 127.5, 3.4999, 3.5001, -128.5, -129.5, 1e9, -1e9, 0.49999997],
+                 dtype=np.float32)
+    want = np.array([0, 2, 2, 0, -2, -2, 126, 127, 3, 4, -128, -128, 127, -128, 0], dtype=np.int8)
+    b = op_desc.DescBuilder("kat_cast_i8")
+    t = b.input([x.size], "float32")
+    text = b.dumps([b.cast(t, "int8")])
+    _, c_out, n_out = build_and_run(text, [x], tmp_path)
+    assert np.array_equal(c_out[0], want)      # truncation toward zero would give 0,1,2,0,-1,-2,126,127,...
+    assert np.array_equal(n_out[0], want)
+
+
+def test_reduce_max_starts_from_minus_largest_finite_not_minus_inf(tmp_path):
+    # a row of -inf must reduce to -FLT_MAX (maxnumf(-FLT_MAX, -inf)), not to -inf
+    b = op_desc.DescBuilder("kat_reduce_max_init")
+    t = b.input([2, 4], "float32")
+    text = b.dumps([b.reduce("ReduceMax", t, [1], True)])
+    x = np.array([[-np.inf] * 4, [1.0, 5.0, -2.0, 3.0]], dtype=np.float32)
+    _, c_out, n_out = build_and_run(text, [x], tmp_path)
+    want = np.array([[-np.finfo(np.float32).max], [5.0]], dtype=np.float32)
+    assert np.array_equal(c_out[0], want)
+    assert np.array_equal(n_out[0], want)
+
+
+def test_reduce_sum_accumulates_in_the_declared_narrow_type(tmp_path):
+    # 4096 ones in float16: a float16 accumulator stalls at 2048 (2048 + 1 rounds back to 2048); an accumulator that is
+    # silently widened to float32 would return 4096.
+    b = op_desc.DescBuilder("kat_reduce_sum_f16")
+    t = b.input([1, 4096], "float16")
+    text = b.dumps([b.reduce("ReduceSum", t, [1], True)])
+    x = np.ones((1, 4096), dtype=np.float16)
+    _, c_out, n_out = build_and_run(text, [x], tmp_path)
+    assert float(c_out[0][0, 0]) == 2048.0
+    assert float(n_out[0][0, 0]) == 2048.0
+
+
+# ---------------------------------------------------------------------------------------------------------
+# fused patterns against closed forms / library routines
+# ---------------------------------------------------------------------------------------------------------
+def run_fixture_both(name, seed):
+    path = os.path.join(FIXTURES, name + ".info")
+    desc = harness.load_desc(path)
+    inputs = harness.make_inputs(desc, seed=seed)
+    c_out = cpu_ref.CpuKernel(path)(inputs)
+    n_out = np_ref.evaluate(desc, inputs)
+    return desc, inputs, c_out, n_out
+
+
+def test_elementwise_chain_matches_float64_closed_form():
+    desc, (a, b, c), c_out, n_out = run_fixture_both("small_ew_tanh_add_mul_f32_7x33", 11)
+    want = np.tanh((a.astype(np.float64) + b) * c)
+    for got in (c_out[0], n_out[0]):
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-7)
+    # a dropped or reordered term is far outside this tolerance
+    assert not np.allclose(np.tanh(a.astype(np.float64) + b * c), want, rtol=1e-3, atol=1e-3)
+
+
+def test_softmax_matches_scipy_and_its_invariants():
+    from scipy.special import softmax
+    desc, (x,), c_out, n_out = run_fixture_both("small_softmax_f16_33x1000", 12)
+    want = softmax(x.astype(np.float64), axis=1)
+    for got in (c_out[0], n_out[0]):
+        g = got.astype(np.float64)
+        assert np.allclose(g, want, rtol=2e-3, atol=1e-6)          # float16 output: 2^-11 relative
+        assert np.allclose(g.sum(axis=1), 1.0, atol=2e-3)
+        assert (g >= 0).all()
+    # shift invariance: adding a per-row constant that is exact in float16 changes nothing but rounding
+    shifted = (x.astype(np.float32) + np.float32(2.0)).astype(np.float16)
+    path = os.path.join(FIXTURES, "small_softmax_f16_33x1000.info")
+    again = cpu_ref.CpuKernel(path)([shifted])[0].astype(np.float64)
+    assert np.allclose(again, want, rtol=6e-3, atol=1e-5)
+
+
+def test_softmax_f32_matches_torch_float64():
+    import torch
+    desc, (x,), c_out, n_out = run_fixture_both("small_softmax_f32_5x77", 13)
+    want = torch.softmax(torch.from_numpy(x).double(), dim=1).numpy()
+    assert np.allclose(c_out[0], want, rtol=1e-5, atol=1e-9)
+    assert np.allclose(n_out[0], want, rtol=1e-5, atol=1e-9)
+
+
+def test_layernorm_residual_matches_torch_float64_and_invariants():
+    import torch
+    desc, (x, g, be, r), c_out, n_out = run_fixture_both("small_layernorm_residual_bf16_19x520", 14)
+    xf, gf, bf, rf = (torch.from_numpy(harness.bf16_bits_to_f32(t)).double() for t in (x, g, be, r))
+    want = (torch.nn.functional.layer_norm(xf, (520,), gf, bf, eps=1e-5) + rf).numpy()
+    for got in (c_out[0], n_out[0]):
+        gotf = harness.bf16_bits_to_f32(got).astype(np.float64)
+        assert np.allclose(gotf, want, rtol=8e-3, atol=1e-6)        # bfloat16 output: 2^-8 relative
+        # undo the affine part: rows must have mean ~0 and variance ~1
+        z = (gotf - rf.numpy() - bf.numpy()) / gf.numpy()
+        assert np.abs(z.mean(axis=1)).max() < 2e-2
+        assert np.abs(z.var(axis=1) - 1.0).max() < 3e-2
+    wrong_unbiased = torch.nn.functional.layer_norm(xf, (520,), gf, bf, eps=1e-5)
+    assert not np.allclose(wrong_unbiased.numpy(), want, rtol=1e-2, atol=1e-2)   # dropping the residual is visible
+
+
+def test_layernorm_float32_against_float64_tight(tmp_path):
+    # the same pattern in float32 end to end, where a wrong epsilon or an N-1 divisor shows at 1e-6
+    import torch
+    text = op_desc.layernorm_residual(6, 64, "float32", eps=1e-5, name="ln_f32_6x64")
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((6, 64)).astype(np.float32) * 1e-2     # small variance: epsilon matters
+    g = rng.uniform(0.5, 1.5, 64).astype(np.float32)
+    be = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    r = rng.standard_normal((6, 64)).astype(np.float32)
+    _, c_out, n_out = build_and_run(text, [x, g, be, r], tmp_path)
+    t = lambda a: torch.from_numpy(a).double()
+    want = (torch.nn.functional.layer_norm(t(x), (64,), t(g), t(be), eps=1e-5) + t(r)).numpy()
+    assert np.allclose(c_out[0], want, rtol=2e-6, atol=2e-6)
+    assert np.allclose(n_out[0], want, rtol=2e-6, atol=2e-6)
+    no_eps = (torch.nn.functional.layer_norm(t(x), (64,), t(g), t(be), eps=0.0) + t(r)).numpy()
+    assert not np.allclose(no_eps, want, rtol=1e-4, atol=1e-4)
+    unbiased = ((t(x) - t(x).mean(1, keepdim=True)) / (t(x).var(1, unbiased=True, keepdim=True) + 1e-5).sqrt() * t(g) + t(be) + t(r)).numpy()
+    assert not np.allclose(unbiased, want, rtol=1e-4, atol=1e-4)
+
+
+def correctly_rounded_f32(fr):
+    """Nearest float32 (ties to even) of an exact Fraction, by comparing against the neighbours' midpoints."""
+    approx = np.float32(float(fr))
+    cands = [np.nextafter(approx, np.float32(-np.inf)), approx, np.nextafter(approx, np.float32(np.inf))]
+    best = min(cands, key=lambda c: (abs(Fraction(float(c)) - fr), int(np.float32(c).view(np.uint32)) & 1))
+    return np.float32(best)
+
+
+def test_quant_brute_force_with_exact_rationals(tmp_path):
+    # tiny case, every quantity recomputed with exact rational arithmetic + explicit correct rounding
+    rows, cols = 3, 8
+    text = op_desc.quant_int8_residual(rows, cols, "bfloat16", name="quant_tiny")
+    rng = np.random.default_rng(5)
+    x = harness.f32_to_bf16_bits(rng.standard_normal((rows, cols)).astype(np.float32) * 3)
+    r = harness.f32_to_bf16_bits(rng.standard_normal((rows, cols)).astype(np.float32))
+    x[0, 0] = harness.f32_to_bf16_bits(np.array([50.0], dtype=np.float32))[0]        # an outlier
+    _, c_out, n_out = build_and_run(text, [x, r], tmp_path)
+    xf, rf = harness.bf16_bits_to_f32(x), harness.bf16_bits_to_f32(r)
+    for i in range(rows):
+        s = [correctly_rounded_f32(Fraction(float(xf[i, j])) + Fraction(float(rf[i, j]))) for j in range(cols)]
+        amax = max(abs(Fraction(float(v))) for v in s)
+        scale = correctly_rounded_f32(amax / 127)
+        assert c_out[1][i] == scale and n_out[1][i] == scale
+        for j in range(cols):
+            q = correctly_rounded_f32(Fraction(float(s[j])) / Fraction(float(scale)))
+            q = min(max(Fraction(float(q)), Fraction(-127)), Fraction(127))
+            fl = q.numerator // q.denominator
+            rem = q - fl
+            n = fl + 1 if (rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1)) else fl
+            assert int(c_out[0][i, j]) == n, (i, j)
+            assert int(n_out[0][i, j]) == n, (i, j)
+
+
+def test_quant_invariants_full_row_width():
+    desc, (x, r), c_out, n_out = run_fixture_both("small_quant_int8_residual_bf16_64x8192", 15)
+    assert np.array_equal(c_out[0], n_out[0]) and np.array_equal(c_out[1], n_out[1])
+    q, scale = c_out
+    s = harness.bf16_bits_to_f32(x) + harness.bf16_bits_to_f32(r)
+    assert np.array_equal(np.abs(q.astype(np.int32)).max(axis=1), np.full(64, 127))      # absmax maps to +-127
+    assert np.allclose(scale, np.abs(s).max(axis=1) / np.float32(127.0), rtol=1e-7)
+    # dequantised value within half a step (plus division rounding) of the source
+    assert (np.abs(q.astype(np.float64) * scale[:, None] - s) <= scale[:, None] * 0.5000001).all()
+
+
+def test_int8_matmul_is_exact_integer_arithmetic(tmp_path):
+    # brute force with Python integers on a tiny case whose products overflow int8 and int16
+    b = op_desc.DescBuilder("mm_tiny")
+    a_t = b.input([3, 5], "int8")
+    b_t = b.input([5, 4], "int8")
+    text = b.dumps([b.matmul(a_t, b_t, "int32")])
+    a = np.array([[127, -127, 100, -100, 77], [1, 2, 3, 4, 5], [-128, -128, -128, -128, -128]], dtype=np.int8)
+    bm = np.array([[127, 1, -1, 0], [-127, 2, -2, 0], [100, 3, -3, 0], [-100, 4, -4, 0], [77, 5, -5, 127]], dtype=np.int8)
+    _, c_out, n_out = build_and_run(text, [a, bm], tmp_path)
+    want = [[sum(int(a[i, k]) * int(bm[k, j]) for k in range(5)) for j in range(4)] for i in range(3)]
+    assert c_out[0].tolist() == want
+    assert n_out[0].tolist() == want
+    assert want[0][0] == 127 * 127 + 127 * 127 + 100 * 100 + 100 * 100 + 77 * 77     # no narrow-type wraparound
+
+
+def test_matmul_transpose_b_reads_b_as_n_by_k(tmp_path):
+    b = op_desc.DescBuilder("mm_tb")
+    a_t = b.input([2, 3], "int8")
+    b_t = b.input([4, 3], "int8")
+    text = b.dumps([b.matmul(a_t, b_t, "int32", transpose_b=True)])
+    a = np.array([[1, 2, 3], [4, 5, 6]], dtype=np.int8)
+    bt = np.array([[1, 0, 0], [0, 1, 0], [0, 0, 1], [1, 1, 1]], dtype=np.int8)
+    _, c_out, n_out = build_and_run(text, [a, bt], tmp_path)
+    want = (a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.int32)
+    assert np.array_equal(c_out[0], want) and np.array_equal(n_out[0], want)
+
+
+def test_gemm_dequant_bias_gelu_matches_torch_float64():
+    import torch
+    desc, (a, sa, w, sb, bias), c_out, n_out = run_fixture_both("small_gemm_i8_dequant_bias_gelu_256x512x256", 16)
+    acc = torch.from_numpy(a).long() @ torch.from_numpy(w).long()
+    x = acc.double() * torch.from_numpy(sa).double() * torch.from_numpy(sb).double() + \
+        torch.from_numpy(harness.bf16_bits_to_f32(bias)).double()
+    want = torch.nn.functional.gelu(x, approximate="tanh").numpy()
+    for got in (c_out[0], n_out[0]):
+        g = harness.bf16_bits_to_f32(got).astype(np.float64)
+        assert np.allclose(g, want, rtol=8e-3, atol=1e-3)
+    # per-row vs per-column scale mix-up would be visible
+    wrong = torch.nn.functional.gelu(acc.double() * torch.from_numpy(sa).double().T * torch.from_numpy(sb).double()[:, None]
+                                     + torch.from_numpy(harness.bf16_bits_to_f32(bias)).double(), approximate="tanh").numpy()
+    assert not np.allclose(wrong, want, rtol=5e-2, atol=5e-2)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# the two restatements against each other on every small fixture
+# ---------------------------------------------------------------------------------------------------------
+SMALL = sorted(f[:-5] for f in os.listdir(FIXTURES) if f.startswith("small_") and f.endswith(".info"))
+
+
+@pytest.mark.parametrize("name", SMALL)
+def test_c_and_numpy_restatements_agree(name):
+    desc, inputs, c_out, n_out = run_fixture_both(name, 21)
+    for d, a, b in zip(desc["output_desc"], c_out, n_out):
+        ok, msg = harness.compare(a, b, d["data_type"])
+        assert ok, "%s %s: %s" % (name, d["tensor_name"], msg)
+        if name.startswith("small_quant") or name.startswith("small_layernorm"):
+            # no transcendental function involved: the two must agree bit for bit
+            assert np.array_equal(a, b)
+
+
+def test_openmp_build_is_bit_identical_to_serial():
+    path = os.path.join(FIXTURES, "small_layernorm_residual_bf16_64x4096.info")
+    inputs = harness.make_inputs(harness.load_desc(path), seed=22)
+    serial = cpu_ref.CpuKernel(path)(inputs)
+    par = cpu_ref.CpuKernel(path, openmp=True)(inputs)
+    assert np.array_equal(serial[0], par[0])
+
+
+def test_generated_c_uses_the_packed_pointer_abi():
+    with open(os.path.join(FIXTURES, "small_quant_int8_residual_bf16_37x1544.info"), "r", encoding="utf-8") as f:
+        src = gen_cpu.generate_c(json.load(f))
+    assert "void small_quant_int8_residual_bf16_37x1544(void **packed)" in src
+    # inputs first, then outputs
+    assert src.index("packed[0]") < src.index("packed[1]") < src.index("packed[2]") < src.index("packed[3]")
