@@ -50,7 +50,7 @@ class GemmEmitter {
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
     note << "gemm_epilogue M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
-         << " tile=256x256x64 mfma=i32_32x32x32_i8 waves=" << wavesM() << "x2 grid=" << k.grid[0];
+         << " tile=256x256x" << stepK() << " mfma=i32_32x32x32_i8 waves=" << wavesM() << "x2 grid=" << k.grid[0];
     k.scheduleNote = note.str();
     return k;
   }
@@ -68,7 +68,9 @@ class GemmEmitter {
   std::ostringstream members_, prepare_, apply_;
 
   // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_GEMM_VARIANT=1.
-  int wavesM() const { return opt_.gemmVariant == 1 ? 2 : 4; }
+  int wavesM() const { return (opt_.gemmVariant & 1) ? 2 : 4; }
+  // K extent of one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
+  int stepK() const { return (opt_.gemmVariant & 2) ? 64 : 128; }
 
   void analyse() {
     for (size_t i = 0; i < g_.ops.size(); ++i) {
@@ -287,7 +289,7 @@ class GemmEmitter {
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
     src_ << "  akg::gemm_i8_256x256<" << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ", " << wavesM() << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
+         << ", " << wavesM() << ", " << stepK() << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
   }
 };
 

@@ -31,13 +31,21 @@ namespace akg {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
+#ifdef AKG_GEMM_STRICT_ORDER
+#define AKG_GEMM_PIN __builtin_amdgcn_sched_barrier(0)
+#else
+#define AKG_GEMM_PIN
+#endif
+
 constexpr int kGemmBM = 256;
 constexpr int kGemmBN = 256;
-constexpr int kGemmBK = 64;
-constexpr int kGemmPitch = 80;  // bytes per LDS row: 64 data + 16 pad
-constexpr int kGemmThreads = 256;
 constexpr int kGemmXcds = 8;
 constexpr int kGemmGroupRows = 8;  // tile-rows per group in the swizzled walk
+
+template <bool B>
+struct BoolTag {
+  static constexpr bool value = B;
+};
 
 // 4 x 4 byte transpose: in r[i] byte j  ->  out t[j] byte i.
 AKG_DEV void transpose4x4_bytes(const u32 (&r)[4], u32 (&t)[4]) {
@@ -60,22 +68,29 @@ constexpr long gemm_i8_grid(long m, long n) {
 // WAVES_M x 2 wavefronts per workgroup: 2 x 2 (one wavefront per SIMD, 128 x 128 per wavefront, 256 accumulator
 // registers) or 4 x 2 (two wavefronts per SIMD, 64 x 128 per wavefront, 128 accumulator registers: the second
 // wavefront's MFMAs cover the first one's loads, transposes and barriers).
-template <long M, long N, long K, bool TRANSB, int WAVES_M, typename Epilogue>
+// BK = K extent of one step: 64 or 128. With 128 every row of A contributes one full 128-byte cache line per step
+// (with 64 each line is fetched from L2 twice), there are half as many barriers, and LDS holds 2 x 72 KiB.
+template <long M, long N, long K, bool TRANSB, int WAVES_M, int BK, typename Epilogue>
 AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B, Epilogue &epi) {
   static_assert(K % 16 == 0, "K must be a multiple of 16");
   static_assert(TRANSB || (N % 4 == 0), "N must be a multiple of 4");
   static_assert(WAVES_M == 2 || WAVES_M == 4, "2 x 2 or 4 x 2 wavefronts");
-  constexpr int kWaves = WAVES_M * 2;
-  constexpr int kThreads = kWaves * 64;
+  static_assert(BK == 64 || BK == 128, "K step of 64 or 128");
+  constexpr int kPitch = BK + 16;                     // LDS row: BK data bytes + 16 pad (odd multiple of 16)
+  constexpr int kSub = BK / 32;                       // MFMA k-substeps per step (2 or 4)
+  constexpr int kChunksPerRow = BK / 16;              // 16-byte chunks per row of a K-contiguous operand tile
+  constexpr int kRowChunks = BK / 16;                 // chunks per staging thread (256 rows * BK/16 / 256 threads)
+  constexpr int kRowStep = 256 / kChunksPerRow;       // rows between two chunks of one thread
+  constexpr int kBlockRows = BK / 4;                  // k-rows of B per staging thread (16 or 32)
   constexpr int kTM = kGemmBM / (32 * WAVES_M);       // MFMA row tiles per wavefront
   constexpr int kWaveRows = kGemmBM / WAVES_M;
   constexpr long kTilesM = (M + kGemmBM - 1) / kGemmBM;
   constexpr long kTilesN = (N + kGemmBN - 1) / kGemmBN;
   constexpr long kTiles = kTilesM * kTilesN;
   constexpr long kPerXcd = (kTiles + kGemmXcds - 1) / kGemmXcds;
-  constexpr long kSteps = (K + kGemmBK - 1) / kGemmBK;
-  constexpr bool kFull = (M % kGemmBM == 0) && (N % kGemmBN == 0) && (K % kGemmBK == 0);
-  constexpr int kTileBytes = kGemmBM * kGemmPitch;  // one operand tile in LDS
+  constexpr long kSteps = (K + BK - 1) / BK;
+  constexpr bool kFull = (M % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
+  constexpr int kTileBytes = kGemmBM * kPitch;        // one operand tile in LDS
 
   __shared__ __attribute__((aligned(16))) u8 lds[2][2][kTileBytes];  // [buffer][A|B]
 
@@ -109,112 +124,154 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
     }
   }
 
-  // ---- staging registers (one K step ahead of LDS, two ahead of the MFMAs)
-  // 2 x 2 wavefronts: every thread stages 4 chunks of A and a 16 x 4 block of B.
-  // 4 x 2 wavefronts: wavefronts 0..3 stage all of B (16 x 4 blocks, 128-bit LDS writes stay conflict free),
-  //                   wavefronts 4..7 stage all of A.
+  // ---- staging registers: the tile of step s+1 travels memory -> registers during step s-1.. s and is written to
+  // LDS at the top of step s.
+  // 2 x 2 wavefronts: every thread stages its share of A (x) and of B (y).
+  // 4 x 2 wavefronts: wavefronts 0..3 stage all of B, wavefronts 4..7 all of A, both in x (the 128-bit LDS writes of
+  //                   the transposed B blocks stay conflict free this way, and x is the only staging array).
   constexpr bool kSplitDuty = (WAVES_M == 4);
-  v4i ga[4];
-  u32 gb[16];   // !TRANSB: 16 k-rows x 4 columns
-  v4i gbt[4];   // TRANSB: like A
+  struct Stage {
+    v4i x[kRowChunks];
+    v4i y[kSplitDuty ? 1 : kRowChunks];
+  };
+  Stage stage;
 
   const int ltid = tid & 255;
   const bool stageA = !kSplitDuty || tid >= 256;
-  const bool stageB = !kSplitDuty || tid < 256;
-  const int aRow = ltid >> 2;   // + 64 * i
-  const int aChunk = ltid & 3;
+  const int aRow = ltid / kChunksPerRow;   // + kRowStep * i
+  const int aChunk = ltid % kChunksPerRow;
   const int bN4 = ltid & 63;
   const int bKq = ltid >> 6;
 
-  const s8 *aSrc = A + (m0 + aRow) * K + aChunk * 16;
-  const s8 *bSrc = TRANSB ? (B + (n0 + aRow) * K + aChunk * 16) : (B + (bKq * 16) * N + n0 + 4 * bN4);
+  // Global loads are buffer loads: the per-lane offset is computed once, everything that changes from load to load
+  // (row block, k-row, K step) is a scalar offset, so the loop spends no vector instructions on addresses (vector
+  // instructions and MFMAs compete for issue cycles). Out-of-range lanes read zero through the descriptor's size.
+  static_assert(M * K < (1L << 31) && N * K < (1L << 31), "operand too large for 32-bit buffer offsets");
+  const __amdgpu_buffer_rsrc_t aRsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<s8 *>(A), 0, static_cast<int>(M * K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t bRsrc = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<s8 *>(B), 0, static_cast<int>(N * K), 0x00020000);
+  const int aVoff = static_cast<int>((m0 + aRow) * K + aChunk * 16);
+  const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
+                           : static_cast<int>((bKq * kBlockRows) * N + n0 + 4 * bN4);
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-  auto loadGlobal = [&](long step) {
-    const long k0 = step * kGemmBK;
-    if (stageA) {
+  auto loadRows = [&](__amdgpu_buffer_rsrc_t rsrc, int voff, long rowBase, long rowLimit, long k0,
+                      v4i (&dst)[kRowChunks]) {
+    // kRowChunks chunks of 16 consecutive k, rows rowBase + kRowStep * i of a K-contiguous operand
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (kFull || (m0 + aRow + 64 * i < M && k0 + aChunk * 16 < K)) {
-          ga[i] = *reinterpret_cast<const v4i *>(aSrc + (64 * i) * K + k0);
-        } else {
-          ga[i] = v4i{0, 0, 0, 0};
-        }
+    for (int i = 0; i < kRowChunks; ++i) {
+      if (kFull || (rowBase + kRowStep * i < rowLimit && k0 + aChunk * 16 < K)) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, static_cast<int>((kRowStep * i) * K + k0), 0);
+        dst[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
+      } else {
+        dst[i] = v4i{0, 0, 0, 0};
       }
     }
-    if (stageB) {
-      if constexpr (TRANSB) {
+  };
+  auto loadBlock = [&](long k0, v4i (&dst)[kRowChunks]) {
+    // kBlockRows k-rows x 4 columns of row-major B, one dword per k-row
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if (kFull || (n0 + aRow + 64 * i < N && k0 + aChunk * 16 < K)) {
-            gbt[i] = *reinterpret_cast<const v4i *>(bSrc + (64 * i) * K + k0);
-          } else {
-            gbt[i] = v4i{0, 0, 0, 0};
-          }
-        }
+    for (int i = 0; i < kBlockRows; ++i) {
+      u32 v = 0u;
+      if (kFull || (n0 + 4 * bN4 < N && k0 + bKq * kBlockRows + i < K)) {
+        v = __builtin_amdgcn_raw_buffer_load_b32(bRsrc, bVoff, static_cast<int>((k0 + i) * N), 0);
+      }
+      dst[i >> 2][i & 3] = static_cast<int>(v);
+    }
+  };
+  auto loadGlobal = [&](long step, Stage &st) {
+    const long k0 = step * BK;
+    if constexpr (kSplitDuty) {
+      if (stageA) {
+        loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
+      } else if constexpr (TRANSB) {
+        loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.x);
       } else {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          if (kFull || (n0 + 4 * bN4 < N && k0 + bKq * 16 + i < K)) {
-            gb[i] = *reinterpret_cast<const u32 *>(bSrc + (k0 + i) * N);
-          } else {
-            gb[i] = 0u;
-          }
-        }
+        loadBlock(k0, st.x);
+      }
+    } else {
+      loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
+      if constexpr (TRANSB) {
+        loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.y);
+      } else {
+        loadBlock(k0, st.y);
       }
     }
   };
 
-  auto storeLds = [&](int buf) {
-    u8 *la = lds[buf][0];
-    u8 *lb = lds[buf][1];
-    if (stageA) {
+  auto storeRowsA = [&](u8 *la, const v4i (&src)[kRowChunks]) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        *reinterpret_cast<v4i *>(la + (aRow + 64 * i) * kGemmPitch + aChunk * 16) = ga[i];
+    for (int i = 0; i < kRowChunks; ++i) {
+      *reinterpret_cast<v4i *>(la + (aRow + kRowStep * i) * kPitch + aChunk * 16) = src[i];
+    }
+  };
+  auto storeRowsBt = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
+#pragma unroll
+    for (int i = 0; i < kRowChunks; ++i) {
+      const int col = aRow + kRowStep * i;           // column of the tile
+      const int r = (col & 3) * 64 + (col >> 2);     // its LDS row
+      *reinterpret_cast<v4i *>(lb + r * kPitch + aChunk * 16) = src[i];
+    }
+  };
+  auto storeBlockB = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
+    // src[g] = 4 k-rows x 4 columns; after the byte transpose t[g][j] = 4 consecutive k of column j
+    u32 t[kRowChunks][4];
+#pragma unroll
+    for (int g = 0; g < kRowChunks; ++g) {
+      const u32 rows[4] = {static_cast<u32>(src[g][0]), static_cast<u32>(src[g][1]), static_cast<u32>(src[g][2]),
+                           static_cast<u32>(src[g][3])};
+      transpose4x4_bytes(rows, t[g]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int h = 0; h < kRowChunks / 4; ++h) {
+        v4i w;
+        w[0] = static_cast<int>(t[4 * h + 0][j]);
+        w[1] = static_cast<int>(t[4 * h + 1][j]);
+        w[2] = static_cast<int>(t[4 * h + 2][j]);
+        w[3] = static_cast<int>(t[4 * h + 3][j]);
+        *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * kBlockRows + h * 16) = w;
       }
     }
-    if (stageB) {
-      if constexpr (TRANSB) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int col = aRow + 64 * i;                 // column of the tile
-          const int r = (col & 3) * 64 + (col >> 2);     // its LDS row
-          *reinterpret_cast<v4i *>(lb + r * kGemmPitch + aChunk * 16) = gbt[i];
-        }
+  };
+  auto storeLds = [&](int buf, const Stage &st) {
+    u8 *la = lds[buf][0];
+    u8 *lb = lds[buf][1];
+    if constexpr (kSplitDuty) {
+      if (stageA) {
+        storeRowsA(la, st.x);
+      } else if constexpr (TRANSB) {
+        storeRowsBt(lb, st.x);
       } else {
-        u32 t[4][4];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const u32 rows[4] = {gb[4 * g], gb[4 * g + 1], gb[4 * g + 2], gb[4 * g + 3]};
-          transpose4x4_bytes(rows, t[g]);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          v4i w;
-          w[0] = static_cast<int>(t[0][j]);
-          w[1] = static_cast<int>(t[1][j]);
-          w[2] = static_cast<int>(t[2][j]);
-          w[3] = static_cast<int>(t[3][j]);
-          *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kGemmPitch + bKq * 16) = w;
-        }
+        storeBlockB(lb, st.x);
+      }
+    } else {
+      storeRowsA(la, st.x);
+      if constexpr (TRANSB) {
+        storeRowsBt(lb, st.y);
+      } else {
+        storeBlockB(lb, st.y);
       }
     }
   };
 
   const int fragRow = lane & 31;
   const int fragHalf = (lane >> 5) * 16;
-  const int aFragOff = (wm * kWaveRows + fragRow) * kGemmPitch + fragHalf;
-  const int bFragOff = (wn * 32 + fragRow) * kGemmPitch + fragHalf;
+  const int aFragOff = (wm * kWaveRows + fragRow) * kPitch + fragHalf;
+  const int bFragOff = (wn * 32 + fragRow) * kPitch + fragHalf;
 
   auto readFrags = [&](int buf, int ks, v4i (&af)[kTM], v4i (&bf)[4]) {
     const u8 *la = lds[buf][0] + aFragOff + ks * 32;
     const u8 *lb = lds[buf][1] + bFragOff + ks * 32;
 #pragma unroll
-    for (int i = 0; i < kTM; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 32 * kGemmPitch);
+    for (int i = 0; i < kTM; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 32 * kPitch);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 64 * kGemmPitch);
+    for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 64 * kPitch);
   };
   auto mfmaAll = [&](const v4i (&af)[kTM], const v4i (&bf)[4]) {
+#ifndef AKG_DIAG_NO_MFMA
 #pragma unroll
     for (int i = 0; i < kTM; ++i) {
 #pragma unroll
@@ -222,50 +279,102 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
         acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
       }
     }
+#endif
   };
 
-  // ---- main loop. Invariant at the top of step s: LDS buffer s&1 holds tile s (complete), the staging registers
-  // hold tile s+1, and f0 holds the fragments of the first half (k 0..31) of tile s.
-  //   a. staged tile s+1 -> LDS buffer (s+1)&1        (its last readers finished before the previous barrier)
+  // ---- main loop. Invariant at the top of step s: LDS buffer s&1 holds tile s (complete), the staging registers hold
+  // tile s+1 (possibly still in flight), and f0 holds the fragments of the first 32 k of tile s.
+  //   a. staged tile s+1 -> LDS buffer (s+1)&1      (its last readers finished before the previous barrier)
   //   b. issue the global loads of tile s+2 into the staging registers
-  //   c. read the second-half fragments f1 of tile s
-  //   d. MFMAs on f0
-  //   e. barrier: everybody has read tile s completely and has written tile s+1
-  //   f. read the first-half fragments of tile s+1     (its latency hides behind the MFMAs of g)
-  //   g. MFMAs on f1
+  //   c. for every k-substep but the last: read the next substep's fragments, MFMAs on the current ones
+  //   d. barrier: everybody has read tile s completely and has written tile s+1
+  //   e. read the first fragments of tile s+1         (their latency hides behind the MFMAs of f)
+  //   f. MFMAs on the last substep's fragments
   v4i f0a[kTM], f0b[4], f1a[kTM], f1b[4];
-  loadGlobal(0);
-  storeLds(0);
-  if (kSteps > 1) loadGlobal(1);
-  __syncthreads();
-  readFrags(0, 0, f0a, f0b);
-  for (long step = 0; step < kSteps; ++step) {
+  // One K step. kStore / kLoad are compile-time so that the steady-state loop body is a single basic block (the
+  // last two steps, which have nothing left to store or load, are peeled off below).
+  auto stepBody = [&](long step, auto storeTag, auto loadTag) {
+    constexpr bool kStore = decltype(storeTag)::value;
+    constexpr bool kLoad = decltype(loadTag)::value;
     const int buf = static_cast<int>(step & 1);
+    // ---- first half: MFMAs on the fragments already in registers; meanwhile fetch the next fragments and move the
+    // staged tile (transposing B) into the other LDS buffer
+#pragma unroll
+    for (int ks = 0; ks + 2 < kSub; ks += 2) {
+      readFrags(buf, ks + 1, f1a, f1b);
+      mfmaAll(f0a, f0b);
+      readFrags(buf, ks + 2, f0a, f0b);
+      mfmaAll(f1a, f1b);
+    }
+    readFrags(buf, kSub - 1, f1a, f1b);
 #ifndef AKG_DIAG_NO_LDS_STORE
-    if (step + 1 < kSteps) storeLds(buf ^ 1);
+    if constexpr (kStore) storeLds(buf ^ 1, stage);
 #endif
-#ifndef AKG_DIAG_NO_GLOBAL_LOAD
-    if (step + 2 < kSteps) loadGlobal(step + 2);
-#endif
-    // Keep the global loads here: left to itself the scheduler sinks them to the end of the step (shorter live
-    // ranges), which exposes the full memory latency at the top of the next step.
-    __builtin_amdgcn_sched_barrier(0);
-#ifndef AKG_DIAG_NO_FRAG_READ
-    readFrags(buf, 1, f1a, f1b);
-#endif
-#ifndef AKG_DIAG_NO_MFMA
     mfmaAll(f0a, f0b);
-#endif
+    if constexpr (!kSplitDuty && kSub == 2 && kStore && !TRANSB) {
+      // Issue order inside the half step (one wavefront per SIMD: nothing else hides latencies). kTM * 4 = 16 MFMAs:
+      //   MFMA 0..7   each followed by one fragment read (ds_read_b128)
+      //   MFMA 8..11  each followed by one A-tile LDS write and 8 of the 32 byte-transpose permutes
+      //   MFMA 12..15 each followed by one B-tile LDS write
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      }
+    }
 #ifndef AKG_DIAG_NO_BARRIER
     __syncthreads();
 #endif
-#ifndef AKG_DIAG_NO_FRAG_READ
-    if (step + 1 < kSteps) readFrags(buf ^ 1, 0, f0a, f0b);
+    // ---- second half: MFMAs on the last fragments of this tile; meanwhile fetch the first fragments of the next
+    // tile and issue the global loads of the tile after it into the (now free) staging registers
+    if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
+#ifndef AKG_DIAG_NO_GLOBAL_LOAD
+    if constexpr (kLoad) loadGlobal(step + 2, stage);
 #endif
-#ifndef AKG_DIAG_NO_MFMA
     mfmaAll(f1a, f1b);
-#endif
+    if constexpr (!kSplitDuty && kSub == 2 && kLoad && !TRANSB) {
+      //   MFMA 0..7   each followed by one fragment read
+      //   MFMA 8..15  each followed by 2-3 of the 20 global loads (4 x 128-bit of A, 16 x 32-bit of B)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 3, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+      }
+    }
+  };
+  loadGlobal(0, stage);
+  storeLds(0, stage);
+  if (kSteps > 1) loadGlobal(1, stage);
+  __syncthreads();
+  readFrags(0, 0, f0a, f0b);
+  long step = 0;
+  for (; step + 2 < kSteps; ++step) stepBody(step, BoolTag<true>(), BoolTag<true>());
+  if (step + 1 < kSteps) {
+    stepBody(step, BoolTag<true>(), BoolTag<false>());
+    ++step;
   }
+  stepBody(step, BoolTag<false>(), BoolTag<false>());
 
   // ---- epilogue: lane owns columns col4 .. col4+3 of 16 * kTM rows
   const long col4 = n0 + 4 * (wn * 32 + fragRow);
