@@ -447,6 +447,13 @@ class TileEmitter {
   int reduceCount_ = 0;
   bool nonTemporal_ = true;
   std::vector<bool> relaxed_;
+  // clamp + integer-cast peephole: ops skipped because a later Cast absorbs them, and what each such Cast computes
+  struct ClampCast {
+    int source = -1;
+    double lo = 0.0, hi = 0.0;
+  };
+  std::vector<bool> absorbed_;            // per op
+  std::vector<ClampCast> clampCast_;      // per op (source < 0: none)
 
   // ------------------------------------------------------------------ analysis
   void analyse() {
@@ -645,6 +652,64 @@ class TileEmitter {
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
   }
 
+  // ------------------------------------------------------------------ peepholes
+  // Cast_to_int8/int16(Minimum(Maximum(x, c0), c1)) (either order) with constant bounds and single-use intermediates
+  // becomes one clamp_cast: 5 vector instructions instead of 11 on the per-token quantisation path.
+  void planPeepholes() {
+    absorbed_.assign(g_.ops.size(), false);
+    clampCast_.assign(g_.ops.size(), ClampCast());
+    std::vector<int> uses(g_.tensors.size(), 0);
+    for (const OpNode &op : g_.ops) {
+      for (int in : op.inputs) ++uses[static_cast<size_t>(in)];
+    }
+    auto constOperand = [&](const OpNode &op, int *other, double *value) {
+      if (op.inputs.size() != 2) return false;
+      for (int side = 0; side < 2; ++side) {
+        const TensorValue &c = g_.tensor(op.inputs[static_cast<size_t>(side)]);
+        if (c.isConst && c.dtype == DType::F32) {
+          *other = op.inputs[static_cast<size_t>(1 - side)];
+          *value = static_cast<double>(static_cast<float>(c.constValue));
+          return true;
+        }
+      }
+      return false;
+    };
+    auto fusable = [&](int tensorId) {
+      const TensorValue &t = g_.tensor(tensorId);
+      return t.producer >= 0 && t.outputIndex < 0 && uses[static_cast<size_t>(tensorId)] == 1 && t.dtype == DType::F32;
+    };
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      const OpNode &cast = g_.ops[k];
+      if (cast.kind != OpKind::Cast || cast.inputs.size() != 1) continue;
+      const DType od = g_.tensor(cast.outputs[0]).dtype;
+      if (od != DType::I8 && od != DType::I16) continue;
+      const int t1 = cast.inputs[0];
+      if (!fusable(t1)) continue;
+      const OpNode &p1 = g_.ops[static_cast<size_t>(g_.tensor(t1).producer)];
+      if (p1.kind != OpKind::Minimum && p1.kind != OpKind::Maximum) continue;
+      int t0 = -1, x = -1;
+      double c1 = 0.0, c0 = 0.0;
+      if (!constOperand(p1, &t0, &c1) || !fusable(t0)) continue;
+      const OpNode &p0 = g_.ops[static_cast<size_t>(g_.tensor(t0).producer)];
+      if ((p0.kind != OpKind::Minimum && p0.kind != OpKind::Maximum) || p0.kind == p1.kind) continue;
+      if (!constOperand(p0, &x, &c0)) continue;
+      if (g_.tensor(x).dtype != DType::F32 || c0 != c0 || c1 != c1) continue;
+      double lo = (p0.kind == OpKind::Maximum) ? c0 : c1;
+      double hi = (p0.kind == OpKind::Minimum) ? c0 : c1;
+      if (lo > hi) continue;  // min(max(x, lo), hi) and max(min(x, hi), lo) differ then: leave it alone
+      const double tlo = (od == DType::I8) ? -128.0 : -32768.0;
+      const double thi = (od == DType::I8) ? 127.0 : 32767.0;
+      lo = std::max(std::nearbyint(lo), tlo);
+      hi = std::min(std::nearbyint(hi), thi);
+      if (lo > hi) continue;
+      absorbed_[static_cast<size_t>(g_.tensor(t1).producer)] = true;
+      absorbed_[static_cast<size_t>(g_.tensor(t0).producer)] = true;
+      clampCast_[k].source = x;
+      clampCast_[k].lo = lo;
+      clampCast_[k].hi = hi;
+    }
+  }
+
   // ------------------------------------------------------------------ emission helpers
   std::string ctOf(int tensorId) const { return computeTypeName(g_.tensor(tensorId).dtype); }
   std::string tagOf(int tensorId) const { return dtypeTag(g_.tensor(tensorId).dtype); }
@@ -697,6 +762,7 @@ class TileEmitter {
   void emit() {
     vals_.assign(g_.tensors.size(), ValInfo());
     relaxed_ = lowering::relaxedPrecisionTensors(g_);
+    planPeepholes();
     const std::string kname = g_.name + "_kernel";
 
     line("// Generated by the akg HIP lowering for gfx950. Op description: " + g_.name);
@@ -778,11 +844,13 @@ class TileEmitter {
       v.ident = lowering::literalFor(tv.dtype, tv.constValue);
     }
     // ops in description order
-    for (const OpNode &op : g_.ops) {
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      const OpNode &op = g_.ops[k];
+      if (absorbed_[k]) continue;
       if (lowering::isReduceKind(op.kind)) {
         emitReduce(op);
       } else {
-        emitElementwise(op);
+        emitElementwise(op, clampCast_[k]);
       }
     }
     // stores
@@ -839,8 +907,11 @@ class TileEmitter {
     }
   }
 
-  void emitElementwise(const OpNode &op) {
-    if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+  void emitElementwise(const OpNode &opIn, const ClampCast &fused) {
+    if (opIn.outputs.size() != 1) throw LoweringError("op " + opIn.name + ": multiple results are not supported");
+    // a Cast that absorbed its clamp reads the clamp's source directly
+    OpNode op = opIn;
+    if (fused.source >= 0) op.inputs[0] = fused.source;
     const int outId = op.outputs[0];
     const TensorValue &outT = g_.tensor(outId);
     ValRank rank = ValRank::Const;
@@ -879,7 +950,10 @@ class TileEmitter {
                                 std::string(computeTypeName(outT.dtype)) == "float" &&
                                 std::string(computeTypeName(g_.tensor(op.inputs[0]).dtype)) == "float" &&
                                 std::string(computeTypeName(g_.tensor(op.inputs[1]).dtype)) == "float";
-    if (uniformDivisor) {
+    if (fused.source >= 0) {
+      expr = "akg::clamp_cast(" + operands[0] + ", " + lowering::literalFor(DType::F32, fused.lo) + ", " +
+             lowering::literalFor(DType::F32, fused.hi) + ")";
+    } else if (uniformDivisor) {
       const std::string hoisted = "d" + std::to_string(outId);
       std::string q;
       if (relaxed) {

@@ -472,6 +472,14 @@ struct Caster<b1, b1> {
   static AKG_DEV bool run(bool x) { return x; }
 };
 
+// Fused clamp + float->int cast: cast(min(max(x, lo), hi)) with constant bounds. Rounding to nearest even is monotonic
+// and maps the bounds to integers, so rounding first and clamping to the rounded bounds (already intersected with the
+// destination range by the lowering) is the same function; NaN propagates through min/max and casts to 0.
+AKG_DEV int clamp_cast(float x, float lo, float hi) {
+  const float r = __builtin_amdgcn_fmed3f(__builtin_rintf(x), lo, hi);
+  return (x != x) ? 0 : static_cast<int>(r);
+}
+
 template <typename DST, typename SRC>
 AKG_DEV typename DST::compute cast(typename SRC::compute x) {
   return Caster<DST, SRC>::run(x);
