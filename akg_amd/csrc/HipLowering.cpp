@@ -446,6 +446,7 @@ class TileEmitter {
   bool raggedCols_ = false, raggedRows_ = false, raggedFlat_ = false;
   int reduceCount_ = 0;
   bool nonTemporal_ = true;
+  bool useBuffers_ = true;
   std::vector<bool> relaxed_;
   // clamp + integer-cast peephole: ops skipped because a later Cast absorbs them, and what each such Cast computes
   struct ClampCast {
@@ -612,12 +613,12 @@ class TileEmitter {
     vec_ = v;
 
     if (rowMode_) {
-      // One row per group of tpr threads: about 16 elements per thread, at most 256 threads per row (wider rows
+      // One row per group of tpr threads: about 16 elements per thread, at most 512 threads per row (wider rows
       // get more chunks per thread instead; measured best on MI355X for 4096- and 8192-wide rows). The row stays
       // in registers across all reductions of the fusion.
       int targetPerThread = std::max(vec_, 16);
       int tpr = opt_.threadsPerRow > 0 ? opt_.threadsPerRow
-                                       : std::min(256, pow2AtLeast(ceilDiv(cols_, targetPerThread)));
+                                       : std::min(512, pow2AtLeast(ceilDiv(cols_, targetPerThread)));
       tpr = std::max(1, std::min(tpr, 1024));
       if ((tpr & (tpr - 1)) != 0) tpr = pow2AtLeast(tpr);
       // never more threads than chunks in a row
@@ -723,6 +724,13 @@ class TileEmitter {
 
   void line(const std::string &s) { src_ << s << "\n"; }
 
+  // Memory operand of argument `arg` ("in0", "out1", ...) at element offset `offset`: a buffer descriptor plus
+  // offset when every tensor of the kernel is below 2 GiB, a plain pointer otherwise.
+  std::string memRef(const std::string &arg, const std::string &offset) const {
+    if (useBuffers_) return "b_" + arg + ", " + offset;
+    return arg + " + " + offset;
+  }
+
   // Offset of the first element of `row` for an input, as an expression in `rowVar`.
   std::string rowOffsetExpr(const InputAccess &a, const std::string &rowVar) const {
     const std::vector<int64_t> &s = a.foldedShape;
@@ -779,6 +787,25 @@ class TileEmitter {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
     line(") {");
+    useBuffers_ = true;
+    for (int id : g_.inputs) {
+      if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
+    }
+    for (int id : g_.outputs) {
+      if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
+    }
+    if (useBuffers_) {
+      for (size_t i = 0; i < g_.inputs.size(); ++i) {
+        const TensorValue &t = g_.tensor(g_.inputs[i]);
+        src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", "
+             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+      }
+      for (size_t i = 0; i < g_.outputs.size(); ++i) {
+        const TensorValue &t = g_.tensor(g_.outputs[i]);
+        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", "
+             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+      }
+    }
     src_ << "  constexpr int V = " << vec_ << ";\n";
     src_ << "  constexpr int NCHUNK = " << chunks_ << ";\n";
     src_ << "  constexpr int BLOCK = " << block_ << ";\n";
@@ -877,9 +904,9 @@ class TileEmitter {
       src_ << "    if (akg_ok[j]) {\n";
       // a tensor as large as the iteration space is read exactly once: stream it
       const bool streamed = nonTemporal_ && (t.numel() == numel_);
-      src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">(in" << i << " + "
-           << rowOffsetExpr(a, "akg_rows[j]")
-           << " + akg_cols[j], " << v.ident << "[j]);\n";
+      src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">("
+           << memRef("in" + std::to_string(i), rowOffsetExpr(a, "akg_rows[j]") + " + akg_cols[j]") << ", " << v.ident
+           << "[j]);\n";
       src_ << "    } else {\n";
       src_ << "      akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(" << tag
            << "::storage()));\n";
@@ -890,8 +917,13 @@ class TileEmitter {
       v.rank = ValRank::Uniform;
       nm << "u_in" << i;
       v.ident = nm.str();
-      src_ << "  const " << ct << " " << v.ident << " = " << tag << "::load(in" << i << "["
-           << rowOffsetExpr(a, "akg_row") << "]);\n";
+      if (useBuffers_) {
+        src_ << "  const " << ct << " " << v.ident << " = akg::load_one<" << tag << ">(b_in" << i << ", "
+             << rowOffsetExpr(a, "akg_row") << ");\n";
+      } else {
+        src_ << "  const " << ct << " " << v.ident << " = " << tag << "::load(in" << i << "["
+             << rowOffsetExpr(a, "akg_row") << "]);\n";
+      }
       (void)t;
     } else {
       // elementwise mode: replicate the per-row element over the chunk
@@ -901,8 +933,13 @@ class TileEmitter {
       src_ << "  " << ct << " " << v.ident << "[NCHUNK][V];\n";
       line("#pragma unroll");
       line("  for (int j = 0; j < NCHUNK; ++j) {");
-      src_ << "    akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(in" << i << "["
-           << rowOffsetExpr(a, "akg_rows[j]") << "]));\n";
+      if (useBuffers_) {
+        src_ << "    akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], akg::load_one<" << tag << ">(b_in" << i << ", "
+             << rowOffsetExpr(a, "akg_rows[j]") << "));\n";
+      } else {
+        src_ << "    akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(in" << i << "["
+             << rowOffsetExpr(a, "akg_rows[j]") << "]));\n";
+      }
       line("  }");
     }
   }
@@ -1124,8 +1161,8 @@ class TileEmitter {
       std::string guard = "akg_ok[j]";
       if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
       std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
-      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (nonTemporal_ ? "true" : "false") << ">(out"
-           << i << " + " << offset << ", " << src
+      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (nonTemporal_ ? "true" : "false") << ">("
+           << memRef("out" + std::to_string(i), offset) << ", " << src
            << "[j]);\n";
       line("  }");
     } else {
@@ -1135,7 +1172,11 @@ class TileEmitter {
       if (v.rank == ValRank::Tile) throw LoweringError("output " + t.name + ": internal rank mismatch");
       std::string guard = "tcol == 0";
       if (raggedRows_) guard += " && akg_row_ok";
-      src_ << "  if (" << guard << ") out" << i << "[akg_row] = " << tag << "::store(" << v.ident << ");\n";
+      if (useBuffers_) {
+        src_ << "  if (" << guard << ") akg::store_one<" << tag << ">(b_out" << i << ", akg_row, " << v.ident << ");\n";
+      } else {
+        src_ << "  if (" << guard << ") out" << i << "[akg_row] = " << tag << "::store(" << v.ident << ");\n";
+      }
     }
   }
 };

@@ -182,6 +182,114 @@ AKG_DEV void store_chunk(typename DT::storage *__restrict__ p, const typename DT
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Buffer-addressed variants (tensors below 2 GiB): a 128-bit descriptor per tensor plus a 32-bit byte offset per
+// access, so address arithmetic is 32-bit, and the cache policy of every access is explicit:
+//   streamed loads   nt            (touched once: do not keep)
+//   streamed stores  sc1 + nt      (write through; measured +2 % over nt alone on a 1 GiB copy)
+//   reused loads     default
+// ---------------------------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t Buffer;
+
+AKG_DEV Buffer make_buffer(const void *p, long bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+constexpr int kAuxDefault = 0;
+constexpr int kAuxStreamLoad = 2;    // nt
+#ifndef AKG_STREAM_STORE_AUX
+#define AKG_STREAM_STORE_AUX 18
+#endif
+constexpr int kAuxStreamStore = AKG_STREAM_STORE_AUX;  // sc1 | nt
+
+template <int BYTES, int AUX>
+struct BufferIo;
+template <int AUX>
+struct BufferIo<16, AUX> {
+  typedef u32 __attribute__((ext_vector_type(4))) type;
+  static AKG_DEV type load(Buffer b, u32 off) { return __builtin_amdgcn_raw_buffer_load_b128(b, off, 0, AUX); }
+  static AKG_DEV void store(type v, Buffer b, u32 off) { __builtin_amdgcn_raw_buffer_store_b128(v, b, off, 0, AUX); }
+};
+template <int AUX>
+struct BufferIo<8, AUX> {
+  typedef u32 __attribute__((ext_vector_type(2))) type;
+  static AKG_DEV type load(Buffer b, u32 off) { return __builtin_amdgcn_raw_buffer_load_b64(b, off, 0, AUX); }
+  static AKG_DEV void store(type v, Buffer b, u32 off) { __builtin_amdgcn_raw_buffer_store_b64(v, b, off, 0, AUX); }
+};
+template <int AUX>
+struct BufferIo<4, AUX> {
+  typedef u32 type;
+  static AKG_DEV type load(Buffer b, u32 off) { return __builtin_amdgcn_raw_buffer_load_b32(b, off, 0, AUX); }
+  static AKG_DEV void store(type v, Buffer b, u32 off) { __builtin_amdgcn_raw_buffer_store_b32(v, b, off, 0, AUX); }
+};
+template <int AUX>
+struct BufferIo<2, AUX> {
+  typedef u16 type;
+  static AKG_DEV type load(Buffer b, u32 off) { return __builtin_amdgcn_raw_buffer_load_b16(b, off, 0, AUX); }
+  static AKG_DEV void store(type v, Buffer b, u32 off) { __builtin_amdgcn_raw_buffer_store_b16(v, b, off, 0, AUX); }
+};
+template <int AUX>
+struct BufferIo<1, AUX> {
+  typedef u8 type;
+  static AKG_DEV type load(Buffer b, u32 off) { return __builtin_amdgcn_raw_buffer_load_b8(b, off, 0, AUX); }
+  static AKG_DEV void store(type v, Buffer b, u32 off) { __builtin_amdgcn_raw_buffer_store_b8(v, b, off, 0, AUX); }
+};
+
+// `index` is an element index; the chunk starts at byte index * sizeof(storage).
+template <typename DT, int V, bool STREAM = false>
+AKG_DEV void load_chunk(Buffer buf, long index, typename DT::compute (&dst)[V]) {
+  typedef typename DT::storage S;
+  constexpr int kBytes = static_cast<int>(sizeof(S)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef BufferIo<kPiece, STREAM ? kAuxStreamLoad : kAuxDefault> Io;
+  typename Io::type raw[kPieces];
+  const u32 off = static_cast<u32>(index) * static_cast<u32>(sizeof(S));
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) raw[k] = Io::load(buf, off + k * kPiece);
+  S tmp[V];
+  __builtin_memcpy(tmp, raw, kBytes);
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(tmp[e]);
+}
+
+template <typename DT, int V, bool STREAM = false>
+AKG_DEV void store_chunk(Buffer buf, long index, const typename DT::compute (&src)[V]) {
+  typedef typename DT::storage S;
+  constexpr int kBytes = static_cast<int>(sizeof(S)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef BufferIo<kPiece, STREAM ? kAuxStreamStore : kAuxDefault> Io;
+  S tmp[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) tmp[e] = DT::store(src[e]);
+  typename Io::type raw[kPieces];
+  __builtin_memcpy(raw, tmp, kBytes);
+  const u32 off = static_cast<u32>(index) * static_cast<u32>(sizeof(S));
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) Io::store(raw[k], buf, off + k * kPiece);
+}
+
+template <typename DT>
+AKG_DEV typename DT::compute load_one(Buffer buf, long index) {
+  typedef typename DT::storage S;
+  typedef BufferIo<static_cast<int>(sizeof(S)), kAuxDefault> Io;
+  const typename Io::type raw = Io::load(buf, static_cast<u32>(index) * static_cast<u32>(sizeof(S)));
+  S s;
+  __builtin_memcpy(&s, &raw, sizeof(S));
+  return DT::load(s);
+}
+
+template <typename DT>
+AKG_DEV void store_one(Buffer buf, long index, typename DT::compute x) {
+  typedef typename DT::storage S;
+  typedef BufferIo<static_cast<int>(sizeof(S)), kAuxDefault> Io;
+  const S s = DT::store(x);
+  typename Io::type raw;
+  __builtin_memcpy(&raw, &s, sizeof(S));
+  Io::store(raw, buf, static_cast<u32>(index) * static_cast<u32>(sizeof(S)));
+}
+
 template <typename DT, int V>
 AKG_DEV void fill_chunk(typename DT::compute (&dst)[V], typename DT::compute x) {
 #pragma unroll
@@ -487,41 +595,74 @@ AKG_DEV typename DST::compute cast(typename SRC::compute x) {
 
 // ---------------------------------------------------------------------------------------------------------
 // Cross-lane reductions. A row is owned by a group of TPR threads (TPR a power of two). Up to one wavefront
-// the reduction is an xor butterfly: every lane ends with the same bits because each step combines the same
-// two partial results in both partners. The two innermost steps are DPP quad permutes; the rest go through
-// the LDS crossbar (ds_bpermute), which touches no LDS memory. Groups wider than a wavefront finish through
-// a small LDS array; every thread then folds the per-wavefront partials in the same fixed order.
+// the reduction is a butterfly of pairwise exchanges: at every step each lane combines its partial result with
+// the partial result of exactly one partner group, and both partners combine the same two values, so every lane
+// ends with the same bits. No step goes through LDS:
+//   partner distance 1, 2   DPP quad_perm
+//   4                       DPP row_half_mirror (lane i <-> 7 - i of its 8-lane half row: the other quad)
+//   8                       DPP row_mirror      (lane i <-> 15 - i of its 16-lane row: the other half row)
+//   16                      v_permlane16_swap   (exchanges odd and even 16-lane rows)
+//   32                      v_permlane32_swap   (exchanges the two 32-lane halves)
+// Groups wider than a wavefront finish through a small LDS array; every thread then folds the per-wavefront
+// partials in the same fixed order.
 // ---------------------------------------------------------------------------------------------------------
-AKG_DEV int lane_xor_bits(int v, int mask) {
-  if (mask == 1) return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
-  if (mask == 2) return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
-  const int lane = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
-  return __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, v);
+template <int STEP>
+AKG_DEV u32 lane_partner_bits(u32 v) {
+  if constexpr (STEP == 1) {
+    return static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, true));  // [1,0,3,2]
+  } else if constexpr (STEP == 2) {
+    return static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, true));  // [2,3,0,1]
+  } else if constexpr (STEP == 4) {
+    return static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x141, 0xF, 0xF, true));
+  } else if constexpr (STEP == 8) {
+    return static_cast<u32>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x140, 0xF, 0xF, true));
+  } else if constexpr (STEP == 16) {
+    // result[0] keeps this lane's value in even rows and receives the partner's in odd rows; result[1] the reverse
+    const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    return r[0] ^ r[1] ^ v;
+  } else {
+    static_assert(STEP == 32, "partner distance must be a power of two up to 32");
+    const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return r[0] ^ r[1] ^ v;
+  }
 }
 
-AKG_DEV float lane_xor(float v, int mask) {
-  return __builtin_bit_cast(float, lane_xor_bits(__builtin_bit_cast(int, v), mask));
+template <int STEP>
+AKG_DEV float lane_partner(float v) {
+  return __builtin_bit_cast(float, lane_partner_bits<STEP>(__builtin_bit_cast(u32, v)));
 }
-AKG_DEV int lane_xor(int v, int mask) { return lane_xor_bits(v, mask); }
-AKG_DEV bool lane_xor(bool v, int mask) { return lane_xor_bits(v ? 1 : 0, mask) != 0; }
-AKG_DEV double lane_xor(double v, int mask) {
-  u64 b = __builtin_bit_cast(u64, v);
-  u32 lo = static_cast<u32>(lane_xor_bits(static_cast<int>(b & 0xffffffffu), mask));
-  u32 hi = static_cast<u32>(lane_xor_bits(static_cast<int>(b >> 32), mask));
+template <int STEP>
+AKG_DEV int lane_partner(int v) {
+  return static_cast<int>(lane_partner_bits<STEP>(static_cast<u32>(v)));
+}
+template <int STEP>
+AKG_DEV bool lane_partner(bool v) {
+  return lane_partner_bits<STEP>(v ? 1u : 0u) != 0u;
+}
+template <int STEP>
+AKG_DEV double lane_partner(double v) {
+  const u64 b = __builtin_bit_cast(u64, v);
+  const u32 lo = lane_partner_bits<STEP>(static_cast<u32>(b & 0xffffffffu));
+  const u32 hi = lane_partner_bits<STEP>(static_cast<u32>(b >> 32));
   return __builtin_bit_cast(double, (static_cast<u64>(hi) << 32) | lo);
 }
-AKG_DEV long long lane_xor(long long v, int mask) {
-  u64 b = static_cast<u64>(v);
-  u32 lo = static_cast<u32>(lane_xor_bits(static_cast<int>(b & 0xffffffffu), mask));
-  u32 hi = static_cast<u32>(lane_xor_bits(static_cast<int>(b >> 32), mask));
+template <int STEP>
+AKG_DEV long long lane_partner(long long v) {
+  const u64 b = static_cast<u64>(v);
+  const u32 lo = lane_partner_bits<STEP>(static_cast<u32>(b & 0xffffffffu));
+  const u32 hi = lane_partner_bits<STEP>(static_cast<u32>(b >> 32));
   return static_cast<long long>((static_cast<u64>(hi) << 32) | lo);
 }
 
 template <typename Red, int WIDTH, typename T>
 AKG_DEV T wave_group_reduce(T v) {
   static_assert(WIDTH <= kWaveSize && (WIDTH & (WIDTH - 1)) == 0, "group width must be a power of two <= 64");
-#pragma unroll
-  for (int m = 1; m < WIDTH; m <<= 1) v = Red::apply(v, lane_xor(v, m));
+  if constexpr (WIDTH > 1) v = Red::apply(v, lane_partner<1>(v));
+  if constexpr (WIDTH > 2) v = Red::apply(v, lane_partner<2>(v));
+  if constexpr (WIDTH > 4) v = Red::apply(v, lane_partner<4>(v));
+  if constexpr (WIDTH > 8) v = Red::apply(v, lane_partner<8>(v));
+  if constexpr (WIDTH > 16) v = Red::apply(v, lane_partner<16>(v));
+  if constexpr (WIDTH > 32) v = Red::apply(v, lane_partner<32>(v));
   return v;
 }
 
