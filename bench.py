@@ -41,10 +41,11 @@ CALIBRATION = "calib_neg_f32_16384x4096"
 # for a plain copy of known size: FETCH_SIZE reads half the bytes, scale 2.0; WRITE_SIZE scale 1.0). Values are the
 # ones of the summaries under profiles/; None = not measured yet.
 MEASURED_TRAFFIC_BYTES = {
-    "c1_ew_tanh_add_mul_f32_1024x4096": 67192508,
-    "c2_softmax_f16_8192x4096": 134251305,
-    "c3_layernorm_residual_bf16_16384x4096": 402778917,
-    "c4_quant_int8_residual_bf16_32768x8192": 1343247471,
+    "c1_ew_tanh_add_mul_f32_1024x4096": 67192334,
+    "c2_softmax_f16_8192x4096": 134251127,
+    "c3_layernorm_residual_bf16_16384x4096": 402799864,
+    "c4_quant_int8_residual_bf16_32768x8192": 1343207389,
+    "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": 470293950,
 }
 
 
