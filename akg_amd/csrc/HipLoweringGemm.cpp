@@ -71,6 +71,7 @@ class GemmEmitter {
   int wavesM() const { return (opt_.gemmVariant & 1) ? 2 : 4; }
   // K extent of one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
   int stepK() const { return (opt_.gemmVariant & 2) ? 64 : 128; }
+  bool splitDuty() const { return (opt_.gemmVariant & 4) != 0 && wavesM() == 4; }
 
   void analyse() {
     for (size_t i = 0; i < g_.ops.size(); ++i) {
@@ -289,7 +290,7 @@ class GemmEmitter {
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
     src_ << "  akg::gemm_i8_256x256<" << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ", " << wavesM() << ", " << stepK() << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
+         << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
   }
 };
 

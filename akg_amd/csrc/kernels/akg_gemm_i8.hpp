@@ -70,18 +70,25 @@ constexpr long gemm_i8_grid(long m, long n) {
 // wavefront's MFMAs cover the first one's loads, transposes and barriers).
 // BK = K extent of one step: 64 or 128. With 128 every row of A contributes one full 128-byte cache line per step
 // (with 64 each line is fetched from L2 twice), there are half as many barriers, and LDS holds 2 x 72 KiB.
-template <long M, long N, long K, bool TRANSB, int WAVES_M, int BK, typename Epilogue>
+template <long M, long N, long K, bool TRANSB, int WAVES_M, int BK, bool SPLIT, typename Epilogue>
 AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B, Epilogue &epi) {
   static_assert(K % 16 == 0, "K must be a multiple of 16");
   static_assert(TRANSB || (N % 4 == 0), "N must be a multiple of 4");
   static_assert(WAVES_M == 2 || WAVES_M == 4, "2 x 2 or 4 x 2 wavefronts");
   static_assert(BK == 64 || BK == 128, "K step of 64 or 128");
+  static_assert(!SPLIT || WAVES_M == 4, "split staging duty needs 8 wavefronts");
+  // Staging (global -> registers -> LDS) is done either by every thread for both operands (uniform control flow:
+  // the whole K step is one basic block, so loads, transposes and LDS writes interleave with the MFMAs), or, with
+  // SPLIT, by wavefronts 0..3 for B and 4..7 for A (fewer, longer bursts per wavefront).
+  constexpr bool kSplitDuty = SPLIT;
+  constexpr int kThreads = WAVES_M * 128;
+  constexpr int kStageThreads = kSplitDuty ? 256 : kThreads;  // threads that share one operand tile
   constexpr int kPitch = BK + 16;                     // LDS row: BK data bytes + 16 pad (odd multiple of 16)
   constexpr int kSub = BK / 32;                       // MFMA k-substeps per step (2 or 4)
   constexpr int kChunksPerRow = BK / 16;              // 16-byte chunks per row of a K-contiguous operand tile
-  constexpr int kRowChunks = BK / 16;                 // chunks per staging thread (256 rows * BK/16 / 256 threads)
-  constexpr int kRowStep = 256 / kChunksPerRow;       // rows between two chunks of one thread
-  constexpr int kBlockRows = BK / 4;                  // k-rows of B per staging thread (16 or 32)
+  constexpr int kRowChunks = 256 * kChunksPerRow / kStageThreads;  // 16-byte chunks per staging thread and operand
+  constexpr int kRowStep = kStageThreads / kChunksPerRow;          // rows between two chunks of one thread
+  constexpr int kBlockRows = 4 * kRowChunks;          // k-rows of B per staging thread (8, 16 or 32), 4 columns each
   constexpr int kTM = kGemmBM / (32 * WAVES_M);       // MFMA row tiles per wavefront
   constexpr int kWaveRows = kGemmBM / WAVES_M;
   constexpr long kTilesM = (M + kGemmBM - 1) / kGemmBM;
@@ -126,17 +133,15 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
 
   // ---- staging registers: the tile of step s+1 travels memory -> registers during step s-1.. s and is written to
   // LDS at the top of step s.
-  // 2 x 2 wavefronts: every thread stages its share of A (x) and of B (y).
-  // 4 x 2 wavefronts: wavefronts 0..3 stage all of B, wavefronts 4..7 all of A, both in x (the 128-bit LDS writes of
-  //                   the transposed B blocks stay conflict free this way, and x is the only staging array).
-  constexpr bool kSplitDuty = (WAVES_M == 4);
+  // Uniform duty: every thread stages its share of A (x) and of B (y).
+  // Split duty:   wavefronts 0..3 stage all of B, wavefronts 4..7 all of A, both in x.
   struct Stage {
     v4i x[kRowChunks];
     v4i y[kSplitDuty ? 1 : kRowChunks];
   };
   Stage stage;
 
-  const int ltid = tid & 255;
+  const int ltid = kSplitDuty ? (tid & 255) : tid;
   const bool stageA = !kSplitDuty || tid >= 256;
   const int aRow = ltid / kChunksPerRow;   // + kRowStep * i
   const int aChunk = ltid % kChunksPerRow;
@@ -223,6 +228,14 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
                            static_cast<u32>(src[g][3])};
       transpose4x4_bytes(rows, t[g]);
     }
+    if constexpr (kRowChunks == 2) {
+      typedef int v2i __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const v2i w = {static_cast<int>(t[0][j]), static_cast<int>(t[1][j])};
+        *reinterpret_cast<v2i *>(lb + (j * 64 + bN4) * kPitch + bKq * kBlockRows) = w;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -285,8 +298,9 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
   // ---- main loop. Invariant at the top of step s: LDS buffer s&1 holds tile s (complete), the staging registers hold
   // tile s+1 (possibly still in flight), and f0 holds the fragments of the first 32 k of tile s.
   //   a. staged tile s+1 -> LDS buffer (s+1)&1      (its last readers finished before the previous barrier)
-  //   b. issue the global loads of tile s+2 into the staging registers
+  //   b. issue the global loads of tile s+2 into the staging registers (they have a whole step to arrive)
   //   c. for every k-substep but the last: read the next substep's fragments, MFMAs on the current ones
+  //      (a and b interleave with the MFMAs of the early substeps)
   //   d. barrier: everybody has read tile s completely and has written tile s+1
   //   e. read the first fragments of tile s+1         (their latency hides behind the MFMAs of f)
   //   f. MFMAs on the last substep's fragments
@@ -297,8 +311,15 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
     constexpr bool kStore = decltype(storeTag)::value;
     constexpr bool kLoad = decltype(loadTag)::value;
     const int buf = static_cast<int>(step & 1);
-    // ---- first half: MFMAs on the fragments already in registers; meanwhile fetch the next fragments and move the
-    // staged tile (transposing B) into the other LDS buffer
+    // The staged tile goes to the other LDS buffer at the very top of the step (its last readers finished before
+    // the previous step's barrier), and the freed staging registers are refilled at once: the LDS writes complete
+    // and the global loads travel while the step's MFMAs run, instead of piling up in front of the barrier.
+#ifndef AKG_DIAG_NO_LDS_STORE
+    if constexpr (kStore) storeLds(buf ^ 1, stage);
+#endif
+#ifndef AKG_DIAG_NO_GLOBAL_LOAD
+    if constexpr (kLoad) loadGlobal(step + 2, stage);
+#endif
 #pragma unroll
     for (int ks = 0; ks + 2 < kSub; ks += 2) {
       readFrags(buf, ks + 1, f1a, f1b);
@@ -306,62 +327,15 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
       readFrags(buf, ks + 2, f0a, f0b);
       mfmaAll(f1a, f1b);
     }
+    if constexpr (kSub > 2) __builtin_amdgcn_sched_barrier(0);  // keep the staging work in the early substeps
     readFrags(buf, kSub - 1, f1a, f1b);
-#ifndef AKG_DIAG_NO_LDS_STORE
-    if constexpr (kStore) storeLds(buf ^ 1, stage);
-#endif
     mfmaAll(f0a, f0b);
-    if constexpr (!kSplitDuty && kSub == 2 && kStore && !TRANSB) {
-      // Issue order inside the half step (one wavefront per SIMD: nothing else hides latencies). kTM * 4 = 16 MFMAs:
-      //   MFMA 0..7   each followed by one fragment read (ds_read_b128)
-      //   MFMA 8..11  each followed by one A-tile LDS write and 8 of the 32 byte-transpose permutes
-      //   MFMA 12..15 each followed by one B-tile LDS write
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-      }
-    }
 #ifndef AKG_DIAG_NO_BARRIER
     __syncthreads();
 #endif
-    // ---- second half: MFMAs on the last fragments of this tile; meanwhile fetch the first fragments of the next
-    // tile and issue the global loads of the tile after it into the (now free) staging registers
+    // ---- after the barrier: MFMAs on the last fragments of this tile; meanwhile fetch the first fragments of the next
     if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
-#ifndef AKG_DIAG_NO_GLOBAL_LOAD
-    if constexpr (kLoad) loadGlobal(step + 2, stage);
-#endif
     mfmaAll(f1a, f1b);
-    if constexpr (!kSplitDuty && kSub == 2 && kLoad && !TRANSB) {
-      //   MFMA 0..7   each followed by one fragment read
-      //   MFMA 8..15  each followed by 2-3 of the 20 global loads (4 x 128-bit of A, 16 x 32-bit of B)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, 3, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-      }
-    }
   };
   loadGlobal(0, stage);
   storeLds(0, stage);
