@@ -40,6 +40,7 @@ CALIBRATION = "calib_neg_f32_16384x4096"
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; scaled by the same counters' reading
 # for a plain copy of known size: FETCH_SIZE reads half the bytes, scale 2.0; WRITE_SIZE scale 1.0). Values are the
 # ones of the summaries under profiles/; None = not measured yet.
+CLOCK_RAMP_MS = 120.0
 MEASURED_TRAFFIC_BYTES = {
     "c1_ew_tanh_add_mul_f32_1024x4096": 67192334,
     "c2_softmax_f16_8192x4096": 134251127,
@@ -69,6 +70,16 @@ def gpu_measure(name, steps, warmup, torch, driver, harness, np):
     ptrs = [[b.data_ptr() for b in bufs] for bufs in sets]
     stream = torch.cuda.current_stream()
     st = stream.cuda_stream
+    # Clock ramp: an idle MI355X sits at a few hundred MHz and needs some tens of milliseconds of sustained work
+    # to reach its steady clocks (the first ~15 ms of launches after idle run 10-25 % slower). The figures reported
+    # are steady-state ones, so the device is kept busy for CLOCK_RAMP_MS before the W warm-up steps.
+    t_ramp = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t_ramp) * 1e3 < CLOCK_RAMP_MS:
+        for _ in range(16):
+            kernel.launch_ptrs(ptrs[i % nsets], st)
+            i += 1
+        torch.cuda.synchronize()
     for i in range(warmup):
         kernel.launch_ptrs(ptrs[i % nsets], st)
     torch.cuda.synchronize()
@@ -149,7 +160,7 @@ def main():
         "vs_baseline": None, "dtype": WORKLOADS.get(name, "f32"), "data": "synthetic",
         "config": {"workload": name, "family": kernel.family, "grid": kernel.grid[0], "block": kernel.block[0],
                    "algorithmic_bytes": kernel.algorithmic_bytes, "algorithmic_ops": kernel.algorithmic_ops,
-                   "buffer_sets_rotated": nsets},
+                   "buffer_sets_rotated": nsets, "clock_ramp_ms": CLOCK_RAMP_MS},
         "roofline": roofline_of(kernel, kernel_ms, name),
         "kernel_ms": round(kernel_ms, 5),
     }
