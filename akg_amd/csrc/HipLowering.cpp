@@ -14,6 +14,7 @@ const char *kernelFamilyName(KernelFamily f) {
     case KernelFamily::Elementwise: return "elementwise";
     case KernelFamily::RowReduce: return "row_reduce";
     case KernelFamily::GemmEpilogue: return "gemm_epilogue";
+    case KernelFamily::StreamReduce: return "stream_reduce";
   }
   return "?";
 }
@@ -159,6 +160,72 @@ std::vector<std::vector<int64_t>> buildShapeArgs(const OpGraph &g) {
 bool isReduceKind(OpKind k) {
   return k == OpKind::ReduceSum || k == OpKind::ReduceMax || k == OpKind::ReduceMin || k == OpKind::ReduceProd ||
          k == OpKind::ReduceAll || k == OpKind::ReduceAny;
+}
+
+ReduceSpec reduceSpec(const OpNode &op, DType od) {
+  ReduceSpec r;
+  r.roundEachStep = (od == DType::F16 || od == DType::BF16 || od == DType::I8 || od == DType::I16);
+  auto largest = [&](bool negative) -> std::string {
+    // largest finite value of the result type (createFloatInitValue, MindSporeToLinalg.cpp:811-827)
+    double v = 0.0;
+    switch (od) {
+      case DType::F16: v = 65504.0; break;
+      case DType::BF16: v = 3.3895313892515355e38; break;
+      case DType::F32: v = 3.4028234663852886e38; break;
+      case DType::F64: v = 1.7976931348623157e308; break;
+      default: break;
+    }
+    return literalFor(od, negative ? -v : v);
+  };
+  auto intLimit = [&](bool minimum) -> std::string {
+    switch (od) {
+      case DType::I8: return minimum ? "(-128)" : "(127)";
+      case DType::I16: return minimum ? "(-32768)" : "(32767)";
+      case DType::I32: return minimum ? "(-2147483647 - 1)" : "(2147483647)";
+      case DType::I64: return minimum ? "(-9223372036854775807LL - 1)" : "(9223372036854775807LL)";
+      default: break;
+    }
+    throw LoweringError("op " + op.name + ": unsupported result type");
+  };
+  switch (op.kind) {
+    case OpKind::ReduceSum:
+      if (od == DType::Bool) throw LoweringError("ReduceSum on bool is not supported");
+      r.combiner = "akg::RedSum";
+      r.init = literalFor(od, 0.0);
+      break;
+    case OpKind::ReduceProd:
+      if (od == DType::Bool) throw LoweringError("ReducePrd on bool is not supported");
+      r.combiner = "akg::RedProd";
+      r.init = literalFor(od, 1.0);
+      break;
+    case OpKind::ReduceMax:
+      if (od == DType::Bool) throw LoweringError("ReduceMax on bool is not supported");
+      r.combiner = "akg::RedMax";
+      r.init = isFloatType(od) ? largest(true) : intLimit(true);
+      r.roundEachStep = false;
+      break;
+    case OpKind::ReduceMin:
+      if (od == DType::Bool) throw LoweringError("ReduceMin on bool is not supported");
+      r.combiner = "akg::RedMin";
+      r.init = isFloatType(od) ? largest(false) : intLimit(false);
+      r.roundEachStep = false;
+      break;
+    case OpKind::ReduceAll:
+      if (od != DType::Bool) throw LoweringError("ReduceAll needs a bool tensor");
+      r.combiner = "akg::RedAll";
+      r.init = "true";
+      r.roundEachStep = false;
+      break;
+    case OpKind::ReduceAny:
+      if (od != DType::Bool) throw LoweringError("ReduceAny needs a bool tensor");
+      r.combiner = "akg::RedAny";
+      r.init = "false";
+      r.roundEachStep = false;
+      break;
+    default:
+      throw LoweringError("internal: not a reduction");
+  }
+  return r;
 }
 
 bool isElementwiseKind(OpKind k) {
@@ -1041,68 +1108,9 @@ class TileEmitter {
     const DType od = g_.tensor(outId).dtype;
     const std::string ct = computeTypeName(od);
     const std::string tag = dtypeTag(od);
-    std::string red, init;
-    bool roundEachStep = (od == DType::F16 || od == DType::BF16 || od == DType::I8 || od == DType::I16);
-    auto largest = [&](bool negative) -> std::string {
-      // largest finite value of the result type (createFloatInitValue, MindSporeToLinalg.cpp:811-827)
-      double v = 0.0;
-      switch (od) {
-        case DType::F16: v = 65504.0; break;
-        case DType::BF16: v = 3.3895313892515355e38; break;
-        case DType::F32: v = 3.4028234663852886e38; break;
-        case DType::F64: v = 1.7976931348623157e308; break;
-        default: break;
-      }
-      return lowering::literalFor(od, negative ? -v : v);
-    };
-    auto intLimit = [&](bool minimum) -> std::string {
-      switch (od) {
-        case DType::I8: return minimum ? "(-128)" : "(127)";
-        case DType::I16: return minimum ? "(-32768)" : "(32767)";
-        case DType::I32: return minimum ? "(-2147483647 - 1)" : "(2147483647)";
-        case DType::I64: return minimum ? "(-9223372036854775807LL - 1)" : "(9223372036854775807LL)";
-        default: break;
-      }
-      throw LoweringError("op " + op.name + ": unsupported result type");
-    };
-    switch (op.kind) {
-      case OpKind::ReduceSum:
-        if (od == DType::Bool) throw LoweringError("ReduceSum on bool is not supported");
-        red = "akg::RedSum";
-        init = lowering::literalFor(od, 0.0);
-        break;
-      case OpKind::ReduceProd:
-        if (od == DType::Bool) throw LoweringError("ReducePrd on bool is not supported");
-        red = "akg::RedProd";
-        init = lowering::literalFor(od, 1.0);
-        break;
-      case OpKind::ReduceMax:
-        if (od == DType::Bool) throw LoweringError("ReduceMax on bool is not supported");
-        red = "akg::RedMax";
-        init = isFloatType(od) ? largest(true) : intLimit(true);
-        roundEachStep = false;
-        break;
-      case OpKind::ReduceMin:
-        if (od == DType::Bool) throw LoweringError("ReduceMin on bool is not supported");
-        red = "akg::RedMin";
-        init = isFloatType(od) ? largest(false) : intLimit(false);
-        roundEachStep = false;
-        break;
-      case OpKind::ReduceAll:
-        if (od != DType::Bool) throw LoweringError("ReduceAll needs a bool tensor");
-        red = "akg::RedAll";
-        init = "true";
-        roundEachStep = false;
-        break;
-      case OpKind::ReduceAny:
-        if (od != DType::Bool) throw LoweringError("ReduceAny needs a bool tensor");
-        red = "akg::RedAny";
-        init = "false";
-        roundEachStep = false;
-        break;
-      default:
-        throw LoweringError("internal: not a reduction");
-    }
+    const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+    const std::string red = spec.combiner, init = spec.init;
+    const bool roundEachStep = spec.roundEachStep;
     if (std::string(computeTypeName(g_.tensor(inId).dtype)) != ct) {
       throw LoweringError("op " + op.name + ": operand and result element types differ");
     }
@@ -1190,6 +1198,7 @@ LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options) {
     if (op.kind == OpKind::MatMul) hasMatMul = true;
   }
   if (hasMatMul) return lowerGemmToHip(graph, options);
+  if (wantsStreamReduce(graph)) return lowerStreamReduceToHip(graph, options);
   TileEmitter emitter(graph, options);
   return emitter.run();
 }

@@ -31,7 +31,7 @@ class LoweringError : public std::runtime_error {
   explicit LoweringError(const std::string &msg) : std::runtime_error(msg) {}
 };
 
-enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue };
+enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce };
 const char *kernelFamilyName(KernelFamily f);
 
 // Tuning knobs; 0 means "let the heuristic decide". They can be set through the environment
@@ -57,12 +57,19 @@ struct LoweredKernel {
   std::string scheduleNote;       // human-readable schedule summary (vec, threads per row, ...)
   // per kernel argument: [offset, sizes..., strides...] as in `<k>_shape_arg.txt`
   std::vector<std::vector<int64_t>> shapeArgs;
+  // Device workspace the kernel takes as one extra trailing pointer argument (0: none). The runtime allocates it
+  // per kernel handle and device and zero-fills it once; the kernel leaves it zeroed where it must be.
+  uint64_t workspaceBytes = 0;
 };
 
 LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options);
 
-// Family-specific entry used by lowerToHip (defined in HipLoweringGemm.cpp).
+// Family-specific entries used by lowerToHip (defined in HipLoweringGemm.cpp and HipLoweringReduce.cpp).
 LoweredKernel lowerGemmToHip(const OpGraph &graph, const LoweringOptions &options);
+LoweredKernel lowerStreamReduceToHip(const OpGraph &graph, const LoweringOptions &options);
+// True when the reductions of `graph` belong to the streaming family: some reduced axis is not the innermost one
+// (direction Y / ALL), or the rows are too long or too few for the register-resident row kernel.
+bool wantsStreamReduce(const OpGraph &graph);
 
 // Shared helpers for the emitters.
 namespace lowering {
@@ -82,6 +89,14 @@ std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vecto
 std::vector<bool> relaxedPrecisionTensors(const OpGraph &g);
 bool isElementwiseKind(OpKind k);
 bool isReduceKind(OpKind k);
+// Combiner functor, initial value and rounding rule of a reduction whose result type is `od`
+// (createInitValueForReduce / createCombinerForReduce, MindSporeToLinalg.cpp:791-901).
+struct ReduceSpec {
+  std::string combiner;        // "akg::RedSum", ...
+  std::string init;            // literal of the compute type
+  bool roundEachStep = false;  // narrow result types accumulate in that type: round after every step
+};
+ReduceSpec reduceSpec(const OpNode &op, DType od);
 }  // namespace lowering
 
 }  // namespace akg

@@ -1,0 +1,778 @@
+/**
+ * Streaming reductions: the kernel family for reductions that the register-resident row kernel cannot take.
+ *
+ *   direction Y  : the reduced axes are not the innermost ones, e.g. [1,5100,3072] -> [1,1,3072] (column sums)
+ *   direction ALL: every axis is reduced, e.g. [768,512] -> [1]
+ *   direction X with rows that are too long for registers, or so few that a row per workgroup leaves the chip idle
+ *
+ * The reference reaches these shapes through its reduce-Y / all-reduce templates and finishes them with atomics on
+ * the result (GpuUseAllReduceWithAtomicReturn, GPUOpt.cpp:226-268; RewriteReduceInMultiLevelMemory.cpp:174-281).
+ * Here the result is deterministic instead: the iteration space is folded to [O, R, I] (outer kept, reduced, inner
+ * kept), SPLIT workgroups share one group of outputs, each streams its slice of R once with 16-byte accesses,
+ * leaves a partial in a workspace, and the last workgroup to arrive combines the partials in a fixed order, applies
+ * the ops that follow the reduction and writes the outputs. Nothing is read twice and no output needs zero-filling.
+ *
+ * Graph shape accepted: elementwise ops on the unreduced tensors ("pre"), any number of reductions over the same axes
+ * of same-shaped operands, elementwise ops on the reduced values ("post"). Outputs may be reduced values or unreduced
+ * ones (stored while streaming). An op that mixes a reduced value with an unreduced one (softmax along Y) would need a
+ * second pass over the data and has no kernel here.
+ */
+#include <algorithm>
+#include <sstream>
+
+#include "HipLowering.h"
+
+namespace akg {
+
+namespace {
+
+using lowering::computeTypeName;
+using lowering::dtypeTag;
+
+int64_t ceilDivL(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+int pow2AtLeastL(int64_t x) {
+  int p = 1;
+  while (p < x) p <<= 1;
+  return p;
+}
+
+// Real (extent > 1) reduced axes of a reduction, as positions in its operand's shape.
+std::vector<size_t> realReducedAxes(const OpGraph &g, const OpNode &op) {
+  const TensorValue &in = g.tensor(op.inputs[0]);
+  std::vector<size_t> out;
+  for (int64_t a : op.axes) {
+    if (a >= 0 && static_cast<size_t>(a) < in.shape.size() && in.shape[static_cast<size_t>(a)] > 1) {
+      out.push_back(static_cast<size_t>(a));
+    }
+  }
+  return out;
+}
+
+enum class Phase { None, Pre, Post };
+
+class StreamReduceEmitter {
+ public:
+  StreamReduceEmitter(const OpGraph &g, const LoweringOptions &o) : g_(g), opt_(o) {}
+
+  LoweredKernel run() {
+    analyse();
+    pickSchedule();
+    emit();
+    LoweredKernel k;
+    k.kernelName = g_.name + "_kernel";
+    k.source = src_.str();
+    k.family = KernelFamily::StreamReduce;
+    k.grid[0] = static_cast<unsigned>(grid_);
+    k.block[0] = static_cast<unsigned>(kBlock);
+    k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
+    k.shapeArgs = lowering::buildShapeArgs(g_);
+    k.workspaceBytes = workspaceBytes_;
+    std::ostringstream note;
+    note << "stream_reduce direction=" << (dirY_ ? "Y" : "X") << " outer=" << O_ << " reduced=" << R_ << " inner=" << I_
+         << " vec=" << vec_ << " lanes=" << lanes_ << " split=" << split_ << " rows_per_split=" << rps_
+         << " block=" << kBlock << " grid=" << grid_ << " workspace=" << workspaceBytes_;
+    k.scheduleNote = note.str();
+    return k;
+  }
+
+ private:
+  static constexpr int kBlock = 256;
+
+  const OpGraph &g_;
+  LoweringOptions opt_;
+  std::ostringstream src_;
+
+  // iteration space: the reduced operand's shape; kind per dim (0 outer kept, 1 reduced, 2 inner kept, -1 unit)
+  std::vector<int64_t> space_;
+  std::vector<int> kind_;
+  int64_t O_ = 1, R_ = 1, I_ = 1;
+  bool dirY_ = false;
+  std::vector<Phase> phase_;  // per tensor
+  std::vector<const OpNode *> reduces_;
+
+  int vec_ = 1, lanes_ = 64, split_ = 1;
+  int64_t strips_ = 1, rps_ = 1, grid_ = 1, groups_ = 1;
+  uint64_t workspaceBytes_ = 0;
+  std::vector<uint64_t> partialOffset_;  // per reduction, bytes from the workspace base
+  bool useBuffers_ = true;
+  std::vector<bool> relaxed_;
+  std::vector<std::string> ident_;  // per tensor: array / scalar name once defined
+
+  void line(const std::string &s) { src_ << s << "\n"; }
+  std::string ctOf(int id) const { return computeTypeName(g_.tensor(id).dtype); }
+  std::string tagOf(int id) const { return dtypeTag(g_.tensor(id).dtype); }
+
+  // ------------------------------------------------------------------ analysis
+  std::vector<int64_t> padTo(const std::vector<int64_t> &shape, const std::string &what) const {
+    std::vector<int64_t> s = shape;
+    const size_t n = space_.size();
+    while (s.size() > n && s.front() == 1) s.erase(s.begin());
+    if (s.size() > n) throw LoweringError(what + ": rank exceeds the reduced operand's");
+    std::vector<int64_t> out(n - s.size(), 1);
+    out.insert(out.end(), s.begin(), s.end());
+    return out;
+  }
+
+  void analyse() {
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::Unknown) {
+        throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
+      }
+      if (op.kind == OpKind::Unsupported || op.kind == OpKind::MatMul) {
+        throw LoweringError("op " + op.name + " cannot be fused into a streaming reduction");
+      }
+      if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+      if (lowering::isReduceKind(op.kind)) reduces_.push_back(&op);
+    }
+    if (reduces_.empty()) throw LoweringError("internal: no reduction");
+    const OpNode &first = *reduces_.front();
+    space_ = g_.tensor(first.inputs[0]).shape;
+    if (space_.empty()) space_.push_back(1);
+    const size_t n = space_.size();
+    std::vector<bool> reduced(n, false);
+    for (size_t a : realReducedAxes(g_, first)) reduced[a] = true;
+    for (const OpNode *op : reduces_) {
+      const TensorValue &in = g_.tensor(op->inputs[0]);
+      if (in.shape.size() != n || padTo(in.shape, "reduce operand " + in.name) != space_) {
+        throw LoweringError("all reductions of one kernel must run over the same tensor shape");
+      }
+      std::vector<bool> r2(n, false);
+      for (size_t a : realReducedAxes(g_, *op)) r2[a] = true;
+      if (r2 != reduced) throw LoweringError("all reductions of one kernel must reduce the same axes");
+      const DType od = g_.tensor(op->outputs[0]).dtype;
+      if (od == DType::Bool) throw LoweringError("op " + op->name + ": bool reductions have no streaming kernel yet");
+      if (std::string(computeTypeName(in.dtype)) != computeTypeName(od)) {
+        throw LoweringError("op " + op->name + ": operand and result element types differ");
+      }
+    }
+    // kinds: kept dims before the first reduced one are "outer", after the last reduced one "inner"
+    kind_.assign(n, -1);
+    size_t firstR = n, lastR = 0;
+    for (size_t d = 0; d < n; ++d) {
+      if (space_[d] > 1 && reduced[d]) {
+        firstR = std::min(firstR, d);
+        lastR = d;
+      }
+    }
+    if (firstR == n) throw LoweringError("reduction over axes of extent 1 only: nothing to reduce");
+    for (size_t d = 0; d < n; ++d) {
+      if (space_[d] <= 1) continue;
+      if (reduced[d]) {
+        kind_[d] = 1;
+      } else if (d < firstR) {
+        kind_[d] = 0;
+      } else if (d > lastR) {
+        kind_[d] = 2;
+      } else {
+        throw LoweringError("reduced axes interleaved with kept ones (e.g. [N,C,HW] over N and HW) have no kernel yet");
+      }
+    }
+    for (size_t d = 0; d < n; ++d) {
+      if (kind_[d] == 0) O_ *= space_[d];
+      if (kind_[d] == 1) R_ *= space_[d];
+      if (kind_[d] == 2) I_ *= space_[d];
+    }
+    dirY_ = I_ > 1;
+
+    // phases by data flow: Post = depends on a reduction result
+    phase_.assign(g_.tensors.size(), Phase::None);
+    for (int id : g_.inputs) phase_[static_cast<size_t>(id)] = Phase::Pre;
+    for (const OpNode &op : g_.ops) {
+      bool anyPost = false, anyPre = false;
+      for (int in : op.inputs) {
+        const TensorValue &t = g_.tensor(in);
+        if (t.isConst) continue;
+        const Phase p = phase_[static_cast<size_t>(in)];
+        if (p == Phase::None) throw LoweringError("op " + op.name + ": operand " + t.name + " is undefined");
+        if (p == Phase::Post) {
+          anyPost = true;
+        } else if (t.producer < 0 && !variesAlongReduced(t)) {
+          // a graph input that does not vary along the reduced axes can be read in either phase
+        } else {
+          anyPre = true;
+        }
+      }
+      const int out = op.outputs[0];
+      if (lowering::isReduceKind(op.kind)) {
+        if (anyPost) throw LoweringError("op " + op.name + ": a reduction of a reduced value needs a second kernel");
+        phase_[static_cast<size_t>(out)] = Phase::Post;
+      } else if (anyPost) {
+        if (anyPre) {
+          throw LoweringError("op " + op.name + " combines a reduced value with an unreduced one: that needs a second "
+                              "pass over the data, which the streaming reduction does not make");
+        }
+        phase_[static_cast<size_t>(out)] = Phase::Post;
+      } else {
+        phase_[static_cast<size_t>(out)] = Phase::Pre;
+      }
+    }
+    const int64_t fullNumel = O_ * R_ * I_;
+    for (int id : g_.outputs) {
+      const TensorValue &t = g_.tensor(id);
+      const Phase p = phase_[static_cast<size_t>(id)];
+      if (p == Phase::Post) {
+        if (t.numel() != O_ * I_) throw LoweringError("output " + t.name + ": not the shape of the reduced value");
+      } else if (p == Phase::Pre) {
+        if (t.producer < 0) throw LoweringError("output " + t.name + " is a kernel input");
+        if (t.numel() != fullNumel) throw LoweringError("output " + t.name + ": shape does not match the reduced operand");
+      } else {
+        throw LoweringError("output " + t.name + " is never computed");
+      }
+    }
+    for (int id : g_.inputs) {
+      const TensorValue &t = g_.tensor(id);
+      const std::vector<int64_t> s = padTo(t.shape, "input " + t.name);
+      for (size_t d = 0; d < n; ++d) {
+        if (s[d] != 1 && s[d] != space_[d]) {
+          throw LoweringError("input " + t.name + " is not broadcast-compatible with the reduced tensor");
+        }
+      }
+    }
+  }
+
+  bool variesAlongReduced(const TensorValue &t) const {
+    const std::vector<int64_t> s = padTo(t.shape, "tensor " + t.name);
+    for (size_t d = 0; d < space_.size(); ++d) {
+      if (kind_[d] == 1 && s[d] != 1) return true;
+    }
+    return false;
+  }
+
+  // Innermost non-unit dim of a group, or -1.
+  int innermostDim(int group) const {
+    for (size_t d = space_.size(); d-- > 0;) {
+      if (kind_[d] == group) return static_cast<int>(d);
+    }
+    return -1;
+  }
+
+  // ------------------------------------------------------------------ schedule
+  void pickSchedule() {
+    size_t widest = 1;
+    for (int id : g_.inputs) widest = std::max(widest, dtypeSize(g_.tensor(id).dtype));
+    for (int id : g_.outputs) widest = std::max(widest, dtypeSize(g_.tensor(id).dtype));
+    int v = opt_.vec > 0 ? opt_.vec : static_cast<int>(16 / widest);
+    v = std::max(1, std::min(v, 16));
+    if ((v & (v - 1)) != 0) v = 1;
+    // chunks run along the innermost dim of the fastest group and must not straddle it
+    const int fastDim = innermostDim(dirY_ ? 2 : 1);
+    const int64_t fastExtent = space_[static_cast<size_t>(fastDim)];
+    while (v > 1 && (fastExtent % v) != 0) v >>= 1;
+    vec_ = v;
+    const int64_t targetGroups = 2048;  // about 8 workgroups per CU
+    if (dirY_) {
+      lanes_ = std::min<int64_t>(64, pow2AtLeastL(ceilDivL(I_, vec_)));
+      const int tr = kBlock / lanes_;
+      strips_ = ceilDivL(I_, static_cast<int64_t>(lanes_) * vec_);
+      groups_ = O_ * strips_;
+      int64_t split = ceilDivL(targetGroups, groups_);
+      const int64_t maxSplit = std::max<int64_t>(1, R_ / (static_cast<int64_t>(tr) * 4));
+      split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), 256));
+      rps_ = ceilDivL(R_, split);
+      split_ = static_cast<int>(ceilDivL(R_, rps_));
+    } else {
+      lanes_ = kBlock;
+      strips_ = 1;
+      groups_ = O_;
+      const int64_t chunk = static_cast<int64_t>(kBlock) * vec_;
+      int64_t split = ceilDivL(targetGroups, groups_);
+      const int64_t maxSplit = std::max<int64_t>(1, R_ / (chunk * 2));
+      split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), kBlock));
+      rps_ = ceilDivL(ceilDivL(R_, split), chunk) * chunk;
+      split_ = static_cast<int>(ceilDivL(R_, rps_));
+    }
+    grid_ = groups_ * split_;
+    if (grid_ > 2147483647LL) throw LoweringError("grid too large");
+    // workspace: one arrival counter per group, then the partials of every reduction
+    workspaceBytes_ = 0;
+    partialOffset_.assign(reduces_.size(), 0);
+    if (split_ > 1) {
+      auto align = [](uint64_t x) { return (x + 255) / 256 * 256; };
+      uint64_t off = align(static_cast<uint64_t>(groups_) * 4);
+      const uint64_t width = dirY_ ? static_cast<uint64_t>(lanes_) * vec_ : 1;
+      for (size_t k = 0; k < reduces_.size(); ++k) {
+        partialOffset_[k] = off;
+        const uint64_t ctSize = std::max<size_t>(4, dtypeSize(g_.tensor(reduces_[k]->outputs[0]).dtype));
+        off = align(off + static_cast<uint64_t>(groups_) * split_ * width * ctSize);
+      }
+      workspaceBytes_ = off;
+    }
+  }
+
+  // ------------------------------------------------------------------ addressing
+  // Element offset of tensor `t` at the point (o, r, i) of the folded space, as an expression in `ov`, `rv`, `iv`
+  // (an empty variable name stands for index 0 of that group).
+  std::string offsetExpr(const TensorValue &t, const std::string &ov, const std::string &rv,
+                         const std::string &iv) const {
+    const std::vector<int64_t> s = padTo(t.shape, "tensor " + t.name);
+    const size_t n = space_.size();
+    std::vector<int64_t> stride(n, 0);
+    int64_t acc = 1;
+    for (size_t d = n; d-- > 0;) {
+      stride[d] = (s[d] == 1) ? 0 : acc;
+      acc *= s[d];
+    }
+    std::ostringstream e;
+    bool firstTerm = true;
+    auto term = [&](const std::string &text) {
+      e << (firstTerm ? "" : " + ") << text;
+      firstTerm = false;
+    };
+    const std::string vars[3] = {ov, rv, iv};
+    for (int group = 0; group < 3; ++group) {
+      const std::string &var = vars[group];
+      if (var.empty()) continue;
+      std::vector<size_t> dims;
+      for (size_t d = 0; d < n; ++d) {
+        if (kind_[d] == group) dims.push_back(d);
+      }
+      if (dims.empty()) continue;
+      // contiguous over the whole group: one multiply
+      bool contiguous = true, allZero = true;
+      for (size_t j = 0; j < dims.size(); ++j) {
+        if (stride[dims[j]] != 0) allZero = false;
+      }
+      int64_t expect = stride[dims.back()];
+      for (size_t j = dims.size(); j-- > 0;) {
+        if (stride[dims[j]] != expect) contiguous = false;
+        expect *= space_[dims[j]];
+      }
+      if (allZero) continue;
+      if (contiguous) {
+        term(var + " * " + std::to_string(stride[dims.back()]) + "L");
+        continue;
+      }
+      int64_t div = 1;
+      for (size_t j = dims.size(); j-- > 0;) {
+        const size_t d = dims[j];
+        if (stride[d] != 0) {
+          term("((" + var + " / " + std::to_string(div) + "L) % " + std::to_string(space_[d]) + "L) * " +
+               std::to_string(stride[d]) + "L");
+        }
+        div *= space_[d];
+      }
+    }
+    if (firstTerm) return "0L";
+    return "(" + e.str() + ")";
+  }
+
+  // Whether V consecutive positions of the fastest group are V consecutive elements of `t` (else: one element).
+  bool chunkContiguous(const TensorValue &t, int group) const {
+    const int d = innermostDim(group);
+    if (d < 0) return false;
+    const std::vector<int64_t> s = padTo(t.shape, "tensor " + t.name);
+    if (s[static_cast<size_t>(d)] == 1) return false;
+    for (size_t k = static_cast<size_t>(d) + 1; k < s.size(); ++k) {
+      if (s[k] != 1) return false;  // a kept/reduced dim of another group lies inside: stride is not 1
+    }
+    return true;
+  }
+
+  std::string memRef(const std::string &arg, const std::string &offset) const {
+    if (useBuffers_) return "b_" + arg + ", " + offset;
+    return arg + " + " + offset;
+  }
+
+  // ------------------------------------------------------------------ emission
+  std::string operandExpr(int id, bool scalarPost) const {
+    const TensorValue &t = g_.tensor(id);
+    if (t.isConst) return lowering::literalFor(t.dtype, t.constValue);
+    const std::string &nm = ident_[static_cast<size_t>(id)];
+    if (nm.empty()) throw LoweringError("internal: operand " + t.name + " used before definition");
+    return scalarPost ? nm : nm + "[e]";
+  }
+
+  void emitInputLoad(size_t index, const std::string &ov, const std::string &rv, const std::string &iv,
+                     const std::string &suffix, bool scalar, const std::string &indent) {
+    const int id = g_.inputs[index];
+    const TensorValue &t = g_.tensor(id);
+    const std::string tag = tagOf(id), ct = ctOf(id);
+    const std::string name = "t_in" + std::to_string(index) + suffix;
+    const std::string arg = "in" + std::to_string(index);
+    const std::string off = offsetExpr(t, ov, rv, iv);
+    const int fastGroup = dirY_ ? 2 : 1;
+    const bool fastVarGiven = !(fastGroup == 2 ? iv : rv).empty();
+    if (scalar) {
+      if (useBuffers_) {
+        src_ << indent << "const " << ct << " " << name << " = akg::load_one<" << tag << ">(b_" << arg << ", " << off << ");\n";
+      } else {
+        src_ << indent << "const " << ct << " " << name << " = " << tag << "::load(" << arg << "[" << off << "]);\n";
+      }
+    } else if (fastVarGiven && chunkContiguous(t, fastGroup)) {
+      const bool streamed = opt_.nonTemporal != 0 && t.numel() == O_ * R_ * I_;
+      src_ << indent << ct << " " << name << "[V];\n";
+      src_ << indent << "akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">(" << memRef(arg, off)
+           << ", " << name << ");\n";
+    } else {
+      src_ << indent << ct << " " << name << "[V];\n";
+      if (useBuffers_) {
+        src_ << indent << "akg::fill_chunk<" << tag << ", V>(" << name << ", akg::load_one<" << tag << ">(b_" << arg
+             << ", " << off << "));\n";
+      } else {
+        src_ << indent << "akg::fill_chunk<" << tag << ", V>(" << name << ", " << tag << "::load(" << arg << "[" << off
+             << "]));\n";
+      }
+    }
+    ident_[static_cast<size_t>(id)] = name;
+  }
+
+  void emitOp(const OpNode &op, bool scalar, const std::string &indent) {
+    const int outId = op.outputs[0];
+    std::vector<std::string> operands;
+    for (int in : op.inputs) operands.push_back(operandExpr(in, scalar));
+    const std::string expr = lowering::elementwiseExpr(g_, op, operands, relaxed_[static_cast<size_t>(outId)]);
+    const std::string name = (scalar ? "u" : "t") + std::to_string(outId);
+    if (scalar) {
+      src_ << indent << "const " << ctOf(outId) << " " << name << " = " << expr << ";  // " << op.name << " -> "
+           << g_.tensor(outId).name << "\n";
+    } else {
+      src_ << indent << ctOf(outId) << " " << name << "[V];  // " << op.name << " -> " << g_.tensor(outId).name << "\n";
+      src_ << indent << "#pragma unroll\n";
+      src_ << indent << "for (int e = 0; e < V; ++e) " << name << "[e] = " << expr << ";\n";
+    }
+    ident_[static_cast<size_t>(outId)] = name;
+  }
+
+  // Inputs that some op of `phase` reads directly.
+  std::vector<size_t> inputsUsedIn(Phase phase) const {
+    std::vector<bool> used(g_.inputs.size(), false);
+    for (const OpNode &op : g_.ops) {
+      const Phase p = phase_[static_cast<size_t>(op.outputs[0])];
+      const bool isReduce = lowering::isReduceKind(op.kind);
+      const Phase opPhase = isReduce ? Phase::Pre : p;  // a reduction consumes its operand in the streaming loop
+      if (opPhase != phase) continue;
+      for (int in : op.inputs) {
+        const TensorValue &t = g_.tensor(in);
+        if (t.inputIndex >= 0 && !t.isConst) used[static_cast<size_t>(t.inputIndex)] = true;
+      }
+    }
+    std::vector<size_t> out;
+    for (size_t i = 0; i < used.size(); ++i) {
+      if (used[i]) out.push_back(i);
+    }
+    return out;
+  }
+
+  void emit() {
+    ident_.assign(g_.tensors.size(), std::string());
+    relaxed_ = lowering::relaxedPrecisionTensors(g_);
+    const std::string kname = g_.name + "_kernel";
+    line("// Generated by the akg HIP lowering for gfx950. Op description: " + g_.name);
+    line("// family: stream_reduce (direction " + std::string(dirY_ ? "Y" : "X") + "), fusion class: " +
+         operatorTemplateName(g_.operatorTemplate));
+    line("#include \"akg_rt.hpp\"");
+    line("");
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << kname << "(";
+    size_t argc = 0;
+    for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
+    }
+    if (split_ > 1) src_ << (argc ? ", " : "") << "unsigned *__restrict__ akg_ws";
+    line(") {");
+    useBuffers_ = true;
+    auto tooLarge = [&](int id) {
+      return g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31);
+    };
+    for (int id : g_.inputs) useBuffers_ = useBuffers_ && !tooLarge(id);
+    for (int id : g_.outputs) useBuffers_ = useBuffers_ && !tooLarge(id);
+    if (useBuffers_) {
+      for (size_t i = 0; i < g_.inputs.size(); ++i) {
+        const TensorValue &t = g_.tensor(g_.inputs[i]);
+        src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", "
+             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+      }
+      for (size_t i = 0; i < g_.outputs.size(); ++i) {
+        const TensorValue &t = g_.tensor(g_.outputs[i]);
+        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", "
+             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+      }
+    }
+    src_ << "  constexpr int V = " << vec_ << ";\n";
+    src_ << "  constexpr int BLOCK = " << kBlock << ";\n";
+    src_ << "  constexpr int LANES = " << lanes_ << ";\n";
+    src_ << "  constexpr long O = " << O_ << "L, R = " << R_ << "L, I = " << I_ << "L;\n";
+    src_ << "  constexpr long STRIPS = " << strips_ << "L;\n";
+    src_ << "  constexpr int SPLIT = " << split_ << ";\n";
+    src_ << "  constexpr long RPS = " << rps_ << "L;\n";
+    line("  (void)O; (void)I; (void)STRIPS;");
+    line("  const int tid = static_cast<int>(threadIdx.x);");
+    line("  const long akg_wg = static_cast<long>(blockIdx.x);");
+    line("  const long akg_s = akg_wg % SPLIT;");
+    line("  const long akg_group = akg_wg / SPLIT;");
+    line("  const long r_begin = akg_s * RPS;");
+    line("  const long r_end = (r_begin + RPS < R) ? (r_begin + RPS) : R;");
+    if (dirY_) {
+      line("  constexpr int TR = BLOCK / LANES;");
+      line("  const int li = tid % LANES;");
+      line("  const int tr = tid / LANES;");
+      line("  const long akg_o = akg_group / STRIPS;");
+      line("  const long akg_i_raw = ((akg_group % STRIPS) * LANES + li) * V;");
+      line("  const bool col_ok = akg_i_raw < I;");
+      line("  const long akg_i = col_ok ? akg_i_raw : 0L;");
+    } else {
+      line("  const long akg_o = akg_group;");
+      line("  __shared__ double akg_scratch[2][BLOCK / 64];");
+    }
+    line("");
+    // accumulators
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      const OpNode &op = *reduces_[k];
+      const DType od = g_.tensor(op.outputs[0]).dtype;
+      const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+      if (dirY_) {
+        src_ << "  " << computeTypeName(od) << " acc" << k << "[V];  // " << op.name << " -> "
+             << g_.tensor(op.outputs[0]).name << "\n";
+        line("#pragma unroll");
+        src_ << "  for (int e = 0; e < V; ++e) acc" << k << "[e] = " << spec.init << ";\n";
+      } else {
+        src_ << "  " << computeTypeName(od) << " acc" << k << " = " << spec.init << ";  // " << op.name << " -> "
+             << g_.tensor(op.outputs[0]).name << "\n";
+      }
+    }
+    // ---- streaming loop
+    line("#pragma unroll 2");
+    if (dirY_) {
+      line("  for (long r = r_begin + tr; r < r_end; r += TR) {");
+    } else {
+      line("  for (long r = r_begin + static_cast<long>(tid) * V; r < r_end; r += static_cast<long>(BLOCK) * V) {");
+    }
+    const std::string in4 = "    ";
+    for (size_t i : inputsUsedIn(Phase::Pre)) emitInputLoad(i, "akg_o", "r", dirY_ ? "akg_i" : "", "", false, in4);
+    for (const OpNode &op : g_.ops) {
+      const int out = op.outputs[0];
+      if (lowering::isReduceKind(op.kind)) {
+        size_t k = 0;
+        while (reduces_[k] != &op) ++k;
+        const DType od = g_.tensor(out).dtype;
+        const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+        const std::string val = operandExpr(op.inputs[0], false);
+        const std::string accName = "acc" + std::to_string(k) + (dirY_ ? "[e]" : "");
+        std::string step = spec.combiner + "::apply(" + accName + ", " + val + ")";
+        if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
+        src_ << in4 << "#pragma unroll\n";
+        src_ << in4 << "for (int e = 0; e < V; ++e) " << accName << " = " << step << ";\n";
+        continue;
+      }
+      if (phase_[static_cast<size_t>(out)] != Phase::Pre) continue;
+      emitOp(op, false, in4);
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      const int id = g_.outputs[i];
+      if (phase_[static_cast<size_t>(id)] != Phase::Pre) continue;
+      const std::string off = dirY_ ? "(akg_o * R + r) * I + akg_i" : "akg_o * R + r";
+      src_ << in4 << (dirY_ ? "if (col_ok) " : "") << "akg::store_chunk<" << tagOf(id) << ", V, "
+           << (opt_.nonTemporal != 0 ? "true" : "false") << ">(" << memRef("out" + std::to_string(i), off) << ", "
+           << ident_[static_cast<size_t>(id)] << ");\n";
+    }
+    line("  }");
+    line("");
+    if (dirY_) {
+      emitCombineY();
+    } else {
+      emitCombineX();
+    }
+    line("}");
+  }
+
+  // Sum of the TR thread-rows of the workgroup into thread-row 0 (fixed order), through LDS.
+  void emitRowCombineY(const std::string &ldsPrefix) {
+    line("  if (TR > 1) {");
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      line("#pragma unroll");
+      src_ << "    for (int e = 0; e < V; ++e) " << ldsPrefix << k << "[tr][li * V + e] = acc" << k << "[e];\n";
+    }
+    line("    __syncthreads();");
+    line("    if (tr == 0) {");
+    line("      for (int t = 1; t < TR; ++t) {");
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      const OpNode &op = *reduces_[k];
+      const DType od = g_.tensor(op.outputs[0]).dtype;
+      const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+      std::string step = spec.combiner + "::apply(acc" + std::to_string(k) + "[e], " + ldsPrefix + std::to_string(k) +
+                         "[t][li * V + e])";
+      if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
+      line("#pragma unroll");
+      src_ << "        for (int e = 0; e < V; ++e) acc" << k << "[e] = " << step << ";\n";
+    }
+    line("      }");
+    line("    }");
+    line("  }");
+  }
+
+  void emitCombineY() {
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      const DType od = g_.tensor(reduces_[k]->outputs[0]).dtype;
+      src_ << "  __shared__ " << computeTypeName(od) << " akg_lds" << k << "[TR > 1 ? TR : 1][LANES * V];\n";
+    }
+    emitRowCombineY("akg_lds");
+    if (split_ > 1) {
+      line("  // ---- partials of this workgroup -> workspace; the last workgroup of the group to arrive finishes the job");
+      line("  unsigned char *akg_wsb = reinterpret_cast<unsigned char *>(akg_ws);");
+      for (size_t k = 0; k < reduces_.size(); ++k) {
+        const std::string ct = computeTypeName(g_.tensor(reduces_[k]->outputs[0]).dtype);
+        src_ << "  " << ct << " *part" << k << " = reinterpret_cast<" << ct << " *>(akg_wsb + " << partialOffset_[k]
+             << "UL) + akg_group * (static_cast<long>(SPLIT) * LANES * V) + li * V;\n";
+        line("  if (tr == 0) {");
+        line("#pragma unroll");
+        src_ << "    for (int e = 0; e < V; ++e) akg::ws_store(part" << k << " + akg_s * (LANES * V) + e, acc" << k
+             << "[e]);\n";
+        line("  }");
+      }
+      line("  __shared__ unsigned akg_flag;");
+      line("  if (!akg::last_workgroup(akg_ws, akg_group, SPLIT, tid, &akg_flag)) return;");
+      for (size_t k = 0; k < reduces_.size(); ++k) {
+        const OpNode &op = *reduces_[k];
+        const DType od = g_.tensor(op.outputs[0]).dtype;
+        const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+        line("#pragma unroll");
+        src_ << "  for (int e = 0; e < V; ++e) acc" << k << "[e] = " << spec.init << ";\n";
+        line("  for (long p = tr; p < SPLIT; p += TR) {");
+        std::string step = spec.combiner + "::apply(acc" + std::to_string(k) + "[e], akg::ws_load(part" +
+                           std::to_string(k) + " + p * (LANES * V) + e))";
+        if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
+        line("#pragma unroll");
+        src_ << "    for (int e = 0; e < V; ++e) acc" << k << "[e] = " << step << ";\n";
+        line("  }");
+      }
+      emitRowCombineY("akg_lds");
+    }
+    // ---- post phase: thread-row 0 holds the reduced values of its V columns
+    line("  if (tr != 0 || !col_ok) return;");
+    emitPost(false);
+  }
+
+  void emitCombineX() {
+    int scratchUse = 0;
+    auto blockReduce = [&](size_t k, const std::string &target) {
+      const OpNode &op = *reduces_[k];
+      const DType od = g_.tensor(op.outputs[0]).dtype;
+      const std::string ct = computeTypeName(od);
+      const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+      src_ << "  " << target << " = " << (spec.roundEachStep ? std::string(dtypeTag(od)) + "::rnd(" : "")
+           << "akg::group_reduce<" << spec.combiner << ", BLOCK>(acc" << k << ", reinterpret_cast<" << ct
+           << " *>(akg_scratch[" << (scratchUse & 1) << "]), tid)" << (spec.roundEachStep ? ")" : "") << ";\n";
+      ++scratchUse;
+    };
+    for (size_t k = 0; k < reduces_.size(); ++k) blockReduce(k, "acc" + std::to_string(k));
+    if (split_ > 1) {
+      line("  // ---- partial of this workgroup -> workspace; the last workgroup of the group to arrive finishes the job");
+      line("  unsigned char *akg_wsb = reinterpret_cast<unsigned char *>(akg_ws);");
+      for (size_t k = 0; k < reduces_.size(); ++k) {
+        const std::string ct = computeTypeName(g_.tensor(reduces_[k]->outputs[0]).dtype);
+        src_ << "  " << ct << " *part" << k << " = reinterpret_cast<" << ct << " *>(akg_wsb + " << partialOffset_[k]
+             << "UL) + akg_group * SPLIT;\n";
+        src_ << "  if (tid == 0) akg::ws_store(part" << k << " + akg_s, acc" << k << ");\n";
+      }
+      line("  __shared__ unsigned akg_flag;");
+      line("  if (!akg::last_workgroup(akg_ws, akg_group, SPLIT, tid, &akg_flag)) return;");
+      for (size_t k = 0; k < reduces_.size(); ++k) {
+        const OpNode &op = *reduces_[k];
+        const lowering::ReduceSpec spec = lowering::reduceSpec(op, g_.tensor(op.outputs[0]).dtype);
+        src_ << "  acc" << k << " = (tid < SPLIT) ? akg::ws_load(part" << k << " + tid) : " << spec.init << ";\n";
+        blockReduce(k, "acc" + std::to_string(k));
+      }
+    }
+    emitPost(true);
+  }
+
+  void emitPost(bool scalar) {
+    const std::string in2 = "  ";
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      const OpNode &op = *reduces_[k];
+      const int out = op.outputs[0];
+      // the accumulator is the value of the reduction's result tensor
+      ident_[static_cast<size_t>(out)] = "acc" + std::to_string(k);
+    }
+    // graph inputs read by post ops: at index 0 of the reduced group
+    for (int id : g_.inputs) ident_[static_cast<size_t>(id)].clear();
+    for (size_t i : inputsUsedIn(Phase::Post)) {
+      emitInputLoad(i, "akg_o", "", scalar ? "" : "akg_i", "_post", scalar, in2);
+    }
+    for (const OpNode &op : g_.ops) {
+      if (lowering::isReduceKind(op.kind)) continue;
+      if (phase_[static_cast<size_t>(op.outputs[0])] != Phase::Post) continue;
+      emitOp(op, scalar, in2);
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      const int id = g_.outputs[i];
+      if (phase_[static_cast<size_t>(id)] != Phase::Post) continue;
+      const std::string tag = tagOf(id);
+      if (scalar) {
+        if (useBuffers_) {
+          src_ << "  if (tid == 0) akg::store_one<" << tag << ">(b_out" << i << ", akg_o, " << ident_[static_cast<size_t>(id)]
+               << ");\n";
+        } else {
+          src_ << "  if (tid == 0) out" << i << "[akg_o] = " << tag << "::store(" << ident_[static_cast<size_t>(id)] << ");\n";
+        }
+      } else {
+        src_ << "  akg::store_chunk<" << tag << ", V, false>(" << memRef("out" + std::to_string(i), "akg_o * I + akg_i")
+             << ", " << ident_[static_cast<size_t>(id)] << ");\n";
+      }
+    }
+  }
+};
+
+}  // namespace
+
+bool wantsStreamReduce(const OpGraph &graph) {
+  const OpNode *first = nullptr;
+  for (const OpNode &op : graph.ops) {
+    if (lowering::isReduceKind(op.kind)) {
+      first = &op;
+      break;
+    }
+  }
+  if (first == nullptr) return false;
+  const TensorValue &in = graph.tensor(first->inputs[0]);
+  const std::vector<size_t> axes = realReducedAxes(graph, *first);
+  if (axes.empty()) return false;
+  // innermost non-unit dim
+  size_t last = in.shape.size();
+  for (size_t d = in.shape.size(); d-- > 0;) {
+    if (in.shape[d] > 1) {
+      last = d;
+      break;
+    }
+  }
+  const bool innermostOnly = axes.size() == 1 && axes[0] == last;
+  if (!innermostOnly) return true;
+  // direction X: the row kernel keeps a whole row in registers and gives every row its own threads. Rows beyond its
+  // capacity, or so few long rows that the chip would idle, stream instead — unless some op needs the row again
+  // after the reduction (softmax, LayerNorm), which only the row kernel can serve.
+  const int64_t cols = in.shape[last];
+  const int64_t rows = in.numel() / cols;
+  const bool tooLong = cols > 131072;
+  const bool tooFew = rows < 64 && cols >= 32768;
+  if (!tooLong && !tooFew) return false;
+  std::vector<bool> post(graph.tensors.size(), false);
+  for (const OpNode &op : graph.ops) {
+    bool anyPost = false, anyFull = false;
+    for (int id : op.inputs) {
+      const TensorValue &t = graph.tensor(id);
+      if (t.isConst) continue;
+      if (post[static_cast<size_t>(id)]) {
+        anyPost = true;
+      } else if (t.numel() == in.numel()) {
+        anyFull = true;
+      }
+    }
+    if (lowering::isReduceKind(op.kind)) {
+      post[static_cast<size_t>(op.outputs[0])] = true;
+    } else if (anyPost) {
+      if (anyFull) return false;  // the row is needed again
+      post[static_cast<size_t>(op.outputs[0])] = true;
+    }
+  }
+  return true;
+}
+
+LoweredKernel lowerStreamReduceToHip(const OpGraph &graph, const LoweringOptions &options) {
+  StreamReduceEmitter emitter(graph, options);
+  return emitter.run();
+}
+
+}  // namespace akg

@@ -45,6 +45,7 @@ struct akg_hip_kernel {
     int device = -1;
     hipModule_t module = nullptr;
     hipFunction_t function = nullptr;
+    void *workspace = nullptr;  // lowered.workspaceBytes of zero-filled device memory, or NULL
   };
   std::vector<Loaded> loaded;
 };
@@ -203,6 +204,7 @@ std::string metaJson(const akg_hip_kernel &k, const std::string &srcDigest) {
   os << "\"schedule\": \"" << jsonEscape(k.lowered.scheduleNote) << "\", ";
   os << "\"algorithmic_bytes\": " << k.lowered.algorithmicBytes << ", ";
   os << "\"algorithmic_ops\": " << k.lowered.algorithmicOps << ", ";
+  os << "\"workspace_bytes\": " << k.lowered.workspaceBytes << ", ";
   os << "\"source_sha256\": \"" << srcDigest << "\"";
   os << "}";
   return os.str();
@@ -286,14 +288,15 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
   return AKG_HIP_OK;
 }
 
-int ensureLoaded(akg_hip_kernel *k, hipFunction_t *fn) {
+// Code object and workspace of `k` on the current device, loaded / allocated on first use.
+int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipGetDevice: " + hipErr(e));
   std::lock_guard<std::mutex> lock(k->mu);
   for (const auto &l : k->loaded) {
     if (l.device == device) {
-      *fn = l.function;
+      *out = l;
       return AKG_HIP_OK;
     }
   }
@@ -306,8 +309,19 @@ int ensureLoaded(akg_hip_kernel *k, hipFunction_t *fn) {
     (void)hipModuleUnload(l.module);
     return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + k->lowered.kernelName + "): " + hipErr(e));
   }
+  if (k->lowered.workspaceBytes > 0) {
+    // Zero-filled once; every launch leaves the arrival counters at zero again. Launches of one handle share the
+    // workspace, so they must not overlap on the device (launch them on one stream, or order the streams).
+    e = hipMalloc(&l.workspace, k->lowered.workspaceBytes);
+    if (e == hipSuccess) e = hipMemset(l.workspace, 0, k->lowered.workspaceBytes);
+    if (e != hipSuccess) {
+      if (l.workspace) (void)hipFree(l.workspace);
+      (void)hipModuleUnload(l.module);
+      return fail(AKG_HIP_ERR_RUNTIME, "workspace of " + std::to_string(k->lowered.workspaceBytes) + " bytes: " + hipErr(e));
+    }
+  }
   k->loaded.push_back(l);
-  *fn = l.function;
+  *out = l;
   return AKG_HIP_OK;
 }
 
@@ -319,15 +333,16 @@ const akg::TensorValue &tensorAt(const akg_hip_kernel *k, int index) {
   return k->graph.tensor(k->graph.outputs[static_cast<size_t>(index) - nin]);
 }
 
-int launchOn(akg_hip_kernel *k, hipFunction_t fn, void *const *devicePtrs, hipStream_t stream) {
-  int n = numTensors(k);
-  std::vector<void *> slots(static_cast<size_t>(n));
-  std::vector<void *> params(static_cast<size_t>(n));
-  for (int i = 0; i < n; ++i) {
-    slots[static_cast<size_t>(i)] = devicePtrs[i];
+int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream) {
+  const int n = numTensors(k);
+  const int nargs = n + (l.workspace ? 1 : 0);  // the workspace is the kernel's trailing argument
+  std::vector<void *> slots(static_cast<size_t>(nargs));
+  std::vector<void *> params(static_cast<size_t>(nargs));
+  for (int i = 0; i < nargs; ++i) {
+    slots[static_cast<size_t>(i)] = i < n ? devicePtrs[i] : l.workspace;
     params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
   }
-  hipError_t e = hipModuleLaunchKernel(fn, k->lowered.grid[0], k->lowered.grid[1], k->lowered.grid[2],
+  hipError_t e = hipModuleLaunchKernel(l.function, k->lowered.grid[0], k->lowered.grid[1], k->lowered.grid[2],
                                        k->lowered.block[0], k->lowered.block[1], k->lowered.block[2], 0, stream,
                                        params.data(), nullptr);
   if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLaunchKernel: " + hipErr(e));
@@ -410,6 +425,7 @@ int akg_hip_kernel_get_info(const akg_hip_kernel_t *kernel, akg_hip_kernel_info 
   info->algorithmic_bytes = kernel->lowered.algorithmicBytes;
   info->algorithmic_ops = kernel->lowered.algorithmicOps;
   info->cache_hit = kernel->cacheHit ? 1 : 0;
+  info->workspace_bytes = kernel->lowered.workspaceBytes;
   return AKG_HIP_OK;
 }
 
@@ -422,16 +438,22 @@ int akg_hip_kernel_source(const akg_hip_kernel_t *kernel, const char **source) {
 int akg_hip_launch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream) {
   int rc = checkPtrs(kernel, device_ptrs, n_ptrs);
   if (rc != AKG_HIP_OK) return rc;
-  hipFunction_t fn = nullptr;
+  akg_hip_kernel::Loaded fn;
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   return launchOn(kernel, fn, device_ptrs, static_cast<hipStream_t>(stream));
 }
 
+int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel) {
+  if (kernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel is NULL");
+  akg_hip_kernel::Loaded l;
+  return ensureLoaded(kernel, &l);
+}
+
 int akg_hip_run_host(akg_hip_kernel_t *kernel, void *const *host_ptrs, int n_ptrs) {
   int rc = checkPtrs(kernel, host_ptrs, n_ptrs);
   if (rc != AKG_HIP_OK) return rc;
-  hipFunction_t fn = nullptr;
+  akg_hip_kernel::Loaded fn;
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   const int n = numTensors(kernel);
@@ -485,7 +507,7 @@ int akg_hip_profile(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_pt
   if (avg_ms == nullptr || number <= 0 || repeat <= 0) {
     return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "number and repeat must be positive and avg_ms non-NULL");
   }
-  hipFunction_t fn = nullptr;
+  akg_hip_kernel::Loaded fn;
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   hipStream_t stream = nullptr;
@@ -525,6 +547,7 @@ int akg_hip_profile(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_pt
 void akg_hip_kernel_destroy(akg_hip_kernel_t *kernel) {
   if (kernel == nullptr) return;
   for (auto &l : kernel->loaded) {
+    if (l.workspace) (void)hipFree(l.workspace);
     if (l.module) (void)hipModuleUnload(l.module);
   }
   delete kernel;

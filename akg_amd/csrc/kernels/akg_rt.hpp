@@ -687,4 +687,39 @@ AKG_DEV T group_reduce(T v, T *scratch, int tid) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Workspace protocol of the streaming reductions. Several workgroups share one group of outputs; each leaves
+// its partial result in device memory and counts its arrival; the workgroup that arrives last reads all the
+// partials back (in slot order, so the result does not depend on the arrival order) and finishes the job.
+// The eight XCDs have private L2 caches: partials are written and read with device-scope accesses, and the
+// arrival counter is an acquire/release device-scope atomic, so the last workgroup sees every partial
+// whichever XCD produced it. The last workgroup puts the counter back to zero: the workspace is zero-filled
+// once when it is allocated and every launch leaves it as it found it.
+// ---------------------------------------------------------------------------------------------------------
+template <typename T>
+AKG_DEV void ws_store(T *p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+AKG_DEV T ws_load(const T *p) {
+  return __hip_atomic_load(const_cast<T *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// True in every thread of exactly one workgroup out of the `split` that share counter `group`: the last to arrive.
+// Must be reached by all threads of the workgroup, after their ws_store calls.
+AKG_DEV bool last_workgroup(unsigned *counters, long group, int split, int tid, unsigned *flag) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned prev = __hip_atomic_fetch_add(counters + group, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = prev == static_cast<unsigned>(split - 1);
+    if (last) __hip_atomic_store(counters + group, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *flag = last ? 1u : 0u;
+  }
+  __syncthreads();
+  const bool last = *flag != 0u;
+  if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  return last;
+}
+
 }  // namespace akg

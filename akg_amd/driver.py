@@ -38,7 +38,7 @@ class _KernelInfo(ctypes.Structure):
     _fields_ = [("kernel_name", ctypes.c_char * 256), ("family", ctypes.c_char * 32),
                 ("operator_type", ctypes.c_char * 32), ("grid", ctypes.c_uint32 * 3), ("block", ctypes.c_uint32 * 3),
                 ("algorithmic_bytes", ctypes.c_uint64), ("algorithmic_ops", ctypes.c_uint64),
-                ("cache_hit", ctypes.c_int32)]
+                ("cache_hit", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64)]
 
 
 _lib = None
@@ -65,6 +65,7 @@ def load_library():
     lib.akg_hip_kernel_tensor.argtypes = [vp, ci, ctypes.POINTER(_TensorDesc)]
     lib.akg_hip_kernel_get_info.argtypes = [vp, ctypes.POINTER(_KernelInfo)]
     lib.akg_hip_kernel_source.argtypes = [vp, ctypes.POINTER(cp)]
+    lib.akg_hip_kernel_prepare.argtypes = [vp]
     lib.akg_hip_launch.argtypes = [vp, ctypes.POINTER(vp), ci, vp]
     lib.akg_hip_run_host.argtypes = [vp, ctypes.POINTER(vp), ci]
     lib.akg_hip_profile.argtypes = [vp, ctypes.POINTER(vp), ci, ci, ci, ctypes.POINTER(ctypes.c_double)]
@@ -137,6 +138,7 @@ class HipKernel:
         self.algorithmic_bytes = int(info.algorithmic_bytes)
         self.algorithmic_ops = int(info.algorithmic_ops)
         self.cache_hit = bool(info.cache_hit)
+        self.workspace_bytes = int(info.workspace_bytes)
 
     @classmethod
     def from_file(cls, info_path, out_dir=DEFAULT_META_DIR):
@@ -166,6 +168,10 @@ class HipKernel:
         if len(ptrs) != len(self.tensors):
             raise ValueError("kernel %s takes %d tensors, %d given" % (self.kernel_name, len(self.tensors), len(ptrs)))
         return (ctypes.c_void_p * len(ptrs))(*ptrs)
+
+    def prepare(self):
+        """Load the code object and allocate the workspace on the current device (later launches allocate nothing)."""
+        _check(self._lib.akg_hip_kernel_prepare(self._handle))
 
     # -- device-resident path (the hot call) -------------------------------------------------------------
     def launch_ptrs(self, device_ptrs, stream=None):

@@ -34,6 +34,19 @@ FIXTURES = {
     "small_quant_int8_residual_bf16_37x1544": lambda n: op_desc.quant_int8_residual(37, 1544, "bfloat16", n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", True, n),
+    # streaming reductions: direction Y, direction ALL, long rows, multi-output
+    "small_reducey_sqsum_f32_1x5100x3072": lambda n: op_desc.square_reduce([1, 5100, 3072], [1], "float32", True, "ReduceSum", n),
+    "small_reducey_sqsum_f32_3x37x50": lambda n: op_desc.square_reduce([3, 37, 50], [1], "float32", False, "ReduceSum", n),
+    "small_reducey_max_f16_130x66": lambda n: op_desc.square_reduce([130, 66], [0], "float16", False, "ReduceMax", n),
+    "small_reduceall_sqsum_f32_768x512": lambda n: op_desc.square_reduce([768, 512], [0, 1], "float32", False, "ReduceSum", n),
+    "small_reduceall_min_f32_7x333": lambda n: op_desc.square_reduce([7, 333], [0, 1], "float32", False, "ReduceMin", n),
+    "small_reducex_long_sqsum_f32_3x300000": lambda n: op_desc.square_reduce([3, 300000], [1], "float32", False, "ReduceSum", n),
+    "small_biasgrad_bf16_2048x1024": lambda n: op_desc.bias_grad(2048, 1024, "bfloat16", n),
+    "small_biasgrad_f32_100x37": lambda n: op_desc.bias_grad(100, 37, "float32", n),
+    "small_sub_exp_reducesum_split_f32_4x96x160": lambda n: op_desc.sub_exp_reduce_y(4, 96, 160, "float32", n),
+    "small_mean_absmax_all_f32_1000x1000": lambda n: op_desc.mean_absmax_all(1000, 1000, "float32", n),
+    # the next measured row: bias / scale gradients of a [16384, 4096] bf16 activation (two column sums in one pass)
+    "n1_biasgrad_bf16_16384x4096": lambda n: op_desc.bias_grad(16384, 4096, "bfloat16", n),
 }
 
 

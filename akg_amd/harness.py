@@ -142,3 +142,29 @@ def compare(actual, expected, dtype):
         err = np.abs(a - e)
         rel = np.nanmax(np.where(np.abs(e) > 0, err / np.abs(e), 0.0)) if a.size else 0.0
     return True, "max abs err %.3g, max rel err %.3g" % (float(np.nanmax(err)) if a.size else 0.0, float(rel))
+
+
+def widen_to_float64(desc):
+    """The same description with every float32 tensor, cast target and constant declared float64: evaluated by the
+    oracle it gives the fused expression with (nearly) exact accumulation, whatever the order of a summation."""
+    text = json.dumps(desc).replace('"float32"', '"float64"')
+    return json.loads(text)
+
+
+def compare_reassociated(actual, exact64, dtype, terms):
+    """Bar for a float32 result that went through a reduction of `terms` values in another order than the serial
+    loop: rtol 1e-5 against the float64-accumulated value, plus an absolute allowance of 1e-6 * sqrt(terms) for
+    sums of O(1) terms that cancel (the float32 rounding of the partial sums, which no order avoids)."""
+    if dtype != "float32":
+        return compare(actual, exact64, dtype)
+    a, e = np.asarray(actual, dtype=np.float64), np.asarray(exact64, dtype=np.float64).reshape(np.shape(actual))
+    atol = 1e-6 * float(np.sqrt(max(1, terms)))
+    close = np.isclose(a, e, rtol=1e-5, atol=atol, equal_nan=True)
+    if not close.all():
+        idx = tuple(np.argwhere(~close)[0])
+        return False, "%d of %d elements outside rtol=1e-5 atol=%g of the float64 value; first at %s: %r vs %r" % (
+            np.count_nonzero(~close), a.size, atol, idx, a[idx], e[idx])
+    err = np.abs(a - e)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        rel = np.nanmax(np.where(np.abs(e) > 0, err / np.abs(e), 0.0)) if a.size else 0.0
+    return True, "vs float64: max abs err %.3g, max rel err %.3g" % (float(err.max()) if a.size else 0.0, float(rel))

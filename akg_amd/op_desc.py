@@ -224,3 +224,54 @@ def gemm_int8_dequant_bias_gelu(m, k, n, out_dtype="bfloat16", transpose_b=False
     g = b.mul(b.mul(x, b.add(b.unary("Tanh", inner), b.const(1.0, "float32"))), b.const(0.5, "float32"))
     out = b.cast(g, out_dtype) if out_dtype != "float32" else g
     return b.dumps([out])
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Streaming-reduction patterns (reduce direction Y and ALL, multi-output fusions).
+# ---------------------------------------------------------------------------------------------------------
+_SHORT = {"float16": "f16", "bfloat16": "bf16", "float32": "f32", "int32": "i32"}
+
+
+def square_reduce(shape, axes, dtype="float32", keep_dims=False, op="ReduceSum", name=None):
+    """out = Reduce(x * x) over `axes`, e.g. [1,5100,3072] over axis 1 (reduce direction Y) or [768,512] over
+    both axes (direction ALL). 16-bit inputs are cast to float32 first and the result is cast back."""
+    b = DescBuilder(name or "Fused_Mul_%s_%s_%s_axes%s" % (
+        op, _SHORT[dtype], "x".join(str(d) for d in shape), "_".join(str(a) for a in axes)))
+    x = b.input(list(shape), dtype)
+    wide = dtype in ("float16", "bfloat16")
+    v = b.cast(x, "float32") if wide else x
+    r = b.reduce(op, b.mul(v, v), list(axes), keep_dims)
+    return b.dumps([b.cast(r, dtype) if wide else r])
+
+
+def bias_grad(rows, cols, dtype="bfloat16", name=None):
+    """Gradients of `y = x * gamma + beta` for dy [rows, cols]: dgamma = sum_rows(dy * x), dbeta = sum_rows(dy),
+    both [cols] float32. Two column reductions (direction Y) of one pass over dy and x."""
+    b = DescBuilder(name or "Fused_Mul_ReduceSum_ReduceSum_biasgrad_%s_%dx%d" % (_SHORT[dtype], rows, cols))
+    dy = b.input([rows, cols], dtype)
+    x = b.input([rows, cols], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    dyf = f(dy)
+    dgamma = b.reduce("ReduceSum", b.mul(dyf, f(x)), [0], False)
+    dbeta = b.reduce("ReduceSum", dyf, [0], False)
+    return b.dumps([dgamma, dbeta])
+
+
+def sub_exp_reduce_y(outer, reduced, inner, dtype="float32", name=None):
+    """Two outputs, as the reference's Fused_Sub_Exp_ReduceSum_split: e = exp(x - m) (full shape, stored while
+    streaming) and s = sum over the middle axis of e, with m broadcast along the reduced axis."""
+    b = DescBuilder(name or "Fused_Sub_Exp_ReduceSum_split_%s_%dx%dx%d" % (_SHORT[dtype], outer, reduced, inner))
+    x = b.input([outer, reduced, inner], dtype)
+    m = b.input([outer, 1, inner], dtype)
+    e = b.unary("Exp", b.sub(x, m))
+    s = b.reduce("ReduceSum", e, [1], True)
+    return b.dumps([e, s])
+
+
+def mean_absmax_all(rows, cols, dtype="float32", name=None):
+    """Two reductions over every axis with ops after them: mean = sum(x) / N and amax = max(|x|), both [1]."""
+    b = DescBuilder(name or "Fused_ReduceSum_Abs_ReduceMax_all_%s_%dx%d" % (_SHORT[dtype], rows, cols))
+    x = b.input([rows, cols], dtype)
+    mean = b.mul(b.reduce("ReduceSum", x, [0, 1], False), b.const(1.0 / (rows * cols), dtype))
+    amax = b.reduce("ReduceMax", b.unary("Abs", x), [0, 1], False)
+    return b.dumps([mean, amax])

@@ -32,6 +32,8 @@ WORKLOADS = {
     "c3_layernorm_residual_bf16_16384x4096": "f32",
     "c4_quant_int8_residual_bf16_32768x8192": "f32",
     "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": "int8",
+    # the row next to the five: two column sums (reduce direction Y) of one pass over two bf16 [16384,4096] tensors
+    "n1_biasgrad_bf16_16384x4096": "f32",
 }
 DEFAULT_WORKLOAD = "c2_softmax_f16_8192x4096"
 # plain streaming kernel of known size (out = -x, 256 MiB in + 256 MiB out): calibrates the HBM traffic counters

@@ -57,13 +57,14 @@ typedef struct akg_hip_tensor_desc {
 
 typedef struct akg_hip_kernel_info {
   char kernel_name[256];              /* "<op>_kernel" (KernelOutliningExt.cpp:433) */
-  char family[32];                    /* "elementwise" | "row_reduce" | "gemm_epilogue" */
+  char family[32];                    /* "elementwise" | "row_reduce" | "stream_reduce" | "gemm_epilogue" */
   char operator_type[32];             /* fusion class, OperatorIdentify.cpp:51-93 */
   uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json */
   uint32_t block[3];                  /* threadIdx.x/y/z extents */
   uint64_t algorithmic_bytes;         /* bytes of every input and output, each counted once */
   uint64_t algorithmic_ops;           /* 2*M*N*K of the contraction, 0 for bandwidth-bound families */
   int32_t cache_hit;                  /* 1 if the code object came from the artifact directory */
+  uint64_t workspace_bytes;           /* device scratch the handle owns per device (streaming reductions), else 0 */
 } akg_hip_kernel_info;
 
 typedef struct akg_hip_kernel akg_hip_kernel_t;
@@ -100,8 +101,18 @@ int akg_hip_kernel_get_info(const akg_hip_kernel_t *kernel, akg_hip_kernel_info 
 int akg_hip_kernel_source(const akg_hip_kernel_t *kernel, const char **source);
 
 /**
+ * Load the code object on the current device and allocate the handle's workspace there (workspace_bytes of
+ * kernel_info; zero for every family but the streaming reductions), so that later launches on this device
+ * allocate nothing. Optional: the first akg_hip_launch on a device does the same. Replaces the cuModuleLoadData /
+ * cuModuleGetFunction prologue of the generated shim (code_template.py:180-203).
+ */
+int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel);
+
+/**
  * The hot call: enqueue the kernel on `stream` (a hipStream_t, NULL for the default stream) with one DEVICE
- * pointer per argument, inputs then outputs. Asynchronous; allocates nothing. Replaces the cuLaunchKernel
+ * pointer per argument, inputs then outputs. Asynchronous; after the first call on a device (or
+ * akg_hip_kernel_prepare) it allocates nothing. Launches of one handle whose workspace_bytes is non-zero share
+ * that workspace and must not overlap on the device. Replaces the cuLaunchKernel
  * step of the generated shim (code_template.py:204) without its per-call context creation, module load,
  * cuMemAlloc and copies.
  */

@@ -496,6 +496,9 @@ class Emitter:
         for k, d in enumerate(par):
             self.emit("for (int64_t i%d = 0; i%d < %dL; ++i%d) {" % (d, d, in_shape[d], d), depth + k)
         depth += len(par)
+        if not par:
+            self.emit("{", depth)  # a reduction over every axis: its accumulator gets a scope of its own
+            depth += 1
         self.emit("%s acc = %s;" % (ct, inits[op.name]), depth)
         for k, d in enumerate(axes):
             self.emit("for (int64_t i%d = 0; i%d < %dL; ++i%d) {" % (d, d, in_shape[d], d), depth + k)
@@ -522,6 +525,8 @@ class Emitter:
         for d in par:
             expr = "i%d" % d if expr is None else "(%s) * %dL + i%d" % (expr, in_shape[d], d)
         self.emit("%s[%s] = %s;" % (out.buffer, expr or "0", self.store_expr(od, "acc")), depth)
+        if not par:
+            self.emit("}", depth - 1)
         for k in range(len(par)):
             self.emit("}", depth - 1 - k)
         _ = order

@@ -16,7 +16,10 @@ from oracle import cpu_ref
 pytestmark = pytest.mark.gpu
 
 FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "akg_amd", "fixtures")
-SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
+STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all")
+ALL_SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
+SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS)]
+STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS)]
 FULL = ["c1_ew_tanh_add_mul_f32_1024x4096.info", "c2_softmax_f16_8192x4096.info",
         "c3_layernorm_residual_bf16_16384x4096.info", "c4_quant_int8_residual_bf16_32768x8192.info"]
 
@@ -62,6 +65,46 @@ def test_small_fixture_matches_oracle(name):
     check_fixture(name, seed=harness.BASE_SEED + 100, openmp=False)
 
 
+def check_stream_reduction(path, seed, repeats=1, family="stream_reduce"):
+    """Streaming reductions (direction Y / ALL, long rows) combine partial results of many workgroups, so float sums
+    are reassociated. Outputs that do not come from a float sum (max / min, the unreduced outputs, 16-bit results)
+    are held to the usual bars against the serial oracle; float32 sums are held to rtol 1e-5 against the float64
+    evaluation of the same description, and the serial float32 oracle is shown for scale. The kernel is launched
+    `repeats` times on the same handle: every launch must leave the workspace ready for the next."""
+    from oracle import np_ref
+    print("case %s seed %d" % (os.path.basename(path), seed), flush=True)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    assert family is None or kernel.family == family
+    inputs = harness.make_inputs(desc, seed=seed)
+    serial = cpu_ref.CpuKernel(path)(inputs)
+    wide_inputs = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+    exact = np_ref.evaluate(harness.widen_to_float64(desc), wide_inputs)
+    in_numel = max(int(np.prod(e[0].get("shape", [1]))) for e in desc["input_desc"])
+    has_sum = any(o["name"] in ("ReduceSum", "ReducePrd") for o in desc["op_desc"])
+    for rep in range(repeats):
+        got = run_on_gpu(kernel, inputs)
+        for d, g, e, x in zip(kernel.outputs, got, serial, exact):
+            terms = max(1, in_numel // max(1, g.size))
+            if d.dtype == "float32" and has_sum and g.size < in_numel:
+                ok, msg = harness.compare_reassociated(g, x, d.dtype, terms)
+                gap = float(np.max(np.abs(np.asarray(e, dtype=np.float64) - np.asarray(x).reshape(e.shape))))
+                msg += " (serial float32 oracle is %.3g away from float64)" % gap
+            else:
+                ok, msg = harness.compare(g, e, d.dtype)
+            print("  launch %d %s %s: %s" % (rep, d.name, d.dtype, msg), flush=True)
+            assert ok, "%s output %s: %s" % (os.path.basename(path), d.name, msg)
+
+
+@pytest.mark.parametrize("name", STREAM)
+def test_streaming_reduction_matches_oracle(name):
+    check_stream_reduction(os.path.join(FIXTURES, name), seed=harness.BASE_SEED + 400, repeats=3)
+
+
+def test_full_size_bias_gradient_column_sums():
+    check_stream_reduction(os.path.join(FIXTURES, "n1_biasgrad_bf16_16384x4096.info"), seed=harness.BASE_SEED + 11)
+
+
 @pytest.mark.parametrize("name", FULL)
 def test_full_size_config_matches_oracle(name):
     # full BASELINE sizes; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)
@@ -70,7 +113,16 @@ def test_full_size_config_matches_oracle(name):
 
 REF_INFO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_info")
 REF_STATIC = sorted(f for f in os.listdir(REF_INFO)
-                    if f.endswith(".info") and ".dynamic." not in f and "13305325157517622155" not in f)
+                    if f.endswith(".info") and ".dynamic." not in f and "ReduceSum_split" not in f)
+REF_STREAM = sorted(f for f in os.listdir(REF_INFO) if f.endswith(".info") and "ReduceSum_split" in f)
+
+
+@pytest.mark.parametrize("name", REF_STREAM)
+def test_reference_repository_all_reduce_descriptions(name):
+    """Fused_Mul_ReduceSum_split_*: the reference's own all-reduce system-test descriptions ([768,512] -> [1] and
+    [3072] -> [1]), unchanged."""
+    check_stream_reduction(os.path.join(REF_INFO, name), seed=harness.BASE_SEED + 200, repeats=2, family=None)
+
 
 
 @pytest.mark.parametrize("name", REF_STATIC)

@@ -141,11 +141,13 @@ def test_error_conventions():
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(_desc(lambda d: d["op_desc"][0]["input_desc"][0][0].update(tensor_name="nowhere")), out_dir=None)
     assert e.value.code == -3 and "nowhere" in str(e.value)
-    # reduce over a non-innermost axis: valid description, no kernel family yet
-    path = os.path.join(REF_INFO, "Fused_Mul_ReduceSum_split_13305325157517622155.info")
+    # softmax along the outer axis: valid description, but the column kernel would need a second pass over the data
+    b = op_desc.DescBuilder("Fused_ReduceMax_Sub_axis0")
+    x = b.input([64, 128], "float32")
+    text = b.dumps([b.sub(x, b.reduce("ReduceMax", x, [0], True))])
     with pytest.raises(driver.AkgHipError) as e:
-        driver.HipKernel.from_file(path, out_dir=None)
-    assert e.value.code == -4
+        driver.HipKernel(text, out_dir=None)
+    assert e.value.code == -4 and "second pass" in str(e.value)
     # path with '..' is refused (checkAndReadJson)
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel.from_file(os.path.join(FIXTURES, "..", "fixtures", "small_softmax_f32_5x77.info"), out_dir=None)
@@ -202,6 +204,31 @@ def test_fusion_class_and_family_per_configuration():
         assert [t.is_output for t in k.tensors] == sorted(t.is_output for t in k.tensors)   # inputs first
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192.info"))
     assert k.algorithmic_ops == 2 * 4096 * 8192 * 8192
+
+
+def test_streaming_reduction_family_and_schedule():
+    """Reduce direction Y / ALL and over-long rows go to the streaming family; its workspace holds one arrival
+    counter per output group plus SPLIT partials per reduction, and is absent when one workgroup owns a group."""
+    k = driver.HipKernel.from_file(os.path.join(REF_INFO, "Fused_Mul_ReduceSum_split_13305325157517622155.info"))
+    assert (k.operator_type, k.family) == ("Reduction", "stream_reduce")
+    assert "direction=X" in _meta_schedule(k) and k.workspace_bytes > 0 and k.grid[0] > 1
+    assert "akg_ws" in k.source and "last_workgroup" in k.source
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_reducey_sqsum_f32_1x5100x3072.info"))
+    assert k.family == "stream_reduce" and "direction=Y" in _meta_schedule(k)
+    assert "outer=1 reduced=5100 inner=3072" in _meta_schedule(k)
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_reducey_sqsum_f32_3x37x50.info"))
+    assert k.workspace_bytes == 0 and "akg_ws" not in k.source      # too little work to split
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n1_biasgrad_bf16_16384x4096.info"))
+    assert k.family == "stream_reduce" and k.algorithmic_bytes == 2 * 16384 * 4096 * 2 + 2 * 4096 * 4
+    assert len(k.outputs) == 2
+    # the same reduction along the innermost axis with rows that fit in registers stays in the row family
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f32_5x77.info"))
+    assert k.family == "row_reduce" and k.workspace_bytes == 0
+
+
+def _meta_schedule(kernel):
+    with open(os.path.join(driver.DEFAULT_META_DIR, kernel.kernel_name[:-len("_kernel")] + ".json"), encoding="utf-8") as f:
+        return json.load(f)["schedule"]
 
 
 def test_artifacts_have_the_reference_layout(tmp_path):
@@ -294,4 +321,8 @@ def test_cli_tool():
     assert r.returncode == 0 and "row_reduce" in r.stdout
     r = subprocess.run([tool, "emit", os.path.join(REF_INFO, "Fused_Mul_ReduceSum_split_13305325157517622155.info")],
                        capture_output=True, text=True)
-    assert r.returncode == 1 and "error -4" in r.stderr
+    assert r.returncode == 0 and "last_workgroup" in r.stdout
+    # a dynamic-shape description is an error with a non-zero exit, never a crash
+    r = subprocess.run([tool, "emit", os.path.join(
+        REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")], capture_output=True, text=True)
+    assert r.returncode == 1 and "error -3" in r.stderr
