@@ -29,6 +29,7 @@ LoweringOptions LoweringOptions::fromEnvironment() {
   o.threadsPerRow = readInt("AKG_HIP_TPR");
   o.chunks = readInt("AKG_HIP_CHUNKS");
   o.block = readInt("AKG_HIP_BLOCK");
+  o.split = readInt("AKG_HIP_SPLIT");
   o.gemmVariant = readInt("AKG_HIP_GEMM_VARIANT");
   if (const char *nt = std::getenv("AKG_HIP_NT")) o.nonTemporal = (nt[0] != '0') ? 1 : 0;
   return o;

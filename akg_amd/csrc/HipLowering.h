@@ -35,12 +35,13 @@ enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce };
 const char *kernelFamilyName(KernelFamily f);
 
 // Tuning knobs; 0 means "let the heuristic decide". They can be set through the environment
-// (AKG_HIP_VEC, AKG_HIP_TPR, AKG_HIP_CHUNKS, AKG_HIP_BLOCK) for sweeps.
+// (AKG_HIP_VEC, AKG_HIP_TPR, AKG_HIP_CHUNKS, AKG_HIP_BLOCK, AKG_HIP_SPLIT) for sweeps.
 struct LoweringOptions {
   int vec = 0;          // elements per chunk
   int threadsPerRow = 0;
   int chunks = 0;       // chunks per thread
   int block = 0;        // threads per workgroup
+  int split = 0;        // streaming reductions: workgroups sharing one group of outputs (AKG_HIP_SPLIT)
   int gemmVariant = 0;  // GEMM tile configuration selector
   int nonTemporal = 1;  // stream once-touched tensors with non-temporal accesses (AKG_HIP_NT=0 turns it off)
   static LoweringOptions fromEnvironment();

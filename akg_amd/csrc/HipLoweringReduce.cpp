@@ -77,7 +77,7 @@ class StreamReduceEmitter {
   }
 
  private:
-  static constexpr int kBlock = 256;
+  int kBlock = 256;  // threads per workgroup (power of two, 64..1024)
 
   const OpGraph &g_;
   LoweringOptions opt_;
@@ -91,7 +91,7 @@ class StreamReduceEmitter {
   std::vector<Phase> phase_;  // per tensor
   std::vector<const OpNode *> reduces_;
 
-  int vec_ = 1, lanes_ = 64, split_ = 1;
+  int vec_ = 1, lanes_ = 64, split_ = 1, unroll_ = 4;
   int64_t strips_ = 1, rps_ = 1, grid_ = 1, groups_ = 1;
   uint64_t workspaceBytes_ = 0;
   std::vector<uint64_t> partialOffset_;  // per reduction, bytes from the workspace base
@@ -249,9 +249,17 @@ class StreamReduceEmitter {
 
   // ------------------------------------------------------------------ schedule
   void pickSchedule() {
-    size_t widest = 1;
-    for (int id : g_.inputs) widest = std::max(widest, dtypeSize(g_.tensor(id).dtype));
-    for (int id : g_.outputs) widest = std::max(widest, dtypeSize(g_.tensor(id).dtype));
+    // 16-byte accesses of the widest tensor that is streamed (as large as the iteration space); the reduced outputs
+    // and broadcast operands are small and do not set the chunk width
+    size_t widest = 0, widestAny = 1;
+    auto consider = [&](int id) {
+      const TensorValue &t = g_.tensor(id);
+      widestAny = std::max(widestAny, dtypeSize(t.dtype));
+      if (t.numel() == O_ * R_ * I_) widest = std::max(widest, dtypeSize(t.dtype));
+    };
+    for (int id : g_.inputs) consider(id);
+    for (int id : g_.outputs) consider(id);
+    if (widest == 0) widest = widestAny;
     int v = opt_.vec > 0 ? opt_.vec : static_cast<int>(16 / widest);
     v = std::max(1, std::min(v, 16));
     if ((v & (v - 1)) != 0) v = 1;
@@ -260,15 +268,31 @@ class StreamReduceEmitter {
     const int64_t fastExtent = space_[static_cast<size_t>(fastDim)];
     while (v > 1 && (fastExtent % v) != 0) v >>= 1;
     vec_ = v;
-    const int64_t targetGroups = 2048;  // about 8 workgroups per CU
+    // Measured on MI355X (256 CUs) with 256 MiB .. 640 MiB inputs: column reductions stream best with 3 workgroups
+    // per CU and two 16-byte loads in flight per thread (75 % of the 8 TB/s peak for two bf16 operands, 89 % for one
+    // float32 operand; 8 workgroups per CU: 55 %); contiguous reductions with 1 workgroup per CU and eight loads
+    // in flight per thread (85 %). More workgroups mean more partials and more end-of-workgroup hand-shakes.
+    int streamedInputs = 0;
+    for (size_t i : inputsUsedIn(Phase::Pre)) {
+      if (g_.tensor(g_.inputs[i]).numel() == O_ * R_ * I_) ++streamedInputs;
+    }
+    streamedInputs = std::max(1, streamedInputs);
+    const int64_t targetGroups = dirY_ ? 768 : 256;
+    unroll_ = opt_.chunks > 0 ? std::min(opt_.chunks, 16) : std::max(1, (dirY_ ? 2 : 8) / streamedInputs);
+    if (opt_.block >= 64 && opt_.block <= 1024 && (opt_.block & (opt_.block - 1)) == 0) kBlock = opt_.block;
     if (dirY_) {
-      lanes_ = std::min<int64_t>(64, pow2AtLeastL(ceilDivL(I_, vec_)));
+      // A workgroup is TR thread-rows of LANES lanes; a lane owns V adjacent columns. Narrow strips (16 lanes = one
+      // 256-byte run per row) give many groups, so few workgroups share a group and the partials stay small.
+      int lanes = opt_.threadsPerRow > 0 ? opt_.threadsPerRow : 16;
+      lanes = std::max(1, std::min(lanes, 64));
+      if ((lanes & (lanes - 1)) != 0) lanes = 16;
+      lanes_ = static_cast<int>(std::min<int64_t>(lanes, pow2AtLeastL(ceilDivL(I_, vec_))));
       const int tr = kBlock / lanes_;
       strips_ = ceilDivL(I_, static_cast<int64_t>(lanes_) * vec_);
       groups_ = O_ * strips_;
-      int64_t split = ceilDivL(targetGroups, groups_);
+      int64_t split = opt_.split > 0 ? opt_.split : ceilDivL(targetGroups, groups_);
       const int64_t maxSplit = std::max<int64_t>(1, R_ / (static_cast<int64_t>(tr) * 4));
-      split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), 256));
+      split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), 1024));
       rps_ = ceilDivL(R_, split);
       split_ = static_cast<int>(ceilDivL(R_, rps_));
     } else {
@@ -276,7 +300,7 @@ class StreamReduceEmitter {
       strips_ = 1;
       groups_ = O_;
       const int64_t chunk = static_cast<int64_t>(kBlock) * vec_;
-      int64_t split = ceilDivL(targetGroups, groups_);
+      int64_t split = opt_.split > 0 ? opt_.split : ceilDivL(targetGroups, groups_);
       const int64_t maxSplit = std::max<int64_t>(1, R_ / (chunk * 2));
       split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), kBlock));
       rps_ = ceilDivL(ceilDivL(R_, split), chunk) * chunk;
@@ -297,6 +321,7 @@ class StreamReduceEmitter {
         off = align(off + static_cast<uint64_t>(groups_) * split_ * width * ctSize);
       }
       workspaceBytes_ = off;
+      if (workspaceBytes_ >= (1ULL << 31)) throw LoweringError("workspace of the streaming reduction exceeds 2 GiB");
     }
   }
 
@@ -501,8 +526,16 @@ class StreamReduceEmitter {
     line("  (void)O; (void)I; (void)STRIPS;");
     line("  const int tid = static_cast<int>(threadIdx.x);");
     line("  const long akg_wg = static_cast<long>(blockIdx.x);");
-    line("  const long akg_s = akg_wg % SPLIT;");
-    line("  const long akg_group = akg_wg / SPLIT;");
+    if (dirY_ && opt_.gemmVariant != 1) {
+      // neighbouring workgroups take neighbouring column strips of the same rows: what is in flight at any time
+      // covers whole rows of the tensor rather than 256-byte pieces 8 KiB apart
+      src_ << "  constexpr long GROUPS = " << groups_ << "L;\n";
+      line("  const long akg_group = akg_wg % GROUPS;");
+      line("  const long akg_s = akg_wg / GROUPS;");
+    } else {
+      line("  const long akg_s = akg_wg % SPLIT;");
+      line("  const long akg_group = akg_wg / SPLIT;");
+    }
     line("  const long r_begin = akg_s * RPS;");
     line("  const long r_end = (r_begin + RPS < R) ? (r_begin + RPS) : R;");
     if (dirY_) {
@@ -534,7 +567,7 @@ class StreamReduceEmitter {
       }
     }
     // ---- streaming loop
-    line("#pragma unroll 2");
+    line("#pragma unroll " + std::to_string(unroll_));
     if (dirY_) {
       line("  for (long r = r_begin + tr; r < r_end; r += TR) {");
     } else {
@@ -611,28 +644,31 @@ class StreamReduceEmitter {
     emitRowCombineY("akg_lds");
     if (split_ > 1) {
       line("  // ---- partials of this workgroup -> workspace; the last workgroup of the group to arrive finishes the job");
-      line("  unsigned char *akg_wsb = reinterpret_cast<unsigned char *>(akg_ws);");
+      src_ << "  const akg::Buffer b_ws = akg::make_buffer(akg_ws, " << workspaceBytes_ << "L);\n";
       for (size_t k = 0; k < reduces_.size(); ++k) {
-        const std::string ct = computeTypeName(g_.tensor(reduces_[k]->outputs[0]).dtype);
-        src_ << "  " << ct << " *part" << k << " = reinterpret_cast<" << ct << " *>(akg_wsb + " << partialOffset_[k]
-             << "UL) + akg_group * (static_cast<long>(SPLIT) * LANES * V) + li * V;\n";
-        line("  if (tr == 0) {");
-        line("#pragma unroll");
-        src_ << "    for (int e = 0; e < V; ++e) akg::ws_store(part" << k << " + akg_s * (LANES * V) + e, acc" << k
-             << "[e]);\n";
-        line("  }");
+        const DType od = g_.tensor(reduces_[k]->outputs[0]).dtype;
+        const uint64_t ctSize = std::max<size_t>(4, dtypeSize(od));
+        // byte offset of partial slot 0 of this lane; slot p is p * LANES * V elements further
+        src_ << "  const unsigned part" << k << " = " << partialOffset_[k] << "u + static_cast<unsigned>((akg_group * "
+             << "(static_cast<long>(SPLIT) * LANES * V) + li * V) * " << ctSize << "L);\n";
+        src_ << "  if (tr == 0) akg::ws_store_chunk<V>(b_ws, part" << k << " + static_cast<unsigned>(akg_s) * (LANES * V * "
+             << ctSize << "u), acc" << k << ");\n";
       }
       line("  __shared__ unsigned akg_flag;");
       line("  if (!akg::last_workgroup(akg_ws, akg_group, SPLIT, tid, &akg_flag)) return;");
       for (size_t k = 0; k < reduces_.size(); ++k) {
         const OpNode &op = *reduces_[k];
         const DType od = g_.tensor(op.outputs[0]).dtype;
+        const uint64_t ctSize = std::max<size_t>(4, dtypeSize(od));
         const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
         line("#pragma unroll");
         src_ << "  for (int e = 0; e < V; ++e) acc" << k << "[e] = " << spec.init << ";\n";
-        line("  for (long p = tr; p < SPLIT; p += TR) {");
-        std::string step = spec.combiner + "::apply(acc" + std::to_string(k) + "[e], akg::ws_load(part" +
-                           std::to_string(k) + " + p * (LANES * V) + e))";
+        line("#pragma unroll 4");
+        line("  for (int p = tr; p < SPLIT; p += TR) {");
+        src_ << "    " << computeTypeName(od) << " pv[V];\n";
+        src_ << "    akg::ws_load_chunk<V>(b_ws, part" << k << " + static_cast<unsigned>(p) * (LANES * V * " << ctSize
+             << "u), pv);\n";
+        std::string step = spec.combiner + "::apply(acc" + std::to_string(k) + "[e], pv[e])";
         if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
         line("#pragma unroll");
         src_ << "    for (int e = 0; e < V; ++e) acc" << k << "[e] = " << step << ";\n";

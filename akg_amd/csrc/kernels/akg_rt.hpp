@@ -691,11 +691,17 @@ AKG_DEV T group_reduce(T v, T *scratch, int tid) {
 // Workspace protocol of the streaming reductions. Several workgroups share one group of outputs; each leaves
 // its partial result in device memory and counts its arrival; the workgroup that arrives last reads all the
 // partials back (in slot order, so the result does not depend on the arrival order) and finishes the job.
-// The eight XCDs have private L2 caches: partials are written and read with device-scope accesses, and the
-// arrival counter is an acquire/release device-scope atomic, so the last workgroup sees every partial
-// whichever XCD produced it. The last workgroup puts the counter back to zero: the workspace is zero-filled
-// once when it is allocated and every launch leaves it as it found it.
+//
+// The eight XCDs have private L2 caches. A device-scope release fence per workgroup would write back and an
+// acquire fence would invalidate a whole L2 each time (measured: about 1 us per workgroup, serialised per XCD),
+// so the protocol uses no fence. Partials are written and read with device-scope (sc1) accesses, which go
+// through the L2 to memory and back; a thread waits for its own stores to be acknowledged (vmcnt 0) before the
+// workgroup barrier, and one thread then counts the arrival with a device-scope atomic. The last workgroup puts
+// the counter back to zero: the workspace is zero-filled once when it is allocated and every launch leaves it
+// as it found it.
 // ---------------------------------------------------------------------------------------------------------
+constexpr int kAuxDeviceScope = 16;  // sc1
+
 template <typename T>
 AKG_DEV void ws_store(T *p, T v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -705,20 +711,44 @@ AKG_DEV T ws_load(const T *p) {
   return __hip_atomic_load(const_cast<T *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// V adjacent partials of one lane at byte offset `off` of the workspace (aligned to min(16, V * sizeof(T))).
+template <int V, typename T>
+AKG_DEV void ws_store_chunk(Buffer ws, u32 off, const T (&v)[V]) {
+  constexpr int kBytes = static_cast<int>(sizeof(T)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef BufferIo<kPiece, kAuxDeviceScope> Io;
+  typename Io::type raw[kPieces];
+  __builtin_memcpy(raw, v, kBytes);
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) Io::store(raw[k], ws, off + k * kPiece);
+}
+template <int V, typename T>
+AKG_DEV void ws_load_chunk(Buffer ws, u32 off, T (&v)[V]) {
+  constexpr int kBytes = static_cast<int>(sizeof(T)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef BufferIo<kPiece, kAuxDeviceScope> Io;
+  typename Io::type raw[kPieces];
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) raw[k] = Io::load(ws, off + k * kPiece);
+  __builtin_memcpy(v, raw, kBytes);
+}
+
 // True in every thread of exactly one workgroup out of the `split` that share counter `group`: the last to arrive.
-// Must be reached by all threads of the workgroup, after their ws_store calls.
+// Must be reached by all threads of the workgroup, after their ws_store / ws_store_chunk calls.
 AKG_DEV bool last_workgroup(unsigned *counters, long group, int split, int tid, unsigned *flag) {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partials have reached memory
   __syncthreads();
   if (tid == 0) {
-    const unsigned prev = __hip_atomic_fetch_add(counters + group, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    const unsigned prev = __hip_atomic_fetch_add(counters + group, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const bool last = prev == static_cast<unsigned>(split - 1);
     if (last) __hip_atomic_store(counters + group, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     *flag = last ? 1u : 0u;
   }
   __syncthreads();
   const bool last = *flag != 0u;
-  if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  asm volatile("" ::: "memory");  // no access to the partials may be moved above the arrival count
   return last;
 }
 
