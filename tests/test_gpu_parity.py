@@ -141,6 +141,37 @@ def test_reference_repository_descriptions_match_oracle(name):
         assert ok, "%s output %s: %s" % (name, d.name, msg)
 
 
+def test_float32_tanh_accuracy_over_the_whole_range():
+    """The float32 tanh of the device op library is an own implementation (series below 0.25, hardware exp2 and
+    reciprocal above): its error against the float64 value is measured on 8M arguments, dense around the branch
+    point and log-spaced over every magnitude, and must stay an order of magnitude inside the 1e-5 bar."""
+    from akg_amd import op_desc
+    rows, cols = 2048, 4096
+    b = op_desc.DescBuilder("Fused_Tanh_accuracy_f32_%dx%d" % (rows, cols))
+    x = b.input([rows, cols], "float32")
+    kernel = driver.HipKernel(b.dumps([b.unary("Tanh", x)]))
+    rng = np.random.default_rng(harness.BASE_SEED + 500)
+    n = rows * cols
+    mag = np.concatenate([
+        np.exp(rng.uniform(np.log(1e-30), np.log(100.0), n // 2)),      # every magnitude
+        rng.uniform(0.0, 12.0, n // 4),                                  # where tanh bends and saturates
+        rng.uniform(0.2, 0.3, n // 4 - 16),                              # around the branch point
+        [0.0, 0.25, np.nextafter(np.float32(0.25), np.float32(0)), 1e-45, 1e-38, 44.0, 45.0, 88.0, 1e30, np.inf,
+         np.nan, 9.0, 9.5, 10.0, 0.5, 1.0]]).astype(np.float32)
+    sign = np.where(rng.random(n) < 0.5, -1.0, 1.0).astype(np.float32)
+    xs = (mag * sign).reshape(rows, cols)
+    got = run_on_gpu(kernel, [xs])[0].astype(np.float64)
+    ref = np.tanh(xs.astype(np.float64))
+    finite = np.isfinite(ref) & (ref != 0)
+    rel = np.abs(got[finite] - ref[finite]) / np.abs(ref[finite])
+    print("  tanh float32: max relative error %.3g over %d arguments" % (rel.max(), rel.size), flush=True)
+    assert rel.max() < 2e-6
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    zero = xs == 0
+    assert np.all(got[zero] == 0) and np.array_equal(np.signbit(got[zero]), np.signbit(xs[zero]))
+    assert np.all(np.abs(got[np.isfinite(got)]) <= 1.0)
+
+
 def test_run_host_reference_style_call_and_driver():
     """Host pointers in, outputs overwritten in place (the reference shim's calling convention), through HipDriver."""
     path = os.path.join(FIXTURES, "small_layernorm_residual_bf16_19x520.info")
