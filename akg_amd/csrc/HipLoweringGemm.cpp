@@ -1,11 +1,16 @@
 /**
- * Lowering of the Matmul fusion class: one int8 MatMul followed by an elementwise epilogue over [M,N].
+ * Lowering of the Matmul fusion class: one MatMul (int8 x int8 -> int32, or bfloat16 / float16 operands with a
+ * float32 accumulator) followed by an elementwise epilogue over [M,N].
  *
  * The reference lowers MatMul to linalg.matmul and then through the same generic loop mapping as everything else
  * (akg-mlir/lib/Conversion/MindSporeToLinalg/MindSporeToLinalg.cpp:1453-1546; no tensor-core path is wired into
- * its GPU pipeline). Here the contraction runs on the MFMA units (kernels/akg_gemm_i8.hpp) and the ops that follow
- * it in the description are emitted as an epilogue functor applied to the int32 accumulators in registers, so the
+ * its GPU pipeline). Here the contraction runs on the MFMA units (kernels/akg_gemm_mfma.hpp) and the ops that follow
+ * it in the description are emitted as an epilogue functor applied to the accumulators in registers, so the
  * [M,N] int32 / float32 intermediates never exist in memory.
+ *
+ * Float MatMul: the reference accumulates in the MatMul's declared result type, element by element in k order
+ * (zero-filled accumulator of the output type, MindSporeToLinalg.cpp:1520-1540). The MFMA accumulates in float32
+ * whatever the declared type; a float16 / bfloat16 result is rounded once, after the whole sum.
  *
  * Epilogue operands are classified by how they vary over the output tile:
  *   Full   [M,N]      4-element chunk per (row, 4 columns), loaded / computed per output chunk
@@ -50,7 +55,8 @@ class GemmEmitter {
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
     note << "gemm_epilogue M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
-         << " tile=256x256x" << stepK() << " mfma=i32_32x32x32_i8 waves=" << wavesM() << "x2 grid=" << k.grid[0];
+         << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
+         << k.grid[0];
     k.scheduleNote = note.str();
     return k;
   }
@@ -67,10 +73,20 @@ class GemmEmitter {
   std::vector<bool> relaxed_;
   std::ostringstream members_, prepare_, apply_;
 
+  DType elem_ = DType::I8;  // operand element type: I8, BF16 or F16
+  int elemBytes() const { return elem_ == DType::I8 ? 1 : 2; }
+  const char *mmaTraits() const {
+    return elem_ == DType::I8 ? "akg::MmaI8" : (elem_ == DType::BF16 ? "akg::MmaBF16" : "akg::MmaF16");
+  }
+  const char *mfmaName() const {
+    return elem_ == DType::I8 ? "i32_32x32x32_i8" : (elem_ == DType::BF16 ? "f32_32x32x16_bf16" : "f32_32x32x16_f16");
+  }
+  const char *accType() const { return elem_ == DType::I8 ? "int" : "float"; }
+  // The tuning variants exist for the 8-bit kernel only; 16-bit operands always use 4 x 2 wavefronts and 128-byte steps.
   // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_GEMM_VARIANT=1.
-  int wavesM() const { return (opt_.gemmVariant & 1) ? 2 : 4; }
-  // K extent of one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
-  int stepK() const { return (opt_.gemmVariant & 2) ? 64 : 128; }
+  int wavesM() const { return (elem_ == DType::I8 && (opt_.gemmVariant & 1)) ? 2 : 4; }
+  // Bytes of K in one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
+  int stepK() const { return (elem_ == DType::I8 && (opt_.gemmVariant & 2)) ? 64 : 128; }
   bool splitDuty() const { return (opt_.gemmVariant & 4) != 0 && wavesM() == 4; }
 
   void analyse() {
@@ -97,8 +113,14 @@ class GemmEmitter {
     if (a.inputIndex < 0 || b.inputIndex < 0) {
       throw LoweringError("MatMul operands must be kernel inputs (prologue fusion is not supported yet)");
     }
-    if (a.dtype != DType::I8 || b.dtype != DType::I8 || c.dtype != DType::I32) {
-      throw LoweringError("MatMul: only int8 x int8 -> int32 has an MFMA kernel yet");
+    if (a.dtype == DType::I8 && b.dtype == DType::I8 && c.dtype == DType::I32) {
+      elem_ = DType::I8;
+    } else if ((a.dtype == DType::BF16 || a.dtype == DType::F16) && b.dtype == a.dtype &&
+               (c.dtype == DType::F32 || c.dtype == a.dtype)) {
+      elem_ = a.dtype;
+    } else {
+      throw LoweringError("MatMul: MFMA kernels exist for int8 x int8 -> int32 and for bfloat16 / float16 operands "
+                          "with a float32 or same-type result");
     }
     if (a.shape.size() != 2 || b.shape.size() != 2 || c.shape.size() != 2) {
       throw LoweringError("MatMul: only rank-2 operands are supported");
@@ -108,7 +130,7 @@ class GemmEmitter {
     n_ = transB_ ? b.shape[0] : b.shape[1];
     const int64_t kb = transB_ ? b.shape[1] : b.shape[0];
     if (kb != k_ || c.shape[0] != m_ || c.shape[1] != n_) throw LoweringError("MatMul: inconsistent shapes");
-    if (k_ % 16 != 0) throw LoweringError("MatMul: K must be a multiple of 16");
+    if ((k_ * elemBytes()) % 16 != 0) throw LoweringError("MatMul: a row of K must be a multiple of 16 bytes");
     if (n_ % 4 != 0) throw LoweringError("MatMul: N must be a multiple of 4");
     for (const OpNode &op : g_.ops) {
       if (op.kind == OpKind::MatMul) continue;
@@ -153,6 +175,13 @@ class GemmEmitter {
     acc.defined = true;
     acc.rank = EpiRank::Full;
     acc.ident = "acc";
+    const DType accDt = g_.tensor(accId_).dtype;
+    if (accDt == DType::F16 || accDt == DType::BF16) {
+      // a 16-bit MatMul result: the float32 sum is rounded to the declared type once
+      acc.ident = "accr";
+      apply_ << "    float accr[4];\n#pragma unroll\n    for (int e = 0; e < 4; ++e) accr[e] = " << dtypeTag(accDt)
+             << "::rnd(acc[e]);\n";
+    }
 
     // constants
     for (size_t t = 0; t < g_.tensors.size(); ++t) {
@@ -269,10 +298,10 @@ class GemmEmitter {
     const std::string kname = g_.name + "_kernel";
     src_ << "// Generated by the akg HIP lowering for gfx950. Op description: " << g_.name << "\n";
     src_ << "// family: gemm_epilogue, fusion class: " << operatorTemplateName(g_.operatorTemplate) << "\n";
-    src_ << "#include \"akg_rt.hpp\"\n#include \"akg_gemm_i8.hpp\"\n\n";
+    src_ << "#include \"akg_rt.hpp\"\n#include \"akg_gemm_mfma.hpp\"\n\n";
     src_ << "namespace {\nstruct Epilogue {\n" << members_.str();
     src_ << "  AKG_DEV void prepare(long col) {\n    (void)col;\n" << prepare_.str() << "  }\n";
-    src_ << "  AKG_DEV void apply(const int (&acc)[4], long row, long col) {\n" << apply_.str() << "  }\n";
+    src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[4], long row, long col) {\n" << apply_.str() << "  }\n";
     src_ << "};\n}  // namespace\n\n";
     src_ << "extern \"C\" __global__ __launch_bounds__(" << wavesM() * 128 << ") void " << kname << "(";
     size_t argc = 0;
@@ -289,7 +318,7 @@ class GemmEmitter {
       src_ << "  epi.in" << i << " = in" << i << ";\n";
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
-    src_ << "  akg::gemm_i8_256x256<" << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
+    src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
          << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
   }
 };

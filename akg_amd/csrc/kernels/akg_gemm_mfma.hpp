@@ -1,11 +1,15 @@
 /**
- * int8 x int8 -> int32 GEMM tile kernel for gfx950 (CDNA4) with a caller-supplied epilogue applied to the
- * int32 accumulators while they are still in registers (dequantise / bias / activation / cast fusions).
+ * MFMA GEMM tile kernel for gfx950 (CDNA4) with a caller-supplied epilogue applied to the accumulators while they
+ * are still in registers (dequantise / bias / activation / cast fusions). The element type is a template
+ * parameter (`Mma`): int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), bfloat16 or float16 -> float32
+ * (v_mfma_f32_32x32x16_bf16 / _f16). Both instruction shapes consume 32 BYTES of K per row and MFMA (a lane holds 16
+ * consecutive bytes), so the kernel is written in bytes along K and the LDS layout, the fragment reads and the A
+ * staging are the same for every element type; only the in-register transpose of a row-major B differs.
  *
  * Shape of the computation (all sizes are compile-time constants of the emitted kernel):
- *   C[M,N] = A[M,K] * B[K,N]            A row-major int8, B row-major int8 ([N,K] when TRANSB)
- *   workgroup = 256 threads = 4 wavefronts (2 x 2), workgroup tile 256 x 256, K step 64
- *   wavefront tile 128 x 128 = 4 x 4 MFMA tiles of v_mfma_i32_32x32x32_i8 (16 accumulator registers each)
+ *   C[M,N] = A[M,K] * B[K,N]            A row-major, B row-major ([N,K] when TRANSB)
+ *   workgroup tile 256 x 256, K step 128 bytes (64 optional), 4 x 2 wavefronts (2 x 2 optional)
+ *   wavefront tile 64 x 128 (128 x 128) = 2 x 4 (4 x 4) MFMA tiles of 32 x 32 (16 accumulator registers each)
  *
  * Data movement:
  *   global -> registers -> LDS, double buffered in LDS (one barrier per K step); the global loads of step
@@ -30,6 +34,34 @@ namespace akg {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// Element-type traits of the contraction: bytes per element, accumulator type, and the MFMA on one 16-byte
+// fragment per operand (32 x 32 outputs, 32 bytes of K).
+struct MmaI8 {
+  static constexpr int kElemBytes = 1;
+  typedef int acc_t;
+  typedef v16i acc_v;
+  static AKG_DEV acc_v mma(v4i a, v4i b, acc_v c) { return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0); }
+};
+struct MmaBF16 {
+  static constexpr int kElemBytes = 2;
+  typedef float acc_t;
+  typedef v16f acc_v;
+  typedef __bf16 frag __attribute__((ext_vector_type(8)));
+  static AKG_DEV acc_v mma(v4i a, v4i b, acc_v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(frag, a), __builtin_bit_cast(frag, b), c, 0, 0, 0);
+  }
+};
+struct MmaF16 {
+  static constexpr int kElemBytes = 2;
+  typedef float acc_t;
+  typedef v16f acc_v;
+  typedef _Float16 frag __attribute__((ext_vector_type(8)));
+  static AKG_DEV acc_v mma(v4i a, v4i b, acc_v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(frag, a), __builtin_bit_cast(frag, b), c, 0, 0, 0);
+  }
+};
 
 #ifdef AKG_GEMM_STRICT_ORDER
 #define AKG_GEMM_PIN __builtin_amdgcn_sched_barrier(0)
@@ -59,20 +91,22 @@ AKG_DEV void transpose4x4_bytes(const u32 (&r)[4], u32 (&t)[4]) {
   t[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
 }
 
-// Number of workgroups to launch for an M x N problem (multiple of the XCD count).
-constexpr long gemm_i8_grid(long m, long n) {
-  const long tiles = ((m + kGemmBM - 1) / kGemmBM) * ((n + kGemmBN - 1) / kGemmBN);
-  return ((tiles + kGemmXcds - 1) / kGemmXcds) * kGemmXcds;
-}
+// 2 x 16-bit pairs: out word = (lo or hi half of x, same half of y).
+AKG_DEV u32 pack_lo16(u32 x, u32 y) { return __builtin_amdgcn_perm(y, x, 0x05040100u); }
+AKG_DEV u32 pack_hi16(u32 x, u32 y) { return __builtin_amdgcn_perm(y, x, 0x07060302u); }
 
 // WAVES_M x 2 wavefronts per workgroup: 2 x 2 (one wavefront per SIMD, 128 x 128 per wavefront, 256 accumulator
 // registers) or 4 x 2 (two wavefronts per SIMD, 64 x 128 per wavefront, 128 accumulator registers: the second
 // wavefront's MFMAs cover the first one's loads, transposes and barriers).
-// BK = K extent of one step: 64 or 128. With 128 every row of A contributes one full 128-byte cache line per step
+// BK = BYTES of K in one step: 64 or 128. With 128 every row of A contributes one full 128-byte cache line per step
 // (with 64 each line is fetched from L2 twice), there are half as many barriers, and LDS holds 2 x 72 KiB.
-template <long M, long N, long K, bool TRANSB, int WAVES_M, int BK, bool SPLIT, typename Epilogue>
-AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B, Epilogue &epi) {
-  static_assert(K % 16 == 0, "K must be a multiple of 16");
+// KE is the K extent in elements; everything below counts K in bytes (K = KE * element size).
+template <typename Mma, long M, long N, long KE, bool TRANSB, int WAVES_M, int BK, bool SPLIT, typename Epilogue>
+AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi) {
+  constexpr int EB = Mma::kElemBytes;
+  constexpr long K = KE * EB;    // bytes of K per row of A (and per column of B)
+  constexpr long NB = N * EB;    // bytes per k-row of a row-major B
+  static_assert(K % 16 == 0, "K must be a multiple of 16 bytes");
   static_assert(TRANSB || (N % 4 == 0), "N must be a multiple of 4");
   static_assert(WAVES_M == 2 || WAVES_M == 4, "2 x 2 or 4 x 2 wavefronts");
   static_assert(BK == 64 || BK == 128, "K step of 64 or 128");
@@ -88,7 +122,7 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
   constexpr int kChunksPerRow = BK / 16;              // 16-byte chunks per row of a K-contiguous operand tile
   constexpr int kRowChunks = 256 * kChunksPerRow / kStageThreads;  // 16-byte chunks per staging thread and operand
   constexpr int kRowStep = kStageThreads / kChunksPerRow;          // rows between two chunks of one thread
-  constexpr int kBlockRows = 4 * kRowChunks;          // k-rows of B per staging thread (8, 16 or 32), 4 columns each
+  constexpr int kBlockRows = 4 * kRowChunks / EB;     // k-rows of B per staging thread, 4 columns each (16 k-bytes per chunk)
   constexpr int kTM = kGemmBM / (32 * WAVES_M);       // MFMA row tiles per wavefront
   constexpr int kWaveRows = kGemmBM / WAVES_M;
   constexpr long kTilesM = (M + kGemmBM - 1) / kGemmBM;
@@ -121,7 +155,7 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
   const int wm = wave >> 1;
   const int wn = wave & 1;
 
-  v16i acc[kTM][4];
+  typename Mma::acc_v acc[kTM][4];
 #pragma unroll
   for (int i = 0; i < kTM; ++i) {
 #pragma unroll
@@ -153,12 +187,12 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
   // instructions and MFMAs compete for issue cycles). Out-of-range lanes read zero through the descriptor's size.
   static_assert(M * K < (1L << 31) && N * K < (1L << 31), "operand too large for 32-bit buffer offsets");
   const __amdgpu_buffer_rsrc_t aRsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<s8 *>(A), 0, static_cast<int>(M * K), 0x00020000);
+      const_cast<void *>(A), 0, static_cast<int>(M * K), 0x00020000);
   const __amdgpu_buffer_rsrc_t bRsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<s8 *>(B), 0, static_cast<int>(N * K), 0x00020000);
+      const_cast<void *>(B), 0, static_cast<int>(N * K), 0x00020000);
   const int aVoff = static_cast<int>((m0 + aRow) * K + aChunk * 16);
   const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
-                           : static_cast<int>((bKq * kBlockRows) * N + n0 + 4 * bN4);
+                           : static_cast<int>((bKq * kBlockRows) * NB + (n0 + 4 * bN4) * EB);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
   auto loadRows = [&](__amdgpu_buffer_rsrc_t rsrc, int voff, long rowBase, long rowLimit, long k0,
@@ -175,14 +209,22 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
     }
   };
   auto loadBlock = [&](long k0, v4i (&dst)[kRowChunks]) {
-    // kBlockRows k-rows x 4 columns of row-major B, one dword per k-row
+    // kBlockRows k-rows x 4 columns of row-major B: one dword (8-bit elements) or two (16-bit) per k-row.
+    // k0 is in bytes of K: the first k-row of the step is k0 / EB.
 #pragma unroll
     for (int i = 0; i < kBlockRows; ++i) {
-      u32 v = 0u;
-      if (kFull || (n0 + 4 * bN4 < N && k0 + bKq * kBlockRows + i < K)) {
-        v = __builtin_amdgcn_raw_buffer_load_b32(bRsrc, bVoff, static_cast<int>((k0 + i) * N), 0);
+      const bool ok = kFull || (n0 + 4 * bN4 < N && k0 / EB + bKq * kBlockRows + i < KE);
+      if constexpr (EB == 1) {
+        u32 v = 0u;
+        if (ok) v = __builtin_amdgcn_raw_buffer_load_b32(bRsrc, bVoff, static_cast<int>((k0 + i) * NB), 0);
+        dst[i >> 2][i & 3] = static_cast<int>(v);
+      } else {
+        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+        u32x2 v = {0u, 0u};
+        if (ok) v = __builtin_amdgcn_raw_buffer_load_b64(bRsrc, bVoff, static_cast<int>((k0 / EB + i) * NB), 0);
+        dst[i >> 1][(i & 1) * 2] = static_cast<int>(v[0]);
+        dst[i >> 1][(i & 1) * 2 + 1] = static_cast<int>(v[1]);
       }
-      dst[i >> 2][i & 3] = static_cast<int>(v);
     }
   };
   auto loadGlobal = [&](long step, Stage &st) {
@@ -219,7 +261,28 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
       *reinterpret_cast<v4i *>(lb + r * kPitch + aChunk * 16) = src[i];
     }
   };
-  auto storeBlockB = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
+  auto storeBlockB16 = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
+    // 16-bit elements: src[g] = k-rows 2g, 2g+1, each as (columns 0 1 | columns 2 3). A column's 8 consecutive k
+    // (16 bytes) are gathered two at a time with v_perm_b32.
+    static_assert(EB != 2 || kRowChunks == 4, "16-bit staging is written for 8 k-rows per thread");
+    if constexpr (EB == 2 && kRowChunks == 4) {
+      v4i w[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const u32 c01a = static_cast<u32>(src[g][0]), c23a = static_cast<u32>(src[g][1]);  // k-row 2g
+        const u32 c01b = static_cast<u32>(src[g][2]), c23b = static_cast<u32>(src[g][3]);  // k-row 2g + 1
+        w[0][g] = static_cast<int>(pack_lo16(c01a, c01b));
+        w[1][g] = static_cast<int>(pack_hi16(c01a, c01b));
+        w[2][g] = static_cast<int>(pack_lo16(c23a, c23b));
+        w[3][g] = static_cast<int>(pack_hi16(c23a, c23b));
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * 16) = w[j];
+      }
+    }
+  };
+  auto storeBlockB8 = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
     // src[g] = 4 k-rows x 4 columns; after the byte transpose t[g][j] = 4 consecutive k of column j
     u32 t[kRowChunks][4];
 #pragma unroll
@@ -247,6 +310,13 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
         w[3] = static_cast<int>(t[4 * h + 3][j]);
         *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * kBlockRows + h * 16) = w;
       }
+    }
+  };
+  auto storeBlockB = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
+    if constexpr (EB == 1) {
+      storeBlockB8(lb, src);
+    } else {
+      storeBlockB16(lb, src);
     }
   };
   auto storeLds = [&](int buf, const Stage &st) {
@@ -289,7 +359,7 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
     for (int i = 0; i < kTM; ++i) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+        acc[i][j] = Mma::mma(af[i], bf[j], acc[i][j]);
       }
     }
 #endif
@@ -360,7 +430,7 @@ AKG_DEV void gemm_i8_256x256(const s8 *__restrict__ A, const s8 *__restrict__ B,
       for (int v = 0; v < 16; ++v) {
         const long row = m0 + wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
         if (kFull || row < M) {
-          const int a4[4] = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+          const typename Mma::acc_t a4[4] = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
           epi.apply(a4, row, col4);
         }
       }

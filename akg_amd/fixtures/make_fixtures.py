@@ -45,6 +45,13 @@ FIXTURES = {
     "small_biasgrad_f32_100x37": lambda n: op_desc.bias_grad(100, 37, "float32", n),
     "small_sub_exp_reducesum_split_f32_4x96x160": lambda n: op_desc.sub_exp_reduce_y(4, 96, 160, "float32", n),
     "small_mean_absmax_all_f32_1000x1000": lambda n: op_desc.mean_absmax_all(1000, 1000, "float32", n),
+    # float MatMul + bias + activation on the bfloat16 / float16 MFMA path
+    "small_gemm_bf16_bias_gelu_256x512x256": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "float32", n),
+    "small_gemm_bf16_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", True, "float32", n),
+    "small_gemm_f16_bias_relu_200x264x136": lambda n: op_desc.gemm_bias_act(200, 264, 136, "float16", "relu", False, "float32", n),
+    "small_gemm_f16_bias_relu_200x264x136_tb": lambda n: op_desc.gemm_bias_act(200, 264, 136, "float16", "relu", True, "float32", n),
+    "small_gemm_bf16_bias_none_520x1024x776": lambda n: op_desc.gemm_bias_act(520, 1024, 776, "bfloat16", "none", False, "float32", n),
+    "n2_gemm_bf16_bias_gelu_4096x8192x8192": lambda n: op_desc.gemm_bias_act(4096, 8192, 8192, "bfloat16", "gelu", False, "float32", n),
     # the next measured row: bias / scale gradients of a [16384, 4096] bf16 activation (two column sums in one pass)
     "n1_biasgrad_bf16_16384x4096": lambda n: op_desc.bias_grad(16384, 4096, "bfloat16", n),
 }

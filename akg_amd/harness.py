@@ -60,7 +60,7 @@ def make_inputs(desc, seed=BASE_SEED, pattern=None):
 
     elementwise: N(0,1).  softmax: N(0, sigma=2).  layernorm: x, r ~ N(0,1), gamma ~ U(0.5,1.5), beta ~ N(0,0.1).
     quant: x, r ~ N(0,1) with 0.1 % of the positions overwritten by +-50.  gemm: int8 ~ U[-127,127], float scales
-    ~ U(0.001,0.02), bias ~ N(0,0.1).  Anything else: N(0,1) floats, small integers."""
+    ~ U(0.001,0.02), bias ~ N(0,0.1), 16-bit float matrix operands ~ N(0, 0.25).  Anything else: N(0,1) floats, small integers."""
     rng = np.random.default_rng(seed)
     pattern = pattern or pattern_of(desc)
     specs = [(e[0]["data_type"], e[0].get("shape", [1])) for e in desc["input_desc"]]
@@ -89,6 +89,8 @@ def make_inputs(desc, seed=BASE_SEED, pattern=None):
             mask = rng.random(size=shape, dtype=np.float32) < 0.001
             sign = np.where(rng.random(size=shape, dtype=np.float32) < 0.5, -50.0, 50.0).astype(np.float32)
             x = np.where(mask, sign, x)
+        elif pattern == "gemm" and len(shape) == 2 and min(shape) > 1 and dt in ("float16", "bfloat16"):
+            x = (rng.standard_normal(shape, dtype=np.float32) * 0.25).astype(np.float32)       # float operands
         elif pattern == "gemm":
             if len(shape) == 1 and dt != "float32":
                 x = (rng.standard_normal(shape, dtype=np.float32) * 0.1).astype(np.float32)   # bias

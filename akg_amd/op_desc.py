@@ -275,3 +275,23 @@ def mean_absmax_all(rows, cols, dtype="float32", name=None):
     mean = b.mul(b.reduce("ReduceSum", x, [0, 1], False), b.const(1.0 / (rows * cols), dtype))
     amax = b.reduce("ReduceMax", b.unary("Abs", x), [0, 1], False)
     return b.dumps([mean, amax])
+
+
+def gemm_bias_act(m, k, n, dtype="bfloat16", act="gelu", transpose_b=False, acc_dtype="float32", name=None):
+    """out = act(A @ B + bias): `dtype` operands (bfloat16 / float16), MatMul result declared `acc_dtype`, bias
+    [n] in `dtype`, activation "gelu" (tanh form, spelled with Mul/Add/Tanh), "relu" (Maximum with 0) or "none"."""
+    b = DescBuilder(name or "Fused_MatMul_Add_%s_%s_%dx%dx%d%s" % (act, _SHORT[dtype], m, k, n, "_tb" if transpose_b else ""))
+    a = b.input([m, k], dtype)
+    w = b.input([n, k] if transpose_b else [k, n], dtype)
+    bias = b.input([n], dtype)
+    x = b.matmul(a, w, acc_dtype, transpose_b=transpose_b)
+    if acc_dtype != "float32":
+        x = b.cast(x, "float32")
+    x = b.add(x, b.cast(bias, "float32"))
+    if act == "gelu":
+        x3 = b.mul(b.mul(x, x), x)
+        inner = b.mul(b.add(x, b.mul(x3, b.const(0.044715, "float32"))), b.const(0.7978845608028654, "float32"))
+        x = b.mul(b.mul(x, b.add(b.unary("Tanh", inner), b.const(1.0, "float32"))), b.const(0.5, "float32"))
+    elif act == "relu":
+        x = b.maximum(x, b.const(0.0, "float32"))
+    return b.dumps([b.cast(x, dtype)])

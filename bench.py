@@ -25,6 +25,7 @@ sys.path.insert(0, ROOT)
 FIXTURES = os.path.join(ROOT, "akg_amd", "fixtures")
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published (no sparsity)
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published (no sparsity)
 
 WORKLOADS = {
     "c1_ew_tanh_add_mul_f32_1024x4096": "f32",
@@ -34,6 +35,8 @@ WORKLOADS = {
     "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": "int8",
     # the row next to the five: two column sums (reduce direction Y) of one pass over two bf16 [16384,4096] tensors
     "n1_biasgrad_bf16_16384x4096": "f32",
+    # bfloat16 MatMul + bias + GELU on the same shape as the int8 fusion (float32 accumulation)
+    "n2_gemm_bf16_bias_gelu_4096x8192x8192": "bf16",
 }
 DEFAULT_WORKLOAD = "c2_softmax_f16_8192x4096"
 # plain streaming kernel of known size (out = -x, 256 MiB in + 256 MiB out): calibrates the HBM traffic counters
@@ -102,8 +105,10 @@ def gpu_measure(name, steps, warmup, torch, driver, harness, np):
 def roofline_of(kernel, kernel_ms, name):
     if kernel.algorithmic_ops:
         achieved = kernel.algorithmic_ops / (kernel_ms * 1e-3) / 1e12
-        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
-                "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+        int8 = WORKLOADS.get(name) == "int8"
+        peak = INT8_MFMA_PEAK_TOPS if int8 else BF16_MFMA_PEAK_TFLOPS
+        return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TOP/s" if int8 else "TFLOP/s",
+                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
     achieved = kernel.algorithmic_bytes / (kernel_ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
@@ -152,7 +157,10 @@ def main():
     is_gemm = bool(kernel.algorithmic_ops)
     if is_gemm:
         value = kernel.algorithmic_ops / (wall_ms * 1e-3) / 1e12
-        unit, metric = "TOP/s", "achieved int8 TOP/s of the fused GEMM (2*M*N*K ops per launch / time)"
+        if WORKLOADS.get(name) == "int8":
+            unit, metric = "TOP/s", "achieved int8 TOP/s of the fused GEMM (2*M*N*K ops per launch / time)"
+        else:
+            unit, metric = "TFLOP/s", "achieved TFLOP/s of the fused GEMM (2*M*N*K flops per launch / time)"
     else:
         value = kernel.algorithmic_bytes / (wall_ms * 1e-3) / 1e9
         unit, metric = "GB/s", "achieved HBM GB/s of the fused op (algorithmic bytes per launch / time)"

@@ -233,6 +233,60 @@ def test_c5_full_size_gemm_fusion():
     assert ok, msg
 
 
+def test_full_size_bf16_gemm_bias_gelu_fusion():
+    """bfloat16 MatMul + bias + GELU at 4096 x 8192 x 8192 (float32 accumulation on the MFMA units):
+    (1) 48 sampled rows against the oracle (float32 products summed serially in k) evaluated on those rows of A;
+    (2) every output against torch on the GPU (float32 matmul of the same bfloat16 values), bfloat16 tolerance."""
+    import torch
+    from oracle import np_ref
+    from akg_amd import op_desc
+    name = "n2_gemm_bf16_bias_gelu_4096x8192x8192.info"
+    path = os.path.join(FIXTURES, name)
+    print("case %s" % name, flush=True)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 6)
+    got = run_on_gpu(kernel, inputs)[0]
+    a, w, bias = inputs
+    rng = np.random.default_rng(98)
+    rows = np.sort(np.concatenate([np.arange(16) * 256 + rng.integers(0, 256, 16), rng.integers(0, 4096, 32)]))
+    sub = json_loads(op_desc.gemm_bias_act(len(rows), 8192, 8192, "bfloat16", "gelu", False, "float32", "n2_rows"))
+    expect_rows = np_ref.evaluate(sub, [a[rows], w, bias])[0]
+    ok, msg = harness.compare(got[rows], expect_rows, "bfloat16")
+    print("  sampled rows vs oracle: %s" % msg, flush=True)
+    assert ok, msg
+    dev = torch.device("cuda:0")
+    as_f32 = lambda bits: torch.from_numpy(harness.bf16_bits_to_f32(bits)).to(dev)
+    allow = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        x = as_f32(a) @ as_f32(w) + as_f32(bias)
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = allow
+    ref = torch.nn.functional.gelu(x, approximate="tanh").to(torch.bfloat16).view(torch.int16).cpu().numpy().view(np.uint16)
+    ok, msg = harness.compare(got, ref, "bfloat16")
+    print("  all outputs vs torch: %s" % msg, flush=True)
+    assert ok, msg
+
+
+def test_sixteen_bit_matmul_result_is_one_rounding_of_the_float32_sum():
+    """A MatMul whose declared result type is float16: the reference accumulates in float16 step by step, the MFMA
+    path sums in float32 and rounds once. Checked against torch float64 on a short K, where a float16 running sum
+    would still be inside the 1e-2 / 1e-3 bar (parity with the reference's own rounding sequence is not claimed)."""
+    from akg_amd import op_desc
+    text = op_desc.gemm_bias_act(128, 64, 96, "float16", "none", False, "float16", "Fused_MatMul_f16_result_128x64x96")
+    desc = json_loads(text)
+    kernel = driver.HipKernel(text)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 7)
+    got = run_on_gpu(kernel, inputs)[0]
+    a, w, bias = [x.astype(np.float64) for x in inputs]
+    acc = (a @ w).astype(np.float16).astype(np.float64)
+    ref = (acc + bias).astype(np.float32).astype(np.float16)
+    ok, msg = harness.compare(got, ref, "float16")
+    print("  float16-result MatMul vs float64: %s" % msg, flush=True)
+    assert ok, msg
+
+
 def json_loads(text):
     import json
     return json.loads(text)
