@@ -15,6 +15,7 @@ const char *kernelFamilyName(KernelFamily f) {
     case KernelFamily::RowReduce: return "row_reduce";
     case KernelFamily::GemmEpilogue: return "gemm_epilogue";
     case KernelFamily::StreamReduce: return "stream_reduce";
+    case KernelFamily::Indexed: return "indexed";
   }
   return "?";
 }
@@ -234,6 +235,12 @@ bool isElementwiseKind(OpKind k) {
     case OpKind::MatMul:
     case OpKind::Unknown:
     case OpKind::Unsupported:
+    case OpKind::Transpose:
+    case OpKind::Tile:
+    case OpKind::Slice:
+    case OpKind::StridedSlice:
+    case OpKind::Pad:
+    case OpKind::Concat:
       return false;
     default:
       return !isReduceKind(k);
@@ -1198,6 +1205,7 @@ LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options) {
   for (const OpNode &op : graph.ops) {
     if (op.kind == OpKind::MatMul) hasMatMul = true;
   }
+  if (wantsIndexedKernel(graph)) return lowerIndexedToHip(graph, options);
   if (hasMatMul) return lowerGemmToHip(graph, options);
   if (wantsStreamReduce(graph)) return lowerStreamReduceToHip(graph, options);
   TileEmitter emitter(graph, options);

@@ -1,0 +1,372 @@
+/**
+ * Indexed elementwise kernels: fusions that contain data-movement ops (Transpose, Tile, Slice, StridedSlice, Pad,
+ * Concat, and Reshape / BroadcastTo between them), where an output element no longer sits at the linear position of
+ * the input elements it is computed from.
+ *
+ * The reference lowers these ops to tosa.transpose / tosa.pad / tosa.concat / tensor.extract_slice / a
+ * linalg.generic with a read map (MindSporeToTosa.cpp:46-58,305-376,479; MindSporeToLinalg.cpp:970-1040;
+ * MindSporeFinalizingLower.cpp:102-140) and materialises every one of them in memory. Here the whole fusion is
+ * one kernel that works backwards from the outputs: a thread owns V consecutive elements of the output's
+ * innermost dimension; for each of them the value of every tensor it depends on is produced on demand at the
+ * index the ops in between map it to, down to scalar loads of the kernel inputs. Nothing intermediate touches
+ * memory and a value needed twice at the same index is computed once. Outputs are stored as V-element chunks.
+ *
+ * Reads of a transposed operand are strided across a wavefront (each lane walks its own row); this family
+ * favours generality, the register-tiled kernels of the other families do not apply to these index maps.
+ */
+#include <map>
+#include <sstream>
+
+#include "HipLowering.h"
+
+namespace akg {
+namespace {
+
+using lowering::computeTypeName;
+using lowering::dtypeTag;
+
+bool isViewKind(OpKind k) {
+  return k == OpKind::Transpose || k == OpKind::Tile || k == OpKind::Slice || k == OpKind::StridedSlice ||
+         k == OpKind::Pad || k == OpKind::Concat;
+}
+
+class IndexedEmitter {
+ public:
+  IndexedEmitter(const OpGraph &g, const LoweringOptions &o) : g_(g), opt_(o) {}
+
+  LoweredKernel run() {
+    analyse();
+    emit();
+    LoweredKernel k;
+    k.kernelName = g_.name + "_kernel";
+    k.source = src_.str();
+    k.family = KernelFamily::Indexed;
+    k.grid[0] = static_cast<unsigned>(grid_);
+    k.block[0] = kBlock;
+    k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
+    k.shapeArgs = lowering::buildShapeArgs(g_);
+    std::ostringstream note;
+    note << "indexed vec=" << vec_ << " block=" << kBlock << " grid=" << grid_ << " rank=" << space_.size();
+    k.scheduleNote = note.str();
+    return k;
+  }
+
+ private:
+  static constexpr int kBlock = 256;
+  typedef std::vector<std::string> Index;  // one C expression per dimension
+
+  const OpGraph &g_;
+  LoweringOptions opt_;
+  std::ostringstream src_;
+  std::vector<int64_t> space_;  // iteration space: the shape of the outputs
+  int vec_ = 1;
+  int64_t grid_ = 1;
+  std::vector<bool> relaxed_;
+  int nextTemp_ = 0;
+  int indent_ = 2;
+  // values already computed in the scopes that are open: (tensor id, index text) -> variable
+  std::vector<std::map<std::string, std::string>> scopes_;
+
+  std::string ctOf(int id) const { return computeTypeName(g_.tensor(id).dtype); }
+  std::string tagOf(int id) const { return dtypeTag(g_.tensor(id).dtype); }
+  void stmt(const std::string &s) { src_ << std::string(static_cast<size_t>(indent_) * 2, ' ') << s << "\n"; }
+  std::string fresh(const char *prefix) { return prefix + std::to_string(nextTemp_++); }
+
+  void analyse() {
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::Unknown) {
+        throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
+      }
+      if (op.kind == OpKind::Unsupported) throw LoweringError("op " + op.name + " has no kernel family yet");
+      if (op.kind == OpKind::MatMul || lowering::isReduceKind(op.kind)) {
+        throw LoweringError("op " + op.name + " cannot be fused with data-movement ops (Transpose, Tile, Slice, Pad, "
+                            "Concat) in one kernel yet");
+      }
+      if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+    }
+    space_ = g_.tensor(g_.outputs[0]).shape;
+    if (space_.empty()) space_.push_back(1);
+    for (int id : g_.outputs) {
+      std::vector<int64_t> s = g_.tensor(id).shape;
+      if (s.empty()) s.push_back(1);
+      if (s != space_) throw LoweringError("outputs of different shapes cannot share an indexed kernel yet");
+      if (g_.tensor(id).producer < 0) throw LoweringError("output " + g_.tensor(id).name + " is a kernel input");
+    }
+    int64_t numel = 1;
+    for (int64_t d : space_) numel *= d;
+    for (const TensorValue &t : g_.tensors) {
+      if (t.numel() >= (1LL << 31)) throw LoweringError("tensor " + t.name + " is too large for 32-bit indexing");
+    }
+    size_t widest = 1;
+    for (int id : g_.outputs) widest = std::max(widest, dtypeSize(g_.tensor(id).dtype));
+    int v = opt_.vec > 0 ? opt_.vec : static_cast<int>(16 / widest);
+    v = std::max(1, std::min(v, 16));
+    if ((v & (v - 1)) != 0) v = 1;
+    while (v > 1 && (space_.back() % v) != 0) v >>= 1;
+    vec_ = v;
+    const int64_t chunks = numel / vec_;
+    grid_ = std::max<int64_t>(1, (chunks + kBlock - 1) / kBlock);
+    if (grid_ > 2147483647LL) throw LoweringError("grid too large");
+  }
+
+  // ---- index helpers ------------------------------------------------------------------------------------
+  static std::string linearize(const Index &idx, const std::vector<int64_t> &shape) {
+    std::string e;
+    for (size_t d = 0; d < shape.size(); ++d) {
+      if (shape[d] == 1) continue;  // the index of a unit dimension is 0
+      e = e.empty() ? idx[d] : "(" + e + ") * " + std::to_string(shape[d]) + " + " + idx[d];
+    }
+    return e.empty() ? "0" : e;
+  }
+
+  // Index of `linear` (a C expression) in a dense tensor of `shape`.
+  Index delinearize(const std::string &linear, const std::vector<int64_t> &shape) {
+    const std::string base = fresh("l");
+    stmt("const int " + base + " = " + linear + ";");
+    Index out(shape.size());
+    int64_t inner = 1;
+    for (size_t d = shape.size(); d-- > 0;) {
+      if (shape[d] == 1) {
+        out[d] = "0";
+      } else {
+        std::string e = inner == 1 ? base : "(" + base + " / " + std::to_string(inner) + ")";
+        int64_t outer = 1;
+        for (size_t k = 0; k < d; ++k) outer *= shape[k];
+        if (outer != 1) e = "(" + e + " % " + std::to_string(shape[d]) + ")";
+        out[d] = e;
+      }
+      inner *= shape[d];
+    }
+    return out;
+  }
+
+  // Index of an operand that numpy-broadcasts (right-aligned) into a result of `outShape`.
+  Index broadcastIndex(const Index &idx, const std::vector<int64_t> &outShape, const std::vector<int64_t> &inShape,
+                       const std::string &what) {
+    std::vector<int64_t> in = inShape;
+    while (in.size() > outShape.size() && in.front() == 1) in.erase(in.begin());
+    if (in.size() > outShape.size()) throw LoweringError(what + ": operand rank exceeds the result's");
+    const size_t off = outShape.size() - in.size();
+    Index out(inShape.size(), "0");
+    const size_t lead = inShape.size() - in.size();
+    for (size_t d = 0; d < in.size(); ++d) {
+      if (in[d] == 1) continue;
+      if (in[d] != outShape[off + d]) throw LoweringError(what + ": operand does not broadcast to the result");
+      out[lead + d] = idx[off + d];
+    }
+    return out;
+  }
+
+  static std::string keyOf(int id, const Index &idx) {
+    std::string k = std::to_string(id) + "@";
+    for (const std::string &s : idx) k += s + ",";
+    return k;
+  }
+
+  const std::string *lookup(const std::string &key) const {
+    for (size_t s = scopes_.size(); s-- > 0;) {
+      auto it = scopes_[s].find(key);
+      if (it != scopes_[s].end()) return &it->second;
+    }
+    return nullptr;
+  }
+
+  // ---- value of tensor `id` at `idx`: emits what is needed and returns a C expression of the compute type ----
+  std::string valueAt(int id, Index idx) {
+    const TensorValue &t = g_.tensor(id);
+    if (t.isConst) return lowering::literalFor(t.dtype, t.constValue);
+    if (idx.size() != std::max<size_t>(1, t.shape.size())) throw LoweringError("internal: index rank of " + t.name);
+    for (size_t d = 0; d < t.shape.size(); ++d) {
+      if (t.shape[d] == 1) idx[d] = "0";
+    }
+    const std::string key = keyOf(id, idx);
+    if (const std::string *known = lookup(key)) return *known;
+    const std::string var = fresh("v");
+    const std::string ct = ctOf(id);
+    if (t.producer < 0) {
+      if (t.inputIndex < 0) throw LoweringError("operand " + t.name + " is undefined");
+      stmt("const " + ct + " " + var + " = " + tagOf(id) + "::load(in" + std::to_string(t.inputIndex) + "[" +
+           linearize(idx, t.shape) + "]);");
+      scopes_.back()[key] = var;
+      return var;
+    }
+    const OpNode &op = g_.ops[static_cast<size_t>(t.producer)];
+    const std::vector<int64_t> outShape = t.shape.empty() ? std::vector<int64_t>{1} : t.shape;
+    auto inShapeOf = [&](size_t i) {
+      const std::vector<int64_t> &s = g_.tensor(op.inputs[i]).shape;
+      return s.empty() ? std::vector<int64_t>{1} : s;
+    };
+    const std::string note = "  // " + op.name + " -> " + t.name;
+    switch (op.kind) {
+      case OpKind::Reshape: {
+        const Index src = delinearize(linearize(idx, outShape), inShapeOf(0));
+        stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
+        break;
+      }
+      case OpKind::BroadcastTo: {
+        const Index src = broadcastIndex(idx, outShape, inShapeOf(0), "op " + op.name);
+        stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
+        break;
+      }
+      case OpKind::Transpose: {
+        Index src(idx.size());
+        for (size_t d = 0; d < idx.size(); ++d) src[static_cast<size_t>(op.perm[d])] = idx[d];
+        stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
+        break;
+      }
+      case OpKind::Tile: {
+        const std::vector<int64_t> in = inShapeOf(0);
+        Index src(idx.size());
+        for (size_t d = 0; d < idx.size(); ++d) {
+          src[d] = in[d] == outShape[d] ? idx[d] : "(" + idx[d] + " % " + std::to_string(in[d]) + ")";
+        }
+        stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
+        break;
+      }
+      case OpKind::Slice:
+      case OpKind::StridedSlice: {
+        Index src(idx.size());
+        for (size_t d = 0; d < idx.size(); ++d) {
+          std::string e = idx[d];
+          if (op.strides[d] != 1) e = e + " * " + std::to_string(op.strides[d]);
+          if (op.begin[d] != 0) e = std::to_string(op.begin[d]) + " + " + e;
+          src[d] = "(" + e + ")";
+        }
+        stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
+        break;
+      }
+      case OpKind::Pad: {
+        const std::vector<int64_t> in = inShapeOf(0);
+        std::string cond;
+        Index src(idx.size());
+        for (size_t d = 0; d < idx.size(); ++d) {
+          src[d] = op.begin[d] == 0 ? idx[d] : "(" + idx[d] + " - " + std::to_string(op.begin[d]) + ")";
+          if (in[d] == outShape[d]) continue;
+          const std::string c = "static_cast<unsigned>(" + src[d] + ") < " + std::to_string(in[d]) + "u";
+          cond = cond.empty() ? c : cond + " && " + c;
+        }
+        const std::string fill = lowering::literalFor(t.dtype, static_cast<double>(op.padValue));
+        if (cond.empty()) {
+          stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
+        } else {
+          stmt(ct + " " + var + " = " + fill + ";" + note);
+          stmt("if (" + cond + ") {");
+          openScope();
+          stmt(var + " = " + valueAt(op.inputs[0], src) + ";");
+          closeScope();
+          stmt("}");
+        }
+        break;
+      }
+      case OpKind::Concat: {
+        const std::vector<int64_t> first = inShapeOf(0);
+        const size_t a = static_cast<size_t>(op.concatAxis);
+        Index second = idx;
+        second[a] = "(" + idx[a] + " - " + std::to_string(first[a]) + ")";
+        stmt(ct + " " + var + ";" + note);
+        stmt("if (" + idx[a] + " < " + std::to_string(first[a]) + ") {");
+        openScope();
+        stmt(var + " = " + valueAt(op.inputs[0], idx) + ";");
+        closeScope();
+        stmt("} else {");
+        openScope();
+        stmt(var + " = " + valueAt(op.inputs[1], second) + ";");
+        closeScope();
+        stmt("}");
+        break;
+      }
+      default: {
+        if (!lowering::isElementwiseKind(op.kind)) throw LoweringError("op " + op.name + " has no indexed lowering");
+        std::vector<std::string> operands;
+        for (size_t i = 0; i < op.inputs.size(); ++i) {
+          const TensorValue &in = g_.tensor(op.inputs[i]);
+          if (in.isConst) {
+            operands.push_back(lowering::literalFor(in.dtype, in.constValue));
+            continue;
+          }
+          operands.push_back(valueAt(op.inputs[i], broadcastIndex(idx, outShape, inShapeOf(i), "op " + op.name)));
+        }
+        const std::string expr = lowering::elementwiseExpr(g_, op, operands, relaxed_[static_cast<size_t>(id)]);
+        stmt("const " + ct + " " + var + " = " + expr + ";" + note);
+        break;
+      }
+    }
+    scopes_.back()[key] = var;
+    return var;
+  }
+
+  void openScope() {
+    scopes_.emplace_back();
+    ++indent_;
+  }
+  void closeScope() {
+    scopes_.pop_back();
+    --indent_;
+  }
+
+  void emit() {
+    relaxed_ = lowering::relaxedPrecisionTensors(g_);
+    const std::string kname = g_.name + "_kernel";
+    src_ << "// Generated by the akg HIP lowering for gfx950. Op description: " << g_.name << "\n";
+    src_ << "// family: indexed, fusion class: " << operatorTemplateName(g_.operatorTemplate) << "\n";
+    src_ << "#include \"akg_rt.hpp\"\n\n";
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << kname << "(";
+    size_t argc = 0;
+    for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
+      src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
+    }
+    src_ << ") {\n";
+    int64_t numel = 1;
+    for (int64_t d : space_) numel *= d;
+    src_ << "  constexpr int V = " << vec_ << ";\n";
+    src_ << "  const int chunk = static_cast<int>(blockIdx.x) * " << kBlock << " + static_cast<int>(threadIdx.x);\n";
+    src_ << "  if (chunk >= " << numel / vec_ << ") return;\n";
+    src_ << "  const int base = chunk * V;  // linear position of this thread's first element\n";
+    indent_ = 1;
+    scopes_.clear();
+    scopes_.emplace_back();
+    // index of the chunk's first element; the innermost coordinate advances with e and never wraps (V divides it)
+    Index start = delinearize("base", space_);
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      stmt(ctOf(g_.outputs[i]) + " o" + std::to_string(i) + "[V];");
+    }
+    stmt("#pragma unroll");
+    stmt("for (int e = 0; e < V; ++e) {");
+    openScope();
+    Index idx = start;
+    if (space_.back() != 1) {
+      stmt("const int inner = " + start.back() + " + e;");
+      idx.back() = "inner";
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      const std::string v = valueAt(g_.outputs[i], idx);
+      stmt("o" + std::to_string(i) + "[e] = " + v + ";");
+    }
+    closeScope();
+    stmt("}");
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, false>(out" + std::to_string(i) + " + base, o" +
+           std::to_string(i) + ");");
+    }
+    src_ << "}\n";
+  }
+};
+
+}  // namespace
+
+bool wantsIndexedKernel(const OpGraph &graph) {
+  for (const OpNode &op : graph.ops) {
+    if (isViewKind(op.kind)) return true;
+  }
+  return false;
+}
+
+LoweredKernel lowerIndexedToHip(const OpGraph &graph, const LoweringOptions &options) {
+  IndexedEmitter emitter(graph, options);
+  return emitter.run();
+}
+
+}  // namespace akg

@@ -83,18 +83,18 @@ const OpTableEntry kOpTable[] = {
   {"ElemAny", OpKind::Unsupported},
   {"ArgMax", OpKind::Unsupported},
   {"BroadcastTo", OpKind::BroadcastTo},
-  {"Slice", OpKind::Unsupported},
-  {"Tile", OpKind::Unsupported},
-  {"Concat", OpKind::Unsupported},
+  {"Slice", OpKind::Slice},
+  {"Tile", OpKind::Tile},
+  {"Concat", OpKind::Concat},
   {"Reshape", OpKind::Reshape},
-  {"Transpose", OpKind::Unsupported},
+  {"Transpose", OpKind::Transpose},
   {"Split", OpKind::Unsupported},
-  {"Pad", OpKind::Unsupported},
+  {"Pad", OpKind::Pad},
   {"Gather", OpKind::Unsupported},
   {"InplaceAssign", OpKind::Unsupported},
   {"Assign", OpKind::Unsupported},
   {"UnsortedSegmentSum", OpKind::Unsupported},
-  {"StridedSlice", OpKind::Unsupported},
+  {"StridedSlice", OpKind::StridedSlice},
   {"AddN", OpKind::AddN},
   {"MatMul", OpKind::MatMul},
   {"BatchMatMul", OpKind::Unsupported},
@@ -281,6 +281,7 @@ class GraphBuilder {
         for (size_t j = 0; j < inputDesc.size(); ++j) {
           if (isIndex1DAttrAsInput(node.name, j)) continue;
           if (node.kind == OpKind::Cast && j > 0) continue;  // convertCastOp keeps the first operand only (:1351-1360)
+          if (node.kind == OpKind::StridedSlice && j > 0) continue;  // begin / end / strides carried as constants
           node.inputs.push_back(operandFor(inputDesc[j][0], node.name));
         }
       }
@@ -314,6 +315,11 @@ class GraphBuilder {
         if (const json::Value *b = findAttr(attrs, kTransposeB)) node.transposeB = b->asBool();
       }
 
+      if (node.kind == OpKind::Transpose || node.kind == OpKind::Tile || node.kind == OpKind::Slice ||
+          node.kind == OpKind::StridedSlice || node.kind == OpKind::Pad || node.kind == OpKind::Concat) {
+        parseDataMovement(&node, attrs, inputDesc, readShape(outputDesc[0]));
+      }
+
       int opIndex = static_cast<int>(graph_.ops.size());
       for (size_t j = 0; j < outputDesc.size(); ++j) {
         const json::Value &d = outputDesc[j];
@@ -325,6 +331,151 @@ class GraphBuilder {
         operandList_[tensorName] = id;
       }
       graph_.ops.push_back(node);
+    }
+  }
+
+  // Attributes of the data-movement ops, checked against the declared result shape.
+  //   Transpose    perm from the second input's value or attr "perm" (convertTransposeOp :965-979)
+  //   Tile         multiples from the second input's value or attr "multiples"; rank stays (convertTileOp
+  //                :1126-1135, MindSporeToLinalg.cpp:970-1040)
+  //   Slice        attrs "begin", "size" (-1: to the end) (convertSliceOp :1089-1101)
+  //   StridedSlice attrs or constant inputs begin / end / strides, negative end counted from the back; the
+  //                lowering uses these three only (MindSporeFinalizingLower.cpp:102-140), so non-zero masks are refused
+  //   Pad          attr "padding" = (before, after) pairs listed from the LAST dimension backwards, "value",
+  //                mode "constant" (MindSporeToTosa.cpp:305-376)
+  //   Concat       two operands, attr "axis" (default 0) (convertConcatOp :1117-1124)
+  void parseDataMovement(OpNode *node, const json::Value &attrs, const json::Value &inputDesc,
+                         const std::vector<int64_t> &outShape) {
+    const std::string &nm = node->name;
+    if (node->inputs.empty()) throw TranslateError("op " + nm + ": missing operand");
+    const std::vector<int64_t> inShape = graph_.tensor(node->inputs[0]).shape;
+    const size_t rank = inShape.size();
+    auto listFrom = [&](size_t inputIdx, const char *attrName) -> std::vector<int64_t> {
+      if (inputDesc.size() > inputIdx && inputDesc[inputIdx][0].contains(kValue)) {
+        const json::Value &v = inputDesc[inputIdx][0].at(kValue);
+        if (v.isArray()) return v.asIntVector();
+        return {static_cast<int64_t>(v.asDouble())};
+      }
+      if (const json::Value *a = findAttr(attrs, attrName)) {
+        if (a->isArray()) return a->asIntVector();
+        return {static_cast<int64_t>(a->asDouble())};
+      }
+      throw TranslateError("op " + nm + ": cannot find attribute " + attrName);
+    };
+    auto needRank = [&](const std::vector<int64_t> &v, const char *what) {
+      if (v.size() != rank) throw TranslateError("op " + nm + ": " + what + " must have one entry per dimension");
+    };
+    std::vector<int64_t> expect(rank, 0);
+    switch (node->kind) {
+      case OpKind::Transpose: {
+        node->perm = listFrom(1, "perm");
+        needRank(node->perm, "perm");
+        std::vector<bool> seen(rank, false);
+        for (size_t d = 0; d < rank; ++d) {
+          int64_t p = node->perm[d];
+          if (p < 0) p += static_cast<int64_t>(rank);
+          if (p < 0 || p >= static_cast<int64_t>(rank) || seen[static_cast<size_t>(p)]) {
+            throw TranslateError("op " + nm + ": perm is not a permutation");
+          }
+          seen[static_cast<size_t>(p)] = true;
+          node->perm[d] = p;
+          expect[d] = inShape[static_cast<size_t>(p)];
+        }
+        break;
+      }
+      case OpKind::Tile: {
+        const std::vector<int64_t> mult = listFrom(1, "multiples");
+        needRank(mult, "multiples");
+        for (size_t d = 0; d < rank; ++d) {
+          if (mult[d] < 1) throw TranslateError("op " + nm + ": multiples must be positive");
+          expect[d] = inShape[d] * mult[d];
+        }
+        break;
+      }
+      case OpKind::Slice: {
+        node->begin = listFrom(99, "begin");
+        std::vector<int64_t> size = listFrom(99, "size");
+        needRank(node->begin, "begin");
+        needRank(size, "size");
+        node->strides.assign(rank, 1);
+        for (size_t d = 0; d < rank; ++d) {
+          if (size[d] == -1) size[d] = inShape[d] - node->begin[d];
+          if (node->begin[d] < 0 || size[d] < 0 || node->begin[d] + size[d] > inShape[d]) {
+            throw TranslateError("op " + nm + ": slice exceeds the operand");
+          }
+          expect[d] = size[d];
+        }
+        break;
+      }
+      case OpKind::StridedSlice: {
+        const bool withAttr = findAttr(attrs, "begin") != nullptr;
+        node->begin = withAttr ? listFrom(99, "begin") : listFrom(1, "begin");
+        std::vector<int64_t> end = withAttr ? listFrom(99, "end") : listFrom(2, "end");
+        node->strides = withAttr ? listFrom(99, "strides") : listFrom(3, "strides");
+        needRank(node->begin, "begin");
+        needRank(end, "end");
+        needRank(node->strides, "strides");
+        for (const char *mask : {"beginMask", "endMask", "ellipsisMask", "newAxisMask", "shrinkAxisMask"}) {
+          const json::Value *m = findAttr(attrs, mask);
+          if (m != nullptr && m->asDouble() != 0.0) {
+            throw TranslateError("op " + nm + ": a non-zero " + mask + " is not supported");
+          }
+        }
+        for (size_t d = 0; d < rank; ++d) {
+          if (end[d] < 0) end[d] += inShape[d];
+          if (node->strides[d] < 1) throw TranslateError("op " + nm + ": strides must be positive");
+          if (node->begin[d] < 0 || end[d] > inShape[d] || end[d] < node->begin[d]) {
+            throw TranslateError("op " + nm + ": slice exceeds the operand");
+          }
+          expect[d] = (end[d] - node->begin[d] + node->strides[d] - 1) / node->strides[d];
+        }
+        break;
+      }
+      case OpKind::Pad: {
+        const std::vector<int64_t> padding = listFrom(99, "padding");
+        if (padding.size() % 2 != 0 || padding.size() / 2 > rank) {
+          throw TranslateError("op " + nm + ": padding must hold (before, after) pairs for at most every dimension");
+        }
+        if (const json::Value *m = findAttr(attrs, "mode")) {
+          if (m->isString() && m->asString() != "constant") {
+            throw TranslateError("op " + nm + ": only constant padding is supported");
+          }
+        }
+        if (const json::Value *v = findAttr(attrs, kValue)) node->padValue = static_cast<int64_t>(v->asDouble());
+        node->begin.assign(rank, 0);
+        std::vector<int64_t> high(rank, 0);
+        for (size_t i = 0; i < padding.size() / 2; ++i) {
+          if (padding[2 * i] < 0 || padding[2 * i + 1] < 0) throw TranslateError("op " + nm + ": negative padding");
+          node->begin[rank - 1 - i] = padding[2 * i];
+          high[rank - 1 - i] = padding[2 * i + 1];
+        }
+        for (size_t d = 0; d < rank; ++d) expect[d] = inShape[d] + node->begin[d] + high[d];
+        break;
+      }
+      case OpKind::Concat: {
+        if (node->inputs.size() != 2) throw TranslateError("op " + nm + ": exactly two operands are supported");
+        int64_t axis = 0;
+        if (const json::Value *a = findAttr(attrs, kAxis)) {
+          axis = a->isArray() ? a->asIntVector().at(0) : static_cast<int64_t>(a->asDouble());
+        }
+        if (axis < 0) axis += static_cast<int64_t>(rank);
+        if (axis < 0 || axis >= static_cast<int64_t>(rank)) throw TranslateError("op " + nm + ": axis out of range");
+        node->concatAxis = axis;
+        const std::vector<int64_t> &other = graph_.tensor(node->inputs[1]).shape;
+        if (other.size() != rank) throw TranslateError("op " + nm + ": operands differ in rank");
+        for (size_t d = 0; d < rank; ++d) {
+          if (static_cast<int64_t>(d) != axis && other[d] != inShape[d]) {
+            throw TranslateError("op " + nm + ": operands differ outside the concatenation axis");
+          }
+          expect[d] = inShape[d] + (static_cast<int64_t>(d) == axis ? other[d] : 0);
+        }
+        break;
+      }
+      default:
+        break;
+    }
+    if (expect != outShape) {
+      throw TranslateError("op " + nm + ": the declared result shape does not follow from the operand and attributes");
     }
   }
 
@@ -373,7 +524,15 @@ OperatorTemplate templateOfOp(const OpGraph &g, const OpNode &op) {
     case OpKind::Reshape:
       return OperatorTemplate::Reshape;
     case OpKind::BroadcastTo:
+    case OpKind::Tile:
       return OperatorTemplate::Broadcast;
+    case OpKind::Transpose:
+      return OperatorTemplate::Transpose;
+    case OpKind::Slice:
+    case OpKind::StridedSlice:
+    case OpKind::Pad:
+    case OpKind::Concat:
+      return OperatorTemplate::Default;  // not classified by getOperatorTemplate (OperatorIdentify.cpp:51-75)
     case OpKind::Unknown:
     case OpKind::Unsupported:
       return OperatorTemplate::Default;
@@ -491,6 +650,12 @@ const char *opKindName(OpKind k) {
     case OpKind::ReduceAny: return "reduce_any";
     case OpKind::Reshape: return "reshape";
     case OpKind::BroadcastTo: return "broadcast_to";
+    case OpKind::Transpose: return "transpose";
+    case OpKind::Tile: return "tile";
+    case OpKind::Slice: return "slice";
+    case OpKind::StridedSlice: return "strided_slice";
+    case OpKind::Pad: return "pad";
+    case OpKind::Concat: return "concat";
     case OpKind::MatMul: return "matmul";
     case OpKind::AddN: return "addn";
     case OpKind::Unsupported: return "unsupported";
@@ -606,6 +771,28 @@ std::string printOpGraph(const OpGraph &g) {
     if (op.kind == OpKind::MatMul) {
       os << " {transpose_a = " << (op.transposeA ? "true" : "false")
          << ", transpose_b = " << (op.transposeB ? "true" : "false") << "}";
+    }
+    auto list = [&](const char *key, const std::vector<int64_t> &v) {
+      os << key << " = [";
+      for (size_t i = 0; i < v.size(); ++i) os << (i ? ", " : "") << v[i];
+      os << "]";
+    };
+    if (op.kind == OpKind::Transpose) {
+      os << " {";
+      list("perm", op.perm);
+      os << "}";
+    } else if (op.kind == OpKind::Slice || op.kind == OpKind::StridedSlice) {
+      os << " {";
+      list("start", op.begin);
+      os << ", ";
+      list("strides", op.strides);
+      os << "}";
+    } else if (op.kind == OpKind::Pad) {
+      os << " {";
+      list("low", op.begin);
+      os << ", value = " << op.padValue << "}";
+    } else if (op.kind == OpKind::Concat) {
+      os << " {axis = " << op.concatAxis << "}";
     }
     if (op.kind == OpKind::Unknown) os << " {ori_op = \"" << op.name << "\"}";
     os << " : " << typeStr(g.tensor(op.outputs[0])) << "\n";

@@ -45,6 +45,8 @@ enum class OpKind {
   ReduceSum, ReduceMax, ReduceMin, ReduceProd, ReduceAll, ReduceAny,
   // shape
   Reshape, BroadcastTo,
+  // data movement: the result is the operand read through an index map
+  Transpose, Tile, Slice, StridedSlice, Pad, Concat,
   // contraction
   MatMul,
   // n-ary
@@ -86,6 +88,12 @@ struct OpNode {
   bool keepDims = false;
   bool transposeA = false;
   bool transposeB = false;
+  // data-movement ops, one entry per dimension of the operand (all normalised by the translator):
+  std::vector<int64_t> perm;       // Transpose: result dim d is operand dim perm[d]
+  std::vector<int64_t> begin;      // Slice / StridedSlice: first index taken; Pad: elements added in front
+  std::vector<int64_t> strides;    // StridedSlice: step (positive); Slice: all ones
+  int64_t padValue = 0;            // Pad: the constant written outside the operand
+  int64_t concatAxis = 0;          // Concat: axis along which the operands follow one another
   std::string ptrAddress;
 };
 

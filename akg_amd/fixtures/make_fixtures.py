@@ -45,6 +45,13 @@ FIXTURES = {
     "small_biasgrad_f32_100x37": lambda n: op_desc.bias_grad(100, 37, "float32", n),
     "small_sub_exp_reducesum_split_f32_4x96x160": lambda n: op_desc.sub_exp_reduce_y(4, 96, 160, "float32", n),
     "small_mean_absmax_all_f32_1000x1000": lambda n: op_desc.mean_absmax_all(1000, 1000, "float32", n),
+    # data-movement ops (indexed family)
+    "small_view_chain_f32": lambda n: op_desc.view_chain(n),
+    "small_transpose_bias_add_bf16_3x20x36": lambda n: op_desc.transpose_bias_add(3, 20, 36, "bfloat16", n),
+    "small_transpose_0213_neg_f16_2x5x6x8": lambda n: op_desc.transpose_0213_neg([2, 5, 6, 8], "float16", n),
+    "small_slice_concat_pad_add_i32": lambda n: op_desc.slice_concat_int(n),
+    "small_transpose_reshape_add_f32_4x6x10": lambda n: op_desc.transpose_reshape_add(n),
+    "n3_transpose_bias_add_bf16_32x2048x1024": lambda n: op_desc.transpose_bias_add(32, 2048, 1024, "bfloat16", n),
     # float MatMul + bias + activation on the bfloat16 / float16 MFMA path
     "small_gemm_bf16_bias_gelu_256x512x256": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "float32", n),
     "small_gemm_bf16_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", True, "float32", n),

@@ -295,3 +295,101 @@ def gemm_bias_act(m, k, n, dtype="bfloat16", act="gelu", transpose_b=False, acc_
     elif act == "relu":
         x = b.maximum(x, b.const(0.0, "float32"))
     return b.dumps([b.cast(x, dtype)])
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Data-movement ops (Transpose, Tile, Slice, StridedSlice, Pad, Concat) on DescBuilder values.
+# ---------------------------------------------------------------------------------------------------------
+def _listint(name, value):
+    return {"data_type": "listInt", "name": name, "value": [int(v) for v in value]}
+
+
+def transpose(b, x, perm):
+    shape = [x.shape[p] for p in perm]
+    return b.op("Transpose", [x], shape, x.dtype, attrs=[_listint("perm", perm)])
+
+
+def tile(b, x, multiples):
+    shape = [d * m for d, m in zip(x.shape, multiples)]
+    return b.op("Tile", [x], shape, x.dtype, attrs=[_listint("multiples", multiples)])
+
+
+def slice_(b, x, begin, size):
+    shape = [x.shape[d] - begin[d] if s == -1 else s for d, s in enumerate(size)]
+    return b.op("Slice", [x], shape, x.dtype, attrs=[_listint("begin", begin), _listint("size", size)])
+
+
+def strided_slice(b, x, begin, end, strides):
+    e = [v + x.shape[d] if v < 0 else v for d, v in enumerate(end)]
+    shape = [(e[d] - begin[d] + strides[d] - 1) // strides[d] for d in range(len(begin))]
+    return b.op("StridedSlice", [x], shape, x.dtype,
+                attrs=[_listint("begin", begin), _listint("end", end), _listint("strides", strides)])
+
+
+def pad(b, x, padding, value=0):
+    """`padding` = (before, after) pairs, the first pair for the last dimension."""
+    shape = list(x.shape)
+    for i in range(len(padding) // 2):
+        shape[len(shape) - 1 - i] += padding[2 * i] + padding[2 * i + 1]
+    return b.op("Pad", [x], shape, x.dtype, attrs=[_listint("padding", padding),
+                                                   {"data_type": "int", "name": "value", "value": int(value)},
+                                                   {"data_type": "str", "name": "mode", "value": "constant"}])
+
+
+def concat(b, x, y, axis):
+    shape = list(x.shape)
+    shape[axis] += y.shape[axis]
+    return b.op("Concat", [x, y], shape, x.dtype, attrs=[{"data_type": "int", "name": "axis", "value": int(axis)}])
+
+
+def transpose_bias_add(batch, rows, cols, dtype="bfloat16", name=None):
+    """out[b, c, r] = x[b, r, c] + bias[r] (bias broadcast along the new innermost axis is [rows]): the layout change
+    in front of an attention score product, fused with an elementwise op."""
+    b = DescBuilder(name or "Fused_Transpose_Add_%s_%dx%dx%d" % (_SHORT[dtype], batch, rows, cols))
+    x = b.input([batch, rows, cols], dtype)
+    bias = b.input([rows], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    y = b.add(f(transpose(b, x, [0, 2, 1])), f(bias))
+    return b.dumps([b.cast(y, dtype) if dtype != "float32" else y])
+
+
+def view_chain(name=None):
+    """Every data-movement op once, on small ragged shapes: pad -> tile -> strided slice -> transpose, a slice of a
+    second input concatenated on, then an elementwise op."""
+    b = DescBuilder(name or "Fused_Pad_Tile_StridedSlice_Transpose_Slice_Concat_Mul_f32")
+    x = b.input([5, 7], "float32")
+    y = b.input([9, 30], "float32")
+    p = pad(b, x, [1, 2, 3, 0], value=2)            # [8, 10]
+    t = tile(b, p, [2, 3])                          # [16, 30]
+    s = strided_slice(b, t, [1, 0], [-1, 30], [2, 1])  # [7, 30]
+    tr = transpose(b, s, [1, 0])                    # [30, 7]
+    ys = slice_(b, y, [2, 0], [4, -1])              # [4, 30]
+    c = concat(b, tr, transpose(b, ys, [1, 0]), 1)  # [30, 11]
+    return b.dumps([b.mul(c, b.const(0.5, "float32"))])
+
+
+def transpose_0213_neg(shape, dtype="float16", name=None):
+    """out = -transpose(x, [0, 2, 1, 3]): the innermost axis stays innermost (head / sequence swap of attention)."""
+    b = DescBuilder(name or "Fused_Transpose_Neg_%s_%s" % (_SHORT[dtype], "x".join(str(d) for d in shape)))
+    x = b.input(list(shape), dtype)
+    return b.dumps([b.unary("Neg", transpose(b, x, [0, 2, 1, 3]))])
+
+
+def slice_concat_int(name=None):
+    """int32: two slices of one input concatenated in swapped order along axis 0, plus a padded second input."""
+    b = DescBuilder(name or "Fused_Slice_Slice_Concat_Pad_Add_i32")
+    x = b.input([12, 16], "int32")
+    y = b.input([10, 12], "int32")
+    top = slice_(b, x, [0, 0], [5, -1])
+    bottom = slice_(b, x, [5, 0], [-1, -1])
+    swapped = concat(b, bottom, top, 0)                 # [12, 16]
+    return b.dumps([b.add(swapped, pad(b, y, [3, 1, 0, 2], value=-7))])
+
+
+def transpose_reshape_add(name=None):
+    """x [4,6,10] -> transpose [1,0,2] -> reshape [24,10] -> + y [24,10]: a Reshape between data-movement ops."""
+    b = DescBuilder(name or "Fused_Transpose_Reshape_Add_f32_4x6x10")
+    x = b.input([4, 6, 10], "float32")
+    y = b.input([24, 10], "float32")
+    t = b.reshape(transpose(b, x, [1, 0, 2]), [24, 10])
+    return b.dumps([b.add(t, y)])

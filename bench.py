@@ -35,6 +35,8 @@ WORKLOADS = {
     "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": "int8",
     # the row next to the five: two column sums (reduce direction Y) of one pass over two bf16 [16384,4096] tensors
     "n1_biasgrad_bf16_16384x4096": "f32",
+    # batched transpose [32,2048,1024] -> [32,1024,2048] fused with a bias add (indexed family)
+    "n3_transpose_bias_add_bf16_32x2048x1024": "f32",
     # bfloat16 MatMul + bias + GELU on the same shape as the int8 fusion (float32 accumulation)
     "n2_gemm_bf16_bias_gelu_4096x8192x8192": "bf16",
 }

@@ -33,6 +33,11 @@ import struct
 import subprocess
 import sys
 
+try:
+    from oracle.view_attrs import VIEW_OPS, view_params
+except ImportError:  # run as a script from inside oracle/
+    from view_attrs import VIEW_OPS, view_params
+
 FLOATS = ("float16", "bfloat16", "float32", "float64")
 INTS = ("int8", "int16", "int32", "int64")
 
@@ -194,6 +199,8 @@ def parse(desc):
                 continue
             if name == "Cast" and idx > 0:
                 continue
+            if name == "StridedSlice" and idx > 0:
+                continue
             d = entry[0]
             if d["tensor_name"] in tensors:
                 ins.append(tensors[d["tensor_name"]])
@@ -212,6 +219,8 @@ def parse(desc):
         o = od["output_desc"][0]
         out = T(o["tensor_name"], o.get("shape", [1]), o["data_type"])
         op = Op(name, ins, out, attrs)
+        if name in VIEW_OPS:
+            op.view = view_params(od, ins[0].shape)
         out.producer = op
         if name in REDUCES:
             if len(od["input_desc"]) == 2:
@@ -263,7 +272,7 @@ class Emitter:
 
     # -- which values live in memory --------------------------------------------------------------------
     def is_elementwise(self, op):
-        return op.name not in REDUCES and op.name not in ("MatMul", "Reshape")
+        return op.name not in REDUCES and op.name not in ("MatMul", "Reshape") and op.name not in VIEW_OPS
 
     def plan(self):
         consumers = {}
@@ -276,11 +285,11 @@ class Emitter:
                 out.alias_of = op.inputs[0]
                 continue
             inline = (self.is_elementwise(op) and out.uses == 1 and not out.is_output
-                      and consumers[out.name][0].name not in ("MatMul", "Reshape"))
+                      and consumers[out.name][0].name not in ("MatMul", "Reshape") + VIEW_OPS)
             out.inline = inline
         # the source of a Reshape view and MatMul operands must be in memory
         for op in self.ops:
-            if op.name in ("Reshape", "MatMul"):
+            if op.name in ("Reshape", "MatMul") + VIEW_OPS:
                 for t in op.inputs:
                     if t.producer is not None and t.producer.name != "Reshape":
                         t.inline = False
@@ -466,6 +475,54 @@ class Emitter:
         self.emit("%s[%s] = %s;" % (out.buffer, self.index_expr(out, shape), self.store_expr(out.dtype, expr)), depth)
         self.close_loops(len(shape), depth)
 
+    def emit_view(self, op):
+        """Data-movement op: a loop nest over the result that copies the operand element its index map names."""
+        out, src, vp = op.output, op.inputs[0], op.view
+        if src.const is not None or out.dtype != src.dtype:
+            raise OracleError("%s: operand must be a tensor of the result's type" % op.name)
+        shape = out.shape
+        rank = len(shape)
+        depth = self.open_loops(shape, True)
+        idx = ["i%d" % d for d in range(rank)]
+
+        def lin(t, terms):
+            expr = None
+            for term, extent in zip(terms, t.shape):
+                expr = term if expr is None else "(%s) * %dL + %s" % (expr, extent, term)
+            return expr or "0"
+
+        def load(t, terms):
+            return self.load_expr(self.root(t), lin(t, terms))
+
+        n = op.name
+        if n == "Transpose":
+            terms = [None] * rank
+            for d, p in enumerate(vp["perm"]):
+                terms[p] = idx[d]
+            value = load(src, terms)
+        elif n == "Tile":
+            value = load(src, ["(%s %% %dL)" % (idx[d], src.shape[d]) for d in range(rank)])
+        elif n in ("Slice", "StridedSlice"):
+            value = load(src, ["(%dL + %s * %dL)" % (vp["begin"][d], idx[d], vp["strides"][d]) for d in range(rank)])
+        elif n == "Pad":
+            cond = " && ".join("%s >= %dL && %s < %dL" % (idx[d], vp["low"][d], idx[d], vp["low"][d] + src.shape[d])
+                               for d in range(rank))
+            inner = load(src, ["(%s - %dL)" % (idx[d], vp["low"][d]) for d in range(rank)])
+            if out.dtype in FLOATS:
+                fill = float_literal(out.dtype, float(vp["value"]))
+            else:
+                fill = "((%s)%dLL)" % (C_COMPUTE[out.dtype], vp["value"])
+            value = "((%s) ? %s : %s)" % (cond, inner, fill)
+        else:
+            other, a = op.inputs[1], vp["axis"]
+            if other.const is not None or other.dtype != out.dtype:
+                raise OracleError("Concat: operands must be tensors of the result's type")
+            second = list(idx)
+            second[a] = "(%s - %dL)" % (idx[a], src.shape[a])
+            value = "((%s < %dL) ? %s : %s)" % (idx[a], src.shape[a], load(src, idx), load(other, second))
+        self.emit("%s[%s] = %s;" % (out.buffer, lin(out, idx), self.store_expr(out.dtype, value)), depth)
+        self.close_loops(rank, depth)
+
     def emit_reduce(self, op):
         src, out = op.inputs[0], op.output
         od = out.dtype
@@ -607,6 +664,8 @@ class Emitter:
                 self.emit_reduce(op)
             elif op.name == "MatMul":
                 self.emit_matmul(op)
+            elif op.name in VIEW_OPS:
+                self.emit_view(op)
             else:
                 self.emit_elementwise(op)
         for b in self.temps:

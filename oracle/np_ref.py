@@ -22,6 +22,8 @@ import json
 
 import numpy as np
 
+from oracle.view_attrs import VIEW_OPS, view_params
+
 FLOATS = ("float16", "bfloat16", "float32", "float64")
 NP_DTYPE = {"bool": np.bool_, "int8": np.int8, "int16": np.int16, "int32": np.int32, "int64": np.int64,
             "float16": np.float16, "bfloat16": np.float32, "float32": np.float32, "float64": np.float64}
@@ -176,6 +178,8 @@ def evaluate(desc, inputs):
                 continue
             if name == "Cast" and idx > 0:
                 continue
+            if name == "StridedSlice" and idx > 0:
+                continue
             d = entry[0]
             tn = d["tensor_name"]
             if tn not in env:
@@ -303,6 +307,21 @@ def evaluate(desc, inputs):
                 else:
                     f = np.logical_and if name == "ReduceAll" else np.logical_or
                     res = f.reduce(x != 0, axis=tuple(axes), keepdims=keep)
+            elif name in VIEW_OPS:
+                x = ins[0]
+                vp = view_params(od, list(x.shape))
+                if name == "Transpose":
+                    res = np.transpose(x, vp["perm"])
+                elif name == "Tile":
+                    res = np.tile(x, vp["multiples"])
+                elif name in ("Slice", "StridedSlice"):
+                    res = x[tuple(slice(b, b + n * st, st) for b, n, st in zip(vp["begin"], vp["size"], vp["strides"]))]
+                elif name == "Pad":
+                    fill = np.asarray(vp["value"]).astype(x.dtype)
+                    res = np.pad(x, list(zip(vp["low"], vp["high"])), mode="constant", constant_values=fill)
+                else:
+                    res = np.concatenate([x, ins[1]], axis=vp["axis"])
+                res = np.ascontiguousarray(res)
             elif name == "MatMul":
                 if attrs.get("transpose_a", False):
                     raise ValueError("TransposeA is not supported")

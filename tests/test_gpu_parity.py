@@ -105,6 +105,11 @@ def test_full_size_bias_gradient_column_sums():
     check_stream_reduction(os.path.join(FIXTURES, "n1_biasgrad_bf16_16384x4096.info"), seed=harness.BASE_SEED + 11)
 
 
+def test_full_size_batched_transpose_bias_add():
+    """[32,2048,1024] -> [32,1024,2048] bfloat16 transpose fused with a bias add (indexed family), every element."""
+    check_fixture("n3_transpose_bias_add_bf16_32x2048x1024.info", seed=harness.BASE_SEED + 12, openmp=True)
+
+
 @pytest.mark.parametrize("name", FULL)
 def test_full_size_config_matches_oracle(name):
     # full BASELINE sizes; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)

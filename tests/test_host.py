@@ -226,6 +226,47 @@ def test_streaming_reduction_family_and_schedule():
     assert k.family == "row_reduce" and k.workspace_bytes == 0
 
 
+def test_data_movement_ops_translate_and_go_to_the_indexed_family():
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_view_chain_f32.info"))
+    assert (k.operator_type, k.family) == ("Transpose", "indexed")
+    text = driver.translate(open(os.path.join(FIXTURES, "small_view_chain_f32.info"), encoding="utf-8").read())
+    for needle in ("mindspore.pad", "mindspore.tile", "mindspore.strided_slice", "mindspore.transpose", "mindspore.slice",
+                   "mindspore.concat", "perm = [1, 0]", "low = [3, 1], value = 2"):
+        assert needle in text, needle
+    # a Tile alone is a Broadcast-class kernel, a Slice alone is unclassified (Default), as in the reference
+    b = op_desc.DescBuilder("Fused_Tile_only")
+    assert driver.HipKernel(b.dumps([op_desc.tile(b, b.input([3, 4], "float32"), [2, 2])]), out_dir=None).operator_type == "Broadcast"
+    b = op_desc.DescBuilder("Fused_Slice_only")
+    assert driver.HipKernel(b.dumps([op_desc.slice_(b, b.input([8, 8], "float32"), [1, 2], [3, -1])]), out_dir=None).operator_type == "Default"
+
+    def broken(mutate):
+        b = op_desc.DescBuilder("Fused_broken")
+        x = b.input([4, 6], "float32")
+        d = b.build([op_desc.transpose(b, x, [1, 0])])
+        mutate(d)
+        return json.dumps(d)
+    with pytest.raises(driver.AkgHipError) as e:   # not a permutation
+        driver.HipKernel(broken(lambda d: d["op_desc"][0]["attr"][0].update(value=[1, 1])), out_dir=None)
+    assert e.value.code == -3 and "permutation" in str(e.value)
+    with pytest.raises(driver.AkgHipError) as e:   # declared shape does not follow from the attributes
+        driver.HipKernel(broken(lambda d: d["op_desc"][0]["output_desc"][0].update(shape=[4, 6])), out_dir=None)
+    assert e.value.code == -3 and "declared result shape" in str(e.value)
+    # a strided slice with a mask set is refused rather than silently read without it
+    b = op_desc.DescBuilder("Fused_masked_slice")
+    x = b.input([8, 8], "float32")
+    d = b.build([op_desc.strided_slice(b, x, [0, 0], [4, 8], [1, 1])])
+    d["op_desc"][0]["attr"].append({"data_type": "int", "name": "shrinkAxisMask", "value": 1})
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(json.dumps(d), out_dir=None)
+    assert e.value.code == -3
+    # a reduction next to a transpose has no single kernel yet: error -4, never a wrong result
+    b = op_desc.DescBuilder("Fused_Transpose_ReduceSum")
+    x = b.input([4, 6], "float32")
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(b.dumps([b.reduce("ReduceSum", op_desc.transpose(b, x, [1, 0]), [1], False)]), out_dir=None)
+    assert e.value.code == -4
+
+
 def _meta_schedule(kernel):
     with open(os.path.join(driver.DEFAULT_META_DIR, kernel.kernel_name[:-len("_kernel")] + ".json"), encoding="utf-8") as f:
         return json.load(f)["schedule"]
