@@ -11,8 +11,13 @@
  * index the ops in between map it to, down to scalar loads of the kernel inputs. Nothing intermediate touches
  * memory and a value needed twice at the same index is computed once. Outputs are stored as V-element chunks.
  *
- * Reads of a transposed operand are strided across a wavefront (each lane walks its own row); this family
- * favours generality, the register-tiled kernels of the other families do not apply to these index maps.
+ * Transposed kernel inputs. Pulled element by element, the reads of a transposed operand are strided across a
+ * wavefront (measured 11 % of the HBM peak on a [32,2048,1024] bfloat16 transpose). When a kernel input X goes
+ * through a Transpose that moves its innermost axis, and the result has the shape of the outputs, the kernel is
+ * tiled instead: a workgroup owns a 64 x 64 patch of the plane spanned by the outputs' innermost axis and the axis
+ * X's innermost one lands on, copies X's side of the patch to LDS with 16-byte loads along X's innermost axis, and
+ * the on-demand read of the transposed value becomes an LDS read (row pitch 64 + 2 elements, so a wavefront's
+ * column reads spread over the banks). Everything else is pulled as before.
  */
 #include <map>
 #include <sstream>
@@ -47,6 +52,7 @@ class IndexedEmitter {
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
     note << "indexed vec=" << vec_ << " block=" << kBlock << " grid=" << grid_ << " rank=" << space_.size();
+    if (!staged_.empty()) note << " lds_tiles=" << staged_.size() << " tile=" << kTile << "x" << kTile << " axis=" << tDim_;
     k.scheduleNote = note.str();
     return k;
   }
@@ -61,6 +67,17 @@ class IndexedEmitter {
   std::vector<int64_t> space_;  // iteration space: the shape of the outputs
   int vec_ = 1;
   int64_t grid_ = 1;
+  // tiled mode (LDS-staged transposed inputs)
+  static constexpr int kTile = 64;
+  struct Staged {
+    int transposed;  // tensor id of the Transpose result
+    int input;       // tensor id of the kernel input it reads
+    int xRowDim;     // dimension of the input that follows the outputs' innermost axis
+    int vecX;        // elements per staging load
+  };
+  std::vector<Staged> staged_;
+  int tDim_ = -1;               // output dimension the staged inputs' innermost axis lands on
+  Index canonical_;             // index of the current output element, by dimension
   std::vector<bool> relaxed_;
   int nextTemp_ = 0;
   int indent_ = 2;
@@ -83,6 +100,13 @@ class IndexedEmitter {
                             "Concat) in one kernel yet");
       }
       if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+      if (isViewKind(op.kind)) {
+        for (int in : op.inputs) {
+          if (g_.tensor(in).dtype != g_.tensor(op.outputs[0]).dtype) {
+            throw LoweringError("op " + op.name + ": operand and result element types differ");
+          }
+        }
+      }
     }
     space_ = g_.tensor(g_.outputs[0]).shape;
     if (space_.empty()) space_.push_back(1);
@@ -106,7 +130,44 @@ class IndexedEmitter {
     vec_ = v;
     const int64_t chunks = numel / vec_;
     grid_ = std::max<int64_t>(1, (chunks + kBlock - 1) / kBlock);
+    pickStaging();
+    if (!staged_.empty()) {
+      grid_ = 1;
+      for (size_t d = 0; d < space_.size(); ++d) {
+        const bool tiledDim = static_cast<int>(d) == tDim_ || d + 1 == space_.size();
+        grid_ *= tiledDim ? (space_[d] + kTile - 1) / kTile : space_[d];
+      }
+    }
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
+  }
+
+  // Transposes of kernel inputs that move the innermost axis and produce a tensor of the outputs' shape. All staged
+  // inputs must agree on the output axis their innermost axis lands on (one tiling plane per kernel).
+  void pickStaging() {
+    if (opt_.gemmVariant == 1) return;  // AKG_HIP_GEMM_VARIANT=1: pull everything (for comparisons)
+    const size_t rank = space_.size();
+    if (rank < 2 || space_.back() < 16) return;
+    for (const OpNode &op : g_.ops) {
+      if (op.kind != OpKind::Transpose || staged_.size() >= 3) continue;
+      const TensorValue &x = g_.tensor(op.inputs[0]);
+      const TensorValue &y = g_.tensor(op.outputs[0]);
+      if (x.inputIndex < 0 || y.shape != space_ || x.shape.size() != rank) continue;
+      if (op.perm[rank - 1] == static_cast<int64_t>(rank) - 1) continue;  // innermost axis stays: reads are contiguous
+      int t = -1;
+      for (size_t d = 0; d < rank; ++d) {
+        if (op.perm[d] == static_cast<int64_t>(rank) - 1) t = static_cast<int>(d);
+      }
+      if (t < 0 || (tDim_ >= 0 && t != tDim_) || space_[static_cast<size_t>(t)] < 16) continue;
+      tDim_ = t;
+      Staged st;
+      st.transposed = op.outputs[0];
+      st.input = op.inputs[0];
+      st.xRowDim = static_cast<int>(op.perm[rank - 1]);
+      int vx = static_cast<int>(16 / dtypeSize(x.dtype));
+      while (vx > 1 && (x.shape.back() % vx) != 0) vx >>= 1;
+      st.vecX = vx;
+      staged_.push_back(st);
+    }
   }
 
   // ---- index helpers ------------------------------------------------------------------------------------
@@ -187,6 +248,14 @@ class IndexedEmitter {
       if (t.inputIndex < 0) throw LoweringError("operand " + t.name + " is undefined");
       stmt("const " + ct + " " + var + " = " + tagOf(id) + "::load(in" + std::to_string(t.inputIndex) + "[" +
            linearize(idx, t.shape) + "]);");
+      scopes_.back()[key] = var;
+      return var;
+    }
+    for (size_t k = 0; k < staged_.size(); ++k) {
+      if (staged_[k].transposed != id || idx != canonical_) continue;
+      // the patch of the transposed input is in LDS: row = position along the outputs' innermost axis
+      stmt("const " + ct + " " + var + " = " + tagOf(id) + "::load(akg_tile" + std::to_string(k) +
+           "[ci * V + e][tt]);  // Transpose -> " + t.name + " (staged)");
       scopes_.back()[key] = var;
       return var;
     }
@@ -295,6 +364,94 @@ class IndexedEmitter {
     return var;
   }
 
+  void emitTiledBody() {
+    const size_t rank = space_.size();
+    const size_t td = static_cast<size_t>(tDim_);
+    const int64_t extentI = space_.back(), extentT = space_[td];
+    const int64_t tilesI = (extentI + kTile - 1) / kTile, tilesT = (extentT + kTile - 1) / kTile;
+    src_ << "  constexpr int V = " << vec_ << ";\n";
+    src_ << "  constexpr int TILE = " << kTile << ";\n";
+    for (size_t k = 0; k < staged_.size(); ++k) {
+      src_ << "  __shared__ " << tagOf(staged_[k].input) << "::storage akg_tile" << k << "[TILE][TILE + "
+           << std::max<size_t>(1, 4 / dtypeSize(g_.tensor(staged_[k].input).dtype)) << "];\n";
+    }
+    src_ << "  const int tid = static_cast<int>(threadIdx.x);\n";
+    // workgroup -> (other dims..., tile along t, tile along the innermost axis); the innermost tile index is fastest
+    src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
+    src_ << "  const int i0 = (akg_w % " << tilesI << ") * TILE;\n  akg_w /= " << tilesI << ";\n";
+    src_ << "  const int t0 = (akg_w % " << tilesT << ") * TILE;\n  akg_w /= " << tilesT << ";\n";
+    canonical_.assign(rank, "0");
+    for (size_t d = rank - 1; d-- > 0;) {
+      if (d == td) continue;
+      if (space_[d] == 1) continue;
+      src_ << "  const int g" << d << " = akg_w % " << space_[d] << ";\n  akg_w /= " << space_[d] << ";\n";
+      canonical_[d] = "g" + std::to_string(d);
+    }
+    canonical_[td] = "gt";
+    canonical_[rank - 1] = "inner";
+    indent_ = 1;
+    scopes_.clear();
+    scopes_.emplace_back();
+    // ---- stage: rows follow the outputs' innermost axis, columns the input's innermost axis (output axis t)
+    for (size_t k = 0; k < staged_.size(); ++k) {
+      const Staged &st = staged_[k];
+      const TensorValue &x = g_.tensor(st.input);
+      const OpNode &op = g_.ops[static_cast<size_t>(g_.tensor(st.transposed).producer)];
+      const int chunksPerRow = kTile / st.vecX;
+      stmt("for (int c = tid; c < TILE * " + std::to_string(chunksPerRow) + "; c += " + std::to_string(kBlock) + ") {");
+      ++indent_;
+      stmt("const int r = c / " + std::to_string(chunksPerRow) + ", q = (c % " + std::to_string(chunksPerRow) + ") * " +
+           std::to_string(st.vecX) + ";");
+      stmt("if (i0 + r < " + std::to_string(extentI) + " && t0 + q < " + std::to_string(extentT) + ") {");
+      ++indent_;
+      // input index: input dim perm[d] takes output index d
+      Index xi(rank, "0");
+      for (size_t d = 0; d < rank; ++d) {
+        std::string v = canonical_[d];
+        if (d == td) v = "(t0 + q)";
+        if (d == rank - 1) v = "(i0 + r)";
+        xi[static_cast<size_t>(op.perm[d])] = v;
+      }
+      stmt("const " + tagOf(st.input) + "::storage *src = in" + std::to_string(x.inputIndex) + " + " +
+           linearize(xi, x.shape) + ";");
+      const size_t bytes = static_cast<size_t>(st.vecX) * dtypeSize(x.dtype);
+      stmt("akg::Raw<" + std::to_string(bytes) + ">::type raw = __builtin_nontemporal_load(reinterpret_cast<const akg::Raw<" +
+           std::to_string(bytes) + ">::type *>(src));");
+      stmt("__builtin_memcpy(&akg_tile" + std::to_string(k) + "[r][q], &raw, " + std::to_string(bytes) + ");");
+      --indent_;
+      stmt("}");
+      --indent_;
+      stmt("}");
+    }
+    stmt("__syncthreads();");
+    // ---- compute: a thread takes V-element chunks of the 64 x 64 output patch
+    const int chunksPerRow = kTile / vec_;
+    stmt("for (int c = tid; c < TILE * " + std::to_string(chunksPerRow) + "; c += " + std::to_string(kBlock) + ") {");
+    ++indent_;
+    stmt("const int tt = c / " + std::to_string(chunksPerRow) + ", ci = c % " + std::to_string(chunksPerRow) + ";");
+    stmt("const int gt = t0 + tt;");
+    stmt("if (gt >= " + std::to_string(extentT) + " || i0 + ci * V >= " + std::to_string(extentI) + ") continue;");
+    for (size_t i = 0; i < g_.outputs.size(); ++i) stmt(ctOf(g_.outputs[i]) + " o" + std::to_string(i) + "[V];");
+    stmt("#pragma unroll");
+    stmt("for (int e = 0; e < V; ++e) {");
+    openScope();
+    stmt("const int inner = i0 + ci * V + e;");
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      const std::string v = valueAt(g_.outputs[i], canonical_);
+      stmt("o" + std::to_string(i) + "[e] = " + v + ";");
+    }
+    closeScope();
+    stmt("}");
+    Index first = canonical_;
+    first[rank - 1] = "(i0 + ci * V)";
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, true>(out" + std::to_string(i) + " + " +
+           linearize(first, space_) + ", o" + std::to_string(i) + ");");
+    }
+    --indent_;
+    stmt("}");
+  }
+
   void openScope() {
     scopes_.emplace_back();
     ++indent_;
@@ -319,6 +476,11 @@ class IndexedEmitter {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
     src_ << ") {\n";
+    if (!staged_.empty()) {
+      emitTiledBody();
+      src_ << "}\n";
+      return;
+    }
     int64_t numel = 1;
     for (int64_t d : space_) numel *= d;
     src_ << "  constexpr int V = " << vec_ << ";\n";

@@ -51,6 +51,9 @@ FIXTURES = {
     "small_transpose_0213_neg_f16_2x5x6x8": lambda n: op_desc.transpose_0213_neg([2, 5, 6, 8], "float16", n),
     "small_slice_concat_pad_add_i32": lambda n: op_desc.slice_concat_int(n),
     "small_transpose_reshape_add_f32_4x6x10": lambda n: op_desc.transpose_reshape_add(n),
+    "small_transpose_bias_add_f32_2x100x200": lambda n: op_desc.transpose_bias_add(2, 100, 200, "float32", n),
+    "small_transpose_sum_f32_2x70x3x80_perm0321": lambda n: op_desc.transpose_sum([2, 70, 3, 80], [0, 3, 2, 1], "float32", n),
+    "small_transpose_sum_f16_130x66_perm10": lambda n: op_desc.transpose_sum([130, 66], [1, 0], "float16", n),
     "n3_transpose_bias_add_bf16_32x2048x1024": lambda n: op_desc.transpose_bias_add(32, 2048, 1024, "bfloat16", n),
     # float MatMul + bias + activation on the bfloat16 / float16 MFMA path
     "small_gemm_bf16_bias_gelu_256x512x256": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "float32", n),

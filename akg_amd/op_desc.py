@@ -393,3 +393,12 @@ def transpose_reshape_add(name=None):
     y = b.input([24, 10], "float32")
     t = b.reshape(transpose(b, x, [1, 0, 2]), [24, 10])
     return b.dumps([b.add(t, y)])
+
+
+def transpose_sum(shape, perm, dtype="float32", name=None):
+    """out = transpose(x, perm) + transpose(y, perm) * 2: two kernel inputs read through the same permutation."""
+    b = DescBuilder(name or "Fused_Transpose_Transpose_Mul_Add_%s_%s_perm%s" % (
+        _SHORT[dtype], "x".join(str(d) for d in shape), "".join(str(p) for p in perm)))
+    x = b.input(list(shape), dtype)
+    y = b.input(list(shape), dtype)
+    return b.dumps([b.add(transpose(b, x, perm), b.mul(transpose(b, y, perm), b.const(2.0, dtype)))])
