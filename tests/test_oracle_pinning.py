@@ -287,6 +287,76 @@ def test_gemm_dequant_bias_gelu_matches_torch_float64():
 
 
 # ---------------------------------------------------------------------------------------------------------
+# data-movement ops, outer-axis reductions, float MatMul
+# ---------------------------------------------------------------------------------------------------------
+def test_data_movement_chain_matches_plain_numpy(tmp_path):
+    """pad -> tile -> strided slice (negative end) -> transpose, slice -> transpose, concat: written out with numpy's
+    own pad / tile / slicing / concatenate. A padding pair applied to the wrong dimension, a perm read as its inverse,
+    an `end` not counted from the back or a swapped concat order changes the result."""
+    text = op_desc.view_chain("pin_view_chain")
+    x = np.arange(35, dtype=np.float32).reshape(5, 7) + 1
+    y = -(np.arange(270, dtype=np.float32).reshape(9, 30) + 1)
+    _, c_out, n_out = build_and_run(text, [x, y], tmp_path)
+    p = np.pad(x, ((3, 0), (1, 2)), constant_values=2)      # padding [1,2,3,0]: (1,2) on the last axis, (3,0) before it
+    t = np.tile(p, (2, 3))
+    s = t[1:15:2, :]                                        # begin 1, end -1 -> 15, stride 2
+    expect = np.concatenate([s.T, y[2:6, :].T], axis=1) * np.float32(0.5)
+    assert expect.shape == (30, 11)
+    assert np.array_equal(c_out[0], expect) and np.array_equal(n_out[0], expect)
+
+
+def test_transpose_perm_is_result_dim_from_operand_dim(tmp_path):
+    """perm [2,0,1]: result dim d has the extent (and the index) of operand dim perm[d] (tosa.transpose), not the inverse."""
+    b = op_desc.DescBuilder("pin_transpose_201")
+    x = b.input([2, 3, 4], "int32")
+    text = b.dumps([op_desc.transpose(b, x, [2, 0, 1])])
+    data = np.arange(24, dtype=np.int32).reshape(2, 3, 4)
+    _, c_out, n_out = build_and_run(text, [data], tmp_path)
+    assert c_out[0].shape == (4, 2, 3)
+    for i in range(4):
+        for j in range(2):
+            for k in range(3):
+                assert c_out[0][i, j, k] == data[j, k, i] == n_out[0][i, j, k]
+
+
+def test_outer_axis_reduction_visits_the_reduced_index_in_order(tmp_path):
+    """ReduceSum over axis 0 in float16: per column, the running sum is rounded after every row (same rule as the row
+    reduction, now with the reduced axis outermost). 4096 ones per column stall at 2048; a float32 accumulator or a
+    pairwise order would give 4096."""
+    b = op_desc.DescBuilder("pin_colsum_f16")
+    x = b.input([4096, 3], "float16")
+    text = b.dumps([b.reduce("ReduceSum", x, [0], False)])
+    _, c_out, n_out = build_and_run(text, [np.ones((4096, 3), dtype=np.float16)], tmp_path)
+    assert np.all(c_out[0] == 2048) and np.all(n_out[0] == 2048)
+    # float32, all axes: the serial order is the row-major order of the operand
+    b = op_desc.DescBuilder("pin_allsum_f32")
+    x = b.input([3, 5], "float32")
+    text = b.dumps([b.reduce("ReduceSum", x, [0, 1], False)])
+    data = np.array([1e8, 1.0, -1e8, 1.0, 1.0] * 3, dtype=np.float32).reshape(3, 5)
+    _, c_out, n_out = build_and_run(text, [data], tmp_path)
+    acc = np.float32(0)
+    for v in data.reshape(-1):
+        acc = np.float32(acc + v)
+    assert c_out[0][0] == acc == n_out[0][0] and acc != np.float32(data.astype(np.float64).sum())
+
+
+def test_bf16_matmul_bias_gelu_matches_torch_float64():
+    import torch
+    name = "small_gemm_bf16_bias_gelu_256x512x256"
+    desc, inputs, c_out, n_out = run_fixture_both(name, 23)
+    a, w, bias = [torch.from_numpy(harness.bf16_bits_to_f32(x).astype(np.float64)) for x in inputs]
+    ref = torch.nn.functional.gelu(a @ w + bias, approximate="tanh").numpy()
+    for out in (c_out[0], n_out[0]):
+        got = harness.bf16_bits_to_f32(out).astype(np.float64)
+        assert np.allclose(got, ref, rtol=1e-2, atol=1e-3)
+    # transposed B: the same numbers read as [N, K]
+    desc, inputs, c_out, _ = run_fixture_both(name + "_tb", 23)
+    a, w, bias = [torch.from_numpy(harness.bf16_bits_to_f32(x).astype(np.float64)) for x in inputs]
+    ref = torch.nn.functional.gelu(a @ w.T + bias, approximate="tanh").numpy()
+    assert np.allclose(harness.bf16_bits_to_f32(c_out[0]).astype(np.float64), ref, rtol=1e-2, atol=1e-3)
+
+
+# ---------------------------------------------------------------------------------------------------------
 # the two restatements against each other on every small fixture
 # ---------------------------------------------------------------------------------------------------------
 SMALL = sorted(f[:-5] for f in os.listdir(FIXTURES) if f.startswith("small_") and f.endswith(".info"))
