@@ -16,6 +16,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <fstream>
+#include <map>
 #include <memory>
 #include <mutex>
 #include <sstream>
@@ -48,6 +49,17 @@ struct akg_hip_kernel {
     void *workspace = nullptr;  // lowered.workspaceBytes of zero-filled device memory, or NULL
   };
   std::vector<Loaded> loaded;
+};
+
+// A dynamic-shape description and the kernels specialised from it so far, keyed by the bound input shapes.
+struct akg_hip_dynamic {
+  std::string jsonText;
+  std::string outDir;
+  bool hasOutDir = false;
+  int numInputs = 0;
+  std::vector<int> inputRanks;
+  std::mutex mu;
+  std::map<std::string, akg_hip_kernel_t *> specializations;
 };
 
 namespace {
@@ -222,12 +234,25 @@ std::string shapeArgText(const akg::LoweredKernel &k) {
   return os.str();
 }
 
-int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel) {
+int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
+              const akg::ShapeBinding *binding = nullptr) {
   if (outKernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "out_kernel is NULL");
   *outKernel = nullptr;
   std::unique_ptr<akg_hip_kernel> k(new akg_hip_kernel());
   try {
-    k->graph = akg::translateJsonToOpGraph(jsonText);
+    k->graph = akg::translateJsonToOpGraph(jsonText, binding);
+    if (binding != nullptr) {
+      // one artifact set per shape: the specialisation is named after a digest of the bound input shapes
+      akg::Sha256 h;
+      for (const auto &shape : binding->inputShapes) {
+        for (int64_t d : shape) {
+          const std::string t = std::to_string(d) + ",";
+          h.update(t.data(), t.size());
+        }
+        h.update(";", 1);
+      }
+      k->graph.name += "_s" + h.hexDigest().substr(0, 12);
+    }
   } catch (const akg::json::ParseError &e) {
     return fail(AKG_HIP_ERR_JSON, e.what());
   } catch (const akg::TranslateError &e) {
@@ -576,6 +601,87 @@ int akg_hip_translate(const char *json_text, size_t json_len, char **out_text) {
 }
 
 void akg_hip_free_string(char *text) { std::free(text); }
+
+int akg_hip_dynamic_create(const char *json_text, size_t json_len, const char *out_dir, akg_hip_dynamic_t **out) {
+  if (json_text == nullptr || out == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  *out = nullptr;
+  try {
+    std::unique_ptr<akg_hip_dynamic> d(new akg_hip_dynamic());
+    d->jsonText.assign(json_text, json_len);
+    if (out_dir != nullptr) {
+      d->outDir = out_dir;
+      d->hasOutDir = true;
+    }
+    const akg::json::Value root = akg::json::Value::parse(d->jsonText);
+    if (!root.isObject() || !root.contains("input_desc") || !root.contains("op_desc") || !root.contains("output_desc")) {
+      return fail(AKG_HIP_ERR_TRANSLATE, "not an op description");
+    }
+    d->numInputs = static_cast<int>(root.at("input_desc").size());
+    for (size_t i = 0; i < root.at("input_desc").size(); ++i) {
+      const akg::json::Value &desc = root.at("input_desc")[i][0];
+      d->inputRanks.push_back(desc.contains("shape") ? static_cast<int>(desc.at("shape").size()) : 1);
+    }
+    *out = d.release();
+    g_lastError.clear();
+    return AKG_HIP_OK;
+  } catch (const akg::json::ParseError &e) {
+    return fail(AKG_HIP_ERR_JSON, e.what());
+  } catch (const std::exception &e) {
+    return fail(AKG_HIP_ERR_TRANSLATE, e.what());
+  }
+}
+
+int akg_hip_dynamic_num_inputs(const akg_hip_dynamic_t *dyn, int *n_inputs) {
+  if (dyn == nullptr || n_inputs == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  *n_inputs = dyn->numInputs;
+  return AKG_HIP_OK;
+}
+
+int akg_hip_dynamic_specialize(akg_hip_dynamic_t *dyn, const int64_t *const *input_shapes, const int32_t *input_ranks,
+                               int n_inputs, akg_hip_kernel_t **out_kernel) {
+  if (dyn == nullptr || input_shapes == nullptr || input_ranks == nullptr || out_kernel == nullptr) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  }
+  *out_kernel = nullptr;
+  if (n_inputs != dyn->numInputs) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "the description has " + std::to_string(dyn->numInputs) + " inputs, " +
+                                                std::to_string(n_inputs) + " shapes given");
+  }
+  akg::ShapeBinding binding;
+  std::string key;
+  for (int i = 0; i < n_inputs; ++i) {
+    if (input_ranks[i] < 0 || input_ranks[i] > AKG_HIP_MAX_RANK || input_shapes[i] == nullptr) {
+      return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "bad rank or NULL shape for input " + std::to_string(i));
+    }
+    std::vector<int64_t> shape(input_shapes[i], input_shapes[i] + input_ranks[i]);
+    for (int64_t d : shape) key += std::to_string(d) + ",";
+    key += ";";
+    binding.inputShapes.push_back(std::move(shape));
+  }
+  std::lock_guard<std::mutex> lock(dyn->mu);
+  auto it = dyn->specializations.find(key);
+  if (it != dyn->specializations.end()) {
+    *out_kernel = it->second;
+    return AKG_HIP_OK;
+  }
+  akg_hip_kernel_t *k = nullptr;
+  int rc;
+  try {
+    rc = doCompile(dyn->jsonText, dyn->hasOutDir ? dyn->outDir.c_str() : nullptr, &k, &binding);
+  } catch (const std::exception &e) {
+    return fail(AKG_HIP_ERR_INTERNAL, std::string("internal error: ") + e.what());
+  }
+  if (rc != AKG_HIP_OK) return rc;
+  dyn->specializations[key] = k;
+  *out_kernel = k;
+  return AKG_HIP_OK;
+}
+
+void akg_hip_dynamic_destroy(akg_hip_dynamic_t *dyn) {
+  if (dyn == nullptr) return;
+  for (auto &kv : dyn->specializations) akg_hip_kernel_destroy(kv.second);
+  delete dyn;
+}
 
 const char *akg_hip_version(void) { return AKG_HIP_VERSION_STRING; }
 

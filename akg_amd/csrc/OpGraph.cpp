@@ -157,7 +157,7 @@ void checkAttrTypes(const json::Value &attrs, const std::string &opName) {
 
 class GraphBuilder {
  public:
-  explicit GraphBuilder(const json::Value &root) : root_(root) {}
+  GraphBuilder(const json::Value &root, const ShapeBinding *binding) : root_(root), binding_(binding) {}
 
   OpGraph build() {
     if (!root_.isObject()) throw TranslateError("op description must be a JSON object");
@@ -179,6 +179,7 @@ class GraphBuilder {
 
  private:
   const json::Value &root_;
+  const ShapeBinding *binding_;
   OpGraph graph_;
   std::map<std::string, int> operandList_;  // tensor_name -> tensor id (operandList, :110)
 
@@ -203,7 +204,23 @@ class GraphBuilder {
       const json::Value &desc = inputs[i][0];
       std::string tensorName = desc.at(kTensorName).asString();
       DType dtype = parseDType(desc.at(kDataType).asString());
-      int id = addTensor(tensorName, dtype, readShape(desc));
+      std::vector<int64_t> shape = readShape(desc);
+      if (binding_ != nullptr) {
+        if (binding_->inputShapes.size() != inputs.size()) {
+          throw TranslateError("shape binding: " + std::to_string(binding_->inputShapes.size()) + " shapes given for " +
+                               std::to_string(inputs.size()) + " kernel inputs");
+        }
+        const std::vector<int64_t> &bound = binding_->inputShapes[i];
+        if (bound.size() != shape.size()) throw TranslateError("shape binding: rank of input " + tensorName + " differs");
+        for (size_t d = 0; d < shape.size(); ++d) {
+          if (bound[d] < 0 || (shape[d] >= 0 && shape[d] != bound[d])) {
+            throw TranslateError("shape binding: dimension " + std::to_string(d) + " of input " + tensorName +
+                                 " contradicts the description");
+          }
+        }
+        shape = bound;
+      }
+      int id = addTensor(tensorName, dtype, shape);
       graph_.tensors[static_cast<size_t>(id)].inputIndex = static_cast<int>(i);
       graph_.inputs.push_back(id);
       operandList_[tensorName] = id;
@@ -315,9 +332,12 @@ class GraphBuilder {
         if (const json::Value *b = findAttr(attrs, kTransposeB)) node.transposeB = b->asBool();
       }
 
+      std::vector<int64_t> inferred;  // result shape derived from the operands (empty: take the declared one)
       if (node.kind == OpKind::Transpose || node.kind == OpKind::Tile || node.kind == OpKind::Slice ||
           node.kind == OpKind::StridedSlice || node.kind == OpKind::Pad || node.kind == OpKind::Concat) {
-        parseDataMovement(&node, attrs, inputDesc, readShape(outputDesc[0]));
+        inferred = parseDataMovement(&node, attrs, inputDesc, readShape(outputDesc[0]));
+      } else if (binding_ != nullptr) {
+        inferred = inferResultShape(node, attrs, inputDesc, readShape(outputDesc[0]));
       }
 
       int opIndex = static_cast<int>(graph_.ops.size());
@@ -325,7 +345,11 @@ class GraphBuilder {
         const json::Value &d = outputDesc[j];
         std::string tensorName = d.at(kTensorName).asString();
         DType dtype = parseDType(d.at(kDataType).asString());
-        int id = addTensor(tensorName, dtype, readShape(d));
+        std::vector<int64_t> shape = readShape(d);
+        bool dynamic = false;
+        for (int64_t e : shape) dynamic = dynamic || e < 0;
+        if (dynamic && binding_ != nullptr && j == 0 && !inferred.empty()) shape = inferred;
+        int id = addTensor(tensorName, dtype, shape);
         graph_.tensors[static_cast<size_t>(id)].producer = opIndex;
         node.outputs.push_back(id);
         operandList_[tensorName] = id;
@@ -344,8 +368,91 @@ class GraphBuilder {
   //   Pad          attr "padding" = (before, after) pairs listed from the LAST dimension backwards, "value",
   //                mode "constant" (MindSporeToTosa.cpp:305-376)
   //   Concat       two operands, attr "axis" (default 0) (convertConcatOp :1117-1124)
-  void parseDataMovement(OpNode *node, const json::Value &attrs, const json::Value &inputDesc,
-                         const std::vector<int64_t> &outShape) {
+  // Result shape of a non-data-movement op from its (already concrete) operands; used under a shape binding for
+  // results declared with -1 dimensions. Elementwise ops broadcast numpy-style; reductions drop or keep their axes;
+  // Reshape solves at most one unknown extent from the element count; MatMul is [M,K] x [K,N] (or [N,K]).
+  std::vector<int64_t> inferResultShape(const OpNode &node, const json::Value &attrs, const json::Value &inputDesc,
+                                        const std::vector<int64_t> &declared) {
+    (void)inputDesc;
+    bool dynamic = false;
+    for (int64_t e : declared) dynamic = dynamic || e < 0;
+    if (!dynamic) return {};
+    auto shapeOf = [&](size_t i) { return graph_.tensor(node.inputs[i]).shape; };
+    if (node.kind == OpKind::Unknown || node.kind == OpKind::Unsupported) {
+      throw TranslateError("op " + node.name + ": cannot derive a dynamic result shape for an op with no lowering");
+    }
+    if (isReduceKind(node.kind)) {
+      const std::vector<int64_t> in = shapeOf(0);
+      std::vector<int64_t> out;
+      for (size_t d = 0; d < in.size(); ++d) {
+        const bool reduced = std::find(node.axes.begin(), node.axes.end(), static_cast<int64_t>(d)) != node.axes.end();
+        if (!reduced) {
+          out.push_back(in[d]);
+        } else if (node.keepDims) {
+          out.push_back(1);
+        }
+      }
+      if (out.empty()) out.push_back(1);
+      return out;
+    }
+    if (node.kind == OpKind::MatMul) {
+      const std::vector<int64_t> a = shapeOf(0), b = shapeOf(1);
+      if (a.size() != 2 || b.size() != 2) throw TranslateError("op " + node.name + ": only rank-2 MatMul is supported");
+      return {a[0], node.transposeB ? b[0] : b[1]};
+    }
+    if (node.kind == OpKind::Reshape || node.kind == OpKind::BroadcastTo) {
+      std::vector<int64_t> out = declared;
+      if (node.kind == OpKind::BroadcastTo) {
+        // unknown extents come from the operand, right-aligned
+        const std::vector<int64_t> in = shapeOf(0);
+        for (size_t d = 0; d < out.size(); ++d) {
+          if (out[d] >= 0) continue;
+          const size_t fromEnd = out.size() - 1 - d;
+          if (fromEnd >= in.size()) throw TranslateError("op " + node.name + ": cannot derive the broadcast shape");
+          out[d] = in[in.size() - 1 - fromEnd];
+        }
+        return out;
+      }
+      int64_t known = 1, total = graph_.tensor(node.inputs[0]).numel();
+      int unknown = 0;
+      for (int64_t e : out) {
+        if (e < 0) {
+          ++unknown;
+        } else {
+          known *= e;
+        }
+      }
+      if (unknown != 1 || known == 0 || total % known != 0) {
+        throw TranslateError("op " + node.name + ": a dynamic Reshape may leave exactly one extent open");
+      }
+      for (int64_t &e : out) {
+        if (e < 0) e = total / known;
+      }
+      return out;
+    }
+    (void)attrs;
+    // elementwise (incl. Cast, Select, AddN): numpy broadcasting over every operand
+    std::vector<int64_t> out;
+    for (size_t i = 0; i < node.inputs.size(); ++i) {
+      const std::vector<int64_t> in = shapeOf(i);
+      if (in.size() > out.size()) out.insert(out.begin(), in.size() - out.size(), 1);
+      for (size_t d = 0; d < in.size(); ++d) {
+        int64_t &o = out[out.size() - in.size() + d];
+        if (o == 1) {
+          o = in[d];
+        } else if (in[d] != 1 && in[d] != o) {
+          throw TranslateError("op " + node.name + ": operands do not broadcast under the shape binding");
+        }
+      }
+    }
+    if (out.size() != declared.size()) {
+      if (out.size() < declared.size()) out.insert(out.begin(), declared.size() - out.size(), 1);
+    }
+    return out;
+  }
+
+  std::vector<int64_t> parseDataMovement(OpNode *node, const json::Value &attrs, const json::Value &inputDesc,
+                                         const std::vector<int64_t> &outShape) {
     const std::string &nm = node->name;
     if (node->inputs.empty()) throw TranslateError("op " + nm + ": missing operand");
     const std::vector<int64_t> inShape = graph_.tensor(node->inputs[0]).shape;
@@ -474,9 +581,12 @@ class GraphBuilder {
       default:
         break;
     }
-    if (expect != outShape) {
+    bool dynamic = false;
+    for (int64_t e : outShape) dynamic = dynamic || e < 0;
+    if (!dynamic && expect != outShape) {
       throw TranslateError("op " + nm + ": the declared result shape does not follow from the operand and attributes");
     }
+    return expect;
   }
 
   void parseOutputs() {
@@ -495,8 +605,14 @@ class GraphBuilder {
       }
       std::vector<int64_t> shape = readShape(desc);
       int64_t n = 1;
-      for (int64_t d : shape) n *= d;
-      if (n != t.numel()) {
+      bool dynamic = false;
+      for (int64_t d : shape) {
+        n *= d;
+        dynamic = dynamic || d < 0;
+      }
+      if (dynamic && binding_ != nullptr) {
+        if (shape.size() != t.shape.size()) throw TranslateError("output " + tensorName + ": rank differs from its producer");
+      } else if (n != t.numel()) {
         throw TranslateError("output " + tensorName + ": shape differs between output_desc and its producer");
       }
       if (t.outputIndex >= 0) throw TranslateError("output " + tensorName + " is listed twice");
@@ -678,9 +794,37 @@ const char *operatorTemplateName(OperatorTemplate t) {
   return "?";
 }
 
-OpGraph translateJsonToOpGraph(const std::string &jsonText) {
+bool descriptionIsDynamic(const std::string &jsonText) {
+  const json::Value root = json::Value::parse(jsonText);
+  auto dyn = [](const json::Value &desc) {
+    if (!desc.contains(kShape)) return false;
+    for (int64_t d : desc.at(kShape).asIntVector()) {
+      if (d < 0) return true;
+    }
+    return false;
+  };
+  if (!root.isObject()) return false;
+  const json::Value &inputs = root.at(kInputDesc);
+  for (size_t i = 0; i < inputs.size(); ++i) {
+    if (dyn(inputs[i][0])) return true;
+  }
+  const json::Value &ops = root.at(kOpDesc);
+  for (size_t i = 0; i < ops.size(); ++i) {
+    const json::Value &outs = ops[i].at(kOutputDesc);
+    for (size_t j = 0; j < outs.size(); ++j) {
+      if (dyn(outs[j])) return true;
+    }
+  }
+  const json::Value &outputs = root.at(kOutputDesc);
+  for (size_t i = 0; i < outputs.size(); ++i) {
+    if (dyn(outputs[i])) return true;
+  }
+  return false;
+}
+
+OpGraph translateJsonToOpGraph(const std::string &jsonText, const ShapeBinding *binding) {
   json::Value root = json::Value::parse(jsonText);
-  GraphBuilder builder(root);
+  GraphBuilder builder(root, binding);
   OpGraph g = builder.build();
   identifyOperator(&g);
   return g;

@@ -113,8 +113,19 @@ struct OpGraph {
   const TensorValue &tensor(int id) const { return tensors[static_cast<size_t>(id)]; }
 };
 
-// JSON text -> op graph. Throws json::ParseError / TranslateError.
-OpGraph translateJsonToOpGraph(const std::string &jsonText);
+// Concrete shapes for the kernel inputs of a dynamic-shape description (dimensions spelled -1), one per input in
+// `input_desc` order. With a binding the translator replaces the -1s of the inputs and derives the shape of every op
+// result from its operands (the job of the reference's shape-inference passes and of the runtime shape arguments of its
+// dynamic kernels, LLVMParameterPacking.cpp:91-194); the result is an ordinary static graph.
+struct ShapeBinding {
+  std::vector<std::vector<int64_t>> inputShapes;
+};
+
+// JSON text -> op graph. Throws json::ParseError / TranslateError. Without a binding a -1 dimension is an error.
+OpGraph translateJsonToOpGraph(const std::string &jsonText, const ShapeBinding *binding = nullptr);
+
+// True if the description has a -1 dimension on any kernel input, op result or kernel output.
+bool descriptionIsDynamic(const std::string &jsonText);
 
 // Fusion-class identification (OperatorIdentify.cpp:51-93) and reduce-direction marking
 // (akg-mlir/lib/Dialect/Linalg/Transforms/MatchAndMarkReductionOps.cpp:51-88). Fills the two fields above.

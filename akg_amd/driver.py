@@ -76,6 +76,12 @@ def load_library():
     lib.akg_hip_free_string.argtypes = [vp]
     lib.akg_hip_free_string.restype = None
     lib.akg_hip_version.restype = cp
+    lib.akg_hip_dynamic_create.argtypes = [cp, ctypes.c_size_t, cp, ctypes.POINTER(vp)]
+    lib.akg_hip_dynamic_num_inputs.argtypes = [vp, ctypes.POINTER(ci)]
+    lib.akg_hip_dynamic_specialize.argtypes = [vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)),
+                                               ctypes.POINTER(ctypes.c_int32), ci, ctypes.POINTER(vp)]
+    lib.akg_hip_dynamic_destroy.argtypes = [vp]
+    lib.akg_hip_dynamic_destroy.restype = None
     _lib = lib
     return lib
 
@@ -97,6 +103,41 @@ def translate(json_text):
         lib.akg_hip_free_string(out)
 
 
+class HipDynamicKernel:
+    """A dynamic-shape description (-1 dimensions), specialised per set of input shapes on demand."""
+
+    def __init__(self, json_text, out_dir=DEFAULT_META_DIR):
+        self._lib = load_library()
+        self._handle = ctypes.c_void_p()
+        raw = json_text.encode("utf-8") if isinstance(json_text, str) else json_text
+        od = out_dir.encode("utf-8") if out_dir else None
+        _check(self._lib.akg_hip_dynamic_create(raw, len(raw), od, ctypes.byref(self._handle)))
+        self._kernels = {}
+
+    def specialize(self, input_shapes):
+        """HipKernel for exactly these input shapes (list of lists, input_desc order); cached per shape set."""
+        key = tuple(tuple(int(d) for d in s) for s in input_shapes)
+        if key in self._kernels:
+            return self._kernels[key]
+        n = len(key)
+        arrays = [(ctypes.c_int64 * max(1, len(s)))(*s) for s in key]
+        ptrs = (ctypes.POINTER(ctypes.c_int64) * n)(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in arrays])
+        ranks = (ctypes.c_int32 * n)(*[len(s) for s in key])
+        out = ctypes.c_void_p()
+        _check(self._lib.akg_hip_dynamic_specialize(self._handle, ptrs, ranks, n, ctypes.byref(out)))
+        k = HipKernel(None, _borrowed=out)
+        k._keepalive = self
+        self._kernels[key] = k
+        return k
+
+    def __del__(self):
+        h = getattr(self, "_handle", None)
+        if h:
+            self._kernels = {}
+            self._lib.akg_hip_dynamic_destroy(h)
+            self._handle = None
+
+
 class TensorDesc:
     def __init__(self, raw):
         self.dtype = DTYPE_NAMES[raw.dtype]
@@ -112,11 +153,14 @@ class TensorDesc:
 class HipKernel:
     """A compiled fused kernel. Construct from JSON text or with `HipKernel.from_file`."""
 
-    def __init__(self, json_text, out_dir=DEFAULT_META_DIR, _path=None):
+    def __init__(self, json_text, out_dir=DEFAULT_META_DIR, _path=None, _borrowed=None):
         self._lib = load_library()
         self._handle = ctypes.c_void_p()
+        self._owned = _borrowed is None
         od = out_dir.encode("utf-8") if out_dir else None
-        if _path is not None:
+        if _borrowed is not None:
+            self._handle = _borrowed      # owned by a HipDynamicKernel
+        elif _path is not None:
             _check(self._lib.akg_hip_compile_file(_path.encode("utf-8"), od, ctypes.byref(self._handle)))
         else:
             raw = json_text.encode("utf-8") if isinstance(json_text, str) else json_text
@@ -146,9 +190,9 @@ class HipKernel:
 
     def __del__(self):
         h = getattr(self, "_handle", None)
-        if h:
+        if h and getattr(self, "_owned", True):
             self._lib.akg_hip_kernel_destroy(h)
-            self._handle = None
+        self._handle = None
 
     @property
     def inputs(self):

@@ -145,6 +145,24 @@ const char *akg_hip_last_error(void);
 int akg_hip_translate(const char *json_text, size_t json_len, char **out_text);
 void akg_hip_free_string(char *text);
 
+/**
+ * Dynamic shapes: a description whose tensors carry -1 dimensions (MindSpore's dynamic-shape graph kernels). The
+ * reference compiles such a description once (`akg-opt --gpu-dyn-opt`), passes sizes and strides as kernel arguments
+ * ([ptrs[], shape/stride[][]] packing, LLVMParameterPacking.cpp:91-194) and solves the launch shape per call in Python
+ * (dynamic_utils.py:269-526). Here every kernel is specialised to its shapes at compile time, so a dynamic description
+ * is kept as text and specialised on demand: akg_hip_dynamic_specialize binds the -1s to the given input shapes,
+ * derives every op's result shape, compiles (or finds in the artifact directory / in memory) the static kernel for
+ * exactly these shapes and returns its handle. The handle is owned by the dynamic object (do not destroy it); it is
+ * launched with akg_hip_launch like any other, and akg_hip_kernel_tensor reports the concrete output shapes.
+ */
+typedef struct akg_hip_dynamic akg_hip_dynamic_t;
+int akg_hip_dynamic_create(const char *json_text, size_t json_len, const char *out_dir, akg_hip_dynamic_t **out);
+int akg_hip_dynamic_num_inputs(const akg_hip_dynamic_t *dyn, int *n_inputs);
+/** input_shapes[i] points at input_ranks[i] extents of kernel input i (input_desc order). */
+int akg_hip_dynamic_specialize(akg_hip_dynamic_t *dyn, const int64_t *const *input_shapes, const int32_t *input_ranks,
+                               int n_inputs, akg_hip_kernel_t **out_kernel);
+void akg_hip_dynamic_destroy(akg_hip_dynamic_t *dyn);
+
 /** Library version string. */
 const char *akg_hip_version(void);
 

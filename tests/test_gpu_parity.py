@@ -146,6 +146,56 @@ def test_reference_repository_descriptions_match_oracle(name):
         assert ok, "%s output %s: %s" % (name, d.name, msg)
 
 
+def _bind_softmax_description(desc, shapes):
+    """The test's own reading of the dynamic description: numpy broadcasting for the elementwise ops, axis 3 kept as 1
+    for the two reductions. Written apart from the product's shape derivation on purpose."""
+    d = json_loads(__import__("json").dumps(desc))
+    env = {}
+    for entry, shape in zip(d["input_desc"], shapes):
+        entry[0]["shape"] = list(shape)
+        env[entry[0]["tensor_name"]] = list(shape)
+    for od in d["op_desc"]:
+        ins = []
+        for entry in od["input_desc"]:
+            if entry[0]["tensor_name"] in env:
+                entry[0]["shape"] = env[entry[0]["tensor_name"]]
+            ins.append(tuple(entry[0]["shape"]))
+        if od["name"].startswith("Reduce"):
+            out = list(ins[0])
+            out[3] = 1
+        else:
+            out = list(np.broadcast_shapes(*ins))
+        od["output_desc"][0]["shape"] = out
+        env[od["output_desc"][0]["tensor_name"]] = out
+    for o in d["output_desc"]:
+        o["shape"] = env[o["tensor_name"]]
+    return d
+
+
+@pytest.mark.parametrize("shapes", [[[32, 1, 48, 48], [32, 12, 48, 48]], [[1, 1, 40, 72], [32, 12, 40, 72]],
+                                    [[32, 1, 7, 1000], [32, 12, 7, 1000]]])
+def test_reference_dynamic_shape_softmax_specialised_per_shape(shapes):
+    """The reference's dynamic-shape system-test description (masked attention softmax, every extent but 32 x 12 open),
+    specialised to three shape sets through akg_hip_dynamic_specialize and checked against the oracle evaluated on the
+    description with the same shapes written in."""
+    from oracle import np_ref
+    path = os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")
+    desc = harness.load_desc(path)
+    dyn = driver.HipDynamicKernel(open(path, encoding="utf-8").read())
+    kernel = dyn.specialize(shapes)
+    bound = _bind_softmax_description(desc, shapes)
+    assert [t.shape for t in kernel.outputs] == [bound["output_desc"][0]["shape"]]
+    rng = np.random.default_rng(harness.BASE_SEED + 600)
+    mask = (rng.random(shapes[0]) < 0.8).astype(np.float32)          # 1 = keep, 0 = masked out by -10000
+    scores = (rng.standard_normal(shapes[1], dtype=np.float32) * 4).astype(np.float32)
+    got = run_on_gpu(kernel, [mask, scores])[0]
+    expect = np_ref.evaluate(bound, [mask, scores])[0]
+    ok, msg = harness.compare(got, expect, "float32")
+    print("  shapes %s: %s" % (shapes, msg), flush=True)
+    assert ok, msg
+    assert np.allclose(got.sum(axis=3), 1.0, atol=1e-5)
+
+
 def test_float32_tanh_accuracy_over_the_whole_range():
     """The float32 tanh of the device op library is an own implementation (series below 0.25, hardware exp2 and
     reciprocal above): its error against the float64 value is measured on 8M arguments, dense around the branch

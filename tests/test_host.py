@@ -267,6 +267,37 @@ def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     assert e.value.code == -4
 
 
+def test_dynamic_description_is_specialised_per_shape(tmp_path):
+    text = open(os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info"),
+                encoding="utf-8").read()
+    dyn = driver.HipDynamicKernel(text, out_dir=str(tmp_path))
+    a = dyn.specialize([[32, 1, 48, 48], [32, 12, 48, 48]])
+    b = dyn.specialize([[1, 1, 40, 72], [32, 12, 40, 72]])       # the mask may also broadcast along the batch
+    assert a.family == b.family == "row_reduce"
+    assert [t.shape for t in a.tensors] == [[32, 1, 48, 48], [32, 12, 48, 48], [32, 12, 48, 48]]
+    assert [t.shape for t in b.tensors] == [[1, 1, 40, 72], [32, 12, 40, 72], [32, 12, 40, 72]]
+    assert a.kernel_name != b.kernel_name and a.kernel_name.startswith("Fused_Sub_Mul_Mul_Add_Softmax_fusion_")
+    assert dyn.specialize([[32, 1, 48, 48], [32, 12, 48, 48]]) is a                 # cached per shape set
+    for k in (a, b):                                                                # one artifact set per shape
+        assert os.path.exists(os.path.join(str(tmp_path), k.kernel_name[:-len("_kernel")] + ".hsaco"))
+    with pytest.raises(driver.AkgHipError) as e:    # a static extent of the description cannot be rebound
+        dyn.specialize([[32, 1, 48, 48], [31, 12, 48, 48]])
+    assert e.value.code == -3 and "contradicts" in str(e.value)
+    with pytest.raises(driver.AkgHipError) as e:    # operands that do not broadcast under the binding
+        dyn.specialize([[32, 1, 48, 48], [32, 12, 48, 47]])
+    assert e.value.code == -3
+    with pytest.raises(driver.AkgHipError) as e:    # wrong number of shapes
+        dyn.specialize([[32, 1, 48, 48]])
+    assert e.value.code == -1
+    # a dynamic Reshape may leave one extent open; reductions and MatMul derive their result shapes
+    b2 = op_desc.DescBuilder("Fused_dyn_matmul")
+    x = b2.input([-1, 64], "bfloat16")
+    w = b2.input([64, 32], "bfloat16")
+    d = b2.build([b2.cast(b2.matmul(x, w, "float32"), "bfloat16")])
+    k = driver.HipDynamicKernel(json.dumps(d), out_dir=None).specialize([[128, 64], [64, 32]])
+    assert k.family == "gemm_epilogue" and k.outputs[0].shape == [128, 32]
+
+
 def _meta_schedule(kernel):
     with open(os.path.join(driver.DEFAULT_META_DIR, kernel.kernel_name[:-len("_kernel")] + ".json"), encoding="utf-8") as f:
         return json.load(f)["schedule"]
