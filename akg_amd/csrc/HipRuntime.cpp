@@ -234,6 +234,27 @@ std::string shapeArgText(const akg::LoweredKernel &k) {
   return os.str();
 }
 
+// <op>_shape_info.json (DumpShapeInfo.cpp:133-142): shapes as the caller sees them and as the kernel addresses them.
+// Kernels here take bare pointers to the caller's dense row-major buffers and carry every extent as a compile-time
+// constant, so both lists are the tensors' own shapes and there are no runtime variables.
+std::string shapeInfoJson(const akg::OpGraph &g) {
+  std::ostringstream shapes;
+  shapes << "[";
+  bool first = true;
+  auto emitShape = [&](int id) {
+    shapes << (first ? "" : ", ") << "[";
+    const auto &s = g.tensor(id).shape;
+    for (size_t i = 0; i < s.size(); ++i) shapes << (i ? ", " : "") << s[i];
+    shapes << "]";
+    first = false;
+  };
+  for (int id : g.inputs) emitShape(id);
+  for (int id : g.outputs) emitShape(id);
+  shapes << "]";
+  return "{\"hostShapes\": " + shapes.str() + ", \"deviceShapes\": " + shapes.str() +
+         ", \"runtimeVars\": [], \"SupportInfo\": {}}";
+}
+
 int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
               const akg::ShapeBinding *binding = nullptr) {
   if (outKernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "out_kernel is NULL");
@@ -300,7 +321,9 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
     if (!base.empty()) {
       std::string meta = metaJson(*k, srcDigest);
       std::string shapeArg = shapeArgText(k->lowered);
-      if (!writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size()) ||
+      std::string shapeInfo = shapeInfoJson(k->graph);
+      if (!writeFile(base + "_shape_info.json", shapeInfo.data(), shapeInfo.size()) ||
+          !writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size()) ||
           !writeFile(base + ".hsaco", k->codeObject.data(), k->codeObject.size()) ||
           !writeFile(base + "_shape_arg.txt", shapeArg.data(), shapeArg.size()) ||
           !writeFile(base + ".json", meta.data(), meta.size())) {

@@ -77,7 +77,8 @@ typedef struct akg_hip_kernel akg_hip_kernel_t;
  * (TranslateToPTX.cpp:67-103).
  * If out_dir is non-NULL the reference's artifact set is written there: <op>.hsaco (in place of <op>.ptx),
  * <op>.json {blockIdx.*, threadIdx.*, kernelName, is_dynamic, sha256} (GPUMapping.cpp:645-665,
- * mlir_driver.py:776-815), <op>_shape_arg.txt (KernelOutliningExt.cpp:384-423), <op>.hip (the emitted
+ * mlir_driver.py:776-815), <op>_shape_arg.txt (KernelOutliningExt.cpp:384-423), <op>_shape_info.json {hostShapes,
+ * deviceShapes, runtimeVars, SupportInfo} (DumpShapeInfo.cpp:133-142), <op>.hip (the emitted
  * source, the counterpart of the <op>_gpu.mlir dump); a matching artifact found there is reused instead
  * of compiling (the reference's KERNEL_META_DIR cache, mlir_driver.py:47-53).
  */

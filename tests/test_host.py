@@ -309,8 +309,11 @@ def test_artifacts_have_the_reference_layout(tmp_path):
     k = driver.HipKernel.from_file(info, out_dir=out)
     assert not k.cache_hit
     name = "small_quant_int8_residual_bf16_37x1544"
-    for ext in (".hsaco", ".json", "_shape_arg.txt", ".hip"):
+    for ext in (".hsaco", ".json", "_shape_arg.txt", "_shape_info.json", ".hip"):
         assert os.path.exists(os.path.join(out, name + ext))
+    shape_info = json.load(open(os.path.join(out, name + "_shape_info.json")))
+    assert shape_info["hostShapes"] == shape_info["deviceShapes"] == [[37, 1544], [37, 1544], [37, 1544], [37]]
+    assert shape_info["runtimeVars"] == [] and "SupportInfo" in shape_info
     meta = json.load(open(os.path.join(out, name + ".json")))
     for key in ("blockIdx.x", "blockIdx.y", "blockIdx.z", "threadIdx.x", "threadIdx.y", "threadIdx.z"):
         assert isinstance(meta[key], int)
