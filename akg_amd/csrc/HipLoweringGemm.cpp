@@ -49,12 +49,14 @@ class GemmEmitter {
     k.family = KernelFamily::GemmEpilogue;
     const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
     k.grid[0] = static_cast<unsigned>(((tiles + 7) / 8) * 8);
+    k.grid[1] = static_cast<unsigned>(batch_);
     k.block[0] = static_cast<unsigned>(wavesM() * 2 * 64);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
-    k.algorithmicOps = 2ull * static_cast<uint64_t>(m_) * static_cast<uint64_t>(n_) * static_cast<uint64_t>(k_);
+    k.algorithmicOps = 2ull * static_cast<uint64_t>(batch_) * static_cast<uint64_t>(m_) * static_cast<uint64_t>(n_) *
+                       static_cast<uint64_t>(k_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
-    note << "gemm_epilogue M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
+    note << "gemm_epilogue batch=" << batch_ << " M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
          << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
          << k.grid[0];
     k.scheduleNote = note.str();
@@ -65,7 +67,7 @@ class GemmEmitter {
   const OpGraph &g_;
   LoweringOptions opt_;
   std::ostringstream src_;
-  int64_t m_ = 0, n_ = 0, k_ = 0;
+  int64_t m_ = 0, n_ = 0, k_ = 0, batch_ = 1;
   bool transB_ = false;
   int matmulOp_ = -1;
   int aId_ = -1, bId_ = -1, accId_ = -1;
@@ -122,14 +124,21 @@ class GemmEmitter {
       throw LoweringError("MatMul: MFMA kernels exist for int8 x int8 -> int32 and for bfloat16 / float16 operands "
                           "with a float32 or same-type result");
     }
-    if (a.shape.size() != 2 || b.shape.size() != 2 || c.shape.size() != 2) {
-      throw LoweringError("MatMul: only rank-2 operands are supported");
+    // [M,K] x [K,N], or one leading batch dimension on all three ([B,M,K] x [B,K,N] -> [B,M,N]: linalg.batch_matmul,
+    // MindSporeToLinalg.cpp:1511-1530); every batch is one grid.y slice of the same tile kernel.
+    const size_t rank = a.shape.size();
+    if ((rank != 2 && rank != 3) || b.shape.size() != rank || c.shape.size() != rank) {
+      throw LoweringError("MatMul: operands and result must all be rank 2, or all rank 3 with one batch dimension");
     }
-    m_ = a.shape[0];
-    k_ = a.shape[1];
-    n_ = transB_ ? b.shape[0] : b.shape[1];
-    const int64_t kb = transB_ ? b.shape[1] : b.shape[0];
-    if (kb != k_ || c.shape[0] != m_ || c.shape[1] != n_) throw LoweringError("MatMul: inconsistent shapes");
+    const size_t o = rank - 2;
+    batch_ = rank == 3 ? a.shape[0] : 1;
+    if (rank == 3 && (b.shape[0] != batch_ || c.shape[0] != batch_)) throw LoweringError("MatMul: batch extents differ");
+    if (batch_ < 1 || batch_ > 65535) throw LoweringError("MatMul: batch extent out of range");
+    m_ = a.shape[o];
+    k_ = a.shape[o + 1];
+    n_ = transB_ ? b.shape[o] : b.shape[o + 1];
+    const int64_t kb = transB_ ? b.shape[o + 1] : b.shape[o];
+    if (kb != k_ || c.shape[o] != m_ || c.shape[o + 1] != n_) throw LoweringError("MatMul: inconsistent shapes");
     if ((k_ * elemBytes()) % 16 != 0) throw LoweringError("MatMul: a row of K must be a multiple of 16 bytes");
     if (n_ % 4 != 0) throw LoweringError("MatMul: N must be a multiple of 4");
     for (const OpNode &op : g_.ops) {
@@ -148,13 +157,24 @@ class GemmEmitter {
 
   EpiRank classifyInput(const TensorValue &t) const {
     if (t.numel() == 1) return EpiRank::Scalar;
+    // the result is addressed as [batch * M, N]: fold a leading batch dimension into the rows
     std::vector<int64_t> s = t.shape;
-    while (s.size() > 2 && s.front() == 1) s.erase(s.begin());
+    while (s.size() > 3 && s.front() == 1) s.erase(s.begin());
+    if (s.size() == 3) {
+      if (s[0] == batch_ && s[1] == m_) {
+        s = {batch_ * m_, s[2]};
+      } else if (s[0] == 1 && (batch_ == 1 || s[1] == 1)) {
+        s = {s[1], s[2]};
+      } else {
+        throw LoweringError("epilogue input " + t.name + " does not broadcast to the MatMul result");
+      }
+    }
     if (s.size() == 1) s.insert(s.begin(), 1);
     if (s.size() != 2) throw LoweringError("epilogue input " + t.name + ": rank exceeds the output's");
-    if (s[0] == m_ && s[1] == n_) return EpiRank::Full;
+    const int64_t rows = batch_ * m_;
+    if (s[0] == rows && s[1] == n_) return EpiRank::Full;
     if (s[0] == 1 && s[1] == n_) return EpiRank::Col;
-    if (s[0] == m_ && s[1] == 1) return EpiRank::Row;
+    if (s[0] == rows && s[1] == 1) return EpiRank::Row;
     throw LoweringError("epilogue input " + t.name + " does not broadcast to the MatMul result");
   }
 
@@ -214,12 +234,12 @@ class GemmEmitter {
           break;
         case EpiRank::Row:
           v.ident = "r_in" + std::to_string(i);
-          apply_ << "    const " << ct << " " << v.ident << " = " << tag << "::load(in" << i << "[row]);\n";
+          apply_ << "    const " << ct << " " << v.ident << " = " << tag << "::load(in" << i << "[grow]);\n";
           break;
         case EpiRank::Full:
           v.ident = "t_in" + std::to_string(i);
           apply_ << "    " << ct << " " << v.ident << "[4];\n";
-          apply_ << "    akg::load_chunk<" << tag << ", 4, " << (nt ? "true" : "false") << ">(in" << i << " + row * " << n_
+          apply_ << "    akg::load_chunk<" << tag << ", 4, " << (nt ? "true" : "false") << ">(in" << i << " + grow * " << n_
                  << "L + col, " << v.ident << ");\n";
           break;
         default:
@@ -288,10 +308,10 @@ class GemmEmitter {
       const TensorValue &t = g_.tensor(id);
       const EpiVal &v = vals_[static_cast<size_t>(id)];
       if (!v.defined) throw LoweringError("output " + t.name + " is never computed");
-      if (t.numel() != m_ * n_ || v.rank != EpiRank::Full) {
+      if (t.numel() != batch_ * m_ * n_ || v.rank != EpiRank::Full) {
         throw LoweringError("output " + t.name + ": only [M,N] outputs of a MatMul fusion are supported");
       }
-      apply_ << "    akg::store_chunk<" << tagOf(id) << ", 4, " << (nt ? "true" : "false") << ">(out" << i << " + row * "
+      apply_ << "    akg::store_chunk<" << tagOf(id) << ", 4, " << (nt ? "true" : "false") << ">(out" << i << " + grow * "
              << n_ << "L + col, " << v.ident << ");\n";
     }
 
@@ -301,7 +321,9 @@ class GemmEmitter {
     src_ << "#include \"akg_rt.hpp\"\n#include \"akg_gemm_mfma.hpp\"\n\n";
     src_ << "namespace {\nstruct Epilogue {\n" << members_.str();
     src_ << "  AKG_DEV void prepare(long col) {\n    (void)col;\n" << prepare_.str() << "  }\n";
-    src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[4], long row, long col) {\n" << apply_.str() << "  }\n";
+    src_ << "  long row0;  // first row of this batch in the [batch * M, N] view of the result\n";
+    src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[4], long row, long col) {\n"
+         << "    const long grow = row0 + row;\n    (void)grow;\n" << apply_.str() << "  }\n";
     src_ << "};\n}  // namespace\n\n";
     src_ << "extern \"C\" __global__ __launch_bounds__(" << wavesM() * 128 << ") void " << kname << "(";
     size_t argc = 0;
@@ -311,7 +333,8 @@ class GemmEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
-    src_ << ") {\n  Epilogue epi;\n";
+    src_ << ") {\n  Epilogue epi;\n  const long akg_batch = static_cast<long>(blockIdx.y);\n"
+         << "  epi.row0 = akg_batch * " << m_ << "L;\n";
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       const int id = g_.inputs[i];
       if (id == aId_ || id == bId_) continue;
@@ -319,7 +342,8 @@ class GemmEmitter {
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
     src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi);\n}\n";
+         << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
+         << " + akg_batch * " << k_ * n_ << "L, epi);\n}\n";
   }
 };
 

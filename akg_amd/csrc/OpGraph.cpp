@@ -97,7 +97,7 @@ const OpTableEntry kOpTable[] = {
   {"StridedSlice", OpKind::StridedSlice},
   {"AddN", OpKind::AddN},
   {"MatMul", OpKind::MatMul},
-  {"BatchMatMul", OpKind::Unsupported},
+  {"BatchMatMul", OpKind::MatMul},
   {"Cast", OpKind::Cast},
 };
 
@@ -397,7 +397,8 @@ class GraphBuilder {
     }
     if (node.kind == OpKind::MatMul) {
       const std::vector<int64_t> a = shapeOf(0), b = shapeOf(1);
-      if (a.size() != 2 || b.size() != 2) throw TranslateError("op " + node.name + ": only rank-2 MatMul is supported");
+      if (a.size() == 3 && b.size() == 3) return {a[0], a[1], node.transposeB ? b[1] : b[2]};
+      if (a.size() != 2 || b.size() != 2) throw TranslateError("op " + node.name + ": MatMul operands must be rank 2 or 3");
       return {a[0], node.transposeB ? b[0] : b[1]};
     }
     if (node.kind == OpKind::Reshape || node.kind == OpKind::BroadcastTo) {

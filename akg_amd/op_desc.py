@@ -402,3 +402,17 @@ def transpose_sum(shape, perm, dtype="float32", name=None):
     x = b.input(list(shape), dtype)
     y = b.input(list(shape), dtype)
     return b.dumps([b.add(transpose(b, x, perm), b.mul(transpose(b, y, perm), b.const(2.0, dtype)))])
+
+
+def batch_matmul_scale_mask(batch, m, k, n, dtype="bfloat16", transpose_b=True, name=None):
+    """Attention scores: out[b] = (Q[b] @ K[b]^T) * scale + mask, Q [batch,m,k], K [batch,n,k] (transpose_b) or
+    [batch,k,n], mask [batch,m,n] in float32, result in `dtype`."""
+    b = DescBuilder(name or "Fused_BatchMatMul_Mul_Add_%s_%dx%dx%dx%d%s" % (_SHORT[dtype], batch, m, k, n, "_tb" if transpose_b else ""))
+    q = b.input([batch, m, k], dtype)
+    kk = b.input([batch, n, k] if transpose_b else [batch, k, n], dtype)
+    mask = b.input([batch, m, n], "float32")
+    attrs = [{"data_type": "bool", "name": "transpose_a", "value": False},
+             {"data_type": "bool", "name": "transpose_b", "value": bool(transpose_b)}]
+    s = b.op("BatchMatMul", [q, kk], [batch, m, n], "float32", attrs=attrs)
+    s = b.add(b.mul(s, b.const(1.0 / (k ** 0.5), "float32")), mask)
+    return b.dumps([b.cast(s, dtype)])

@@ -55,6 +55,7 @@ INT_RANGE = {"int8": (-128, 127), "int16": (-32768, 32767), "int32": (-214748364
 UNARY_MATH = {"Exp": "exp", "Log": "log", "Tanh": "tanh", "Sqrt": "sqrt", "Floor": "floor", "Sin": "sin", "Cos": "cos",
               "ASin": "asin", "ACos": "acos", "Atan": "atan", "Asinh": "asinh", "Acosh": "acosh"}
 COMPARE = {"Equal": "==", "NotEqual": "!=", "Greater": ">", "GreaterEqual": ">=", "Less": "<", "LessEqual": "<="}
+MATMULS = ("MatMul", "BatchMatMul")
 REDUCES = ("ReduceSum", "ReduceMax", "ReduceMin", "ReducePrd", "ReduceAll", "ReduceAny")
 ATTR_AS_INPUT = ("Reshape", "BroadcastTo", "ReduceMax", "ReduceMin", "ReduceSum", "ReducePrd", "ReduceAll", "ReduceAny",
                  "ArgMax", "Transpose", "Tile")
@@ -272,7 +273,7 @@ class Emitter:
 
     # -- which values live in memory --------------------------------------------------------------------
     def is_elementwise(self, op):
-        return op.name not in REDUCES and op.name not in ("MatMul", "Reshape") and op.name not in VIEW_OPS
+        return op.name not in REDUCES and op.name not in MATMULS + ("Reshape",) and op.name not in VIEW_OPS
 
     def plan(self):
         consumers = {}
@@ -285,11 +286,11 @@ class Emitter:
                 out.alias_of = op.inputs[0]
                 continue
             inline = (self.is_elementwise(op) and out.uses == 1 and not out.is_output
-                      and consumers[out.name][0].name not in ("MatMul", "Reshape") + VIEW_OPS)
+                      and consumers[out.name][0].name not in MATMULS + ("Reshape",) + VIEW_OPS)
             out.inline = inline
         # the source of a Reshape view and MatMul operands must be in memory
         for op in self.ops:
-            if op.name in ("Reshape", "MatMul") + VIEW_OPS:
+            if op.name in MATMULS + ("Reshape",) + VIEW_OPS:
                 for t in op.inputs:
                     if t.producer is not None and t.producer.name != "Reshape":
                         t.inline = False
@@ -593,35 +594,41 @@ class Emitter:
         if op.attrs.get("transpose_a", False):
             raise OracleError("TransposeA is not supported (MindSporeToLinalg.cpp:1508-1510)")
         tb = bool(op.attrs.get("transpose_b", False))
-        if len(a.shape) != 2 or len(b.shape) != 2:
-            raise OracleError("only rank-2 MatMul is restated")
-        m, k = a.shape
-        n = b.shape[0] if tb else b.shape[1]
+        if len(a.shape) not in (2, 3) or len(b.shape) != len(a.shape):
+            raise OracleError("MatMul operands must both be rank 2, or both rank 3 with one batch dimension")
+        # BatchMatMul (linalg.batch_matmul, MindSporeToLinalg.cpp:1511-1530): the same loop nest per batch index
+        batch = a.shape[0] if len(a.shape) == 3 else 1
+        if len(a.shape) == 3 and b.shape[0] != batch:
+            raise OracleError("batch extents differ")
+        m, k = a.shape[-2], a.shape[-1]
+        n = b.shape[-2] if tb else b.shape[-1]
         od = out.dtype
         ct = C_COMPUTE[od]
         ra, rb = self.root(a), self.root(b)
-        aidx = "i * %dL + k" % k
-        bidx = ("j * %dL + k" % k) if tb else ("k * %dL + j" % n)
+        aidx = "(bt * %dL + i) * %dL + k" % (m, k)
+        bidx = ("(bt * %dL + j) * %dL + k" % (n, k)) if tb else ("(bt * %dL + k) * %dL + j" % (k, n))
         prod = "(%s)%s * (%s)%s" % (ct, self.load_expr(ra, aidx), ct, self.load_expr(rb, bidx))
-        cidx = "i * %dL + j" % n
+        cidx = "(bt * %dL + i) * %dL + j" % (m, n)
         # zero-filled accumulator of the output type
-        self.emit("memset(%s, 0, sizeof(%s) * %dL);" % (out.buffer, C_STORAGE[od], m * n))
-        if self.openmp:
-            self.emit("#pragma omp parallel for schedule(static)")
-        self.emit("for (int64_t i = 0; i < %dL; ++i) {" % m)
+        self.emit("memset(%s, 0, sizeof(%s) * %dL);" % (out.buffer, C_STORAGE[od], batch * m * n))
         if od in FLOATS and od not in ("float32", "float64"):
             raise OracleError("MatMul accumulating in %s is not restated" % od)
+        self.emit("for (int64_t bt = 0; bt < %dL; ++bt) {" % batch)
+        if self.openmp:
+            self.emit("#pragma omp parallel for schedule(static)", 2)
+        self.emit("for (int64_t i = 0; i < %dL; ++i) {" % m, 2)
         if self.matmul_order == "ijk":
-            self.emit("for (int64_t j = 0; j < %dL; ++j) {" % n, 2)
-            self.emit("for (int64_t k = 0; k < %dL; ++k) {" % k, 3)
-        else:
-            self.emit("for (int64_t k = 0; k < %dL; ++k) {" % k, 2)
             self.emit("for (int64_t j = 0; j < %dL; ++j) {" % n, 3)
+            self.emit("for (int64_t k = 0; k < %dL; ++k) {" % k, 4)
+        else:
+            self.emit("for (int64_t k = 0; k < %dL; ++k) {" % k, 3)
+            self.emit("for (int64_t j = 0; j < %dL; ++j) {" % n, 4)
         if od in INTS:
             ut = "uint64_t" if od == "int64" else "uint32_t"
-            self.emit("%s[%s] = (%s)((%s)%s[%s] + (%s)(%s));" % (out.buffer, cidx, C_STORAGE[od], ut, out.buffer, cidx, ut, prod), 4)
+            self.emit("%s[%s] = (%s)((%s)%s[%s] + (%s)(%s));" % (out.buffer, cidx, C_STORAGE[od], ut, out.buffer, cidx, ut, prod), 5)
         else:
-            self.emit("%s[%s] = %s[%s] + %s;" % (out.buffer, cidx, out.buffer, cidx, prod), 4)
+            self.emit("%s[%s] = %s[%s] + %s;" % (out.buffer, cidx, out.buffer, cidx, prod), 5)
+        self.emit("}", 4)
         self.emit("}", 3)
         self.emit("}", 2)
         self.emit("}")
@@ -662,7 +669,7 @@ class Emitter:
             self.emit("/* %s -> %s */" % (op.name, out.name))
             if op.name in REDUCES:
                 self.emit_reduce(op)
-            elif op.name == "MatMul":
+            elif op.name in MATMULS:
                 self.emit_matmul(op)
             elif op.name in VIEW_OPS:
                 self.emit_view(op)

@@ -322,21 +322,29 @@ def evaluate(desc, inputs):
                 else:
                     res = np.concatenate([x, ins[1]], axis=vp["axis"])
                 res = np.ascontiguousarray(res)
-            elif name == "MatMul":
+            elif name in ("MatMul", "BatchMatMul"):
                 if attrs.get("transpose_a", False):
                     raise ValueError("TransposeA is not supported")
                 a, b = ins[0], ins[1]
+                if a.ndim == 2:
+                    a, b = a[None], b[None]
                 if attrs.get("transpose_b", False):
-                    b = b.T
-                if odt == "int32" and in_dt[0] == "int8" and in_dt[1] == "int8":
-                    res = matmul_exact_i32(a, b)
-                elif odt in ("float32", "float64"):
-                    # serial k order in the output type
-                    res = np.zeros((a.shape[0], b.shape[1]), dtype=NP_DTYPE[odt])
-                    for k in range(a.shape[1]):
-                        res = res + np.outer(a[:, k].astype(res.dtype), b[k, :].astype(res.dtype))
-                else:
-                    raise ValueError("MatMul %s x %s -> %s is not restated" % (in_dt[0], in_dt[1], odt))
+                    b = np.swapaxes(b, 1, 2)
+                slices = []
+                for a2, b2 in zip(a, b):      # one matrix product per batch index
+                    if odt == "int32" and in_dt[0] == "int8" and in_dt[1] == "int8":
+                        slices.append(matmul_exact_i32(a2, b2))
+                    elif odt in ("float32", "float64"):
+                        # serial k order in the output type
+                        acc = np.zeros((a2.shape[0], b2.shape[1]), dtype=NP_DTYPE[odt])
+                        for k in range(a2.shape[1]):
+                            acc = acc + np.outer(a2[:, k].astype(acc.dtype), b2[k, :].astype(acc.dtype))
+                        slices.append(acc)
+                    else:
+                        raise ValueError("MatMul %s x %s -> %s is not restated" % (in_dt[0], in_dt[1], odt))
+                res = np.stack(slices)
+                if ins[0].ndim == 2:
+                    res = res[0]
             else:
                 raise ValueError("op %s is not supported by the numpy restatement" % name)
         res = finish(res, odt) if name not in ("Cast",) else res

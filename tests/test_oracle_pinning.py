@@ -356,6 +356,18 @@ def test_bf16_matmul_bias_gelu_matches_torch_float64():
     assert np.allclose(harness.bf16_bits_to_f32(c_out[0]).astype(np.float64), ref, rtol=1e-2, atol=1e-3)
 
 
+def test_batch_matmul_is_one_product_per_batch_index():
+    """BatchMatMul against torch float64 bmm: batches must not mix and transpose_b must read [batch, n, k]."""
+    import torch
+    for name, tb, dt in (("small_batchmatmul_scale_mask_bf16_3x200x64x136_tb", True, "bfloat16"),
+                         ("small_batchmatmul_scale_mask_f16_2x256x128x256", False, "float16")):
+        desc, inputs, c_out, n_out = run_fixture_both(name, 24)
+        q, k, mask = (torch.from_numpy(harness.to_float(x, d)) for x, d in zip(inputs, (dt, dt, "float32")))
+        ref = (torch.bmm(q, k.transpose(1, 2) if tb else k) / (q.shape[-1] ** 0.5) + mask).numpy()
+        for out in (c_out[0], n_out[0]):
+            assert np.allclose(harness.to_float(out, dt), ref, rtol=1e-2, atol=1e-3)
+
+
 # ---------------------------------------------------------------------------------------------------------
 # the two restatements against each other on every small fixture
 # ---------------------------------------------------------------------------------------------------------
