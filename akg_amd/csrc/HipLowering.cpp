@@ -589,7 +589,8 @@ class TileEmitter {
     access_.resize(g_.inputs.size());
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       const TensorValue &t = g_.tensor(g_.inputs[i]);
-      std::vector<int64_t> s = padShape(t.shape, r, "input " + t.name);
+      // an input nothing reads takes no part in the iteration space
+      std::vector<int64_t> s = padShape(t.used ? t.shape : std::vector<int64_t>{1}, r, "input " + t.name);
       for (size_t d = 0; d < r; ++d) {
         if (s[d] != 1 && s[d] != space[d]) {
           throw LoweringError("input " + t.name + " is not broadcast-compatible with the reduced tensor");
@@ -611,7 +612,7 @@ class TileEmitter {
     std::vector<std::vector<int64_t>> padded;
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       const TensorValue &t = g_.tensor(g_.inputs[i]);
-      std::vector<int64_t> s = padShape(t.shape, r, "input " + t.name);
+      std::vector<int64_t> s = padShape(t.used ? t.shape : std::vector<int64_t>{1}, r, "input " + t.name);
       for (size_t d = 0; d < r; ++d) {
         if (s[d] != 1 && s[d] != space[d]) {
           throw LoweringError("input " + t.name + " is not broadcast-compatible with the output shape");

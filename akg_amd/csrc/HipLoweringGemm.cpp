@@ -215,6 +215,7 @@ class GemmEmitter {
       const int id = g_.inputs[i];
       if (id == aId_ || id == bId_) continue;
       const TensorValue &t = g_.tensor(id);
+      if (!t.used) continue;
       const EpiRank r = classifyInput(t);
       EpiVal &v = vals_[static_cast<size_t>(id)];
       v.defined = true;
@@ -337,7 +338,7 @@ class GemmEmitter {
          << "  epi.row0 = akg_batch * " << m_ << "L;\n";
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       const int id = g_.inputs[i];
-      if (id == aId_ || id == bId_) continue;
+      if (id == aId_ || id == bId_ || !g_.tensor(id).used) continue;
       src_ << "  epi.in" << i << " = in" << i << ";\n";
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";

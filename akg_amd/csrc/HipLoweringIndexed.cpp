@@ -520,10 +520,21 @@ class IndexedEmitter {
 }  // namespace
 
 bool wantsIndexedKernel(const OpGraph &graph) {
+  bool reshapes = false, contraction = false;
   for (const OpNode &op : graph.ops) {
     if (isViewKind(op.kind)) return true;
+    if (op.kind == OpKind::MatMul || lowering::isReduceKind(op.kind)) contraction = true;
+    if (op.kind == OpKind::Reshape) {
+      // A Reshape that only adds or drops leading unit dimensions keeps every operand right-aligned with the
+      // outputs, which is what the chunked elementwise kernel relies on; any other Reshape changes how the
+      // dimensions of operands in front of it line up with the outputs' and needs real index arithmetic.
+      std::vector<int64_t> a = graph.tensor(op.inputs[0]).shape, b = graph.tensor(op.outputs[0]).shape;
+      while (a.size() > 1 && a.front() == 1) a.erase(a.begin());
+      while (b.size() > 1 && b.front() == 1) b.erase(b.begin());
+      if (a != b) reshapes = true;
+    }
   }
-  return false;
+  return reshapes && !contraction;
 }
 
 LoweredKernel lowerIndexedToHip(const OpGraph &graph, const LoweringOptions &options) {

@@ -222,6 +222,7 @@ class StreamReduceEmitter {
     }
     for (int id : g_.inputs) {
       const TensorValue &t = g_.tensor(id);
+      if (!t.used) continue;
       const std::vector<int64_t> s = padTo(t.shape, "input " + t.name);
       for (size_t d = 0; d < n; ++d) {
         if (s[d] != 1 && s[d] != space_[d]) {
@@ -776,6 +777,8 @@ bool wantsStreamReduce(const OpGraph &graph) {
   }
   const bool innermostOnly = axes.size() == 1 && axes[0] == last;
   if (!innermostOnly) return true;
+  // trailing unit dimensions ([33,1] over axis 0): the row kernel aligns operands on the last dimension
+  if (last + 1 != in.shape.size()) return true;
   // direction X: the row kernel keeps a whole row in registers and gives every row its own threads. Rows beyond its
   // capacity, or so few long rows that the chip would idle, stream instead — unless some op needs the row again
   // after the reduction (softmax, LayerNorm), which only the row kernel can serve.

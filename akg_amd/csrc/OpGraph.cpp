@@ -827,8 +827,52 @@ OpGraph translateJsonToOpGraph(const std::string &jsonText, const ShapeBinding *
   json::Value root = json::Value::parse(jsonText);
   GraphBuilder builder(root, binding);
   OpGraph g = builder.build();
+  removeRedundantReduces(&g);
+  pruneDeadOps(&g);
   identifyOperator(&g);
   return g;
+}
+
+void removeRedundantReduces(OpGraph *graph) {
+  for (OpNode &op : graph->ops) {
+    if (!isReduceKind(op.kind) || op.inputs.empty()) continue;
+    const std::vector<int64_t> &in = graph->tensor(op.inputs[0]).shape;
+    bool redundant = true;
+    for (int64_t a : op.axes) {
+      if (a >= 0 && static_cast<size_t>(a) < in.size() && in[static_cast<size_t>(a)] != 1) redundant = false;
+    }
+    if (!redundant || graph->tensor(op.inputs[0]).dtype != graph->tensor(op.outputs[0]).dtype) continue;
+    op.kind = OpKind::Reshape;
+    op.axes.clear();
+    op.inputs.resize(1);
+  }
+}
+
+void pruneDeadOps(OpGraph *graph) {
+  std::vector<bool> live(graph->tensors.size(), false);
+  for (int id : graph->outputs) live[static_cast<size_t>(id)] = true;
+  std::vector<bool> keep(graph->ops.size(), false);
+  for (size_t k = graph->ops.size(); k-- > 0;) {
+    const OpNode &op = graph->ops[k];
+    bool needed = op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported;  // keep what must be reported
+    for (int out : op.outputs) needed = needed || live[static_cast<size_t>(out)];
+    if (!needed) continue;
+    keep[k] = true;
+    for (int in : op.inputs) live[static_cast<size_t>(in)] = true;
+  }
+  std::vector<int> newIndex(graph->ops.size(), -1);
+  std::vector<OpNode> kept;
+  for (size_t k = 0; k < graph->ops.size(); ++k) {
+    if (!keep[k]) continue;
+    newIndex[k] = static_cast<int>(kept.size());
+    kept.push_back(graph->ops[k]);
+  }
+  graph->ops.swap(kept);
+  for (size_t t = 0; t < graph->tensors.size(); ++t) {
+    TensorValue &tv = graph->tensors[t];
+    if (tv.producer >= 0) tv.producer = newIndex[static_cast<size_t>(tv.producer)];
+    if (tv.inputIndex >= 0) tv.used = live[t];
+  }
 }
 
 void identifyOperator(OpGraph *graph) {

@@ -76,6 +76,7 @@ struct TensorValue {
   int producer = -1;          // index into OpGraph::ops, -1 for graph inputs and constants
   int inputIndex = -1;        // position in the kernel signature if this is a graph input
   int outputIndex = -1;       // position among the outputs if this is a graph output
+  bool used = true;           // false for a kernel input that no op on the way to an output reads
   int64_t numel() const;
 };
 
@@ -126,6 +127,15 @@ OpGraph translateJsonToOpGraph(const std::string &jsonText, const ShapeBinding *
 
 // True if the description has a -1 dimension on any kernel input, op result or kernel output.
 bool descriptionIsDynamic(const std::string &jsonText);
+
+// A reduction whose reduced axes all have extent 1 folds nothing: it becomes a Reshape of its operand
+// (RemoveRedundantReduce.cpp:46-75 replaces the keep_dims form by the operand; the other form differs from its operand
+// only in shape). Differs from evaluating the one-step reduction only for NaN under max / min and for -0.0 under sum.
+void removeRedundantReduces(OpGraph *graph);
+
+// Removes ops whose results no kernel output depends on and marks kernel inputs that nothing reads any more (they stay
+// in the signature). The reference gets the same effect from MLIR's dead-code elimination in its canonicalisation runs.
+void pruneDeadOps(OpGraph *graph);
 
 // Fusion-class identification (OperatorIdentify.cpp:51-93) and reduce-direction marking
 // (akg-mlir/lib/Dialect/Linalg/Transforms/MatchAndMarkReductionOps.cpp:51-88). Fills the two fields above.

@@ -1,0 +1,165 @@
+"""Seeded random fused-op descriptions for differential tests (product kernel against the CPU oracle).
+
+A description is grown op by op from two to four kernel inputs of broadcast-compatible shapes. Every value carries two
+facts the generator respects: its value range is tame (inputs are N(0,1); Exp / Reciprocal / RealDiv get bounded
+operands), and whether it is `exact`, i.e. computed only through correctly rounded operations. Ops that are
+discontinuous in their operand (comparisons, Select conditions, rounding to a narrower type) are only applied to exact
+values: two correct implementations may differ by an ulp after tanh or exp, and a discontinuity would turn that ulp
+into a different result.
+"""
+import numpy as np
+
+from akg_amd import op_desc
+
+FLOATS = ("float32", "float16", "bfloat16")
+
+
+class Val:
+    def __init__(self, t, exact=True, positive=False, bounded=True):
+        self.t = t
+        self.exact = exact
+        self.positive = positive   # values >= some margin above zero
+        self.bounded = bounded     # |values| small enough for Exp
+
+
+def _variant_shape(rng, base):
+    """A shape that broadcasts to `base`: some extents set to 1, leading dims possibly dropped."""
+    s = [d if rng.random() < 0.7 else 1 for d in base]
+    drop = int(rng.integers(0, len(s)))
+    if rng.random() < 0.3:
+        s = s[drop:] or [1]
+    return s
+
+
+def random_description(seed, allow_views=True, allow_reduce=True):
+    """Returns (json_text, notes). Deterministic in `seed`."""
+    rng = np.random.default_rng(seed)
+    rank = int(rng.integers(1, 5))
+    extents = [1, 2, 3, 4, 5, 7, 8, 9, 16, 33]
+    base = [int(rng.choice(extents)) for _ in range(rank)]
+    if rng.random() < 0.5:
+        base[-1] = int(rng.choice([8, 16, 32, 40, 64, 100]))
+    dtype = str(rng.choice(FLOATS))
+    b = op_desc.DescBuilder("Fused_random_%d" % seed)
+    f32 = lambda v: b.cast(v.t, "float32") if v.t.dtype != "float32" else v.t  # noqa: E731
+
+    vals = [Val(b.input(base, dtype))]
+    for _ in range(int(rng.integers(1, 4))):
+        vals.append(Val(b.input(_variant_shape(rng, base), dtype)))
+    # compute in float32 like the measured fusions do
+    work = [Val(f32(v), True) for v in vals]
+    notes = []
+    used_view = False
+
+    def pick(pred=lambda v: True):
+        cands = [v for v in work if pred(v)]
+        return cands[int(rng.integers(0, len(cands)))] if cands else None
+
+    n_ops = int(rng.integers(3, 10))
+    for _ in range(n_ops):
+        kind = rng.random()
+        x = pick()
+        if kind < 0.30:      # binary arithmetic with broadcasting
+            y = pick()
+            name = str(rng.choice(["Add", "Sub", "Mul", "Maximum", "Minimum"]))
+            try:
+                t = b.binary(name, x.t, y.t)
+            except ValueError:
+                continue
+            work.append(Val(t, x.exact and y.exact, bounded=False if name == "Mul" else x.bounded and y.bounded))
+            notes.append(name)
+        elif kind < 0.45:    # unary, correctly rounded
+            name = str(rng.choice(["Abs", "Neg", "Square"]))
+            work.append(Val(b.unary(name, x.t), x.exact, bounded=x.bounded and name != "Square"))
+            notes.append(name)
+        elif kind < 0.58:    # transcendental on a bounded operand
+            xb = pick(lambda v: v.bounded)
+            if xb is None:
+                continue
+            clipped = b.minimum(b.maximum(xb.t, b.const(-6.0, "float32")), b.const(6.0, "float32"))
+            name = str(rng.choice(["Tanh", "Exp"]))
+            work.append(Val(b.unary(name, clipped), False, positive=name == "Exp", bounded=name == "Tanh"))
+            notes.append(name)
+        elif kind < 0.66:    # division / reciprocal / sqrt with a safe operand
+            safe = b.add(b.unary("Abs", x.t), b.const(0.5, "float32"))
+            name = str(rng.choice(["RealDiv", "Reciprocal", "Sqrt", "Rsqrt"]))
+            if name == "RealDiv":
+                y = pick()
+                try:
+                    t = b.binary("RealDiv", y.t, safe)
+                except ValueError:
+                    continue
+                work.append(Val(t, x.exact and y.exact, bounded=False))
+            else:
+                work.append(Val(b.unary(name, safe), x.exact, positive=True, bounded=x.bounded))
+            notes.append(name)
+        elif kind < 0.76:    # comparison + Select on exact operands
+            xe, ye = pick(lambda v: v.exact), pick(lambda v: v.exact)
+            if xe is None or ye is None:
+                continue
+            try:
+                cmp_ = b.binary(str(rng.choice(["Greater", "LessEqual", "Equal", "NotEqual"])), xe.t, ye.t, dtype="bool")
+                a2, b2 = pick(), pick()
+                shape = b._broadcast(b._broadcast(cmp_.shape, a2.t.shape), b2.t.shape)
+            except ValueError:
+                continue
+            t = b.op("Select", [cmp_, a2.t, b2.t], shape, "float32")
+            work.append(Val(t, a2.exact and b2.exact, bounded=a2.bounded and b2.bounded))
+            notes.append("Select")
+        elif kind < 0.82:    # round trip through a narrow type (a rounding step: exact operands only)
+            x = pick(lambda v: v.exact)
+            if x is None:
+                continue
+            nt = str(rng.choice(["float16", "bfloat16"]))
+            work.append(Val(b.cast(b.cast(x.t, nt), "float32"), x.exact, bounded=x.bounded))
+            notes.append("Cast-" + nt)
+        elif allow_views and len(x.t.shape) >= 1 and kind < 1.0:
+            t = x.t
+            which = str(rng.choice(["Transpose", "Slice", "StridedSlice", "Pad", "Tile", "Concat", "Reshape"]))
+            r = len(t.shape)
+            if which == "Transpose" and r >= 2:
+                t = op_desc.transpose(b, t, [int(p) for p in rng.permutation(r)])
+            elif which == "Slice" and max(t.shape) >= 2:
+                begin = [int(rng.integers(0, d)) for d in t.shape]
+                size = [int(rng.integers(1, d - s + 1)) for d, s in zip(t.shape, begin)]
+                t = op_desc.slice_(b, t, begin, size)
+            elif which == "StridedSlice" and max(t.shape) >= 3:
+                begin = [int(rng.integers(0, max(1, d // 2))) for d in t.shape]
+                end = [int(rng.integers(s + 1, d + 1)) for d, s in zip(t.shape, begin)]
+                strides = [int(rng.integers(1, 4)) for _ in t.shape]
+                t = op_desc.strided_slice(b, t, begin, end, strides)
+            elif which == "Pad":
+                pairs = int(rng.integers(1, r + 1))
+                t = op_desc.pad(b, t, [int(rng.integers(0, 4)) for _ in range(2 * pairs)], value=int(rng.integers(-3, 4)))
+            elif which == "Tile" and int(np.prod(t.shape)) <= 4096:
+                t = op_desc.tile(b, t, [int(rng.integers(1, 3)) for _ in t.shape])
+            elif which == "Concat":
+                y = pick(lambda v: v.t.shape == x.t.shape)
+                t = op_desc.concat(b, t, y.t, int(rng.integers(0, r)))
+                x = Val(t, x.exact and y.exact, bounded=x.bounded and y.bounded)
+            elif which == "Reshape" and int(np.prod(t.shape)) > 1:
+                n = int(np.prod(t.shape))
+                divs = [d for d in range(1, n + 1) if n % d == 0]
+                d0 = int(rng.choice(divs))
+                t = b.reshape(t, [d0, n // d0])
+            else:
+                continue
+            work.append(Val(t, x.exact, x.positive, x.bounded))
+            used_view = True
+            notes.append(which)
+    out = work[-1]
+    outs = [out.t]
+    if allow_reduce and not used_view and rng.random() < 0.5 and len(out.t.shape) >= 1:
+        axis = [len(out.t.shape) - 1] if rng.random() < 0.6 else [int(rng.integers(0, len(out.t.shape)))]
+        name = str(rng.choice(["ReduceSum", "ReduceMax", "ReduceMin"]))
+        notes.append("%s%s" % (name, axis))
+        if rng.random() < 0.4 and axis == [len(out.t.shape) - 1]:
+            # use the reduced value again on the row it came from (softmax-like): only the row kernel can serve that
+            outs = [b.sub(out.t, b.reduce(name, out.t, axis, True))]
+            notes.append("Sub-after-reduce")
+        else:
+            outs = [b.reduce(name, out.t, axis, bool(rng.random() < 0.5))]
+    final = []
+    for t in outs:
+        final.append(b.cast(t, dtype) if dtype != "float32" and rng.random() < 0.7 else t)
+    return b.dumps(final), notes
