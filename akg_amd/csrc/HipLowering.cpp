@@ -241,6 +241,7 @@ bool isElementwiseKind(OpKind k) {
     case OpKind::StridedSlice:
     case OpKind::Pad:
     case OpKind::Concat:
+    case OpKind::Gather:
       return false;
     default:
       return !isReduceKind(k);

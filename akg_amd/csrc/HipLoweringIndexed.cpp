@@ -32,7 +32,7 @@ using lowering::dtypeTag;
 
 bool isViewKind(OpKind k) {
   return k == OpKind::Transpose || k == OpKind::Tile || k == OpKind::Slice || k == OpKind::StridedSlice ||
-         k == OpKind::Pad || k == OpKind::Concat;
+         k == OpKind::Pad || k == OpKind::Concat || k == OpKind::Gather;
 }
 
 class IndexedEmitter {
@@ -102,6 +102,7 @@ class IndexedEmitter {
       if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
       if (isViewKind(op.kind)) {
         for (int in : op.inputs) {
+          if (op.kind == OpKind::Gather && in == op.inputs[1]) continue;  // the indices
           if (g_.tensor(in).dtype != g_.tensor(op.outputs[0]).dtype) {
             throw LoweringError("op " + op.name + ": operand and result element types differ");
           }
@@ -325,6 +326,25 @@ class IndexedEmitter {
           closeScope();
           stmt("}");
         }
+        break;
+      }
+      case OpKind::Gather: {
+        // result index = data index with the gathered axis replaced by the indices' dimensions; the looked-up
+        // position is clamped into the axis (the reference reads out of bounds there, which must not fault a GPU)
+        const std::vector<int64_t> data = inShapeOf(0), ind = inShapeOf(1);
+        const size_t a = static_cast<size_t>(op.concatAxis);
+        const size_t indRank = g_.tensor(op.inputs[1]).shape.size();
+        Index where(ind.size(), "0");
+        for (size_t d = 0; d < indRank && d < ind.size(); ++d) where[d] = idx[a + d];
+        const std::string pos = fresh("g");
+        stmt("int " + pos + " = static_cast<int>(" + valueAt(op.inputs[1], where) + ");");
+        stmt(pos + " = " + pos + " < 0 ? 0 : (" + pos + " > " + std::to_string(data[a] - 1) + " ? " +
+             std::to_string(data[a] - 1) + " : " + pos + ");");
+        Index src(data.size());
+        for (size_t d = 0; d < a; ++d) src[d] = idx[d];
+        src[a] = pos;
+        for (size_t d = a + 1; d < data.size(); ++d) src[d] = idx[d - 1 + indRank];
+        stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
         break;
       }
       case OpKind::Concat: {

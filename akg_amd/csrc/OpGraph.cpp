@@ -80,7 +80,7 @@ const OpTableEntry kOpTable[] = {
   {"ReducePrd", OpKind::ReduceProd},
   {"ReduceAll", OpKind::ReduceAll},
   {"ReduceAny", OpKind::ReduceAny},
-  {"ElemAny", OpKind::Unsupported},
+  {"ElemAny", OpKind::ReduceAny},
   {"ArgMax", OpKind::Unsupported},
   {"BroadcastTo", OpKind::BroadcastTo},
   {"Slice", OpKind::Slice},
@@ -90,7 +90,7 @@ const OpTableEntry kOpTable[] = {
   {"Transpose", OpKind::Transpose},
   {"Split", OpKind::Unsupported},
   {"Pad", OpKind::Pad},
-  {"Gather", OpKind::Unsupported},
+  {"Gather", OpKind::Gather},
   {"InplaceAssign", OpKind::Unsupported},
   {"Assign", OpKind::Unsupported},
   {"UnsortedSegmentSum", OpKind::Unsupported},
@@ -299,6 +299,7 @@ class GraphBuilder {
           if (isIndex1DAttrAsInput(node.name, j)) continue;
           if (node.kind == OpKind::Cast && j > 0) continue;  // convertCastOp keeps the first operand only (:1351-1360)
           if (node.kind == OpKind::StridedSlice && j > 0) continue;  // begin / end / strides carried as constants
+          if (node.kind == OpKind::Gather && j > 1) continue;        // the axis carried as a constant
           node.inputs.push_back(operandFor(inputDesc[j][0], node.name));
         }
       }
@@ -334,7 +335,8 @@ class GraphBuilder {
 
       std::vector<int64_t> inferred;  // result shape derived from the operands (empty: take the declared one)
       if (node.kind == OpKind::Transpose || node.kind == OpKind::Tile || node.kind == OpKind::Slice ||
-          node.kind == OpKind::StridedSlice || node.kind == OpKind::Pad || node.kind == OpKind::Concat) {
+          node.kind == OpKind::StridedSlice || node.kind == OpKind::Pad || node.kind == OpKind::Concat ||
+          node.kind == OpKind::Gather) {
         inferred = parseDataMovement(&node, attrs, inputDesc, readShape(outputDesc[0]));
       } else if (binding_ != nullptr) {
         inferred = inferResultShape(node, attrs, inputDesc, readShape(outputDesc[0]));
@@ -560,6 +562,30 @@ class GraphBuilder {
         for (size_t d = 0; d < rank; ++d) expect[d] = inShape[d] + node->begin[d] + high[d];
         break;
       }
+      case OpKind::Gather: {
+        // out = data.shape[:axis] + indices.shape + data.shape[axis+1:]; axis from the third input's value or attr
+        // "axis"; batch_dims must be 0 (convertGatherOp :1208-1233, MindSporeToLinalg.cpp:526-594)
+        if (node->inputs.size() != 2) throw TranslateError("op " + nm + ": needs a data and an indices operand");
+        int64_t axis = 0;
+        if (inputDesc.size() > 2 && inputDesc[2][0].contains(kValue)) {
+          const json::Value &v = inputDesc[2][0].at(kValue);
+          axis = v.isArray() ? v.asIntVector().at(0) : static_cast<int64_t>(v.asDouble());
+        } else if (const json::Value *a = findAttr(attrs, kAxis)) {
+          axis = a->isArray() ? a->asIntVector().at(0) : static_cast<int64_t>(a->asDouble());
+        }
+        if (const json::Value *bd = findAttr(attrs, "batch_dims")) {
+          if (bd->asDouble() != 0.0) throw TranslateError("op " + nm + ": batch_dims other than 0 is not supported");
+        }
+        if (axis < 0) axis += static_cast<int64_t>(rank);
+        if (axis < 0 || axis >= static_cast<int64_t>(rank)) throw TranslateError("op " + nm + ": axis out of range");
+        node->concatAxis = axis;
+        const TensorValue &idx = graph_.tensor(node->inputs[1]);
+        if (isFloatType(idx.dtype) || idx.dtype == DType::Bool) throw TranslateError("op " + nm + ": indices must be integers");
+        expect.assign(inShape.begin(), inShape.begin() + axis);
+        expect.insert(expect.end(), idx.shape.begin(), idx.shape.end());
+        expect.insert(expect.end(), inShape.begin() + axis + 1, inShape.end());
+        break;
+      }
       case OpKind::Concat: {
         if (node->inputs.size() != 2) throw TranslateError("op " + nm + ": exactly two operands are supported");
         int64_t axis = 0;
@@ -649,6 +675,7 @@ OperatorTemplate templateOfOp(const OpGraph &g, const OpNode &op) {
     case OpKind::StridedSlice:
     case OpKind::Pad:
     case OpKind::Concat:
+    case OpKind::Gather:
       return OperatorTemplate::Default;  // not classified by getOperatorTemplate (OperatorIdentify.cpp:51-75)
     case OpKind::Unknown:
     case OpKind::Unsupported:
@@ -773,6 +800,7 @@ const char *opKindName(OpKind k) {
     case OpKind::StridedSlice: return "strided_slice";
     case OpKind::Pad: return "pad";
     case OpKind::Concat: return "concat";
+    case OpKind::Gather: return "gather";
     case OpKind::MatMul: return "matmul";
     case OpKind::AddN: return "addn";
     case OpKind::Unsupported: return "unsupported";
@@ -980,7 +1008,7 @@ std::string printOpGraph(const OpGraph &g) {
       os << " {";
       list("low", op.begin);
       os << ", value = " << op.padValue << "}";
-    } else if (op.kind == OpKind::Concat) {
+    } else if (op.kind == OpKind::Concat || op.kind == OpKind::Gather) {
       os << " {axis = " << op.concatAxis << "}";
     }
     if (op.kind == OpKind::Unknown) os << " {ori_op = \"" << op.name << "\"}";

@@ -46,7 +46,7 @@ enum class OpKind {
   // shape
   Reshape, BroadcastTo,
   // data movement: the result is the operand read through an index map
-  Transpose, Tile, Slice, StridedSlice, Pad, Concat,
+  Transpose, Tile, Slice, StridedSlice, Pad, Concat, Gather,
   // contraction
   MatMul,
   // n-ary
@@ -94,7 +94,7 @@ struct OpNode {
   std::vector<int64_t> begin;      // Slice / StridedSlice: first index taken; Pad: elements added in front
   std::vector<int64_t> strides;    // StridedSlice: step (positive); Slice: all ones
   int64_t padValue = 0;            // Pad: the constant written outside the operand
-  int64_t concatAxis = 0;          // Concat: axis along which the operands follow one another
+  int64_t concatAxis = 0;          // Concat: axis along which the operands follow one another; Gather: gathered axis
   std::string ptrAddress;
 };
 

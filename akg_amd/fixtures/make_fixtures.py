@@ -34,6 +34,7 @@ FIXTURES = {
     "small_quant_int8_residual_bf16_37x1544": lambda n: op_desc.quant_int8_residual(37, 1544, "bfloat16", n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", True, n),
+    "small_elemany_greater_f32_9x130": lambda n: op_desc.any_greater(9, 130, 2.5, "ElemAny", n),
     # streaming reductions: direction Y, direction ALL, long rows, multi-output
     "small_reducey_sqsum_f32_1x5100x3072": lambda n: op_desc.square_reduce([1, 5100, 3072], [1], "float32", True, "ReduceSum", n),
     "small_reducey_sqsum_f32_3x37x50": lambda n: op_desc.square_reduce([3, 37, 50], [1], "float32", False, "ReduceSum", n),
@@ -54,6 +55,8 @@ FIXTURES = {
     "small_transpose_bias_add_f32_2x100x200": lambda n: op_desc.transpose_bias_add(2, 100, 200, "float32", n),
     "small_transpose_sum_f32_2x70x3x80_perm0321": lambda n: op_desc.transpose_sum([2, 70, 3, 80], [0, 3, 2, 1], "float32", n),
     "small_transpose_sum_f16_130x66_perm10": lambda n: op_desc.transpose_sum([130, 66], [1, 0], "float16", n),
+    "small_embedding_lookup_bf16_1000x96_ids5x33": lambda n: op_desc.embedding_lookup_scale(1000, 96, 5, 33, "bfloat16", n),
+    "small_embedding_lookup_f32_50x7_ids3x4": lambda n: op_desc.embedding_lookup_scale(50, 7, 3, 4, "float32", n),
     "n3_transpose_bias_add_bf16_32x2048x1024": lambda n: op_desc.transpose_bias_add(32, 2048, 1024, "bfloat16", n),
     # float MatMul + bias + activation on the bfloat16 / float16 MFMA path
     "small_gemm_bf16_bias_gelu_256x512x256": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "float32", n),

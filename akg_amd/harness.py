@@ -44,6 +44,8 @@ def pattern_of(desc):
     names = [o["name"] for o in desc["op_desc"]]
     if "MatMul" in names:
         return "gemm"
+    if "Gather" in names:
+        return "gather"
     if "ReduceMax" in names and "Exp" in names:
         return "softmax"
     if "Rsqrt" in names and "ReduceSum" in names:
@@ -68,6 +70,13 @@ def make_inputs(desc, seed=BASE_SEED, pattern=None):
     for idx, (dt, shape) in enumerate(specs):
         if dt in ("int8", "uint8"):
             out.append(rng.integers(-127, 128, size=shape, dtype=np.int8))
+            continue
+        if dt in ("int16", "int32", "int64") and pattern == "gather":
+            # positions along the gathered axis, a few of them just outside it (those are clamped)
+            op = next(o for o in desc["op_desc"] if o["name"] == "Gather")
+            attrs = {a["name"]: a["value"] for a in (op.get("attr") or [])}
+            extent = op["input_desc"][0][0]["shape"][int(attrs.get("axis", 0))]
+            out.append(rng.integers(-2, extent + 2, size=shape).astype(dt))
             continue
         if dt in ("int16", "int32", "int64"):
             out.append(rng.integers(-100, 101, size=shape).astype(dt))

@@ -416,3 +416,30 @@ def batch_matmul_scale_mask(batch, m, k, n, dtype="bfloat16", transpose_b=True, 
     s = b.op("BatchMatMul", [q, kk], [batch, m, n], "float32", attrs=attrs)
     s = b.add(b.mul(s, b.const(1.0 / (k ** 0.5), "float32")), mask)
     return b.dumps([b.cast(s, dtype)])
+
+
+def gather(b, data, indices, axis):
+    shape = list(data.shape[:axis]) + list(indices.shape) + list(data.shape[axis + 1:])
+    return b.op("Gather", [data, indices], shape, data.dtype,
+                attrs=[{"data_type": "int", "name": "axis", "value": int(axis)},
+                       {"data_type": "int", "name": "batch_dims", "value": 0}])
+
+
+def embedding_lookup_scale(vocab, width, batch, seq, dtype="bfloat16", name=None):
+    """out[b, s, :] = table[ids[b, s], :] * scale + pos[s, :]: an embedding gather fused with its scale and the
+    positional term."""
+    b = DescBuilder(name or "Fused_Gather_Mul_Add_%s_%dx%d_ids%dx%d" % (_SHORT[dtype], vocab, width, batch, seq))
+    table = b.input([vocab, width], dtype)
+    ids = b.input([batch, seq], "int32")
+    pos = b.input([seq, width], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    x = b.add(b.mul(f(gather(b, table, ids, 0)), b.const(float(width) ** 0.5, "float32")), f(pos))
+    return b.dumps([b.cast(x, dtype) if dtype != "float32" else x])
+
+
+def any_greater(rows, cols, threshold=2.5, op="ElemAny", name=None):
+    """out[r] = any(x[r, :] > threshold), spelled with `ElemAny` (the reference maps it to its ReduceAny op)."""
+    b = DescBuilder(name or "Fused_Greater_%s_f32_%dx%d" % (op, rows, cols))
+    x = b.input([rows, cols], "float32")
+    hit = b.binary("Greater", x, b.const(threshold, "float32"), dtype="bool")
+    return b.dumps([b.reduce(op, hit, [1], False)])

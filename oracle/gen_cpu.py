@@ -193,6 +193,8 @@ def parse(desc):
     ops = []
     for od in desc["op_desc"]:
         name = od["name"]
+        if name == "ElemAny":  # same mindspore op as ReduceAny (TranslateToMindsporeDialect.cpp:463)
+            name = "ReduceAny"
         attrs = {a["name"]: a["value"] for a in (od.get("attr") or [])}
         ins = []
         for idx, entry in enumerate(od["input_desc"]):
@@ -201,6 +203,8 @@ def parse(desc):
             if name == "Cast" and idx > 0:
                 continue
             if name == "StridedSlice" and idx > 0:
+                continue
+            if name == "Gather" and idx > 1:
                 continue
             d = entry[0]
             if d["tensor_name"] in tensors:
@@ -514,6 +518,13 @@ class Emitter:
             else:
                 fill = "((%s)%dLL)" % (C_COMPUTE[out.dtype], vp["value"])
             value = "((%s) ? %s : %s)" % (cond, inner, fill)
+        elif n == "Gather":
+            ind, a = op.inputs[1], vp["axis"]
+            nind = len(ind.shape)
+            pos = load(ind, idx[a:a + nind])
+            hi = src.shape[a] - 1
+            clamped = "((%s) < 0 ? 0 : ((%s) > %dL ? %dL : (int64_t)(%s)))" % (pos, pos, hi, hi, pos)
+            value = load(src, idx[:a] + [clamped] + idx[a + nind:])
         else:
             other, a = op.inputs[1], vp["axis"]
             if other.const is not None or other.dtype != out.dtype:

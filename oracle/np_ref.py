@@ -171,6 +171,8 @@ def evaluate(desc, inputs):
         dtypes[d["tensor_name"]] = dt
     for od in desc["op_desc"]:
         name = od["name"]
+        if name == "ElemAny":  # same mindspore op as ReduceAny (TranslateToMindsporeDialect.cpp:463)
+            name = "ReduceAny"
         attrs = {a["name"]: a["value"] for a in (od.get("attr") or [])}
         ins, in_dt = [], []
         for idx, entry in enumerate(od["input_desc"]):
@@ -179,6 +181,8 @@ def evaluate(desc, inputs):
             if name == "Cast" and idx > 0:
                 continue
             if name == "StridedSlice" and idx > 0:
+                continue
+            if name == "Gather" and idx > 1:
                 continue
             d = entry[0]
             tn = d["tensor_name"]
@@ -319,6 +323,8 @@ def evaluate(desc, inputs):
                 elif name == "Pad":
                     fill = np.asarray(vp["value"]).astype(x.dtype)
                     res = np.pad(x, list(zip(vp["low"], vp["high"])), mode="constant", constant_values=fill)
+                elif name == "Gather":
+                    res = np.take(x, ins[1].astype(np.int64), axis=vp["axis"], mode="clip")
                 else:
                     res = np.concatenate([x, ins[1]], axis=vp["axis"])
                 res = np.ascontiguousarray(res)

@@ -14,9 +14,13 @@ Rules followed (reference file:line):
                 ...; attr "value" (integer), constant mode (MindSporeToTosa.cpp:305-376)
   Concat        two operands, attr "axis" (default 0) (TranslateToMindsporeDialect.cpp:1117-1124,
                 MindSporeToTosa.cpp:46-58)
+  Gather        data, integer indices, axis from a third constant input or attr "axis", batch_dims 0; result shape
+                data[:axis] + indices + data[axis+1:], element = data[..., indices[...], ...]
+                (TranslateToMindsporeDialect.cpp:1208-1233, MindSporeToLinalg.cpp:526-594). Out-of-range positions are
+                undefined in the reference (tensor.extract); both restatements and the kernels clamp them into the axis.
 """
 
-VIEW_OPS = ("Transpose", "Tile", "Slice", "StridedSlice", "Pad", "Concat")
+VIEW_OPS = ("Transpose", "Tile", "Slice", "StridedSlice", "Pad", "Concat", "Gather")
 
 
 def _ints(v):
@@ -68,5 +72,14 @@ def view_params(od, in_shape):
     if name == "Concat":
         axis = attrs.get("axis", 0)
         axis = int(axis[0] if isinstance(axis, list) else axis)
+        return {"axis": axis + rank if axis < 0 else axis}
+    if name == "Gather":
+        ins = od["input_desc"]
+        if len(ins) > 2 and "value" in ins[2][0]:
+            axis = ins[2][0]["value"]
+        else:
+            axis = attrs.get("axis", 0)
+        axis = int(axis[0] if isinstance(axis, list) else axis)
+        assert int(attrs.get("batch_dims", 0)) == 0, "batch_dims other than 0 is not restated"
         return {"axis": axis + rank if axis < 0 else axis}
     raise ValueError("not a data-movement op: %s" % name)

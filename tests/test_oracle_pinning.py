@@ -356,6 +356,24 @@ def test_bf16_matmul_bias_gelu_matches_torch_float64():
     assert np.allclose(harness.bf16_bits_to_f32(c_out[0]).astype(np.float64), ref, rtol=1e-2, atol=1e-3)
 
 
+def test_gather_takes_rows_by_index_and_clamps(tmp_path):
+    """Gather along axis 1 of a rank-3 tensor with rank-2 indices: result shape data[:1] + indices + data[2:], written
+    out element by element; positions outside the axis are clamped (undefined in the reference)."""
+    b = op_desc.DescBuilder("pin_gather_axis1")
+    data = b.input([2, 5, 3], "int32")
+    ind = b.input([2, 2], "int32")
+    text = b.dumps([op_desc.gather(b, data, ind, 1)])
+    x = np.arange(30, dtype=np.int32).reshape(2, 5, 3)
+    idx = np.array([[4, 0], [7, -1]], dtype=np.int32)
+    _, c_out, n_out = build_and_run(text, [x, idx], tmp_path)
+    assert c_out[0].shape == (2, 2, 2, 3)
+    for i in range(2):
+        for j in range(2):
+            for k in range(2):
+                row = min(max(int(idx[j, k]), 0), 4)
+                assert np.array_equal(c_out[0][i, j, k], x[i, row]) and np.array_equal(n_out[0][i, j, k], x[i, row])
+
+
 def test_batch_matmul_is_one_product_per_batch_index():
     """BatchMatMul against torch float64 bmm: batches must not mix and transpose_b must read [batch, n, k]."""
     import torch
