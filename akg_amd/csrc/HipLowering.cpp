@@ -278,6 +278,10 @@ std::vector<bool> relaxedPrecisionTensors(const OpGraph &g) {
           inDemand = 1;
         }
         break;
+      case OpKind::Assign:
+        // the value also lands in the destination buffer: a float32 / integer destination needs it exact
+        if (!(od == DType::F16 || od == DType::BF16)) inDemand = 2;
+        break;
       case OpKind::Equal: case OpKind::NotEqual: case OpKind::Greater: case OpKind::GreaterEqual:
       case OpKind::Less: case OpKind::LessEqual: case OpKind::Floor: case OpKind::IsNan: case OpKind::IsInf:
       case OpKind::IsFinite: case OpKind::LogicalNot: case OpKind::LogicalAnd: case OpKind::LogicalOr:
@@ -429,6 +433,9 @@ std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vecto
     case OpKind::BroadcastTo:
       need(1);
       return conv(0);
+    case OpKind::Assign:
+      need(2);
+      return conv(1);  // the value; the store over the destination is the emitter's job
     default:
       break;
   }
@@ -857,8 +864,12 @@ class TileEmitter {
     line("");
     src_ << "extern \"C\" __global__ __launch_bounds__(" << block_ << ") void " << kname << "(";
     size_t argc = 0;
+    std::vector<bool> assigned(g_.inputs.size(), false);
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::Assign) assigned[static_cast<size_t>(g_.tensor(op.inputs[0]).inputIndex)] = true;
+    }
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
-      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+      src_ << (argc ? ", " : "") << (assigned[i] ? "" : "const ") << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
@@ -957,8 +968,12 @@ class TileEmitter {
         emitElementwise(op, clampCast_[k]);
       }
     }
-    // stores
+    // stores: the outputs, then the destinations of Assign ops (every thread has read its part of a destination
+    // into registers above, and writes exactly the positions it read)
     for (size_t i = 0; i < g_.outputs.size(); ++i) emitOutputStore(i);
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::Assign) emitAssignStore(op);
+    }
     line("}");
   }
 
@@ -1153,6 +1168,26 @@ class TileEmitter {
     v.ident = nm.str();
     const TensorValue &outT = g_.tensor(outId);
     v.rowvecNoKeep = outT.numel() != 1 && !outT.shape.empty() && outT.shape.back() != 1;
+  }
+
+  void emitAssignStore(const OpNode &op) {
+    const TensorValue &dst = g_.tensor(op.inputs[0]);
+    const int valueId = op.outputs[0];
+    const ValInfo &v = vals_[static_cast<size_t>(valueId)];
+    if (!v.defined) throw LoweringError("op " + op.name + ": value is never computed");
+    if (dst.numel() != numel_ || v.rank != ValRank::Tile) {
+      throw LoweringError("op " + op.name + ": only destinations as large as the kernel's iteration space are supported");
+    }
+    const std::string tag = tagOf(valueId);
+    line("#pragma unroll");
+    line("  for (int j = 0; j < NCHUNK; ++j) {");
+    std::string guard = "akg_ok[j]";
+    if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
+    const std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
+    src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (nonTemporal_ ? "true" : "false") << ">("
+         << memRef("in" + std::to_string(dst.inputIndex), offset) << ", " << v.ident << "[j]);  // " << op.name << " -> "
+         << dst.name << "\n";
+    line("  }");
   }
 
   void emitOutputStore(size_t i) {

@@ -99,7 +99,7 @@ class GemmEmitter {
         matmulOp_ = static_cast<int>(i);
       } else if (op.kind == OpKind::Unknown) {
         throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
-      } else if (op.kind == OpKind::Unsupported || lowering::isReduceKind(op.kind)) {
+      } else if (op.kind == OpKind::Unsupported || op.kind == OpKind::Assign || lowering::isReduceKind(op.kind)) {
         throw LoweringError("op " + op.name + " cannot be fused into a MatMul epilogue yet");
       }
     }

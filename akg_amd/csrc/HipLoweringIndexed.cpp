@@ -95,6 +95,7 @@ class IndexedEmitter {
         throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
       }
       if (op.kind == OpKind::Unsupported) throw LoweringError("op " + op.name + " has no kernel family yet");
+      if (op.kind == OpKind::Assign) throw LoweringError("op " + op.name + " has no lowering in the indexed family yet");
       if (op.kind == OpKind::MatMul || lowering::isReduceKind(op.kind)) {
         throw LoweringError("op " + op.name + " cannot be fused with data-movement ops (Transpose, Tile, Slice, Pad, "
                             "Concat) in one kernel yet");

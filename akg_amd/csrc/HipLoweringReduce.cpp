@@ -123,6 +123,7 @@ class StreamReduceEmitter {
         throw LoweringError("op " + op.name + " cannot be fused into a streaming reduction");
       }
       if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
+      if (op.kind == OpKind::Assign) throw LoweringError("op " + op.name + " has no lowering in the streaming-reduction family yet");
       if (lowering::isReduceKind(op.kind)) reduces_.push_back(&op);
     }
     if (reduces_.empty()) throw LoweringError("internal: no reduction");

@@ -91,8 +91,8 @@ const OpTableEntry kOpTable[] = {
   {"Split", OpKind::Unsupported},
   {"Pad", OpKind::Pad},
   {"Gather", OpKind::Gather},
-  {"InplaceAssign", OpKind::Unsupported},
-  {"Assign", OpKind::Unsupported},
+  {"InplaceAssign", OpKind::Assign},
+  {"Assign", OpKind::Assign},
   {"UnsortedSegmentSum", OpKind::Unsupported},
   {"StridedSlice", OpKind::StridedSlice},
   {"AddN", OpKind::AddN},
@@ -273,9 +273,11 @@ class GraphBuilder {
       static const json::Value kNoAttrs;
       const json::Value &attrs = (opDesc.contains(kAttr) && opDesc.at(kAttr).isArray()) ? opDesc.at(kAttr) : kNoAttrs;
       checkAttrTypes(attrs, node.name);
+      bool fakeOutput = false;
       if (const json::Value *fake = findAttr(attrs, "fake_output")) {
-        if (fake->isBool() && fake->asBool()) {
-          throw TranslateError("op " + node.name + ": fake_output (in-place aliasing) is not supported");
+        fakeOutput = fake->isBool() && fake->asBool();
+        if (fakeOutput && node.kind != OpKind::Assign) {
+          throw TranslateError("op " + node.name + ": fake_output is only meaningful on Assign / InplaceAssign");
         }
       }
       if (opDesc.contains(kPtrAddress) && opDesc.at(kPtrAddress).isString()) {
@@ -300,6 +302,7 @@ class GraphBuilder {
           if (node.kind == OpKind::Cast && j > 0) continue;  // convertCastOp keeps the first operand only (:1351-1360)
           if (node.kind == OpKind::StridedSlice && j > 0) continue;  // begin / end / strides carried as constants
           if (node.kind == OpKind::Gather && j > 1) continue;        // the axis carried as a constant
+          if (node.kind == OpKind::Assign && j > 1) continue;        // convertInplaceAssignOp keeps two operands (:1104-1115)
           node.inputs.push_back(operandFor(inputDesc[j][0], node.name));
         }
       }
@@ -333,6 +336,16 @@ class GraphBuilder {
         if (const json::Value *b = findAttr(attrs, kTransposeB)) node.transposeB = b->asBool();
       }
 
+      if (node.kind == OpKind::Assign) {
+        if (node.inputs.size() != 2) throw TranslateError("op " + node.name + ": needs a destination and a value operand");
+        const TensorValue &dst = graph_.tensor(node.inputs[0]);
+        const TensorValue &src = graph_.tensor(node.inputs[1]);
+        if (dst.inputIndex < 0) throw TranslateError("op " + node.name + ": the destination must be a kernel input");
+        if (dst.dtype != src.dtype || dst.numel() != src.numel()) {
+          throw TranslateError("op " + node.name + ": destination and value differ in type or size");
+        }
+      }
+      (void)fakeOutput;
       std::vector<int64_t> inferred;  // result shape derived from the operands (empty: take the declared one)
       if (node.kind == OpKind::Transpose || node.kind == OpKind::Tile || node.kind == OpKind::Slice ||
           node.kind == OpKind::StridedSlice || node.kind == OpKind::Pad || node.kind == OpKind::Concat ||
@@ -351,6 +364,7 @@ class GraphBuilder {
         bool dynamic = false;
         for (int64_t e : shape) dynamic = dynamic || e < 0;
         if (dynamic && binding_ != nullptr && j == 0 && !inferred.empty()) shape = inferred;
+        if (node.kind == OpKind::Assign) shape = graph_.tensor(node.inputs[0]).shape;  // (:359-364, :398-404)
         int id = addTensor(tensorName, dtype, shape);
         graph_.tensors[static_cast<size_t>(id)].producer = opIndex;
         node.outputs.push_back(id);
@@ -637,7 +651,10 @@ class GraphBuilder {
         n *= d;
         dynamic = dynamic || d < 0;
       }
-      if (dynamic && binding_ != nullptr) {
+      const bool assigned = t.producer >= 0 && graph_.ops[static_cast<size_t>(t.producer)].kind == OpKind::Assign;
+      if (assigned) {
+        // a fake output: its declared shape is not binding, the destination's is (:398-404)
+      } else if (dynamic && binding_ != nullptr) {
         if (shape.size() != t.shape.size()) throw TranslateError("output " + tensorName + ": rank differs from its producer");
       } else if (n != t.numel()) {
         throw TranslateError("output " + tensorName + ": shape differs between output_desc and its producer");
@@ -803,6 +820,7 @@ const char *opKindName(OpKind k) {
     case OpKind::Gather: return "gather";
     case OpKind::MatMul: return "matmul";
     case OpKind::AddN: return "addn";
+    case OpKind::Assign: return "inplace_assign";
     case OpKind::Unsupported: return "unsupported";
     case OpKind::Unknown: return "unknown";
   }
@@ -882,7 +900,8 @@ void pruneDeadOps(OpGraph *graph) {
   std::vector<bool> keep(graph->ops.size(), false);
   for (size_t k = graph->ops.size(); k-- > 0;) {
     const OpNode &op = graph->ops[k];
-    bool needed = op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported;  // keep what must be reported
+    // keep what must be reported, and what has a side effect
+    bool needed = op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported || op.kind == OpKind::Assign;
     for (int out : op.outputs) needed = needed || live[static_cast<size_t>(out)];
     if (!needed) continue;
     keep[k] = true;

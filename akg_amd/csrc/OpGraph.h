@@ -51,6 +51,9 @@ enum class OpKind {
   MatMul,
   // n-ary
   AddN,
+  // Assign / InplaceAssign: the result is the second operand; as a side effect it is also written over the first
+  // operand, which must be a kernel input (linalg.copy ins=input1 outs=input0, MindSporeToLinalg.cpp:495-524)
+  Assign,
   // anything in the reference's factory that this backend has no kernel family for, and names outside the
   // factory (the reference turns those into mindspore.unknown, :874-876,939-946)
   Unsupported,

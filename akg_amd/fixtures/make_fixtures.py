@@ -34,6 +34,8 @@ FIXTURES = {
     "small_quant_int8_residual_bf16_37x1544": lambda n: op_desc.quant_int8_residual(37, 1544, "bfloat16", n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", True, n),
+    "small_momentum_update_f32_37x130": lambda n: op_desc.momentum_update(37, 130, "float32", name=n),
+    "small_momentum_update_bf16_64x256": lambda n: op_desc.momentum_update(64, 256, "bfloat16", name=n),
     "small_elemany_greater_f32_9x130": lambda n: op_desc.any_greater(9, 130, 2.5, "ElemAny", n),
     # streaming reductions: direction Y, direction ALL, long rows, multi-output
     "small_reducey_sqsum_f32_1x5100x3072": lambda n: op_desc.square_reduce([1, 5100, 3072], [1], "float32", True, "ReduceSum", n),

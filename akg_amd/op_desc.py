@@ -443,3 +443,20 @@ def any_greater(rows, cols, threshold=2.5, op="ElemAny", name=None):
     x = b.input([rows, cols], "float32")
     hit = b.binary("Greater", x, b.const(threshold, "float32"), dtype="bool")
     return b.dumps([b.reduce(op, hit, [1], False)])
+
+
+def momentum_update(rows, cols, dtype="float32", lr=0.01, mu=0.9, name=None):
+    """SGD with momentum, in place: v <- mu * v + g (Assign), p <- p - lr * v (Assign). Kernel inputs p, v, g; the two
+    Assign results are the (fake) outputs."""
+    b = DescBuilder(name or "Fused_Mul_Add_Assign_Mul_Sub_Assign_%s_%dx%d" % (_SHORT[dtype], rows, cols))
+    p = b.input([rows, cols], dtype)
+    v = b.input([rows, cols], dtype)
+    g = b.input([rows, cols], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    back = (lambda t: b.cast(t, dtype)) if dtype != "float32" else (lambda t: t)
+    v_new = b.add(b.mul(f(v), b.const(mu, "float32")), f(g))
+    v_out = b.op("Assign", [v, back(v_new)], [rows, cols], dtype)
+    p_new = b.sub(f(p), b.mul(v_new, b.const(lr, "float32")))
+    p_out = b.op("InplaceAssign", [p, back(p_new), back(v_new)], [rows, cols], dtype,
+                 attrs=[{"data_type": "bool", "name": "fake_output", "value": True}])
+    return b.dumps([v_out, p_out])

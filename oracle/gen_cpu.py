@@ -56,6 +56,10 @@ UNARY_MATH = {"Exp": "exp", "Log": "log", "Tanh": "tanh", "Sqrt": "sqrt", "Floor
               "ASin": "asin", "ACos": "acos", "Atan": "atan", "Asinh": "asinh", "Acosh": "acosh"}
 COMPARE = {"Equal": "==", "NotEqual": "!=", "Greater": ">", "GreaterEqual": ">=", "Less": "<", "LessEqual": "<="}
 MATMULS = ("MatMul", "BatchMatMul")
+# Assign / InplaceAssign: linalg.copy ins=input1 outs=input0 (MindSporeToLinalg.cpp:495-524): the value is written over
+# the first operand's buffer (a kernel input) and is also the op's result; the result has the destination's shape
+# (TranslateToMindsporeDialect.cpp:359-364,398-404)
+ASSIGNS = ("Assign", "InplaceAssign")
 REDUCES = ("ReduceSum", "ReduceMax", "ReduceMin", "ReducePrd", "ReduceAll", "ReduceAny")
 ATTR_AS_INPUT = ("Reshape", "BroadcastTo", "ReduceMax", "ReduceMin", "ReduceSum", "ReducePrd", "ReduceAll", "ReduceAny",
                  "ArgMax", "Transpose", "Tile")
@@ -206,6 +210,8 @@ def parse(desc):
                 continue
             if name == "Gather" and idx > 1:
                 continue
+            if name in ASSIGNS and idx > 1:
+                continue
             d = entry[0]
             if d["tensor_name"] in tensors:
                 ins.append(tensors[d["tensor_name"]])
@@ -222,7 +228,7 @@ def parse(desc):
             tensors[c.name] = c
             ins.append(c)
         o = od["output_desc"][0]
-        out = T(o["tensor_name"], o.get("shape", [1]), o["data_type"])
+        out = T(o["tensor_name"], ins[0].shape if name in ASSIGNS else o.get("shape", [1]), o["data_type"])
         op = Op(name, ins, out, attrs)
         if name in VIEW_OPS:
             op.view = view_params(od, ins[0].shape)
@@ -277,7 +283,7 @@ class Emitter:
 
     # -- which values live in memory --------------------------------------------------------------------
     def is_elementwise(self, op):
-        return op.name not in REDUCES and op.name not in MATMULS + ("Reshape",) and op.name not in VIEW_OPS
+        return op.name not in REDUCES and op.name not in MATMULS + ("Reshape",) and op.name not in VIEW_OPS + ASSIGNS
 
     def plan(self):
         consumers = {}
@@ -478,6 +484,19 @@ class Emitter:
         depth = self.open_loops(shape, True)
         expr = self.op_expr(op, shape)
         self.emit("%s[%s] = %s;" % (out.buffer, self.index_expr(out, shape), self.store_expr(out.dtype, expr)), depth)
+        self.close_loops(len(shape), depth)
+
+    def emit_assign(self, op):
+        dst, src, out = op.inputs[0], op.inputs[1], op.output
+        if not dst.is_input or dst.dtype != out.dtype:
+            raise OracleError("%s: the destination must be a kernel input of the value's type" % op.name)
+        shape = dst.shape
+        depth = self.open_loops(shape, True)
+        value = self.value_expr(src, shape)
+        self.emit("const %s v = %s;" % (C_STORAGE[out.dtype], self.store_expr(out.dtype, value)), depth)
+        idx = self.index_expr(dst, shape)
+        self.emit("((%s *)%s)[%s] = v;" % (C_STORAGE[dst.dtype], dst.buffer, idx), depth)
+        self.emit("%s[%s] = v;" % (out.buffer, idx), depth)
         self.close_loops(len(shape), depth)
 
     def emit_view(self, op):
@@ -684,6 +703,8 @@ class Emitter:
                 self.emit_matmul(op)
             elif op.name in VIEW_OPS:
                 self.emit_view(op)
+            elif op.name in ASSIGNS:
+                self.emit_assign(op)
             else:
                 self.emit_elementwise(op)
         for b in self.temps:

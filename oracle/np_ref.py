@@ -153,9 +153,10 @@ def matmul_exact_i32(a, b):
     return acc.astype(np.int32)   # two's complement wrap, as i32 accumulation would
 
 
-def evaluate(desc, inputs):
+def evaluate(desc, inputs, updates=None):
     """Evaluate the description on `inputs` (list of external arrays in input_desc order); returns the list of
-    external output arrays in output_desc order."""
+    external output arrays in output_desc order. Assign / InplaceAssign overwrite a kernel input: pass a dict as
+    `updates` to receive {input position: new external array} (the caller's arrays are left alone)."""
     if isinstance(desc, str):
         desc = json.loads(desc)
     env = {}
@@ -183,6 +184,8 @@ def evaluate(desc, inputs):
             if name == "StridedSlice" and idx > 0:
                 continue
             if name == "Gather" and idx > 1:
+                continue
+            if name in ("Assign", "InplaceAssign") and idx > 1:
                 continue
             d = entry[0]
             tn = d["tensor_name"]
@@ -328,6 +331,15 @@ def evaluate(desc, inputs):
                 else:
                     res = np.concatenate([x, ins[1]], axis=vp["axis"])
                 res = np.ascontiguousarray(res)
+            elif name in ("Assign", "InplaceAssign"):
+                # linalg.copy ins=input1 outs=input0 (MindSporeToLinalg.cpp:495-524)
+                dst_name = od["input_desc"][0][0]["tensor_name"]
+                res = np.array(ins[1]).reshape(ins[0].shape)
+                env[dst_name] = res
+                oshape = list(ins[0].shape)
+                if updates is not None:
+                    pos = [e[0]["tensor_name"] for e in desc["input_desc"]].index(dst_name)
+                    updates[pos] = to_external(res, odt).reshape(ins[0].shape)
             elif name in ("MatMul", "BatchMatMul"):
                 if attrs.get("transpose_a", False):
                     raise ValueError("TransposeA is not supported")

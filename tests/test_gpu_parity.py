@@ -196,6 +196,38 @@ def test_reference_dynamic_shape_softmax_specialised_per_shape(shapes):
     assert np.allclose(got.sum(axis=3), 1.0, atol=1e-5)
 
 
+@pytest.mark.parametrize("name", ["small_momentum_update_f32_37x130", "small_momentum_update_bf16_64x256"])
+def test_assign_overwrites_its_destination_inputs(name):
+    """Assign / InplaceAssign write their value over a kernel INPUT (the momentum and the parameter of an optimizer
+    step) besides returning it: the device copies of those inputs must hold the oracle's updated values afterwards, the
+    untouched input must be unchanged, and a second launch must apply a second step."""
+    import torch
+    path = os.path.join(FIXTURES, name + ".info")
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 700)
+    dev = torch.device("cuda:0")
+    ins = [_torch_view(a.copy()).to(dev) for a in inputs]
+    outs = [torch.empty(d.nbytes, dtype=torch.uint8, device=dev) for d in kernel.outputs]
+    oracle = cpu_ref.CpuKernel(path)
+    host = [a.copy() for a in inputs]
+    for step in range(2):
+        kernel.launch(ins + outs)
+        torch.cuda.synchronize()
+        expect_out = oracle(host)                       # updates host[0] (parameter) and host[1] (momentum) in place
+        for d, o, e in zip(kernel.outputs, outs, expect_out):
+            got = o.cpu().numpy().view(driver.NP_HOST_DTYPE[d.dtype]).reshape(d.shape)
+            ok, msg = harness.compare(got, e, d.dtype)
+            assert ok, "step %d output %s: %s" % (step, d.name, msg)
+        for i, (t, h) in enumerate(zip(ins, host)):
+            got = t.cpu().numpy().view(h.dtype).reshape(h.shape)
+            ok, msg = harness.compare(got, h, desc["input_desc"][i][0]["data_type"])
+            print("  step %d input %d: %s" % (step, i, msg), flush=True)
+            assert ok, "step %d input %d: %s" % (step, i, msg)
+        assert np.array_equal(host[2], inputs[2])       # the gradient is only read
+    assert not np.array_equal(host[0], inputs[0]) and not np.array_equal(host[1], inputs[1])
+
+
 def test_float32_tanh_accuracy_over_the_whole_range():
     """The float32 tanh of the device op library is an own implementation (series below 0.25, hardware exp2 and
     reciprocal above): its error against the float64 value is measured on 8M arguments, dense around the branch

@@ -125,7 +125,7 @@ def run_fixture_both(name, seed):
     path = os.path.join(FIXTURES, name + ".info")
     desc = harness.load_desc(path)
     inputs = harness.make_inputs(desc, seed=seed)
-    c_out = cpu_ref.CpuKernel(path)(inputs)
+    c_out = cpu_ref.CpuKernel(path)([a.copy() for a in inputs])   # Assign ops overwrite their destination input
     n_out = np_ref.evaluate(desc, inputs)
     return desc, inputs, c_out, n_out
 
@@ -372,6 +372,24 @@ def test_gather_takes_rows_by_index_and_clamps(tmp_path):
             for k in range(2):
                 row = min(max(int(idx[j, k]), 0), 4)
                 assert np.array_equal(c_out[0][i, j, k], x[i, row]) and np.array_equal(n_out[0][i, j, k], x[i, row])
+
+
+def test_assign_writes_the_value_over_its_first_operand(tmp_path):
+    """Momentum step in float32 against the formula written out in numpy: v <- 0.9 v + g, p <- p - 0.01 v. The C
+    restatement updates the caller's input arrays in place, the numpy one reports the updates."""
+    text = op_desc.momentum_update(5, 9, "float32", name="pin_momentum")
+    rng = np.random.default_rng(5)
+    p0, v0, g0 = (rng.standard_normal((5, 9), dtype=np.float32) for _ in range(3))
+    ins = [p0.copy(), v0.copy(), g0.copy()]
+    updates = {}
+    n_out = np_ref.evaluate(json.loads(text), [p0, v0, g0], updates)
+    _, c_out, _ = build_and_run(text, ins, tmp_path)
+    v1 = (np.float32(0.9) * v0 + g0).astype(np.float32)
+    p1 = (p0 - np.float32(0.01) * v1).astype(np.float32)
+    assert np.array_equal(ins[1], v1) and np.array_equal(ins[0], p1) and np.array_equal(ins[2], g0)
+    assert np.array_equal(updates[1], v1) and np.array_equal(updates[0], p1) and sorted(updates) == [0, 1]
+    assert np.array_equal(c_out[0], v1) and np.array_equal(c_out[1], p1)
+    assert np.array_equal(n_out[0], v1) and np.array_equal(n_out[1], p1)
 
 
 def test_batch_matmul_is_one_product_per_batch_index():
