@@ -11,6 +11,14 @@
  * index the ops in between map it to, down to scalar loads of the kernel inputs. Nothing intermediate touches
  * memory and a value needed twice at the same index is computed once. Outputs are stored as V-element chunks.
  *
+ * Vector loads. Every index component carries how it varies over the V elements of a thread's chunk: not at all,
+ * as `u + e` with a chunk-uniform `u` (and whether `u` is a multiple of V), or arbitrarily. Slices, pads, concats and
+ * tiles whose offsets and extents are multiples of V keep the second form, conditions on such components hold for
+ * the whole chunk or for none of it, and a kernel input whose innermost index has that form (all other components
+ * uniform, every enclosing condition chunk-uniform) is read once per chunk with one 16-byte load placed in front of
+ * the element loop. Index loads of a Gather whose position is chunk-uniform are placed there too, so an embedding
+ * lookup reads its table rows with vector loads. Anything else falls back to scalar loads inside the element loop.
+ *
  * Transposed kernel inputs. Pulled element by element, the reads of a transposed operand are strided across a
  * wavefront (measured 11 % of the HBM peak on a [32,2048,1024] bfloat16 transpose). When a kernel input X goes
  * through a Transpose that moves its innermost axis, and the result has the shape of the outputs, the kernel is
@@ -59,7 +67,32 @@ class IndexedEmitter {
 
  private:
   static constexpr int kBlock = 256;
-  typedef std::vector<std::string> Index;  // one C expression per dimension
+  // One component of a tensor index at the element a thread is working on.
+  struct Ix {
+    std::string s;         // C expression for the current element
+    int kind = 0;          // 0: same for all V elements of the chunk; 1: u + e; 2: anything else
+    std::string u;         // kind 1: the chunk-uniform part
+    bool aligned = false;  // kind 1: u is known to be a multiple of V
+    bool early = true;     // kind 0 (s) / kind 1 (u): only uses variables that exist in front of the element loop
+    Ix() : s("0") {}
+    Ix(const std::string &text, bool isEarly = true) : s(text), early(isEarly) {}  // NOLINT(runtime/explicit)
+    Ix(const char *text) : s(text) {}                                             // NOLINT(runtime/explicit)
+    bool operator==(const Ix &o) const { return s == o.s; }
+    bool operator!=(const Ix &o) const { return s != o.s; }
+  };
+  typedef std::vector<Ix> Index;  // one component per dimension
+  static Ix affine(const std::string &u, bool aligned, bool early) {
+    Ix x("(" + u + " + e)", early);
+    x.kind = 1;
+    x.u = u;
+    x.aligned = aligned;
+    return x;
+  }
+  static Ix perElement(const std::string &text) {
+    Ix x(text, false);
+    x.kind = 2;
+    return x;
+  }
 
   const OpGraph &g_;
   LoweringOptions opt_;
@@ -83,10 +116,23 @@ class IndexedEmitter {
   int indent_ = 2;
   // values already computed in the scopes that are open: (tensor id, index text) -> variable
   std::vector<std::map<std::string, std::string>> scopes_;
+  // Statements go to `src_` until the element loop is opened; its body is collected in `body_` and statements that
+  // belong in front of it (chunk-wide loads, chunk-uniform gather positions) in `hoist_`.
+  std::ostringstream body_, hoist_;
+  std::ostringstream *out_ = &src_;
+  int hoistIndent_ = 1;
+  bool inLoop_ = false;
+  struct Cond {
+    std::string chunkText;  // the condition for the whole chunk, if uniform
+    bool uniformEarly;      // holds for all V elements or none, and can be evaluated in front of the loop
+  };
+  std::vector<Cond> conds_;
+  std::map<std::string, std::string> hoistedLoads_;  // (input, chunk offset, guard) -> array
 
   std::string ctOf(int id) const { return computeTypeName(g_.tensor(id).dtype); }
   std::string tagOf(int id) const { return dtypeTag(g_.tensor(id).dtype); }
-  void stmt(const std::string &s) { src_ << std::string(static_cast<size_t>(indent_) * 2, ' ') << s << "\n"; }
+  void stmt(const std::string &s) { *out_ << std::string(static_cast<size_t>(indent_) * 2, ' ') << s << "\n"; }
+  void hoisted(const std::string &s) { hoist_ << std::string(static_cast<size_t>(hoistIndent_) * 2, ' ') << s << "\n"; }
   std::string fresh(const char *prefix) { return prefix + std::to_string(nextTemp_++); }
 
   void analyse() {
@@ -177,26 +223,31 @@ class IndexedEmitter {
     std::string e;
     for (size_t d = 0; d < shape.size(); ++d) {
       if (shape[d] == 1) continue;  // the index of a unit dimension is 0
-      e = e.empty() ? idx[d] : "(" + e + ") * " + std::to_string(shape[d]) + " + " + idx[d];
+      e = e.empty() ? idx[d].s : "(" + e + ") * " + std::to_string(shape[d]) + " + " + idx[d].s;
     }
     return e.empty() ? "0" : e;
   }
 
-  // Index of `linear` (a C expression) in a dense tensor of `shape`.
-  Index delinearize(const std::string &linear, const std::vector<int64_t> &shape) {
+  // Index of `linear` (a C expression) in a dense tensor of `shape`. `early`: the expression only uses variables that
+  // exist in front of the element loop, so the temporary can be defined there.
+  Index delinearize(const std::string &linear, const std::vector<int64_t> &shape, bool uniform = true, bool early = true) {
     const std::string base = fresh("l");
-    stmt("const int " + base + " = " + linear + ";");
+    const bool hoist = inLoop_ && uniform && early;
+    if (hoist) {
+      hoisted("const int " + base + " = " + linear + ";");
+    } else {
+      stmt("const int " + base + " = " + linear + ";");
+    }
+    const bool resultEarly = !inLoop_ || hoist;
     Index out(shape.size());
     int64_t inner = 1;
     for (size_t d = shape.size(); d-- > 0;) {
-      if (shape[d] == 1) {
-        out[d] = "0";
-      } else {
+      if (shape[d] != 1) {
         std::string e = inner == 1 ? base : "(" + base + " / " + std::to_string(inner) + ")";
         int64_t outer = 1;
         for (size_t k = 0; k < d; ++k) outer *= shape[k];
         if (outer != 1) e = "(" + e + " % " + std::to_string(shape[d]) + ")";
-        out[d] = e;
+        out[d] = uniform ? Ix(e, resultEarly) : perElement(e);
       }
       inner *= shape[d];
     }
@@ -210,7 +261,7 @@ class IndexedEmitter {
     while (in.size() > outShape.size() && in.front() == 1) in.erase(in.begin());
     if (in.size() > outShape.size()) throw LoweringError(what + ": operand rank exceeds the result's");
     const size_t off = outShape.size() - in.size();
-    Index out(inShape.size(), "0");
+    Index out(inShape.size());
     const size_t lead = inShape.size() - in.size();
     for (size_t d = 0; d < in.size(); ++d) {
       if (in[d] == 1) continue;
@@ -220,9 +271,40 @@ class IndexedEmitter {
     return out;
   }
 
+  // idx + delta (delta a compile-time constant), keeping the chunk form where it survives
+  Ix shifted(const Ix &x, int64_t delta) const {
+    if (delta == 0) return x;
+    const std::string d = delta > 0 ? " + " + std::to_string(delta) : " - " + std::to_string(-delta);
+    if (x.kind == 0) return Ix("(" + x.s + d + ")", x.early);
+    if (x.kind == 1) return affine("(" + x.u + d + ")", x.aligned && (delta % vec_) == 0, x.early);
+    return perElement("(" + x.s + d + ")");
+  }
+
+  // `x` compared against the half-open range [0, extent): per-element text, and whether it is one answer per chunk
+  Cond rangeCond(const Ix &x, int64_t extent, std::string *text) const {
+    *text = "static_cast<unsigned>(" + x.s + ") < " + std::to_string(extent) + "u";
+    if (x.kind == 0) return Cond{*text, x.early};
+    if (x.kind == 1 && x.aligned && (extent % vec_) == 0) {
+      return Cond{"static_cast<unsigned>(" + x.u + ") < " + std::to_string(extent) + "u", x.early};
+    }
+    return Cond{"", false};
+  }
+
+  bool condsHoistable() const {
+    for (const Cond &c : conds_) {
+      if (!c.uniformEarly) return false;
+    }
+    return true;
+  }
+  std::string guardText() const {
+    std::string g;
+    for (const Cond &c : conds_) g = g.empty() ? "(" + c.chunkText + ")" : g + " && (" + c.chunkText + ")";
+    return g;
+  }
+
   static std::string keyOf(int id, const Index &idx) {
     std::string k = std::to_string(id) + "@";
-    for (const std::string &s : idx) k += s + ",";
+    for (const Ix &x : idx) k += x.s + ",";
     return k;
   }
 
@@ -240,7 +322,7 @@ class IndexedEmitter {
     if (t.isConst) return lowering::literalFor(t.dtype, t.constValue);
     if (idx.size() != std::max<size_t>(1, t.shape.size())) throw LoweringError("internal: index rank of " + t.name);
     for (size_t d = 0; d < t.shape.size(); ++d) {
-      if (t.shape[d] == 1) idx[d] = "0";
+      if (t.shape[d] == 1) idx[d] = Ix();
     }
     const std::string key = keyOf(id, idx);
     if (const std::string *known = lookup(key)) return *known;
@@ -248,6 +330,11 @@ class IndexedEmitter {
     const std::string ct = ctOf(id);
     if (t.producer < 0) {
       if (t.inputIndex < 0) throw LoweringError("operand " + t.name + " is undefined");
+      const std::string chunkLoad = inLoop_ ? tryChunkLoad(id, idx) : std::string();
+      if (!chunkLoad.empty()) {
+        scopes_.back()[key] = chunkLoad;
+        return chunkLoad;
+      }
       stmt("const " + ct + " " + var + " = " + tagOf(id) + "::load(in" + std::to_string(t.inputIndex) + "[" +
            linearize(idx, t.shape) + "]);");
       scopes_.back()[key] = var;
@@ -270,7 +357,29 @@ class IndexedEmitter {
     const std::string note = "  // " + op.name + " -> " + t.name;
     switch (op.kind) {
       case OpKind::Reshape: {
-        const Index src = delinearize(linearize(idx, outShape), inShapeOf(0));
+        const std::vector<int64_t> in = inShapeOf(0);
+        bool allUniform = true, allEarly = true, outerUniform = true, outerEarly = true;
+        for (size_t d = 0; d < idx.size(); ++d) {
+          const bool uni = idx[d].kind == 0;
+          allUniform = allUniform && uni;
+          allEarly = allEarly && idx[d].early;
+          if (d + 1 < idx.size()) {
+            outerUniform = outerUniform && uni;
+            outerEarly = outerEarly && idx[d].early;
+          }
+        }
+        Index src;
+        if (allUniform) {
+          src = delinearize(linearize(idx, outShape), in, true, allEarly);
+        } else if (outerUniform && in.back() == outShape.back() && in.back() != 1) {
+          // the innermost axis is untouched: re-derive the outer coordinates only, keep the innermost component
+          Index outerIdx(idx.begin(), idx.end() - 1);
+          const std::vector<int64_t> outerOut(outShape.begin(), outShape.end() - 1), outerIn(in.begin(), in.end() - 1);
+          src = delinearize(linearize(outerIdx, outerOut), outerIn, true, outerEarly);
+          src.push_back(idx.back());
+        } else {
+          src = delinearize(linearize(idx, outShape), in, false, false);
+        }
         stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
         break;
       }
@@ -289,7 +398,17 @@ class IndexedEmitter {
         const std::vector<int64_t> in = inShapeOf(0);
         Index src(idx.size());
         for (size_t d = 0; d < idx.size(); ++d) {
-          src[d] = in[d] == outShape[d] ? idx[d] : "(" + idx[d] + " % " + std::to_string(in[d]) + ")";
+          const Ix &x = idx[d];
+          const std::string m = " % " + std::to_string(in[d]) + ")";
+          if (in[d] == outShape[d]) {
+            src[d] = x;
+          } else if (x.kind == 0) {
+            src[d] = Ix("(" + x.s + m, x.early);
+          } else if (x.kind == 1 && x.aligned && (in[d] % vec_) == 0) {
+            src[d] = affine("(" + x.u + m, true, x.early);  // a chunk never straddles a period that V divides
+          } else {
+            src[d] = perElement("(" + x.s + m);
+          }
         }
         stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
         break;
@@ -298,10 +417,12 @@ class IndexedEmitter {
       case OpKind::StridedSlice: {
         Index src(idx.size());
         for (size_t d = 0; d < idx.size(); ++d) {
-          std::string e = idx[d];
-          if (op.strides[d] != 1) e = e + " * " + std::to_string(op.strides[d]);
-          if (op.begin[d] != 0) e = std::to_string(op.begin[d]) + " + " + e;
-          src[d] = "(" + e + ")";
+          if (op.strides[d] == 1) {
+            src[d] = shifted(idx[d], op.begin[d]);
+            continue;
+          }
+          const std::string e = "(" + std::to_string(op.begin[d]) + " + " + idx[d].s + " * " + std::to_string(op.strides[d]) + ")";
+          src[d] = idx[d].kind == 0 ? Ix(e, idx[d].early) : perElement(e);
         }
         stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
         break;
@@ -309,12 +430,16 @@ class IndexedEmitter {
       case OpKind::Pad: {
         const std::vector<int64_t> in = inShapeOf(0);
         std::string cond;
+        Cond chunk{"", true};
         Index src(idx.size());
         for (size_t d = 0; d < idx.size(); ++d) {
-          src[d] = op.begin[d] == 0 ? idx[d] : "(" + idx[d] + " - " + std::to_string(op.begin[d]) + ")";
+          src[d] = shifted(idx[d], -op.begin[d]);
           if (in[d] == outShape[d]) continue;
-          const std::string c = "static_cast<unsigned>(" + src[d] + ") < " + std::to_string(in[d]) + "u";
+          std::string c;
+          const Cond one = rangeCond(src[d], in[d], &c);
           cond = cond.empty() ? c : cond + " && " + c;
+          chunk.uniformEarly = chunk.uniformEarly && one.uniformEarly;
+          chunk.chunkText = chunk.chunkText.empty() ? one.chunkText : chunk.chunkText + " && " + one.chunkText;
         }
         const std::string fill = lowering::literalFor(t.dtype, static_cast<double>(op.padValue));
         if (cond.empty()) {
@@ -323,7 +448,9 @@ class IndexedEmitter {
           stmt(ct + " " + var + " = " + fill + ";" + note);
           stmt("if (" + cond + ") {");
           openScope();
+          conds_.push_back(chunk);
           stmt(var + " = " + valueAt(op.inputs[0], src) + ";");
+          conds_.pop_back();
           closeScope();
           stmt("}");
         }
@@ -335,15 +462,41 @@ class IndexedEmitter {
         const std::vector<int64_t> data = inShapeOf(0), ind = inShapeOf(1);
         const size_t a = static_cast<size_t>(op.concatAxis);
         const size_t indRank = g_.tensor(op.inputs[1]).shape.size();
-        Index where(ind.size(), "0");
-        for (size_t d = 0; d < indRank && d < ind.size(); ++d) where[d] = idx[a + d];
+        Index where(ind.size());
+        bool uniform = true, early = true;
+        for (size_t d = 0; d < indRank && d < ind.size(); ++d) {
+          where[d] = idx[a + d];
+          uniform = uniform && where[d].kind == 0;
+          early = early && where[d].early;
+        }
         const std::string pos = fresh("g");
-        stmt("int " + pos + " = static_cast<int>(" + valueAt(op.inputs[1], where) + ");");
-        stmt(pos + " = " + pos + " < 0 ? 0 : (" + pos + " > " + std::to_string(data[a] - 1) + " ? " +
-             std::to_string(data[a] - 1) + " : " + pos + ");");
+        const std::string clampHi = std::to_string(data[a] - 1);
+        // One position for the whole chunk, computable in front of the element loop: do it there, so that the data
+        // read below can become a chunk-wide load (embedding lookups).
+        const bool hoist = inLoop_ && uniform && early && conds_.empty();
+        if (hoist) {
+          // evaluate the position in the scope that encloses the element loop, writing in front of the loop
+          std::ostringstream *savedOut = out_;
+          const int savedIndent = indent_;
+          std::vector<std::map<std::string, std::string>> inner(scopes_.begin() + static_cast<long>(loopScope_), scopes_.end());
+          scopes_.resize(loopScope_);
+          out_ = &hoist_;
+          indent_ = hoistIndent_;
+          inLoop_ = false;
+          const std::string raw = valueAt(op.inputs[1], where);
+          stmt("int " + pos + " = static_cast<int>(" + raw + ");");
+          stmt(pos + " = " + pos + " < 0 ? 0 : (" + pos + " > " + clampHi + " ? " + clampHi + " : " + pos + ");");
+          inLoop_ = true;
+          scopes_.insert(scopes_.end(), inner.begin(), inner.end());
+          out_ = savedOut;
+          indent_ = savedIndent;
+        } else {
+          stmt("int " + pos + " = static_cast<int>(" + valueAt(op.inputs[1], where) + ");");
+          stmt(pos + " = " + pos + " < 0 ? 0 : (" + pos + " > " + clampHi + " ? " + clampHi + " : " + pos + ");");
+        }
         Index src(data.size());
         for (size_t d = 0; d < a; ++d) src[d] = idx[d];
-        src[a] = pos;
+        src[a] = uniform ? Ix(pos, hoist || !inLoop_) : perElement(pos);
         for (size_t d = a + 1; d < data.size(); ++d) src[d] = idx[d - 1 + indRank];
         stmt("const " + ct + " " + var + " = " + valueAt(op.inputs[0], src) + ";" + note);
         break;
@@ -352,15 +505,25 @@ class IndexedEmitter {
         const std::vector<int64_t> first = inShapeOf(0);
         const size_t a = static_cast<size_t>(op.concatAxis);
         Index second = idx;
-        second[a] = "(" + idx[a] + " - " + std::to_string(first[a]) + ")";
+        second[a] = shifted(idx[a], -first[a]);
+        Cond chunk{"", false};
+        if (idx[a].kind == 0) {
+          chunk = Cond{idx[a].s + " < " + std::to_string(first[a]), idx[a].early};
+        } else if (idx[a].kind == 1 && idx[a].aligned && (first[a] % vec_) == 0) {
+          chunk = Cond{idx[a].u + " < " + std::to_string(first[a]), idx[a].early};
+        }
         stmt(ct + " " + var + ";" + note);
-        stmt("if (" + idx[a] + " < " + std::to_string(first[a]) + ") {");
+        stmt("if (" + idx[a].s + " < " + std::to_string(first[a]) + ") {");
         openScope();
+        conds_.push_back(chunk);
         stmt(var + " = " + valueAt(op.inputs[0], idx) + ";");
+        conds_.pop_back();
         closeScope();
         stmt("} else {");
         openScope();
+        conds_.push_back(Cond{"!(" + chunk.chunkText + ")", chunk.uniformEarly});
         stmt(var + " = " + valueAt(op.inputs[1], second) + ";");
+        conds_.pop_back();
         closeScope();
         stmt("}");
         break;
@@ -385,6 +548,61 @@ class IndexedEmitter {
     return var;
   }
 
+  // A kernel input read at `idx`: if its V elements for this chunk are V consecutive, aligned elements in memory and
+  // the read happens for the whole chunk or not at all, load them once in front of the element loop and return the
+  // expression of the current element; otherwise return "".
+  std::string tryChunkLoad(int id, const Index &idx) {
+    const TensorValue &t = g_.tensor(id);
+    if (vec_ < 2 || t.shape.empty() || idx.empty() || opt_.gemmVariant == 2) return std::string();
+    const Ix &last = idx.back();
+    if (last.kind != 1 || !last.aligned || !last.early || (t.shape.back() % vec_) != 0) return std::string();
+    for (size_t d = 0; d + 1 < idx.size(); ++d) {
+      if (idx[d].kind != 0 || !idx[d].early) return std::string();
+    }
+    if (!condsHoistable()) return std::string();
+    Index first = idx;
+    first.back() = Ix(last.u);
+    const std::string offset = linearize(first, t.shape);
+    const std::string guard = guardText();
+    const std::string key = std::to_string(id) + "@" + offset + "?" + guard;
+    auto it = hoistedLoads_.find(key);
+    if (it == hoistedLoads_.end()) {
+      const std::string arr = fresh("w");
+      const std::string tag = tagOf(id);
+      hoisted(ctOf(id) + " " + arr + "[V] = {};");
+      hoisted(std::string(guard.empty() ? "" : "if (" + guard + ") ") + "akg::load_chunk<" + tag + ", V, false>(in" +
+              std::to_string(t.inputIndex) + " + " + offset + ", " + arr + ");");
+      it = hoistedLoads_.emplace(key, arr).first;
+    }
+    return it->second + "[e]";
+  }
+
+  // Opens the element loop: what follows goes to the loop body until closeElementLoop writes hoisted statements,
+  // loop header and body to `src_`.
+  size_t loopScope_ = 0;
+  void openElementLoop(int indentOfLoop) {
+    body_.str(std::string());
+    hoist_.str(std::string());
+    hoistedLoads_.clear();
+    conds_.clear();
+    hoistIndent_ = indentOfLoop;
+    indent_ = indentOfLoop;
+    out_ = &body_;
+    inLoop_ = true;
+    loopScope_ = scopes_.size();
+    openScope();
+  }
+  void closeElementLoop() {
+    closeScope();
+    inLoop_ = false;
+    out_ = &src_;
+    src_ << hoist_.str();
+    stmt("#pragma unroll");
+    stmt("for (int e = 0; e < V; ++e) {");
+    src_ << body_.str();
+    stmt("}");
+  }
+
   void emitTiledBody() {
     const size_t rank = space_.size();
     const size_t td = static_cast<size_t>(tDim_);
@@ -401,15 +619,15 @@ class IndexedEmitter {
     src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
     src_ << "  const int i0 = (akg_w % " << tilesI << ") * TILE;\n  akg_w /= " << tilesI << ";\n";
     src_ << "  const int t0 = (akg_w % " << tilesT << ") * TILE;\n  akg_w /= " << tilesT << ";\n";
-    canonical_.assign(rank, "0");
+    canonical_.assign(rank, Ix());
     for (size_t d = rank - 1; d-- > 0;) {
       if (d == td) continue;
       if (space_[d] == 1) continue;
       src_ << "  const int g" << d << " = akg_w % " << space_[d] << ";\n  akg_w /= " << space_[d] << ";\n";
-      canonical_[d] = "g" + std::to_string(d);
+      canonical_[d] = Ix("g" + std::to_string(d));
     }
-    canonical_[td] = "gt";
-    canonical_[rank - 1] = "inner";
+    canonical_[td] = Ix("gt");
+    canonical_[rank - 1] = affine("inner0", true, true);
     indent_ = 1;
     scopes_.clear();
     scopes_.emplace_back();
@@ -426,11 +644,11 @@ class IndexedEmitter {
       stmt("if (i0 + r < " + std::to_string(extentI) + " && t0 + q < " + std::to_string(extentT) + ") {");
       ++indent_;
       // input index: input dim perm[d] takes output index d
-      Index xi(rank, "0");
+      Index xi(rank);
       for (size_t d = 0; d < rank; ++d) {
-        std::string v = canonical_[d];
-        if (d == td) v = "(t0 + q)";
-        if (d == rank - 1) v = "(i0 + r)";
+        Ix v = canonical_[d];
+        if (d == td) v = Ix("(t0 + q)");
+        if (d == rank - 1) v = Ix("(i0 + r)");
         xi[static_cast<size_t>(op.perm[d])] = v;
       }
       stmt("const " + tagOf(st.input) + "::storage *src = in" + std::to_string(x.inputIndex) + " + " +
@@ -453,18 +671,15 @@ class IndexedEmitter {
     stmt("const int gt = t0 + tt;");
     stmt("if (gt >= " + std::to_string(extentT) + " || i0 + ci * V >= " + std::to_string(extentI) + ") continue;");
     for (size_t i = 0; i < g_.outputs.size(); ++i) stmt(ctOf(g_.outputs[i]) + " o" + std::to_string(i) + "[V];");
-    stmt("#pragma unroll");
-    stmt("for (int e = 0; e < V; ++e) {");
-    openScope();
-    stmt("const int inner = i0 + ci * V + e;");
+    stmt("const int inner0 = i0 + ci * V;");
+    openElementLoop(indent_);
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       const std::string v = valueAt(g_.outputs[i], canonical_);
       stmt("o" + std::to_string(i) + "[e] = " + v + ";");
     }
-    closeScope();
-    stmt("}");
+    closeElementLoop();
     Index first = canonical_;
-    first[rank - 1] = "(i0 + ci * V)";
+    first[rank - 1] = Ix("inner0");
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, true>(out" + std::to_string(i) + " + " +
            linearize(first, space_) + ", o" + std::to_string(i) + ");");
@@ -516,20 +731,17 @@ class IndexedEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       stmt(ctOf(g_.outputs[i]) + " o" + std::to_string(i) + "[V];");
     }
-    stmt("#pragma unroll");
-    stmt("for (int e = 0; e < V; ++e) {");
-    openScope();
     Index idx = start;
     if (space_.back() != 1) {
-      stmt("const int inner = " + start.back() + " + e;");
-      idx.back() = "inner";
+      stmt("const int inner0 = " + start.back().s + ";  // a multiple of V: V divides the innermost extent");
+      idx.back() = affine("inner0", true, true);
     }
+    openElementLoop(indent_);
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       const std::string v = valueAt(g_.outputs[i], idx);
       stmt("o" + std::to_string(i) + "[e] = " + v + ";");
     }
-    closeScope();
-    stmt("}");
+    closeElementLoop();
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, false>(out" + std::to_string(i) + " + base, o" +
            std::to_string(i) + ");");
