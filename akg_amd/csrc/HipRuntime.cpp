@@ -362,6 +362,9 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
     // workspace, so they must not overlap on the device (launch them on one stream, or order the streams).
     e = hipMalloc(&l.workspace, k->lowered.workspaceBytes);
     if (e == hipSuccess) e = hipMemset(l.workspace, 0, k->lowered.workspaceBytes);
+    // the fill runs on the null stream and may still be in flight when hipMemset returns; the first launch may go to
+    // a stream that does not wait for the null stream
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess) {
       if (l.workspace) (void)hipFree(l.workspace);
       (void)hipModuleUnload(l.module);
