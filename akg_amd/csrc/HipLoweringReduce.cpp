@@ -142,7 +142,6 @@ class StreamReduceEmitter {
       for (size_t a : realReducedAxes(g_, *op)) r2[a] = true;
       if (r2 != reduced) throw LoweringError("all reductions of one kernel must reduce the same axes");
       const DType od = g_.tensor(op->outputs[0]).dtype;
-      if (od == DType::Bool) throw LoweringError("op " + op->name + ": bool reductions have no streaming kernel yet");
       if (std::string(computeTypeName(in.dtype)) != computeTypeName(od)) {
         throw LoweringError("op " + op->name + ": operand and result element types differ");
       }

@@ -298,6 +298,12 @@ class GraphBuilder {
         }
       } else {
         for (size_t j = 0; j < inputDesc.size(); ++j) {
+          if (node.kind == OpKind::Concat) {
+            // the operands of a Concat are the tensors of its input entries, normally ONE entry holding the whole
+            // list (handleConcatOperands :772-791)
+            for (size_t t = 0; t < inputDesc[j].size(); ++t) node.inputs.push_back(operandFor(inputDesc[j][t], node.name));
+            continue;
+          }
           if (isIndex1DAttrAsInput(node.name, j)) continue;
           if (node.kind == OpKind::Cast && j > 0) continue;  // convertCastOp keeps the first operand only (:1351-1360)
           if (node.kind == OpKind::StridedSlice && j > 0) continue;  // begin / end / strides carried as constants

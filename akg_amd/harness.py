@@ -82,7 +82,10 @@ def make_inputs(desc, seed=BASE_SEED, pattern=None):
             out.append(rng.integers(-100, 101, size=shape).astype(dt))
             continue
         if dt == "bool":
-            out.append(rng.integers(0, 2, size=shape).astype(np.bool_))
+            if any(o["name"] == "ReduceAll" for o in desc["op_desc"]):
+                out.append(rng.random(size=shape) < 0.999)      # mostly true, so that some results are true
+            else:
+                out.append(rng.integers(0, 2, size=shape).astype(np.bool_))
             continue
         if pattern == "softmax":
             x = rng.standard_normal(shape, dtype=np.float32) * 2.0

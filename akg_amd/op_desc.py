@@ -337,9 +337,14 @@ def pad(b, x, padding, value=0):
 
 
 def concat(b, x, y, axis):
+    """The operands of a Concat travel as ONE input entry holding the list of tensors (TranslateToMindsporeDialect.cpp
+    :772-791), unlike every other op, where each operand is an entry of its own."""
     shape = list(x.shape)
     shape[axis] += y.shape[axis]
-    return b.op("Concat", [x, y], shape, x.dtype, attrs=[{"data_type": "int", "name": "axis", "value": int(axis)}])
+    out = b.op("Concat", [x, y], shape, x.dtype, attrs=[{"data_type": "int", "name": "axis", "value": int(axis)},
+                                                         {"data_type": "int", "name": "inputNums", "value": 2}])
+    b.ops[-1]["input_desc"] = [[x.desc(), y.desc()]]
+    return out
 
 
 def transpose_bias_add(batch, rows, cols, dtype="bfloat16", name=None):

@@ -176,7 +176,10 @@ def evaluate(desc, inputs, updates=None):
             name = "ReduceAny"
         attrs = {a["name"]: a["value"] for a in (od.get("attr") or [])}
         ins, in_dt = [], []
-        for idx, entry in enumerate(od["input_desc"]):
+        entries = od["input_desc"]
+        if name == "Concat":  # one entry holding the list of operands (TranslateToMindsporeDialect.cpp:772-791)
+            entries = [[d] for entry in entries for d in entry]
+        for idx, entry in enumerate(entries):
             if idx == 1 and name in ATTR_AS_INPUT:
                 continue
             if name == "Cast" and idx > 0:

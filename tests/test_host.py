@@ -64,7 +64,13 @@ def test_null_arguments_are_rejected_not_crashed_on():
 # ---------------------------------------------------------------------------------------------------------
 # translator vs an independent JSON reader, on the reference's own fixture files
 # ---------------------------------------------------------------------------------------------------------
-STATIC_REF = sorted(f for f in os.listdir(REF_INFO) if f.endswith(".info") and ".dynamic." not in f)
+def _static(name):
+    d = harness.load_desc(os.path.join(REF_INFO, name))
+    return not any(x < 0 for e in d["input_desc"] for x in e[0].get("shape", [1]))
+
+
+# every static description of the reference's test tree but the Split one (two results share a tensor name there)
+STATIC_REF = sorted(f for f in os.listdir(REF_INFO) if ".info" in f and not f.startswith("Fused_Split_") and _static(f))
 
 
 @pytest.mark.parametrize("name", STATIC_REF)
