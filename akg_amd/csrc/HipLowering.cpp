@@ -16,6 +16,7 @@ const char *kernelFamilyName(KernelFamily f) {
     case KernelFamily::GemmEpilogue: return "gemm_epilogue";
     case KernelFamily::StreamReduce: return "stream_reduce";
     case KernelFamily::Indexed: return "indexed";
+    case KernelFamily::SegmentSum: return "segment_sum";
   }
   return "?";
 }
@@ -242,6 +243,7 @@ bool isElementwiseKind(OpKind k) {
     case OpKind::Pad:
     case OpKind::Concat:
     case OpKind::Gather:
+    case OpKind::SegmentSum:
       return false;
     default:
       return !isReduceKind(k);
@@ -1243,6 +1245,9 @@ LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options) {
   bool hasMatMul = false;
   for (const OpNode &op : graph.ops) {
     if (op.kind == OpKind::MatMul) hasMatMul = true;
+  }
+  for (const OpNode &op : graph.ops) {
+    if (op.kind == OpKind::SegmentSum) return lowerSegmentSumToHip(graph, options);
   }
   if (wantsIndexedKernel(graph)) return lowerIndexedToHip(graph, options);
   if (hasMatMul) return lowerGemmToHip(graph, options);

@@ -31,7 +31,7 @@ class LoweringError : public std::runtime_error {
   explicit LoweringError(const std::string &msg) : std::runtime_error(msg) {}
 };
 
-enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce, Indexed };
+enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce, Indexed, SegmentSum };
 const char *kernelFamilyName(KernelFamily f);
 
 // Tuning knobs; 0 means "let the heuristic decide". They can be set through the environment
@@ -69,6 +69,7 @@ LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerGemmToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerStreamReduceToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerIndexedToHip(const OpGraph &graph, const LoweringOptions &options);
+LoweredKernel lowerSegmentSumToHip(const OpGraph &graph, const LoweringOptions &options);
 // True when the graph contains a data-movement op (Transpose, Tile, Slice, StridedSlice, Pad, Concat).
 bool wantsIndexedKernel(const OpGraph &graph);
 // True when the reductions of `graph` belong to the streaming family: some reduced axis is not the innermost one

@@ -93,7 +93,7 @@ const OpTableEntry kOpTable[] = {
   {"Gather", OpKind::Gather},
   {"InplaceAssign", OpKind::Assign},
   {"Assign", OpKind::Assign},
-  {"UnsortedSegmentSum", OpKind::Unsupported},
+  {"UnsortedSegmentSum", OpKind::SegmentSum},
   {"StridedSlice", OpKind::StridedSlice},
   {"AddN", OpKind::AddN},
   {"MatMul", OpKind::MatMul},
@@ -308,6 +308,7 @@ class GraphBuilder {
           if (node.kind == OpKind::Cast && j > 0) continue;  // convertCastOp keeps the first operand only (:1351-1360)
           if (node.kind == OpKind::StridedSlice && j > 0) continue;  // begin / end / strides carried as constants
           if (node.kind == OpKind::Gather && j > 1) continue;        // the axis carried as a constant
+          if (node.kind == OpKind::SegmentSum && j > 1) continue;    // the segment count carried as a constant
           if (node.kind == OpKind::Assign && j > 1) continue;        // convertInplaceAssignOp keeps two operands (:1104-1115)
           node.inputs.push_back(operandFor(inputDesc[j][0], node.name));
         }
@@ -342,6 +343,36 @@ class GraphBuilder {
         if (const json::Value *b = findAttr(attrs, kTransposeB)) node.transposeB = b->asBool();
       }
 
+      if (node.kind == OpKind::SegmentSum) {
+        // segment count: third input's value, else attr "numSegments" (convertUnsortedSegmentSumOp :981-1017); the
+        // reference's own test descriptions spell it "num_segments", which is accepted too
+        if (node.inputs.size() != 2) throw TranslateError("op " + node.name + ": needs a data and a segment-id operand");
+        int64_t segments = 0;
+        if (inputDesc.size() > 2 && inputDesc[2][0].contains(kValue)) {
+          const json::Value &v = inputDesc[2][0].at(kValue);
+          segments = v.isArray() ? v.asIntVector().at(0) : static_cast<int64_t>(v.asDouble());
+        } else if (const json::Value *a = findAttr(attrs, "numSegments")) {
+          segments = a->isArray() ? a->asIntVector().at(0) : static_cast<int64_t>(a->asDouble());
+        } else if (const json::Value *b = findAttr(attrs, "num_segments")) {
+          segments = b->isArray() ? b->asIntVector().at(0) : static_cast<int64_t>(b->asDouble());
+        }
+        if (segments <= 0) throw TranslateError("UnsortedSegmentSumOp must have attr: numSegments");
+        const TensorValue &data = graph_.tensor(node.inputs[0]);
+        const TensorValue &ids = graph_.tensor(node.inputs[1]);
+        if (isFloatType(ids.dtype) || ids.dtype == DType::Bool) throw TranslateError("op " + node.name + ": segment ids must be integers");
+        if (ids.shape.size() > data.shape.size() ||
+            !std::equal(ids.shape.begin(), ids.shape.end(), data.shape.begin())) {
+          throw TranslateError("op " + node.name + ": the segment ids must have the leading dimensions of the data");
+        }
+        std::vector<int64_t> expect{segments};
+        expect.insert(expect.end(), data.shape.begin() + static_cast<long>(ids.shape.size()), data.shape.end());
+        const std::vector<int64_t> declared = readShape(outputDesc[0]);
+        int64_t n = 1, m = 1;
+        for (int64_t d : expect) n *= d;
+        for (int64_t d : declared) m *= d;
+        if (n != m) throw TranslateError("op " + node.name + ": the declared result shape does not follow from the operands");
+        node.padValue = segments;
+      }
       if (node.kind == OpKind::Assign) {
         if (node.inputs.size() != 2) throw TranslateError("op " + node.name + ": needs a destination and a value operand");
         const TensorValue &dst = graph_.tensor(node.inputs[0]);
@@ -699,6 +730,7 @@ OperatorTemplate templateOfOp(const OpGraph &g, const OpNode &op) {
     case OpKind::Pad:
     case OpKind::Concat:
     case OpKind::Gather:
+    case OpKind::SegmentSum:
       return OperatorTemplate::Default;  // not classified by getOperatorTemplate (OperatorIdentify.cpp:51-75)
     case OpKind::Unknown:
     case OpKind::Unsupported:
@@ -824,6 +856,7 @@ const char *opKindName(OpKind k) {
     case OpKind::Pad: return "pad";
     case OpKind::Concat: return "concat";
     case OpKind::Gather: return "gather";
+    case OpKind::SegmentSum: return "unsorted_segment_sum";
     case OpKind::MatMul: return "matmul";
     case OpKind::AddN: return "addn";
     case OpKind::Assign: return "inplace_assign";

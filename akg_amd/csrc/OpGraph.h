@@ -47,6 +47,8 @@ enum class OpKind {
   Reshape, BroadcastTo,
   // data movement: the result is the operand read through an index map
   Transpose, Tile, Slice, StridedSlice, Pad, Concat, Gather,
+  // UnsortedSegmentSum: out[ids[i], ...] += data[i, ...] over the index positions i in increasing order
+  SegmentSum,
   // contraction
   MatMul,
   // n-ary
@@ -96,7 +98,7 @@ struct OpNode {
   std::vector<int64_t> perm;       // Transpose: result dim d is operand dim perm[d]
   std::vector<int64_t> begin;      // Slice / StridedSlice: first index taken; Pad: elements added in front
   std::vector<int64_t> strides;    // StridedSlice: step (positive); Slice: all ones
-  int64_t padValue = 0;            // Pad: the constant written outside the operand
+  int64_t padValue = 0;            // Pad: the constant written outside the operand; SegmentSum: number of segments
   int64_t concatAxis = 0;          // Concat: axis along which the operands follow one another; Gather: gathered axis
   std::string ptrAddress;
 };

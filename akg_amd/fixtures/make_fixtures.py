@@ -59,6 +59,11 @@ FIXTURES = {
     "small_transpose_sum_f16_130x66_perm10": lambda n: op_desc.transpose_sum([130, 66], [1, 0], "float16", n),
     "small_embedding_lookup_bf16_1000x96_ids5x33": lambda n: op_desc.embedding_lookup_scale(1000, 96, 5, 33, "bfloat16", n),
     "small_embedding_lookup_f32_50x7_ids3x4": lambda n: op_desc.embedding_lookup_scale(50, 7, 3, 4, "float32", n),
+    # UnsortedSegmentSum (segment_sum family): short slices, a wide slice tiled over workgroups, 16-bit accumulation
+    "small_segment_sum_f32_700x3_by_1x3_seg50": lambda n: op_desc.unsorted_segment_sum([700, 3], [1, 3], 50, "float32", "int32", n),
+    "small_segment_sum_f32_300_by_10000_seg7": lambda n: op_desc.unsorted_segment_sum([300], [10000], 7, "float32", "int64", n),
+    "small_segment_sum_bf16_4096_by_200_seg1000": lambda n: op_desc.unsorted_segment_sum([4096], [200], 1000, "bfloat16", "int32", n),
+    "small_segment_sum_i32_1000_by_65_seg3": lambda n: op_desc.unsorted_segment_sum([1000], [65], 3, "int32", "int32", n),
     "n3_transpose_bias_add_bf16_32x2048x1024": lambda n: op_desc.transpose_bias_add(32, 2048, 1024, "bfloat16", n),
     # float MatMul + bias + activation on the bfloat16 / float16 MFMA path
     "small_gemm_bf16_bias_gelu_256x512x256": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "float32", n),

@@ -78,6 +78,10 @@ def make_inputs(desc, seed=BASE_SEED, pattern=None):
             extent = op["input_desc"][0][0]["shape"][int(attrs.get("axis", 0))]
             out.append(rng.integers(-2, extent + 2, size=shape).astype(dt))
             continue
+        if dt in ("int16", "int32", "int64") and any(o["name"] == "UnsortedSegmentSum" for o in desc["op_desc"]):
+            op = next(o for o in desc["op_desc"] if o["name"] == "UnsortedSegmentSum")
+            out.append(rng.integers(0, op["output_desc"][0]["shape"][0], size=shape).astype(dt))
+            continue
         if dt in ("int16", "int32", "int64"):
             out.append(rng.integers(-100, 101, size=shape).astype(dt))
             continue

@@ -442,6 +442,18 @@ def embedding_lookup_scale(vocab, width, batch, seq, dtype="bfloat16", name=None
     return b.dumps([b.cast(x, dtype) if dtype != "float32" else x])
 
 
+def unsorted_segment_sum(index_shape, slice_shape, segments, dtype="float32", ids_dtype="int32", name=None):
+    """out[ids[i...], :] += data[i..., :] over the index positions in row-major order (an embedding-table gradient, a
+    graph-network aggregation). The segment count is carried as the attribute the reference's test descriptions use."""
+    b = DescBuilder(name or "Fused_UnsortedSegmentSum_%s_%s_seg%d" % (
+        _SHORT[dtype], "x".join(str(d) for d in list(index_shape) + list(slice_shape)), segments))
+    data = b.input(list(index_shape) + list(slice_shape), dtype)
+    ids = b.input(list(index_shape), ids_dtype)
+    out = b.op("UnsortedSegmentSum", [data, ids], [segments] + list(slice_shape), dtype,
+               attrs=[{"data_type": "int", "name": "num_segments", "value": int(segments)}])
+    return b.dumps([out])
+
+
 def any_greater(rows, cols, threshold=2.5, op="ElemAny", name=None):
     """out[r] = any(x[r, :] > threshold), spelled with `ElemAny` (the reference maps it to its ReduceAny op)."""
     b = DescBuilder(name or "Fused_Greater_%s_f32_%dx%d" % (op, rows, cols))

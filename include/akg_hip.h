@@ -57,7 +57,7 @@ typedef struct akg_hip_tensor_desc {
 
 typedef struct akg_hip_kernel_info {
   char kernel_name[256];              /* "<op>_kernel" (KernelOutliningExt.cpp:433) */
-  char family[32];                    /* "elementwise" | "row_reduce" | "stream_reduce" | "gemm_epilogue" | "indexed" */
+  char family[32];                    /* "elementwise" | "row_reduce" | "stream_reduce" | "gemm_epilogue" | "indexed" | "segment_sum" */
   char operator_type[32];             /* fusion class, OperatorIdentify.cpp:51-93 */
   uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json */
   uint32_t block[3];                  /* threadIdx.x/y/z extents */

@@ -60,6 +60,7 @@ MATMULS = ("MatMul", "BatchMatMul")
 # the first operand's buffer (a kernel input) and is also the op's result; the result has the destination's shape
 # (TranslateToMindsporeDialect.cpp:359-364,398-404)
 ASSIGNS = ("Assign", "InplaceAssign")
+SEGMENTS = ("UnsortedSegmentSum",)
 REDUCES = ("ReduceSum", "ReduceMax", "ReduceMin", "ReducePrd", "ReduceAll", "ReduceAny")
 ATTR_AS_INPUT = ("Reshape", "BroadcastTo", "ReduceMax", "ReduceMin", "ReduceSum", "ReducePrd", "ReduceAll", "ReduceAny",
                  "ArgMax", "Transpose", "Tile")
@@ -215,6 +216,8 @@ def parse(desc):
                 continue
             if name in ASSIGNS and idx > 1:
                 continue
+            if name in SEGMENTS and idx > 1:
+                continue
             d = entry[0]
             if d["tensor_name"] in tensors:
                 ins.append(tensors[d["tensor_name"]])
@@ -286,7 +289,7 @@ class Emitter:
 
     # -- which values live in memory --------------------------------------------------------------------
     def is_elementwise(self, op):
-        return op.name not in REDUCES and op.name not in MATMULS + ("Reshape",) and op.name not in VIEW_OPS + ASSIGNS
+        return op.name not in REDUCES + MATMULS + ("Reshape",) + VIEW_OPS + ASSIGNS + SEGMENTS
 
     def plan(self):
         consumers = {}
@@ -299,11 +302,11 @@ class Emitter:
                 out.alias_of = op.inputs[0]
                 continue
             inline = (self.is_elementwise(op) and out.uses == 1 and not out.is_output
-                      and consumers[out.name][0].name not in MATMULS + ("Reshape",) + VIEW_OPS)
+                      and consumers[out.name][0].name not in MATMULS + ("Reshape",) + VIEW_OPS + SEGMENTS)
             out.inline = inline
         # the source of a Reshape view and MatMul operands must be in memory
         for op in self.ops:
-            if op.name in MATMULS + ("Reshape",) + VIEW_OPS:
+            if op.name in MATMULS + ("Reshape",) + VIEW_OPS + SEGMENTS:
                 for t in op.inputs:
                     if t.producer is not None and t.producer.name != "Reshape":
                         t.inline = False
@@ -501,6 +504,41 @@ class Emitter:
         self.emit("((%s *)%s)[%s] = v;" % (C_STORAGE[dst.dtype], dst.buffer, idx), depth)
         self.emit("%s[%s] = v;" % (out.buffer, idx), depth)
         self.close_loops(len(shape), depth)
+
+    def emit_segment_sum(self, op):
+        """UnsortedSegmentSum (MindSporeToLinalg.cpp:596-745): the index dimensions collapse into one, the result is
+        zero-filled, and ONE serial loop over the index positions adds data[i, :] to result[ids[i], :], rounding to the
+        result's type after every addition. The reference indexes the result with the id as it is; ids outside
+        [0, segments) are dropped here (parity unpinned for those: the reference's access would be out of bounds)."""
+        data, ids, out = op.inputs[0], op.inputs[1], op.output
+        if data.const is not None or ids.const is not None or data.dtype != out.dtype or ids.dtype in FLOATS + ("bool",):
+            raise OracleError("UnsortedSegmentSum: needs a data tensor of the result's type and integer segment ids")
+        if list(data.shape[:len(ids.shape)]) != list(ids.shape):
+            raise OracleError("UnsortedSegmentSum: the ids must have the leading dimensions of the data")
+        positions = max(1, ids.numel)
+        slice_ = data.numel // positions
+        segments = out.numel // slice_
+        want = op.attrs.get("numSegments", op.attrs.get("num_segments", segments))
+        if isinstance(want, list):
+            want = want[0]
+        if int(want) != segments:
+            raise OracleError("UnsortedSegmentSum: the result shape does not follow from the segment count")
+        rd, ri = self.root(data), self.root(ids)
+        od = out.dtype
+        self.emit("memset(%s, 0, sizeof(%s) * %dL);" % (out.buffer, C_STORAGE[od], out.numel))
+        self.emit("for (int64_t i = 0; i < %dL; ++i) {" % positions)
+        self.emit("const int64_t id = (int64_t)%s[i];" % ri.buffer, 2)
+        self.emit("if (id < 0 || id >= %dL) continue;" % segments, 2)
+        self.emit("for (int64_t j = 0; j < %dL; ++j) {" % slice_, 2)
+        x = self.load_expr(rd, "i * %dL + j" % slice_)
+        acc = self.load_expr(out, "id * %dL + j" % slice_)
+        if od in FLOATS:
+            step = self.rnd(od, "(%s + %s)" % (x, acc))
+        else:
+            step = self.rnd(od, "((%s)((uint64_t)%s + (uint64_t)%s))" % (C_COMPUTE[od], x, acc))
+        self.emit("%s[id * %dL + j] = %s;" % (out.buffer, slice_, self.store_expr(od, step)), 3)
+        self.emit("}", 2)
+        self.emit("}")
 
     def emit_view(self, op):
         """Data-movement op: a loop nest over the result that copies the operand element its index map names."""
@@ -708,6 +746,8 @@ class Emitter:
                 self.emit_view(op)
             elif op.name in ASSIGNS:
                 self.emit_assign(op)
+            elif op.name in SEGMENTS:
+                self.emit_segment_sum(op)
             else:
                 self.emit_elementwise(op)
         for b in self.temps:

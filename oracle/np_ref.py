@@ -190,6 +190,8 @@ def evaluate(desc, inputs, updates=None):
                 continue
             if name in ("Assign", "InplaceAssign") and idx > 1:
                 continue
+            if name == "UnsortedSegmentSum" and idx > 1:
+                continue
             d = entry[0]
             tn = d["tensor_name"]
             if tn not in env:
@@ -334,6 +336,21 @@ def evaluate(desc, inputs, updates=None):
                 else:
                     res = np.concatenate([x, ins[1]], axis=vp["axis"])
                 res = np.ascontiguousarray(res)
+            elif name == "UnsortedSegmentSum":
+                # serial loop over the collapsed index positions, accumulating in the result's type
+                # (MindSporeToLinalg.cpp:596-745); ids outside [0, segments) are dropped
+                ids_flat = np.asarray(ins[1]).astype(np.int64).reshape(-1)
+                rows = cv[0].reshape(ids_flat.size, -1)
+                segments = int(np.prod(oshape)) // max(1, rows.shape[1])
+                res = np.zeros((segments, rows.shape[1]), dtype=rows.dtype)
+                if odt in ("float16", "bfloat16", "int8", "int16"):
+                    for i, sid in enumerate(ids_flat):     # rounds after every addition
+                        if 0 <= sid < segments:
+                            res[sid] = compute_view(finish(rows[i] + res[sid], odt), odt)
+                else:
+                    ok = (ids_flat >= 0) & (ids_flat < segments)
+                    np.add.at(res, ids_flat[ok], rows[ok])  # unbuffered: applied in index order
+                res = res.reshape(oshape)
             elif name in ("Assign", "InplaceAssign"):
                 # linalg.copy ins=input1 outs=input0 (MindSporeToLinalg.cpp:495-524)
                 dst_name = od["input_desc"][0][0]["tensor_name"]

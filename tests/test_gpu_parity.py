@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "akg_amd", "fixtures")
 STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all")
 ALL_SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
-SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS)]
+SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS) and "segment_sum" not in n]
 STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS)]
 FULL = ["c1_ew_tanh_add_mul_f32_1024x4096.info", "c2_softmax_f16_8192x4096.info",
         "c3_layernorm_residual_bf16_16384x4096.info", "c4_quant_int8_residual_bf16_32768x8192.info"]
@@ -119,8 +119,8 @@ def test_full_size_config_matches_oracle(name):
 REF_INFO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_info")
 # Every op description of the reference's own test tree (akg-mlir/tests/st/**), copied as data under their own names
 # (".info_failed" / ".info.failed" are the reference's markers for cases its CPU pipeline does not pass).
-# Not run: Split (the reference has no lowering for mindspore.split either) and UnsortedSegmentSum (no kernel here).
-REF_SKIPPED = ("Fused_Split_", "Fused_UnsortedSegmentSum_")
+# Not run: Split (the reference has no lowering for mindspore.split either).
+REF_SKIPPED = ("Fused_Split_",)
 
 
 def _is_dynamic(path):
@@ -131,7 +131,8 @@ def _is_dynamic(path):
 REF_ALL = sorted(f for f in os.listdir(REF_INFO) if ".info" in f and not f.startswith(REF_SKIPPED))
 REF_DYNAMIC = [f for f in REF_ALL if _is_dynamic(os.path.join(REF_INFO, f))]
 REF_STREAM = [f for f in REF_ALL if f not in REF_DYNAMIC and "ReduceSum_split" in f]
-REF_STATIC = [f for f in REF_ALL if f not in REF_DYNAMIC and f not in REF_STREAM]
+REF_SEGMENT = [f for f in REF_ALL if f.startswith("Fused_UnsortedSegmentSum_")]
+REF_STATIC = [f for f in REF_ALL if f not in REF_DYNAMIC and f not in REF_STREAM and f not in REF_SEGMENT]
 
 
 @pytest.mark.parametrize("name", REF_STREAM)
@@ -156,6 +157,49 @@ def test_reference_repository_descriptions_match_oracle(name):
         ok, msg = harness.compare(g, e, d.dtype)
         print("  %s %s: %s" % (d.name, d.dtype, msg), flush=True)
         assert ok, "%s output %s: %s" % (name, d.name, msg)
+
+
+def check_segment_sum(path, seed, repeats=2):
+    """UnsortedSegmentSum keeps the serial order of the additions per output element: bit-exact against the oracle,
+    float types included, and on every launch (nothing may be left over from the one before)."""
+    print("case %s seed %d" % (os.path.basename(path), seed), flush=True)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    assert kernel.family == "segment_sum"
+    inputs = harness.make_inputs(desc, seed=seed)
+    expect = cpu_ref.CpuKernel(path)(inputs)
+    for rep in range(repeats):
+        got = run_on_gpu(kernel, inputs)
+        assert len(got) == 1 and got[0].shape == expect[0].shape
+        same = np.array_equal(np.ascontiguousarray(got[0]).view(np.uint8), np.ascontiguousarray(expect[0]).view(np.uint8))
+        print("  launch %d: %s" % (rep, "bit-exact" if same else "DIFFERS"), flush=True)
+        assert same, os.path.basename(path)
+    return inputs, expect
+
+
+@pytest.mark.parametrize("name", REF_SEGMENT)
+def test_reference_repository_segment_sum_descriptions(name):
+    """Fused_UnsortedSegmentSum_split_*: the reference's own descriptions (marked failed for its CPU pipeline), up to
+    24.5 million index positions scattered into [4954, 1, 3]."""
+    check_segment_sum(os.path.join(REF_INFO, name), seed=harness.BASE_SEED + 300)
+
+
+@pytest.mark.parametrize("name", [n for n in ALL_SMALL if "segment_sum" in n])
+def test_segment_sum_is_bit_exact(name):
+    check_segment_sum(os.path.join(FIXTURES, name), seed=harness.BASE_SEED + 301)
+
+
+def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero():
+    path = os.path.join(FIXTURES, "small_segment_sum_f32_700x3_by_1x3_seg50.info")
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 302)
+    ids = inputs[1]
+    ids[ids == 17] = 50          # nobody names row 17; 50 and -3 are outside [0, 50)
+    ids[::7] = -3
+    expect = cpu_ref.CpuKernel(path)(inputs)
+    got = run_on_gpu(kernel, inputs)
+    assert np.array_equal(got[0], expect[0]) and not got[0][17].any() and got[0].any()
 
 
 # Shapes the dynamic descriptions of the reference's test tree are specialised to (input_desc order).

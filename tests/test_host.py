@@ -232,6 +232,36 @@ def test_streaming_reduction_family_and_schedule():
     assert k.family == "row_reduce" and k.workspace_bytes == 0
 
 
+def test_unsorted_segment_sum_translates_and_gets_its_own_family():
+    path = os.path.join(REF_INFO, "Fused_UnsortedSegmentSum_split_11686736348673473318.info_failed")
+    k = driver.HipKernel.from_file(path)
+    assert k.family == "segment_sum" and k.workspace_bytes == 0
+    assert [t.shape for t in k.outputs] == [[4954, 1, 3]]
+    assert "mindspore.unsorted_segment_sum" in driver.translate(open(path, encoding="utf-8").read())
+    # the kernel scans ids 64 at a time and keeps the accumulators of its segments in LDS
+    assert "__ballot" in k.source and "__shared__" in k.source and "atomic" not in k.source
+    d = json.loads(op_desc.unsorted_segment_sum([12], [5], 4, "float32"))
+    d["op_desc"][0]["attr"] = None              # no segment count anywhere: the reference's own message
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(json.dumps(d), out_dir=None)
+    assert e.value.code == -3 and "numSegments" in str(e.value)
+    d = json.loads(op_desc.unsorted_segment_sum([12], [5], 4, "float32"))
+    d["op_desc"][0]["attr"][0]["name"] = "numSegments"      # the spelling the reference's translator reads
+    assert driver.HipKernel(json.dumps(d), out_dir=None).family == "segment_sum"
+    d["op_desc"][0]["input_desc"][1][0]["shape"] = [6]      # ids must cover the leading dimensions of the data
+    d["input_desc"][1][0]["shape"] = [6]
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(json.dumps(d), out_dir=None)
+    assert e.value.code == -3 and "leading dimensions" in str(e.value)
+    # fused with a neighbour: no kernel yet, said so
+    b = op_desc.DescBuilder("Fused_UnsortedSegmentSum_Neg")
+    data, ids = b.input([12, 5], "float32"), b.input([12], "int32")
+    seg = b.op("UnsortedSegmentSum", [data, ids], [4, 5], "float32", attrs=[{"data_type": "int", "name": "num_segments", "value": 4}])
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(b.dumps([b.unary("Neg", seg)]), out_dir=None)
+    assert e.value.code == -4 and "kernel of its own" in str(e.value)
+
+
 def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_view_chain_f32.info"))
     assert (k.operator_type, k.family) == ("Transpose", "indexed")

@@ -374,6 +374,36 @@ def test_gather_takes_rows_by_index_and_clamps(tmp_path):
                 assert np.array_equal(c_out[0][i, j, k], x[i, row]) and np.array_equal(n_out[0][i, j, k], x[i, row])
 
 
+def test_unsorted_segment_sum_adds_slices_in_index_order(tmp_path):
+    """UnsortedSegmentSum against a dictionary of Python lists: every slice lands in the row its id names, rows no id
+    names stay zero, and the additions happen in index order in the result's type. The order is pinned by a row that
+    receives 1, 2^24 and -2^24 in that order: float32 gives 0 (1 + 2^24 rounds to 2^24), any other order gives 1.
+    Ids outside [0, segments) are dropped (undefined in the reference)."""
+    text = op_desc.unsorted_segment_sum([3, 2], [2], 5, "float32", name="pin_segment_sum")
+    data = np.array([[[1, 10], [5, 50]], [[2.0 ** 24, 20], [7, 70]], [[-2.0 ** 24, 30], [9, 90]]], dtype=np.float32)
+    ids = np.array([[2, 0], [2, 7], [2, -1]], dtype=np.int32)
+    _, c_out, n_out = build_and_run(text, [data, ids], tmp_path)
+    rows = {}
+    for pos in range(6):
+        sid = int(ids.reshape(-1)[pos])
+        if 0 <= sid < 5:
+            rows.setdefault(sid, []).append(data.reshape(6, 2)[pos])
+    expect = np.zeros((5, 2), dtype=np.float32)
+    for sid, parts in rows.items():
+        acc = np.zeros(2, dtype=np.float32)
+        for part in parts:
+            acc = (acc + part).astype(np.float32)
+        expect[sid] = acc
+    assert expect[2, 0] == 0.0 and expect[2, 1] == 60.0 and expect[0, 0] == 5.0
+    assert np.array_equal(c_out[0], expect) and np.array_equal(np.asarray(n_out[0]).reshape(5, 2), expect)
+    # bfloat16 accumulates in bfloat16: 256 ones in one row stop growing at 256 (257 is not representable)
+    text = op_desc.unsorted_segment_sum([300], [1], 2, "bfloat16", name="pin_segment_sum_bf16")
+    ones = harness.f32_to_bf16_bits(np.ones((300, 1), dtype=np.float32))
+    _, c_out, n_out = build_and_run(text, [ones, np.zeros(300, dtype=np.int32)], tmp_path)
+    assert harness.bf16_bits_to_f32(c_out[0]).reshape(-1).tolist() == [256.0, 0.0]
+    assert harness.bf16_bits_to_f32(n_out[0]).reshape(-1).tolist() == [256.0, 0.0]
+
+
 def test_assign_writes_the_value_over_its_first_operand(tmp_path):
     """Momentum step in float32 against the formula written out in numpy: v <- 0.9 v + g, p <- p - 0.01 v. The C
     restatement updates the caller's input arrays in place, the numpy one reports the updates."""
