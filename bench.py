@@ -49,14 +49,14 @@ CALIBRATION = "calib_neg_f32_16384x4096"
 # ones of the summaries under profiles/; None = not measured yet.
 CLOCK_RAMP_MS = 120.0
 MEASURED_TRAFFIC_BYTES = {
-    "c1_ew_tanh_add_mul_f32_1024x4096": 67142575,
-    "c2_softmax_f16_8192x4096": 134248003,
-    "c3_layernorm_residual_bf16_16384x4096": 402799591,
-    "c4_quant_int8_residual_bf16_32768x8192": 1343213382,
-    "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": 470265416,
-    "n1_biasgrad_bf16_16384x4096": 270924749,
-    "n2_gemm_bf16_bias_gelu_4096x8192x8192": 872783522,
-    "n3_transpose_bias_add_bf16_32x2048x1024": 268461174,
+    "c1_ew_tanh_add_mul_f32_1024x4096": 67142582,
+    "c2_softmax_f16_8192x4096": 134243913,
+    "c3_layernorm_residual_bf16_16384x4096": 402797563,
+    "c4_quant_int8_residual_bf16_32768x8192": 1343173505,
+    "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": 470254548,
+    "n1_biasgrad_bf16_16384x4096": 270924759,
+    "n2_gemm_bf16_bias_gelu_4096x8192x8192": 872910920,
+    "n3_transpose_bias_add_bf16_32x2048x1024": 268462651,
 }
 
 
