@@ -511,6 +511,8 @@ class TileEmitter {
     note << kernelFamilyName(k.family) << " rows=" << rows_ << " cols=" << cols_ << " vec=" << vec_
          << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
          << " block=" << block_ << " grid=" << grid_;
+    if (overlap_ > 0) note << " tail_overlap=" << overlap_;
+    if (multiPass_) note << " walks_of_groups=" << groups_;
     k.scheduleNote = note.str();
     return k;
   }
@@ -530,6 +532,17 @@ class TileEmitter {
   int64_t grid_ = 1;
   bool raggedCols_ = false, raggedRows_ = false, raggedFlat_ = false;
   int reduceCount_ = 0;
+  // Rows too long to stay in registers: the row is walked in `groups_` groups of NCHUNK chunks per thread, once per
+  // reduction of the fusion and once more for the outputs; every walk recomputes the element values it needs from
+  // the kernel inputs (re-read from L2 / the last-level cache after the first walk).
+  // Rows whose length is not a multiple of the chunk: chunks keep their full width (the accesses are then only
+  // element-aligned, which the hardware serves), and the last chunk of a row starts at COLS - V, overlapping its
+  // neighbour by overlap_ elements that reductions skip and that are stored twice with the same value.
+  int overlap_ = 0;
+  bool multiPass_ = false;
+  int64_t groups_ = 1;
+  int pass_ = 0;                           // walk being emitted
+  std::vector<int> lastPassOfInput_;       // per graph input: the last walk that reads it
   bool nonTemporal_ = true;
   bool useBuffers_ = true;
   std::vector<bool> relaxed_;
@@ -676,6 +689,13 @@ class TileEmitter {
 
   // ------------------------------------------------------------------ schedule
   void pickSchedule() {
+    useBuffers_ = true;
+    for (int id : g_.inputs) {
+      if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
+    }
+    for (int id : g_.outputs) {
+      if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
+    }
     // Chunk width: 16 bytes of the widest element type that is moved chunk-wise, so no tensor needs more than one
     // 128-bit access per chunk (narrower tensors use 64- or 32-bit accesses, which still coalesce fully). Measured
     // on MI355X: many small contiguous accesses per wave beat fewer, wider ones.
@@ -694,8 +714,14 @@ class TileEmitter {
     if (!any) minSize = 4;
     int v = opt_.vec > 0 ? opt_.vec : static_cast<int>(16 / minSize);
     v = std::max(1, std::min(v, 16));
-    while (v > 1 && (cols_ % v) != 0) v >>= 1;
     if ((v & (v - 1)) != 0) v = 1;
+    bool inPlace = false;
+    for (const OpNode &op : g_.ops) inPlace = inPlace || op.kind == OpKind::Assign;
+    if (rowMode_ && useBuffers_ && !inPlace && opt_.vec == 0 && (cols_ % v) != 0 && cols_ >= 2 * v) {
+      overlap_ = static_cast<int>(v - cols_ % v);
+    } else {
+      while (v > 1 && (cols_ % v) != 0) v >>= 1;
+    }
     vec_ = v;
 
     if (rowMode_) {
@@ -704,18 +730,48 @@ class TileEmitter {
       // 79.5 % of the HBM peak with 1024 threads per row against 75.8 % with 512; 4096-wide f16 rows 75.0 % with 512
       // against 73.9 % with 256; 4096-wide bf16 rows with two streamed inputs the same either way. The row stays in
       // registers across all reductions of the fusion.
-      int targetPerThread = std::max(vec_, 8);
-      int tpr = opt_.threadsPerRow > 0 ? opt_.threadsPerRow
-                                       : std::min(1024, pow2AtLeast(ceilDiv(cols_, targetPerThread)));
-      tpr = std::max(1, std::min(tpr, 1024));
-      if ((tpr & (tpr - 1)) != 0) tpr = pow2AtLeast(tpr);
-      // never more threads than chunks in a row
-      while (tpr > 1 && static_cast<int64_t>(tpr) * vec_ > cols_ * 2) tpr >>= 1;
+      // Threads per row must be a power of two (butterfly reductions). Among the (threads, chunks per thread) pairs
+      // with at least 8 elements and at most 8 chunks per thread, the one that leaves the fewest idle chunk slots
+      // wins; between pairs within 3 % of each other the one with fewer chunks per thread. Measured on MI355X
+      // (% of the HBM peak): 4096-wide f16 rows 512 x 1 75.0, 256 x 2 73.9; 8192-wide bf16 rows 1024 x 1 79.5,
+      // 512 x 2 75.8; 4096-wide f32 rows 512 x 2 78.4, 1024 x 1 69.0; 768-wide bf16 LayerNorm 32 x 3 80.5, 128 x 1
+      // (25 % idle) 60.3; 5120-wide 128 x 5 78.7, 1024 x 1 (37 % idle) 50.3; 11008-wide f32 softmax 1024 x 3 72.6,
+      // 256 x 11 68.2.
+      const int64_t rowChunks = ceilDiv(cols_, vec_);
+      int tpr = 0;
+      if (opt_.threadsPerRow > 0) {
+        tpr = pow2AtLeast(std::max(1, std::min(opt_.threadsPerRow, 1024)));
+      } else {
+        const int64_t minChunks = std::max(1, 8 / vec_);
+        double best = 0;
+        for (int t = 1024; t >= 1; t >>= 1) {
+          const int64_t c = ceilDiv(rowChunks, t);
+          if (c < minChunks && t > 1) continue;
+          if (c > 8 && tpr != 0) break;
+          const double slots = static_cast<double>(t) * static_cast<double>(c) / static_cast<double>(rowChunks);
+          // candidates come with growing chunks per thread: a later one must be clearly better to win
+          if (tpr == 0 || slots < best / 1.03) {
+            tpr = t;
+            best = slots;
+          }
+        }
+      }
       tpr_ = tpr;
-      chunks_ = static_cast<int>(ceilDiv(cols_, static_cast<int64_t>(tpr_) * vec_));
-      if (static_cast<int64_t>(chunks_) * vec_ > 256) {
-        throw LoweringError("row of " + std::to_string(cols_) +
-                            " elements does not fit the register-resident row kernel (max 262144 per row)");
+      int64_t perThread = ceilDiv(cols_, static_cast<int64_t>(tpr_) * vec_);
+      // More than 64 values per thread and tensor do not stay in registers (measured: 65536-wide bf16 LayerNorm rows
+      // 22 % of the HBM peak, 131072-wide 11 %): walk the row in groups of `chunks` chunks per thread instead.
+      const int rowPasses = opt_.gemmVariant;  // 1: force the register-resident row, 2: force the walks
+      multiPass_ = rowPasses == 2 || (rowPasses != 1 && perThread * vec_ > 64);
+      if (multiPass_) {
+        const int64_t perGroup = opt_.chunks > 0 ? opt_.chunks : std::max<int64_t>(1, 32 / vec_);
+        chunks_ = static_cast<int>(std::min<int64_t>(perGroup, perThread));
+        groups_ = ceilDiv(perThread, chunks_);
+      } else {
+        if (perThread * vec_ > 256) {
+          throw LoweringError("row of " + std::to_string(cols_) + " elements does not fit the register-resident row kernel");
+        }
+        chunks_ = static_cast<int>(perThread);
+        groups_ = 1;
       }
       block_ = opt_.block > 0 ? opt_.block : 256;
       block_ = std::max(block_, tpr_);
@@ -723,7 +779,7 @@ class TileEmitter {
       if (block_ % tpr_ != 0 || block_ % 64 != 0) block_ = std::max(tpr_, 64);
       rowsPerBlock_ = block_ / tpr_;
       grid_ = ceilDiv(rows_, rowsPerBlock_);
-      raggedCols_ = (static_cast<int64_t>(chunks_) * tpr_ * vec_ != cols_);
+      raggedCols_ = (groups_ * chunks_ * tpr_ != rowChunks);
       raggedRows_ = (rows_ % rowsPerBlock_) != 0;
     } else {
       block_ = opt_.block > 0 ? opt_.block : 256;
@@ -879,13 +935,6 @@ class TileEmitter {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
     line(") {");
-    useBuffers_ = true;
-    for (int id : g_.inputs) {
-      if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
-    }
-    for (int id : g_.outputs) {
-      if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
-    }
     if (useBuffers_) {
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
         const TensorValue &t = g_.tensor(g_.inputs[i]);
@@ -919,14 +968,13 @@ class TileEmitter {
         line("  __shared__ double akg_scratch[2][BLOCK / 64];");
       }
       line("  long akg_rows[NCHUNK];");
-      line("  long akg_cols[NCHUNK];");
-      line("  bool akg_ok[NCHUNK];");
       line("#pragma unroll");
-      line("  for (int j = 0; j < NCHUNK; ++j) {");
-      line("    akg_rows[j] = akg_row;");
-      line("    akg_cols[j] = (static_cast<long>(j) * TPR + tcol) * V;");
-      line(std::string("    akg_ok[j] = ") + (raggedCols_ ? "akg_cols[j] < COLS;" : "true;"));
-      line("  }");
+      line("  for (int j = 0; j < NCHUNK; ++j) akg_rows[j] = akg_row;");
+      if (multiPass_) {
+        src_ << "  constexpr int GROUPS = " << groups_ << ";\n";
+      } else {
+        emitColumnsOfGroup("0");
+      }
     } else {
       line("  constexpr long NUMEL = ROWS * COLS;");
       line("  const long akg_base = static_cast<long>(blockIdx.x) * (static_cast<long>(BLOCK) * V * NCHUNK);");
@@ -951,8 +999,6 @@ class TileEmitter {
     }
     line("");
 
-    // loads of kernel inputs
-    for (size_t i = 0; i < g_.inputs.size(); ++i) emitInputLoad(i);
     // constants
     for (size_t t = 0; t < g_.tensors.size(); ++t) {
       const TensorValue &tv = g_.tensors[t];
@@ -962,12 +1008,21 @@ class TileEmitter {
       v.rank = ValRank::Const;
       v.ident = lowering::literalFor(tv.dtype, tv.constValue);
     }
+    if (multiPass_) {
+      emitWalks();
+      line("}");
+      return;
+    }
+    // loads of kernel inputs
+    for (size_t i = 0; i < g_.inputs.size(); ++i) emitInputLoad(i);
     // ops in description order
     for (size_t k = 0; k < g_.ops.size(); ++k) {
       const OpNode &op = g_.ops[k];
       if (absorbed_[k]) continue;
       if (lowering::isReduceKind(op.kind)) {
-        emitReduce(op);
+        emitReduceAccumulator(op);
+        emitReduceAccumulate(op);
+        emitReduceFinish(op);
       } else {
         emitElementwise(op, clampCast_[k]);
       }
@@ -979,6 +1034,150 @@ class TileEmitter {
       if (op.kind == OpKind::Assign) emitAssignStore(op);
     }
     line("}");
+  }
+
+  // Column of every chunk of the thread in group `group` of the row (an expression; "0" for the only group).
+  void emitColumnsOfGroup(const std::string &group) {
+    line("  long akg_cols[NCHUNK];");
+    line("  bool akg_ok[NCHUNK];");
+    if (overlap_ > 0) line("  bool akg_tail[NCHUNK];");
+    line("#pragma unroll");
+    line("  for (int j = 0; j < NCHUNK; ++j) {");
+    line("    akg_cols[j] = ((static_cast<long>(" + group + ") * NCHUNK + j) * TPR + tcol) * V;");
+    line(std::string("    akg_ok[j] = ") + (raggedCols_ ? "akg_cols[j] < COLS;" : "true;"));
+    if (overlap_ > 0) {
+      line("    akg_tail[j] = akg_cols[j] > COLS - V;");
+      line("    if (akg_tail[j]) akg_cols[j] = COLS - V;");
+    }
+    line("  }");
+  }
+
+  // Would the value be a per-element (Tile) value? Inputs that span the row are, and whatever is computed from one.
+  std::vector<bool> tileRanks() const {
+    std::vector<bool> tile(g_.tensors.size(), false);
+    for (size_t i = 0; i < g_.inputs.size(); ++i) tile[static_cast<size_t>(g_.inputs[i])] = access_[i].lastDimFull;
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      const OpNode &op = g_.ops[k];
+      if (lowering::isReduceKind(op.kind)) continue;
+      bool any = false;
+      for (int in : operandsOf(k)) any = any || tile[static_cast<size_t>(in)];
+      for (int out : op.outputs) tile[static_cast<size_t>(out)] = any;
+    }
+    return tile;
+  }
+
+  // Operands an op really reads (a Cast that absorbed its clamp reads the clamp's source).
+  std::vector<int> operandsOf(size_t k) const {
+    std::vector<int> in = g_.ops[k].inputs;
+    if (clampCast_[k].source >= 0) in[0] = clampCast_[k].source;
+    return in;
+  }
+
+  struct Walk {
+    std::vector<bool> ops;     // per op: recomputed in this walk
+    std::vector<bool> inputs;  // per graph input: loaded in this walk
+  };
+
+  // What a walk must load and recompute to have `targets` as per-element values.
+  Walk planWalk(const std::vector<int> &targets, const std::vector<bool> &tile) const {
+    Walk w;
+    w.ops.assign(g_.ops.size(), false);
+    w.inputs.assign(g_.inputs.size(), false);
+    std::vector<int> producer(g_.tensors.size(), -1);
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      for (int out : g_.ops[k].outputs) producer[static_cast<size_t>(out)] = static_cast<int>(k);
+    }
+    std::vector<int> todo = targets;
+    while (!todo.empty()) {
+      const int id = todo.back();
+      todo.pop_back();
+      if (!tile[static_cast<size_t>(id)]) continue;
+      const TensorValue &t = g_.tensor(id);
+      if (t.inputIndex >= 0 && producer[static_cast<size_t>(id)] < 0) {
+        w.inputs[static_cast<size_t>(t.inputIndex)] = true;
+        continue;
+      }
+      const int k = producer[static_cast<size_t>(id)];
+      if (k < 0 || w.ops[static_cast<size_t>(k)]) continue;
+      w.ops[static_cast<size_t>(k)] = true;
+      for (int in : operandsOf(static_cast<size_t>(k))) todo.push_back(in);
+    }
+    return w;
+  }
+
+  void emitWalkBody(const Walk &w) {
+    emitColumnsOfGroup("akg_g");
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      if (w.inputs[i]) emitInputLoad(i);
+    }
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      if (w.ops[k] && !absorbed_[k]) emitElementwise(g_.ops[k], clampCast_[k]);
+    }
+  }
+
+  // The row in several walks: per-row values (inputs with one element per row, reduce results and what is computed
+  // from them alone) are emitted once, in description order; every reduction gets a walk over the row that recomputes
+  // the elements it sums, and a last walk computes and stores the outputs.
+  void emitWalks() {
+    const std::vector<bool> tile = tileRanks();
+    std::vector<Walk> walks;
+    std::vector<size_t> walkOfOp(g_.ops.size(), 0);
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      if (absorbed_[k] || !lowering::isReduceKind(g_.ops[k].kind)) continue;
+      walkOfOp[k] = walks.size();
+      walks.push_back(planWalk({g_.ops[k].inputs[0]}, tile));
+    }
+    std::vector<int> finals;
+    for (int id : g_.outputs) {
+      if (g_.tensor(id).numel() == numel_) finals.push_back(id);
+    }
+    for (const OpNode &op : g_.ops) {
+      if (op.kind == OpKind::Assign) finals.push_back(op.outputs[0]);
+    }
+    walks.push_back(planWalk(finals, tile));
+    lastPassOfInput_.assign(g_.inputs.size(), -1);
+    for (size_t p = 0; p < walks.size(); ++p) {
+      for (size_t i = 0; i < g_.inputs.size(); ++i) {
+        if (walks[p].inputs[i]) lastPassOfInput_[i] = static_cast<int>(p);
+      }
+    }
+    // inputs with one element per row
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      if (!access_[i].lastDimFull) emitInputLoad(i);
+    }
+    for (size_t k = 0; k < g_.ops.size(); ++k) {
+      const OpNode &op = g_.ops[k];
+      if (absorbed_[k]) continue;
+      if (lowering::isReduceKind(op.kind)) {
+        if (!tile[static_cast<size_t>(op.inputs[0])]) {
+          throw LoweringError("op " + op.name + ": the reduced operand must span the innermost axis");
+        }
+        pass_ = static_cast<int>(walkOfOp[k]);
+        emitReduceAccumulator(op);
+        line("  for (int akg_g = 0; akg_g < GROUPS; ++akg_g) {");
+        emitWalkBody(walks[walkOfOp[k]]);
+        emitReduceAccumulate(op);
+        line("  }");
+        emitReduceFinish(op);
+      } else if (!tile[static_cast<size_t>(op.outputs[0])]) {
+        emitElementwise(op, clampCast_[k]);
+      }
+    }
+    pass_ = static_cast<int>(walks.size()) - 1;
+    if (!finals.empty()) {
+      line("  for (int akg_g = 0; akg_g < GROUPS; ++akg_g) {");
+      emitWalkBody(walks.back());
+      for (size_t i = 0; i < g_.outputs.size(); ++i) {
+        if (g_.tensor(g_.outputs[i]).numel() == numel_) emitOutputStore(i);
+      }
+      for (const OpNode &op : g_.ops) {
+        if (op.kind == OpKind::Assign) emitAssignStore(op);
+      }
+      line("  }");
+    }
+    for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      if (g_.tensor(g_.outputs[i]).numel() != numel_) emitOutputStore(i);
+    }
   }
 
   void emitInputLoad(size_t i) {
@@ -999,7 +1198,8 @@ class TileEmitter {
       line("  for (int j = 0; j < NCHUNK; ++j) {");
       src_ << "    if (akg_ok[j]) {\n";
       // a tensor as large as the iteration space is read exactly once: stream it
-      const bool streamed = nonTemporal_ && (t.numel() == numel_);
+      const bool streamed = nonTemporal_ && (t.numel() == numel_) &&
+                            (!multiPass_ || lastPassOfInput_[i] == pass_);
       src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">("
            << memRef("in" + std::to_string(i), rowOffsetExpr(a, "akg_rows[j]") + " + akg_cols[j]") << ", " << v.ident
            << "[j]);\n";
@@ -1127,7 +1327,20 @@ class TileEmitter {
     }
   }
 
-  void emitReduce(const OpNode &op) {
+  void emitReduceAccumulator(const OpNode &op) {
+    const int inId = op.inputs[0];
+    const int outId = op.outputs[0];
+    const DType od = g_.tensor(outId).dtype;
+    const std::string ct = computeTypeName(od);
+    const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+    if (std::string(computeTypeName(g_.tensor(inId).dtype)) != ct) {
+      throw LoweringError("op " + op.name + ": operand and result element types differ");
+    }
+    src_ << "  " << ct << " acc" << outId << " = " << spec.init << ";  // " << op.name << " -> " << g_.tensor(outId).name
+         << "\n";
+  }
+
+  void emitReduceAccumulate(const OpNode &op) {
     const int inId = op.inputs[0];
     const int outId = op.outputs[0];
     const ValInfo &in = vals_[static_cast<size_t>(inId)];
@@ -1135,32 +1348,38 @@ class TileEmitter {
       throw LoweringError("op " + op.name + ": the reduced operand must span the innermost axis");
     }
     const DType od = g_.tensor(outId).dtype;
-    const std::string ct = computeTypeName(od);
     const std::string tag = dtypeTag(od);
     const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
-    const std::string red = spec.combiner, init = spec.init;
-    const bool roundEachStep = spec.roundEachStep;
-    if (std::string(computeTypeName(g_.tensor(inId).dtype)) != ct) {
-      throw LoweringError("op " + op.name + ": operand and result element types differ");
-    }
-    ValInfo &v = vals_[static_cast<size_t>(outId)];
-    std::ostringstream nm;
-    nm << "u" << outId;
     const std::string acc = "acc" + std::to_string(outId);
-    src_ << "  " << ct << " " << acc << " = " << init << ";  // " << op.name << " -> " << g_.tensor(outId).name << "\n";
     line("#pragma unroll");
     line("  for (int j = 0; j < NCHUNK; ++j) {");
     line("#pragma unroll");
     line("    for (int e = 0; e < V; ++e) {");
-    std::string step = red + "::apply(" + acc + ", " + in.ident + "[j][e])";
-    if (roundEachStep) step = tag + "::rnd(" + step + ")";
-    if (raggedCols_) {
+    std::string step = spec.combiner + "::apply(" + acc + ", " + in.ident + "[j][e])";
+    if (spec.roundEachStep) step = tag + "::rnd(" + step + ")";
+    if (overlap_ > 0) {
+      src_ << "      if (akg_ok[j] && (!akg_tail[j] || e >= " << overlap_ << ")) " << acc << " = " << step << ";\n";
+    } else if (raggedCols_) {
       src_ << "      if (akg_ok[j]) " << acc << " = " << step << ";\n";
     } else {
       src_ << "      " << acc << " = " << step << ";\n";
     }
     line("    }");
     line("  }");
+  }
+
+  void emitReduceFinish(const OpNode &op) {
+    const int outId = op.outputs[0];
+    const DType od = g_.tensor(outId).dtype;
+    const std::string ct = computeTypeName(od);
+    const std::string tag = dtypeTag(od);
+    const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
+    const std::string red = spec.combiner;
+    const bool roundEachStep = spec.roundEachStep;
+    const std::string acc = "acc" + std::to_string(outId);
+    ValInfo &v = vals_[static_cast<size_t>(outId)];
+    std::ostringstream nm;
+    nm << "u" << outId;
     std::string scratch = tpr_ > 64 ? "reinterpret_cast<" + ct + " *>(akg_scratch[" + std::to_string(reduceCount_ & 1) + "])"
                                     : "static_cast<" + ct + " *>(nullptr)";
     src_ << "  const " << ct << " " << nm.str() << " = " << (roundEachStep ? tag + "::rnd(" : "")

@@ -32,6 +32,19 @@ FIXTURES = {
     "small_layernorm_residual_bf16_19x520": lambda n: op_desc.layernorm_residual(19, 520, "bfloat16", 1e-5, n),
     "small_quant_int8_residual_bf16_64x8192": lambda n: op_desc.quant_int8_residual(64, 8192, "bfloat16", n),
     "small_quant_int8_residual_bf16_37x1544": lambda n: op_desc.quant_int8_residual(37, 1544, "bfloat16", n),
+    # rows that are not a power of two of chunks (3, 5 and 6 chunks per thread) and rows too long for registers
+    # (walked in groups, once per reduction and once for the outputs; ragged last group)
+    "small_softmax_f16_9x768": lambda n: op_desc.softmax_last_axis(9, 768, "float16", n),
+    "small_layernorm_residual_bf16_5x5120": lambda n: op_desc.layernorm_residual(5, 5120, "bfloat16", 1e-5, n),
+    "small_layernorm_residual_bf16_3x11008": lambda n: op_desc.layernorm_residual(3, 11008, "bfloat16", 1e-5, n),
+    # rows that are not a multiple of the 16-byte chunk: element-aligned full-width accesses, overlapping last chunk
+    "small_softmax_f16_7x4095": lambda n: op_desc.softmax_last_axis(7, 4095, "float16", n),
+    "small_layernorm_residual_bf16_4x1001": lambda n: op_desc.layernorm_residual(4, 1001, "bfloat16", 1e-5, n),
+    "small_quant_int8_residual_bf16_3x2051": lambda n: op_desc.quant_int8_residual(3, 2051, "bfloat16", n),
+    "small_softmax_f16_3x70000": lambda n: op_desc.softmax_last_axis(3, 70000, "float16", n),
+    "small_softmax_f32_2x50257": lambda n: op_desc.softmax_last_axis(2, 50257, "float32", n),
+    "small_layernorm_residual_bf16_2x66000": lambda n: op_desc.layernorm_residual(2, 66000, "bfloat16", 1e-5, n),
+    "small_quant_int8_residual_bf16_2x131080": lambda n: op_desc.quant_int8_residual(2, 131080, "bfloat16", n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", True, n),
     "small_momentum_update_f32_37x130": lambda n: op_desc.momentum_update(37, 130, "float32", name=n),

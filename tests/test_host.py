@@ -398,10 +398,37 @@ def test_streamed_tensors_use_non_temporal_accesses_broadcast_vectors_do_not():
 
 
 def test_ragged_shapes_get_guards_and_aligned_shapes_do_not():
-    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f32_5x77.info")).source
-    assert "akg_ok[j] = akg_cols[j] < COLS;" in src and "akg_row_ok" in src
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f32_5x77.info"))
+    assert "akg_row_ok" in k.source
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f16_33x1000.info")).source
+    assert "akg_ok[j] = akg_cols[j] < COLS;" in src          # 125 chunks on 128 threads
+    # 77 is not a multiple of the 4-element chunk: chunks stay 4 wide, the last one starts at COLS - V and the three
+    # elements it shares with its neighbour are left out of the reductions
+    assert "constexpr int V = 4;" in k.source and "if (akg_tail[j]) akg_cols[j] = COLS - V;" in k.source
+    assert "(!akg_tail[j] || e >= 3)" in k.source
     src = driver.HipKernel.from_file(os.path.join(FIXTURES, "c2_softmax_f16_8192x4096.info")).source
-    assert "akg_ok[j] = true;" in src and "akg_row_ok" not in src
+    assert "akg_ok[j] = true;" in src and "akg_row_ok" not in src and "akg_tail" not in src
+
+
+def test_row_schedules_for_odd_and_long_rows():
+    def consts(name):
+        src = driver.HipKernel.from_file(os.path.join(FIXTURES, name + ".info")).source
+        return {m[0]: int(m[1]) for m in re.findall(r"constexpr int (\w+) = (\d+);", src)}, src
+    c, _ = consts("small_softmax_f16_9x768")                  # 96 chunks: 32 threads x 3, no idle slot
+    assert (c["TPR"], c["NCHUNK"], c["V"]) == (32, 3, 8)
+    c, _ = consts("small_layernorm_residual_bf16_5x5120")     # 640 chunks: 128 x 5
+    assert (c["TPR"], c["NCHUNK"]) == (128, 5)
+    c, _ = consts("small_layernorm_residual_bf16_3x11008")    # 1376 chunks: 512 x 3 (10 % idle) beats 1024 x 2 (33 %)
+    assert (c["TPR"], c["NCHUNK"]) == (512, 3)
+    c, _ = consts("c2_softmax_f16_8192x4096")
+    assert (c["TPR"], c["NCHUNK"]) == (512, 1)
+    # rows beyond 64 values per thread are walked in groups: one walk per reduction and one for the outputs, the
+    # input streamed (non-temporal) only in the last walk that reads it
+    c, src = consts("small_softmax_f16_3x70000")
+    assert (c["TPR"], c["NCHUNK"], c["GROUPS"]) == (1024, 4, 3) and src.count("for (int akg_g = 0; akg_g < GROUPS") == 3
+    assert re.findall(r"load_chunk<akg::f16, V, (true|false)>\(b_in0", src) == ["false", "false", "true"]
+    c, src = consts("small_layernorm_residual_bf16_2x66000")
+    assert c["GROUPS"] == 3 and src.count("for (int akg_g = 0; akg_g < GROUPS") == 3
 
 
 def test_elementwise_dimension_folding():
