@@ -758,10 +758,17 @@ class TileEmitter {
       }
       tpr_ = tpr;
       int64_t perThread = ceilDiv(cols_, static_cast<int64_t>(tpr_) * vec_);
-      // More than 64 values per thread and tensor do not stay in registers (measured: 65536-wide bf16 LayerNorm rows
-      // 22 % of the HBM peak, 131072-wide 11 %): walk the row in groups of `chunks` chunks per thread instead.
+      // More than 64 values per thread of one row-sized input, or 96 over all of them, do not stay in registers: walk the row in groups of
+      // `chunks` chunks per thread instead. The walks after the first re-read the row from HBM (rows in flight exceed
+      // L2), so the register-resident row is kept as long as it fits. Measured, % of the HBM peak, resident / walks:
+      // 65536-wide f16 softmax (1 input, 64 values) 62.6 / 46.2; 65536-wide bf16 LayerNorm (2 inputs) 21.9 / 61.3;
+      // 32768-wide LayerNorm 70.2 / 63.2; 131072-wide LayerNorm 10.6 / 50.0, softmax 30.1 / 42.3.
       const int rowPasses = opt_.gemmVariant;  // 1: force the register-resident row, 2: force the walks
-      multiPass_ = rowPasses == 2 || (rowPasses != 1 && perThread * vec_ > 64);
+      int64_t rowInputs = 0;
+      for (size_t i = 0; i < g_.inputs.size(); ++i) {
+        if (access_[i].lastDimFull && g_.tensor(g_.inputs[i]).numel() == numel_) ++rowInputs;
+      }
+      multiPass_ = rowPasses == 2 || (rowPasses != 1 && (perThread * vec_ > 64 || perThread * vec_ * rowInputs > 96));
       if (multiPass_) {
         const int64_t perGroup = opt_.chunks > 0 ? opt_.chunks : std::max<int64_t>(1, 32 / vec_);
         chunks_ = static_cast<int>(std::min<int64_t>(perGroup, perThread));
@@ -957,7 +964,10 @@ class TileEmitter {
       src_ << "  constexpr int TPR = " << tpr_ << ";\n";
       src_ << "  constexpr int RPB = " << rowsPerBlock_ << ";\n";
       line("  const int tcol = tid % TPR;");
-      line("  const long akg_row_raw = static_cast<long>(blockIdx.x) * RPB + (tid / TPR);");
+      // Launch order is kept even where rows share cache lines with their neighbours: giving every XCD a contiguous
+      // range of rows was measured slower (1000-wide f16 softmax 73.1 -> 67.8 % of the HBM peak, 4095-wide 63.0 -> 59.9).
+      line("  const int akg_wg = static_cast<int>(blockIdx.x);");
+      line("  const long akg_row_raw = static_cast<long>(akg_wg) * RPB + (tid / TPR);");
       if (raggedRows_) {
         line("  const bool akg_row_ok = akg_row_raw < ROWS;");
         line("  const long akg_row = akg_row_ok ? akg_row_raw : (ROWS - 1);");
@@ -1034,6 +1044,17 @@ class TileEmitter {
       if (op.kind == OpKind::Assign) emitAssignStore(op);
     }
     line("}");
+  }
+
+  // Non-temporal accesses pay off when a workgroup moves whole cache lines. Rows of a row kernel that are not a
+  // multiple of 64 bytes share their first and last line with the neighbouring rows, which other workgroups move:
+  // with the hint such a line is dropped before the neighbour comes for it (measured on 1000-wide bf16 rows:
+  // LayerNorm 62.8 % of the HBM peak with the hint, 68.4 % without; int8 quantisation 58.9 % and 66.9 %).
+  bool streamsWholeLines(int tensorId) const {
+    if (!nonTemporal_) return false;
+    if (!rowMode_) return true;
+    const int64_t rowBytes = cols_ * static_cast<int64_t>(dtypeSize(g_.tensor(tensorId).dtype));
+    return rowBytes % 64 == 0 || rowBytes >= 16384;  // two shared lines in 256 or more do not matter
   }
 
   // Column of every chunk of the thread in group `group` of the row (an expression; "0" for the only group).
@@ -1198,7 +1219,7 @@ class TileEmitter {
       line("  for (int j = 0; j < NCHUNK; ++j) {");
       src_ << "    if (akg_ok[j]) {\n";
       // a tensor as large as the iteration space is read exactly once: stream it
-      const bool streamed = nonTemporal_ && (t.numel() == numel_) &&
+      const bool streamed = streamsWholeLines(id) && (t.numel() == numel_) &&
                             (!multiPass_ || lastPassOfInput_[i] == pass_);
       src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">("
            << memRef("in" + std::to_string(i), rowOffsetExpr(a, "akg_rows[j]") + " + akg_cols[j]") << ", " << v.ident
@@ -1407,7 +1428,7 @@ class TileEmitter {
     std::string guard = "akg_ok[j]";
     if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
     const std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
-    src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (nonTemporal_ ? "true" : "false") << ">("
+    src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (streamsWholeLines(op.inputs[0]) ? "true" : "false") << ">("
          << memRef("in" + std::to_string(dst.inputIndex), offset) << ", " << v.ident << "[j]);  // " << op.name << " -> "
          << dst.name << "\n";
     line("  }");
@@ -1437,7 +1458,7 @@ class TileEmitter {
       std::string guard = "akg_ok[j]";
       if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
       std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
-      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (nonTemporal_ ? "true" : "false") << ">("
+      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (streamsWholeLines(id) ? "true" : "false") << ">("
            << memRef("out" + std::to_string(i), offset) << ", " << src
            << "[j]);\n";
       line("  }");

@@ -616,7 +616,14 @@ class IndexedEmitter {
     }
     src_ << "  const int tid = static_cast<int>(threadIdx.x);\n";
     // workgroup -> (other dims..., tile along t, tile along the innermost axis); the innermost tile index is fastest
-    src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
+    // output rows that are not whole cache lines: tiles that write parts of one line next to each other on one XCD
+    // (64 x 1000 x 1024 -> 64 x 1024 x 1000 bf16: 33.5 % of the HBM peak in launch order)
+    const int64_t outRowBytes = space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[0]).dtype));
+    if (outRowBytes % 64 != 0 && opt_.gemmVariant != 3 && grid_ >= 64) {
+      src_ << "  int akg_w = akg::xcd_contiguous_id(static_cast<int>(blockIdx.x), " << grid_ << ");\n";
+    } else {
+      src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
+    }
     src_ << "  const int i0 = (akg_w % " << tilesI << ") * TILE;\n  akg_w /= " << tilesI << ";\n";
     src_ << "  const int t0 = (akg_w % " << tilesT << ") * TILE;\n  akg_w /= " << tilesT << ";\n";
     canonical_.assign(rank, Ix());
@@ -654,7 +661,10 @@ class IndexedEmitter {
       stmt("const " + tagOf(st.input) + "::storage *src = in" + std::to_string(x.inputIndex) + " + " +
            linearize(xi, x.shape) + ";");
       const size_t bytes = static_cast<size_t>(st.vecX) * dtypeSize(x.dtype);
-      stmt("akg::Raw<" + std::to_string(bytes) + ">::type raw = __builtin_nontemporal_load(reinterpret_cast<const akg::Raw<" +
+      // the hint only where the tile rows are whole 64-byte pieces of a line (see the stores below)
+      const bool ntIn = opt_.nonTemporal != 0 && (x.shape.back() * static_cast<int64_t>(dtypeSize(x.dtype))) % 64 == 0;
+      stmt("akg::Raw<" + std::to_string(bytes) + ">::type raw = " +
+           (ntIn ? "__builtin_nontemporal_load(" : "*(") + "reinterpret_cast<const akg::Raw<" +
            std::to_string(bytes) + ">::type *>(src));");
       stmt("__builtin_memcpy(&akg_tile" + std::to_string(k) + "[r][q], &raw, " + std::to_string(bytes) + ");");
       --indent_;
@@ -681,8 +691,12 @@ class IndexedEmitter {
     Index first = canonical_;
     first[rank - 1] = Ix("inner0");
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
-      stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, true>(out" + std::to_string(i) + " + " +
-           linearize(first, space_) + ", o" + std::to_string(i) + ");");
+      // Non-temporal stores leave L2 at once: fine for whole lines, but a row segment that ends inside a line would
+      // reach memory as a partial write before the neighbouring tile adds the rest of the line.
+      const bool ntOut = opt_.nonTemporal != 0 &&
+                         (space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[i]).dtype))) % 64 == 0;
+      stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, " + (ntOut ? "true" : "false") + ">(out" + std::to_string(i) +
+           " + " + linearize(first, space_) + ", o" + std::to_string(i) + ");");
     }
     --indent_;
     stmt("}");

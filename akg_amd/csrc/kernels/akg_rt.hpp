@@ -290,6 +290,16 @@ AKG_DEV void store_one(Buffer buf, long index, typename DT::compute x) {
   Io::store(raw, buf, static_cast<u32>(index) * static_cast<u32>(sizeof(S)));
 }
 
+// Workgroups are handed to the 8 XCDs round robin (workgroup w runs on XCD w % 8), and every XCD has an L2 of its own.
+// When neighbouring workgroups write parts of the same cache line (rows that are not a multiple of the line), the two
+// parts end up in two L2s and reach memory as two partial writes. This renumbering gives every XCD one contiguous
+// range of the logical workgroup ids instead, so that neighbours share an L2: XCD x owns grid / 8 ids (one more for
+// the first grid % 8 XCDs), in launch order.
+AKG_DEV int xcd_contiguous_id(int w, int grid) {
+  const int q = grid / 8, r = grid % 8, x = w % 8;
+  return x * q + (x < r ? x : r) + w / 8;
+}
+
 template <typename DT, int V>
 AKG_DEV void fill_chunk(typename DT::compute (&dst)[V], typename DT::compute x) {
 #pragma unroll

@@ -391,10 +391,13 @@ def test_math_selection_follows_the_precision_demand():
 
 
 def test_streamed_tensors_use_non_temporal_accesses_broadcast_vectors_do_not():
-    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_layernorm_residual_bf16_19x520.info")).source
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_layernorm_residual_bf16_64x4096.info")).source
     loads = re.findall(r"load_chunk<akg::bf16, V, (true|false)>\(b_in(\d)", src)
     assert dict((i, nt) for nt, i in loads) == {"0": "true", "1": "false", "2": "false", "3": "true"}
     assert "store_chunk<akg::bf16, V, true>" in src
+    # rows of 1040 bytes share cache lines with their neighbours: no hint
+    src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_layernorm_residual_bf16_19x520.info")).source
+    assert "V, true>" not in src
 
 
 def test_ragged_shapes_get_guards_and_aligned_shapes_do_not():
