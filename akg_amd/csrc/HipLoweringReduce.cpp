@@ -70,7 +70,7 @@ class StreamReduceEmitter {
     k.workspaceBytes = workspaceBytes_;
     std::ostringstream note;
     note << "stream_reduce direction=" << (dirY_ ? "Y" : "X") << " outer=" << O_ << " reduced=" << R_ << " inner=" << I_
-         << " vec=" << vec_ << " lanes=" << lanes_ << " split=" << split_ << " rows_per_split=" << rps_
+         << " vec=" << vec_ << (overlapTail_ ? " (overlapping last chunk)" : "") << " lanes=" << lanes_ << " split=" << split_ << " rows_per_split=" << rps_
          << " block=" << kBlock << " grid=" << grid_ << " workspace=" << workspaceBytes_;
     k.scheduleNote = note.str();
     return k;
@@ -92,6 +92,7 @@ class StreamReduceEmitter {
   std::vector<const OpNode *> reduces_;
 
   int vec_ = 1, lanes_ = 64, split_ = 1, unroll_ = 4;
+  bool overlapTail_ = false;  // direction Y, I not a multiple of V: the last chunk of a row starts at I - V
   int64_t strips_ = 1, rps_ = 1, grid_ = 1, groups_ = 1;
   uint64_t workspaceBytes_ = 0;
   std::vector<uint64_t> partialOffset_;  // per reduction, bytes from the workspace base
@@ -267,7 +268,21 @@ class StreamReduceEmitter {
     // chunks run along the innermost dim of the fastest group and must not straddle it
     const int fastDim = innermostDim(dirY_ ? 2 : 1);
     const int64_t fastExtent = space_[static_cast<size_t>(fastDim)];
-    while (v > 1 && (fastExtent % v) != 0) v >>= 1;
+    // Column reductions over rows that are not a multiple of the chunk keep the full chunk width (accesses are then
+    // only element-aligned, which the hardware serves): the last lane of a row starts at I - V and shares columns
+    // with its neighbour; both sum them in the same order and write the same result. 4095-wide bf16 rows with
+    // single-element accesses reach 15 % of the HBM peak.
+    bool allBuffers = true;
+    auto tooLargeForBuffer = [&](int id) {
+      return g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31);
+    };
+    for (int id : g_.inputs) allBuffers = allBuffers && !tooLargeForBuffer(id);
+    for (int id : g_.outputs) allBuffers = allBuffers && !tooLargeForBuffer(id);
+    if (dirY_ && allBuffers && opt_.vec == 0 && fastExtent == I_ && (I_ % v) != 0 && I_ >= 2 * v) {
+      overlapTail_ = true;
+    } else {
+      while (v > 1 && (fastExtent % v) != 0) v >>= 1;
+    }
     vec_ = v;
     // Measured on MI355X (256 CUs) with 256 MiB .. 640 MiB inputs: column reductions stream best with 3 workgroups
     // per CU and two 16-byte loads in flight per thread (75 % of the 8 TB/s peak for two bf16 operands, 89 % for one
@@ -546,7 +561,11 @@ class StreamReduceEmitter {
       line("  const long akg_o = akg_group / STRIPS;");
       line("  const long akg_i_raw = ((akg_group % STRIPS) * LANES + li) * V;");
       line("  const bool col_ok = akg_i_raw < I;");
-      line("  const long akg_i = col_ok ? akg_i_raw : 0L;");
+      if (overlapTail_) {
+        line("  const long akg_i = col_ok ? (akg_i_raw < I - V ? akg_i_raw : I - V) : 0L;");
+      } else {
+        line("  const long akg_i = col_ok ? akg_i_raw : 0L;");
+      }
     } else {
       line("  const long akg_o = akg_group;");
       line("  __shared__ double akg_scratch[2][BLOCK / 64];");

@@ -58,6 +58,7 @@ FIXTURES = {
     "small_reduceall_min_f32_7x333": lambda n: op_desc.square_reduce([7, 333], [0, 1], "float32", False, "ReduceMin", n),
     "small_reducex_long_sqsum_f32_3x300000": lambda n: op_desc.square_reduce([3, 300000], [1], "float32", False, "ReduceSum", n),
     "small_biasgrad_bf16_2048x1024": lambda n: op_desc.bias_grad(2048, 1024, "bfloat16", n),
+    "small_biasgrad_bf16_1000x4095": lambda n: op_desc.bias_grad(1000, 4095, "bfloat16", n),
     "small_biasgrad_f32_100x37": lambda n: op_desc.bias_grad(100, 37, "float32", n),
     "small_sub_exp_reducesum_split_f32_4x96x160": lambda n: op_desc.sub_exp_reduce_y(4, 96, 160, "float32", n),
     "small_mean_absmax_all_f32_1000x1000": lambda n: op_desc.mean_absmax_all(1000, 1000, "float32", n),
