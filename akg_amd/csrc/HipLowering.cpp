@@ -134,8 +134,29 @@ std::string literalFor(DType t, double value) {
 }
 
 uint64_t countAlgorithmicBytes(const OpGraph &g) {
+  // Every kernel input and output once. An input that is only read through Slice / StridedSlice / Gather (of which it
+  // is the data operand) counts with the bytes those ops take out of it, if that is less: the rest of it is never
+  // needed, and counting it would overstate the bandwidth of a kernel that rightly leaves it alone.
   uint64_t bytes = 0;
-  for (int id : g.inputs) bytes += static_cast<uint64_t>(g.tensor(id).numel()) * dtypeSize(g.tensor(id).dtype);
+  for (int id : g.inputs) {
+    const TensorValue &t = g.tensor(id);
+    const uint64_t whole = static_cast<uint64_t>(t.numel()) * dtypeSize(t.dtype);
+    uint64_t taken = 0;
+    bool onlyTaken = true, used = false;
+    for (const OpNode &op : g.ops) {
+      for (size_t i = 0; i < op.inputs.size(); ++i) {
+        if (op.inputs[i] != id) continue;
+        used = true;
+        const bool takes = (op.kind == OpKind::Slice || op.kind == OpKind::StridedSlice || op.kind == OpKind::Gather) && i == 0;
+        if (!takes) {
+          onlyTaken = false;
+        } else {
+          taken += static_cast<uint64_t>(g.tensor(op.outputs[0]).numel()) * dtypeSize(t.dtype);
+        }
+      }
+    }
+    bytes += (used && onlyTaken) ? std::min(whole, taken) : whole;
+  }
   for (int id : g.outputs) bytes += static_cast<uint64_t>(g.tensor(id).numel()) * dtypeSize(g.tensor(id).dtype);
   return bytes;
 }

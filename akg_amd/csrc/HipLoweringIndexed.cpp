@@ -99,6 +99,8 @@ class IndexedEmitter {
   std::ostringstream src_;
   std::vector<int64_t> space_;  // iteration space: the shape of the outputs
   int vec_ = 1;
+  bool overlapTail_ = false;   // V does not divide the innermost extent: the last chunk of a row overlaps its neighbour
+  int64_t chunksPerRow_ = 1;
   int64_t grid_ = 1;
   // tiled mode (LDS-staged transposed inputs)
   static constexpr int kTile = 64;
@@ -174,11 +176,25 @@ class IndexedEmitter {
     int v = opt_.vec > 0 ? opt_.vec : static_cast<int>(16 / widest);
     v = std::max(1, std::min(v, 16));
     if ((v & (v - 1)) != 0) v = 1;
-    while (v > 1 && (space_.back() % v) != 0) v >>= 1;
+    // An innermost extent that V does not divide keeps the full chunk width: the last chunk of a row then starts
+    // at extent - V and shares elements with its neighbour (both write the same values); such chunks are only
+    // element-aligned in memory.
+    if (opt_.vec == 0 && (space_.back() % v) != 0 && space_.back() >= 2 * v) {
+      overlapTail_ = true;
+    } else {
+      while (v > 1 && (space_.back() % v) != 0) v >>= 1;
+    }
     vec_ = v;
-    const int64_t chunks = numel / vec_;
+    chunksPerRow_ = (space_.back() + vec_ - 1) / vec_;
+    const int64_t chunks = numel / space_.back() * chunksPerRow_;
     grid_ = std::max<int64_t>(1, (chunks + kBlock - 1) / kBlock);
     pickStaging();
+    if (!staged_.empty() && overlapTail_) {
+      // the LDS-tiled transposes keep their own chunking: narrower chunks instead
+      overlapTail_ = false;
+      while (vec_ > 1 && (space_.back() % vec_) != 0) vec_ >>= 1;
+      chunksPerRow_ = space_.back() / vec_;
+    }
     if (!staged_.empty()) {
       grid_ = 1;
       for (size_t d = 0; d < space_.size(); ++d) {
@@ -548,14 +564,15 @@ class IndexedEmitter {
     return var;
   }
 
-  // A kernel input read at `idx`: if its V elements for this chunk are V consecutive, aligned elements in memory and
-  // the read happens for the whole chunk or not at all, load them once in front of the element loop and return the
+  // A kernel input read at `idx`: if its V elements for this chunk are V consecutive elements in memory (aligned or
+  // not) and the read happens for the whole chunk or not at all, load them once in front of the element loop and return the
   // expression of the current element; otherwise return "".
   std::string tryChunkLoad(int id, const Index &idx) {
     const TensorValue &t = g_.tensor(id);
     if (vec_ < 2 || t.shape.empty() || idx.empty() || opt_.gemmVariant == 2) return std::string();
     const Ix &last = idx.back();
-    if (last.kind != 1 || !last.aligned || !last.early || (t.shape.back() % vec_) != 0) return std::string();
+    if (last.kind != 1 || !last.early || t.shape.back() < vec_) return std::string();
+    const bool alignedAccess = last.aligned && (t.shape.back() % vec_) == 0;
     for (size_t d = 0; d + 1 < idx.size(); ++d) {
       if (idx[d].kind != 0 || !idx[d].early) return std::string();
     }
@@ -570,7 +587,8 @@ class IndexedEmitter {
       const std::string arr = fresh("w");
       const std::string tag = tagOf(id);
       hoisted(ctOf(id) + " " + arr + "[V] = {};");
-      hoisted(std::string(guard.empty() ? "" : "if (" + guard + ") ") + "akg::load_chunk<" + tag + ", V, false>(in" +
+      hoisted(std::string(guard.empty() ? "" : "if (" + guard + ") ") +
+              (alignedAccess ? "akg::load_chunk<" + tag + ", V, false>(in" : "akg::load_chunk_unaligned<" + tag + ", V>(in") +
               std::to_string(t.inputIndex) + " + " + offset + ", " + arr + ");");
       it = hoistedLoads_.emplace(key, arr).first;
     }
@@ -735,20 +753,28 @@ class IndexedEmitter {
     for (int64_t d : space_) numel *= d;
     src_ << "  constexpr int V = " << vec_ << ";\n";
     src_ << "  const int chunk = static_cast<int>(blockIdx.x) * " << kBlock << " + static_cast<int>(threadIdx.x);\n";
-    src_ << "  if (chunk >= " << numel / vec_ << ") return;\n";
-    src_ << "  const int base = chunk * V;  // linear position of this thread's first element\n";
+    src_ << "  if (chunk >= " << numel / space_.back() * chunksPerRow_ << ") return;\n";
+    if (overlapTail_) {
+      src_ << "  int akg_inner = (chunk % " << chunksPerRow_ << ") * V;\n";
+      src_ << "  if (akg_inner > " << space_.back() - vec_ << ") akg_inner = " << space_.back() - vec_ << ";\n";
+      src_ << "  const int base = (chunk / " << chunksPerRow_ << ") * " << space_.back()
+           << " + akg_inner;  // linear position of this thread's first element\n";
+    } else {
+      src_ << "  const int base = chunk * V;  // linear position of this thread's first element\n";
+    }
     indent_ = 1;
     scopes_.clear();
     scopes_.emplace_back();
-    // index of the chunk's first element; the innermost coordinate advances with e and never wraps (V divides it)
+    // index of the chunk's first element; the innermost coordinate advances with e and never wraps
     Index start = delinearize("base", space_);
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       stmt(ctOf(g_.outputs[i]) + " o" + std::to_string(i) + "[V];");
     }
     Index idx = start;
     if (space_.back() != 1) {
-      stmt("const int inner0 = " + start.back().s + ";  // a multiple of V: V divides the innermost extent");
-      idx.back() = affine("inner0", true, true);
+      stmt("const int inner0 = " + start.back().s + ";" +
+           (overlapTail_ ? "" : "  // a multiple of V: V divides the innermost extent"));
+      idx.back() = affine("inner0", !overlapTail_, true);
     }
     openElementLoop(indent_);
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
@@ -757,8 +783,8 @@ class IndexedEmitter {
     }
     closeElementLoop();
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
-      stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, false>(out" + std::to_string(i) + " + base, o" +
-           std::to_string(i) + ");");
+      stmt(std::string("akg::store_chunk") + (overlapTail_ ? "_unaligned<" : "<") + tagOf(g_.outputs[i]) + ", V" +
+           (overlapTail_ ? "" : ", false") + ">(out" + std::to_string(i) + " + base, o" + std::to_string(i) + ");");
     }
     src_ << "}\n";
   }

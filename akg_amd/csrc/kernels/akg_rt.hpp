@@ -182,6 +182,25 @@ AKG_DEV void store_chunk(typename DT::storage *__restrict__ p, const typename DT
   }
 }
 
+// Chunks that are only element-aligned (a slice that starts at an odd column, rows that are not a multiple of the
+// chunk): gfx950 serves unaligned 16-byte global accesses, and with the alignment stated truthfully the compiler still
+// issues one wide instruction.
+template <typename DT, int V>
+AKG_DEV void load_chunk_unaligned(const typename DT::storage *__restrict__ p, typename DT::compute (&dst)[V]) {
+  typename DT::storage tmp[V];
+  __builtin_memcpy(tmp, p, sizeof(tmp));
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(tmp[e]);
+}
+
+template <typename DT, int V>
+AKG_DEV void store_chunk_unaligned(typename DT::storage *__restrict__ p, const typename DT::compute (&src)[V]) {
+  typename DT::storage tmp[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) tmp[e] = DT::store(src[e]);
+  __builtin_memcpy(p, tmp, sizeof(tmp));
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // Buffer-addressed variants (tensors below 2 GiB): a 128-bit descriptor per tensor plus a 32-bit byte offset per
 // access, so address arithmetic is 32-bit, and the cache policy of every access is explicit:

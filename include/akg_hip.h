@@ -61,7 +61,8 @@ typedef struct akg_hip_kernel_info {
   char operator_type[32];             /* fusion class, OperatorIdentify.cpp:51-93 */
   uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json */
   uint32_t block[3];                  /* threadIdx.x/y/z extents */
-  uint64_t algorithmic_bytes;         /* bytes of every input and output, each counted once */
+  uint64_t algorithmic_bytes;         /* bytes of every input and output, each counted once (an input that is only
+                                         sliced or gathered from: the bytes taken out of it) */
   uint64_t algorithmic_ops;           /* 2*M*N*K of the contraction, 0 for bandwidth-bound families */
   int32_t cache_hit;                  /* 1 if the code object came from the artifact directory */
   uint64_t workspace_bytes;           /* device scratch the handle owns per device (streaming reductions), else 0 */
