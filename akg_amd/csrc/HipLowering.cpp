@@ -533,7 +533,7 @@ class TileEmitter {
          << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
          << " block=" << block_ << " grid=" << grid_;
     if (overlap_ > 0) note << " tail_overlap=" << overlap_;
-    if (multiPass_) note << " walks_of_groups=" << groups_;
+    if (multiPass_) note << " walks_of_groups=" << groups_ << (packedRow_ ? " (row packed in registers)" : "");
     k.scheduleNote = note.str();
     return k;
   }
@@ -561,6 +561,10 @@ class TileEmitter {
   // neighbour by overlap_ elements that reductions skip and that are stored twice with the same value.
   int overlap_ = 0;
   bool multiPass_ = false;
+  // Walks over a row of 16-bit inputs that fits the registers in its memory image (half its float image): the row
+  // is loaded once, kept packed, and every walk unpacks the group it works on.
+  bool packedRow_ = false;
+  std::vector<bool> packedInput_;          // per graph input: held packed in registers across the walks
   int64_t groups_ = 1;
   int pass_ = 0;                           // walk being emitted
   std::vector<int> lastPassOfInput_;       // per graph input: the last walk that reads it
@@ -784,14 +788,38 @@ class TileEmitter {
       // L2), so the register-resident row is kept as long as it fits. Measured, % of the HBM peak, resident / walks:
       // 65536-wide f16 softmax (1 input, 64 values) 62.6 / 46.2; 65536-wide bf16 LayerNorm (2 inputs) 21.9 / 61.3;
       // 32768-wide LayerNorm 70.2 / 63.2; 131072-wide LayerNorm 10.6 / 50.0, softmax 30.1 / 42.3.
-      const int rowPasses = opt_.gemmVariant;  // 1: force the register-resident row, 2: force the walks
+      const int rowPasses = opt_.gemmVariant;  // 1: force the register-resident row, 2: force the walks, 4: walks, packed if possible
       int64_t rowInputs = 0;
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
         if (access_[i].lastDimFull && g_.tensor(g_.inputs[i]).numel() == numel_) ++rowInputs;
       }
-      multiPass_ = rowPasses == 2 || (rowPasses != 1 && (perThread * vec_ > 64 || perThread * vec_ * rowInputs > 96));
+      multiPass_ = rowPasses == 2 || rowPasses == 4 || (rowPasses != 1 && (perThread * vec_ > 64 || perThread * vec_ * rowInputs > 96));
+      packedInput_.assign(g_.inputs.size(), false);
+      // Measured, % of the HBM peak, float values resident / packed walks: 32768-wide bf16 quantisation 61.6 / 73.0,
+      // 32768-wide f16 softmax 67.8 / 70.0, 65536-wide 62.1 / 66.4, 32768-wide LayerNorm 69.6 / 67.4; at 16384 and
+      // below the same within a point or two. So rows of 16-bit inputs on 1024 threads go packed from 64 values per
+      // thread on.
+      const bool preferPacked = rowPasses == 0 && tpr_ == 1024 && perThread * vec_ * rowInputs >= 64;
+      if ((multiPass_ || preferPacked) && useBuffers_ && rowPasses != 2) {
+        // registers (32-bit) per thread for the packed row; 64 leave room for one group's float values
+        int64_t packedRegs = 0;
+        bool narrowOnly = true;
+        for (size_t i = 0; i < g_.inputs.size(); ++i) {
+          const TensorValue &t = g_.tensor(g_.inputs[i]);
+          if (!(access_[i].lastDimFull && t.numel() == numel_)) continue;
+          if (dtypeSize(t.dtype) > 2) narrowOnly = false;
+          packedRegs += perThread * ((vec_ * static_cast<int64_t>(dtypeSize(t.dtype)) + 3) / 4);
+        }
+        if (narrowOnly && packedRegs > 0 && packedRegs <= 64) {
+          packedRow_ = true;
+          multiPass_ = true;
+          for (size_t i = 0; i < g_.inputs.size(); ++i) {
+            packedInput_[i] = access_[i].lastDimFull && g_.tensor(g_.inputs[i]).numel() == numel_;
+          }
+        }
+      }
       if (multiPass_) {
-        const int64_t perGroup = opt_.chunks > 0 ? opt_.chunks : std::max<int64_t>(1, 32 / vec_);
+        const int64_t perGroup = opt_.chunks > 0 ? opt_.chunks : std::max<int64_t>(1, (packedRow_ ? 16 : 32) / vec_);
         chunks_ = static_cast<int>(std::min<int64_t>(perGroup, perThread));
         groups_ = ceilDiv(perThread, chunks_);
       } else {
@@ -1187,6 +1215,30 @@ class TileEmitter {
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       if (!access_[i].lastDimFull) emitInputLoad(i);
     }
+    if (packedRow_) {
+      // the row, once, as it lies in memory
+      for (size_t i = 0; i < g_.inputs.size(); ++i) {
+        if (packedInput_[i]) src_ << "  akg::RawChunk<" << tagOf(g_.inputs[i]) << ", V> r_in" << i << "[GROUPS * NCHUNK];\n";
+      }
+      line("#pragma unroll");
+      line("  for (int akg_g = 0; akg_g < GROUPS; ++akg_g) {");
+      emitColumnsOfGroup("akg_g");
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      for (size_t i = 0; i < g_.inputs.size(); ++i) {
+        if (!packedInput_[i]) continue;
+        const std::string tag = tagOf(g_.inputs[i]);
+        src_ << "    if (akg_ok[j]) {\n";
+        src_ << "      akg::load_raw_chunk<" << tag << ", V, " << (streamsWholeLines(g_.inputs[i]) ? "true" : "false") << ">(b_in"
+             << i << ", " << rowOffsetExpr(access_[i], "akg_rows[j]") << " + akg_cols[j], r_in" << i
+             << "[akg_g * NCHUNK + j]);\n";
+        src_ << "    } else {\n";
+        src_ << "      akg::zero_raw_chunk<" << tag << ", V>(r_in" << i << "[akg_g * NCHUNK + j]);\n";
+        src_ << "    }\n";
+      }
+      line("  }");
+      line("  }");
+    }
     for (size_t k = 0; k < g_.ops.size(); ++k) {
       const OpNode &op = g_.ops[k];
       if (absorbed_[k]) continue;
@@ -1196,17 +1248,27 @@ class TileEmitter {
         }
         pass_ = static_cast<int>(walkOfOp[k]);
         emitReduceAccumulator(op);
+        if (packedRow_) line("#pragma unroll");
         line("  for (int akg_g = 0; akg_g < GROUPS; ++akg_g) {");
         emitWalkBody(walks[walkOfOp[k]]);
         emitReduceAccumulate(op);
         line("  }");
         emitReduceFinish(op);
+        if (packedRow_) {
+          for (size_t i = 0; i < g_.inputs.size(); ++i) {
+            if (!packedInput_[i]) continue;
+            line("#pragma unroll");
+            src_ << "  for (int c = 0; c < GROUPS * NCHUNK; ++c) akg::forget_unpacked<" << tagOf(g_.inputs[i]) << ", V>(r_in" << i
+                 << "[c]);\n";
+          }
+        }
       } else if (!tile[static_cast<size_t>(op.outputs[0])]) {
         emitElementwise(op, clampCast_[k]);
       }
     }
     pass_ = static_cast<int>(walks.size()) - 1;
     if (!finals.empty()) {
+      if (packedRow_) line("#pragma unroll");
       line("  for (int akg_g = 0; akg_g < GROUPS; ++akg_g) {");
       emitWalkBody(walks.back());
       for (size_t i = 0; i < g_.outputs.size(); ++i) {
@@ -1231,6 +1293,16 @@ class TileEmitter {
     const std::string tag = tagOf(id);
     const std::string ct = ctOf(id);
     std::ostringstream nm;
+    if (a.lastDimFull && packedRow_ && packedInput_[i]) {
+      v.rank = ValRank::Tile;
+      nm << "t_in" << i;
+      v.ident = nm.str();
+      src_ << "  " << ct << " " << v.ident << "[NCHUNK][V];\n";
+      line("#pragma unroll");
+      src_ << "  for (int j = 0; j < NCHUNK; ++j) akg::unpack_chunk<" << tag << ", V>(r_in" << i << "[akg_g * NCHUNK + j], "
+           << v.ident << "[j]);\n";
+      return;
+    }
     if (a.lastDimFull) {
       v.rank = ValRank::Tile;
       nm << "t_in" << i;

@@ -289,6 +289,47 @@ AKG_DEV void store_chunk(Buffer buf, long index, const typename DT::compute (&sr
   for (int k = 0; k < kPieces; ++k) Io::store(raw[k], buf, off + k * kPiece);
 }
 
+// A chunk kept as it came from memory (a 16-bit row held in registers takes half the space of its float image);
+// unpack_chunk converts it whenever the values are needed.
+template <typename DT, int V>
+struct RawChunk {
+  static constexpr int kBytes = static_cast<int>(sizeof(typename DT::storage)) * V;
+  static constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  static constexpr int kPieces = kBytes / kPiece;
+  typename BufferIo<kPiece, kAuxDefault>::type raw[kPieces];
+};
+
+template <typename DT, int V, bool STREAM = false>
+AKG_DEV void load_raw_chunk(Buffer buf, long index, RawChunk<DT, V> &dst) {
+  typedef RawChunk<DT, V> R;
+  typedef BufferIo<R::kPiece, STREAM ? kAuxStreamLoad : kAuxDefault> Io;
+  const u32 off = static_cast<u32>(index) * static_cast<u32>(sizeof(typename DT::storage));
+#pragma unroll
+  for (int k = 0; k < R::kPieces; ++k) dst.raw[k] = Io::load(buf, off + k * R::kPiece);
+}
+
+template <typename DT, int V>
+AKG_DEV void zero_raw_chunk(RawChunk<DT, V> &dst) {
+#pragma unroll
+  for (int k = 0; k < RawChunk<DT, V>::kPieces; ++k) dst.raw[k] = {};
+}
+
+// Makes the compiler forget what it knows about the registers of a packed chunk, so that the float values unpacked
+// from it in one walk over the row are not kept alive for the next walk (which would defeat the packing).
+template <typename DT, int V>
+AKG_DEV void forget_unpacked(RawChunk<DT, V> &c) {
+#pragma unroll
+  for (int k = 0; k < RawChunk<DT, V>::kPieces; ++k) asm volatile("" : "+v"(c.raw[k]));
+}
+
+template <typename DT, int V>
+AKG_DEV void unpack_chunk(const RawChunk<DT, V> &src, typename DT::compute (&dst)[V]) {
+  typename DT::storage tmp[V];
+  __builtin_memcpy(tmp, src.raw, RawChunk<DT, V>::kBytes);
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(tmp[e]);
+}
+
 template <typename DT>
 AKG_DEV typename DT::compute load_one(Buffer buf, long index) {
   typedef typename DT::storage S;

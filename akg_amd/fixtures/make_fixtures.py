@@ -43,6 +43,7 @@ FIXTURES = {
     "small_quant_int8_residual_bf16_3x2051": lambda n: op_desc.quant_int8_residual(3, 2051, "bfloat16", n),
     "small_softmax_f16_3x70000": lambda n: op_desc.softmax_last_axis(3, 70000, "float16", n),
     "small_softmax_f32_2x50257": lambda n: op_desc.softmax_last_axis(2, 50257, "float32", n),
+    "small_layernorm_residual_bf16_2x57000": lambda n: op_desc.layernorm_residual(2, 57000, "bfloat16", 1e-5, n),
     "small_layernorm_residual_bf16_2x66000": lambda n: op_desc.layernorm_residual(2, 66000, "bfloat16", 1e-5, n),
     "small_quant_int8_residual_bf16_2x131080": lambda n: op_desc.quant_int8_residual(2, 131080, "bfloat16", n),
     "small_gemm_i8_dequant_bias_gelu_256x512x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(256, 512, 256, "bfloat16", False, n),

@@ -425,13 +425,18 @@ def test_row_schedules_for_odd_and_long_rows():
     assert (c["TPR"], c["NCHUNK"]) == (512, 3)
     c, _ = consts("c2_softmax_f16_8192x4096")
     assert (c["TPR"], c["NCHUNK"]) == (512, 1)
-    # rows beyond 64 values per thread are walked in groups: one walk per reduction and one for the outputs, the
-    # input streamed (non-temporal) only in the last walk that reads it
+    # rows beyond 64 values per thread are walked in groups: one walk per reduction and one for the outputs. A row of
+    # 16-bit inputs that fits 64 registers per thread in its memory image is loaded once and kept packed ...
     c, src = consts("small_softmax_f16_3x70000")
-    assert (c["TPR"], c["NCHUNK"], c["GROUPS"]) == (1024, 4, 3) and src.count("for (int akg_g = 0; akg_g < GROUPS") == 3
-    assert re.findall(r"load_chunk<akg::f16, V, (true|false)>\(b_in0", src) == ["false", "false", "true"]
+    assert (c["TPR"], c["NCHUNK"], c["GROUPS"]) == (1024, 2, 5) and src.count("for (int akg_g = 0; akg_g < GROUPS") == 4
+    assert src.count("load_raw_chunk<akg::f16, V, true>(b_in0") == 1 and src.count("unpack_chunk<akg::f16, V>(r_in0") == 3
+    assert "load_chunk<akg::f16" not in src and src.count("forget_unpacked") == 2
+    c, src = consts("small_layernorm_residual_bf16_2x57000")
+    assert c["GROUPS"] == 4 and "r_in0[GROUPS * NCHUNK]" in src and "r_in3[GROUPS * NCHUNK]" in src and "r_in1" not in src
+    # ... a longer one is re-read by every walk, with the non-temporal hint only in the last walk that reads it
     c, src = consts("small_layernorm_residual_bf16_2x66000")
-    assert c["GROUPS"] == 3 and src.count("for (int akg_g = 0; akg_g < GROUPS") == 3
+    assert c["GROUPS"] == 3 and src.count("for (int akg_g = 0; akg_g < GROUPS") == 3 and "RawChunk" not in src
+    assert re.findall(r"load_chunk<akg::bf16, V, (true|false)>\(b_in0", src) == ["false", "false", "true"]
 
 
 def test_elementwise_dimension_folding():
