@@ -58,6 +58,11 @@ FIXTURES = {
     "small_reduceall_sqsum_f32_768x512": lambda n: op_desc.square_reduce([768, 512], [0, 1], "float32", False, "ReduceSum", n),
     "small_reduceall_min_f32_7x333": lambda n: op_desc.square_reduce([7, 333], [0, 1], "float32", False, "ReduceMin", n),
     "small_reducex_long_sqsum_f32_3x300000": lambda n: op_desc.square_reduce([3, 300000], [1], "float32", False, "ReduceSum", n),
+    # kept axes between reduced ones: batch-norm statistics (contiguous runs of H*W), and a [4,5,6,16] sum over axes 0, 2
+    "small_bnstats_bf16_8x6x7x12": lambda n: op_desc.batchnorm_stats(8, 6, 7, 12, "bfloat16", n),
+    "small_bnstats_f32_32x16x28x28": lambda n: op_desc.batchnorm_stats(32, 16, 28, 28, "float32", n),
+    "small_reducey_sqsum_f32_4x5x6x16_axes02": lambda n: op_desc.square_reduce([4, 5, 6, 16], [0, 2], "float32", False, "ReduceSum", n),
+    "small_reducey_max_f16_3x4x50x9_axes02_keep": lambda n: op_desc.square_reduce([3, 4, 50, 9], [0, 2], "float16", True, "ReduceMax", n),
     "small_biasgrad_bf16_2048x1024": lambda n: op_desc.bias_grad(2048, 1024, "bfloat16", n),
     "small_biasgrad_bf16_1000x4095": lambda n: op_desc.bias_grad(1000, 4095, "bfloat16", n),
     "small_biasgrad_f32_100x37": lambda n: op_desc.bias_grad(100, 37, "float32", n),

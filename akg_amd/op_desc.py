@@ -257,6 +257,17 @@ def bias_grad(rows, cols, dtype="bfloat16", name=None):
     return b.dumps([dgamma, dbeta])
 
 
+def batchnorm_stats(n, c, h, w, dtype="bfloat16", name=None):
+    """Per-channel sum and sum of squares of x[N,C,H,W] over N, H and W (the statistics pass of a training batch norm):
+    the kept axis lies between the reduced ones."""
+    b = DescBuilder(name or "Fused_Cast_ReduceSum_Mul_ReduceSum_bnstats_%s_%dx%dx%dx%d" % (_SHORT[dtype], n, c, h, w))
+    x = b.input([n, c, h, w], dtype)
+    xf = b.cast(x, "float32") if dtype != "float32" else x
+    s1 = b.reduce("ReduceSum", xf, [0, 2, 3], False)
+    s2 = b.reduce("ReduceSum", b.mul(xf, xf), [0, 2, 3], False)
+    return b.dumps([s1, s2])
+
+
 def sub_exp_reduce_y(outer, reduced, inner, dtype="float32", name=None):
     """Two outputs, as the reference's Fused_Sub_Exp_ReduceSum_split: e = exp(x - m) (full shape, stored while
     streaming) and s = sum over the middle axis of e, with m broadcast along the reduced axis."""

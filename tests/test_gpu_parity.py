@@ -16,7 +16,7 @@ from oracle import cpu_ref
 pytestmark = pytest.mark.gpu
 
 FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "akg_amd", "fixtures")
-STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all")
+STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all", "bnstats")
 ALL_SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
 SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS) and "segment_sum" not in n]
 STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS)]
