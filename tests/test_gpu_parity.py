@@ -10,7 +10,7 @@ import os
 import numpy as np
 import pytest
 
-from akg_amd import driver, harness
+from akg_amd import driver, harness, op_desc
 from oracle import cpu_ref
 
 pytestmark = pytest.mark.gpu
@@ -108,6 +108,56 @@ def test_full_size_bias_gradient_column_sums():
 def test_full_size_batched_transpose_bias_add():
     """[32,2048,1024] -> [32,1024,2048] bfloat16 transpose fused with a bias add (indexed family), every element."""
     check_fixture("n3_transpose_bias_add_bf16_32x2048x1024.info", seed=harness.BASE_SEED + 12, openmp=True)
+
+
+def test_tensors_of_two_gib_and_more_are_addressed_with_64_bit_offsets(tmp_path):
+    """float32 [34000, 16384] is 2.08 GiB: beyond what a buffer descriptor with 32-bit offsets reaches, so the kernels
+    address it through plain pointers. Elementwise (bias add, every element against the oracle's OpenMP build), column
+    sums (against float64 numpy) and a softmax over f16 [34000, 32768] (first and last rows against the oracle of a
+    64-row description: rows are independent, and a wrapped offset would show at the far end)."""
+    rows, cols = 34000, 16384
+    b = op_desc.DescBuilder("big_bias_add_f32_%dx%d" % (rows, cols))
+    x, v = b.input([rows, cols], "float32"), b.input([cols], "float32")
+    text = b.dumps([b.add(x, v)])
+    path = os.path.join(str(tmp_path), "big_bias_add.info")
+    open(path, "w").write(text)
+    rng = np.random.default_rng(7)
+    xs = rng.standard_normal((rows, cols), dtype=np.float32)
+    vs = rng.standard_normal(cols, dtype=np.float32)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert "make_buffer" not in kernel.source
+    print("case big bias add", flush=True)
+    got = run_on_gpu(kernel, [xs, vs])[0]
+    expect = cpu_ref.CpuKernel(path, openmp=True, rebuild=True)([xs, vs])[0]
+    assert np.array_equal(got, expect)
+    del got, expect
+    print("case big column sum", flush=True)
+    text = op_desc.square_reduce([rows, cols], [0], "float32", False, "ReduceSum", name="big_colsum_f32_%dx%d" % (rows, cols))
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family == "stream_reduce" and "make_buffer(in0" not in kernel.source
+    got = run_on_gpu(kernel, [xs])[0]
+    exact = np.einsum("rc,rc->c", xs, xs, dtype=np.float64)
+    ok, msg = harness.compare_reassociated(got, exact, "float32", rows)
+    print("  column sums: %s" % msg, flush=True)
+    assert ok, msg
+    del xs
+    print("case big softmax", flush=True)
+    rows, cols = 34000, 32768
+    kernel = driver.HipKernel(op_desc.softmax_last_axis(rows, cols, "float16"), out_dir=None)
+    assert "make_buffer" not in kernel.source
+    xh = (rng.standard_normal((rows, cols), dtype=np.float32) * 2.0).astype(np.float16)
+    got = run_on_gpu(kernel, [xh])[0]
+    small = op_desc.softmax_last_axis(64, cols, "float16", name="big_softmax_rows_sample")
+    spath = os.path.join(str(tmp_path), "big_softmax_rows_sample.info")
+    open(spath, "w").write(small)
+    ref = cpu_ref.CpuKernel(spath, openmp=True, rebuild=True)
+    for first in (0, rows // 2, rows - 64):
+        expect = ref([np.ascontiguousarray(xh[first:first + 64])])[0]
+        ok, msg = harness.compare(got[first:first + 64], expect, "float16")
+        print("  rows %d..%d: %s" % (first, first + 63, msg), flush=True)
+        assert ok, msg
+    sums = got[::997].astype(np.float64).sum(axis=1)
+    assert np.all(np.abs(sums - 1.0) < 2e-2)      # every sampled row is a distribution
 
 
 @pytest.mark.parametrize("name", FULL)
