@@ -88,7 +88,7 @@ const OpTableEntry kOpTable[] = {
   {"Concat", OpKind::Concat},
   {"Reshape", OpKind::Reshape},
   {"Transpose", OpKind::Transpose},
-  {"Split", OpKind::Unsupported},
+  {"Split", OpKind::Slice},   // becomes one Slice per result (see the translator)
   {"Pad", OpKind::Pad},
   {"Gather", OpKind::Gather},
   {"InplaceAssign", OpKind::Assign},
@@ -384,7 +384,9 @@ class GraphBuilder {
       }
       (void)fakeOutput;
       std::vector<int64_t> inferred;  // result shape derived from the operands (empty: take the declared one)
-      if (node.kind == OpKind::Transpose || node.kind == OpKind::Tile || node.kind == OpKind::Slice ||
+      if (node.name == "Split") {
+        // handled below, once the result tensors exist
+      } else if (node.kind == OpKind::Transpose || node.kind == OpKind::Tile || node.kind == OpKind::Slice ||
           node.kind == OpKind::StridedSlice || node.kind == OpKind::Pad || node.kind == OpKind::Concat ||
           node.kind == OpKind::Gather) {
         inferred = parseDataMovement(&node, attrs, inputDesc, readShape(outputDesc[0]));
@@ -407,8 +409,47 @@ class GraphBuilder {
         node.outputs.push_back(id);
         operandList_[tensorName] = id;
       }
+      if (node.name == "Split") {
+        splitIntoSlices(node, attrs);
+        continue;
+      }
       graph_.ops.push_back(node);
     }
+  }
+
+  // Split (convertSplitOp :1206-1232 reads attr "axis"; the reference has no lowering for mindspore.split): result k
+  // is the piece of the operand along `axis` that follows the pieces before it, each as long as its declared shape
+  // says. One Slice node per result, all named Split.
+  void splitIntoSlices(const OpNode &node, const json::Value &attrs) {
+    if (node.inputs.size() != 1) throw TranslateError("op Split: needs exactly one operand");
+    const TensorValue x = graph_.tensor(node.inputs[0]);
+    const size_t rank = x.shape.size();
+    int64_t axis = 0;
+    if (const json::Value *a = findAttr(attrs, "axis")) axis = a->isArray() ? a->asIntVector().at(0) : static_cast<int64_t>(a->asDouble());
+    if (axis < 0) axis += static_cast<int64_t>(rank);
+    if (axis < 0 || axis >= static_cast<int64_t>(rank)) throw TranslateError("op Split: axis out of range");
+    int64_t offset = 0;
+    for (int out : node.outputs) {
+      const TensorValue &y = graph_.tensor(out);
+      if (y.dtype != x.dtype) throw TranslateError("op Split: operand and result element types differ");
+      if (y.shape.size() != rank) throw TranslateError("op Split: a result must have the rank of the operand");
+      for (size_t d = 0; d < rank; ++d) {
+        if (static_cast<int64_t>(d) != axis && y.shape[d] != x.shape[d]) {
+          throw TranslateError("op Split: a result differs from the operand outside the split axis");
+        }
+      }
+      OpNode piece = node;
+      piece.kind = OpKind::Slice;
+      piece.outputs.assign(1, out);
+      piece.begin.assign(rank, 0);
+      piece.begin[static_cast<size_t>(axis)] = offset;
+      piece.strides.assign(rank, 1);
+      offset += y.shape[static_cast<size_t>(axis)];
+      if (offset > x.shape[static_cast<size_t>(axis)]) throw TranslateError("op Split: the results exceed the operand");
+      graph_.tensors[static_cast<size_t>(out)].producer = static_cast<int>(graph_.ops.size());
+      graph_.ops.push_back(piece);
+    }
+    if (offset != x.shape[static_cast<size_t>(axis)]) throw TranslateError("op Split: the results do not cover the operand");
   }
 
   // Attributes of the data-movement ops, checked against the declared result shape.
@@ -696,9 +737,10 @@ class GraphBuilder {
       } else if (n != t.numel()) {
         throw TranslateError("output " + tensorName + ": shape differs between output_desc and its producer");
       }
-      if (t.outputIndex >= 0) throw TranslateError("output " + tensorName + " is listed twice");
+      // A value may be returned more than once (the reference looks every output up by name and returns what it
+      // finds; its own Split test description lists one result twice): every listing gets an output buffer.
       if (t.inputIndex >= 0) throw TranslateError("output " + tensorName + " aliases a kernel input");
-      t.outputIndex = static_cast<int>(i);
+      if (t.outputIndex < 0) t.outputIndex = static_cast<int>(i);
       graph_.outputs.push_back(it->second);
     }
     if (graph_.outputs.empty()) throw TranslateError("op description has no outputs");

@@ -77,6 +77,8 @@ FIXTURES = {
     "small_transpose_bias_add_f32_2x100x200": lambda n: op_desc.transpose_bias_add(2, 100, 200, "float32", n),
     "small_transpose_sum_f32_2x70x3x80_perm0321": lambda n: op_desc.transpose_sum([2, 70, 3, 80], [0, 3, 2, 1], "float32", n),
     "small_transpose_sum_f16_130x66_perm10": lambda n: op_desc.transpose_sum([130, 66], [1, 0], "float16", n),
+    "small_split_swiglu_bf16_37x264": lambda n: op_desc.split_swiglu(37, 264, "bfloat16", n),
+    "small_split_swiglu_f32_5x9": lambda n: op_desc.split_swiglu(5, 9, "float32", n),
     "small_embedding_lookup_bf16_1000x96_ids5x33": lambda n: op_desc.embedding_lookup_scale(1000, 96, 5, 33, "bfloat16", n),
     "small_embedding_lookup_f32_50x7_ids3x4": lambda n: op_desc.embedding_lookup_scale(50, 7, 3, 4, "float32", n),
     # UnsortedSegmentSum (segment_sum family): short slices, a wide slice tiled over workgroups, 16-bit accumulation

@@ -358,6 +358,36 @@ def concat(b, x, y, axis):
     return out
 
 
+def split(b, x, sizes, axis):
+    """One Split op with len(sizes) results: consecutive pieces of `x` along `axis`."""
+    outs = []
+    for n in sizes:
+        shape = list(x.shape)
+        shape[axis] = int(n)
+        outs.append(Tensor("output_0_%d" % b._n_out, shape, x.dtype))
+        b._n_out += 1
+    b.ops.append({
+        "attr": [{"data_type": "int", "name": "output_num", "value": len(sizes)},
+                 {"data_type": "listInt", "name": "size_splits", "value": [int(n) for n in sizes]},
+                 {"data_type": "int", "name": "axis", "value": int(axis)}],
+        "impl_path": "", "input_desc": [[x.desc()]], "name": "Split",
+        "output_desc": [t.desc(with_value=False) for t in outs]})
+    return outs
+
+
+def split_swiglu(rows, width, dtype="bfloat16", name=None):
+    """SwiGLU on a fused projection: x[rows, 2*width] is split into gate and up halves along the last axis,
+    out = gate * sigmoid(gate) * up."""
+    b = DescBuilder(name or "Fused_Split_SwiGLU_%s_%dx%d" % (_SHORT[dtype], rows, width))
+    x = b.input([rows, 2 * width], dtype)
+    gate, up = split(b, x, [width, width], 1)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    gf, uf = f(gate), f(up)
+    sig = b.unary("Reciprocal", b.add(b.unary("Exp", b.unary("Neg", gf)), b.const(1.0, "float32")))
+    y = b.mul(b.mul(gf, sig), uf)
+    return b.dumps([b.cast(y, dtype) if dtype != "float32" else y])
+
+
 def transpose_bias_add(batch, rows, cols, dtype="bfloat16", name=None):
     """out[b, c, r] = x[b, r, c] + bias[r] (bias broadcast along the new innermost axis is [rows]): the layout change
     in front of an attention score product, fused with an elementwise op."""

@@ -34,9 +34,9 @@ import subprocess
 import sys
 
 try:
-    from oracle.view_attrs import VIEW_OPS, view_params
+    from oracle.view_attrs import VIEW_OPS, view_params, expand_split
 except ImportError:  # run as a script from inside oracle/
-    from view_attrs import VIEW_OPS, view_params
+    from view_attrs import VIEW_OPS, view_params, expand_split
 
 FLOATS = ("float16", "bfloat16", "float32", "float64")
 INTS = ("int8", "int16", "int32", "int64")
@@ -187,6 +187,7 @@ class Op:
 def parse(desc):
     """JSON document -> (name, inputs, ops, outputs); same reading rules as the reference translator
     (TranslateToMindsporeDialect.cpp:295-415, 793-808, 1273-1318)."""
+    desc = expand_split(desc)
     tensors = {}
     inputs = []
     for entry in desc["input_desc"]:
@@ -715,9 +716,14 @@ class Emitter:
             t.buffer = "in%d" % arg
             self.emit("const %s *%s = (const %s *)packed[%d];" % (C_STORAGE[t.dtype], t.buffer, C_STORAGE[t.dtype], arg))
             arg += 1
+        copies = []  # a value listed more than once among the outputs: the later listings are copies of the first
         for k, t in enumerate(self.outputs):
-            t.buffer = "out%d" % k
-            self.emit("%s *%s = (%s *)packed[%d];" % (C_STORAGE[t.dtype], t.buffer, C_STORAGE[t.dtype], arg))
+            if t in self.outputs[:k]:
+                self.emit("%s *dup%d = (%s *)packed[%d];" % (C_STORAGE[t.dtype], k, C_STORAGE[t.dtype], arg))
+                copies.append((k, t))
+            else:
+                t.buffer = "out%d" % k
+                self.emit("%s *%s = (%s *)packed[%d];" % (C_STORAGE[t.dtype], t.buffer, C_STORAGE[t.dtype], arg))
             arg += 1
         for op in self.ops:
             out = op.output
@@ -750,6 +756,8 @@ class Emitter:
                 self.emit_segment_sum(op)
             else:
                 self.emit_elementwise(op)
+        for k, t in copies:
+            self.emit("memcpy(dup%d, %s, sizeof(%s) * %dL);" % (k, t.buffer, C_STORAGE[t.dtype], max(1, t.numel)))
         for b in self.temps:
             self.emit("free(%s);" % b)
         L.append("}")

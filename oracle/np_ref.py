@@ -22,7 +22,7 @@ import json
 
 import numpy as np
 
-from oracle.view_attrs import VIEW_OPS, view_params
+from oracle.view_attrs import VIEW_OPS, view_params, expand_split
 
 FLOATS = ("float16", "bfloat16", "float32", "float64")
 NP_DTYPE = {"bool": np.bool_, "int8": np.int8, "int16": np.int16, "int32": np.int32, "int64": np.int64,
@@ -159,6 +159,7 @@ def evaluate(desc, inputs, updates=None):
     `updates` to receive {input position: new external array} (the caller's arrays are left alone)."""
     if isinstance(desc, str):
         desc = json.loads(desc)
+    desc = expand_split(desc)
     env = {}
     dtypes = {}
     shapes = {}

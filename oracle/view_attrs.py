@@ -20,6 +20,38 @@ Rules followed (reference file:line):
                 undefined in the reference (tensor.extract); both restatements and the kernels clamp them into the axis.
 """
 
+def expand_split(desc):
+    """Split -> one Slice per result. The reference translates Split (attr "axis", TranslateToMindsporeDialect.cpp
+    :1206-1232) but has no lowering for it, so the meaning restated here is the operator's own: result k is the piece of
+    the operand along `axis` that follows the pieces before it, as long as its declared shape says. Returns a
+    description without Split entries (the same object if there is none)."""
+    if not any(od["name"] == "Split" for od in desc["op_desc"]):
+        return desc
+    out = dict(desc)
+    out["op_desc"] = []
+    for od in desc["op_desc"]:
+        if od["name"] != "Split":
+            out["op_desc"].append(od)
+            continue
+        attrs = {a["name"]: a["value"] for a in (od.get("attr") or [])}
+        src = od["input_desc"][0][0]
+        rank = len(src["shape"])
+        axis = attrs.get("axis", 0)
+        axis = int(axis[0] if isinstance(axis, list) else axis)
+        axis = axis + rank if axis < 0 else axis
+        offset = 0
+        for piece in od["output_desc"]:
+            begin = [0] * rank
+            begin[axis] = offset
+            offset += piece["shape"][axis]
+            out["op_desc"].append({
+                "name": "Slice", "impl_path": "", "input_desc": [[src]], "output_desc": [piece],
+                "attr": [{"data_type": "listInt", "name": "begin", "value": begin},
+                         {"data_type": "listInt", "name": "size", "value": list(piece["shape"])}]})
+        assert offset == src["shape"][axis], "Split: the results do not cover the operand"
+    return out
+
+
 VIEW_OPS = ("Transpose", "Tile", "Slice", "StridedSlice", "Pad", "Concat", "Gather")
 
 

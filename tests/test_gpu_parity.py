@@ -169,8 +169,7 @@ def test_full_size_config_matches_oracle(name):
 REF_INFO = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "ref_info")
 # Every op description of the reference's own test tree (akg-mlir/tests/st/**), copied as data under their own names
 # (".info_failed" / ".info.failed" are the reference's markers for cases its CPU pipeline does not pass).
-# Not run: Split (the reference has no lowering for mindspore.split either).
-REF_SKIPPED = ("Fused_Split_",)
+REF_SKIPPED = ()
 
 
 def _is_dynamic(path):
@@ -178,7 +177,7 @@ def _is_dynamic(path):
     return any(x < 0 for e in d["input_desc"] for x in e[0].get("shape", [1]))
 
 
-REF_ALL = sorted(f for f in os.listdir(REF_INFO) if ".info" in f and not f.startswith(REF_SKIPPED))
+REF_ALL = sorted(f for f in os.listdir(REF_INFO) if ".info" in f and not (REF_SKIPPED and f.startswith(REF_SKIPPED)))
 REF_DYNAMIC = [f for f in REF_ALL if _is_dynamic(os.path.join(REF_INFO, f))]
 REF_STREAM = [f for f in REF_ALL if f not in REF_DYNAMIC and "ReduceSum_split" in f]
 REF_SEGMENT = [f for f in REF_ALL if f.startswith("Fused_UnsortedSegmentSum_")]

@@ -69,8 +69,8 @@ def _static(name):
     return not any(x < 0 for e in d["input_desc"] for x in e[0].get("shape", [1]))
 
 
-# every static description of the reference's test tree but the Split one (two results share a tensor name there)
-STATIC_REF = sorted(f for f in os.listdir(REF_INFO) if ".info" in f and not f.startswith("Fused_Split_") and _static(f))
+# every static description of the reference's test tree
+STATIC_REF = sorted(f for f in os.listdir(REF_INFO) if ".info" in f and _static(f))
 
 
 @pytest.mark.parametrize("name", STATIC_REF)

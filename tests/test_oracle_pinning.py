@@ -404,6 +404,22 @@ def test_unsorted_segment_sum_adds_slices_in_index_order(tmp_path):
     assert harness.bf16_bits_to_f32(n_out[0]).reshape(-1).tolist() == [256.0, 0.0]
 
 
+def test_split_gives_consecutive_pieces_along_the_axis(tmp_path):
+    """Split into three unequal pieces along axis 1 against numpy's split; each piece goes through an op of its own so
+    that a swapped or shifted piece shows. (The reference translates Split but has no lowering for it.)"""
+    b = op_desc.DescBuilder("pin_split")
+    x = b.input([3, 10, 2], "float32")
+    p0, p1, p2 = op_desc.split(b, x, [2, 5, 3], 1)
+    text = b.dumps([b.unary("Neg", p0), b.mul(p1, b.const(3.0, "float32")), b.unary("Abs", p2)])
+    data = np.arange(60, dtype=np.float32).reshape(3, 10, 2) - 17.0
+    _, c_out, n_out = build_and_run(text, [data], tmp_path)
+    a0, a1, a2 = np.split(data, [2, 7], axis=1)
+    for got in (c_out, n_out):
+        assert np.array_equal(np.asarray(got[0]).reshape(a0.shape), -a0)
+        assert np.array_equal(np.asarray(got[1]).reshape(a1.shape), a1 * 3.0)
+        assert np.array_equal(np.asarray(got[2]).reshape(a2.shape), np.abs(a2))
+
+
 def test_assign_writes_the_value_over_its_first_operand(tmp_path):
     """Momentum step in float32 against the formula written out in numpy: v <- 0.9 v + g, p <- p - 0.01 v. The C
     restatement updates the caller's input arrays in place, the numpy one reports the updates."""
