@@ -265,6 +265,7 @@ bool isElementwiseKind(OpKind k) {
     case OpKind::Concat:
     case OpKind::Gather:
     case OpKind::SegmentSum:
+    case OpKind::ArgMax:
       return false;
     default:
       return !isReduceKind(k);
@@ -1129,7 +1130,7 @@ class TileEmitter {
     for (size_t k = 0; k < g_.ops.size(); ++k) {
       const OpNode &op = g_.ops[k];
       if (lowering::isReduceKind(op.kind)) continue;
-      bool any = false;
+      bool any = op.kind == OpKind::Iota;
       for (int in : operandsOf(k)) any = any || tile[static_cast<size_t>(in)];
       for (int out : op.outputs) tile[static_cast<size_t>(out)] = any;
     }
@@ -1375,6 +1376,10 @@ class TileEmitter {
       if (vi.rowvecNoKeep) anyNoKeep = true;
     }
     if (rank == ValRank::Const) rank = ValRank::Uniform;
+    if (op.kind == OpKind::Iota) {
+      if (!rowMode_) throw LoweringError("op Iota: only produced for ArgMax over the innermost axis");
+      rank = ValRank::Tile;
+    }
     if (anyTile && anyNoKeep) {
       throw LoweringError("op " + op.name + ": a reduce result without keep_dims cannot be broadcast against the "
                           "reduced tensor; reshape it to [...,1] first");
@@ -1397,7 +1402,9 @@ class TileEmitter {
                                 std::string(computeTypeName(outT.dtype)) == "float" &&
                                 std::string(computeTypeName(g_.tensor(op.inputs[0]).dtype)) == "float" &&
                                 std::string(computeTypeName(g_.tensor(op.inputs[1]).dtype)) == "float";
-    if (fused.source >= 0) {
+    if (op.kind == OpKind::Iota) {
+      expr = "static_cast<int>(akg_cols[j] + e)";   // the column of the element: the innermost axis of the row space
+    } else if (fused.source >= 0) {
       expr = "akg::clamp_cast(" + operands[0] + ", " + lowering::literalFor(DType::F32, fused.lo) + ", " +
              lowering::literalFor(DType::F32, fused.hi) + ")";
     } else if (uniformDivisor) {
@@ -1573,8 +1580,34 @@ class TileEmitter {
 
 }  // namespace
 
-LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options) {
-  if (graph.ops.empty()) throw LoweringError("op description has no ops");
+LoweredKernel lowerToHip(const OpGraph &described, const LoweringOptions &options) {
+  if (described.ops.empty()) throw LoweringError("op description has no ops");
+  bool hasArgMax = false;
+  for (const OpNode &op : described.ops) hasArgMax = hasArgMax || op.kind == OpKind::ArgMax;
+  OpGraph expanded;
+  if (hasArgMax) {
+    expanded = described;
+    try {
+      expandArgMax(&expanded);
+    } catch (const TranslateError &e) {
+      throw LoweringError(e.what());
+    }
+    for (const OpNode &op : expanded.ops) {
+      if (op.kind != OpKind::Iota) continue;
+      const std::vector<int64_t> &shape = expanded.tensor(op.outputs[0]).shape;
+      size_t last = shape.size();
+      for (size_t d = shape.size(); d-- > 0;) {
+        if (shape[d] > 1) {
+          last = d;
+          break;
+        }
+      }
+      if (static_cast<size_t>(op.concatAxis) != last || last + 1 != shape.size()) {
+        throw LoweringError("op ArgMax: only the innermost axis has a kernel yet");
+      }
+    }
+  }
+  const OpGraph &graph = hasArgMax ? expanded : described;
   bool hasMatMul = false;
   for (const OpNode &op : graph.ops) {
     if (op.kind == OpKind::MatMul) hasMatMul = true;

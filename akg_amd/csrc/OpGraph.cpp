@@ -81,7 +81,7 @@ const OpTableEntry kOpTable[] = {
   {"ReduceAll", OpKind::ReduceAll},
   {"ReduceAny", OpKind::ReduceAny},
   {"ElemAny", OpKind::ReduceAny},
-  {"ArgMax", OpKind::Unsupported},
+  {"ArgMax", OpKind::ArgMax},
   {"BroadcastTo", OpKind::BroadcastTo},
   {"Slice", OpKind::Slice},
   {"Tile", OpKind::Tile},
@@ -314,7 +314,7 @@ class GraphBuilder {
         }
       }
 
-      if (isReduceKind(node.kind)) {
+      if (isReduceKind(node.kind) || node.kind == OpKind::ArgMax) {
         // Axis from the second input's value or from attr "axis" (:1280-1300); keep_dims defaults to false.
         std::vector<int64_t> axes;
         if (inputDesc.size() == 2) {
@@ -777,6 +777,10 @@ OperatorTemplate templateOfOp(const OpGraph &g, const OpNode &op) {
     case OpKind::Unknown:
     case OpKind::Unsupported:
       return OperatorTemplate::Default;
+    case OpKind::ArgMax:
+      return OperatorTemplate::Reduction;
+    case OpKind::Iota:
+      return OperatorTemplate::Elementwise;
     default: {
       // Elementwise when every operand has the result's shape, Broadcast otherwise (elementwiseMatch,
       // OperatorIdentify.cpp:34-48).
@@ -898,6 +902,8 @@ const char *opKindName(OpKind k) {
     case OpKind::Pad: return "pad";
     case OpKind::Concat: return "concat";
     case OpKind::Gather: return "gather";
+    case OpKind::ArgMax: return "argmax";
+    case OpKind::Iota: return "iota";
     case OpKind::SegmentSum: return "unsorted_segment_sum";
     case OpKind::MatMul: return "matmul";
     case OpKind::AddN: return "addn";
@@ -958,6 +964,89 @@ OpGraph translateJsonToOpGraph(const std::string &jsonText, const ShapeBinding *
   pruneDeadOps(&g);
   identifyOperator(&g);
   return g;
+}
+
+void expandArgMax(OpGraph *graph) {
+  bool any = false;
+  for (const OpNode &op : graph->ops) any = any || op.kind == OpKind::ArgMax;
+  if (!any) return;
+  const double kBig = 2147483647.0;
+  std::vector<OpNode> ops;
+  std::vector<int> newIndex;  // not needed by callers: producers are re-derived below
+  auto addTensor = [&](const std::string &name, DType dtype, const std::vector<int64_t> &shape) {
+    TensorValue t;
+    t.name = name;
+    t.dtype = dtype;
+    t.shape = shape;
+    graph->tensors.push_back(t);
+    return static_cast<int>(graph->tensors.size()) - 1;
+  };
+  auto addConst = [&](const std::string &name, double value) {
+    const int id = addTensor(name, DType::I32, {1});
+    graph->tensors[static_cast<size_t>(id)].isConst = true;
+    graph->tensors[static_cast<size_t>(id)].constValue = value;
+    return id;
+  };
+  auto emit = [&](OpKind kind, const char *name, std::vector<int> inputs, int output) {
+    OpNode n;
+    n.kind = kind;
+    n.name = name;
+    n.inputs = std::move(inputs);
+    n.outputs.assign(1, output);
+    ops.push_back(n);
+    return &ops.back();
+  };
+  int serial = 0;
+  for (const OpNode &op : graph->ops) {
+    if (op.kind != OpKind::ArgMax) {
+      ops.push_back(op);
+      continue;
+    }
+    const int x = op.inputs.at(0);
+    const int out = op.outputs.at(0);
+    const std::vector<int64_t> inShape = graph->tensor(x).shape;
+    const DType xType = graph->tensor(x).dtype, outType = graph->tensor(out).dtype;
+    if (op.axes.size() != 1) throw TranslateError("op ArgMax: exactly one axis is supported");
+    if (isFloatType(outType) || outType == DType::Bool) throw TranslateError("op ArgMax: the result must be an integer tensor");
+    if (xType == DType::Bool) throw TranslateError("op ArgMax: a bool operand is not supported");
+    const size_t axis = static_cast<size_t>(op.axes[0]);
+    if (inShape[axis] >= (1LL << 31) - 1) throw TranslateError("op ArgMax: axis too long");
+    std::vector<int64_t> kept = inShape;
+    kept[axis] = 1;
+    const std::string base = "argmax" + std::to_string(serial++) + "_";
+    const int m = addTensor(base + "max", xType, kept);
+    OpNode *r = emit(OpKind::ReduceMax, "ReduceMax", {x}, m);
+    r->axes = op.axes;
+    r->keepDims = true;
+    const int eq = addTensor(base + "hit", DType::Bool, inShape);
+    emit(OpKind::Equal, "Equal", {x, m}, eq);
+    const int iota = addTensor(base + "iota", DType::I32, inShape);
+    emit(OpKind::Iota, "Iota", {}, iota)->concatAxis = static_cast<int64_t>(axis);
+    const int big = addConst(base + "big", kBig);
+    const int sel = addTensor(base + "pos", DType::I32, inShape);
+    emit(OpKind::Select, "Select", {eq, iota, big}, sel);
+    const std::vector<int64_t> outShape = graph->tensor(out).shape;
+    const int first = addTensor(base + "first", DType::I32, outShape);
+    r = emit(OpKind::ReduceMin, "ReduceMin", {sel}, first);
+    r->axes = op.axes;
+    r->keepDims = op.keepDims;
+    const int none = addTensor(base + "none", DType::Bool, outShape);
+    emit(OpKind::Equal, "Equal", {first, big}, none);
+    const int zero = addConst(base + "zero", 0.0);
+    if (outType == DType::I32) {
+      emit(OpKind::Select, "Select", {none, zero, first}, out);
+    } else {
+      const int fixed = addTensor(base + "fixed", DType::I32, outShape);
+      emit(OpKind::Select, "Select", {none, zero, first}, fixed);
+      emit(OpKind::Cast, "Cast", {fixed}, out);
+    }
+  }
+  graph->ops.swap(ops);
+  for (TensorValue &t : graph->tensors) t.producer = -1;
+  for (size_t k = 0; k < graph->ops.size(); ++k) {
+    for (int id : graph->ops[k].outputs) graph->tensors[static_cast<size_t>(id)].producer = static_cast<int>(k);
+  }
+  (void)newIndex;
 }
 
 void removeRedundantReduces(OpGraph *graph) {

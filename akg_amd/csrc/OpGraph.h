@@ -49,6 +49,10 @@ enum class OpKind {
   Transpose, Tile, Slice, StridedSlice, Pad, Concat, Gather,
   // UnsortedSegmentSum: out[ids[i], ...] += data[i, ...] over the index positions i in increasing order
   SegmentSum,
+  // ArgMax over one axis: position of the first greatest element (integer result). Lowered by expandArgMax.
+  ArgMax,
+  // the index of every element along one axis of its (result) shape, int32; only produced by expandArgMax
+  Iota,
   // contraction
   MatMul,
   // n-ary
@@ -132,6 +136,13 @@ OpGraph translateJsonToOpGraph(const std::string &jsonText, const ShapeBinding *
 
 // True if the description has a -1 dimension on any kernel input, op result or kernel output.
 bool descriptionIsDynamic(const std::string &jsonText);
+
+// ArgMax(x, axis) as ops the kernel families have: m = ReduceMax(x) (keep_dims), i = ReduceMin(Select(x == m, Iota, BIG)),
+// result = Cast(Select(i == BIG, 0, i)). This restates upstream tosa.argmax's linalg lowering (LLVM 19.1.7
+// TosaToLinalg ArgMaxConverter: start at index 0 with the lowest finite value, take a later element only if it is
+// strictly greater under an ordered comparison): the first of equal maxima wins, NaNs are never taken, and a row that
+// holds nothing above the lowest finite value gives 0. The graph's other ops are untouched.
+void expandArgMax(OpGraph *graph);
 
 // A reduction whose reduced axes all have extent 1 folds nothing: it becomes a Reshape of its operand
 // (RemoveRedundantReduce.cpp:46-75 replaces the keep_dims form by the operand; the other form differs from its operand

@@ -79,6 +79,10 @@ FIXTURES = {
     "small_transpose_sum_f16_130x66_perm10": lambda n: op_desc.transpose_sum([130, 66], [1, 0], "float16", n),
     "small_split_swiglu_bf16_37x264": lambda n: op_desc.split_swiglu(37, 264, "bfloat16", n),
     "small_split_swiglu_f32_5x9": lambda n: op_desc.split_swiglu(5, 9, "float32", n),
+    # ArgMax over the innermost axis (row family: max, then the least position that holds it)
+    "small_argmax_f32_37x1000": lambda n: op_desc.argmax_last_axis([37, 1000], "float32", False, "int32", None, n),
+    "small_argmax_f16_3x5x333_keep_i64": lambda n: op_desc.argmax_last_axis([3, 5, 333], "float16", True, "int64", None, n),
+    "small_argmax_bf16_scaled_4x70000": lambda n: op_desc.argmax_last_axis([4, 70000], "bfloat16", False, "int32", 0.5, n),
     "small_embedding_lookup_bf16_1000x96_ids5x33": lambda n: op_desc.embedding_lookup_scale(1000, 96, 5, 33, "bfloat16", n),
     "small_embedding_lookup_f32_50x7_ids3x4": lambda n: op_desc.embedding_lookup_scale(50, 7, 3, 4, "float32", n),
     # UnsortedSegmentSum (segment_sum family): short slices, a wide slice tiled over workgroups, 16-bit accumulation

@@ -495,6 +495,25 @@ def unsorted_segment_sum(index_shape, slice_shape, segments, dtype="float32", id
     return b.dumps([out])
 
 
+def argmax(b, x, axis, keep_dims=False, dtype="int32"):
+    axis = axis % len(x.shape)
+    shape = [1 if i == axis else d for i, d in enumerate(x.shape)] if keep_dims else \
+            [d for i, d in enumerate(x.shape) if i != axis] or [1]
+    return b.op("ArgMax", [x], shape, dtype, attrs=[{"data_type": "listInt", "name": "axis", "value": [int(axis)]},
+                                                    {"data_type": "bool", "name": "keep_dims", "value": bool(keep_dims)}])
+
+
+def argmax_last_axis(shape, dtype="float32", keep_dims=False, index_dtype="int32", scale=None, name=None):
+    """Greedy decoding step: index of the greatest logit per row (optionally after a scale, so that an elementwise op
+    is fused in front)."""
+    b = DescBuilder(name or "Fused_ArgMax_%s_%s" % (_SHORT[dtype], "x".join(str(d) for d in shape)))
+    x = b.input(list(shape), dtype)
+    y = x
+    if scale is not None:
+        y = b.mul(b.cast(x, "float32") if dtype != "float32" else x, b.const(float(scale), "float32"))
+    return b.dumps([argmax(b, y, len(shape) - 1, keep_dims, index_dtype)])
+
+
 def any_greater(rows, cols, threshold=2.5, op="ElemAny", name=None):
     """out[r] = any(x[r, :] > threshold), spelled with `ElemAny` (the reference maps it to its ReduceAny op)."""
     b = DescBuilder(name or "Fused_Greater_%s_f32_%dx%d" % (op, rows, cols))

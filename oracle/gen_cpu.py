@@ -240,7 +240,7 @@ def parse(desc):
         if name in VIEW_OPS:
             op.view = view_params(od, ins[0].shape)
         out.producer = op
-        if name in REDUCES:
+        if name in REDUCES + ("ArgMax",):
             if len(od["input_desc"]) == 2:
                 axes = od["input_desc"][1][0]["value"]
             else:
@@ -290,7 +290,7 @@ class Emitter:
 
     # -- which values live in memory --------------------------------------------------------------------
     def is_elementwise(self, op):
-        return op.name not in REDUCES + MATMULS + ("Reshape",) + VIEW_OPS + ASSIGNS + SEGMENTS
+        return op.name not in REDUCES + MATMULS + ("Reshape", "ArgMax") + VIEW_OPS + ASSIGNS + SEGMENTS
 
     def plan(self):
         consumers = {}
@@ -596,6 +596,45 @@ class Emitter:
         self.emit("%s[%s] = %s;" % (out.buffer, lin(out, idx), self.store_expr(out.dtype, value)), depth)
         self.close_loops(rank, depth)
 
+    def emit_argmax(self, op):
+        """ArgMax over one axis. The reference hands it to tosa.argmax (MindSporeToTosa.cpp:497) with attributes that op
+        does not have, so what is restated is upstream's lowering of tosa.argmax itself (LLVM 19.1.7, TosaToLinalg
+        ArgMaxConverter): index 0 and the lowest finite value to start with, a later element replaces them only if
+        it is greater under an ordered comparison (so the first of equal maxima wins and NaN never does)."""
+        src, out = op.inputs[0], op.output
+        if len(op.axes) != 1 or out.dtype not in INTS or src.dtype == "bool":
+            raise OracleError("ArgMax: one axis, an integer result and a non-bool operand are required")
+        axis = op.axes[0]
+        in_shape = src.shape
+        par = [d for d in range(len(in_shape)) if d != axis]
+        sd = src.dtype
+        if sd in FLOATS:
+            big = {"float16": 65504.0, "bfloat16": 3.3895313892515355e38, "float32": 3.4028234663852886e38,
+                   "float64": 1.7976931348623157e308}[sd]
+            lowest = float_literal(sd, -big)
+        else:
+            lo = INT_RANGE[sd][0]
+            lowest = "INT64_MIN" if sd == "int64" else ("INT32_MIN" if lo <= -2147483648 else "%d" % lo)
+        depth = 1
+        for k, d in enumerate(par):
+            self.emit("for (int64_t i%d = 0; i%d < %dL; ++i%d) {" % (d, d, in_shape[d], d), depth + k)
+        depth += len(par)
+        self.emit("{", depth)
+        self.emit("%s best = %s;" % (C_COMPUTE[sd], lowest), depth + 1)
+        self.emit("int64_t where = 0;", depth + 1)
+        self.emit("for (int64_t i%d = 0; i%d < %dL; ++i%d) {" % (axis, axis, in_shape[axis], axis), depth + 1)
+        x = self.value_expr(src, in_shape)
+        self.emit("const %s v = %s;" % (C_COMPUTE[sd], x), depth + 2)
+        self.emit("if (v > best) { best = v; where = i%d; }" % axis, depth + 2)
+        self.emit("}", depth + 1)
+        expr = None
+        for d in par:
+            expr = "i%d" % d if expr is None else "(%s) * %dL + i%d" % (expr, in_shape[d], d)
+        self.emit("%s[%s] = (%s)where;" % (out.buffer, expr or "0", C_STORAGE[out.dtype]), depth + 1)
+        self.emit("}", depth)
+        for k in range(len(par)):
+            self.emit("}", depth - 1 - k)
+
     def emit_reduce(self, op):
         src, out = op.inputs[0], op.output
         od = out.dtype
@@ -746,6 +785,8 @@ class Emitter:
             self.emit("/* %s -> %s */" % (op.name, out.name))
             if op.name in REDUCES:
                 self.emit_reduce(op)
+            elif op.name == "ArgMax":
+                self.emit_argmax(op)
             elif op.name in MATMULS:
                 self.emit_matmul(op)
             elif op.name in VIEW_OPS:

@@ -290,6 +290,25 @@ def evaluate(desc, inputs, updates=None):
                 res = ins[0].reshape(oshape)
             elif name == "BroadcastTo":
                 res = np.broadcast_to(ins[0], oshape)
+            elif name == "ArgMax":
+                # upstream tosa.argmax lowering (LLVM 19.1.7): start at index 0 with the lowest finite value, a later
+                # element wins only if it is greater (ordered comparison: never a NaN, never an equal one)
+                axes = od["input_desc"][1][0]["value"] if len(od["input_desc"]) == 2 else attrs["axis"]
+                axes = axes if isinstance(axes, list) else [axes]
+                assert len(axes) == 1, "ArgMax: one axis"
+                axis = axes[0] + ins[0].ndim if axes[0] < 0 else axes[0]
+                x = np.moveaxis(cv[0], axis, -1)
+                if in_dt[0] in FLOATS:
+                    best = np.full(x.shape[:-1], -LARGEST[in_dt[0]], dtype=x.dtype)
+                else:
+                    best = np.full(x.shape[:-1], np.iinfo(x.dtype).min, dtype=x.dtype)
+                where = np.zeros(x.shape[:-1], dtype=np.int64)
+                for k in range(x.shape[-1]):
+                    v = x[..., k]
+                    hit = v > best
+                    best = np.where(hit, v, best)
+                    where = np.where(hit, k, where)
+                res = where.reshape(oshape)
             elif name in ("ReduceSum", "ReduceMax", "ReduceMin", "ReducePrd", "ReduceAll", "ReduceAny"):
                 if len(od["input_desc"]) == 2:
                     axes = od["input_desc"][1][0]["value"]

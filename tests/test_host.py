@@ -262,6 +262,25 @@ def test_unsorted_segment_sum_translates_and_gets_its_own_family():
     assert e.value.code == -4 and "kernel of its own" in str(e.value)
 
 
+def test_argmax_becomes_a_max_and_a_least_position_in_the_row_family():
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_argmax_f32_37x1000.info"))
+    assert k.family == "row_reduce" and [t.dtype for t in k.outputs] == ["int32"]
+    assert "mindspore.argmax" in driver.translate(open(os.path.join(FIXTURES, "small_argmax_f32_37x1000.info")).read())
+    assert k.source.count("group_reduce<akg::RedMax") == 1 and k.source.count("group_reduce<akg::RedMin") == 1
+    assert "static_cast<int>(akg_cols[j] + e)" in k.source
+    # a row too long for registers: the position pass is one more walk over the (packed) row
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_argmax_bf16_scaled_4x70000.info"))
+    assert k.source.count("for (int akg_g = 0; akg_g < GROUPS") == 3 and "RawChunk" in k.source
+    b = op_desc.DescBuilder("Fused_ArgMax_axis0")
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(b.dumps([op_desc.argmax(b, b.input([8, 16], "float32"), 0)]), out_dir=None)
+    assert e.value.code == -4 and "innermost axis" in str(e.value)
+    b = op_desc.DescBuilder("Fused_ArgMax_float_result")
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(b.dumps([op_desc.argmax(b, b.input([8, 16], "float32"), 1, dtype="float32")]), out_dir=None)
+    assert "integer" in str(e.value)
+
+
 def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_view_chain_f32.info"))
     assert (k.operator_type, k.family) == ("Transpose", "indexed")

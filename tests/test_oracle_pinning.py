@@ -420,6 +420,33 @@ def test_split_gives_consecutive_pieces_along_the_axis(tmp_path):
         assert np.array_equal(np.asarray(got[2]).reshape(a2.shape), np.abs(a2))
 
 
+def test_argmax_takes_the_first_greatest_element_and_never_a_nan(tmp_path):
+    """ArgMax against numpy.argmax on rows without NaN (numpy also takes the first of equal maxima), and the cases
+    upstream's lowering of tosa.argmax fixes: NaN is never taken, a row of -inf or of NaN only gives 0 (nothing is
+    greater than the lowest finite value it starts with)."""
+    b = op_desc.DescBuilder("pin_argmax")
+    x = b.input([6, 7], "float32")
+    text = b.dumps([op_desc.argmax(b, x, 1)])
+    inf, nan = np.inf, np.nan
+    data = np.array([[1, 5, 3, 5, 0, -2, 5],            # three equal maxima: the first
+                     [nan, 2, 9, nan, 9, 1, 0],         # NaN skipped, first 9
+                     [-inf] * 7,                        # nothing above the lowest finite value
+                     [nan] * 7,
+                     [-3, -2, -1, -0.5, -7, -0.5, -9],  # negative values
+                     [0, 0, 0, 0, 0, 0, inf]], dtype=np.float32)
+    _, c_out, n_out = build_and_run(text, [data], tmp_path)
+    expect = [1, 2, 0, 0, 3, 6]
+    assert c_out[0].tolist() == expect and np.asarray(n_out[0]).reshape(-1).tolist() == expect
+    rng = np.random.default_rng(9)
+    b = op_desc.DescBuilder("pin_argmax_axis0")
+    x = b.input([50, 4, 9], "float32")
+    text = b.dumps([op_desc.argmax(b, x, 0, keep_dims=True, dtype="int64")])
+    data = rng.integers(-5, 6, size=(50, 4, 9)).astype(np.float32)       # many ties
+    _, c_out, n_out = build_and_run(text, [data], tmp_path)
+    want = np.argmax(data, axis=0).reshape(1, 4, 9)
+    assert np.array_equal(c_out[0], want) and np.array_equal(np.asarray(n_out[0]).reshape(1, 4, 9), want)
+
+
 def test_assign_writes_the_value_over_its_first_operand(tmp_path):
     """Momentum step in float32 against the formula written out in numpy: v <- 0.9 v + g, p <- p - 0.01 v. The C
     restatement updates the caller's input arrays in place, the numpy one reports the updates."""
