@@ -150,7 +150,14 @@ def random_description(seed, allow_views=True, allow_reduce=True):
     out = work[-1]
     outs = [out.t]
     if allow_reduce and not used_view and rng.random() < 0.5 and len(out.t.shape) >= 1:
-        axis = [len(out.t.shape) - 1] if rng.random() < 0.6 else [int(rng.integers(0, len(out.t.shape)))]
+        r = len(out.t.shape)
+        pick_axes = rng.random()
+        if pick_axes < 0.5:
+            axis = [r - 1]
+        elif pick_axes < 0.8 or r < 2:
+            axis = [int(rng.integers(0, r))]
+        else:   # several axes, possibly with kept ones in between ([N,C,HW] over N and HW)
+            axis = sorted(int(a) for a in rng.choice(r, size=int(rng.integers(2, r + 1)), replace=False))
         name = str(rng.choice(["ReduceSum", "ReduceMax", "ReduceMin"]))
         notes.append("%s%s" % (name, axis))
         if rng.random() < 0.4 and axis == [len(out.t.shape) - 1]:
