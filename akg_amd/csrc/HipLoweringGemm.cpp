@@ -18,6 +18,7 @@
  *   Row    [M,1]      one value per output row
  *   Scalar [1]        one value
  */
+#include <algorithm>
 #include <sstream>
 
 #include "HipLowering.h"
@@ -42,13 +43,19 @@ class GemmEmitter {
 
   LoweredKernel run() {
     analyse();
+    pickSplit();
     emit();
     LoweredKernel k;
     k.kernelName = g_.name + "_kernel";
     k.source = src_.str();
     k.family = KernelFamily::GemmEpilogue;
     const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
-    k.grid[0] = static_cast<unsigned>(((tiles + 7) / 8) * 8);
+    const int64_t gridTiles = ((tiles + 7) / 8) * 8;
+    k.grid[0] = static_cast<unsigned>(gridTiles * kSplit_);
+    if (kSplit_ > 1) {
+      const int64_t partRows = std::min<int64_t>(m_, 256);
+      k.workspaceBytes = static_cast<uint64_t>((gridTiles * 4 + 255) / 256 * 256 + tiles * kSplit_ * partRows * 256 * 4);
+    }
     k.grid[1] = static_cast<unsigned>(batch_);
     k.block[0] = static_cast<unsigned>(wavesM() * 2 * 64);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
@@ -59,6 +66,7 @@ class GemmEmitter {
     note << "gemm_epilogue batch=" << batch_ << " M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
          << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
          << k.grid[0];
+    if (kSplit_ > 1) note << " k_splits=" << kSplit_;
     k.scheduleNote = note.str();
     return k;
   }
@@ -68,6 +76,7 @@ class GemmEmitter {
   LoweringOptions opt_;
   std::ostringstream src_;
   int64_t m_ = 0, n_ = 0, k_ = 0, batch_ = 1;
+  int kSplit_ = 1;  // workgroups per tile, each with a range of K steps (see pickSplit)
   bool transB_ = false;
   int matmulOp_ = -1;
   int aId_ = -1, bId_ = -1, accId_ = -1;
@@ -90,6 +99,28 @@ class GemmEmitter {
   // Bytes of K in one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
   int stepK() const { return (elem_ == DType::I8 && (opt_.gemmVariant & 2)) ? 64 : 128; }
   bool splitDuty() const { return (opt_.gemmVariant & 4) != 0 && wavesM() == 4; }
+
+  // Few tiles and a long K (a skinny activation in front of a big weight matrix: M = 16 .. 1024 against 8192 x 8192
+  // leaves 32 .. 128 of 256 CUs busy, and the time is that of streaming the weights through those few): split K over
+  // enough workgroups to fill the chip, at least four K steps each.
+  void pickSplit() {
+    kSplit_ = 1;
+    if (batch_ != 1) return;
+    const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
+    const int64_t steps = (k_ * elemBytes() + stepK() - 1) / stepK();
+    int64_t want = opt_.split > 0 ? opt_.split : (tiles >= 192 ? 1 : std::min<int64_t>(16, (256 + tiles - 1) / tiles));
+    want = std::max<int64_t>(1, std::min<int64_t>(want, opt_.split > 0 ? steps : steps / 4));
+    while (want > 1 && (want - 1) * ((steps + want - 1) / want) >= steps) --want;   // no empty split
+    const int64_t partRows = std::min<int64_t>(m_, 256);
+    while (want > 1 && tiles * want * partRows * 256 * 4 >= (1LL << 30)) --want;
+    if (opt_.split <= 0) {
+      // the partials are written and read once: not more of them than four times the operands (2048^3 int8 with four
+      // splits moved 134 MB of partials for 8 MB of operands and lost 12 %; bf16 with twice the operands gained 26 %)
+      const int64_t operandBytes = (m_ * k_ + k_ * n_) * elemBytes();
+      while (want > 1 && 2 * tiles * want * partRows * 256 * 4 > 4 * operandBytes) --want;
+    }
+    kSplit_ = static_cast<int>(std::max<int64_t>(1, want));
+  }
 
   void analyse() {
     for (size_t i = 0; i < g_.ops.size(); ++i) {
@@ -334,6 +365,7 @@ class GemmEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
+    if (kSplit_ > 1) src_ << ", unsigned *__restrict__ akg_ws";
     src_ << ") {\n  Epilogue epi;\n  const long akg_batch = static_cast<long>(blockIdx.y);\n"
          << "  epi.row0 = akg_batch * " << m_ << "L;\n";
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
@@ -343,8 +375,9 @@ class GemmEmitter {
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
     src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
-         << " + akg_batch * " << k_ * n_ << "L, epi);\n}\n";
+         << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ", Epilogue, " << kSplit_
+         << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
+         << " + akg_batch * " << k_ * n_ << "L, epi" << (kSplit_ > 1 ? ", akg_ws" : "") << ");\n}\n";
   }
 };
 

@@ -101,8 +101,15 @@ AKG_DEV u32 pack_hi16(u32 x, u32 y) { return __builtin_amdgcn_perm(y, x, 0x07060
 // BK = BYTES of K in one step: 64 or 128. With 128 every row of A contributes one full 128-byte cache line per step
 // (with 64 each line is fetched from L2 twice), there are half as many barriers, and LDS holds 2 x 72 KiB.
 // KE is the K extent in elements; everything below counts K in bytes (K = KE * element size).
-template <typename Mma, long M, long N, long KE, bool TRANSB, int WAVES_M, int BK, bool SPLIT, typename Epilogue>
-AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi) {
+// KSPLIT > 1 (few tiles, long K: a skinny A in front of a big weight matrix) gives every tile to KSPLIT workgroups,
+// each with a contiguous range of K steps; they leave their accumulators in the workspace `ws` (one arrival counter per
+// tile, then kPartRows x 256 accumulators per tile and split), and the last one to arrive adds the partials in split
+// order and runs the epilogue: deterministic, and the weight matrix is still read exactly once. The launch has
+// KSPLIT times the workgroups; the counters are left at zero.
+template <typename Mma, long M, long N, long KE, bool TRANSB, int WAVES_M, int BK, bool SPLIT, typename Epilogue,
+          int KSPLIT = 1>
+AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi,
+                          unsigned *__restrict__ ws = nullptr) {
   constexpr int EB = Mma::kElemBytes;
   constexpr long K = KE * EB;    // bytes of K per row of A (and per column of B)
   constexpr long NB = N * EB;    // bytes per k-row of a row-major B
@@ -136,9 +143,16 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   __shared__ __attribute__((aligned(16))) u8 lds[2][2][kTileBytes];  // [buffer][A|B]
 
   // ---- workgroup -> tile
-  const long wg = static_cast<long>(blockIdx.x);
+  constexpr long kGridTiles = kPerXcd * kGemmXcds;   // workgroups per K split (a multiple of the XCD count)
+  const long wgAll = static_cast<long>(blockIdx.x);
+  const long ksplit = KSPLIT > 1 ? wgAll / kGridTiles : 0;
+  const long wg = KSPLIT > 1 ? wgAll % kGridTiles : wgAll;
   const long linear = (wg % kGemmXcds) * kPerXcd + wg / kGemmXcds;
   if (linear >= kTiles) return;
+  constexpr long kStepsPer = (kSteps + KSPLIT - 1) / KSPLIT;
+  static_assert((KSPLIT - 1) * kStepsPer < kSteps, "every K split needs at least one step");
+  const long stepBase = ksplit * kStepsPer;
+  const long mySteps = KSPLIT == 1 ? kSteps : ((kSteps - stepBase) < kStepsPer ? (kSteps - stepBase) : kStepsPer);
   constexpr long kGroupSize = kGemmGroupRows * kTilesN;
   const long group = linear / kGroupSize;
   const long firstRow = group * kGemmGroupRows;
@@ -228,7 +242,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     }
   };
   auto loadGlobal = [&](long step, Stage &st) {
-    const long k0 = step * BK;
+    const long k0 = (stepBase + step) * BK;
     if constexpr (kSplitDuty) {
       if (stageA) {
         loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
@@ -409,12 +423,12 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   };
   loadGlobal(0, stage);
   storeLds(0, stage);
-  if (kSteps > 1) loadGlobal(1, stage);
+  if (mySteps > 1) loadGlobal(1, stage);
   __syncthreads();
   readFrags(0, 0, f0a, f0b);
   long step = 0;
-  for (; step + 2 < kSteps; ++step) stepBody(step, BoolTag<true>(), BoolTag<true>());
-  if (step + 1 < kSteps) {
+  for (; step + 2 < mySteps; ++step) stepBody(step, BoolTag<true>(), BoolTag<true>());
+  if (step + 1 < mySteps) {
     stepBody(step, BoolTag<true>(), BoolTag<false>());
     ++step;
   }
@@ -422,6 +436,55 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 
   // ---- epilogue: lane owns columns col4 .. col4+3 of 16 * kTM rows
   const long col4 = n0 + 4 * (wn * 32 + fragRow);
+  if constexpr (KSPLIT > 1) {
+    constexpr long kPartRows = M < kGemmBM ? M : kGemmBM;            // rows of a tile that can hold results
+    constexpr long kCounterBytes = (kGridTiles * 4 + 255) / 256 * 256;
+    constexpr long kPartBytes = kPartRows * kGemmBN * static_cast<long>(sizeof(typename Mma::acc_t));
+    constexpr long kWsBytes = kCounterBytes + kTiles * KSPLIT * kPartBytes;
+    static_assert(kWsBytes < (1L << 31), "split-K workspace too large");
+    const Buffer wsBuf = make_buffer(ws, kWsBytes);
+    const u32 tileBase = static_cast<u32>(kCounterBytes + linear * KSPLIT * kPartBytes);
+    const bool colOk = kFull || col4 < N;
+    auto partOffset = [&](int i, int v) {
+      const long rowInTile = wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+      return static_cast<long>((rowInTile * kGemmBN + (col4 - n0)) * static_cast<long>(sizeof(typename Mma::acc_t)));
+    };
+    auto rowOk = [&](int i, int v) {
+      const long rowInTile = wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+      return rowInTile < kPartRows && m0 + rowInTile < M;
+    };
+#pragma unroll
+    for (int i = 0; i < kTM; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        if (colOk && rowOk(i, v)) {
+          const typename Mma::acc_t a4[4] = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+          ws_store_chunk<4>(wsBuf, tileBase + static_cast<u32>(ksplit * kPartBytes + partOffset(i, v)), a4);
+        }
+      }
+    }
+    __shared__ unsigned akg_gemm_flag;
+    if (!last_workgroup(ws, linear, KSPLIT, tid, &akg_gemm_flag)) return;
+    if (!colOk) return;
+    epi.prepare(col4);
+#pragma unroll
+    for (int i = 0; i < kTM; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        if (!rowOk(i, v)) continue;
+        typename Mma::acc_t sum[4] = {0, 0, 0, 0};
+        for (int p = 0; p < KSPLIT; ++p) {
+          typename Mma::acc_t part[4];
+          ws_load_chunk<4>(wsBuf, tileBase + static_cast<u32>(p * kPartBytes + partOffset(i, v)), part);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sum[c] += part[c];
+        }
+        const long row = m0 + wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+        epi.apply(sum, row, col4);
+      }
+    }
+    return;
+  }
   if (kFull || col4 < N) {
     epi.prepare(col4);
 #pragma unroll

@@ -97,6 +97,11 @@ FIXTURES = {
     "small_gemm_f16_bias_relu_200x264x136": lambda n: op_desc.gemm_bias_act(200, 264, 136, "float16", "relu", False, "float32", n),
     "small_gemm_f16_bias_relu_200x264x136_tb": lambda n: op_desc.gemm_bias_act(200, 264, 136, "float16", "relu", True, "float32", n),
     "small_gemm_bf16_bias_none_520x1024x776": lambda n: op_desc.gemm_bias_act(520, 1024, 776, "bfloat16", "none", False, "float32", n),
+    # few tiles, long K: K split over several workgroups per tile (partials in the workspace, last one finishes)
+    "small_gemm_i8_dequant_bias_gelu_64x4096x256": lambda n: op_desc.gemm_int8_dequant_bias_gelu(64, 4096, 256, "bfloat16", False, n),
+    "small_gemm_i8_dequant_bias_gelu_300x2064x520_tb": lambda n: op_desc.gemm_int8_dequant_bias_gelu(300, 2064, 520, "bfloat16", True, n),
+    "small_gemm_bf16_bias_gelu_100x2048x520": lambda n: op_desc.gemm_bias_act(100, 2048, 520, "bfloat16", "gelu", False, "float32", n),
+    "small_gemm_f16_bias_relu_16x3000x264_tb": lambda n: op_desc.gemm_bias_act(16, 3000, 264, "float16", "relu", True, "float32", n),
     "small_batchmatmul_scale_mask_bf16_3x200x64x136_tb": lambda n: op_desc.batch_matmul_scale_mask(3, 200, 64, 136, "bfloat16", True, n),
     "small_batchmatmul_scale_mask_f16_2x256x128x256": lambda n: op_desc.batch_matmul_scale_mask(2, 256, 128, 256, "float16", False, n),
     "n2_gemm_bf16_bias_gelu_4096x8192x8192": lambda n: op_desc.gemm_bias_act(4096, 8192, 8192, "bfloat16", "gelu", False, "float32", n),
