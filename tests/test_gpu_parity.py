@@ -160,6 +160,62 @@ def test_tensors_of_two_gib_and_more_are_addressed_with_64_bit_offsets(tmp_path)
     assert np.all(np.abs(sums - 1.0) < 2e-2)      # every sampled row is a distribution
 
 
+def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
+    """After `prepare` a launch allocates nothing and records no memset, so a serving loop can capture a chain of
+    kernels once and replay it: a softmax, a column reduction (workspace + arrival counters) and a split-K GEMM
+    (workspace) are captured in one graph and replayed four times on fresh inputs, with eager work and
+    synchronisations in between; every replay must equal the eager launches bit for bit (the counters and partials
+    of one replay must be ready for the next)."""
+    import torch
+    dev = torch.device("cuda:0")
+    names = ["small_softmax_f16_64x4096", "small_biasgrad_bf16_2048x1024", "small_gemm_bf16_bias_gelu_100x2048x520"]
+    kernels, descs = [], []
+    for n in names:
+        path = os.path.join(FIXTURES, n + ".info")
+        k = driver.HipKernel.from_file(path)
+        k.prepare()
+        kernels.append(k)
+        descs.append(harness.load_desc(path))
+    assert kernels[1].workspace_bytes > 0 and kernels[2].workspace_bytes > 0
+
+    def buffers(k):
+        return [torch.zeros(t.nbytes, dtype=torch.uint8, device=dev) for t in k.tensors]
+    static = [buffers(k) for k in kernels]          # the graph's own buffers
+    eager = [buffers(k) for k in kernels]
+
+    def upload(bufs, k, inputs):
+        for b, a in zip(bufs, inputs):
+            b.copy_(torch.from_numpy(a.view(np.uint8).reshape(-1)))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                   # warm-up launches outside the capture
+        for k, bufs in zip(kernels, static):
+            k.launch(bufs)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for k, bufs in zip(kernels, static):
+            k.launch(bufs)
+    for replay in range(4):
+        print("replay %d" % replay, flush=True)
+        for k, d, sb, eb in zip(kernels, descs, static, eager):
+            inputs = harness.make_inputs(d, seed=harness.BASE_SEED + 900 + replay)
+            upload(sb, k, inputs)
+            upload(eb, k, inputs)
+            for b in sb[len(inputs):]:
+                b.fill_(0x7B)                        # stale results of the previous replay must not survive
+        graph.replay()
+        torch.cuda.synchronize()
+        for k, eb in zip(kernels, eager):            # the program's own eager work between replays
+            k.launch(eb)
+        torch.cuda.synchronize()
+        for k, sb, eb in zip(kernels, static, eager):
+            n_in = len(k.tensors) - len(k.outputs)
+            for a, b in zip(sb[n_in:], eb[n_in:]):
+                assert torch.equal(a, b), "replay %d of %s differs from the eager launch" % (replay, k.kernel_name)
+
+
 @pytest.mark.parametrize("name", FULL)
 def test_full_size_config_matches_oracle(name):
     # full BASELINE sizes; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)
