@@ -68,6 +68,7 @@ LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options);
 // Family-specific entries used by lowerToHip (HipLoweringGemm.cpp, HipLoweringReduce.cpp, HipLoweringIndexed.cpp).
 LoweredKernel lowerGemmToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerStreamReduceToHip(const OpGraph &graph, const LoweringOptions &options);
+LoweredKernel lowerTileToHip(const OpGraph &graph, const LoweringOptions &options);      // elementwise, row_reduce
 LoweredKernel lowerIndexedToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerSegmentSumToHip(const OpGraph &graph, const LoweringOptions &options);
 // True when the graph contains a data-movement op (Transpose, Tile, Slice, StridedSlice, Pad, Concat).
