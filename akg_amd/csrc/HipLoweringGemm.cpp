@@ -95,7 +95,7 @@ class GemmEmitter {
   const char *accType() const { return elem_ == DType::I8 ? "int" : "float"; }
   // The tuning variants exist for the 8-bit kernel only; 16-bit operands always use 4 x 2 wavefronts and 128-byte steps.
   // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_GEMM_VARIANT=1.
-  int wavesM() const { return (elem_ == DType::I8 && (opt_.gemmVariant & 1)) ? 2 : 4; }
+  int wavesM() const { return (opt_.gemmVariant & 1) ? 2 : 4; }
   // Bytes of K in one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
   int stepK() const { return (elem_ == DType::I8 && (opt_.gemmVariant & 2)) ? 64 : 128; }
   bool splitDuty() const { return (opt_.gemmVariant & 4) != 0 && wavesM() == 4; }

@@ -277,22 +277,25 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   };
   auto storeBlockB16 = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
     // 16-bit elements: src[g] = k-rows 2g, 2g+1, each as (columns 0 1 | columns 2 3). A column's 8 consecutive k
-    // (16 bytes) are gathered two at a time with v_perm_b32.
-    static_assert(EB != 2 || kRowChunks == 4, "16-bit staging is written for 8 k-rows per thread");
-    if constexpr (EB == 2 && kRowChunks == 4) {
-      v4i w[4];
+    // (16 bytes) are gathered two at a time with v_perm_b32; a thread holds 8 k-rows (4 x 2 wavefronts) or 16 (2 x 2).
+    static_assert(EB != 2 || kRowChunks == 4 || kRowChunks == 8, "16-bit staging is written for 8 or 16 k-rows per thread");
+    if constexpr (EB == 2 && (kRowChunks == 4 || kRowChunks == 8)) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const u32 c01a = static_cast<u32>(src[g][0]), c23a = static_cast<u32>(src[g][1]);  // k-row 2g
-        const u32 c01b = static_cast<u32>(src[g][2]), c23b = static_cast<u32>(src[g][3]);  // k-row 2g + 1
-        w[0][g] = static_cast<int>(pack_lo16(c01a, c01b));
-        w[1][g] = static_cast<int>(pack_hi16(c01a, c01b));
-        w[2][g] = static_cast<int>(pack_lo16(c23a, c23b));
-        w[3][g] = static_cast<int>(pack_hi16(c23a, c23b));
-      }
+      for (int h = 0; h < kRowChunks / 4; ++h) {
+        v4i w[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * 16) = w[j];
+        for (int g = 0; g < 4; ++g) {
+          const u32 c01a = static_cast<u32>(src[4 * h + g][0]), c23a = static_cast<u32>(src[4 * h + g][1]);  // k-row 2g
+          const u32 c01b = static_cast<u32>(src[4 * h + g][2]), c23b = static_cast<u32>(src[4 * h + g][3]);  // k-row 2g + 1
+          w[0][g] = static_cast<int>(pack_lo16(c01a, c01b));
+          w[1][g] = static_cast<int>(pack_hi16(c01a, c01b));
+          w[2][g] = static_cast<int>(pack_lo16(c23a, c23b));
+          w[3][g] = static_cast<int>(pack_hi16(c23a, c23b));
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * (kRowChunks * 4) + h * 16) = w[j];
+        }
       }
     }
   };
