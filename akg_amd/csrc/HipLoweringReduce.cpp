@@ -70,7 +70,7 @@ class StreamReduceEmitter {
     k.workspaceBytes = workspaceBytes_;
     std::ostringstream note;
     note << "stream_reduce direction=" << (dirY_ ? "Y" : "X") << " outer=" << O_ << " reduced=" << R_ << " inner=" << I_
-         << " vec=" << vec_ << (overlapTail_ ? " (overlapping last chunk)" : "") << " lanes=" << lanes_ << " split=" << split_ << " rows_per_split=" << rps_
+         << " vec=" << vec_ << ((overlapTail_ || overlapRun_) ? " (overlapping last chunk)" : "") << " lanes=" << lanes_ << " split=" << split_ << " rows_per_split=" << rps_
          << " block=" << kBlock << " grid=" << grid_ << " workspace=" << workspaceBytes_;
     k.scheduleNote = note.str();
     return k;
@@ -85,6 +85,8 @@ class StreamReduceEmitter {
 
   // iteration space: the reduced operand's shape; kind per dim (0 outer kept, 1 reduced, 2 inner kept, -1 unit)
   std::vector<int64_t> space_;
+  std::vector<int> foldOf_;            // per dim of the reduced operand: the dim of space_ it was folded into
+  std::vector<bool> reducedFolded_;    // per dim of space_
   std::vector<int> kind_;
   int64_t O_ = 1, R_ = 1, I_ = 1;
   bool dirY_ = false;
@@ -93,6 +95,12 @@ class StreamReduceEmitter {
 
   int vec_ = 1, lanes_ = 64, split_ = 1, unroll_ = 4;
   bool overlapTail_ = false;  // direction Y, I not a multiple of V: the last chunk of a row starts at I - V
+  // Direction X over contiguous runs whose length V does not divide (7 x 7 images, odd row lengths): the reduced
+  // extent is walked in chunk slots, runChunks_ per run of runLength_ elements, the last one starting at
+  // runLength_ - V; the elements it shares with its neighbour are left out of the reductions.
+  bool xcdContiguous_ = false;
+  bool overlapRun_ = false;
+  int64_t runLength_ = 1, runChunks_ = 1;
   int64_t strips_ = 1, rps_ = 1, grid_ = 1, groups_ = 1;
   uint64_t workspaceBytes_ = 0;
   std::vector<uint64_t> partialOffset_;  // per reduction, bytes from the workspace base
@@ -105,13 +113,21 @@ class StreamReduceEmitter {
   std::string tagOf(int id) const { return dtypeTag(g_.tensor(id).dtype); }
 
   // ------------------------------------------------------------------ analysis
-  std::vector<int64_t> padTo(const std::vector<int64_t> &shape, const std::string &what) const {
+  // Shape of a tensor in the kernel's iteration space: right-aligned with the reduced operand's shape, then folded
+  // like it (foldOf_: for every dim of the operand the dim of the space it went into).
+  std::vector<int64_t> padOriginal(const std::vector<int64_t> &shape, const std::string &what) const {
     std::vector<int64_t> s = shape;
-    const size_t n = space_.size();
+    const size_t n = foldOf_.size();
     while (s.size() > n && s.front() == 1) s.erase(s.begin());
     if (s.size() > n) throw LoweringError(what + ": rank exceeds the reduced operand's");
     std::vector<int64_t> out(n - s.size(), 1);
     out.insert(out.end(), s.begin(), s.end());
+    return out;
+  }
+  std::vector<int64_t> padTo(const std::vector<int64_t> &shape, const std::string &what) const {
+    const std::vector<int64_t> s = padOriginal(shape, what);
+    std::vector<int64_t> out(space_.size(), 1);
+    for (size_t d = 0; d < s.size(); ++d) out[static_cast<size_t>(foldOf_[d])] *= s[d];
     return out;
   }
 
@@ -129,24 +145,66 @@ class StreamReduceEmitter {
     }
     if (reduces_.empty()) throw LoweringError("internal: no reduction");
     const OpNode &first = *reduces_.front();
-    space_ = g_.tensor(first.inputs[0]).shape;
-    if (space_.empty()) space_.push_back(1);
-    const size_t n = space_.size();
-    std::vector<bool> reduced(n, false);
-    for (size_t a : realReducedAxes(g_, first)) reduced[a] = true;
+    std::vector<int64_t> original = g_.tensor(first.inputs[0]).shape;
+    if (original.empty()) original.push_back(1);
+    const size_t n0 = original.size();
+    std::vector<bool> reduced0(n0, false);
+    for (size_t a : realReducedAxes(g_, first)) reduced0[a] = true;
+    foldOf_.assign(n0, 0);
+    for (size_t d = 0; d < n0; ++d) foldOf_[d] = static_cast<int>(d);   // identity while the operands are compared
+    space_ = original;
     for (const OpNode *op : reduces_) {
       const TensorValue &in = g_.tensor(op->inputs[0]);
-      if (in.shape.size() != n || padTo(in.shape, "reduce operand " + in.name) != space_) {
+      if (in.shape.size() != n0 || padOriginal(in.shape, "reduce operand " + in.name) != original) {
         throw LoweringError("all reductions of one kernel must run over the same tensor shape");
       }
-      std::vector<bool> r2(n, false);
+      std::vector<bool> r2(n0, false);
       for (size_t a : realReducedAxes(g_, *op)) r2[a] = true;
-      if (r2 != reduced) throw LoweringError("all reductions of one kernel must reduce the same axes");
+      if (r2 != reduced0) throw LoweringError("all reductions of one kernel must reduce the same axes");
       const DType od = g_.tensor(op->outputs[0]).dtype;
       if (std::string(computeTypeName(in.dtype)) != computeTypeName(od)) {
         throw LoweringError("op " + op->name + ": operand and result element types differ");
       }
     }
+    // Fold: neighbouring dims that are both reduced or both kept, and that every input spans or broadcasts together,
+    // become one dim ([N,C,H,W] over N, H, W is [N,C,H*W]: chunks may then run across H). Unit dims join their
+    // left neighbour.
+    {
+      std::vector<std::vector<int64_t>> shapes;
+      for (int id : g_.inputs) {
+        const TensorValue &t = g_.tensor(id);
+        if (t.used) shapes.push_back(padOriginal(t.shape, "input " + t.name));
+      }
+      std::vector<int64_t> folded;
+      std::vector<bool> foldedReduced;
+      int lastReal = -1;   // last non-unit dim of the current group
+      for (size_t d = 0; d < n0; ++d) {
+        bool join = !folded.empty();
+        if (join && original[d] > 1 && lastReal >= 0) {
+          const size_t p = static_cast<size_t>(lastReal);
+          if (reduced0[d] != reduced0[p]) join = false;
+          for (const auto &sh : shapes) {
+            if ((sh[d] == 1) != (sh[p] == 1)) join = false;
+          }
+        }
+        if (join) {
+          folded.back() *= original[d];
+        } else {
+          folded.push_back(original[d]);
+          foldedReduced.push_back(false);
+          lastReal = -1;
+        }
+        if (original[d] > 1) {
+          lastReal = static_cast<int>(d);
+          foldedReduced.back() = reduced0[d];
+        }
+        foldOf_[d] = static_cast<int>(folded.size()) - 1;
+      }
+      space_ = folded;
+      reducedFolded_ = foldedReduced;
+    }
+    const size_t n = space_.size();
+    const std::vector<bool> &reduced = reducedFolded_;
     // kinds: kept dims before the last reduced one are "outer", after it "inner"
     kind_.assign(n, -1);
     size_t firstR = n, lastR = 0;
@@ -282,6 +340,10 @@ class StreamReduceEmitter {
     for (int id : g_.outputs) allBuffers = allBuffers && !tooLargeForBuffer(id);
     if (dirY_ && allBuffers && opt_.vec == 0 && fastExtent == I_ && (I_ % v) != 0 && I_ >= 2 * v) {
       overlapTail_ = true;
+    } else if (!dirY_ && allBuffers && opt_.vec == 0 && (fastExtent % v) != 0 && fastExtent >= 2 * v && R_ < (1LL << 30)) {
+      overlapRun_ = true;
+      runLength_ = fastExtent;
+      runChunks_ = ceilDivL(fastExtent, v);
     } else {
       while (v > 1 && (fastExtent % v) != 0) v >>= 1;
     }
@@ -332,15 +394,21 @@ class StreamReduceEmitter {
       lanes_ = kBlock;
       strips_ = 1;
       groups_ = O_;
-      const int64_t chunk = static_cast<int64_t>(kBlock) * vec_;
+      // what a workgroup's slice of the reduced extent is counted in: elements, or chunk slots (one per thread)
+      const int64_t extent = overlapRun_ ? (R_ / runLength_) * runChunks_ : R_;
+      const int64_t chunk = overlapRun_ ? static_cast<int64_t>(kBlock) : static_cast<int64_t>(kBlock) * vec_;
       int64_t split = opt_.split > 0 ? opt_.split : ceilDivL(targetGroups, groups_);
-      const int64_t maxSplit = std::max<int64_t>(1, R_ / (chunk * 2));
+      const int64_t maxSplit = std::max<int64_t>(1, extent / (chunk * 2));
       split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), kBlock));
-      rps_ = ceilDivL(ceilDivL(R_, split), chunk) * chunk;
-      split_ = static_cast<int>(ceilDivL(R_, rps_));
+      rps_ = ceilDivL(ceilDivL(extent, split), chunk) * chunk;
+      split_ = static_cast<int>(ceilDivL(extent, rps_));
     }
     grid_ = groups_ * split_;
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
+    // Runs shorter than a few cache lines that do not end on line boundaries ([N,C,7,7]: 98 bytes per channel and
+    // image): the lines are shared with the neighbouring outputs' runs.
+    xcdContiguous_ = !dirY_ && scatteredR && grid_ >= 64 && opt_.gemmVariant != 3 &&
+                     (fastExtent * static_cast<int64_t>(widest)) % 128 != 0 && fastExtent * static_cast<int64_t>(widest) < 2048;
     // workspace: one arrival counter per group, then the partials of every reduction
     workspaceBytes_ = 0;
     partialOffset_.assign(reduces_.size(), 0);
@@ -571,7 +639,12 @@ class StreamReduceEmitter {
     src_ << "  constexpr long RPS = " << rps_ << "L;\n";
     line("  (void)O; (void)I; (void)STRIPS;");
     line("  const int tid = static_cast<int>(threadIdx.x);");
-    line("  const long akg_wg = static_cast<long>(blockIdx.x);");
+    if (!dirY_ && xcdContiguous_) {
+      // neighbouring outputs read neighbouring runs that share cache lines: keep them on one XCD (one L2)
+      src_ << "  const long akg_wg = akg::xcd_contiguous_id(static_cast<int>(blockIdx.x), " << grid_ << ");\n";
+    } else {
+      line("  const long akg_wg = static_cast<long>(blockIdx.x);");
+    }
     if (dirY_ && opt_.gemmVariant != 1) {
       // neighbouring workgroups take neighbouring column strips of the same rows: what is in flight at any time
       // covers whole rows of the tensor rather than 256-byte pieces 8 KiB apart
@@ -582,8 +655,16 @@ class StreamReduceEmitter {
       line("  const long akg_s = akg_wg % SPLIT;");
       line("  const long akg_group = akg_wg / SPLIT;");
     }
-    line("  const long r_begin = akg_s * RPS;");
-    line("  const long r_end = (r_begin + RPS < R) ? (r_begin + RPS) : R;");
+    if (overlapRun_) {
+      src_ << "  constexpr int RUN = " << runLength_ << ", RUN_CHUNKS = " << runChunks_ << ", OVERLAP = "
+           << runChunks_ * vec_ - runLength_ << ";\n";
+      src_ << "  constexpr long SLOTS = " << (R_ / runLength_) * runChunks_ << "L;\n";
+      line("  const long r_begin = akg_s * RPS;   // in chunk slots");
+      line("  const long r_end = (r_begin + RPS < SLOTS) ? (r_begin + RPS) : SLOTS;");
+    } else {
+      line("  const long r_begin = akg_s * RPS;");
+      line("  const long r_end = (r_begin + RPS < R) ? (r_begin + RPS) : R;");
+    }
     if (dirY_) {
       line("  constexpr int TR = BLOCK / LANES;");
       line("  const int li = tid % LANES;");
@@ -620,6 +701,13 @@ class StreamReduceEmitter {
     line("#pragma unroll " + std::to_string(unroll_));
     if (dirY_) {
       line("  for (long r = r_begin + tr; r < r_end; r += TR) {");
+    } else if (overlapRun_) {
+      line("  for (long akg_slot = r_begin + tid; akg_slot < r_end; akg_slot += BLOCK) {");
+      line("    const int akg_run = static_cast<int>(akg_slot) / RUN_CHUNKS;");
+      line("    int akg_start = (static_cast<int>(akg_slot) % RUN_CHUNKS) * V;");
+      line("    const bool akg_tail = akg_start > RUN - V;");
+      line("    if (akg_tail) akg_start = RUN - V;");
+      line("    const long r = static_cast<long>(akg_run) * RUN + akg_start;");
     } else {
       line("  for (long r = r_begin + static_cast<long>(tid) * V; r < r_end; r += static_cast<long>(BLOCK) * V) {");
     }
@@ -637,7 +725,8 @@ class StreamReduceEmitter {
         std::string step = spec.combiner + "::apply(" + accName + ", " + val + ")";
         if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
         src_ << in4 << "#pragma unroll\n";
-        src_ << in4 << "for (int e = 0; e < V; ++e) " << accName << " = " << step << ";\n";
+        src_ << in4 << "for (int e = 0; e < V; ++e) " << (overlapRun_ ? "if (!akg_tail || e >= OVERLAP) " : "") << accName
+             << " = " << step << ";\n";
         continue;
       }
       if (phase_[static_cast<size_t>(out)] != Phase::Pre) continue;
