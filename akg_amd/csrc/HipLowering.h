@@ -44,6 +44,10 @@ struct LoweringOptions {
   int split = 0;        // streaming reductions: workgroups sharing one group of outputs (AKG_HIP_SPLIT)
   int gemmVariant = 0;  // GEMM tile configuration selector
   int nonTemporal = 1;  // stream once-touched tensors with non-temporal accesses (AKG_HIP_NT=0 turns it off)
+  // Dynamic-shape descriptions: the elementwise / row-reduction kernels take their row count (or, when everything
+  // folds into one dimension, their element count) as a kernel argument instead of a constant, so that shape sets
+  // that differ only there share one code object (the source no longer depends on them).
+  bool extentAsArgument = false;
   static LoweringOptions fromEnvironment();
 };
 
@@ -58,6 +62,8 @@ struct LoweredKernel {
   std::string scheduleNote;       // human-readable schedule summary (vec, threads per row, ...)
   // per kernel argument: [offset, sizes..., strides...] as in `<k>_shape_arg.txt`
   std::vector<std::vector<int64_t>> shapeArgs;
+  // 64-bit scalar kernel arguments that follow the tensor pointers (before the workspace pointer, if any)
+  std::vector<int64_t> scalarArgs;
   // Device workspace the kernel takes as one extra trailing pointer argument (0: none). The runtime allocates it
   // per kernel handle and device and zero-fills it once; the kernel leaves it zeroed where it must be.
   uint64_t workspaceBytes = 0;

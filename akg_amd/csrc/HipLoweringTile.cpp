@@ -75,6 +75,7 @@ class TileEmitter {
     k.block[0] = static_cast<unsigned>(block_);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
+    if (extentArg_) k.scalarArgs.push_back(extentIsCols_ ? cols_ : rows_);
     std::ostringstream note;
     note << kernelFamilyName(k.family) << " rows=" << rows_ << " cols=" << cols_ << " vec=" << vec_
          << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
@@ -93,6 +94,8 @@ class TileEmitter {
   bool rowMode_ = false;
   std::vector<int64_t> full_;     // iteration space (folded in elementwise mode)
   int64_t rows_ = 1, cols_ = 1, numel_ = 1;
+  bool extentArg_ = false;     // the row count (or COLS when everything folded into one dim) is a kernel argument
+  bool extentIsCols_ = false;
   std::vector<InputAccess> access_;  // per graph input
   std::vector<ValInfo> vals_;        // per tensor
 
@@ -261,6 +264,8 @@ class TileEmitter {
 
   // ------------------------------------------------------------------ schedule
   void pickSchedule() {
+    extentArg_ = opt_.extentAsArgument;
+    extentIsCols_ = extentArg_ && !rowMode_ && rows_ == 1;
     useBuffers_ = true;
     for (int id : g_.inputs) {
       if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
@@ -383,7 +388,7 @@ class TileEmitter {
       rowsPerBlock_ = block_ / tpr_;
       grid_ = ceilDiv(rows_, rowsPerBlock_);
       raggedCols_ = (groups_ * chunks_ * tpr_ != rowChunks);
-      raggedRows_ = (rows_ % rowsPerBlock_) != 0;
+      raggedRows_ = (rows_ % rowsPerBlock_) != 0 || extentArg_;
     } else {
       block_ = opt_.block > 0 ? opt_.block : 256;
       if (block_ % 64 != 0 || block_ > 1024) block_ = 256;
@@ -395,7 +400,7 @@ class TileEmitter {
       rowsPerBlock_ = 1;
       int64_t perBlock = static_cast<int64_t>(block_) * vec_ * chunks_;
       grid_ = std::max<int64_t>(1, ceilDiv(numel_, perBlock));
-      raggedFlat_ = (numel_ % perBlock) != 0;
+      raggedFlat_ = (numel_ % perBlock) != 0 || extentArg_;
     }
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
   }
@@ -537,24 +542,34 @@ class TileEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
+    if (extentArg_) src_ << ", const long akg_extent";
     line(") {");
+    if (extentArg_ && extentIsCols_) {
+      line("  constexpr long ROWS = 1L;");
+      line("  const long COLS = akg_extent;   // everything folds into one dimension: the element count");
+    } else if (extentArg_) {
+      src_ << "  constexpr long COLS = " << cols_ << "L;\n";
+      line("  const long ROWS = akg_extent;   // product of the leading dimensions");
+    } else {
+      src_ << "  constexpr long COLS = " << cols_ << "L;\n";
+      src_ << "  constexpr long ROWS = " << rows_ << "L;\n";
+    }
     if (useBuffers_) {
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
         const TensorValue &t = g_.tensor(g_.inputs[i]);
         src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", "
-             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+             << bytesExpr(access_[i].foldedShape, t) << ");\n";
       }
       for (size_t i = 0; i < g_.outputs.size(); ++i) {
         const TensorValue &t = g_.tensor(g_.outputs[i]);
-        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", "
-             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+        std::vector<int64_t> folded = full_;
+        if (t.numel() != numel_) folded.back() = 1;   // one value per row
+        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", " << bytesExpr(folded, t) << ");\n";
       }
     }
     src_ << "  constexpr int V = " << vec_ << ";\n";
     src_ << "  constexpr int NCHUNK = " << chunks_ << ";\n";
     src_ << "  constexpr int BLOCK = " << block_ << ";\n";
-    src_ << "  constexpr long COLS = " << cols_ << "L;\n";
-    src_ << "  constexpr long ROWS = " << rows_ << "L;\n";
     line("  const int tid = static_cast<int>(threadIdx.x);");
     if (rowMode_) {
       src_ << "  constexpr int TPR = " << tpr_ << ";\n";
@@ -582,7 +597,7 @@ class TileEmitter {
         emitColumnsOfGroup("0");
       }
     } else {
-      line("  constexpr long NUMEL = ROWS * COLS;");
+      line("  const long NUMEL = ROWS * COLS;");
       line("  const long akg_base = static_cast<long>(blockIdx.x) * (static_cast<long>(BLOCK) * V * NCHUNK);");
       line("  long akg_rows[NCHUNK];");
       line("  long akg_cols[NCHUNK];");
@@ -640,6 +655,27 @@ class TileEmitter {
       if (op.kind == OpKind::Assign) emitAssignStore(op);
     }
     line("}");
+  }
+
+  // Size in bytes of a tensor with the given shape in the (folded) iteration space, as a C expression: a number, or,
+  // when the extent is a kernel argument, a multiple of it for tensors that span all leading dimensions (or the one
+  // folded dimension). A tensor that spans only some of the leading dimensions keeps its number: such a source is
+  // specific to the shape set, which is correct, just not shared.
+  std::string bytesExpr(const std::vector<int64_t> &folded, const TensorValue &t) const {
+    const int64_t bytes = t.numel() * static_cast<int64_t>(dtypeSize(t.dtype));
+    const std::string number = std::to_string(bytes) + "L";
+    if (!extentArg_ || folded.size() != full_.size()) return number;
+    if (extentIsCols_) {
+      return folded.back() == cols_ ? "akg_extent * " + std::to_string(dtypeSize(t.dtype)) + "L" : number;
+    }
+    bool leadFull = true, leadOne = true;
+    for (size_t d = 0; d + 1 < folded.size(); ++d) {
+      if (folded[d] != full_[d]) leadFull = false;
+      if (folded[d] != 1) leadOne = false;
+    }
+    if (leadOne && rows_ != 1) return number;
+    if (!leadFull) return number;
+    return "akg_extent * " + std::to_string(folded.back() * static_cast<int64_t>(dtypeSize(t.dtype))) + "L";
   }
 
   // Non-temporal accesses pay off when a workgroup moves whole cache lines. Rows of a row kernel that are not a

@@ -51,6 +51,12 @@ struct akg_hip_kernel {
   std::vector<Loaded> loaded;
 };
 
+// Code objects compiled in this process, by the digest of their source (identical sources arise when a dynamic
+// description is specialised to shape sets that its kernel takes as an argument, and when one description is compiled
+// twice).
+std::mutex g_codeCacheMutex;
+std::map<std::string, std::vector<char>> g_codeCache;
+
 // A dynamic-shape description and the kernels specialised from it so far, keyed by the bound input shapes.
 struct akg_hip_dynamic {
   std::string jsonText;
@@ -260,6 +266,7 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
   if (outKernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "out_kernel is NULL");
   *outKernel = nullptr;
   std::unique_ptr<akg_hip_kernel> k(new akg_hip_kernel());
+  std::string artifactSuffix;
   try {
     k->graph = akg::translateJsonToOpGraph(jsonText, binding);
     if (binding != nullptr) {
@@ -272,7 +279,7 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
         }
         h.update(";", 1);
       }
-      k->graph.name += "_s" + h.hexDigest().substr(0, 12);
+      artifactSuffix = "_s" + h.hexDigest().substr(0, 12);
     }
   } catch (const akg::json::ParseError &e) {
     return fail(AKG_HIP_ERR_JSON, e.what());
@@ -280,11 +287,16 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
     return fail(AKG_HIP_ERR_TRANSLATE, e.what());
   }
   try {
-    k->lowered = akg::lowerToHip(k->graph, akg::LoweringOptions::fromEnvironment());
+    akg::LoweringOptions options = akg::LoweringOptions::fromEnvironment();
+    options.extentAsArgument = binding != nullptr;
+    k->lowered = akg::lowerToHip(k->graph, options);
+    // the kernel keeps the description's name (shape sets may share its code object); the artifacts are per shape set
+    k->graph.name += artifactSuffix;
   } catch (const akg::LoweringError &e) {
     return fail(AKG_HIP_ERR_UNSUPPORTED, std::string("kernel ") + k->graph.name + ": " + e.what());
   }
   const std::string srcDigest = sourceDigest(k->lowered.source);
+  bool fromMemory = false;
 
   std::string dir = outDir ? std::string(outDir) : std::string();
   std::string base;
@@ -308,9 +320,22 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
       }
     }
   }
-  if (!k->cacheHit) {
+  if (!k->cacheHit && !(std::getenv("AKG_HIP_NO_CACHE") && std::getenv("AKG_HIP_NO_CACHE")[0] == '1')) {
+    // code objects compiled earlier in this process, by source digest
+    std::lock_guard<std::mutex> lock(g_codeCacheMutex);
+    auto it = g_codeCache.find(srcDigest);
+    if (it != g_codeCache.end()) {
+      k->codeObject = it->second;
+      akg::Sha256 h;
+      h.update(k->codeObject.data(), k->codeObject.size());
+      k->codeSha256 = h.hexDigest();
+      k->cacheHit = true;
+      fromMemory = true;
+    }
+  }
+  if (!k->cacheHit || (fromMemory && !base.empty())) {
     std::string log;
-    int rc = compileToCodeObject(k->lowered, &k->codeObject, &log);
+    int rc = fromMemory ? AKG_HIP_OK : compileToCodeObject(k->lowered, &k->codeObject, &log);
     if (rc != AKG_HIP_OK) {
       if (!base.empty()) (void)writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size());
       return fail(rc, "device compilation of " + k->lowered.kernelName + " failed:\n" + log);
@@ -318,6 +343,10 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
     akg::Sha256 h;
     h.update(k->codeObject.data(), k->codeObject.size());
     k->codeSha256 = h.hexDigest();
+    if (!fromMemory) {
+      std::lock_guard<std::mutex> lock(g_codeCacheMutex);
+      if (g_codeCache.size() < 4096) g_codeCache[srcDigest] = k->codeObject;
+    }
     if (!base.empty()) {
       std::string meta = metaJson(*k, srcDigest);
       std::string shapeArg = shapeArgText(k->lowered);
@@ -385,13 +414,22 @@ const akg::TensorValue &tensorAt(const akg_hip_kernel *k, int index) {
 }
 
 int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream) {
+  // kernel arguments: the tensor pointers, then the 64-bit scalars of the lowering, then the workspace
   const int n = numTensors(k);
-  const int nargs = n + (l.workspace ? 1 : 0);  // the workspace is the kernel's trailing argument
+  const int nscalar = static_cast<int>(k->lowered.scalarArgs.size());
+  const int nargs = n + nscalar + (l.workspace ? 1 : 0);
   std::vector<void *> slots(static_cast<size_t>(nargs));
   std::vector<void *> params(static_cast<size_t>(nargs));
   for (int i = 0; i < nargs; ++i) {
-    slots[static_cast<size_t>(i)] = i < n ? devicePtrs[i] : l.workspace;
-    params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
+    if (i < n) {
+      slots[static_cast<size_t>(i)] = devicePtrs[i];
+      params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
+    } else if (i < n + nscalar) {
+      params[static_cast<size_t>(i)] = const_cast<int64_t *>(&k->lowered.scalarArgs[static_cast<size_t>(i - n)]);
+    } else {
+      slots[static_cast<size_t>(i)] = l.workspace;
+      params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
+    }
   }
   hipError_t e = hipModuleLaunchKernel(l.function, k->lowered.grid[0], k->lowered.grid[1], k->lowered.grid[2],
                                        k->lowered.block[0], k->lowered.block[1], k->lowered.block[2], 0, stream,

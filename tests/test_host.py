@@ -322,6 +322,29 @@ def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     assert e.value.code == -4
 
 
+def test_shape_sets_that_differ_in_the_leading_dimensions_share_one_code_object(tmp_path):
+    """The elementwise / row kernels of a dynamic description take their row count as a kernel argument, so their
+    source does not depend on it: a second shape set with the same row length is served by the code object of the first
+    (no device compilation), with its own grid."""
+    text = open(os.path.join(REF_INFO, "Fused_ReduceMax_fusion_2054638663855723468.info_failed"), encoding="utf-8").read()
+    dyn = driver.HipDynamicKernel(text, out_dir=str(tmp_path))
+    a = dyn.specialize([[100, 768]])
+    b = dyn.specialize([[3, 768]])
+    c = dyn.specialize([[5000, 768]])
+    assert a.source == b.source == c.source
+    assert "const long akg_extent" in a.source and "const long ROWS = akg_extent;" in a.source
+    assert (a.cache_hit, b.cache_hit, c.cache_hit) == (False, True, True)
+    assert len({a.grid, b.grid, c.grid}) == 3 and a.family == "row_reduce"
+    # the static entry point keeps constants
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f16_33x1000.info"), out_dir=None)
+    assert "akg_extent" not in k.source and "constexpr long ROWS = 33L;" in k.source
+    # everything folds into one dimension: the element count is the argument
+    text = open(os.path.join(REF_INFO, "Fused_Sub_Mul_split_1454621004286351279.info_failed"), encoding="utf-8").read()
+    dyn = driver.HipDynamicKernel(text, out_dir=None)
+    a, b = dyn.specialize([[32, 1, 48, 48]]), dyn.specialize([[32, 1, 7, 100]])
+    assert a.source == b.source and "const long COLS = akg_extent;" in a.source and b.cache_hit
+
+
 def test_dynamic_description_is_specialised_per_shape(tmp_path):
     text = open(os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info"),
                 encoding="utf-8").read()
@@ -331,10 +354,11 @@ def test_dynamic_description_is_specialised_per_shape(tmp_path):
     assert a.family == b.family == "row_reduce"
     assert [t.shape for t in a.tensors] == [[32, 1, 48, 48], [32, 12, 48, 48], [32, 12, 48, 48]]
     assert [t.shape for t in b.tensors] == [[1, 1, 40, 72], [32, 12, 40, 72], [32, 12, 40, 72]]
-    assert a.kernel_name != b.kernel_name and a.kernel_name.startswith("Fused_Sub_Mul_Mul_Add_Softmax_fusion_")
+    assert a.kernel_name == b.kernel_name == "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957_kernel"
+    assert a.source != b.source                                                     # 48 and 72 columns: two kernels
     assert dyn.specialize([[32, 1, 48, 48], [32, 12, 48, 48]]) is a                 # cached per shape set
-    for k in (a, b):                                                                # one artifact set per shape
-        assert os.path.exists(os.path.join(str(tmp_path), k.kernel_name[:-len("_kernel")] + ".hsaco"))
+    made = sorted(f for f in os.listdir(str(tmp_path)) if f.endswith(".hsaco"))     # one artifact set per shape set
+    assert len(made) == 2 and all(re.match(r"Fused_Sub_Mul_Mul_Add_Softmax_fusion_\d+_s[0-9a-f]{12}\.hsaco$", f) for f in made)
     with pytest.raises(driver.AkgHipError) as e:    # a static extent of the description cannot be rebound
         dyn.specialize([[32, 1, 48, 48], [31, 12, 48, 48]])
     assert e.value.code == -3 and "contradicts" in str(e.value)
@@ -359,11 +383,14 @@ def _meta_schedule(kernel):
 
 
 def test_artifacts_have_the_reference_layout(tmp_path):
-    info = os.path.join(FIXTURES, "small_quant_int8_residual_bf16_37x1544.info")
+    # under a name of its own: code objects are also remembered per process, by the digest of their source
+    name = "artifact_layout_quant_int8_residual_bf16_37x1544"
+    info = str(tmp_path / (name + ".info"))
+    with open(info, "w", encoding="utf-8") as f:
+        f.write(op_desc.quant_int8_residual(37, 1544, "bfloat16", name))
     out = str(tmp_path / "meta")
     k = driver.HipKernel.from_file(info, out_dir=out)
     assert not k.cache_hit
-    name = "small_quant_int8_residual_bf16_37x1544"
     for ext in (".hsaco", ".json", "_shape_arg.txt", "_shape_info.json", ".hip"):
         assert os.path.exists(os.path.join(out, name + ext))
     shape_info = json.load(open(os.path.join(out, name + "_shape_info.json")))
@@ -380,11 +407,20 @@ def test_artifacts_have_the_reference_layout(tmp_path):
     # [offset, sizes..., strides...] per kernel argument, inputs then outputs
     shape_arg = json.load(open(os.path.join(out, name + "_shape_arg.txt")))
     assert shape_arg == [[0, 37, 1544, 1544, 1], [0, 37, 1544, 1544, 1], [0, 37, 1544, 1544, 1], [0, 37, 1]]
-    # second compile reuses the artifact; a corrupted code object is detected and rebuilt
+    # second compile reuses the artifact; a corrupted code object is detected and replaced
     assert driver.HipKernel.from_file(info, out_dir=out).cache_hit
     with open(os.path.join(out, name + ".hsaco"), "ab") as f:
         f.write(b"x")
-    assert not driver.HipKernel.from_file(info, out_dir=out).cache_hit
+    os.environ["AKG_HIP_NO_CACHE"] = "1"      # no artifact probe and no per-process memory: a device compilation
+    try:
+        assert not driver.HipKernel.from_file(info, out_dir=out).cache_hit
+    finally:
+        del os.environ["AKG_HIP_NO_CACHE"]
+    assert open(os.path.join(out, name + ".hsaco"), "rb").read() == code
+    with open(os.path.join(out, name + ".hsaco"), "ab") as f:
+        f.write(b"x")
+    assert driver.HipKernel.from_file(info, out_dir=out).cache_hit      # served from memory, the file repaired
+    assert open(os.path.join(out, name + ".hsaco"), "rb").read() == code
 
 
 def test_math_selection_follows_the_precision_demand():
