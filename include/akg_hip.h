@@ -64,8 +64,10 @@ typedef struct akg_hip_kernel_info {
   uint64_t algorithmic_bytes;         /* bytes of every input and output, each counted once (an input that is only
                                          sliced or gathered from: the bytes taken out of it) */
   uint64_t algorithmic_ops;           /* 2*M*N*K of the contraction, 0 for bandwidth-bound families */
-  int32_t cache_hit;                  /* 1 if the code object came from the artifact directory */
-  uint64_t workspace_bytes;           /* device scratch the handle owns per device (streaming reductions), else 0 */
+  int32_t cache_hit;                  /* 1 if no device compilation was needed: the code object came from the
+                                         artifact directory or from this process's memory (same source digest) */
+  uint64_t workspace_bytes;           /* device scratch the handle owns per device (streaming reductions, GEMMs
+                                         with K split over workgroups), else 0 */
 } akg_hip_kernel_info;
 
 typedef struct akg_hip_kernel akg_hip_kernel_t;
@@ -151,10 +153,11 @@ void akg_hip_free_string(char *text);
  * Dynamic shapes: a description whose tensors carry -1 dimensions (MindSpore's dynamic-shape graph kernels). The
  * reference compiles such a description once (`akg-opt --gpu-dyn-opt`), passes sizes and strides as kernel arguments
  * ([ptrs[], shape/stride[][]] packing, LLVMParameterPacking.cpp:91-194) and solves the launch shape per call in Python
- * (dynamic_utils.py:269-526). Here every kernel is specialised to its shapes at compile time, so a dynamic description
- * is kept as text and specialised on demand: akg_hip_dynamic_specialize binds the -1s to the given input shapes,
- * derives every op's result shape, compiles (or finds in the artifact directory / in memory) the static kernel for
- * exactly these shapes and returns its handle. The handle is owned by the dynamic object (do not destroy it); it is
+ * (dynamic_utils.py:269-526). Here a dynamic description is kept as text and specialised on demand:
+ * akg_hip_dynamic_specialize binds the -1s to the given input shapes, derives every op's result shape, lowers the
+ * kernel for these shapes and returns its handle. Elementwise and row-reduction kernels take the product of their
+ * leading dimensions as a kernel argument, so shape sets that differ only there share one code object and the second
+ * one needs no device compilation; anything else compiles once per shape set (or is found in the artifact directory). The handle is owned by the dynamic object (do not destroy it); it is
  * launched with akg_hip_launch like any other, and akg_hip_kernel_tensor reports the concrete output shapes.
  */
 typedef struct akg_hip_dynamic akg_hip_dynamic_t;
