@@ -218,7 +218,7 @@ def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
 
 @pytest.mark.parametrize("name", FULL)
 def test_full_size_config_matches_oracle(name):
-    # full BASELINE sizes; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)
+    # the full sizes of the measured configurations; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)
     check_fixture(name, seed=harness.BASE_SEED + 1 + FULL.index(name), openmp=True)
 
 
