@@ -110,7 +110,6 @@ class GemmEmitter {
     const int64_t steps = (k_ * elemBytes() + stepK() - 1) / stepK();
     int64_t want = opt_.split > 0 ? opt_.split : (tiles >= 192 ? 1 : std::min<int64_t>(16, (256 + tiles - 1) / tiles));
     want = std::max<int64_t>(1, std::min<int64_t>(want, opt_.split > 0 ? steps : steps / 4));
-    while (want > 1 && (want - 1) * ((steps + want - 1) / want) >= steps) --want;   // no empty split
     const int64_t partRows = std::min<int64_t>(m_, 256);
     while (want > 1 && tiles * want * partRows * 256 * 4 >= (1LL << 30)) --want;
     if (opt_.split <= 0) {
@@ -119,6 +118,7 @@ class GemmEmitter {
       const int64_t operandBytes = (m_ * k_ + k_ * n_) * elemBytes();
       while (want > 1 && 2 * tiles * want * partRows * 256 * 4 > 4 * operandBytes) --want;
     }
+    while (want > 1 && (want - 1) * ((steps + want - 1) / want) >= steps) --want;   // no empty split
     kSplit_ = static_cast<int>(std::max<int64_t>(1, want));
   }
 

@@ -160,6 +160,41 @@ def test_tensors_of_two_gib_and_more_are_addressed_with_64_bit_offsets(tmp_path)
     assert np.all(np.abs(sums - 1.0) < 2e-2)      # every sampled row is a distribution
 
 
+def _random_gemm_cases(count, seed=123):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(count):
+        kind = str(rng.choice(["i8", "bf16", "f16"]))
+        m = int(rng.choice([1, 3, 16, 33, 64, 100, 200, 256, 257, 300, 511]))
+        n = int(rng.choice([4, 8, 136, 256, 260, 520, 776]))
+        k = int(rng.choice([16, 64, 272, 512, 1008, 2048, 3008, 4096, 8192] if kind == "i8" else
+                           [16, 64, 264, 512, 1000, 2048, 3000, 4096, 8192]))
+        cases.append((kind, m, k, n, bool(rng.integers(0, 2)), str(rng.choice(["gelu", "relu", "none"]))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_gemm_cases(20), ids=lambda c: "%s_%dx%dx%d%s" % (c[0], c[1], c[2], c[3], "_tb" if c[4] else ""))
+def test_gemm_family_on_ragged_shapes_with_and_without_split_k(case, tmp_path):
+    """MatMul fusions on shapes that are no multiple of the tile in any direction, K from one step to 64 (split over up
+    to 16 workgroups per tile when K is long and the tiles are few), both operand layouts."""
+    kind, m, k, n, tb, act = case
+    name = "ragged_gemm_%s_%dx%dx%d%s" % (kind, m, k, n, "_tb" if tb else "")
+    if kind == "i8":
+        text = op_desc.gemm_int8_dequant_bias_gelu(m, k, n, "bfloat16", tb, name)
+    else:
+        text = op_desc.gemm_bias_act(m, k, n, "bfloat16" if kind == "bf16" else "float16", act, tb, "float32", name)
+    path = os.path.join(str(tmp_path), name + ".info")
+    open(path, "w").write(text)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel(text, out_dir=None)
+    print("case %s grid %d workspace %d" % (name, kernel.grid[0], kernel.workspace_bytes), flush=True)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 700)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path, openmp=True, rebuild=True)(inputs)
+    ok, msg = harness.compare(got[0], expect[0], kernel.outputs[0].dtype)
+    assert ok, "%s: %s" % (name, msg)
+
+
 def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
     """After `prepare` a launch allocates nothing and records no memset, so a serving loop can capture a chain of
     kernels once and replay it: a softmax, a column reduction (workspace + arrival counters) and a split-K GEMM
