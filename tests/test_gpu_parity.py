@@ -160,6 +160,47 @@ def test_tensors_of_two_gib_and_more_are_addressed_with_64_bit_offsets(tmp_path)
     assert np.all(np.abs(sums - 1.0) < 2e-2)      # every sampled row is a distribution
 
 
+ODD_LONG_ROWS = {
+    "softmax_f16_3x70001": lambda n: op_desc.softmax_last_axis(3, 70001, "float16", n),
+    "layernorm_bf16_2x57001": lambda n: op_desc.layernorm_residual(2, 57001, "bfloat16", 1e-5, n),
+    "quant_bf16_2x131081": lambda n: op_desc.quant_int8_residual(2, 131081, "bfloat16", n),
+    "argmax_f16_2x100003": lambda n: op_desc.argmax_last_axis([2, 100003], "float16", False, "int32", None, n),
+    "softmax_f32_2x300001": lambda n: op_desc.softmax_last_axis(2, 300001, "float32", n),
+    "layernorm_bf16_3x16391": lambda n: op_desc.layernorm_residual(3, 16391, "bfloat16", 1e-5, n),
+}
+
+
+@pytest.mark.parametrize("case", sorted(ODD_LONG_ROWS))
+def test_rows_that_are_long_and_odd_at_once(case, tmp_path):
+    """Row kernels where the walks over a long row, the packed row and the overlapping last chunk meet."""
+    name = "odd_long_" + case
+    text = ODD_LONG_ROWS[case](name)
+    path = os.path.join(str(tmp_path), name + ".info")
+    open(path, "w").write(text)
+    print("case %s" % name, flush=True)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family == "row_reduce" and "akg_tail" in kernel.source
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 800)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    cols = desc["input_desc"][0][0]["shape"][-1]
+    for d, g, e in zip(kernel.outputs, got, expect):
+        if d.dtype == "float32":
+            # a serial float32 sum of 300 001 terms is itself 1e-4 away from the exact one: float32 results are held
+            # to rtol 1e-5 against the float64 evaluation of the same description instead
+            from oracle import np_ref
+            wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+            exact = np_ref.evaluate(harness.widen_to_float64(desc), wide)[kernel.outputs.index(d)]
+            ok, msg = harness.compare_reassociated(g, exact, d.dtype, cols)
+            gap = float(np.max(np.abs(np.asarray(e, dtype=np.float64) - np.asarray(exact).reshape(e.shape))))
+            msg += " (serial float32 oracle is %.3g away from float64)" % gap
+        else:
+            ok, msg = harness.compare(g, e, d.dtype)
+        print("  %s %s: %s" % (d.name, d.dtype, msg), flush=True)
+        assert ok, "%s output %s: %s" % (name, d.name, msg)
+
+
 def _random_gemm_cases(count, seed=123):
     rng = np.random.default_rng(seed)
     cases = []
