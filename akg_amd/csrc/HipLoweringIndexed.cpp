@@ -783,8 +783,12 @@ class IndexedEmitter {
     }
     closeElementLoop();
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
+      // results are written once and never read by this kernel: non-temporal where whole 64-byte pieces are stored
+      const bool ntOut = opt_.nonTemporal != 0 && opt_.gemmVariant != 5 &&
+                         (space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[i]).dtype))) % 64 == 0;
       stmt(std::string("akg::store_chunk") + (overlapTail_ ? "_unaligned<" : "<") + tagOf(g_.outputs[i]) + ", V" +
-           (overlapTail_ ? "" : ", false") + ">(out" + std::to_string(i) + " + base, o" + std::to_string(i) + ");");
+           (overlapTail_ ? "" : (ntOut ? ", true" : ", false")) + ">(out" + std::to_string(i) + " + base, o" +
+           std::to_string(i) + ");");
     }
     src_ << "}\n";
   }
