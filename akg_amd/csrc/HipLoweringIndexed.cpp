@@ -99,6 +99,7 @@ class IndexedEmitter {
   std::ostringstream src_;
   std::vector<int64_t> space_;  // iteration space: the shape of the outputs
   int vec_ = 1;
+  std::vector<bool> streamedInput_;  // per kernel input: read at most once per element by the whole grid
   bool overlapTail_ = false;   // V does not divide the innermost extent: the last chunk of a row overlaps its neighbour
   int64_t chunksPerRow_ = 1;
   int64_t grid_ = 1;
@@ -189,6 +190,7 @@ class IndexedEmitter {
     const int64_t chunks = numel / space_.back() * chunksPerRow_;
     grid_ = std::max<int64_t>(1, (chunks + kBlock - 1) / kBlock);
     pickStaging();
+    findStreamedInputs();
     if (!staged_.empty() && overlapTail_) {
       // the LDS-tiled transposes keep their own chunking: narrower chunks instead
       overlapTail_ = false;
@@ -203,6 +205,61 @@ class IndexedEmitter {
       }
     }
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
+  }
+
+  // Kernel inputs every element of which is read at most once by the whole grid: they have one consumer, and from
+  // there to a kernel output every op either maps elements one to one (Transpose, Slice, StridedSlice, Pad, Concat,
+  // Reshape, Cast and other elementwise ops on operands of the result's size) or drops some (the slices). A Tile, a
+  // broadcast, a Gather's data operand or a second consumer mean re-use, and such inputs keep ordinary loads.
+  void findStreamedInputs() {
+    streamedInput_.assign(g_.inputs.size(), false);
+    if (opt_.nonTemporal == 0 || opt_.gemmVariant == 5) return;
+    std::vector<int> uses(g_.tensors.size(), 0);
+    for (const OpNode &op : g_.ops) {
+      for (int in : op.inputs) ++uses[static_cast<size_t>(in)];
+    }
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      int id = g_.inputs[i];
+      bool once = true;
+      while (once) {
+        if (uses[static_cast<size_t>(id)] != 1) {
+          once = uses[static_cast<size_t>(id)] == 0 && g_.tensor(id).outputIndex >= 0;   // reached an output
+          break;
+        }
+        const OpNode *consumer = nullptr;
+        for (const OpNode &op : g_.ops) {
+          for (int in : op.inputs) {
+            if (in == id) consumer = &op;
+          }
+        }
+        const TensorValue &from = g_.tensor(id), &to = g_.tensor(consumer->outputs[0]);
+        switch (consumer->kind) {
+          case OpKind::Transpose:
+          case OpKind::Slice:
+          case OpKind::StridedSlice:
+          case OpKind::Pad:
+          case OpKind::Concat:
+          case OpKind::Reshape:
+            break;
+          case OpKind::Tile:
+          case OpKind::BroadcastTo:
+          case OpKind::Gather:
+            once = false;
+            break;
+          default:
+            once = lowering::isElementwiseKind(consumer->kind) && from.numel() == to.numel();
+            break;
+        }
+        if (g_.tensor(consumer->outputs[0]).outputIndex >= 0 && uses[static_cast<size_t>(consumer->outputs[0])] == 0) {
+          break;
+        }
+        id = consumer->outputs[0];
+      }
+      // whole 64-byte pieces only (see the result stores)
+      const TensorValue &t = g_.tensor(g_.inputs[i]);
+      const int64_t rowBytes = (t.shape.empty() ? 1 : t.shape.back()) * static_cast<int64_t>(dtypeSize(t.dtype));
+      streamedInput_[i] = once && rowBytes % 64 == 0;
+    }
   }
 
   // Transposes of kernel inputs that move the innermost axis and produce a tensor of the outputs' shape. All staged
@@ -588,7 +645,9 @@ class IndexedEmitter {
       const std::string tag = tagOf(id);
       hoisted(ctOf(id) + " " + arr + "[V] = {};");
       hoisted(std::string(guard.empty() ? "" : "if (" + guard + ") ") +
-              (alignedAccess ? "akg::load_chunk<" + tag + ", V, false>(in" : "akg::load_chunk_unaligned<" + tag + ", V>(in") +
+              (alignedAccess ? "akg::load_chunk<" + tag + ", V, " +
+                                   (streamedInput_[static_cast<size_t>(t.inputIndex)] ? "true" : "false") + ">(in"
+                             : "akg::load_chunk_unaligned<" + tag + ", V>(in") +
               std::to_string(t.inputIndex) + " + " + offset + ", " + arr + ");");
       it = hoistedLoads_.emplace(key, arr).first;
     }
