@@ -32,7 +32,8 @@ LoweringOptions LoweringOptions::fromEnvironment() {
   o.chunks = readInt("AKG_HIP_CHUNKS");
   o.block = readInt("AKG_HIP_BLOCK");
   o.split = readInt("AKG_HIP_SPLIT");
-  o.gemmVariant = readInt("AKG_HIP_GEMM_VARIANT");
+  o.variant = readInt("AKG_HIP_VARIANT");
+  if (o.variant == 0) o.variant = readInt("AKG_HIP_GEMM_VARIANT");   // the switch's earlier name
   if (const char *nt = std::getenv("AKG_HIP_NT")) o.nonTemporal = (nt[0] != '0') ? 1 : 0;
   return o;
 }

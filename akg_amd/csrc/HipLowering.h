@@ -42,7 +42,12 @@ struct LoweringOptions {
   int chunks = 0;       // chunks per thread
   int block = 0;        // threads per workgroup
   int split = 0;        // streaming reductions: workgroups sharing one group of outputs (AKG_HIP_SPLIT)
-  int gemmVariant = 0;  // GEMM tile configuration selector
+  // Experiment switch (AKG_HIP_VARIANT), read by whichever family lowers the kernel; 0 = the measured default.
+  //   gemm_epilogue  bit 0: 2 x 2 wavefronts per workgroup, bit 1: 64-byte K steps (8-bit only), bit 2: split staging duty
+  //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
+  //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs
+  //   indexed        1: no LDS-tiled transposes, 2: no chunk-wide loads, 3: launch order of tiles, 5: no non-temporal hints
+  int variant = 0;
   int nonTemporal = 1;  // stream once-touched tensors with non-temporal accesses (AKG_HIP_NT=0 turns it off)
   // Dynamic-shape descriptions: the elementwise / row-reduction kernels take their row count (or, when everything
   // folds into one dimension, their element count) as a kernel argument instead of a constant, so that shape sets

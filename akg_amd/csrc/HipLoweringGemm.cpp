@@ -94,11 +94,11 @@ class GemmEmitter {
   }
   const char *accType() const { return elem_ == DType::I8 ? "int" : "float"; }
   // The tuning variants exist for the 8-bit kernel only; 16-bit operands always use 4 x 2 wavefronts and 128-byte steps.
-  // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_GEMM_VARIANT=1.
-  int wavesM() const { return (opt_.gemmVariant & 1) ? 2 : 4; }
-  // Bytes of K in one step: 128 by default, 64 with bit 1 of AKG_HIP_GEMM_VARIANT set.
-  int stepK() const { return (elem_ == DType::I8 && (opt_.gemmVariant & 2)) ? 64 : 128; }
-  bool splitDuty() const { return (opt_.gemmVariant & 4) != 0 && wavesM() == 4; }
+  // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_VARIANT=1.
+  int wavesM() const { return (opt_.variant & 1) ? 2 : 4; }
+  // Bytes of K in one step: 128 by default, 64 with bit 1 of AKG_HIP_VARIANT set.
+  int stepK() const { return (elem_ == DType::I8 && (opt_.variant & 2)) ? 64 : 128; }
+  bool splitDuty() const { return (opt_.variant & 4) != 0 && wavesM() == 4; }
 
   // Few tiles and a long K (a skinny activation in front of a big weight matrix: M = 16 .. 1024 against 8192 x 8192
   // leaves 32 .. 128 of 256 CUs busy, and the time is that of streaming the weights through those few): split K over

@@ -213,7 +213,7 @@ class IndexedEmitter {
   // broadcast, a Gather's data operand or a second consumer mean re-use, and such inputs keep ordinary loads.
   void findStreamedInputs() {
     streamedInput_.assign(g_.inputs.size(), false);
-    if (opt_.nonTemporal == 0 || opt_.gemmVariant == 5) return;
+    if (opt_.nonTemporal == 0 || opt_.variant == 5) return;
     std::vector<int> uses(g_.tensors.size(), 0);
     for (const OpNode &op : g_.ops) {
       for (int in : op.inputs) ++uses[static_cast<size_t>(in)];
@@ -265,7 +265,7 @@ class IndexedEmitter {
   // Transposes of kernel inputs that move the innermost axis and produce a tensor of the outputs' shape. All staged
   // inputs must agree on the output axis their innermost axis lands on (one tiling plane per kernel).
   void pickStaging() {
-    if (opt_.gemmVariant == 1) return;  // AKG_HIP_GEMM_VARIANT=1: pull everything (for comparisons)
+    if (opt_.variant == 1) return;  // AKG_HIP_VARIANT=1: pull everything (for comparisons)
     const size_t rank = space_.size();
     if (rank < 2 || space_.back() < 16) return;
     for (const OpNode &op : g_.ops) {
@@ -626,7 +626,7 @@ class IndexedEmitter {
   // expression of the current element; otherwise return "".
   std::string tryChunkLoad(int id, const Index &idx) {
     const TensorValue &t = g_.tensor(id);
-    if (vec_ < 2 || t.shape.empty() || idx.empty() || opt_.gemmVariant == 2) return std::string();
+    if (vec_ < 2 || t.shape.empty() || idx.empty() || opt_.variant == 2) return std::string();
     const Ix &last = idx.back();
     if (last.kind != 1 || !last.early || t.shape.back() < vec_) return std::string();
     const bool alignedAccess = last.aligned && (t.shape.back() % vec_) == 0;
@@ -696,7 +696,7 @@ class IndexedEmitter {
     // output rows that are not whole cache lines: tiles that write parts of one line next to each other on one XCD
     // (64 x 1000 x 1024 -> 64 x 1024 x 1000 bf16: 33.5 % of the HBM peak in launch order)
     const int64_t outRowBytes = space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[0]).dtype));
-    if (outRowBytes % 64 != 0 && opt_.gemmVariant != 3 && grid_ >= 64) {
+    if (outRowBytes % 64 != 0 && opt_.variant != 3 && grid_ >= 64) {
       src_ << "  int akg_w = akg::xcd_contiguous_id(static_cast<int>(blockIdx.x), " << grid_ << ");\n";
     } else {
       src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
@@ -843,7 +843,7 @@ class IndexedEmitter {
     closeElementLoop();
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       // results are written once and never read by this kernel: non-temporal where whole 64-byte pieces are stored
-      const bool ntOut = opt_.nonTemporal != 0 && opt_.gemmVariant != 5 &&
+      const bool ntOut = opt_.nonTemporal != 0 && opt_.variant != 5 &&
                          (space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[i]).dtype))) % 64 == 0;
       stmt(std::string("akg::store_chunk") + (overlapTail_ ? "_unaligned<" : "<") + tagOf(g_.outputs[i]) + ", V" +
            (overlapTail_ ? "" : (ntOut ? ", true" : ", false")) + ">(out" + std::to_string(i) + " + base, o" +

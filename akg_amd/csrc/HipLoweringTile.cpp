@@ -340,7 +340,7 @@ class TileEmitter {
       // L2), so the register-resident row is kept as long as it fits. Measured, % of the HBM peak, resident / walks:
       // 65536-wide f16 softmax (1 input, 64 values) 62.6 / 46.2; 65536-wide bf16 LayerNorm (2 inputs) 21.9 / 61.3;
       // 32768-wide LayerNorm 70.2 / 63.2; 131072-wide LayerNorm 10.6 / 50.0, softmax 30.1 / 42.3.
-      const int rowPasses = opt_.gemmVariant;  // 1: force the register-resident row, 2: force the walks, 4: walks, packed if possible
+      const int rowPasses = opt_.variant;  // 1: force the register-resident row, 2: force the walks, 4: walks, packed if possible
       int64_t rowInputs = 0;
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
         if (access_[i].lastDimFull && g_.tensor(g_.inputs[i]).numel() == numel_) ++rowInputs;

@@ -345,7 +345,7 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
     k->codeSha256 = h.hexDigest();
     if (!fromMemory) {
       std::lock_guard<std::mutex> lock(g_codeCacheMutex);
-      if (g_codeCache.size() < 4096) g_codeCache[srcDigest] = k->codeObject;
+      if (g_codeCache.size() < 1024) g_codeCache[srcDigest] = k->codeObject;   // bounded: some tens of MB at most
     }
     if (!base.empty()) {
       std::string meta = metaJson(*k, srcDigest);
