@@ -115,7 +115,7 @@ def random_description(seed, allow_views=True, allow_reduce=True):
             notes.append("Cast-" + nt)
         elif allow_views and len(x.t.shape) >= 1 and kind < 1.0:
             t = x.t
-            which = str(rng.choice(["Transpose", "Slice", "StridedSlice", "Pad", "Tile", "Concat", "Reshape"]))
+            which = str(rng.choice(["Transpose", "Slice", "StridedSlice", "Pad", "Tile", "Concat", "Reshape", "Split"]))
             r = len(t.shape)
             if which == "Transpose" and r >= 2:
                 t = op_desc.transpose(b, t, [int(p) for p in rng.permutation(r)])
@@ -137,6 +137,14 @@ def random_description(seed, allow_views=True, allow_reduce=True):
                 y = pick(lambda v: v.t.shape == x.t.shape)
                 t = op_desc.concat(b, t, y.t, int(rng.integers(0, r)))
                 x = Val(t, x.exact and y.exact, bounded=x.bounded and y.bounded)
+            elif which == "Split" and max(t.shape) >= 2:
+                ax = int(rng.choice([d for d in range(r) if t.shape[d] >= 2]))
+                if t.shape[ax] % 2 == 0 and rng.random() < 0.5:     # two equal pieces, both used
+                    lo, hi = op_desc.split(b, t, [t.shape[ax] // 2] * 2, ax)
+                    t = b.sub(lo, hi)
+                else:                                               # unequal pieces, one of them used
+                    cut = int(rng.integers(1, t.shape[ax]))
+                    t = op_desc.split(b, t, [cut, t.shape[ax] - cut], ax)[int(rng.integers(0, 2))]
             elif which == "Reshape" and int(np.prod(t.shape)) > 1:
                 n = int(np.prod(t.shape))
                 divs = [d for d in range(1, n + 1) if n % d == 0]
@@ -166,6 +174,13 @@ def random_description(seed, allow_views=True, allow_reduce=True):
             notes.append("Sub-after-reduce")
         else:
             outs = [b.reduce(name, out.t, axis, bool(rng.random() < 0.5))]
+    if allow_reduce and not used_view and len(outs) == 1 and outs[0] is out.t and out.exact and out.t.shape[-1] >= 2 \
+            and rng.random() < 0.15:
+        # position of the greatest element of every row; only on exactly computed values (a tie broken by an ulp
+        # would name another position), ties themselves are welcome: the first one wins
+        notes.append("ArgMax")
+        return b.dumps([op_desc.argmax(b, out.t, len(out.t.shape) - 1, bool(rng.random() < 0.5),
+                                       str(rng.choice(["int32", "int64"])))]), notes
     final = []
     for t in outs:
         final.append(b.cast(t, dtype) if dtype != "float32" and rng.random() < 0.7 else t)
