@@ -362,7 +362,12 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const int aFragOff = (wm * kWaveRows + fragRow) * kPitch + fragHalf;
   const int bFragOff = (wn * 32 + fragRow) * kPitch + fragHalf;
 
+  // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
+  // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
+  constexpr bool kAllRowsReal = (M % kGemmBM == 0);
+  const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
   auto readFrags = [&](int buf, int ks, v4i (&af)[kTM], v4i (&bf)[4]) {
+    if (!kAllRowsReal && !waveHasRows) return;
     const u8 *la = lds[buf][0] + aFragOff + ks * 32;
     const u8 *lb = lds[buf][1] + bFragOff + ks * 32;
 #pragma unroll
@@ -371,6 +376,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 64 * kPitch);
   };
   auto mfmaAll = [&](const v4i (&af)[kTM], const v4i (&bf)[4]) {
+    if (!kAllRowsReal && !waveHasRows) return;
 #ifndef AKG_DIAG_NO_MFMA
 #pragma unroll
     for (int i = 0; i < kTM; ++i) {
