@@ -106,6 +106,9 @@ FIXTURES = {
     "small_batchmatmul_scale_mask_f16_2x256x128x256": lambda n: op_desc.batch_matmul_scale_mask(2, 256, 128, 256, "float16", False, n),
     "n2_gemm_bf16_bias_gelu_4096x8192x8192": lambda n: op_desc.gemm_bias_act(4096, 8192, 8192, "bfloat16", "gelu", False, "float32", n),
     # the next measured row: bias / scale gradients of a [16384, 4096] bf16 activation (two column sums in one pass)
+    "n4_softmax_f16_512x131072": lambda n: op_desc.softmax_last_axis(512, 131072, "float16", n),
+    "n5_bnstats_bf16_256x64x56x56": lambda n: op_desc.batchnorm_stats(256, 64, 56, 56, "bfloat16", n),
+    "n6_gemm_bf16_bias_gelu_16x8192x8192": lambda n: op_desc.gemm_bias_act(16, 8192, 8192, "bfloat16", "gelu", False, "float32", n),
     "n1_biasgrad_bf16_16384x4096": lambda n: op_desc.bias_grad(16384, 4096, "bfloat16", n),
 }
 

@@ -39,6 +39,11 @@ WORKLOADS = {
     "n3_transpose_bias_add_bf16_32x2048x1024": "f32",
     # bfloat16 MatMul + bias + GELU on the same shape as the int8 fusion (float32 accumulation)
     "n2_gemm_bf16_bias_gelu_4096x8192x8192": "bf16",
+    # shapes off the measured ones: a softmax row of 131072 (kept packed in registers across three walks), batch-norm
+    # statistics (kept axis between reduced ones), a skinny MatMul (K split over workgroups: bound by the weight stream)
+    "n4_softmax_f16_512x131072": "f32",
+    "n5_bnstats_bf16_256x64x56x56": "f32",
+    "n6_gemm_bf16_bias_gelu_16x8192x8192": "bf16",
 }
 DEFAULT_WORKLOAD = "c2_softmax_f16_8192x4096"
 # plain streaming kernel of known size (out = -x, 256 MiB in + 256 MiB out): calibrates the HBM traffic counters
@@ -57,6 +62,9 @@ MEASURED_TRAFFIC_BYTES = {
     "n1_biasgrad_bf16_16384x4096": 270924759,
     "n2_gemm_bf16_bias_gelu_4096x8192x8192": 872910920,
     "n3_transpose_bias_add_bf16_32x2048x1024": 268462651,
+    "n4_softmax_f16_512x131072": 268593234,
+    "n5_bnstats_bf16_256x64x56x56": 102898801,
+    "n6_gemm_bf16_bias_gelu_16x8192x8192": 145144376,
 }
 
 
@@ -108,10 +116,13 @@ def gpu_measure(name, steps, warmup, torch, driver, harness, np):
 
 
 def roofline_of(kernel, kernel_ms, name):
-    if kernel.algorithmic_ops:
+    int8 = WORKLOADS.get(name) == "int8"
+    mfma_peak = INT8_MFMA_PEAK_TOPS if int8 else BF16_MFMA_PEAK_TFLOPS
+    # the bound that takes longer at its peak decides: a contraction with a skinny operand is bound by its operand stream
+    mfma_bound = kernel.algorithmic_ops / (mfma_peak * 1e12) > kernel.algorithmic_bytes / (HBM_PEAK_GBS * 1e9)
+    if kernel.algorithmic_ops and mfma_bound:
         achieved = kernel.algorithmic_ops / (kernel_ms * 1e-3) / 1e12
-        int8 = WORKLOADS.get(name) == "int8"
-        peak = INT8_MFMA_PEAK_TOPS if int8 else BF16_MFMA_PEAK_TFLOPS
+        peak = mfma_peak
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TOP/s" if int8 else "TFLOP/s",
                 "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
     achieved = kernel.algorithmic_bytes / (kernel_ms * 1e-3) / 1e9

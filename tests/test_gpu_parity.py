@@ -105,6 +105,19 @@ def test_full_size_bias_gradient_column_sums():
     check_stream_reduction(os.path.join(FIXTURES, "n1_biasgrad_bf16_16384x4096.info"), seed=harness.BASE_SEED + 11)
 
 
+def test_full_size_long_row_softmax():
+    """f16 [512, 131072]: the row is kept packed in registers across the three walks."""
+    check_fixture("n4_softmax_f16_512x131072.info", seed=harness.BASE_SEED + 13, openmp=True)
+
+
+def test_full_size_batchnorm_statistics():
+    check_stream_reduction(os.path.join(FIXTURES, "n5_bnstats_bf16_256x64x56x56.info"), seed=harness.BASE_SEED + 14)
+
+
+def test_full_size_skinny_matmul_with_split_k():
+    check_fixture("n6_gemm_bf16_bias_gelu_16x8192x8192.info", seed=harness.BASE_SEED + 15, openmp=True)
+
+
 def test_full_size_batched_transpose_bias_add():
     """[32,2048,1024] -> [32,1024,2048] bfloat16 transpose fused with a bias add (indexed family), every element."""
     check_fixture("n3_transpose_bias_add_bf16_32x2048x1024.info", seed=harness.BASE_SEED + 12, openmp=True)
