@@ -170,7 +170,7 @@ def main():
 
     name = args.workload
     kernel, inputs, wall_ms, kernel_ms, nsets = gpu_measure(name, args.steps, args.warmup, torch, driver, harness, np)
-    is_gemm = bool(kernel.algorithmic_ops)
+    is_gemm = roofline_of(kernel, kernel_ms, name)["bound"] == "mfma"
     if is_gemm:
         value = kernel.algorithmic_ops / (wall_ms * 1e-3) / 1e12
         if WORKLOADS.get(name) == "int8":
