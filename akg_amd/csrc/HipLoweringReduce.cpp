@@ -86,11 +86,15 @@ class StreamReduceEmitter {
   // iteration space: the reduced operand's shape; kind per dim (0 outer kept, 1 reduced, 2 inner kept, -1 unit)
   std::vector<int64_t> space_;
   std::vector<int> foldOf_;            // per dim of the reduced operand: the dim of space_ it was folded into
+  std::vector<int64_t> originalSpace_; // the reduced operand's shape, and which of its dims are reduced
+  std::vector<bool> reducedOriginal_;
   std::vector<bool> reducedFolded_;    // per dim of space_
   std::vector<int> kind_;
   int64_t O_ = 1, R_ = 1, I_ = 1;
   bool dirY_ = false;
   std::vector<Phase> phase_;  // per tensor
+  std::vector<bool> invariant_;            // per tensor: computed without anything that varies along the reduced axes
+  std::vector<bool> neededPre_, neededPost_;   // per invariant tensor: read in the streaming loop / after the reduction
   std::vector<const OpNode *> reduces_;
 
   int vec_ = 1, lanes_ = 64, split_ = 1, unroll_ = 4;
@@ -122,6 +126,32 @@ class StreamReduceEmitter {
     if (s.size() > n) throw LoweringError(what + ": rank exceeds the reduced operand's");
     std::vector<int64_t> out(n - s.size(), 1);
     out.insert(out.end(), s.begin(), s.end());
+    // A tensor of the reduced value's shape without keep_dims ([C] next to [N,C,H,W] reduced over N, H, W: running
+    // statistics, per-channel parameters used after the reduction) does not right-align with the operand: its dims are
+    // the kept ones, in order.
+    bool aligned = originalSpace_.size() != n;
+    if (!aligned) {
+      aligned = true;
+      for (size_t d = 0; d < n; ++d) aligned = aligned && (out[d] == 1 || out[d] == originalSpace_[d]);
+    }
+    if (!aligned) {
+      std::vector<int64_t> t = shape;
+      while (!t.empty() && t.front() == 1) t.erase(t.begin());
+      std::vector<size_t> kept;
+      for (size_t d = 0; d < n; ++d) {
+        if (!reducedOriginal_[d] && originalSpace_[d] > 1) kept.push_back(d);
+      }
+      if (t.size() <= kept.size()) {
+        std::vector<int64_t> mapped(n, 1);
+        bool ok = true;
+        for (size_t j = 0; j < t.size(); ++j) {
+          const size_t d = kept[kept.size() - t.size() + j];
+          ok = ok && (t[j] == 1 || t[j] == originalSpace_[d]);
+          mapped[d] = t[j];
+        }
+        if (ok) return mapped;
+      }
+    }
     return out;
   }
   std::vector<int64_t> padTo(const std::vector<int64_t> &shape, const std::string &what) const {
@@ -140,7 +170,8 @@ class StreamReduceEmitter {
         throw LoweringError("op " + op.name + " cannot be fused into a streaming reduction");
       }
       if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
-      if (op.kind == OpKind::Assign) throw LoweringError("op " + op.name + " has no lowering in the streaming-reduction family yet");
+      // Assign / InplaceAssign: allowed after the reduction (running statistics updated from the reduced values);
+      // checked once the phases are known
       if (lowering::isReduceKind(op.kind)) reduces_.push_back(&op);
     }
     if (reduces_.empty()) throw LoweringError("internal: no reduction");
@@ -152,6 +183,8 @@ class StreamReduceEmitter {
     for (size_t a : realReducedAxes(g_, first)) reduced0[a] = true;
     foldOf_.assign(n0, 0);
     for (size_t d = 0; d < n0; ++d) foldOf_[d] = static_cast<int>(d);   // identity while the operands are compared
+    originalSpace_ = original;
+    reducedOriginal_ = reduced0;
     space_ = original;
     for (const OpNode *op : reduces_) {
       const TensorValue &in = g_.tensor(op->inputs[0]);
@@ -236,9 +269,15 @@ class StreamReduceEmitter {
     }
     dirY_ = I_ > 1;
 
-    // phases by data flow: Post = depends on a reduction result
+    // phases by data flow: Post = depends on a reduction result. Values computed only from constants and from kernel
+    // inputs that do not vary along the reduced axes (running statistics, per-channel scales) belong to neither: they
+    // are computed wherever they are needed, before the reduction, after it, or both.
     phase_.assign(g_.tensors.size(), Phase::None);
-    for (int id : g_.inputs) phase_[static_cast<size_t>(id)] = Phase::Pre;
+    invariant_.assign(g_.tensors.size(), false);
+    for (int id : g_.inputs) {
+      phase_[static_cast<size_t>(id)] = Phase::Pre;
+      invariant_[static_cast<size_t>(id)] = !variesAlongReduced(g_.tensor(id));
+    }
     for (const OpNode &op : g_.ops) {
       bool anyPost = false, anyPre = false;
       for (int in : op.inputs) {
@@ -246,10 +285,9 @@ class StreamReduceEmitter {
         if (t.isConst) continue;
         const Phase p = phase_[static_cast<size_t>(in)];
         if (p == Phase::None) throw LoweringError("op " + op.name + ": operand " + t.name + " is undefined");
+        if (invariant_[static_cast<size_t>(in)]) continue;
         if (p == Phase::Post) {
           anyPost = true;
-        } else if (t.producer < 0 && !variesAlongReduced(t)) {
-          // a graph input that does not vary along the reduced axes can be read in either phase
         } else {
           anyPre = true;
         }
@@ -266,6 +304,37 @@ class StreamReduceEmitter {
         phase_[static_cast<size_t>(out)] = Phase::Post;
       } else {
         phase_[static_cast<size_t>(out)] = Phase::Pre;
+        invariant_[static_cast<size_t>(out)] = !anyPre && op.kind != OpKind::Assign;
+      }
+    }
+    // where the invariant values are needed: by ops of the streaming loop, by ops after the reduction, as outputs
+    neededPre_.assign(g_.tensors.size(), false);
+    neededPost_.assign(g_.tensors.size(), false);
+    for (int id : g_.outputs) {
+      if (invariant_[static_cast<size_t>(id)]) neededPost_[static_cast<size_t>(id)] = true;
+    }
+    for (size_t k = g_.ops.size(); k-- > 0;) {
+      const OpNode &op = g_.ops[k];
+      const size_t out = static_cast<size_t>(op.outputs[0]);
+      const bool inLoop = lowering::isReduceKind(op.kind) || (!invariant_[out] && phase_[out] == Phase::Pre) ||
+                          (invariant_[out] && neededPre_[out]);
+      const bool after = (!lowering::isReduceKind(op.kind) && !invariant_[out] && phase_[out] == Phase::Post) ||
+                         (invariant_[out] && neededPost_[out]);
+      for (int in : op.inputs) {
+        if (!invariant_[static_cast<size_t>(in)]) continue;
+        if (inLoop) neededPre_[static_cast<size_t>(in)] = true;
+        if (after) neededPost_[static_cast<size_t>(in)] = true;
+      }
+    }
+    for (const OpNode &op : g_.ops) {
+      if (op.kind != OpKind::Assign) continue;
+      const TensorValue &dst = g_.tensor(op.inputs[0]);
+      if (phase_[static_cast<size_t>(op.outputs[0])] != Phase::Post) {
+        throw LoweringError("op " + op.name + ": only values computed from the reduced results can be assigned in a "
+                            "streaming reduction");
+      }
+      if (dst.inputIndex < 0 || dst.numel() != O_ * I_ || variesAlongReduced(dst)) {
+        throw LoweringError("op " + op.name + ": the destination must be a kernel input of the reduced value's shape");
       }
     }
     const int64_t fullNumel = O_ * R_ * I_;
@@ -573,14 +642,20 @@ class StreamReduceEmitter {
     ident_[static_cast<size_t>(outId)] = name;
   }
 
+  // Is the (non-reduce) op emitted in `phase`? An invariant op is emitted wherever its result is needed.
+  bool emittedIn(const OpNode &op, Phase phase) const {
+    const size_t out = static_cast<size_t>(op.outputs[0]);
+    if (invariant_[out]) return phase == Phase::Pre ? neededPre_[out] : neededPost_[out];
+    return phase_[out] == phase;
+  }
+
   // Inputs that some op of `phase` reads directly.
   std::vector<size_t> inputsUsedIn(Phase phase) const {
     std::vector<bool> used(g_.inputs.size(), false);
     for (const OpNode &op : g_.ops) {
-      const Phase p = phase_[static_cast<size_t>(op.outputs[0])];
       const bool isReduce = lowering::isReduceKind(op.kind);
-      const Phase opPhase = isReduce ? Phase::Pre : p;  // a reduction consumes its operand in the streaming loop
-      if (opPhase != phase) continue;
+      // a reduction consumes its operand in the streaming loop
+      if (isReduce ? phase != Phase::Pre : !emittedIn(op, phase)) continue;
       for (int in : op.inputs) {
         const TensorValue &t = g_.tensor(in);
         if (t.inputIndex >= 0 && !t.isConst) used[static_cast<size_t>(t.inputIndex)] = true;
@@ -605,7 +680,11 @@ class StreamReduceEmitter {
     src_ << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << kname << "(";
     size_t argc = 0;
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
-      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+      bool assigned = false;
+      for (const OpNode &op : g_.ops) {
+        assigned = assigned || (op.kind == OpKind::Assign && g_.tensor(op.inputs[0]).inputIndex == static_cast<int>(i));
+      }
+      src_ << (argc ? ", " : "") << (assigned ? "" : "const ") << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
@@ -729,7 +808,7 @@ class StreamReduceEmitter {
              << " = " << step << ";\n";
         continue;
       }
-      if (phase_[static_cast<size_t>(out)] != Phase::Pre) continue;
+      if (!emittedIn(op, Phase::Pre)) continue;
       emitOp(op, false, in4);
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
@@ -869,8 +948,28 @@ class StreamReduceEmitter {
     }
     for (const OpNode &op : g_.ops) {
       if (lowering::isReduceKind(op.kind)) continue;
-      if (phase_[static_cast<size_t>(op.outputs[0])] != Phase::Post) continue;
+      if (!emittedIn(op, Phase::Post)) continue;
       emitOp(op, scalar, in2);
+    }
+    // Assign: the value also goes over its destination (every element of which this thread has read, if at all,
+    // further up: the post phase runs once per output element, in the last workgroup of its group)
+    for (const OpNode &op : g_.ops) {
+      if (op.kind != OpKind::Assign) continue;
+      const TensorValue &dst = g_.tensor(op.inputs[0]);
+      const std::string tag = tagOf(op.outputs[0]);
+      const std::string arg = "in" + std::to_string(dst.inputIndex);
+      const std::string &value = ident_[static_cast<size_t>(op.outputs[0])];
+      if (scalar) {
+        if (useBuffers_) {
+          src_ << "  if (tid == 0) akg::store_one<" << tag << ">(b_" << arg << ", akg_o, " << value << ");  // " << op.name
+               << " -> " << dst.name << "\n";
+        } else {
+          src_ << "  if (tid == 0) " << arg << "[akg_o] = " << tag << "::store(" << value << ");\n";
+        }
+      } else {
+        src_ << "  akg::store_chunk<" << tag << ", V, false>(" << memRef(arg, "akg_o * I + akg_i") << ", " << value << ");  // "
+             << op.name << " -> " << dst.name << "\n";
+      }
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       const int id = g_.outputs[i];

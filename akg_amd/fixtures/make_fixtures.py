@@ -60,6 +60,8 @@ FIXTURES = {
     "small_reducex_long_sqsum_f32_3x300000": lambda n: op_desc.square_reduce([3, 300000], [1], "float32", False, "ReduceSum", n),
     # kept axes between reduced ones: batch-norm statistics (contiguous runs of H*W), and a [4,5,6,16] sum over axes 0, 2
     "small_bnstats_bf16_8x6x7x12": lambda n: op_desc.batchnorm_stats(8, 6, 7, 12, "bfloat16", n),
+    "small_bnstats_update_bf16_8x6x7x12": lambda n: op_desc.batchnorm_stats_update(8, 6, 7, 12, "bfloat16", 0.9, n),
+    "small_bnstats_update_f32_32x16x28x28": lambda n: op_desc.batchnorm_stats_update(32, 16, 28, 28, "float32", 0.9, n),
     "small_bnstats_f32_32x16x28x28": lambda n: op_desc.batchnorm_stats(32, 16, 28, 28, "float32", n),
     "small_reducey_sqsum_f32_4x5x6x16_axes02": lambda n: op_desc.square_reduce([4, 5, 6, 16], [0, 2], "float32", False, "ReduceSum", n),
     "small_reducey_max_f16_3x4x50x9_axes02_keep": lambda n: op_desc.square_reduce([3, 4, 50, 9], [0, 2], "float16", True, "ReduceMax", n),

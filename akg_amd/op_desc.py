@@ -268,6 +268,27 @@ def batchnorm_stats(n, c, h, w, dtype="bfloat16", name=None):
     return b.dumps([s1, s2])
 
 
+def batchnorm_stats_update(n, c, h, w, dtype="float32", momentum=0.9, name=None):
+    """Training batch norm, statistics half: per-channel mean and variance of x[N,C,H,W] over N, H, W, and the running
+    statistics updated in place from them (two Assigns on [C] inputs). Outputs: mean, variance, and the two assigned
+    values."""
+    b = DescBuilder(name or "Fused_bnstats_update_%s_%dx%dx%dx%d" % (_SHORT[dtype], n, c, h, w))
+    x = b.input([n, c, h, w], dtype)
+    run_mean = b.input([c], "float32")
+    run_var = b.input([c], "float32")
+    xf = b.cast(x, "float32") if dtype != "float32" else x
+    inv = b.const(1.0 / (n * h * w), "float32")
+    mean = b.mul(b.reduce("ReduceSum", xf, [0, 2, 3], False), inv)
+    sq = b.mul(b.reduce("ReduceSum", b.mul(xf, xf), [0, 2, 3], False), inv)
+    var = b.sub(sq, b.mul(mean, mean))
+    keep, take = b.const(momentum, "float32"), b.const(1.0 - momentum, "float32")
+    new_mean = b.add(b.mul(run_mean, keep), b.mul(mean, take))
+    new_var = b.add(b.mul(run_var, keep), b.mul(var, take))
+    a0 = b.op("Assign", [run_mean, new_mean], [c], "float32")
+    a1 = b.op("Assign", [run_var, new_var], [c], "float32")
+    return b.dumps([mean, var, a0, a1])
+
+
 def sub_exp_reduce_y(outer, reduced, inner, dtype="float32", name=None):
     """Two outputs, as the reference's Fused_Sub_Exp_ReduceSum_split: e = exp(x - m) (full shape, stored while
     streaming) and s = sum over the middle axis of e, with m broadcast along the reduced axis."""

@@ -19,7 +19,7 @@ FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__
 STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all", "bnstats")
 ALL_SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
 SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS) and "segment_sum" not in n]
-STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS)]
+STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS) and "bnstats_update" not in n]
 FULL = ["c1_ew_tanh_add_mul_f32_1024x4096.info", "c2_softmax_f16_8192x4096.info",
         "c3_layernorm_residual_bf16_16384x4096.info", "c4_quant_int8_residual_bf16_32768x8192.info"]
 
@@ -552,6 +552,44 @@ def test_assign_overwrites_its_destination_inputs(name):
             assert ok, "step %d input %d: %s" % (step, i, msg)
         assert np.array_equal(host[2], inputs[2])       # the gradient is only read
     assert not np.array_equal(host[0], inputs[0]) and not np.array_equal(host[1], inputs[1])
+
+
+@pytest.mark.parametrize("name", ["small_bnstats_update_f32_32x16x28x28", "small_bnstats_update_bf16_8x6x7x12"])
+def test_running_statistics_are_assigned_after_the_reduction(name):
+    """Batch-norm statistics with the running mean and variance updated in place (Assign after a streaming reduction):
+    mean, variance and the updated running statistics against the float64 evaluation; two launches apply two updates;
+    the activations are only read."""
+    import torch
+    from oracle import np_ref
+    path = os.path.join(FIXTURES, name + ".info")
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    assert kernel.family == "stream_reduce"
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 710)
+    inputs[2] = np.abs(inputs[2]) + 0.5                               # a running variance
+    dev = torch.device("cuda:0")
+    ins = [_torch_view(a.copy()).to(dev) for a in inputs]
+    outs = [torch.empty(d.nbytes, dtype=torch.uint8, device=dev) for d in kernel.outputs]
+    host = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+    terms = int(np.prod(desc["input_desc"][0][0]["shape"])) // host[1].size
+    for step in range(2):
+        kernel.launch(ins + outs)
+        torch.cuda.synchronize()
+        updates = {}
+        exact = np_ref.evaluate(harness.widen_to_float64(desc), host, updates)
+        for d, o, e in zip(kernel.outputs, outs, exact):
+            got = o.cpu().numpy().view(driver.NP_HOST_DTYPE[d.dtype]).reshape(d.shape)
+            ok, msg = harness.compare_reassociated(got, e, d.dtype, terms)
+            print("  step %d %s: %s" % (step, d.name, msg), flush=True)
+            assert ok, "step %d output %s: %s" % (step, d.name, msg)
+        assert sorted(updates) == [1, 2]
+        for i, new in updates.items():
+            host[i] = np.asarray(new, dtype=np.float64)
+            got = ins[i].cpu().numpy().view(np.float32).reshape(host[i].shape)
+            ok, msg = harness.compare_reassociated(got, host[i], "float32", terms)
+            assert ok, "step %d running statistic %d: %s" % (step, i, msg)
+        assert np.array_equal(ins[0].cpu().numpy().view(inputs[0].dtype).reshape(inputs[0].shape), inputs[0])
+    assert not np.allclose(host[1], inputs[1])
 
 
 def test_float32_tanh_accuracy_over_the_whole_range():

@@ -232,6 +232,26 @@ def test_streaming_reduction_family_and_schedule():
     assert k.family == "row_reduce" and k.workspace_bytes == 0
 
 
+def test_assign_after_a_streaming_reduction_stores_over_its_input():
+    """Running statistics of a batch norm: the Assigns take values that exist only after the reduction, so their stores
+    sit in the kernel's last phase, over parameters that are not const; the activations stay read-only. An Assign
+    over the streamed tensor itself with a value built from the reduced result needs a second pass and is refused."""
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_bnstats_update_f32_32x16x28x28.info"))
+    assert k.family == "stream_reduce" and len(k.outputs) == 4
+    params = re.search(r"void\s+\w+_kernel\((.*?)\)\s*\{", k.source, flags=re.S).group(1)
+    assert "const akg::f32::storage *__restrict__ in0" in params
+    assert ", akg::f32::storage *__restrict__ in1" in params
+    assert ", akg::f32::storage *__restrict__ in2" in params
+    post = k.source[k.source.rindex("last_workgroup"):] if "last_workgroup" in k.source else k.source
+    assert "akg::store_one<akg::f32>(b_in1," in post and "akg::store_one<akg::f32>(b_in2," in post
+    b = op_desc.DescBuilder("assign_over_streamed")
+    x = b.input([64, 4096], "float32")
+    s = b.reduce("ReduceSum", x, [0], True)
+    a = b.op("Assign", [x, b.add(x, s)], [64, 4096], "float32")
+    with pytest.raises(driver.AkgHipError):
+        driver.HipKernel(b.dumps([a]))
+
+
 def test_unsorted_segment_sum_translates_and_gets_its_own_family():
     path = os.path.join(REF_INFO, "Fused_UnsortedSegmentSum_split_11686736348673473318.info_failed")
     k = driver.HipKernel.from_file(path)

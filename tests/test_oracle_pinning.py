@@ -465,6 +465,26 @@ def test_assign_writes_the_value_over_its_first_operand(tmp_path):
     assert np.array_equal(n_out[0], v1) and np.array_equal(n_out[1], p1)
 
 
+def test_assign_after_a_reduction_updates_running_statistics(tmp_path):
+    """Batch-norm statistics with the running mean and variance assigned from them, against numpy's own mean and var
+    over (N, H, W) in float64: a reduction over the wrong axes, a biased/unbiased mix-up or swapped momentum weights
+    would each show."""
+    text = op_desc.batchnorm_stats_update(6, 5, 4, 7, "float32", momentum=0.9, name="pin_bn_update")
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((6, 5, 4, 7), dtype=np.float32) * 2 + 1
+    rm, rv = rng.standard_normal(5, dtype=np.float32), rng.random(5, dtype=np.float32) + 0.5
+    ins = [x.copy(), rm.copy(), rv.copy()]
+    updates = {}
+    n_out = np_ref.evaluate(json.loads(text), [x, rm, rv], updates)
+    _, c_out, _ = build_and_run(text, ins, tmp_path)
+    mean, var = x.astype(np.float64).mean(axis=(0, 2, 3)), x.astype(np.float64).var(axis=(0, 2, 3))
+    want = [mean, var, 0.9 * rm + 0.1 * mean, 0.9 * rv + 0.1 * var]
+    for got_c, got_n, w in zip(c_out, n_out, want):
+        assert np.allclose(got_c, w, rtol=2e-5, atol=2e-5) and np.allclose(np.asarray(got_n), w, rtol=2e-5, atol=2e-5)
+    assert np.array_equal(ins[1], c_out[2]) and np.array_equal(ins[2], c_out[3]) and np.array_equal(ins[0], x)
+    assert sorted(updates) == [1, 2] and np.allclose(updates[1], want[2], rtol=2e-5, atol=2e-5)
+
+
 def test_batch_matmul_is_one_product_per_batch_index():
     """BatchMatMul against torch float64 bmm: batches must not mix and transpose_b must read [batch, n, k]."""
     import torch
