@@ -46,6 +46,7 @@ struct LoweringOptions {
   //   gemm_epilogue  bit 0: 2 x 2 wavefronts per workgroup, bit 1: 64-byte K steps (8-bit only), bit 2: split staging duty
   //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
   //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs
+  //   segment_sum    1: every workgroup scans all ids, 2: positions grouped by segment first (whatever the size)
   //   indexed        1: no LDS-tiled transposes, 2: no chunk-wide loads, 3: launch order of tiles, 5: no non-temporal hints
   int variant = 0;
   int nonTemporal = 1;  // stream once-touched tensors with non-temporal accesses (AKG_HIP_NT=0 turns it off)
@@ -56,8 +57,18 @@ struct LoweringOptions {
   static LoweringOptions fromEnvironment();
 };
 
+// A launch that precedes the kernel proper (same arguments, same stream, in order).
+struct KernelPhase {
+  std::string kernelName;
+  unsigned grid[3] = {1, 1, 1};
+  unsigned block[3] = {1, 1, 1};
+};
+
 struct LoweredKernel {
   std::string kernelName;  // "<op>_kernel", as the reference names its outlined gpu.func
+  // Kernels of the same code object that run before `kernelName`, in this order (empty for all families but the
+  // grouped segment sum). Grid, block and name of the kernel proper stay in the fields below.
+  std::vector<KernelPhase> earlierPhases;
   std::string source;      // HIP translation unit
   KernelFamily family = KernelFamily::Elementwise;
   unsigned grid[3] = {1, 1, 1};

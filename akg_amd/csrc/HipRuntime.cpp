@@ -46,6 +46,7 @@ struct akg_hip_kernel {
     int device = -1;
     hipModule_t module = nullptr;
     hipFunction_t function = nullptr;
+    std::vector<hipFunction_t> earlier;  // lowered.earlierPhases, in their order
     void *workspace = nullptr;  // lowered.workspaceBytes of zero-filled device memory, or NULL
   };
   std::vector<Loaded> loaded;
@@ -223,6 +224,17 @@ std::string metaJson(const akg_hip_kernel &k, const std::string &srcDigest) {
   os << "\"algorithmic_bytes\": " << k.lowered.algorithmicBytes << ", ";
   os << "\"algorithmic_ops\": " << k.lowered.algorithmicOps << ", ";
   os << "\"workspace_bytes\": " << k.lowered.workspaceBytes << ", ";
+  if (!k.lowered.earlierPhases.empty()) {
+    // kernels of the same code object to launch before kernelName, in this order, with the same arguments
+    os << "\"earlier_phases\": [";
+    for (size_t i = 0; i < k.lowered.earlierPhases.size(); ++i) {
+      const akg::KernelPhase &ph = k.lowered.earlierPhases[i];
+      os << (i ? ", " : "") << "{\"kernelName\": \"" << jsonEscape(ph.kernelName) << "\", \"blockIdx.x\": " << ph.grid[0]
+         << ", \"blockIdx.y\": " << ph.grid[1] << ", \"blockIdx.z\": " << ph.grid[2] << ", \"threadIdx.x\": " << ph.block[0]
+         << ", \"threadIdx.y\": " << ph.block[1] << ", \"threadIdx.z\": " << ph.block[2] << "}";
+    }
+    os << "], ";
+  }
   os << "\"source_sha256\": \"" << srcDigest << "\"";
   os << "}";
   return os.str();
@@ -386,6 +398,15 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
     (void)hipModuleUnload(l.module);
     return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + k->lowered.kernelName + "): " + hipErr(e));
   }
+  for (const akg::KernelPhase &ph : k->lowered.earlierPhases) {
+    hipFunction_t f = nullptr;
+    e = hipModuleGetFunction(&f, l.module, ph.kernelName.c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(l.module);
+      return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + ph.kernelName + "): " + hipErr(e));
+    }
+    l.earlier.push_back(f);
+  }
   if (k->lowered.workspaceBytes > 0) {
     // Zero-filled once; every launch leaves the arrival counters at zero again. Launches of one handle share the
     // workspace, so they must not overlap on the device (launch them on one stream, or order the streams).
@@ -430,6 +451,12 @@ int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *de
       slots[static_cast<size_t>(i)] = l.workspace;
       params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
     }
+  }
+  for (size_t i = 0; i < l.earlier.size(); ++i) {
+    const akg::KernelPhase &ph = k->lowered.earlierPhases[i];
+    hipError_t pe = hipModuleLaunchKernel(l.earlier[i], ph.grid[0], ph.grid[1], ph.grid[2], ph.block[0], ph.block[1],
+                                          ph.block[2], 0, stream, params.data(), nullptr);
+    if (pe != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLaunchKernel(" + ph.kernelName + "): " + hipErr(pe));
   }
   hipError_t e = hipModuleLaunchKernel(l.function, k->lowered.grid[0], k->lowered.grid[1], k->lowered.grid[2],
                                        k->lowered.block[0], k->lowered.block[1], k->lowered.block[2], 0, stream,

@@ -92,6 +92,10 @@ FIXTURES = {
     "small_segment_sum_f32_300_by_10000_seg7": lambda n: op_desc.unsorted_segment_sum([300], [10000], 7, "float32", "int64", n),
     "small_segment_sum_bf16_4096_by_200_seg1000": lambda n: op_desc.unsorted_segment_sum([4096], [200], 1000, "bfloat16", "int32", n),
     "small_segment_sum_i32_1000_by_65_seg3": lambda n: op_desc.unsorted_segment_sum([1000], [65], 3, "int32", "int32", n),
+    # many positions: grouped by segment first (short rows moved, wide rows through their positions)
+    "small_segment_sum_f32_300000_by_3_seg5000": lambda n: op_desc.unsorted_segment_sum([300000], [3], 5000, "float32", "int32", n),
+    "small_segment_sum_f16_150001_by_4_seg300": lambda n: op_desc.unsorted_segment_sum([150001], [4], 300, "float16", "int64", n),
+    "small_segment_sum_f32_140000_by_40_seg129": lambda n: op_desc.unsorted_segment_sum([140000], [40], 129, "float32", "int32", n),
     "n3_transpose_bias_add_bf16_32x2048x1024": lambda n: op_desc.transpose_bias_add(32, 2048, 1024, "bfloat16", n),
     # float MatMul + bias + activation on the bfloat16 / float16 MFMA path
     "small_gemm_bf16_bias_gelu_256x512x256": lambda n: op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "float32", n),

@@ -59,7 +59,8 @@ typedef struct akg_hip_kernel_info {
   char kernel_name[256];              /* "<op>_kernel" (KernelOutliningExt.cpp:433) */
   char family[32];                    /* "elementwise" | "row_reduce" | "stream_reduce" | "gemm_epilogue" | "indexed" | "segment_sum" */
   char operator_type[32];             /* fusion class, OperatorIdentify.cpp:51-93 */
-  uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json */
+  uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json (of the kernel proper when
+                                         earlier launches precede it: segment sums over many positions) */
   uint32_t block[3];                  /* threadIdx.x/y/z extents */
   uint64_t algorithmic_bytes;         /* bytes of every input and output, each counted once (an input that is only
                                          sliced or gathered from: the bytes taken out of it) */
@@ -67,7 +68,7 @@ typedef struct akg_hip_kernel_info {
   int32_t cache_hit;                  /* 1 if no device compilation was needed: the code object came from the
                                          artifact directory or from this process's memory (same source digest) */
   uint64_t workspace_bytes;           /* device scratch the handle owns per device (streaming reductions, GEMMs
-                                         with K split over workgroups), else 0 */
+                                         with K split over workgroups, grouped segment sums), else 0 */
 } akg_hip_kernel_info;
 
 typedef struct akg_hip_kernel akg_hip_kernel_t;

@@ -251,13 +251,14 @@ def test_gemm_family_on_ragged_shapes_with_and_without_split_k(case, tmp_path):
 
 def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
     """After `prepare` a launch allocates nothing and records no memset, so a serving loop can capture a chain of
-    kernels once and replay it: a softmax, a column reduction (workspace + arrival counters) and a split-K GEMM
-    (workspace) are captured in one graph and replayed four times on fresh inputs, with eager work and
+    kernels once and replay it: a softmax, a column reduction (workspace + arrival counters), a split-K GEMM
+    (workspace) and a grouped segment sum (five launches over one workspace) are captured in one graph and replayed four times on fresh inputs, with eager work and
     synchronisations in between; every replay must equal the eager launches bit for bit (the counters and partials
     of one replay must be ready for the next)."""
     import torch
     dev = torch.device("cuda:0")
-    names = ["small_softmax_f16_64x4096", "small_biasgrad_bf16_2048x1024", "small_gemm_bf16_bias_gelu_100x2048x520"]
+    names = ["small_softmax_f16_64x4096", "small_biasgrad_bf16_2048x1024", "small_gemm_bf16_bias_gelu_100x2048x520",
+             "small_segment_sum_f16_150001_by_4_seg300"]
     kernels, descs = [], []
     for n in names:
         path = os.path.join(FIXTURES, n + ".info")
@@ -265,7 +266,7 @@ def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
         k.prepare()
         kernels.append(k)
         descs.append(harness.load_desc(path))
-    assert kernels[1].workspace_bytes > 0 and kernels[2].workspace_bytes > 0
+    assert kernels[1].workspace_bytes > 0 and kernels[2].workspace_bytes > 0 and kernels[3].workspace_bytes > 0
 
     def buffers(k):
         return [torch.zeros(t.nbytes, dtype=torch.uint8, device=dev) for t in k.tensors]
@@ -383,10 +384,14 @@ def test_segment_sum_is_bit_exact(name):
     check_segment_sum(os.path.join(FIXTURES, name), seed=harness.BASE_SEED + 301)
 
 
-def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero():
+@pytest.mark.parametrize("schedule", ["scan", "grouped"])
+def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero(schedule, monkeypatch, tmp_path):
+    """Both schedules (every workgroup scanning all ids; positions grouped by segment first) on the same small case."""
+    monkeypatch.setenv("AKG_HIP_VARIANT", "1" if schedule == "scan" else "2")
     path = os.path.join(FIXTURES, "small_segment_sum_f32_700x3_by_1x3_seg50.info")
     desc = harness.load_desc(path)
-    kernel = driver.HipKernel.from_file(path)
+    kernel = driver.HipKernel.from_file(path, out_dir=str(tmp_path))
+    assert ("grouped by segment" in kernel.source) == (schedule == "grouped")
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 302)
     ids = inputs[1]
     ids[ids == 17] = 50          # nobody names row 17; 50 and -3 are outside [0, 50)

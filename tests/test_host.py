@@ -282,6 +282,35 @@ def test_unsorted_segment_sum_translates_and_gets_its_own_family():
     assert e.value.code == -4 and "kernel of its own" in str(e.value)
 
 
+def test_segment_sum_over_many_positions_is_grouped_by_segment_first(tmp_path):
+    """From 65536 positions on: four launches that sort the positions by segment (integer counters only) precede the
+    kernel proper; they are listed in the artifact's JSON in launch order, and the handle owns the workspace they
+    share. Short rows are moved into segment order, wide ones stay where they are."""
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_300000_by_3_seg5000.info"), out_dir=str(tmp_path))
+    meta = json.load(open(os.path.join(str(tmp_path), k.kernel_name[:-len("_kernel")] + ".json")))
+    assert k.family == "segment_sum" and "grouped by segment" in meta["schedule"]
+    runs = 300000 // 1024
+    run_length = -(-(-(-300000 // runs)) // 64) * 64
+    runs = -(-300000 // run_length)
+    words = runs * 5000 + 5000 + 5000 + 1
+    words = -(-words // 4) * 4 + 300000 * 3
+    assert k.workspace_bytes == 4 * words
+    names = [p["kernelName"] for p in meta["earlier_phases"]]
+    stem = k.kernel_name[:-len("_kernel")]
+    assert names == [stem + "_count", stem + "_offsets", stem + "_starts", stem + "_place"]
+    assert [p["blockIdx.x"] for p in meta["earlier_phases"]] == [runs, -(-5000 // 16), 1, runs]
+    assert meta["kernelName"] == k.kernel_name and meta["workspace_bytes"] == k.workspace_bytes
+    for n in names + [k.kernel_name]:
+        assert 'void %s(' % n in k.source
+    assert "placed[at + rank] = row[u]" in k.source and "float" in k.source
+    # no float atomics anywhere: the only atomic is the integer count in LDS
+    assert k.source.count("atomicAdd(&akg_cnt[id], 1u)") == 1 and k.source.count("atomic") == 1
+    wide = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_140000_by_40_seg129.info"), out_dir=None)
+    assert "akg_ws[W_SORTED + at + rank] = " in wide.source and "placed" not in wide.source
+    small = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_700x3_by_1x3_seg50.info"), out_dir=None)
+    assert small.workspace_bytes == 0 and "grouped" not in small.source
+
+
 def test_argmax_becomes_a_max_and_a_least_position_in_the_row_family():
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_argmax_f32_37x1000.info"))
     assert k.family == "row_reduce" and [t.dtype for t in k.outputs] == ["int32"]
