@@ -218,23 +218,29 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
   s << "  const int p0 = run * RUN, p1 = p0 + RUN < POSITIONS ? p0 + RUN : POSITIONS;\n";
   s << "  const unsigned long long below = (1ull << lane) - 1ull;\n";
   if (staged) {
-    s << "  constexpr int ROW = " << slice << ";\n";
-    s << "  struct row_t { " << tag << "::storage v[ROW]; };\n";
-    s << "  const row_t *__restrict__ rows = reinterpret_cast<const row_t *>(" << dataName << ");\n";
-    s << "  row_t *__restrict__ placed = reinterpret_cast<row_t *>(akg_ws + W_SORTED);\n";
+    // rows are copied in the widest unit that divides them (their values are not looked at)
+    const int64_t rowBytes = slice * elemBytes;
+    const int unitBytes = rowBytes % 4 == 0 ? 4 : rowBytes % 2 == 0 ? 2 : 1;
+    s << "  using unit_t = " << (unitBytes == 4 ? "unsigned" : unitBytes == 2 ? "unsigned short" : "unsigned char") << ";\n";
+    s << "  constexpr int UNITS = " << rowBytes / unitBytes << ";\n";
+    s << "  const unit_t *__restrict__ rows = reinterpret_cast<const unit_t *>(" << dataName << ");\n";
+    s << "  unit_t *__restrict__ placed = reinterpret_cast<unit_t *>(akg_ws + W_SORTED);\n";
   }
   s << "  for (int base = p0; base < p1; base += 64 * U) {\n";
   s << "    int id[U];\n";
-  if (staged) s << "    row_t row[U];\n";
+  if (staged) s << "    unit_t row[U][UNITS];\n";
   s << "#pragma unroll\n";
   s << "    for (int u = 0; u < U; ++u) {\n";
   s << "      const int p = base + u * 64 + lane;\n";
   s << "      id[u] = p < p1 ? as_segment(" << idTag << "::load(" << idsName << "[p])) : -1;\n";
-  if (staged) s << "      if (p < p1) row[u] = rows[p];\n";
+  if (staged) {
+    s << "#pragma unroll\n";
+    s << "      for (int c = 0; c < UNITS; ++c) row[u][c] = p < p1 ? rows[static_cast<long>(p) * UNITS + c] : unit_t(0);\n";
+  }
   s << "    }\n";
   s << "#pragma unroll\n";
   s << "    for (int u = 0; u < U; ++u) {\n";
-  s << "      if (base + u * 64 >= p1) break;\n";
+  s << "      if (base + u * 64 < p1) {   // (uniform; a guard and not a break, so that the tiles stay in registers)\n";
   s << "      // lanes of this tile with the same id as mine\n";
   s << "      unsigned long long same = __ballot(id[u] >= 0);\n";
   s << "#pragma unroll\n";
@@ -247,11 +253,13 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
   s << "        const unsigned at = akg_next[id[u]];\n";
   s << "        const unsigned rank = static_cast<unsigned>(__popcll(same & below));\n";
   if (staged) {
-    s << "        placed[at + rank] = row[u];\n";
+    s << "#pragma unroll\n";
+    s << "        for (int c = 0; c < UNITS; ++c) placed[static_cast<long>(at + rank) * UNITS + c] = row[u][c];\n";
   } else {
     s << "        akg_ws[W_SORTED + at + rank] = static_cast<unsigned>(base + u * 64 + lane);\n";
   }
   s << "        if ((same >> lane) >> 1 == 0ull) akg_next[id[u]] = at + rank + 1u;   // the group's highest lane\n";
+  s << "      }\n";
   s << "      }\n";
   s << "    }\n";
   s << "  }\n";

@@ -116,6 +116,8 @@ FIXTURES = {
     "n5_bnstats_bf16_256x64x56x56": lambda n: op_desc.batchnorm_stats(256, 64, 56, 56, "bfloat16", n),
     "n6_gemm_bf16_bias_gelu_16x8192x8192": lambda n: op_desc.gemm_bias_act(16, 8192, 8192, "bfloat16", "gelu", False, "float32", n),
     "n1_biasgrad_bf16_16384x4096": lambda n: op_desc.bias_grad(16384, 4096, "bfloat16", n),
+    # the shape of the reference's largest UnsortedSegmentSum description: 24.5 million positions of 3 floats into 4954 rows
+    "n7_segment_sum_f32_4954x4953_by_1x3_seg4954": lambda n: op_desc.unsorted_segment_sum([4954, 4953], [1, 3], 4954, "float32", "int32", n),
 }
 
 

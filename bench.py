@@ -44,6 +44,8 @@ WORKLOADS = {
     "n4_softmax_f16_512x131072": "f32",
     "n5_bnstats_bf16_256x64x56x56": "f32",
     "n6_gemm_bf16_bias_gelu_16x8192x8192": "bf16",
+    # 24.5 million index positions of 3 floats added into 4954 rows in the serial order (five launches per step)
+    "n7_segment_sum_f32_4954x4953_by_1x3_seg4954": "f32",
 }
 DEFAULT_WORKLOAD = "c2_softmax_f16_8192x4096"
 # plain streaming kernel of known size (out = -x, 256 MiB in + 256 MiB out): calibrates the HBM traffic counters
@@ -65,6 +67,7 @@ MEASURED_TRAFFIC_BYTES = {
     "n4_softmax_f16_512x131072": 268593234,
     "n5_bnstats_bf16_256x64x56x56": 102898801,
     "n6_gemm_bf16_bias_gelu_16x8192x8192": 145144376,
+    "n7_segment_sum_f32_4954x4953_by_1x3_seg4954": 2127240577,
 }
 
 

@@ -302,7 +302,7 @@ def test_segment_sum_over_many_positions_is_grouped_by_segment_first(tmp_path):
     assert meta["kernelName"] == k.kernel_name and meta["workspace_bytes"] == k.workspace_bytes
     for n in names + [k.kernel_name]:
         assert 'void %s(' % n in k.source
-    assert "placed[at + rank] = row[u]" in k.source and "float" in k.source
+    assert "placed[static_cast<long>(at + rank) * UNITS + c] = row[u][c]" in k.source
     # no float atomics anywhere: the only atomic is the integer count in LDS
     assert k.source.count("atomicAdd(&akg_cnt[id], 1u)") == 1 and k.source.count("atomic") == 1
     wide = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_140000_by_40_seg129.info"), out_dir=None)
