@@ -306,6 +306,48 @@ def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
                 assert torch.equal(a, b), "replay %d of %s differs from the eager launch" % (replay, k.kernel_name)
 
 
+def test_handles_launched_from_several_threads_on_their_own_streams():
+    """Four threads, each with a handle and a stream of its own (one of them with a workspace, one with five launches
+    per step), launch 40 times at once; every thread's result must equal what the same handle gives alone."""
+    import threading
+    import torch
+    dev = torch.device("cuda:0")
+    names = ["small_softmax_f16_64x4096", "small_biasgrad_bf16_2048x1024", "small_segment_sum_f16_150001_by_4_seg300",
+             "small_gemm_bf16_bias_gelu_100x2048x520"]
+    jobs = []
+    for i, n in enumerate(names):
+        path = os.path.join(FIXTURES, n + ".info")
+        k = driver.HipKernel.from_file(path)
+        k.prepare()
+        inputs = harness.make_inputs(harness.load_desc(path), seed=harness.BASE_SEED + 950 + i)
+        alone = run_on_gpu(k, inputs)
+        ins = [_torch_view(a).to(dev) for a in inputs]
+        outs = [torch.zeros(d.nbytes, dtype=torch.uint8, device=dev) for d in k.outputs]
+        jobs.append((k, ins, outs, alone, torch.cuda.Stream()))
+    torch.cuda.synchronize()
+    failures = []
+
+    def work(job):
+        k, ins, outs, _, stream = job
+        try:
+            for _ in range(40):
+                k.launch(ins + outs, stream=stream)
+            stream.synchronize()
+        except Exception as exc:                                  # noqa: BLE001 - reported by the main thread
+            failures.append((k.kernel_name, repr(exc)))
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not failures, failures
+    for k, _, outs, alone, _ in jobs:
+        for d, o, a in zip(k.outputs, outs, alone):
+            got = o.cpu().numpy().view(driver.NP_HOST_DTYPE[d.dtype]).reshape(d.shape)
+            assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(a).view(np.uint8)), k.kernel_name
+
+
 @pytest.mark.parametrize("name", FULL)
 def test_full_size_config_matches_oracle(name):
     # the full sizes of the measured configurations; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)

@@ -562,6 +562,46 @@ def test_hip_driver_mirrors_the_reference_driver_interface(tmp_path):
         driver.HipDriver(input_file=info, backend="cuda")
 
 
+def test_compiling_from_several_threads_gives_the_serial_results(tmp_path, monkeypatch):
+    """The reference compiles one kernel per process (its schedule tools are process-wide singletons,
+    GlobalVars.hpp:129-132) and forks workers over a directory (benchmark.py:304-317). This library is called from
+    threads instead: eight threads compile different descriptions at once, twice each, into one artifact directory;
+    every code object must equal the one a single thread produces, and errors stay with the thread that made them."""
+    import threading
+    monkeypatch.setenv("AKG_HIP_NO_CACHE", "1")
+    names = ["small_softmax_f16_64x4096", "small_biasgrad_bf16_2048x1024", "small_segment_sum_f32_700x3_by_1x3_seg50",
+             "small_reducey_sqsum_f32_3x37x50", "small_softmax_f32_5x77", "small_gemm_bf16_bias_gelu_100x2048x520",
+             "small_segment_sum_f32_300000_by_3_seg5000", "small_bnstats_update_f32_32x16x28x28"]
+    texts = [open(os.path.join(FIXTURES, n + ".info"), encoding="utf-8").read() for n in names]
+    serial_dir, threaded_dir = str(tmp_path / "serial"), str(tmp_path / "threaded")
+    os.makedirs(serial_dir), os.makedirs(threaded_dir)
+
+    def digest(d, n):
+        return json.load(open(os.path.join(d, n + ".json")))["sha256"]
+    for t in texts:
+        driver.HipKernel(t, out_dir=serial_dir)
+    want = [digest(serial_dir, n) for n in names]
+    failures = []
+
+    def work(i):
+        try:
+            for _ in range(2):
+                k = driver.HipKernel(texts[i], out_dir=threaded_dir)
+                assert k.kernel_name == names[i] + "_kernel"
+                with pytest.raises(driver.AkgHipError) as e:      # this thread's own error text
+                    driver.HipKernel('{"op": "broken_%d"' % i, out_dir=None)
+                assert "broken" in str(e.value) or e.value.code < 0
+        except Exception as exc:                                  # noqa: BLE001 - reported by the main thread
+            failures.append((names[i], repr(exc)))
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(len(names))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
+    assert [digest(threaded_dir, n) for n in names] == want
+
+
 def test_cli_tool():
     tool = os.path.join(ROOT, "akg_amd", "akg-hip")
     info = os.path.join(FIXTURES, "small_softmax_f32_5x77.info")
