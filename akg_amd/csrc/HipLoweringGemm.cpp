@@ -51,21 +51,35 @@ class GemmEmitter {
     k.family = KernelFamily::GemmEpilogue;
     const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
     const int64_t gridTiles = ((tiles + 7) / 8) * 8;
-    k.grid[0] = static_cast<unsigned>(gridTiles * kSplit_);
-    if (kSplit_ > 1) {
-      const int64_t partRows = std::min<int64_t>(m_, 256);
-      k.workspaceBytes = static_cast<uint64_t>((gridTiles * 4 + 255) / 256 * 256 + tiles * kSplit_ * partRows * 256 * 4);
+    if (skinny_) {
+      const int64_t strips = (n_ + 127) / 128;
+      k.grid[0] = static_cast<unsigned>(strips * kSplit_);
+      if (kSplit_ > 1) {
+        const int64_t groups = strips * batch_;
+        k.workspaceBytes = static_cast<uint64_t>((groups * 4 + 255) / 256 * 256 + groups * kSplit_ * m_ * 128 * 4);
+      }
+      k.block[0] = static_cast<unsigned>(skinnyWaves() * 64);
+    } else {
+      k.grid[0] = static_cast<unsigned>(gridTiles * kSplit_);
+      if (kSplit_ > 1) {
+        const int64_t partRows = std::min<int64_t>(m_, 256);
+        k.workspaceBytes = static_cast<uint64_t>((gridTiles * 4 + 255) / 256 * 256 + tiles * kSplit_ * partRows * 256 * 4);
+      }
+      k.block[0] = static_cast<unsigned>(wavesM() * 2 * 64);
     }
     k.grid[1] = static_cast<unsigned>(batch_);
-    k.block[0] = static_cast<unsigned>(wavesM() * 2 * 64);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.algorithmicOps = 2ull * static_cast<uint64_t>(batch_) * static_cast<uint64_t>(m_) * static_cast<uint64_t>(n_) *
                        static_cast<uint64_t>(k_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
-    note << "gemm_epilogue batch=" << batch_ << " M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0)
-         << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
-         << k.grid[0];
+    note << "gemm_epilogue batch=" << batch_ << " M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0);
+    if (skinny_) {
+      note << " skinny: strips of 128 columns, B straight into MFMA operands, mfma=" << mfmaName() << " waves=4 grid=" << k.grid[0];
+    } else {
+      note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
+           << k.grid[0];
+    }
     if (kSplit_ > 1) note << " k_splits=" << kSplit_;
     k.scheduleNote = note.str();
     return k;
@@ -77,6 +91,9 @@ class GemmEmitter {
   std::ostringstream src_;
   int64_t m_ = 0, n_ = 0, k_ = 0, batch_ = 1;
   int kSplit_ = 1;  // workgroups per tile, each with a range of K steps (see pickSplit)
+  int skinnyWaves() const { return opt_.block == 512 ? 8 : 4; }
+  int skinnyUnroll() const { return opt_.chunks > 0 ? opt_.chunks : 2; }
+  bool skinny_ = false;  // M <= 32: the kernel that streams B straight into MFMA operands (gemm_skinny)
   bool transB_ = false;
   int matmulOp_ = -1;
   int aId_ = -1, bId_ = -1, accId_ = -1;
@@ -105,6 +122,21 @@ class GemmEmitter {
   // enough workgroups to fill the chip, at least four K steps each.
   void pickSplit() {
     kSplit_ = 1;
+    // At most 32 rows of A (and K a multiple of 32 bytes): the time is that of streaming B, which gemm_skinny reads
+    // straight into MFMA operands; 256 workgroups of four wavefronts (one per CU: 16 x 8192 x 8192 bf16 reaches 66 % of
+    // the HBM peak with 4 splits of 64 strips, 59 % with 8, 48 % with 2; 8 wavefronts or more steps in flight change
+    // nothing), each wavefront with at least 4 MFMA steps.
+    // AKG_HIP_VARIANT bit 3 keeps the 256 x 256 tile kernel.
+    skinny_ = m_ <= 32 && (k_ * elemBytes()) % 32 == 0 && (transB_ || n_ % 4 == 0) && !(opt_.variant & 8);
+    if (skinny_) {
+      const int64_t strips = (n_ + 127) / 128, steps = k_ * elemBytes() / 32;
+      int64_t want = opt_.split > 0 ? opt_.split : std::max<int64_t>(1, 256 / (strips * batch_));
+      want = std::min<int64_t>(want, std::max<int64_t>(1, opt_.split > 0 ? steps : steps / 16));
+      want = std::min<int64_t>(want, 64);
+      while (want > 1 && strips * batch_ * want * m_ * 128 * 4 >= (1LL << 30)) --want;
+      kSplit_ = static_cast<int>(want);
+      return;
+    }
     if (batch_ != 1) return;
     const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
     const int64_t steps = (k_ * elemBytes() + stepK() - 1) / stepK();
@@ -357,7 +389,7 @@ class GemmEmitter {
     src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[4], long row, long col) {\n"
          << "    const long grow = row0 + row;\n    (void)grow;\n" << apply_.str() << "  }\n";
     src_ << "};\n}  // namespace\n\n";
-    src_ << "extern \"C\" __global__ __launch_bounds__(" << wavesM() * 128 << ") void " << kname << "(";
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << (skinny_ ? skinnyWaves() * 64 : wavesM() * 128) << ") void " << kname << "(";
     size_t argc = 0;
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
@@ -374,6 +406,13 @@ class GemmEmitter {
       src_ << "  epi.in" << i << " = in" << i << ";\n";
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
+    if (skinny_) {
+      src_ << "  akg::gemm_skinny<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
+           << ", Epilogue, " << kSplit_ << ", " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (opt_.nonTemporal != 0 ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in"
+           << g_.tensor(bId_).inputIndex << " + akg_batch * " << k_ * n_ << "L, epi, " << (kSplit_ > 1 ? "akg_ws" : "nullptr")
+           << ", akg_batch * " << (n_ + 127) / 128 << "L);\n}\n";
+      return;
+    }
     src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
          << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ", Epilogue, " << kSplit_
          << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex

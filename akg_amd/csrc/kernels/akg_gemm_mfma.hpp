@@ -510,4 +510,203 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Skinny A (M <= 32 rows: a decoding step, a GEMV): the time is that of streaming B once, so B goes from global memory
+// straight into MFMA operands, without LDS and without barriers in the main loop.
+//   workgroup = 4 wavefronts, one strip of 128 columns, one range of K (KSPLIT ranges per strip)
+//   wavefront w takes the MFMA steps (32 bytes of K each) w, w + 4, ... of that range, two steps' loads in flight
+//   lane (n = lane % 32, g = lane / 32) owns the 4 ADJACENT columns 4n .. 4n+3 of the strip and the 16 bytes
+//   [32 t + 16 g, +16) of K: for a row-major B it loads a (16 bytes of K) x (4 columns) block (8 rows x 8 bytes or
+//   16 rows x 4 bytes) and transposes it in registers into four operands, for [N,K] it loads the four operands as they
+//   are; one MFMA per column of the four, all against the same A operand (rows beyond M repeat row M-1 and are dropped)
+// The four wavefronts add their accumulators through LDS (only the M real rows), the KSPLIT workgroups of a strip
+// through the workspace in split order (counter per strip, then M x 128 partials per strip and split), and the thread
+// that owns (row, 4 columns) runs the epilogue on the sums. Deterministic; B is read exactly once.
+template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT, int WAVES = 4, int UNROLL = 2, bool NT = false>
+AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ Bv, Epilogue &epi,
+                         unsigned *__restrict__ ws, long group0) {
+  constexpr int EB = Mma::kElemBytes;
+  constexpr long K = KE * EB;   // bytes of K per row of A
+  constexpr long NB = N * EB;   // bytes per k-row of a row-major B
+  static_assert(M >= 1 && M <= 32, "at most 32 rows");
+  static_assert(K % 32 == 0, "K must be a multiple of 32 bytes");
+  static_assert(TRANSB || N % 4 == 0, "N must be a multiple of 4");
+  constexpr long kSteps = K / 32;
+  constexpr long kStrips = (N + 127) / 128;
+  constexpr int kWaves = WAVES, U = UNROLL;
+  static_assert(WAVES == 4 || WAVES == 8, "4 or 8 wavefronts");
+  constexpr int kRawWords = 16;   // dwords a lane loads per step: 64 bytes whatever the layout
+  typedef typename Mma::acc_t acc_t;
+  typedef typename Mma::acc_v acc_v;
+  const int tid = static_cast<int>(threadIdx.x), lane = tid & 63, wave = tid >> 6;
+  const long strip = static_cast<long>(blockIdx.x) % kStrips;   // neighbours in launch order read neighbouring columns
+  const int ksplit = static_cast<int>(static_cast<long>(blockIdx.x) / kStrips);
+  const long t0 = kSteps * ksplit / KSPLIT, t1 = kSteps * (ksplit + 1) / KSPLIT;
+  const int n32 = lane & 31, kg = lane >> 5;
+  const long myCol = strip * 128 + 4 * n32;
+  const long ldCol = myCol + 3 < N ? myCol : 0;   // columns beyond N: load something valid, the results are dropped
+  const long rowA = n32 < M ? n32 : M - 1;
+  const char *__restrict__ A = static_cast<const char *>(Av) + rowA * K + kg * 16;
+  const char *__restrict__ B = static_cast<const char *>(Bv);
+  acc_v acc[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[c][v] = 0;
+  }
+  struct Raw {
+    v4i a;
+    u32 w[kRawWords];
+  };
+  auto load = [&](long t, Raw &r) {
+    const long kb = t * 32 + kg * 16;   // this lane's first byte of K
+    r.a = *reinterpret_cast<const v4i *>(A + t * 32);
+    if constexpr (TRANSB) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const v4i *bp = reinterpret_cast<const v4i *>(B + (ldCol + c) * K + kb);
+        const v4i q = NT ? __builtin_nontemporal_load(bp) : *bp;
+        r.w[4 * c + 0] = static_cast<u32>(q[0]);
+        r.w[4 * c + 1] = static_cast<u32>(q[1]);
+        r.w[4 * c + 2] = static_cast<u32>(q[2]);
+        r.w[4 * c + 3] = static_cast<u32>(q[3]);
+      }
+    } else if constexpr (EB == 2) {
+      const long k0 = kb / 2;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        typedef u32 v2u __attribute__((ext_vector_type(2)));
+        const v2u *bp = reinterpret_cast<const v2u *>(B + (k0 + j) * NB + ldCol * 2);
+        const v2u q = NT ? __builtin_nontemporal_load(bp) : *bp;
+        r.w[2 * j] = q[0];
+        r.w[2 * j + 1] = q[1];
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const u32 *bp = reinterpret_cast<const u32 *>(B + (kb + j) * NB + ldCol);
+        r.w[j] = NT ? __builtin_nontemporal_load(bp) : *bp;
+      }
+    }
+  };
+  auto mfma = [&](const Raw &r) {
+    v4i b[4];
+    if constexpr (TRANSB) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b[c][i] = static_cast<int>(r.w[4 * c + i]);
+      }
+    } else if constexpr (EB == 2) {
+      // rows 2i, 2i+1 of the block -> word i of every column's operand
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        b[0][i] = static_cast<int>(pack_lo16(r.w[4 * i], r.w[4 * i + 2]));
+        b[1][i] = static_cast<int>(pack_hi16(r.w[4 * i], r.w[4 * i + 2]));
+        b[2][i] = static_cast<int>(pack_lo16(r.w[4 * i + 1], r.w[4 * i + 3]));
+        b[3][i] = static_cast<int>(pack_hi16(r.w[4 * i + 1], r.w[4 * i + 3]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const u32 rows[4] = {r.w[4 * i], r.w[4 * i + 1], r.w[4 * i + 2], r.w[4 * i + 3]};
+        u32 cols[4];
+        transpose4x4_bytes(rows, cols);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) b[c][i] = static_cast<int>(cols[c]);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = Mma::mma(r.a, b[c], acc[c]);
+  };
+  for (long t = t0 + wave; t < t1; t += kWaves * U) {   // (uniform per wavefront)
+    Raw r[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (t + u * kWaves < t1) load(t + u * kWaves, r[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (t + u * kWaves < t1) mfma(r[u]);
+    }
+  }
+
+  // ---- the four wavefronts' sums, rows below M only, 16 rows at a time: accumulator v of a lane is row
+  // 8 (v / 4) + 4 g + v % 4; thread (c4, r0) then owns 4 columns of the strip and the rows r0, r0 + 8, ...
+  constexpr int kHalfRows = M < 16 ? static_cast<int>(M) : 16;
+  __shared__ acc_t akg_skinny_sum[kWaves][kHalfRows][128];
+  const int c4 = tid & 31, r0 = (tid >> 5) & 7;
+  const long col = strip * 128 + 4 * c4;
+  const bool colOk = col < N && tid < 256;   // (of 8 wavefronts the first four finish the sums)
+  constexpr int kRowsPerThread = (M + 7) / 8;
+  acc_t sum[kRowsPerThread][4];
+#pragma unroll
+  for (int h = 0; h < (M + 15) / 16; ++h) {
+    if (h > 0) __syncthreads();
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      if ((v >> 3) != h) continue;                  // rows 16 h .. 16 h + 15 are the accumulators 8 h .. 8 h + 7
+      const int row = 8 * (v >> 2) + 4 * kg + (v & 3);
+      if (row < M) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) akg_skinny_sum[wave][row - 16 * h][4 * n32 + c] = acc[c][v];
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 2 * h; i < 2 * h + 2 && i < kRowsPerThread; ++i) {
+      const int row = r0 + 8 * i;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        sum[i][c] = 0;
+        if (row < M) {
+#pragma unroll
+          for (int w = 0; w < kWaves; ++w) sum[i][c] += akg_skinny_sum[w][row - 16 * h][4 * c4 + c];
+        }
+      }
+    }
+  }
+  if constexpr (KSPLIT > 1) {
+    constexpr long kPartBytes = M * 128 * static_cast<long>(sizeof(acc_t));
+    const long group = group0 + strip;
+    // layout: [groups x 4 bytes of counters, rounded up to 256][group][split][M][128]
+    const long groups = static_cast<long>(gridDim.y) * kStrips;
+    const long counterBytes = (groups * 4 + 255) / 256 * 256;
+    const Buffer wsBuf = make_buffer(ws, counterBytes + groups * KSPLIT * kPartBytes);
+    const u32 base = static_cast<u32>(counterBytes + group * KSPLIT * kPartBytes);
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; ++i) {
+      const int row = r0 + 8 * i;
+      if (row < M && colOk) {
+        ws_store_chunk<4>(wsBuf, base + static_cast<u32>(ksplit * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))), sum[i]);
+      }
+    }
+    __shared__ unsigned akg_skinny_flag;
+    if (!last_workgroup(ws, group, KSPLIT, tid, &akg_skinny_flag)) return;
+    if (!colOk) return;
+    epi.prepare(col);
+#pragma unroll
+    for (int i = 0; i < kRowsPerThread; ++i) {
+      const int row = r0 + 8 * i;
+      if (row >= M) continue;
+      acc_t total[4] = {0, 0, 0, 0};
+      for (int p = 0; p < KSPLIT; ++p) {
+        acc_t part[4];
+        ws_load_chunk<4>(wsBuf, base + static_cast<u32>(p * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))), part);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) total[c] += part[c];
+      }
+      epi.apply(total, row, col);
+    }
+    return;
+  }
+  if (!colOk) return;
+  epi.prepare(col);
+#pragma unroll
+  for (int i = 0; i < kRowsPerThread; ++i) {
+    const int row = r0 + 8 * i;
+    if (row < M) epi.apply(sum[i], row, col);
+  }
+}
+
 }  // namespace akg

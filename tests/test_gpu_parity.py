@@ -214,6 +214,38 @@ def test_rows_that_are_long_and_odd_at_once(case, tmp_path):
         assert ok, "%s output %s: %s" % (name, d.name, msg)
 
 
+SKINNY_CASES = [("bf16", 1, 1024, 520, False), ("bf16", 16, 4096, 1024, False), ("f16", 16, 2048, 264, True),
+                ("i8", 32, 4096, 260, False), ("i8", 7, 64, 128, True), ("i8", 1, 32, 4, False), ("f16", 5, 16, 136, False),
+                ("bf16", 32, 8192, 136, True), ("batch_bf16", 3, 256, 520, True), ("batch_bf16", 32, 2048, 260, False)]
+
+
+@pytest.mark.parametrize("case", SKINNY_CASES, ids=lambda c: "%s_%dx%dx%d%s" % (c[0], c[1], c[2], c[3], "_tb" if c[4] else ""))
+def test_skinny_matmul_streams_b_into_mfma_operands(case, tmp_path):
+    """At most 32 rows of A: strips of 128 columns, B loaded straight into MFMA operands (transposed in registers when
+    row-major), K split over wavefronts and workgroups. One row to 32, one K step to 256, ragged N, both layouts, all
+    three element types, batched; against the oracle, and twice (the workspace must be left ready)."""
+    kind, m, k, n, tb = case
+    name = "skinny_gemm_%s_%dx%dx%d%s" % (kind, m, k, n, "_tb" if tb else "")
+    if kind == "i8":
+        text = op_desc.gemm_int8_dequant_bias_gelu(m, k, n, "bfloat16", tb, name)
+    elif kind == "batch_bf16":
+        text = op_desc.batch_matmul_scale_mask(5, m, k, n, "bfloat16", tb, name)
+    else:
+        text = op_desc.gemm_bias_act(m, k, n, "bfloat16" if kind == "bf16" else "float16", "gelu", tb, "float32", name)
+    path = os.path.join(str(tmp_path), name + ".info")
+    open(path, "w").write(text)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert "gemm_skinny" in kernel.source
+    print("case %s grid %d x %d workspace %d" % (name, kernel.grid[0], kernel.grid[1], kernel.workspace_bytes), flush=True)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 720)
+    expect = cpu_ref.CpuKernel(path, openmp=True, rebuild=True)(inputs)
+    for launch in range(2):
+        got = run_on_gpu(kernel, inputs)
+        ok, msg = harness.compare(got[0], expect[0], kernel.outputs[0].dtype)
+        assert ok, "%s launch %d: %s" % (name, launch, msg)
+
+
 def _random_gemm_cases(count, seed=123):
     rng = np.random.default_rng(seed)
     cases = []

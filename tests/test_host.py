@@ -562,6 +562,21 @@ def test_hip_driver_mirrors_the_reference_driver_interface(tmp_path):
         driver.HipDriver(input_file=info, backend="cuda")
 
 
+def test_skinny_matmul_gets_the_streaming_kernel():
+    """At most 32 rows of A and K a multiple of 32 bytes: B goes straight into MFMA operands (no 256 x 256 tile), strips
+    of 128 columns times K splits make about 256 workgroups, and the workspace holds a counter per strip plus M x 128
+    partials per strip and split. Other shapes keep the tile kernel."""
+    k = driver.HipKernel(op_desc.gemm_bias_act(16, 8192, 8192, "bfloat16", "gelu", False, "float32", "skinny_a"), out_dir=None)
+    assert "akg::gemm_skinny<akg::MmaBF16, 16L, 8192L, 8192L, false, Epilogue, 4, 4, 2, true>" in k.source
+    assert (k.grid[0], k.block[0]) == (64 * 4, 256) and k.workspace_bytes == 256 + 64 * 4 * 16 * 128 * 4
+    k = driver.HipKernel(op_desc.gemm_int8_dequant_bias_gelu(1, 64, 128, "bfloat16", True, "skinny_b"), out_dir=None)
+    assert "akg::gemm_skinny<akg::MmaI8, 1L, 128L, 64L, true, Epilogue, 1, " in k.source and k.workspace_bytes == 0
+    k = driver.HipKernel(op_desc.gemm_bias_act(33, 1024, 256, "bfloat16", "gelu", False, "float32", "not_skinny_rows"), out_dir=None)
+    assert "gemm_skinny" not in k.source and "gemm_256x256" in k.source
+    k = driver.HipKernel(op_desc.gemm_bias_act(16, 3000, 264, "float16", "relu", True, "float32", "not_skinny_k"), out_dir=None)
+    assert "gemm_skinny" not in k.source                    # 6000 bytes of K: not a multiple of 32
+
+
 def test_compiling_from_several_threads_gives_the_serial_results(tmp_path, monkeypatch):
     """The reference compiles one kernel per process (its schedule tools are process-wide singletons,
     GlobalVars.hpp:129-132) and forks workers over a directory (benchmark.py:304-317). This library is called from
