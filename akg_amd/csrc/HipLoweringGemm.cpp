@@ -91,9 +91,10 @@ class GemmEmitter {
   std::ostringstream src_;
   int64_t m_ = 0, n_ = 0, k_ = 0, batch_ = 1;
   int kSplit_ = 1;  // workgroups per tile, each with a range of K steps (see pickSplit)
+  int skinnyRows() const { return (opt_.variant & 16) ? 32 : 64; }
   int skinnyWaves() const { return opt_.block == 512 ? 8 : 4; }
   int skinnyUnroll() const { return opt_.chunks > 0 ? opt_.chunks : 2; }
-  bool skinny_ = false;  // M <= 32: the kernel that streams B straight into MFMA operands (gemm_skinny)
+  bool skinny_ = false;  // M <= 64: the kernel that streams B straight into MFMA operands (gemm_skinny)
   bool transB_ = false;
   int matmulOp_ = -1;
   int aId_ = -1, bId_ = -1, accId_ = -1;
@@ -122,12 +123,12 @@ class GemmEmitter {
   // enough workgroups to fill the chip, at least four K steps each.
   void pickSplit() {
     kSplit_ = 1;
-    // At most 32 rows of A (and K a multiple of 32 bytes): the time is that of streaming B, which gemm_skinny reads
+    // At most 64 rows of A (and K a multiple of 32 bytes): the time is that of streaming B, which gemm_skinny reads
     // straight into MFMA operands; 256 workgroups of four wavefronts (one per CU: 16 x 8192 x 8192 bf16 reaches 66 % of
     // the HBM peak with 4 splits of 64 strips, 59 % with 8, 48 % with 2; 8 wavefronts or more steps in flight change
     // nothing), each wavefront with at least 4 MFMA steps.
     // AKG_HIP_VARIANT bit 3 keeps the 256 x 256 tile kernel.
-    skinny_ = m_ <= 32 && (k_ * elemBytes()) % 32 == 0 && (transB_ || n_ % 4 == 0) && !(opt_.variant & 8);
+    skinny_ = m_ <= skinnyRows() && (k_ * elemBytes()) % 32 == 0 && (transB_ || n_ % 4 == 0) && !(opt_.variant & 8);
     if (skinny_) {
       const int64_t strips = (n_ + 127) / 128, steps = k_ * elemBytes() / 32;
       int64_t want = opt_.split > 0 ? opt_.split : std::max<int64_t>(1, 256 / (strips * batch_));

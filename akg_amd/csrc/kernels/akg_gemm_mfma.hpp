@@ -511,14 +511,14 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Skinny A (M <= 32 rows: a decoding step, a GEMV): the time is that of streaming B once, so B goes from global memory
+// Skinny A (M <= 64 rows: a decoding step, a GEMV): the time is that of streaming B once, so B goes from global memory
 // straight into MFMA operands, without LDS and without barriers in the main loop.
 //   workgroup = 4 wavefronts, one strip of 128 columns, one range of K (KSPLIT ranges per strip)
 //   wavefront w takes the MFMA steps (32 bytes of K each) w, w + 4, ... of that range, two steps' loads in flight
 //   lane (n = lane % 32, g = lane / 32) owns the 4 ADJACENT columns 4n .. 4n+3 of the strip and the 16 bytes
 //   [32 t + 16 g, +16) of K: for a row-major B it loads a (16 bytes of K) x (4 columns) block (8 rows x 8 bytes or
 //   16 rows x 4 bytes) and transposes it in registers into four operands, for [N,K] it loads the four operands as they
-//   are; one MFMA per column of the four, all against the same A operand (rows beyond M repeat row M-1 and are dropped)
+//   are; one MFMA per column of the four, all against the same one or two A operands (32 rows each; rows beyond M repeat row M-1 and are dropped)
 // The four wavefronts add their accumulators through LDS (only the M real rows), the KSPLIT workgroups of a strip
 // through the workspace in split order (counter per strip, then M x 128 partials per strip and split), and the thread
 // that owns (row, 4 columns) runs the epilogue on the sums. Deterministic; B is read exactly once.
@@ -528,7 +528,8 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
   constexpr int EB = Mma::kElemBytes;
   constexpr long K = KE * EB;   // bytes of K per row of A
   constexpr long NB = N * EB;   // bytes per k-row of a row-major B
-  static_assert(M >= 1 && M <= 32, "at most 32 rows");
+  static_assert(M >= 1 && M <= 64, "at most 64 rows");
+  constexpr int kRowTiles = M > 32 ? 2 : 1;   // MFMA tiles of 32 rows
   static_assert(K % 32 == 0, "K must be a multiple of 32 bytes");
   static_assert(TRANSB || N % 4 == 0, "N must be a multiple of 4");
   constexpr long kSteps = K / 32;
@@ -545,22 +546,30 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
   const int n32 = lane & 31, kg = lane >> 5;
   const long myCol = strip * 128 + 4 * n32;
   const long ldCol = myCol + 3 < N ? myCol : 0;   // columns beyond N: load something valid, the results are dropped
-  const long rowA = n32 < M ? n32 : M - 1;
-  const char *__restrict__ A = static_cast<const char *>(Av) + rowA * K + kg * 16;
+  const char *__restrict__ A[kRowTiles];
+#pragma unroll
+  for (int rt = 0; rt < kRowTiles; ++rt) {
+    const long rowA = 32 * rt + n32 < M ? 32 * rt + n32 : M - 1;
+    A[rt] = static_cast<const char *>(Av) + rowA * K + kg * 16;
+  }
   const char *__restrict__ B = static_cast<const char *>(Bv);
-  acc_v acc[4];
+  acc_v acc[kRowTiles][4];
 #pragma unroll
-  for (int c = 0; c < 4; ++c) {
+  for (int rt = 0; rt < kRowTiles; ++rt) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[c][v] = 0;
+    for (int c = 0; c < 4; ++c) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[rt][c][v] = 0;
+    }
   }
   struct Raw {
-    v4i a;
+    v4i a[kRowTiles];
     u32 w[kRawWords];
   };
   auto load = [&](long t, Raw &r) {
     const long kb = t * 32 + kg * 16;   // this lane's first byte of K
-    r.a = *reinterpret_cast<const v4i *>(A + t * 32);
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt) r.a[rt] = *reinterpret_cast<const v4i *>(A[rt] + t * 32);
     if constexpr (TRANSB) {
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
@@ -617,7 +626,10 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
       }
     }
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] = Mma::mma(r.a, b[c], acc[c]);
+    for (int rt = 0; rt < kRowTiles; ++rt) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[rt][c] = Mma::mma(r.a[rt], b[c], acc[rt][c]);
+    }
   };
   for (long t = t0 + wave; t < t1; t += kWaves * U) {   // (uniform per wavefront)
     Raw r[U];
@@ -645,11 +657,11 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
     if (h > 0) __syncthreads();
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      if ((v >> 3) != h) continue;                  // rows 16 h .. 16 h + 15 are the accumulators 8 h .. 8 h + 7
-      const int row = 8 * (v >> 2) + 4 * kg + (v & 3);
+      if ((v >> 3) != (h & 1)) continue;            // rows 16 h .. 16 h + 15: tile h / 2, accumulators 8 (h % 2) .. + 7
+      const int row = 32 * (h >> 1) + 8 * (v >> 2) + 4 * kg + (v & 3);
       if (row < M) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) akg_skinny_sum[wave][row - 16 * h][4 * n32 + c] = acc[c][v];
+        for (int c = 0; c < 4; ++c) akg_skinny_sum[wave][row - 16 * h][4 * n32 + c] = acc[h >> 1][c][v];
       }
     }
     __syncthreads();

@@ -216,13 +216,15 @@ def test_rows_that_are_long_and_odd_at_once(case, tmp_path):
 
 SKINNY_CASES = [("bf16", 1, 1024, 520, False), ("bf16", 16, 4096, 1024, False), ("f16", 16, 2048, 264, True),
                 ("i8", 32, 4096, 260, False), ("i8", 7, 64, 128, True), ("i8", 1, 32, 4, False), ("f16", 5, 16, 136, False),
-                ("bf16", 32, 8192, 136, True), ("batch_bf16", 3, 256, 520, True), ("batch_bf16", 32, 2048, 260, False)]
+                ("bf16", 32, 8192, 136, True), ("batch_bf16", 3, 256, 520, True), ("batch_bf16", 32, 2048, 260, False),
+                ("bf16", 33, 2048, 264, False), ("i8", 64, 4096, 520, False), ("f16", 48, 1024, 136, True),
+                ("i8", 50, 8192, 128, True), ("batch_bf16", 64, 512, 260, False)]
 
 
 @pytest.mark.parametrize("case", SKINNY_CASES, ids=lambda c: "%s_%dx%dx%d%s" % (c[0], c[1], c[2], c[3], "_tb" if c[4] else ""))
 def test_skinny_matmul_streams_b_into_mfma_operands(case, tmp_path):
-    """At most 32 rows of A: strips of 128 columns, B loaded straight into MFMA operands (transposed in registers when
-    row-major), K split over wavefronts and workgroups. One row to 32, one K step to 256, ragged N, both layouts, all
+    """At most 64 rows of A: strips of 128 columns, B loaded straight into MFMA operands (transposed in registers when
+    row-major), K split over wavefronts and workgroups. One row to 64, one K step to 256, ragged N, both layouts, all
     three element types, batched; against the oracle, and twice (the workspace must be left ready)."""
     kind, m, k, n, tb = case
     name = "skinny_gemm_%s_%dx%dx%d%s" % (kind, m, k, n, "_tb" if tb else "")

@@ -563,7 +563,7 @@ def test_hip_driver_mirrors_the_reference_driver_interface(tmp_path):
 
 
 def test_skinny_matmul_gets_the_streaming_kernel():
-    """At most 32 rows of A and K a multiple of 32 bytes: B goes straight into MFMA operands (no 256 x 256 tile), strips
+    """At most 64 rows of A and K a multiple of 32 bytes: B goes straight into MFMA operands (no 256 x 256 tile), strips
     of 128 columns times K splits make about 256 workgroups, and the workspace holds a counter per strip plus M x 128
     partials per strip and split. Other shapes keep the tile kernel."""
     k = driver.HipKernel(op_desc.gemm_bias_act(16, 8192, 8192, "bfloat16", "gelu", False, "float32", "skinny_a"), out_dir=None)
@@ -571,7 +571,7 @@ def test_skinny_matmul_gets_the_streaming_kernel():
     assert (k.grid[0], k.block[0]) == (64 * 4, 256) and k.workspace_bytes == 256 + 64 * 4 * 16 * 128 * 4
     k = driver.HipKernel(op_desc.gemm_int8_dequant_bias_gelu(1, 64, 128, "bfloat16", True, "skinny_b"), out_dir=None)
     assert "akg::gemm_skinny<akg::MmaI8, 1L, 128L, 64L, true, Epilogue, 1, " in k.source and k.workspace_bytes == 0
-    k = driver.HipKernel(op_desc.gemm_bias_act(33, 1024, 256, "bfloat16", "gelu", False, "float32", "not_skinny_rows"), out_dir=None)
+    k = driver.HipKernel(op_desc.gemm_bias_act(65, 1024, 256, "bfloat16", "gelu", False, "float32", "not_skinny_rows"), out_dir=None)
     assert "gemm_skinny" not in k.source and "gemm_256x256" in k.source
     k = driver.HipKernel(op_desc.gemm_bias_act(16, 3000, 264, "float16", "relu", True, "float32", "not_skinny_k"), out_dir=None)
     assert "gemm_skinny" not in k.source                    # 6000 bytes of K: not a multiple of 32
