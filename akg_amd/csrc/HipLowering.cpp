@@ -17,6 +17,7 @@ const char *kernelFamilyName(KernelFamily f) {
     case KernelFamily::StreamReduce: return "stream_reduce";
     case KernelFamily::Indexed: return "indexed";
     case KernelFamily::SegmentSum: return "segment_sum";
+    case KernelFamily::Staged: return "staged";
   }
   return "?";
 }

@@ -31,7 +31,7 @@ class LoweringError : public std::runtime_error {
   explicit LoweringError(const std::string &msg) : std::runtime_error(msg) {}
 };
 
-enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce, Indexed, SegmentSum };
+enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce, Indexed, SegmentSum, Staged };
 const char *kernelFamilyName(KernelFamily f);
 
 // Tuning knobs; 0 means "let the heuristic decide". They can be set through the environment

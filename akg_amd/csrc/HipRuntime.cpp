@@ -25,6 +25,7 @@
 
 #include "../../include/akg_hip.h"
 #include "HipLowering.h"
+#include "Staging.h"
 #include "Json.h"
 #include "OpGraph.h"
 #include "Sha256.h"
@@ -50,6 +51,14 @@ struct akg_hip_kernel {
     void *workspace = nullptr;  // lowered.workspaceBytes of zero-filled device memory, or NULL
   };
   std::vector<Loaded> loaded;
+  // A description run as a sequence of kernels (Staging.h): each stage is a handle of its own; this handle owns
+  // them and the temporaries between them (its workspace), and has no code object itself.
+  struct Stage {
+    akg_hip_kernel *kernel = nullptr;
+    std::vector<akg::StageArg> args;
+  };
+  std::vector<Stage> stages;
+  std::vector<uint64_t> tempOffsets;
 };
 
 // Code objects compiled in this process, by the digest of their source (identical sources arise when a dynamic
@@ -224,6 +233,29 @@ std::string metaJson(const akg_hip_kernel &k, const std::string &srcDigest) {
   os << "\"algorithmic_bytes\": " << k.lowered.algorithmicBytes << ", ";
   os << "\"algorithmic_ops\": " << k.lowered.algorithmicOps << ", ";
   os << "\"workspace_bytes\": " << k.lowered.workspaceBytes << ", ";
+  if (!k.stages.empty()) {
+    // the description runs as these kernels, in this order, each with artifacts of its own under its name; "args" says
+    // where each tensor of a stage's signature lives: input i / output j of this description, or temporary t at a byte
+    // offset of the workspace
+    os << "\"stages\": [";
+    for (size_t i = 0; i < k.stages.size(); ++i) {
+      const auto &st = k.stages[i];
+      os << (i ? ", " : "") << "{\"kernelName\": \"" << jsonEscape(st.kernel->lowered.kernelName) << "\", \"args\": [";
+      for (size_t a = 0; a < st.args.size(); ++a) {
+        const akg::StageArg &sa = st.args[a];
+        os << (a ? ", " : "");
+        if (sa.kind == akg::StageArg::Kind::Input) {
+          os << "{\"input\": " << sa.index << "}";
+        } else if (sa.kind == akg::StageArg::Kind::Output) {
+          os << "{\"output\": " << sa.index << "}";
+        } else {
+          os << "{\"workspace_offset\": " << k.tempOffsets[static_cast<size_t>(sa.index)] << "}";
+        }
+      }
+      os << "]}";
+    }
+    os << "], ";
+  }
   if (!k.lowered.earlierPhases.empty()) {
     // kernels of the same code object to launch before kernelName, in this order, with the same arguments
     os << "\"earlier_phases\": [";
@@ -274,7 +306,89 @@ std::string shapeInfoJson(const akg::OpGraph &g) {
 }
 
 int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
-              const akg::ShapeBinding *binding = nullptr) {
+              const akg::ShapeBinding *binding = nullptr, bool allowStages = true);
+
+void destroyKernel(akg_hip_kernel *kernel);
+
+// The description as a sequence of kernels. `k` holds the translated graph; `reason` is why no single kernel serves it.
+int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k, const char *outDir,
+                  akg_hip_kernel_t **outKernel, const std::string &reason) {
+  const std::string refusal = std::string("kernel ") + k->graph.name + ": " + reason;
+  akg::StagingPlan plan;
+  std::string why;
+  try {
+    if (!akg::planStages(jsonText, k->graph, &plan, &why)) {
+      return fail(AKG_HIP_ERR_UNSUPPORTED, refusal + " (and it cannot run as several kernels: " + why + ")");
+    }
+  } catch (const std::exception &e) {
+    return fail(AKG_HIP_ERR_UNSUPPORTED, refusal);
+  }
+  bool allHits = true;
+  std::ostringstream source, note;
+  note << "staged: " << plan.stages.size() << " kernels";
+  for (const akg::StagePlan &sp : plan.stages) {
+    akg_hip_kernel_t *stage = nullptr;
+    const int rc = doCompile(sp.jsonText, outDir, &stage, nullptr, false);
+    if (rc != AKG_HIP_OK) {
+      const std::string inner = g_lastError;
+      for (auto &st : k->stages) destroyKernel(st.kernel);
+      k->stages.clear();
+      return fail(AKG_HIP_ERR_UNSUPPORTED, refusal + " (and as several kernels: " + inner + ")");
+    }
+    if (!stage->stages.empty()) {      // a stage must be one kernel
+      destroyKernel(stage);
+      for (auto &st : k->stages) destroyKernel(st.kernel);
+      k->stages.clear();
+      return fail(AKG_HIP_ERR_UNSUPPORTED, refusal);
+    }
+    akg_hip_kernel::Stage st;
+    st.kernel = stage;
+    st.args = sp.args;
+    k->stages.push_back(st);
+    allHits = allHits && stage->cacheHit;
+    source << "// ---- " << stage->lowered.kernelName << "\n" << stage->lowered.source << "\n";
+    note << " | " << stage->lowered.kernelName << ": " << akg::kernelFamilyName(stage->lowered.family) << " grid="
+         << stage->lowered.grid[0] << " block=" << stage->lowered.block[0];
+  }
+  uint64_t offset = 0;
+  for (uint64_t bytes : plan.tempBytes) {
+    k->tempOffsets.push_back(offset);
+    offset += (bytes + 255) / 256 * 256;
+  }
+  const akg_hip_kernel *last = k->stages.back().kernel;
+  k->lowered = akg::LoweredKernel();
+  k->lowered.kernelName = last->lowered.kernelName;
+  k->lowered.family = akg::KernelFamily::Staged;
+  for (int d = 0; d < 3; ++d) {
+    k->lowered.grid[d] = last->lowered.grid[d];
+    k->lowered.block[d] = last->lowered.block[d];
+  }
+  k->lowered.source = source.str();
+  k->lowered.scheduleNote = note.str();
+  k->lowered.algorithmicBytes = akg::lowering::countAlgorithmicBytes(k->graph);
+  k->lowered.shapeArgs = akg::lowering::buildShapeArgs(k->graph);
+  k->lowered.workspaceBytes = offset;
+  k->cacheHit = allHits;
+  if (outDir != nullptr && outDir[0] != 0) {
+    const std::string base = std::string(outDir) + "/" + k->graph.name;
+    const std::string meta = metaJson(*k, sourceDigest(k->lowered.source));
+    const std::string shapeArg = shapeArgText(k->lowered);
+    const std::string shapeInfo = shapeInfoJson(k->graph);
+    if (!writeFile(base + "_shape_info.json", shapeInfo.data(), shapeInfo.size()) ||
+        !writeFile(base + "_shape_arg.txt", shapeArg.data(), shapeArg.size()) ||
+        !writeFile(base + ".json", meta.data(), meta.size())) {
+      for (auto &st : k->stages) destroyKernel(st.kernel);
+      k->stages.clear();
+      return fail(AKG_HIP_ERR_IO, std::string("cannot write artifacts under ") + outDir);
+    }
+  }
+  *outKernel = k.release();
+  g_lastError.clear();
+  return AKG_HIP_OK;
+}
+
+int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
+              const akg::ShapeBinding *binding, bool allowStages) {
   if (outKernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "out_kernel is NULL");
   *outKernel = nullptr;
   std::unique_ptr<akg_hip_kernel> k(new akg_hip_kernel());
@@ -305,6 +419,9 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
     // the kernel keeps the description's name (shape sets may share its code object); the artifacts are per shape set
     k->graph.name += artifactSuffix;
   } catch (const akg::LoweringError &e) {
+    if (binding == nullptr && allowStages) {
+      return compileStaged(jsonText, std::move(k), outDir, outKernel, e.what());
+    }
     return fail(AKG_HIP_ERR_UNSUPPORTED, std::string("kernel ") + k->graph.name + ": " + e.what());
   }
   const std::string srcDigest = sourceDigest(k->lowered.source);
@@ -391,12 +508,20 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
   }
   akg_hip_kernel::Loaded l;
   l.device = device;
-  e = hipModuleLoadData(&l.module, k->codeObject.data());
-  if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLoadData: " + hipErr(e));
-  e = hipModuleGetFunction(&l.function, l.module, k->lowered.kernelName.c_str());
-  if (e != hipSuccess) {
-    (void)hipModuleUnload(l.module);
-    return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + k->lowered.kernelName + "): " + hipErr(e));
+  if (!k->stages.empty()) {
+    for (auto &st : k->stages) {
+      akg_hip_kernel::Loaded ls;
+      const int rc = ensureLoaded(st.kernel, &ls);
+      if (rc != AKG_HIP_OK) return rc;
+    }
+  } else {
+    e = hipModuleLoadData(&l.module, k->codeObject.data());
+    if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLoadData: " + hipErr(e));
+    e = hipModuleGetFunction(&l.function, l.module, k->lowered.kernelName.c_str());
+    if (e != hipSuccess) {
+      (void)hipModuleUnload(l.module);
+      return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + k->lowered.kernelName + "): " + hipErr(e));
+    }
   }
   for (const akg::KernelPhase &ph : k->lowered.earlierPhases) {
     hipFunction_t f = nullptr;
@@ -417,13 +542,23 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
     if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
     if (e != hipSuccess) {
       if (l.workspace) (void)hipFree(l.workspace);
-      (void)hipModuleUnload(l.module);
+      if (l.module) (void)hipModuleUnload(l.module);
       return fail(AKG_HIP_ERR_RUNTIME, "workspace of " + std::to_string(k->lowered.workspaceBytes) + " bytes: " + hipErr(e));
     }
   }
   k->loaded.push_back(l);
   *out = l;
   return AKG_HIP_OK;
+}
+
+void destroyKernel(akg_hip_kernel *kernel) {
+  if (kernel == nullptr) return;
+  for (auto &st : kernel->stages) destroyKernel(st.kernel);
+  for (auto &l : kernel->loaded) {
+    if (l.workspace) (void)hipFree(l.workspace);
+    if (l.module) (void)hipModuleUnload(l.module);
+  }
+  delete kernel;
 }
 
 int numTensors(const akg_hip_kernel *k) { return static_cast<int>(k->graph.inputs.size() + k->graph.outputs.size()); }
@@ -435,6 +570,28 @@ const akg::TensorValue &tensorAt(const akg_hip_kernel *k, int index) {
 }
 
 int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream) {
+  if (!k->stages.empty()) {
+    const size_t nin = k->graph.inputs.size();
+    for (auto &st : k->stages) {
+      akg_hip_kernel::Loaded ls;
+      int rc = ensureLoaded(st.kernel, &ls);
+      if (rc != AKG_HIP_OK) return rc;
+      std::vector<void *> ptrs(st.args.size());
+      for (size_t a = 0; a < st.args.size(); ++a) {
+        const akg::StageArg &sa = st.args[a];
+        if (sa.kind == akg::StageArg::Kind::Input) {
+          ptrs[a] = devicePtrs[sa.index];
+        } else if (sa.kind == akg::StageArg::Kind::Output) {
+          ptrs[a] = devicePtrs[nin + static_cast<size_t>(sa.index)];
+        } else {
+          ptrs[a] = static_cast<char *>(l.workspace) + k->tempOffsets[static_cast<size_t>(sa.index)];
+        }
+      }
+      rc = launchOn(st.kernel, ls, ptrs.data(), stream);
+      if (rc != AKG_HIP_OK) return rc;
+    }
+    return AKG_HIP_OK;
+  }
   // kernel arguments: the tensor pointers, then the 64-bit scalars of the lowering, then the workspace
   const int n = numTensors(k);
   const int nscalar = static_cast<int>(k->lowered.scalarArgs.size());
@@ -660,14 +817,7 @@ int akg_hip_profile(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_pt
   return rc;
 }
 
-void akg_hip_kernel_destroy(akg_hip_kernel_t *kernel) {
-  if (kernel == nullptr) return;
-  for (auto &l : kernel->loaded) {
-    if (l.workspace) (void)hipFree(l.workspace);
-    if (l.module) (void)hipModuleUnload(l.module);
-  }
-  delete kernel;
-}
+void akg_hip_kernel_destroy(akg_hip_kernel_t *kernel) { destroyKernel(kernel); }
 
 const char *akg_hip_last_error(void) { return g_lastError.c_str(); }
 

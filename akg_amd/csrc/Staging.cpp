@@ -1,0 +1,269 @@
+#include "Staging.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <map>
+#include <set>
+#include <sstream>
+
+#include "HipLowering.h"
+#include "Json.h"
+
+namespace akg {
+namespace {
+
+std::string quote(const std::string &s) {
+  std::string o = "\"";
+  for (char c : s) {
+    switch (c) {
+      case '"': o += "\\\""; break;
+      case '\\': o += "\\\\"; break;
+      case '\n': o += "\\n"; break;
+      case '\r': o += "\\r"; break;
+      case '\t': o += "\\t"; break;
+      default:
+        if (static_cast<unsigned char>(c) < 0x20) {
+          char buf[8];
+          std::snprintf(buf, sizeof(buf), "\\u%04x", c);
+          o += buf;
+        } else {
+          o += c;
+        }
+    }
+  }
+  return o + "\"";
+}
+
+// The document model back to text (numbers written as integers stay integers, others keep 17 digits).
+std::string dump(const json::Value &v) {
+  switch (v.kind()) {
+    case json::Value::Kind::Null: return "null";
+    case json::Value::Kind::Bool: return v.asBool() ? "true" : "false";
+    case json::Value::Kind::Number: {
+      if (v.isInteger()) return std::to_string(v.asInt());
+      char buf[40];
+      std::snprintf(buf, sizeof(buf), "%.17g", v.asDouble());
+      return buf;
+    }
+    case json::Value::Kind::String: return quote(v.asString());
+    case json::Value::Kind::Array: {
+      std::string o = "[";
+      for (size_t i = 0; i < v.size(); ++i) o += (i ? ", " : "") + dump(v[i]);
+      return o + "]";
+    }
+    case json::Value::Kind::Object: {
+      std::string o = "{";
+      bool first = true;
+      for (const auto &m : v.members()) {
+        o += (first ? "" : ", ") + quote(m.first) + ": " + dump(m.second);
+        first = false;
+      }
+      return o + "}";
+    }
+  }
+  return "null";
+}
+
+std::string tensorEntry(const TensorValue &t) {
+  std::ostringstream o;
+  o << "{\"data_type\": " << quote(dtypeName(t.dtype)) << ", \"format\": \"DefaultFormat\", \"shape\": [";
+  for (size_t i = 0; i < t.shape.size(); ++i) o << (i ? ", " : "") << t.shape[i];
+  o << "], \"tensor_name\": " << quote(t.name) << "}";
+  return o.str();
+}
+
+}  // namespace
+
+bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan, std::string *why) {
+  plan->stages.clear();
+  plan->tempBytes.clear();
+  const json::Value doc = json::Value::parse(jsonText);
+  if (!doc.contains("op_desc") || doc.at("op_desc").size() != g.ops.size()) {
+    *why = "its op entries do not map one to one onto the translated ops";
+    return false;
+  }
+  const json::Value &opDesc = doc.at("op_desc");
+  for (size_t i = 0; i < g.ops.size(); ++i) {
+    const OpNode &op = g.ops[i];
+    if (!opDesc[i].contains("name") || opDesc[i].at("name").asString() != op.name) {
+      *why = "its op entries do not map one to one onto the translated ops";
+      return false;
+    }
+    if (op.kind == OpKind::Assign || op.kind == OpKind::MatMul || op.kind == OpKind::SegmentSum ||
+        op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported) {
+      *why = "op " + op.name + " is not cut into stages";
+      return false;
+    }
+    if (op.outputs.size() != 1) {
+      *why = "op " + op.name + " has several results";
+      return false;
+    }
+  }
+  {
+    std::set<int> distinct(g.outputs.begin(), g.outputs.end());
+    if (distinct.size() != g.outputs.size()) {
+      *why = "an output is listed twice";
+      return false;
+    }
+  }
+  const size_t nt = g.tensors.size();
+  std::vector<int> level(nt, 0);
+  std::vector<bool> reduced(nt, false);
+  for (const OpNode &op : g.ops) {
+    int lv = 0;
+    for (int in : op.inputs) lv = std::max(lv, level[static_cast<size_t>(in)]);
+    const bool isReduce = lowering::isReduceKind(op.kind);
+    for (int out : op.outputs) {
+      level[static_cast<size_t>(out)] = lv + (isReduce ? 1 : 0);
+      reduced[static_cast<size_t>(out)] = isReduce;
+    }
+  }
+  // tensors some output of the description depends on
+  std::vector<bool> needed(nt, false);
+  {
+    std::vector<int> work(g.outputs.begin(), g.outputs.end());
+    while (!work.empty()) {
+      const int t = work.back();
+      work.pop_back();
+      if (needed[static_cast<size_t>(t)]) continue;
+      needed[static_cast<size_t>(t)] = true;
+      const int p = g.tensor(t).producer;
+      if (p >= 0) {
+        for (int in : g.ops[static_cast<size_t>(p)].inputs) work.push_back(in);
+      }
+    }
+  }
+  int maxLevel = 0;
+  for (int t : g.outputs) maxLevel = std::max(maxLevel, level[static_cast<size_t>(t)]);
+
+  // where the reduction results live
+  std::map<int, int> tempOf;
+  for (size_t t = 0; t < nt; ++t) {
+    if (!reduced[t] || !needed[t] || g.tensors[t].outputIndex >= 0) continue;
+    tempOf[static_cast<int>(t)] = static_cast<int>(plan->tempBytes.size());
+    plan->tempBytes.push_back(static_cast<uint64_t>(g.tensors[t].numel()) * dtypeSize(g.tensors[t].dtype));
+  }
+
+  // one kernel per target group
+  auto addKernel = [&](const std::vector<int> &targets, int stage) {
+    // ops on the way to the targets, cut at the description's inputs and at reduction results of earlier stages
+    std::set<int> targetSet(targets.begin(), targets.end());
+    std::vector<bool> opUsed(g.ops.size(), false);
+    std::set<int> cutInputs;       // reduction results read from memory
+    std::set<int> graphInputs;     // description inputs read
+    std::vector<int> work(targets.begin(), targets.end());
+    std::set<int> seen;
+    while (!work.empty()) {
+      const int t = work.back();
+      work.pop_back();
+      if (!seen.insert(t).second) continue;
+      const TensorValue &tv = g.tensor(t);
+      if (tv.isConst) continue;
+      if (tv.inputIndex >= 0) {
+        graphInputs.insert(tv.inputIndex);
+        continue;
+      }
+      const bool earlier = reduced[static_cast<size_t>(t)] && level[static_cast<size_t>(t)] <= stage && !targetSet.count(t);
+      if (earlier) {
+        cutInputs.insert(t);
+        continue;
+      }
+      if (tv.producer < 0) continue;
+      opUsed[static_cast<size_t>(tv.producer)] = true;
+      for (int in : g.ops[static_cast<size_t>(tv.producer)].inputs) work.push_back(in);
+    }
+    StagePlan sp;
+    std::ostringstream o;
+    const std::string name = g.name + "_stage" + std::to_string(plan->stages.size());
+    o << "{\"op\": " << quote(name);
+    for (const char *key : {"process", "platform", "composite", "version", "target_info"}) {
+      if (doc.contains(key)) o << ", " << quote(key) << ": " << dump(doc.at(key));
+    }
+    o << ", \"input_desc\": [";
+    bool first = true;
+    for (int idx : graphInputs) {
+      o << (first ? "" : ", ") << "[" << tensorEntry(g.tensor(g.inputs[static_cast<size_t>(idx)])) << "]";
+      first = false;
+      StageArg a;
+      a.kind = StageArg::Kind::Input;
+      a.index = idx;
+      sp.args.push_back(a);
+    }
+    for (int t : cutInputs) {
+      o << (first ? "" : ", ") << "[" << tensorEntry(g.tensor(t)) << "]";
+      first = false;
+      StageArg a;
+      if (g.tensor(t).outputIndex >= 0) {
+        a.kind = StageArg::Kind::Output;
+        a.index = g.tensor(t).outputIndex;
+      } else {
+        a.kind = StageArg::Kind::Temp;
+        a.index = tempOf.at(t);
+      }
+      sp.args.push_back(a);
+    }
+    o << "], \"op_desc\": [";
+    first = true;
+    for (size_t i = 0; i < g.ops.size(); ++i) {
+      if (!opUsed[i]) continue;
+      o << (first ? "" : ", ") << dump(opDesc[i]);
+      first = false;
+    }
+    o << "], \"output_desc\": [";
+    first = true;
+    for (int t : targets) {
+      o << (first ? "" : ", ") << tensorEntry(g.tensor(t));
+      first = false;
+      StageArg a;
+      if (g.tensor(t).outputIndex >= 0) {
+        a.kind = StageArg::Kind::Output;
+        a.index = g.tensor(t).outputIndex;
+      } else {
+        a.kind = StageArg::Kind::Temp;
+        a.index = tempOf.at(t);
+      }
+      sp.args.push_back(a);
+    }
+    o << "]}";
+    sp.jsonText = o.str();
+    plan->stages.push_back(sp);
+  };
+
+  for (int s = 0; s <= maxLevel; ++s) {
+    // the reductions over operands of level s, grouped by operand shape and axes (one reduction space per kernel)
+    std::map<std::string, std::vector<int>> reduceGroups;
+    for (const OpNode &op : g.ops) {
+      if (!lowering::isReduceKind(op.kind)) continue;
+      const int out = op.outputs[0];
+      if (!needed[static_cast<size_t>(out)] || level[static_cast<size_t>(out)] != s + 1) continue;
+      std::ostringstream key;
+      for (int64_t d : g.tensor(op.inputs[0]).shape) key << d << "x";
+      key << "/";
+      for (int64_t a : op.axes) key << a << ",";
+      key << (op.keepDims ? "k" : "");
+      reduceGroups[key.str()].push_back(out);
+    }
+    for (const auto &kv : reduceGroups) addKernel(kv.second, s);
+    // the description's other outputs of this level, one kernel per shape
+    std::map<std::string, std::vector<int>> outputGroups;
+    for (int t : g.outputs) {
+      if (level[static_cast<size_t>(t)] != s || reduced[static_cast<size_t>(t)]) continue;
+      if (g.tensor(t).inputIndex >= 0 || g.tensor(t).isConst) {
+        *why = "an output is an input of the description";
+        return false;
+      }
+      std::ostringstream key;
+      for (int64_t d : g.tensor(t).shape) key << d << "x";
+      std::vector<int> &grp = outputGroups[key.str()];
+      if (std::find(grp.begin(), grp.end(), t) == grp.end()) grp.push_back(t);
+    }
+    for (const auto &kv : outputGroups) addKernel(kv.second, s);
+  }
+  if (plan->stages.size() < 2) {
+    *why = "it has no reduction result to cut at";
+    return false;
+  }
+  return true;
+}
+
+}  // namespace akg

@@ -92,6 +92,12 @@ FIXTURES = {
     "small_segment_sum_f32_300_by_10000_seg7": lambda n: op_desc.unsorted_segment_sum([300], [10000], 7, "float32", "int64", n),
     "small_segment_sum_bf16_4096_by_200_seg1000": lambda n: op_desc.unsorted_segment_sum([4096], [200], 1000, "bfloat16", "int32", n),
     "small_segment_sum_i32_1000_by_65_seg3": lambda n: op_desc.unsorted_segment_sum([1000], [65], 3, "int32", "int32", n),
+    # descriptions no single kernel serves: run as a sequence of kernels cut at the reduction results
+    "small_staged_softmax_f32_32x12x24x40_axis1": lambda n: op_desc.softmax_over_axis([32, 12, 24, 40], 1, "float32", n),
+    "small_staged_softmax_f16_50x3000_axis0": lambda n: op_desc.softmax_over_axis([50, 3000], 0, "float16", n),
+    "small_staged_bn_train_forward_f32_16x8x14x14": lambda n: op_desc.batchnorm_train_forward(16, 8, 14, 14, "float32", 1e-5, n),
+    "small_staged_bn_train_forward_bf16_8x6x7x12": lambda n: op_desc.batchnorm_train_forward(8, 6, 7, 12, "bfloat16", 1e-5, n),
+    "small_staged_layernorm_axis1_bf16_8x64x49": lambda n: op_desc.layernorm_over_axis1(8, 64, 49, "bfloat16", 1e-5, n),
     # many positions: grouped by segment first (short rows moved, wide rows through their positions)
     "small_segment_sum_f32_300000_by_3_seg5000": lambda n: op_desc.unsorted_segment_sum([300000], [3], 5000, "float32", "int32", n),
     "small_segment_sum_f16_150001_by_4_seg300": lambda n: op_desc.unsorted_segment_sum([150001], [4], 300, "float16", "int64", n),

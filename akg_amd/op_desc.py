@@ -169,6 +169,52 @@ def softmax_last_axis(rows, cols, dtype="float16", name=None):
     return b.dumps([out])
 
 
+def softmax_over_axis(shape, axis, dtype="float32", name=None):
+    """Softmax over any one axis of `shape` (the channel axis of an NCHW tensor, say). Over an axis that is not the last
+    one no single kernel serves it: the max, the sum and the quotient each need a pass of their own."""
+    b = DescBuilder(name or "Fused_ReduceMax_Sub_Exp_ReduceSum_RealDiv_softmax_%s_%s_axis%d" % (
+        _SHORT[dtype], "x".join(str(d) for d in shape), axis))
+    x = b.input(list(shape), dtype)
+    xf = b.cast(x, "float32") if dtype != "float32" else x
+    mx = b.reduce("ReduceMax", xf, [axis], True)
+    e = b.unary("Exp", b.sub(xf, mx))
+    p = b.div(e, b.reduce("ReduceSum", e, [axis], True))
+    return b.dumps([b.cast(p, dtype) if dtype != "float32" else p])
+
+
+def batchnorm_train_forward(n, c, h, w, dtype="float32", eps=1e-5, name=None):
+    """Training batch norm in one description: per-channel mean and variance of x[N,C,H,W] over N, H, W (keep_dims),
+    y = (x - mean) * rsqrt(var + eps) * gamma + beta. Outputs: y, mean, variance."""
+    b = DescBuilder(name or "Fused_bn_train_forward_%s_%dx%dx%dx%d" % (_SHORT[dtype], n, c, h, w))
+    x = b.input([n, c, h, w], dtype)
+    gamma = b.input([1, c, 1, 1], "float32")
+    beta = b.input([1, c, 1, 1], "float32")
+    xf = b.cast(x, "float32") if dtype != "float32" else x
+    inv = b.const(1.0 / (n * h * w), "float32")
+    mean = b.mul(b.reduce("ReduceSum", xf, [0, 2, 3], True), inv)
+    xc = b.sub(xf, mean)
+    var = b.mul(b.reduce("ReduceSum", b.mul(xc, xc), [0, 2, 3], True), inv)
+    y = b.add(b.mul(b.mul(xc, b.unary("Rsqrt", b.add(var, b.const(eps, "float32")))), gamma), beta)
+    return b.dumps([b.cast(y, dtype) if dtype != "float32" else y, mean, var])
+
+
+def layernorm_over_axis1(outer, width, inner, dtype="bfloat16", eps=1e-5, name=None):
+    """LayerNorm over the middle axis of [outer, width, inner] (channels-first activations) with gamma / beta
+    [width, 1]."""
+    b = DescBuilder(name or "Fused_LayerNorm_axis1_%s_%dx%dx%d" % (_SHORT[dtype], outer, width, inner))
+    x = b.input([outer, width, inner], dtype)
+    gamma = b.input([width, 1], dtype)
+    beta = b.input([width, 1], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    xf = f(x)
+    inv = b.const(1.0 / width, "float32")
+    mean = b.mul(b.reduce("ReduceSum", xf, [1], True), inv)
+    xc = b.sub(xf, mean)
+    var = b.mul(b.reduce("ReduceSum", b.mul(xc, xc), [1], True), inv)
+    y = b.add(b.mul(b.mul(xc, b.unary("Rsqrt", b.add(var, b.const(eps, "float32")))), f(gamma)), f(beta))
+    return b.dumps([b.cast(y, dtype) if dtype != "float32" else y])
+
+
 def layernorm_residual(rows, cols, dtype="bfloat16", eps=1e-5, name=None):
     """out = LayerNorm(x) * gamma + beta + r over the last axis, float32 internals."""
     b = DescBuilder(name or "Fused_LayerNorm_Residual_%s_%dx%d" % (

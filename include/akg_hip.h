@@ -57,7 +57,9 @@ typedef struct akg_hip_tensor_desc {
 
 typedef struct akg_hip_kernel_info {
   char kernel_name[256];              /* "<op>_kernel" (KernelOutliningExt.cpp:433) */
-  char family[32];                    /* "elementwise" | "row_reduce" | "stream_reduce" | "gemm_epilogue" | "indexed" | "segment_sum" */
+  char family[32];                    /* "elementwise" | "row_reduce" | "stream_reduce" | "gemm_epilogue" | "indexed" | "segment_sum" |
+                                         "staged" (a sequence of kernels of the other families; kernel_name, grid and
+                                         block are those of the last one) */
   char operator_type[32];             /* fusion class, OperatorIdentify.cpp:51-93 */
   uint32_t grid[3];                   /* blockIdx.x/y/z extents, as written to <k>.json (of the kernel proper when
                                          earlier launches precede it: segment sums over many positions) */

@@ -18,8 +18,9 @@ pytestmark = pytest.mark.gpu
 FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "akg_amd", "fixtures")
 STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all", "bnstats")
 ALL_SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
-SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS) and "segment_sum" not in n]
-STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS) and "bnstats_update" not in n]
+STAGED = [n for n in ALL_SMALL if "_staged_" in n]
+SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS) and "segment_sum" not in n and n not in STAGED]
+STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS) and "bnstats_update" not in n and n not in STAGED]
 FULL = ["c1_ew_tanh_add_mul_f32_1024x4096.info", "c2_softmax_f16_8192x4096.info",
         "c3_layernorm_residual_bf16_16384x4096.info", "c4_quant_int8_residual_bf16_32768x8192.info"]
 
@@ -94,6 +95,34 @@ def check_stream_reduction(path, seed, repeats=1, family="stream_reduce"):
                 ok, msg = harness.compare(g, e, d.dtype)
             print("  launch %d %s %s: %s" % (rep, d.name, d.dtype, msg), flush=True)
             assert ok, "%s output %s: %s" % (os.path.basename(path), d.name, msg)
+
+
+@pytest.mark.parametrize("name", STAGED)
+def test_descriptions_cut_into_several_kernels_match_the_oracle(name):
+    """A softmax or a normalisation over an outer axis, batch-norm statistics and their use in one description: no
+    single kernel serves them, so the handle runs one kernel per reduction level (temporaries in its workspace).
+    float32 results against the float64 evaluation (the sums are reassociated), 16-bit ones against the serial
+    oracle; three launches of one handle."""
+    from oracle import np_ref
+    path = os.path.join(FIXTURES, name)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    assert kernel.family == "staged" and kernel.source.count("extern \"C\" __global__") >= 3
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 730)
+    serial = cpu_ref.CpuKernel(path)(inputs)
+    wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+    exact = np_ref.evaluate(harness.widen_to_float64(desc), wide)
+    in_numel = max(int(np.prod(e[0].get("shape", [1]))) for e in desc["input_desc"])
+    terms = max(1, in_numel // min(int(np.prod(d.shape)) for d in kernel.outputs))
+    for launch in range(3):
+        got = run_on_gpu(kernel, inputs)
+        for d, g, e, x in zip(kernel.outputs, got, serial, exact):
+            if d.dtype == "float32":
+                ok, msg = harness.compare_reassociated(g, x, d.dtype, max(terms, 64))
+            else:
+                ok, msg = harness.compare(g, e, d.dtype)
+            print("  launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
+            assert ok, "%s output %s: %s" % (name, d.name, msg)
 
 
 @pytest.mark.parametrize("name", STREAM)

@@ -147,13 +147,18 @@ def test_error_conventions():
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(_desc(lambda d: d["op_desc"][0]["input_desc"][0][0].update(tensor_name="nowhere")), out_dir=None)
     assert e.value.code == -3 and "nowhere" in str(e.value)
-    # softmax along the outer axis: valid description, but the column kernel would need a second pass over the data
+    # a reduced value that meets an unreduced one along an outer axis needs a second pass: such a description runs as
+    # several kernels, unless it also holds an op that is not cut (an Assign), and then both reasons are given
     b = op_desc.DescBuilder("Fused_ReduceMax_Sub_axis0")
     x = b.input([64, 128], "float32")
     text = b.dumps([b.sub(x, b.reduce("ReduceMax", x, [0], True))])
+    assert driver.HipKernel(text, out_dir=None).family == "staged"
+    b = op_desc.DescBuilder("Fused_ReduceMax_Sub_Assign_axis0")
+    x = b.input([64, 128], "float32")
+    text = b.dumps([b.op("Assign", [x, b.sub(x, b.reduce("ReduceMax", x, [0], True))], [64, 128], "float32")])
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(text, out_dir=None)
-    assert e.value.code == -4 and "second pass" in str(e.value)
+    assert e.value.code == -4 and "second pass" in str(e.value) and "Assign is not cut into stages" in str(e.value)
     # path with '..' is refused (checkAndReadJson)
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel.from_file(os.path.join(FIXTURES, "..", "fixtures", "small_softmax_f32_5x77.info"), out_dir=None)
@@ -560,6 +565,36 @@ def test_hip_driver_mirrors_the_reference_driver_interface(tmp_path):
     assert [t.dtype for t in k.tensors] == ["float32", "float32"]
     with pytest.raises(ValueError):
         driver.HipDriver(input_file=info, backend="cuda")
+
+
+def test_description_no_single_kernel_serves_is_cut_at_its_reduction_results(tmp_path):
+    """Training batch norm in one description: mean (level 1), variance (level 2, it needs x - mean) and the normalised
+    tensor (level 2). The handle runs a kernel per reduction level plus one per output shape; every stage is a
+    description of its own made of the original op entries, compiled through the ordinary pipeline into artifacts of
+    its own; reduction results that are no outputs live in the handle's workspace."""
+    path = os.path.join(FIXTURES, "small_staged_bn_train_forward_f32_16x8x14x14.info")
+    k = driver.HipKernel.from_file(path, out_dir=str(tmp_path))
+    name = "small_staged_bn_train_forward_f32_16x8x14x14"
+    meta = json.load(open(os.path.join(str(tmp_path), name + ".json")))
+    assert k.family == "staged" and meta["family"] == "staged"
+    stages = meta["stages"]
+    assert [s["kernelName"] for s in stages] == ["%s_stage%d_kernel" % (name, i) for i in range(5)]
+    assert meta["kernelName"] == stages[-1]["kernelName"] == k.kernel_name
+    # two temporaries (the raw sums, [1,8,1,1] float32 each, 256-byte slots); stage 0 reads x and writes the first sum
+    assert k.workspace_bytes == 512
+    assert stages[0]["args"] == [{"input": 0}, {"workspace_offset": 0}]
+    assert stages[1]["args"] == [{"input": 0}, {"workspace_offset": 0}, {"workspace_offset": 256}]
+    written = sorted(a["output"] for s in stages for a in s["args"][-1:] if "output" in a)
+    assert written == [0, 1, 2]
+    for i in range(5):
+        stage_meta = json.load(open(os.path.join(str(tmp_path), "%s_stage%d.json" % (name, i))))
+        assert stage_meta["family"] in ("stream_reduce", "elementwise")
+        assert os.path.exists(os.path.join(str(tmp_path), "%s_stage%d.hsaco" % (name, i)))
+    assert not os.path.exists(os.path.join(str(tmp_path), name + ".hsaco"))      # the handle itself has no code object
+    assert k.source.count('extern "C" __global__') == 5
+    # the last axis needs no cut: one row kernel
+    one = driver.HipKernel(op_desc.softmax_over_axis([32, 12, 24, 40], 3, "float32", "sm_last"), out_dir=None)
+    assert one.family == "row_reduce"
 
 
 def test_skinny_matmul_gets_the_streaming_kernel():
