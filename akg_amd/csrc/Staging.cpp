@@ -78,17 +78,21 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
   plan->stages.clear();
   plan->tempBytes.clear();
   const json::Value doc = json::Value::parse(jsonText);
-  if (!doc.contains("op_desc") || doc.at("op_desc").size() != g.ops.size()) {
-    *why = "its op entries do not map one to one onto the translated ops";
+  if (!doc.contains("op_desc")) {
+    *why = "it has no op entries";
     return false;
   }
+  // the op entry behind every translated op, by the name of its result (the translator may have dropped unused entries)
   const json::Value &opDesc = doc.at("op_desc");
+  std::map<std::string, size_t> entryOf;
+  for (size_t i = 0; i < opDesc.size(); ++i) {
+    if (!opDesc[i].contains("output_desc") || opDesc[i].at("output_desc").size() != 1) continue;
+    const json::Value &out = opDesc[i].at("output_desc")[0];
+    if (out.contains("tensor_name")) entryOf[out.at("tensor_name").asString()] = i;
+  }
+  std::vector<size_t> entry(g.ops.size(), 0);
   for (size_t i = 0; i < g.ops.size(); ++i) {
     const OpNode &op = g.ops[i];
-    if (!opDesc[i].contains("name") || opDesc[i].at("name").asString() != op.name) {
-      *why = "its op entries do not map one to one onto the translated ops";
-      return false;
-    }
     if (op.kind == OpKind::Assign || op.kind == OpKind::MatMul || op.kind == OpKind::SegmentSum ||
         op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported) {
       *why = "op " + op.name + " is not cut into stages";
@@ -98,6 +102,12 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
       *why = "op " + op.name + " has several results";
       return false;
     }
+    const auto it = entryOf.find(g.tensor(op.outputs[0]).name);
+    if (it == entryOf.end() || !opDesc[it->second].contains("name") || opDesc[it->second].at("name").asString() != op.name) {
+      *why = "its op entries do not map one to one onto the translated ops";
+      return false;
+    }
+    entry[i] = it->second;
   }
   {
     std::set<int> distinct(g.outputs.begin(), g.outputs.end());
@@ -206,7 +216,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
     first = true;
     for (size_t i = 0; i < g.ops.size(); ++i) {
       if (!opUsed[i]) continue;
-      o << (first ? "" : ", ") << dump(opDesc[i]);
+      o << (first ? "" : ", ") << dump(opDesc[entry[i]]);
       first = false;
     }
     o << "], \"output_desc\": [";

@@ -168,8 +168,9 @@ def random_description(seed, allow_views=True, allow_reduce=True):
             axis = sorted(int(a) for a in rng.choice(r, size=int(rng.integers(2, r + 1)), replace=False))
         name = str(rng.choice(["ReduceSum", "ReduceMax", "ReduceMin"]))
         notes.append("%s%s" % (name, axis))
-        if rng.random() < 0.4 and axis == [len(out.t.shape) - 1]:
-            # use the reduced value again on the row it came from (softmax-like): only the row kernel can serve that
+        if rng.random() < 0.4 and (axis == [len(out.t.shape) - 1] or name != "ReduceSum"):
+            # use the reduced value again on the elements it came from (softmax-like): the row kernel serves the last
+            # axis, other axes need a kernel per pass (max / min only there: they do not depend on the order)
             outs = [b.sub(out.t, b.reduce(name, out.t, axis, True))]
             notes.append("Sub-after-reduce")
         else:

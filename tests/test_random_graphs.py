@@ -43,7 +43,7 @@ def test_random_description_compiles_and_oracles_agree(seed, tmp_path):
     text, notes = random_description(seed)
     desc, path = _write(tmp_path, text)
     kernel = driver.HipKernel(text, out_dir=None)
-    assert kernel.family in ("elementwise", "row_reduce", "stream_reduce", "indexed"), notes
+    assert kernel.family in ("elementwise", "row_reduce", "stream_reduce", "indexed", "staged"), notes
     inputs = harness.make_inputs(desc, seed=seed)
     c_out = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
     n_out = np_ref.evaluate(desc, inputs)
