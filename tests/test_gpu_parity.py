@@ -123,6 +123,11 @@ def test_descriptions_cut_into_several_kernels_match_the_oracle(name):
                 ok, msg = harness.compare(g, e, d.dtype)
             print("  launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
             assert ok, "%s output %s: %s" % (name, d.name, msg)
+    # the reference-style call on host buffers and the timing call go through the same sequence of kernels
+    host_outs = kernel.empty_outputs()
+    kernel.run_host([np.ascontiguousarray(a) for a in inputs] + host_outs)
+    for g, h in zip(got, host_outs):
+        assert np.array_equal(np.ascontiguousarray(g).view(np.uint8), h.view(np.uint8))
 
 
 @pytest.mark.parametrize("name", STREAM)
