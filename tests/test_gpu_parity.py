@@ -320,13 +320,14 @@ def test_gemm_family_on_ragged_shapes_with_and_without_split_k(case, tmp_path):
 def test_launches_can_be_captured_in_a_hip_graph_and_replayed():
     """After `prepare` a launch allocates nothing and records no memset, so a serving loop can capture a chain of
     kernels once and replay it: a softmax, a column reduction (workspace + arrival counters), a split-K GEMM
-    (workspace) and a grouped segment sum (five launches over one workspace) are captured in one graph and replayed four times on fresh inputs, with eager work and
+    (workspace), a grouped segment sum (five launches over one workspace) and a softmax over an outer axis (three
+    kernels with temporaries between them) are captured in one graph and replayed four times on fresh inputs, with eager work and
     synchronisations in between; every replay must equal the eager launches bit for bit (the counters and partials
     of one replay must be ready for the next)."""
     import torch
     dev = torch.device("cuda:0")
     names = ["small_softmax_f16_64x4096", "small_biasgrad_bf16_2048x1024", "small_gemm_bf16_bias_gelu_100x2048x520",
-             "small_segment_sum_f16_150001_by_4_seg300"]
+             "small_segment_sum_f16_150001_by_4_seg300", "small_staged_softmax_f32_32x12x24x40_axis1"]
     kernels, descs = [], []
     for n in names:
         path = os.path.join(FIXTURES, n + ".info")
