@@ -312,7 +312,7 @@ void destroyKernel(akg_hip_kernel *kernel);
 
 // The description as a sequence of kernels. `k` holds the translated graph; `reason` is why no single kernel serves it.
 int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k, const char *outDir,
-                  akg_hip_kernel_t **outKernel, const std::string &reason) {
+                  akg_hip_kernel_t **outKernel, const std::string &reason, bool dynamic, const std::string &artifactSuffix) {
   const std::string refusal = std::string("kernel ") + k->graph.name + ": " + reason;
   akg::StagingPlan plan;
   std::string why;
@@ -328,7 +328,13 @@ int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k
   note << "staged: " << plan.stages.size() << " kernels";
   for (const akg::StagePlan &sp : plan.stages) {
     akg_hip_kernel_t *stage = nullptr;
-    const int rc = doCompile(sp.jsonText, outDir, &stage, nullptr, false);
+    // a stage of a dynamic description is specialised to the shapes its tensors have in the bound graph (its op
+    // entries still carry the open dimensions)
+    akg::ShapeBinding stageBinding;
+    if (dynamic) {
+      stageBinding.inputShapes.assign(sp.shapes.begin(), sp.shapes.end() - static_cast<long>(sp.numOutputs));
+    }
+    const int rc = doCompile(sp.jsonText, outDir, &stage, dynamic ? &stageBinding : nullptr, false);
     if (rc != AKG_HIP_OK) {
       const std::string inner = g_lastError;
       for (auto &st : k->stages) destroyKernel(st.kernel);
@@ -356,6 +362,7 @@ int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k
     offset += (bytes + 255) / 256 * 256;
   }
   const akg_hip_kernel *last = k->stages.back().kernel;
+  k->graph.name += artifactSuffix;
   k->lowered = akg::LoweredKernel();
   k->lowered.kernelName = last->lowered.kernelName;
   k->lowered.family = akg::KernelFamily::Staged;
@@ -419,8 +426,8 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
     // the kernel keeps the description's name (shape sets may share its code object); the artifacts are per shape set
     k->graph.name += artifactSuffix;
   } catch (const akg::LoweringError &e) {
-    if (binding == nullptr && allowStages) {
-      return compileStaged(jsonText, std::move(k), outDir, outKernel, e.what());
+    if (allowStages) {
+      return compileStaged(jsonText, std::move(k), outDir, outKernel, e.what(), binding != nullptr, artifactSuffix);
     }
     return fail(AKG_HIP_ERR_UNSUPPORTED, std::string("kernel ") + k->graph.name + ": " + e.what());
   }

@@ -198,6 +198,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
       a.kind = StageArg::Kind::Input;
       a.index = idx;
       sp.args.push_back(a);
+      sp.shapes.push_back(g.tensor(g.inputs[static_cast<size_t>(idx)]).shape);
     }
     for (int t : cutInputs) {
       o << (first ? "" : ", ") << "[" << tensorEntry(g.tensor(t)) << "]";
@@ -211,6 +212,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
         a.index = tempOf.at(t);
       }
       sp.args.push_back(a);
+      sp.shapes.push_back(g.tensor(t).shape);
     }
     o << "], \"op_desc\": [";
     first = true;
@@ -233,6 +235,8 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
         a.index = tempOf.at(t);
       }
       sp.args.push_back(a);
+      sp.shapes.push_back(g.tensor(t).shape);
+      ++sp.numOutputs;
     }
     o << "]}";
     sp.jsonText = o.str();

@@ -33,6 +33,8 @@ struct StageArg {
 struct StagePlan {
   std::string jsonText;        // the stage as a description of its own, named "<op>_stage<k>"
   std::vector<StageArg> args;  // where each tensor of its signature lives (its inputs, then its outputs)
+  std::vector<std::vector<int64_t>> shapes;  // shape of each of them in the translated graph
+  size_t numOutputs = 0;
 };
 
 struct StagingPlan {

@@ -130,6 +130,38 @@ def test_descriptions_cut_into_several_kernels_match_the_oracle(name):
         assert np.array_equal(np.ascontiguousarray(g).view(np.uint8), h.view(np.uint8))
 
 
+def test_dynamic_description_that_needs_several_kernels(tmp_path):
+    """A softmax over axis 1 with an open leading dimension: every shape set is specialised into its own sequence of
+    kernels (stage artifacts carry the shape digest); results against the oracle of the same description written with
+    the bound shape."""
+    text = op_desc.softmax_over_axis([32, 12, 24, 40], 1, "float32", "dyn_softmax_axis1")
+    d = json_loads(text)
+
+    def open_leading(e):
+        if isinstance(e, dict):
+            if e.get("shape") and e["shape"][0] == 32:
+                e["shape"][0] = -1
+            for v in e.values():
+                open_leading(v)
+        elif isinstance(e, list):
+            for v in e:
+                open_leading(v)
+    open_leading(d)
+    dyn = driver.HipDynamicKernel(__import__("json").dumps(d), out_dir=str(tmp_path))
+    for lead in (32, 7, 32):
+        kernel = dyn.specialize([[lead, 12, 24, 40]])
+        assert kernel.family == "staged" and [t.shape for t in kernel.tensors] == [[lead, 12, 24, 40]] * 2
+        static = op_desc.softmax_over_axis([lead, 12, 24, 40], 1, "float32", "static_softmax_axis1_%d" % lead)
+        path = os.path.join(str(tmp_path), "static_%d.info" % lead)
+        open(path, "w").write(static)
+        inputs = harness.make_inputs(json_loads(static), seed=harness.BASE_SEED + 740 + lead)
+        got = run_on_gpu(kernel, inputs)
+        expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+        ok, msg = harness.compare(got[0], expect[0], "float32")
+        assert ok, "leading dimension %d: %s" % (lead, msg)
+    assert len([f for f in os.listdir(str(tmp_path)) if f.startswith("dyn_softmax_axis1_stage0_s") and f.endswith(".hsaco")]) == 2
+
+
 @pytest.mark.parametrize("name", STREAM)
 def test_streaming_reduction_matches_oracle(name):
     check_stream_reduction(os.path.join(FIXTURES, name), seed=harness.BASE_SEED + 400, repeats=3)
