@@ -528,8 +528,8 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
   constexpr int EB = Mma::kElemBytes;
   constexpr long K = KE * EB;   // bytes of K per row of A
   constexpr long NB = N * EB;   // bytes per k-row of a row-major B
-  static_assert(M >= 1 && M <= 64, "at most 64 rows");
-  constexpr int kRowTiles = M > 32 ? 2 : 1;   // MFMA tiles of 32 rows
+  static_assert(M >= 1 && M <= 128, "at most 128 rows");
+  constexpr int kRowTiles = static_cast<int>((M + 31) / 32);   // MFMA tiles of 32 rows
   static_assert(K % 32 == 0, "K must be a multiple of 32 bytes");
   static_assert(TRANSB || N % 4 == 0, "N must be a multiple of 4");
   constexpr long kSteps = K / 32;
