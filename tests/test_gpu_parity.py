@@ -544,6 +544,33 @@ def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero(sc
     assert np.array_equal(got[0], expect[0]) and not got[0][17].any() and got[0].any()
 
 
+@pytest.mark.parametrize("pattern", ["one_segment", "sorted", "runs_of_64", "mostly_outside"])
+def test_grouped_segment_sum_on_skewed_ids(pattern):
+    """The grouped schedule where the ids are far from uniform: every position in one segment (every lane of a tile
+    ranks behind its neighbours, one chain of 300000 additions), ids already sorted (a run touches few segments), whole
+    tiles of equal ids, and nine ids in ten outside [0, segments). Bit-exact against the serial loop."""
+    path = os.path.join(FIXTURES, "small_segment_sum_f32_300000_by_3_seg5000.info")
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    assert "grouped by segment" in kernel.source
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 760)
+    ids = inputs[1]
+    rng = np.random.default_rng(harness.BASE_SEED + 761)
+    if pattern == "one_segment":
+        ids[...] = 4999
+    elif pattern == "sorted":
+        ids[...] = np.sort(ids.reshape(-1)).reshape(ids.shape)
+    elif pattern == "runs_of_64":
+        ids[...] = np.repeat(rng.integers(0, 5000, size=(ids.size + 63) // 64), 64)[:ids.size].reshape(ids.shape)
+    else:
+        outside = rng.random(ids.shape) < 0.9
+        ids[outside] = rng.choice(np.array([-1, -70000, 5000, 2 ** 31 - 1], dtype=ids.dtype), size=int(outside.sum()))
+    expect = cpu_ref.CpuKernel(path)(inputs)
+    for launch in range(2):
+        got = run_on_gpu(kernel, inputs)
+        assert np.array_equal(got[0].view(np.uint8), expect[0].view(np.uint8)), "%s launch %d" % (pattern, launch)
+
+
 # Shapes the dynamic descriptions of the reference's test tree are specialised to (input_desc order).
 REF_DYNAMIC_SHAPES = {
     "Fused_Cast_Sub_Mul_split_14802837530264465372": [[[32, 1, 48, 48]], [[32, 1, 5, 1000]]],
