@@ -15,6 +15,7 @@ from oracle import cpu_ref
 
 pytestmark = pytest.mark.gpu
 
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "akg_amd", "fixtures")
 STREAM_MARKS = ("reducey", "reduceall", "reducex_long", "biasgrad", "sub_exp_reducesum", "mean_absmax_all", "bnstats")
 ALL_SMALL = sorted(os.path.basename(p) for p in glob.glob(os.path.join(FIXTURES, "small_*.info")))
@@ -447,6 +448,29 @@ def test_handles_launched_from_several_threads_on_their_own_streams():
         for d, o, a in zip(k.outputs, outs, alone):
             got = o.cpu().numpy().view(driver.NP_HOST_DTYPE[d.dtype]).reshape(d.shape)
             assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(a).view(np.uint8)), k.kernel_name
+
+
+def test_cli_runs_a_description_on_the_gpu():
+    """`akg-hip run X.info`: seeded inputs, NaN-prefilled outputs, a call on host buffers and timed launches. Two runs
+    give the same checksums (one kernel, a sequence of kernels, and a kernel that must leave unnamed rows zero) and no NaN
+    is left in the outputs."""
+    import subprocess
+    tool = os.path.join(ROOT, "akg_amd", "akg-hip")
+    for fixture in ("small_softmax_f16_64x4096.info", "small_staged_softmax_f32_32x12x24x40_axis1.info",
+                    "small_segment_sum_f32_700x3_by_1x3_seg50.info"):
+        runs = []
+        for _ in range(2):
+            p = subprocess.run([tool, "run", os.path.join(FIXTURES, fixture), "-n", "5", "-r", "2"], capture_output=True,
+                               text=True, timeout=120)
+            assert p.returncode == 0, p.stderr
+            runs.append(p.stdout)
+        lines = [l for l in runs[0].splitlines() if l.startswith("output ")]
+        assert lines and lines == [l for l in runs[1].splitlines() if l.startswith("output ")]
+        assert all(l.split()[-1] in ("0", "-1") for l in lines), runs[0]
+        ms = float([l for l in runs[0].splitlines() if l.startswith("time")][0].split()[1])
+        assert 0.0 < ms < 50.0
+    p = subprocess.run([tool, "run", os.path.join(FIXTURES, "no_such.info")], capture_output=True, text=True, timeout=60)
+    assert p.returncode == 1 and "cannot read" in p.stderr
 
 
 @pytest.mark.parametrize("name", FULL)
