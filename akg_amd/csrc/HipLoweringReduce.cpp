@@ -276,6 +276,7 @@ class StreamReduceEmitter {
     invariant_.assign(g_.tensors.size(), false);
     for (int id : g_.inputs) {
       phase_[static_cast<size_t>(id)] = Phase::Pre;
+      if (!g_.tensor(id).used) continue;   // (an input nothing reads may have any shape)
       invariant_[static_cast<size_t>(id)] = !variesAlongReduced(g_.tensor(id));
     }
     for (const OpNode &op : g_.ops) {

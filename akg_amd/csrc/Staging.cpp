@@ -64,6 +64,23 @@ std::string dump(const json::Value &v) {
   return "null";
 }
 
+// Ops whose result is read through an index map: kept out of the kernels that reduce.
+bool isViewOp(OpKind k) {
+  switch (k) {
+    case OpKind::Transpose:
+    case OpKind::Tile:
+    case OpKind::Slice:
+    case OpKind::StridedSlice:
+    case OpKind::Pad:
+    case OpKind::Concat:
+    case OpKind::Gather:
+    case OpKind::Reshape:
+      return true;
+    default:
+      return false;
+  }
+}
+
 std::string tensorEntry(const TensorValue &t) {
   std::ostringstream o;
   o << "{\"data_type\": " << quote(dtypeName(t.dtype)) << ", \"format\": \"DefaultFormat\", \"shape\": [";
@@ -86,9 +103,11 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
   const json::Value &opDesc = doc.at("op_desc");
   std::map<std::string, size_t> entryOf;
   for (size_t i = 0; i < opDesc.size(); ++i) {
-    if (!opDesc[i].contains("output_desc") || opDesc[i].at("output_desc").size() != 1) continue;
-    const json::Value &out = opDesc[i].at("output_desc")[0];
-    if (out.contains("tensor_name")) entryOf[out.at("tensor_name").asString()] = i;
+    if (!opDesc[i].contains("output_desc")) continue;
+    for (size_t o = 0; o < opDesc[i].at("output_desc").size(); ++o) {   // (a Split entry has one result per piece)
+      const json::Value &out = opDesc[i].at("output_desc")[o];
+      if (out.contains("tensor_name")) entryOf[out.at("tensor_name").asString()] = i;
+    }
   }
   std::vector<size_t> entry(g.ops.size(), 0);
   for (size_t i = 0; i < g.ops.size(); ++i) {
@@ -103,7 +122,10 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
       return false;
     }
     const auto it = entryOf.find(g.tensor(op.outputs[0]).name);
-    if (it == entryOf.end() || !opDesc[it->second].contains("name") || opDesc[it->second].at("name").asString() != op.name) {
+    // (the translator turns a Split entry into one Slice per piece that is used)
+    const bool named = it != entryOf.end() && opDesc[it->second].contains("name");
+    const std::string entryName = named ? opDesc[it->second].at("name").asString() : std::string();
+    if (!named || (entryName != op.name && !(entryName == "Split" && op.kind == OpKind::Slice))) {
       *why = "its op entries do not map one to one onto the translated ops";
       return false;
     }
@@ -117,15 +139,16 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
     }
   }
   const size_t nt = g.tensors.size();
+  // `reduced`: the tensor is the result of a cut op (a reduction, or a data-movement op) and lives in memory
   std::vector<int> level(nt, 0);
   std::vector<bool> reduced(nt, false);
   for (const OpNode &op : g.ops) {
     int lv = 0;
     for (int in : op.inputs) lv = std::max(lv, level[static_cast<size_t>(in)]);
-    const bool isReduce = lowering::isReduceKind(op.kind);
+    const bool cut = lowering::isReduceKind(op.kind) || isViewOp(op.kind);
     for (int out : op.outputs) {
-      level[static_cast<size_t>(out)] = lv + (isReduce ? 1 : 0);
-      reduced[static_cast<size_t>(out)] = isReduce;
+      level[static_cast<size_t>(out)] = lv + (cut ? 1 : 0);
+      reduced[static_cast<size_t>(out)] = cut;
     }
   }
   // tensors some output of the description depends on
@@ -216,8 +239,9 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
     }
     o << "], \"op_desc\": [";
     first = true;
+    std::set<size_t> written;
     for (size_t i = 0; i < g.ops.size(); ++i) {
-      if (!opUsed[i]) continue;
+      if (!opUsed[i] || !written.insert(entry[i]).second) continue;
       o << (first ? "" : ", ") << dump(opDesc[entry[i]]);
       first = false;
     }
@@ -247,14 +271,19 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
     // the reductions over operands of level s, grouped by operand shape and axes (one reduction space per kernel)
     std::map<std::string, std::vector<int>> reduceGroups;
     for (const OpNode &op : g.ops) {
-      if (!lowering::isReduceKind(op.kind)) continue;
+      const bool isReduce = lowering::isReduceKind(op.kind);
+      if (!isReduce && !isViewOp(op.kind)) continue;
       const int out = op.outputs[0];
       if (!needed[static_cast<size_t>(out)] || level[static_cast<size_t>(out)] != s + 1) continue;
       std::ostringstream key;
-      for (int64_t d : g.tensor(op.inputs[0]).shape) key << d << "x";
-      key << "/";
-      for (int64_t a : op.axes) key << a << ",";
-      key << (op.keepDims ? "k" : "");
+      if (isReduce) {
+        for (int64_t d : g.tensor(op.inputs[0]).shape) key << d << "x";
+        key << "/";
+        for (int64_t a : op.axes) key << a << ",";
+        key << (op.keepDims ? "k" : "");
+      } else {
+        key << "view" << out;   // a kernel of its own per data-movement result
+      }
       reduceGroups[key.str()].push_back(out);
     }
     for (const auto &kv : reduceGroups) addKernel(kv.second, s);
@@ -274,7 +303,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
     for (const auto &kv : outputGroups) addKernel(kv.second, s);
   }
   if (plan->stages.size() < 2) {
-    *why = "it has no reduction result to cut at";
+    *why = "it has no reduction or data-movement result to cut at";
     return false;
   }
   return true;

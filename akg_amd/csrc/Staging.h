@@ -7,7 +7,9 @@
  * same way: at the results of its reductions.
  *
  * Every tensor gets a level: inputs 0, an elementwise result the greatest level of its operands, a reduction's result
- * one more than its operand. The kernels of level s compute the reductions whose operands have level s (from the
+ * one more than its operand; so does the result of a data-movement op (Transpose, Slice, Pad, Concat, Tile, Gather,
+ * Reshape), which no kernel that reduces takes in: it gets a kernel of its own (with the elementwise ops in front of
+ * it) and the reduction reads its result from memory. The kernels of level s compute the reductions whose operands have level s (from the
  * description's inputs and the reduction results of earlier levels, recomputing the elementwise ops in between) and
  * the description's outputs of level s. Reduction results that are not outputs of the description live in a temporary
  * buffer the handle owns. Each kernel is an ordinary description made of the original's op entries and goes through

@@ -157,7 +157,7 @@ def random_description(seed, allow_views=True, allow_reduce=True):
             notes.append(which)
     out = work[-1]
     outs = [out.t]
-    if allow_reduce and not used_view and rng.random() < 0.5 and len(out.t.shape) >= 1:
+    if allow_reduce and rng.random() < 0.5 and len(out.t.shape) >= 1:
         r = len(out.t.shape)
         pick_axes = rng.random()
         if pick_axes < 0.5:

@@ -368,11 +368,16 @@ def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(json.dumps(d), out_dir=None)
     assert e.value.code == -3
-    # a reduction next to a transpose has no single kernel yet: error -4, never a wrong result
+    # a reduction next to a transpose has no single kernel: the transpose gets a kernel of its own and the reduction
+    # reads its result from the handle's workspace; next to a MatMul it is error -4, never a wrong result
     b = op_desc.DescBuilder("Fused_Transpose_ReduceSum")
     x = b.input([4, 6], "float32")
+    k = driver.HipKernel(b.dumps([b.reduce("ReduceSum", op_desc.transpose(b, x, [1, 0]), [1], False)]), out_dir=None)
+    assert k.family == "staged" and k.workspace_bytes == 256 and k.source.count('extern "C" __global__') == 2
+    b = op_desc.DescBuilder("Fused_Transpose_MatMul")
+    x, w = b.input([64, 32], "bfloat16"), b.input([64, 128], "bfloat16")
     with pytest.raises(driver.AkgHipError) as e:
-        driver.HipKernel(b.dumps([b.reduce("ReduceSum", op_desc.transpose(b, x, [1, 0]), [1], False)]), out_dir=None)
+        driver.HipKernel(b.dumps([b.matmul(op_desc.transpose(b, x, [1, 0]), w, "float32")]), out_dir=None)
     assert e.value.code == -4
 
 

@@ -75,6 +75,13 @@ def test_random_description_matches_oracle_on_gpu(seed, tmp_path):
             # after a subtraction of nearly equal tanh / exp values two correct float32 evaluations differ by that much
             e64 = np.asarray(x, dtype=np.float64).reshape(e.shape)
             slack = 16.0 * np.abs(e.astype(np.float64) - e64)
+            if any(n in ("Exp", "Tanh", "Sqrt", "Rsqrt", "Reciprocal", "RealDiv") for n in notes):
+                # the device's exp / tanh (and its hardware square roots and reciprocals where relaxed) are good to
+                # an ulp or two of their own results, which here are of the inputs' order of magnitude (operands are
+                # clipped to [-6, 6] in front of exp / tanh); a subtraction of two such values keeps that absolute
+                # error however small its result is, and the oracle may happen to be exact at that element
+                scale = max([1.0] + [float(np.max(np.abs(a.astype(np.float64)))) for a in inputs if a.dtype.kind == "f" and a.size])
+                slack = slack + 2.0 * float(np.finfo(np.float32).eps) * scale
             bad = np.abs(g.astype(np.float64) - e.astype(np.float64)) > 1e-5 * np.abs(e) + 1e-8 + slack
             bad &= ~(np.isnan(g) & np.isnan(e))
             ok, msg = not bad.any(), "%d of %d elements outside rtol 1e-5 + conditioning slack" % (bad.sum(), bad.size)
