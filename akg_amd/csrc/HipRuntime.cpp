@@ -58,7 +58,7 @@ struct akg_hip_kernel {
     std::vector<akg::StageArg> args;
   };
   std::vector<Stage> stages;
-  std::vector<uint64_t> tempOffsets;
+  std::vector<uint64_t> tempBytes, tempOffsets;
 };
 
 // Code objects compiled in this process, by the digest of their source (identical sources arise when a dynamic
@@ -317,15 +317,18 @@ int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k
   akg::StagingPlan plan;
   std::string why;
   try {
-    if (!akg::planStages(jsonText, k->graph, &plan, &why)) {
+    // first only behind contractions and data-movement ops (the pieces are compiled with staging allowed again, so a
+    // piece that still needs it is cut at its reductions); if there is no such cut, at the reductions
+    if (!akg::planStages(jsonText, k->graph, false, &plan, &why) && !akg::planStages(jsonText, k->graph, true, &plan, &why)) {
       return fail(AKG_HIP_ERR_UNSUPPORTED, refusal + " (and it cannot run as several kernels: " + why + ")");
     }
   } catch (const std::exception &e) {
     return fail(AKG_HIP_ERR_UNSUPPORTED, refusal);
   }
+  k->tempBytes = plan.tempBytes;
   bool allHits = true;
   std::ostringstream source, note;
-  note << "staged: " << plan.stages.size() << " kernels";
+  note << "staged:";
   for (const akg::StagePlan &sp : plan.stages) {
     akg_hip_kernel_t *stage = nullptr;
     // a stage of a dynamic description is specialised to the shapes its tensors have in the bound graph (its op
@@ -334,30 +337,54 @@ int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k
     if (dynamic) {
       stageBinding.inputShapes.assign(sp.shapes.begin(), sp.shapes.end() - static_cast<long>(sp.numOutputs));
     }
-    const int rc = doCompile(sp.jsonText, outDir, &stage, dynamic ? &stageBinding : nullptr, false);
+    const int rc = doCompile(sp.jsonText, outDir, &stage, dynamic ? &stageBinding : nullptr, true);
     if (rc != AKG_HIP_OK) {
       const std::string inner = g_lastError;
       for (auto &st : k->stages) destroyKernel(st.kernel);
       k->stages.clear();
       return fail(AKG_HIP_ERR_UNSUPPORTED, refusal + " (and as several kernels: " + inner + ")");
     }
-    if (!stage->stages.empty()) {      // a stage must be one kernel
-      destroyKernel(stage);
-      for (auto &st : k->stages) destroyKernel(st.kernel);
-      k->stages.clear();
-      return fail(AKG_HIP_ERR_UNSUPPORTED, refusal);
-    }
-    akg_hip_kernel::Stage st;
-    st.kernel = stage;
-    st.args = sp.args;
-    k->stages.push_back(st);
     allHits = allHits && stage->cacheHit;
-    source << "// ---- " << stage->lowered.kernelName << "\n" << stage->lowered.source << "\n";
-    note << " | " << stage->lowered.kernelName << ": " << akg::kernelFamilyName(stage->lowered.family) << " grid="
-         << stage->lowered.grid[0] << " block=" << stage->lowered.block[0];
+    std::vector<akg_hip_kernel::Stage> pieces;
+    if (stage->stages.empty()) {
+      akg_hip_kernel::Stage st;
+      st.kernel = stage;
+      st.args = sp.args;
+      pieces.push_back(st);
+    } else {
+      // the piece needed stages of its own: they become stages of this handle, their tensors found through the piece's
+      // bindings and their temporaries appended to this handle's
+      const size_t pieceInputs = sp.args.size() - sp.numOutputs;
+      const int tempBase = static_cast<int>(k->tempBytes.size());
+      k->tempBytes.insert(k->tempBytes.end(), stage->tempBytes.begin(), stage->tempBytes.end());
+      for (auto &inner : stage->stages) {
+        akg_hip_kernel::Stage st;
+        st.kernel = inner.kernel;
+        for (const akg::StageArg &a : inner.args) {
+          akg::StageArg m = a;
+          if (a.kind == akg::StageArg::Kind::Input) {
+            m = sp.args[static_cast<size_t>(a.index)];
+          } else if (a.kind == akg::StageArg::Kind::Output) {
+            m = sp.args[pieceInputs + static_cast<size_t>(a.index)];
+          } else {
+            m.index = tempBase + a.index;
+          }
+          st.args.push_back(m);
+        }
+        pieces.push_back(st);
+      }
+      stage->stages.clear();   // ownership moved
+      destroyKernel(stage);
+    }
+    for (const auto &st : pieces) {
+      k->stages.push_back(st);
+      source << "// ---- " << st.kernel->lowered.kernelName << "\n" << st.kernel->lowered.source << "\n";
+      note << " | " << st.kernel->lowered.kernelName << ": " << akg::kernelFamilyName(st.kernel->lowered.family) << " grid="
+           << st.kernel->lowered.grid[0] << " block=" << st.kernel->lowered.block[0];
+    }
   }
   uint64_t offset = 0;
-  for (uint64_t bytes : plan.tempBytes) {
+  for (uint64_t bytes : k->tempBytes) {
     k->tempOffsets.push_back(offset);
     offset += (bytes + 255) / 256 * 256;
   }

@@ -91,7 +91,10 @@ std::string tensorEntry(const TensorValue &t) {
 
 }  // namespace
 
-bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan, std::string *why) {
+bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsToo, StagingPlan *plan, std::string *why) {
+  const auto isCut = [reductionsToo](OpKind k) {
+    return (reductionsToo && lowering::isReduceKind(k)) || isViewOp(k) || k == OpKind::MatMul;
+  };
   plan->stages.clear();
   plan->tempBytes.clear();
   const json::Value doc = json::Value::parse(jsonText);
@@ -112,8 +115,8 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
   std::vector<size_t> entry(g.ops.size(), 0);
   for (size_t i = 0; i < g.ops.size(); ++i) {
     const OpNode &op = g.ops[i];
-    if (op.kind == OpKind::Assign || op.kind == OpKind::MatMul || op.kind == OpKind::SegmentSum ||
-        op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported) {
+    if (op.kind == OpKind::Assign || op.kind == OpKind::SegmentSum || op.kind == OpKind::Unknown ||
+        op.kind == OpKind::Unsupported) {
       *why = "op " + op.name + " is not cut into stages";
       return false;
     }
@@ -145,7 +148,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
   for (const OpNode &op : g.ops) {
     int lv = 0;
     for (int in : op.inputs) lv = std::max(lv, level[static_cast<size_t>(in)]);
-    const bool cut = lowering::isReduceKind(op.kind) || isViewOp(op.kind);
+    const bool cut = isCut(op.kind);
     for (int out : op.outputs) {
       level[static_cast<size_t>(out)] = lv + (cut ? 1 : 0);
       reduced[static_cast<size_t>(out)] = cut;
@@ -168,6 +171,11 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
   }
   int maxLevel = 0;
   for (int t : g.outputs) maxLevel = std::max(maxLevel, level[static_cast<size_t>(t)]);
+  if (maxLevel == 0) {   // (outputs of different shapes alone are no reason for several kernels)
+    *why = reductionsToo ? "it has no reduction, contraction or data-movement result to cut at"
+                         : "it has no contraction or data-movement result to cut at";
+    return false;
+  }
 
   // where the reduction results live
   std::map<int, int> tempOf;
@@ -272,7 +280,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
     std::map<std::string, std::vector<int>> reduceGroups;
     for (const OpNode &op : g.ops) {
       const bool isReduce = lowering::isReduceKind(op.kind);
-      if (!isReduce && !isViewOp(op.kind)) continue;
+      if (!isCut(op.kind)) continue;
       const int out = op.outputs[0];
       if (!needed[static_cast<size_t>(out)] || level[static_cast<size_t>(out)] != s + 1) continue;
       std::ostringstream key;
@@ -282,7 +290,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, StagingPlan *plan
         for (int64_t a : op.axes) key << a << ",";
         key << (op.keepDims ? "k" : "");
       } else {
-        key << "view" << out;   // a kernel of its own per data-movement result
+        key << "own" << out;   // a kernel of its own per data-movement result and per contraction
       }
       reduceGroups[key.str()].push_back(out);
     }

@@ -531,6 +531,22 @@ def batch_matmul_scale_mask(batch, m, k, n, dtype="bfloat16", transpose_b=True, 
     return b.dumps([b.cast(s, dtype)])
 
 
+def attention_probabilities(batch, m, k, n, dtype="bfloat16", name=None):
+    """softmax((Q[b] @ K[b]^T) * scale + mask) over the last axis in one description: Q [batch,m,k], K [batch,n,k],
+    mask [batch,m,n] float32, probabilities in `dtype`."""
+    b = DescBuilder(name or "Fused_BatchMatMul_Mul_Add_softmax_%s_%dx%dx%dx%d" % (_SHORT[dtype], batch, m, k, n))
+    q = b.input([batch, m, k], dtype)
+    kk = b.input([batch, n, k], dtype)
+    mask = b.input([batch, m, n], "float32")
+    attrs = [{"data_type": "bool", "name": "transpose_a", "value": False},
+             {"data_type": "bool", "name": "transpose_b", "value": True}]
+    s = b.op("BatchMatMul", [q, kk], [batch, m, n], "float32", attrs=attrs)
+    s = b.add(b.mul(s, b.const(1.0 / (k ** 0.5), "float32")), mask)
+    e = b.unary("Exp", b.sub(s, b.reduce("ReduceMax", s, [2], True)))
+    p = b.div(e, b.reduce("ReduceSum", e, [2], True))
+    return b.dumps([b.cast(p, dtype)])
+
+
 def gather(b, data, indices, axis):
     shape = list(data.shape[:axis]) + list(indices.shape) + list(data.shape[axis + 1:])
     return b.op("Gather", [data, indices], shape, data.dtype,

@@ -108,7 +108,7 @@ def test_descriptions_cut_into_several_kernels_match_the_oracle(name):
     path = os.path.join(FIXTURES, name)
     desc = harness.load_desc(path)
     kernel = driver.HipKernel.from_file(path)
-    assert kernel.family == "staged" and kernel.source.count("extern \"C\" __global__") >= 3
+    assert kernel.family == "staged" and kernel.source.count("extern \"C\" __global__") >= 2
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 730)
     serial = cpu_ref.CpuKernel(path)(inputs)
     wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]

@@ -368,17 +368,16 @@ def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(json.dumps(d), out_dir=None)
     assert e.value.code == -3
-    # a reduction next to a transpose has no single kernel: the transpose gets a kernel of its own and the reduction
-    # reads its result from the handle's workspace; next to a MatMul it is error -4, never a wrong result
+    # a reduction or a MatMul next to a transpose has no single kernel: the transpose gets a kernel of its own and the
+    # other reads its result from the handle's workspace
     b = op_desc.DescBuilder("Fused_Transpose_ReduceSum")
     x = b.input([4, 6], "float32")
     k = driver.HipKernel(b.dumps([b.reduce("ReduceSum", op_desc.transpose(b, x, [1, 0]), [1], False)]), out_dir=None)
     assert k.family == "staged" and k.workspace_bytes == 256 and k.source.count('extern "C" __global__') == 2
     b = op_desc.DescBuilder("Fused_Transpose_MatMul")
     x, w = b.input([64, 32], "bfloat16"), b.input([64, 128], "bfloat16")
-    with pytest.raises(driver.AkgHipError) as e:
-        driver.HipKernel(b.dumps([b.matmul(op_desc.transpose(b, x, [1, 0]), w, "float32")]), out_dir=None)
-    assert e.value.code == -4
+    k = driver.HipKernel(b.dumps([b.matmul(op_desc.transpose(b, x, [1, 0]), w, "float32")]), out_dir=None)
+    assert k.family == "staged" and "gemm_skinny" in k.source and "stage0_kernel" in k.source
 
 
 def test_shape_sets_that_differ_in_the_leading_dimensions_share_one_code_object(tmp_path):
@@ -600,6 +599,30 @@ def test_description_no_single_kernel_serves_is_cut_at_its_reduction_results(tmp
     # the last axis needs no cut: one row kernel
     one = driver.HipKernel(op_desc.softmax_over_axis([32, 12, 24, 40], 3, "float32", "sm_last"), out_dir=None)
     assert one.family == "row_reduce"
+
+
+def test_matmul_next_to_a_softmax_is_cut_behind_the_contraction(tmp_path):
+    """Attention probabilities in one description: the contraction (with nothing fused behind it) leaves the float32
+    scores in the workspace, and everything behind it, scale, mask and softmax, is ONE row kernel: the cut is made
+    behind contractions and data-movement ops first, and at reductions only where a piece still needs it."""
+    text = op_desc.attention_probabilities(4, 128, 64, 256, "bfloat16", "attn_probs")
+    k = driver.HipKernel(text, out_dir=str(tmp_path))
+    meta = json.load(open(os.path.join(str(tmp_path), "attn_probs.json")))
+    assert k.family == "staged" and [s["kernelName"] for s in meta["stages"]] == ["attn_probs_stage0_kernel", "attn_probs_stage1_kernel"]
+    assert k.workspace_bytes == 4 * 128 * 256 * 4
+    fams = [json.load(open(os.path.join(str(tmp_path), "attn_probs_stage%d.json" % i)))["family"] for i in range(2)]
+    assert fams == ["gemm_epilogue", "row_reduce"]
+    assert meta["stages"][1]["args"] == [{"input": 2}, {"workspace_offset": 0}, {"output": 0}]
+    # a piece that needs cuts of its own: its stages are spliced in, temporaries appended
+    b = op_desc.DescBuilder("transpose_then_softmax_axis0")
+    x = b.input([64, 96], "float32")
+    t = op_desc.transpose(b, x, [1, 0])
+    e = b.unary("Exp", b.sub(t, b.reduce("ReduceMax", t, [0], True)))
+    k = driver.HipKernel(b.dumps([b.div(e, b.reduce("ReduceSum", e, [0], True))]), out_dir=str(tmp_path))
+    meta = json.load(open(os.path.join(str(tmp_path), "transpose_then_softmax_axis0.json")))
+    assert [s["kernelName"] for s in meta["stages"]] == ["transpose_then_softmax_axis0_stage0_kernel"] + [
+        "transpose_then_softmax_axis0_stage1_stage%d_kernel" % i for i in range(3)]
+    assert k.workspace_bytes == 96 * 64 * 4 + 256 + 256
 
 
 def test_skinny_matmul_gets_the_streaming_kernel():
