@@ -92,9 +92,7 @@ std::string tensorEntry(const TensorValue &t) {
 }  // namespace
 
 bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsToo, StagingPlan *plan, std::string *why) {
-  const auto isCut = [reductionsToo](OpKind k) {
-    return (reductionsToo && lowering::isReduceKind(k)) || isViewOp(k) || k == OpKind::MatMul;
-  };
+
   plan->stages.clear();
   plan->tempBytes.clear();
   const json::Value doc = json::Value::parse(jsonText);
@@ -143,12 +141,39 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
   }
   const size_t nt = g.tensors.size();
   // `reduced`: the tensor is the result of a cut op (a reduction, or a data-movement op) and lives in memory
+  // Which results are cut (live in memory): those of data-movement ops; of reductions when asked for; of a
+  // contraction when a reduction depends on it (otherwise the ops behind it are its epilogue, in the same kernel); and
+  // the operands of a contraction that are computed (the GEMM kernel reads its operands from memory).
+  std::vector<bool> cutResult(nt, false);
+  {
+    std::vector<bool> feedsReduction(nt, false);
+    for (size_t i = g.ops.size(); i-- > 0;) {
+      const OpNode &op = g.ops[i];
+      bool feeds = lowering::isReduceKind(op.kind);
+      for (int out : op.outputs) feeds = feeds || feedsReduction[static_cast<size_t>(out)];
+      if (feeds) {
+        for (int in : op.inputs) feedsReduction[static_cast<size_t>(in)] = true;
+      }
+    }
+    for (const OpNode &op : g.ops) {
+      const int out = op.outputs[0];
+      if (isViewOp(op.kind) || (reductionsToo && lowering::isReduceKind(op.kind)) ||
+          (op.kind == OpKind::MatMul && feedsReduction[static_cast<size_t>(out)])) {
+        cutResult[static_cast<size_t>(out)] = true;
+      }
+      if (op.kind == OpKind::MatMul) {
+        for (int in : op.inputs) {
+          if (g.tensor(in).producer >= 0) cutResult[static_cast<size_t>(in)] = true;
+        }
+      }
+    }
+  }
   std::vector<int> level(nt, 0);
   std::vector<bool> reduced(nt, false);
   for (const OpNode &op : g.ops) {
     int lv = 0;
     for (int in : op.inputs) lv = std::max(lv, level[static_cast<size_t>(in)]);
-    const bool cut = isCut(op.kind);
+    const bool cut = cutResult[static_cast<size_t>(op.outputs[0])];
     for (int out : op.outputs) {
       level[static_cast<size_t>(out)] = lv + (cut ? 1 : 0);
       reduced[static_cast<size_t>(out)] = cut;
@@ -280,11 +305,11 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
     std::map<std::string, std::vector<int>> reduceGroups;
     for (const OpNode &op : g.ops) {
       const bool isReduce = lowering::isReduceKind(op.kind);
-      if (!isCut(op.kind)) continue;
+      if (!cutResult[static_cast<size_t>(op.outputs[0])]) continue;
       const int out = op.outputs[0];
       if (!needed[static_cast<size_t>(out)] || level[static_cast<size_t>(out)] != s + 1) continue;
       std::ostringstream key;
-      if (isReduce) {
+      if (isReduce && reductionsToo) {
         for (int64_t d : g.tensor(op.inputs[0]).shape) key << d << "x";
         key << "/";
         for (int64_t a : op.axes) key << a << ",";

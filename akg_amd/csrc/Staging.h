@@ -9,8 +9,9 @@
  * Every tensor gets a level: inputs 0, an elementwise result the greatest level of its operands, a reduction's result
  * one more than its operand; so does the result of a data-movement op (Transpose, Slice, Pad, Concat, Tile, Gather,
  * Reshape), which no kernel that reduces takes in: it gets a kernel of its own (with the elementwise ops in front of
- * it) and the reduction reads its result from memory. A MatMul next to a reduction (attention scores and their softmax)
- * is cut the same way: the contraction leaves its result in memory, the ops behind it run in the next kernel. The kernels of level s compute the reductions whose operands have level s (from the
+ * it) and the reduction reads its result from memory. A MatMul that a reduction depends on (attention scores and their
+ * softmax) is cut the same way: the contraction leaves its result in memory, the ops behind it run in the next kernel;
+ * operands of a contraction that are computed in the description are cut too (the GEMM kernel reads memory). The kernels of level s compute the reductions whose operands have level s (from the
  * description's inputs and the reduction results of earlier levels, recomputing the elementwise ops in between) and
  * the description's outputs of level s. Reduction results that are not outputs of the description live in a temporary
  * buffer the handle owns. Each kernel is an ordinary description made of the original's op entries and goes through

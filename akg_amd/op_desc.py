@@ -547,6 +547,18 @@ def attention_probabilities(batch, m, k, n, dtype="bfloat16", name=None):
     return b.dumps([b.cast(p, dtype)])
 
 
+def transposed_a_matmul_bias_relu(m, k, n, dtype="bfloat16", name=None):
+    """relu(A^T @ B + bias) with A stored [k, m]: the reference's MatMul refuses transpose_a
+    (MindSporeToLinalg.cpp:1508-1510), so the description spells the transpose as an op of its own."""
+    b = DescBuilder(name or "Fused_Transpose_MatMul_Add_relu_%s_%dx%dx%d" % (_SHORT[dtype], m, k, n))
+    a = b.input([k, m], dtype)
+    w = b.input([k, n], dtype)
+    bias = b.input([n], dtype)
+    acc = b.matmul(transpose(b, a, [1, 0]), w, "float32")
+    y = b.maximum(b.add(acc, b.cast(bias, "float32")), b.const(0.0, "float32"))
+    return b.dumps([b.cast(y, dtype)])
+
+
 def gather(b, data, indices, axis):
     shape = list(data.shape[:axis]) + list(indices.shape) + list(data.shape[axis + 1:])
     return b.op("Gather", [data, indices], shape, data.dtype,
