@@ -113,8 +113,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
   std::vector<size_t> entry(g.ops.size(), 0);
   for (size_t i = 0; i < g.ops.size(); ++i) {
     const OpNode &op = g.ops[i];
-    if (op.kind == OpKind::Assign || op.kind == OpKind::SegmentSum || op.kind == OpKind::Unknown ||
-        op.kind == OpKind::Unsupported) {
+    if (op.kind == OpKind::SegmentSum || op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported) {
       *why = "op " + op.name + " is not cut into stages";
       return false;
     }
@@ -210,6 +209,9 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
     plan->tempBytes.push_back(static_cast<uint64_t>(g.tensors[t].numel()) * dtypeSize(g.tensors[t].dtype));
   }
 
+  // per kernel: the description inputs it reads and the Assign ops it holds (for the ordering check at the end)
+  std::vector<std::set<int>> kernelReads;
+  std::vector<std::vector<size_t>> kernelAssigns;
   // one kernel per target group
   auto addKernel = [&](const std::vector<int> &targets, int stage) {
     // ops on the way to the targets, cut at the description's inputs and at reduction results of earlier stages
@@ -298,6 +300,12 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
     o << "]}";
     sp.jsonText = o.str();
     plan->stages.push_back(sp);
+    kernelReads.push_back(graphInputs);
+    std::vector<size_t> assigns;
+    for (size_t i = 0; i < g.ops.size(); ++i) {
+      if (opUsed[i] && g.ops[i].kind == OpKind::Assign) assigns.push_back(i);
+    }
+    kernelAssigns.push_back(assigns);
   };
 
   for (int s = 0; s <= maxLevel; ++s) {
@@ -334,6 +342,29 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
       if (std::find(grp.begin(), grp.end(), t) == grp.end()) grp.push_back(t);
     }
     for (const auto &kv : outputGroups) addKernel(kv.second, s);
+  }
+  // Assign writes over an input of the description. The kernels recompute from the inputs, so the write must come after
+  // every other kernel's reads of that input, must happen once, and must not be lost.
+  for (size_t i = 0; i < g.ops.size(); ++i) {
+    if (g.ops[i].kind != OpKind::Assign) continue;
+    const int dst = g.tensor(g.ops[i].inputs[0]).inputIndex;
+    int holder = -1, holders = 0;
+    for (size_t kx = 0; kx < kernelAssigns.size(); ++kx) {
+      if (std::find(kernelAssigns[kx].begin(), kernelAssigns[kx].end(), i) != kernelAssigns[kx].end()) {
+        holder = static_cast<int>(kx);
+        ++holders;
+      }
+    }
+    if (holders != 1 || dst < 0) {
+      *why = holders == 0 ? "the result of an Assign is not among the outputs" : "an Assign would run in several kernels";
+      return false;
+    }
+    for (size_t kx = 0; kx < kernelReads.size(); ++kx) {
+      if (static_cast<int>(kx) > holder && kernelReads[kx].count(dst)) {
+        *why = "a kernel behind an Assign would read the input it overwrites";
+        return false;
+      }
+    }
   }
   if (plan->stages.size() < 2) {
     *why = "it has no reduction or data-movement result to cut at";

@@ -102,6 +102,8 @@ FIXTURES = {
     "small_staged_attention_probs_f16_3x40x64x136": lambda n: op_desc.attention_probabilities(3, 40, 64, 136, "float16", n),
     "small_staged_transposed_a_matmul_bf16_48x512x264": lambda n: op_desc.transposed_a_matmul_bias_relu(48, 512, 264, "bfloat16", n),
     "small_staged_transposed_a_matmul_f16_300x256x136": lambda n: op_desc.transposed_a_matmul_bias_relu(300, 256, 136, "float16", n),
+    "small_sgdclip_update_f32_300x130": lambda n: op_desc.sgd_clip_by_global_norm(300, 130, "float32", 0.01, 1.0, n),
+    "small_sgdclip_update_bf16_64x256": lambda n: op_desc.sgd_clip_by_global_norm(64, 256, "bfloat16", 0.01, 1.0, n),
     # many positions: grouped by segment first (short rows moved, wide rows through their positions)
     "small_segment_sum_f32_300000_by_3_seg5000": lambda n: op_desc.unsorted_segment_sum([300000], [3], 5000, "float32", "int32", n),
     "small_segment_sum_f16_150001_by_4_seg300": lambda n: op_desc.unsorted_segment_sum([150001], [4], 300, "float16", "int64", n),

@@ -547,6 +547,22 @@ def attention_probabilities(batch, m, k, n, dtype="bfloat16", name=None):
     return b.dumps([b.cast(p, dtype)])
 
 
+def sgd_clip_by_global_norm(rows, cols, dtype="float32", lr=0.01, clip=1.0, name=None):
+    """p <- p - lr * g * min(1, clip / ||g||): the norm is a reduction over the whole gradient, the update an Assign over
+    the parameter. Outputs: the assigned parameter and the norm."""
+    b = DescBuilder(name or "Fused_sgd_clip_global_norm_%s_%dx%d" % (_SHORT[dtype], rows, cols))
+    p = b.input([rows, cols], dtype)
+    g = b.input([rows, cols], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    gf = f(g)
+    norm = b.unary("Sqrt", b.reduce("ReduceSum", b.mul(gf, gf), [0, 1], True))
+    scale = b.minimum(b.div(b.const(clip, "float32"), b.add(norm, b.const(1e-6, "float32"))), b.const(1.0, "float32"))
+    new_p = b.sub(f(p), b.mul(b.mul(gf, scale), b.const(lr, "float32")))
+    new_p = b.cast(new_p, dtype) if dtype != "float32" else new_p
+    a = b.op("Assign", [p, new_p], [rows, cols], dtype)
+    return b.dumps([a, norm])
+
+
 def transposed_a_matmul_bias_relu(m, k, n, dtype="bfloat16", name=None):
     """relu(A^T @ B + bias) with A stored [k, m]: the reference's MatMul refuses transpose_a
     (MindSporeToLinalg.cpp:1508-1510), so the description spells the transpose as an op of its own."""
