@@ -186,3 +186,53 @@ def random_description(seed, allow_views=True, allow_reduce=True):
     for t in outs:
         final.append(b.cast(t, dtype) if dtype != "float32" and rng.random() < 0.7 else t)
     return b.dumps(final), notes
+
+
+def random_matmul_description(seed):
+    """A MatMul in the middle of a random description: an optional Cast or Transpose in front of its first operand,
+    bias and activation behind it, and optionally a softmax over the rows, column sums or a row maximum of the result,
+    so that the contraction's neighbours are sometimes its epilogue and sometimes kernels of their own. 16-bit results
+    (the accumulation order of the matrix units differs from the serial loop's). Returns (json_text, notes)."""
+    rng = np.random.default_rng(100000 + seed)
+    m = int(rng.choice([1, 7, 40, 64, 130]))
+    k = int(rng.choice([32, 64, 256]))
+    n = int(rng.choice([8, 136, 256]))
+    dtype = str(rng.choice(["bfloat16", "float16"]))
+    tb = bool(rng.integers(0, 2))
+    b = op_desc.DescBuilder("Fused_random_matmul_%d" % seed)
+    notes = ["%dx%dx%d" % (m, k, n), dtype]
+    front = str(rng.choice(["none", "cast", "transpose"]))
+    if front == "cast":
+        a = b.cast(b.input([m, k], "float32"), dtype)
+    elif front == "transpose":
+        a = op_desc.transpose(b, b.input([k, m], dtype), [1, 0])
+    else:
+        a = b.input([m, k], dtype)
+    notes.append("front-" + front)
+    w = b.input([n, k] if tb else [k, n], dtype)
+    acc = b.matmul(a, w, "float32", transpose_b=tb)
+    notes.append("tb" if tb else "nt")
+    y = acc
+    if rng.random() < 0.7:
+        y = b.add(y, b.cast(b.input([n], dtype), "float32"))
+        notes.append("bias")
+    act = str(rng.choice(["none", "relu", "tanh"]))
+    if act == "relu":
+        y = b.maximum(y, b.const(0.0, "float32"))
+    elif act == "tanh":
+        y = b.unary("Tanh", b.mul(y, b.const(0.125, "float32")))
+    notes.append(act)
+    outs = []
+    tail = str(rng.choice(["none", "none", "softmax", "colsum", "rowmax"]))
+    notes.append("tail-" + tail)
+    if tail == "softmax":
+        s = b.mul(y, b.const(1.0 / (k ** 0.5), "float32"))
+        e = b.unary("Exp", b.sub(s, b.reduce("ReduceMax", s, [1], True)))
+        outs.append(b.div(e, b.reduce("ReduceSum", e, [1], True)))
+    elif tail == "colsum":
+        outs += [y, b.mul(b.reduce("ReduceSum", y, [0], True), b.const(1.0 / m, "float32"))]
+    elif tail == "rowmax":
+        outs += [y, b.reduce("ReduceMax", y, [1], False)]
+    else:
+        outs.append(y)
+    return b.dumps([b.cast(t, dtype) for t in outs]), notes

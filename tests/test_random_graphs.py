@@ -11,7 +11,7 @@ import pytest
 
 from akg_amd import driver, harness
 from oracle import cpu_ref, np_ref
-from random_graphs import random_description
+from random_graphs import random_description, random_matmul_description
 
 # AKG_RANDOM_GRAPHS=N widens the sweep for a one-off soak on the CPU oracle / a GPU box
 SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_GRAPHS", "40"))))
@@ -87,5 +87,33 @@ def test_random_description_matches_oracle_on_gpu(seed, tmp_path):
             ok, msg = not bad.any(), "%d of %d elements outside rtol 1e-5 + conditioning slack" % (bad.sum(), bad.size)
         else:
             ok, msg = harness.compare(g, e, d.dtype)
+        print("  %s %s %s: %s" % (kernel.family, d.name, d.dtype, msg), flush=True)
+        assert ok, "seed %d (%s) output %s: %s" % (seed, " ".join(notes), d.name, msg)
+
+
+MATMUL_SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_MATMULS", "40"))))
+
+
+@pytest.mark.parametrize("seed", MATMUL_SEEDS[:12])
+def test_random_matmul_description_compiles(seed):
+    text, notes = random_matmul_description(seed)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family in ("gemm_epilogue", "staged"), notes
+    assert "gemm_" in kernel.source
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", MATMUL_SEEDS)
+def test_random_matmul_description_matches_oracle_on_gpu(seed, tmp_path):
+    from test_gpu_parity import run_on_gpu
+    text, notes = random_matmul_description(seed)
+    desc, path = _write(tmp_path, text)
+    print("seed %d: %s" % (seed, " ".join(notes)), flush=True)
+    kernel = driver.HipKernel(text, out_dir=None)
+    inputs = harness.make_inputs(desc, seed=seed)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    for d, g, e in zip(kernel.outputs, got, expect):
+        ok, msg = harness.compare(g, e, d.dtype)
         print("  %s %s %s: %s" % (kernel.family, d.name, d.dtype, msg), flush=True)
         assert ok, "seed %d (%s) output %s: %s" % (seed, " ".join(notes), d.name, msg)
