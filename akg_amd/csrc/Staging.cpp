@@ -113,7 +113,7 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
   std::vector<size_t> entry(g.ops.size(), 0);
   for (size_t i = 0; i < g.ops.size(); ++i) {
     const OpNode &op = g.ops[i];
-    if (op.kind == OpKind::SegmentSum || op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported) {
+    if (op.kind == OpKind::Unknown || op.kind == OpKind::Unsupported) {
       *why = "op " + op.name + " is not cut into stages";
       return false;
     }
@@ -140,7 +140,8 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
   }
   const size_t nt = g.tensors.size();
   // `reduced`: the tensor is the result of a cut op (a reduction, or a data-movement op) and lives in memory
-  // Which results are cut (live in memory): those of data-movement ops; of reductions when asked for; of a
+  // Which results are cut (live in memory): those of data-movement ops and of UnsortedSegmentSum (a kernel of its
+  // own); of reductions when asked for; of a
   // contraction when a reduction depends on it (otherwise the ops behind it are its epilogue, in the same kernel); and
   // the operands of a contraction that are computed (the GEMM kernel reads its operands from memory).
   std::vector<bool> cutResult(nt, false);
@@ -157,10 +158,10 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
     for (const OpNode &op : g.ops) {
       const int out = op.outputs[0];
       if (isViewOp(op.kind) || (reductionsToo && lowering::isReduceKind(op.kind)) ||
-          (op.kind == OpKind::MatMul && feedsReduction[static_cast<size_t>(out)])) {
+          (op.kind == OpKind::MatMul && feedsReduction[static_cast<size_t>(out)]) || op.kind == OpKind::SegmentSum) {
         cutResult[static_cast<size_t>(out)] = true;
       }
-      if (op.kind == OpKind::MatMul) {
+      if (op.kind == OpKind::MatMul || op.kind == OpKind::SegmentSum) {   // (their kernels read operands from memory)
         for (int in : op.inputs) {
           if (g.tensor(in).producer >= 0) cutResult[static_cast<size_t>(in)] = true;
         }

@@ -47,7 +47,7 @@ struct StagingPlan {
 };
 
 // False (with the reason in *why) when the description cannot be cut: fewer than two kernels would result, its op
-// entries do not match the translated graph one to one, it holds an UnsortedSegmentSum, or an Assign whose write could
+// entries do not match the translated graph one to one, or it holds an Assign whose write could
 // not be ordered behind every other kernel's reads of the input it overwrites.
 // `reductionsToo` false: cut only behind contractions and data-movement ops (what is left between two cuts may still be
 // one kernel: a softmax behind a MatMul); true: at reduction results as well.

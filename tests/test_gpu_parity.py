@@ -569,6 +569,26 @@ def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero(sc
     assert np.array_equal(got[0], expect[0]) and not got[0][17].any() and got[0].any()
 
 
+def test_segment_sum_with_neighbours_runs_as_stages_and_stays_bit_exact(tmp_path):
+    """out = -UnsortedSegmentSum(2 * data, ids): the scaling, the segment sum and the negation are three kernels; the
+    additions keep their serial order, so the result equals the oracle's bit for bit (scaling by two and negation are
+    exact)."""
+    b = op_desc.DescBuilder("Fused_Mul_UnsortedSegmentSum_Neg")
+    data, ids = b.input([70000, 3], "float32"), b.input([70000], "int32")
+    seg = b.op("UnsortedSegmentSum", [b.mul(data, b.const(2.0, "float32")), ids], [500, 3], "float32",
+               attrs=[{"data_type": "int", "name": "num_segments", "value": 500}])
+    text = b.dumps([b.unary("Neg", seg)])
+    path = os.path.join(str(tmp_path), "Fused_Mul_UnsortedSegmentSum_Neg.info")
+    open(path, "w").write(text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family == "staged" and "grouped by segment" in kernel.source
+    inputs = harness.make_inputs(json_loads(text), seed=harness.BASE_SEED + 780)
+    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    for launch in range(2):
+        got = run_on_gpu(kernel, inputs)
+        assert np.array_equal(got[0].view(np.uint8), expect[0].view(np.uint8)), "launch %d" % launch
+
+
 @pytest.mark.parametrize("pattern", ["one_segment", "sorted", "runs_of_64", "mostly_outside"])
 def test_grouped_segment_sum_on_skewed_ids(pattern):
     """The grouped schedule where the ids are far from uniform: every position in one segment (every lane of a tile
