@@ -104,19 +104,22 @@ int akg_hip_kernel_tensor(const akg_hip_kernel_t *kernel, int index, akg_hip_ten
 /** Launch shape, family, algorithmic work. Replaces get_gpu_setting_by_input (dynamic_utils.py:564-577). */
 int akg_hip_kernel_get_info(const akg_hip_kernel_t *kernel, akg_hip_kernel_info *info);
 
-/** Emitted HIP source of the kernel (NUL-terminated, owned by the handle). */
+/** Emitted HIP source of the kernel (NUL-terminated, owned by the handle); for a description that runs as several
+ *  kernels, their sources one after the other. */
 int akg_hip_kernel_source(const akg_hip_kernel_t *kernel, const char **source);
 
 /**
  * Load the code object on the current device and allocate the handle's workspace there (workspace_bytes of
- * kernel_info; zero for every family but the streaming reductions), so that later launches on this device
+ * kernel_info: partial results of streaming reductions and split-K GEMMs, the sorted positions of large segment
+ * sums, the tensors between the kernels of a staged description), so that later launches on this device
  * allocate nothing. Optional: the first akg_hip_launch on a device does the same. Replaces the cuModuleLoadData /
  * cuModuleGetFunction prologue of the generated shim (code_template.py:180-203).
  */
 int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel);
 
 /**
- * The hot call: enqueue the kernel on `stream` (a hipStream_t, NULL for the default stream) with one DEVICE
+ * The hot call: enqueue the kernel (or, for a description that needs several, its kernels in order) on `stream`
+ * (a hipStream_t, NULL for the default stream) with one DEVICE
  * pointer per argument, inputs then outputs. Asynchronous; after the first call on a device (or
  * akg_hip_kernel_prepare) it allocates nothing. Launches of one handle whose workspace_bytes is non-zero share
  * that workspace and must not overlap on the device. Replaces the cuLaunchKernel
