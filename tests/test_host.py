@@ -609,6 +609,23 @@ def test_description_no_single_kernel_serves_is_cut_at_its_reduction_results(tmp
     assert one.family == "row_reduce"
 
 
+def test_descriptions_that_cannot_be_cut_say_both_reasons():
+    """Staging refuses what it cannot order or name: an output listed twice (two kernels would write one buffer) keeps the
+    single-kernel refusal and adds its own reason; nothing crashes."""
+    b = op_desc.DescBuilder("twice_listed_outer_softmax")
+    x = b.input([64, 128], "float32")
+    y = b.sub(x, b.reduce("ReduceMax", x, [0], True))
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(b.dumps([y, y]), out_dir=None)
+    assert e.value.code == -4 and "second pass" in str(e.value) and "listed twice" in str(e.value)
+    # an op outside the op table is refused before any cut is tried
+    d = json.loads(op_desc.softmax_over_axis([8, 16], 0, "float32", "unknown_op_outer"))
+    d["op_desc"][1]["name"] = "Frobnicate"
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(json.dumps(d), out_dir=None)
+    assert e.value.code in (-3, -4) and "Frobnicate" in str(e.value)
+
+
 def test_matmul_next_to_a_softmax_is_cut_behind_the_contraction(tmp_path):
     """Attention probabilities in one description: the contraction (with nothing fused behind it) leaves the float32
     scores in the workspace, and everything behind it, scale, mask and softmax, is ONE row kernel: the cut is made
