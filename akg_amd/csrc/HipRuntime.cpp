@@ -29,6 +29,7 @@
 #include "Json.h"
 #include "OpGraph.h"
 #include "Sha256.h"
+#include "StaticScratch.h"
 
 // Text of the device-side headers, generated at build time from kernels/*.hpp.
 #include "KernelLibEmbed.inc"
@@ -603,12 +604,49 @@ const akg::TensorValue &tensorAt(const akg_hip_kernel *k, int index) {
   return k->graph.tensor(k->graph.outputs[static_cast<size_t>(index) - nin]);
 }
 
-int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream) {
+uint64_t alignScratch(uint64_t bytes) { return (bytes + 255) / 256 * 256; }
+
+// Device memory beyond inputs and outputs that one launch of `k` uses: its own workspace (for a staged description the
+// tensors between its kernels) followed by the workspaces of its stages, each piece a multiple of 256 bytes.
+uint64_t scratchBytesNeeded(const akg_hip_kernel *k) {
+  uint64_t total = alignScratch(k->lowered.workspaceBytes);
+  for (const auto &st : k->stages) total += scratchBytesNeeded(st.kernel);
+  return total;
+}
+
+// Code object of `k` (and of its stages) on `device`, if it has been loaded there; loads nothing.
+bool findLoaded(akg_hip_kernel *k, int device, akg_hip_kernel::Loaded *out) {
+  for (auto &st : k->stages) {
+    akg_hip_kernel::Loaded ls;
+    if (!findLoaded(st.kernel, device, &ls)) return false;
+  }
+  std::lock_guard<std::mutex> lock(k->mu);
+  for (const auto &l : k->loaded) {
+    if (l.device == device) {
+      *out = l;
+      return true;
+    }
+  }
+  return false;
+}
+
+// Enqueues the kernel(s) of `k`. With `scratchBase` NULL the handle's own workspaces are used; otherwise the launch
+// takes its scratchBytesNeeded(k) bytes from `scratchBase` (laid out as that function says) and nothing is loaded or
+// allocated: every code object must be on the device already.
+int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream,
+             char *scratchBase = nullptr) {
+  void *const workspace = scratchBase != nullptr ? (k->lowered.workspaceBytes > 0 ? scratchBase : nullptr) : l.workspace;
   if (!k->stages.empty()) {
     const size_t nin = k->graph.inputs.size();
+    char *stageScratch = scratchBase != nullptr ? scratchBase + alignScratch(k->lowered.workspaceBytes) : nullptr;
     for (auto &st : k->stages) {
       akg_hip_kernel::Loaded ls;
-      int rc = ensureLoaded(st.kernel, &ls);
+      int rc = AKG_HIP_OK;
+      if (scratchBase != nullptr) {
+        if (!findLoaded(st.kernel, l.device, &ls)) return fail(AKG_HIP_ERR_INTERNAL, "stage not loaded");
+      } else {
+        rc = ensureLoaded(st.kernel, &ls);
+      }
       if (rc != AKG_HIP_OK) return rc;
       std::vector<void *> ptrs(st.args.size());
       for (size_t a = 0; a < st.args.size(); ++a) {
@@ -618,18 +656,19 @@ int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *de
         } else if (sa.kind == akg::StageArg::Kind::Output) {
           ptrs[a] = devicePtrs[nin + static_cast<size_t>(sa.index)];
         } else {
-          ptrs[a] = static_cast<char *>(l.workspace) + k->tempOffsets[static_cast<size_t>(sa.index)];
+          ptrs[a] = static_cast<char *>(workspace) + k->tempOffsets[static_cast<size_t>(sa.index)];
         }
       }
-      rc = launchOn(st.kernel, ls, ptrs.data(), stream);
+      rc = launchOn(st.kernel, ls, ptrs.data(), stream, stageScratch);
       if (rc != AKG_HIP_OK) return rc;
+      if (stageScratch != nullptr) stageScratch += scratchBytesNeeded(st.kernel);
     }
     return AKG_HIP_OK;
   }
   // kernel arguments: the tensor pointers, then the 64-bit scalars of the lowering, then the workspace
   const int n = numTensors(k);
   const int nscalar = static_cast<int>(k->lowered.scalarArgs.size());
-  const int nargs = n + nscalar + (l.workspace ? 1 : 0);
+  const int nargs = n + nscalar + (workspace ? 1 : 0);
   std::vector<void *> slots(static_cast<size_t>(nargs));
   std::vector<void *> params(static_cast<size_t>(nargs));
   for (int i = 0; i < nargs; ++i) {
@@ -639,7 +678,7 @@ int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *de
     } else if (i < n + nscalar) {
       params[static_cast<size_t>(i)] = const_cast<int64_t *>(&k->lowered.scalarArgs[static_cast<size_t>(i - n)]);
     } else {
-      slots[static_cast<size_t>(i)] = l.workspace;
+      slots[static_cast<size_t>(i)] = workspace;
       params[static_cast<size_t>(i)] = &slots[static_cast<size_t>(i)];
     }
   }
@@ -749,6 +788,42 @@ int akg_hip_launch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptr
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   return launchOn(kernel, fn, device_ptrs, static_cast<hipStream_t>(stream));
+}
+
+int akg_hip_launch_static_scratch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream) {
+  int rc = checkPtrs(kernel, device_ptrs, n_ptrs);
+  if (rc != AKG_HIP_OK) return rc;
+  const uint64_t need = scratchBytesNeeded(kernel);
+  if (need > AKG_HIP_STATIC_SCRATCH_BYTES) {
+    return fail(AKG_HIP_ERR_UNSUPPORTED, "kernel " + kernel->graph.name + " needs " + std::to_string(need) +
+                                           " bytes of scratch, the static array holds " +
+                                           std::to_string(AKG_HIP_STATIC_SCRATCH_BYTES) + ": use akg_hip_launch");
+  }
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipGetDevice: " + hipErr(e));
+  akg_hip_kernel::Loaded fn;
+  if (!findLoaded(kernel, device, &fn)) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel " + kernel->graph.name + " is not loaded on device " +
+                                                std::to_string(device) +
+                                                ": call akg_hip_kernel_prepare once before the launches that must not allocate");
+  }
+  char *base = nullptr;
+  if (need > 0) {
+    void *p = nullptr;
+    e = akg::staticScratchOnCurrentDevice(&p);
+    if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "address of the static scratch array: " + hipErr(e));
+    base = static_cast<char *>(p);
+    // The array keeps whatever the last launch on this device left (another handle's partial results, or counters of
+    // a launch that failed half way), and the kernels expect their arrival counters at zero: clear the part used.
+    e = akg::staticScratchClear(base, need, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "clearing the static scratch array: " + hipErr(e));
+  } else {
+    // no kernel of this handle uses scratch; a non-NULL base only tells launchOn to load and allocate nothing
+    static char unused;
+    base = &unused;
+  }
+  return launchOn(kernel, fn, device_ptrs, static_cast<hipStream_t>(stream), base);
 }
 
 int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel) {

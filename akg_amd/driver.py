@@ -67,6 +67,7 @@ def load_library():
     lib.akg_hip_kernel_source.argtypes = [vp, ctypes.POINTER(cp)]
     lib.akg_hip_kernel_prepare.argtypes = [vp]
     lib.akg_hip_launch.argtypes = [vp, ctypes.POINTER(vp), ci, vp]
+    lib.akg_hip_launch_static_scratch.argtypes = [vp, ctypes.POINTER(vp), ci, vp]
     lib.akg_hip_run_host.argtypes = [vp, ctypes.POINTER(vp), ci]
     lib.akg_hip_profile.argtypes = [vp, ctypes.POINTER(vp), ci, ci, ci, ctypes.POINTER(ctypes.c_double)]
     lib.akg_hip_kernel_destroy.argtypes = [vp]
@@ -221,6 +222,11 @@ class HipKernel:
     def launch_ptrs(self, device_ptrs, stream=None):
         arr = self._ptr_array(device_ptrs)
         _check(self._lib.akg_hip_launch(self._handle, arr, len(device_ptrs), ctypes.c_void_p(stream or 0)))
+
+    def launch_static_scratch_ptrs(self, device_ptrs, stream=None):
+        """`launch_ptrs` through the entry point that allocates nothing (needs `prepare()` on the device first)."""
+        arr = self._ptr_array(device_ptrs)
+        _check(self._lib.akg_hip_launch_static_scratch(self._handle, arr, len(device_ptrs), ctypes.c_void_p(stream or 0)))
 
     def launch(self, tensors, stream=None):
         """Launch on torch device tensors (inputs then outputs), on `stream` (a torch stream) or the current one."""

@@ -129,6 +129,25 @@ int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel);
 int akg_hip_launch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream);
 
 /**
+ * akg_hip_launch for callers that cannot allocate device memory: code under HIP graph capture, serving loops with a
+ * frozen memory plan, harnesses that forbid hipMalloc. It has no counterpart in the reference (whose shim allocates
+ * and frees every tensor on every call, code_template.py:160-211). Same arguments and results as akg_hip_launch, but
+ * the device memory that the kernels use beyond inputs and outputs (arrival counters and partial results of streaming
+ * reductions and split-K GEMMs, grouped segment sums, the tensors between the kernels of a staged description) is a
+ * fixed array of AKG_HIP_STATIC_SCRATCH_MAX bytes inside the library's own code object instead of the handle's
+ * workspace, and the call allocates, loads and frees nothing:
+ *  - akg_hip_kernel_prepare must have been called for this handle on the current device (it loads the code objects);
+ *    otherwise AKG_HIP_ERR_INVALID_ARGUMENT;
+ *  - a handle that needs more than AKG_HIP_STATIC_SCRATCH_MAX bytes is refused with AKG_HIP_ERR_UNSUPPORTED;
+ *  - the part of the array the handle uses is cleared by a fill kernel on `stream` in front of the launch;
+ *  - every call on a device shares that device's array, whatever the handle: calls that overlap on one device race.
+ *    Order them on one stream or with events.
+ * Each device holds the array (16 MiB) from the first such call until the process ends.
+ */
+#define AKG_HIP_STATIC_SCRATCH_MAX (16u << 20)
+int akg_hip_launch_static_scratch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream);
+
+/**
  * Reference-style execution with HOST pointers: allocate device buffers, copy every tensor in (outputs
  * too, as the reference does, gen_runtime_code.py:95-97), launch, copy the outputs back, free. Replaces
  * `extern "C" cuda_runtime_exec(T0* data_0, ...)` (code_template.py:160-211) called from MlirDriver.run_gpu

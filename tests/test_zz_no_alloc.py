@@ -1,0 +1,108 @@
+"""The launch entry point that allocates nothing (akg_hip_launch_static_scratch) against akg_hip_launch.
+
+Kernels that need device memory beyond inputs and outputs take it from a fixed array inside the library instead of the
+handle's workspace. Both entry points run the same kernels in the same order and the partial results are combined in a
+fixed order, so the outputs must be identical bit for bit (which is inside every bar of the parity tests). Calls follow
+each other on one stream; the second description of each sequence is smaller than the first, so it finds the array
+holding the first one's leftovers.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from akg_amd import driver, harness
+
+pytestmark = pytest.mark.gpu
+
+FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "akg_amd", "fixtures")
+
+# (larger first, smaller second) - streaming reductions, a GEMM with K split over workgroups, descriptions that run as
+# several kernels, a grouped segment sum (several launches of one code object sharing the scratch)
+SEQUENCES = [
+    ("small_biasgrad_bf16_2048x1024.info", "small_reducey_max_f16_130x66.info"),
+    ("small_reducey_sqsum_f32_1x5100x3072.info", "small_reduceall_sqsum_f32_768x512.info"),
+    ("small_gemm_i8_dequant_bias_gelu_300x2064x520_tb.info", "small_gemm_bf16_bias_gelu_256x512x256.info"),
+    ("small_staged_softmax_f32_32x12x24x40_axis1.info", "small_staged_layernorm_axis1_bf16_8x64x49.info"),
+    ("small_segment_sum_f16_150001_by_4_seg300.info", "small_bnstats_f32_32x16x28x28.info"),
+]
+
+
+def _device_buffers(kernel, inputs):
+    import torch
+    dev = torch.device("cuda:0")
+    ins = [torch.from_numpy(a.view(np.int16) if a.dtype == np.uint16 else a).to(dev) for a in inputs]
+    outs = []
+    for d in kernel.outputs:
+        t = torch.empty(d.nbytes, dtype=torch.uint8, device=dev)
+        t.fill_(0xFF if d.dtype in ("float16", "bfloat16", "float32", "float64") else 0x7B)
+        outs.append(t)
+    return ins, outs
+
+
+def _run(kernel, inputs, static):
+    import torch
+    ins, outs = _device_buffers(kernel, inputs)
+    ptrs = [t.data_ptr() for t in ins + outs]
+    stream = torch.cuda.current_stream().cuda_stream
+    if static:
+        kernel.launch_static_scratch_ptrs(ptrs, stream)
+    else:
+        kernel.launch_ptrs(ptrs, stream)
+    torch.cuda.synchronize()
+    # Assign / InplaceAssign descriptions also write an input: compare those too
+    return [t.cpu().numpy().view(np.uint8).copy() for t in outs + ins]
+
+
+@pytest.mark.parametrize("first,second", SEQUENCES)
+def test_static_scratch_launch_equals_the_allocating_launch(first, second):
+    cases = []
+    for name in (first, second):
+        path = os.path.join(FIXTURES, name)
+        kernel = driver.HipKernel.from_file(path)
+        assert kernel.workspace_bytes > 0, "%s uses no scratch: it proves nothing here" % name
+        inputs = harness.make_inputs(harness.load_desc(path), seed=harness.BASE_SEED + 4242)
+        kernel.prepare()
+        cases.append((name, kernel, inputs))
+    expected = [_run(k, i, static=False) for _, k, i in cases]
+    # twice through the sequence: the second round starts on an array that every kernel of the first has used
+    for round_no in range(2):
+        for (name, kernel, inputs), want in zip(cases, expected):
+            print("case %s round %d" % (name, round_no), flush=True)
+            got = _run(kernel, inputs, static=True)
+            for idx, (g, w) in enumerate(zip(got, want)):
+                assert np.array_equal(g, w), "%s round %d: buffer %d differs from akg_hip_launch's" % (name, round_no, idx)
+
+
+def test_static_scratch_launch_needs_a_prepared_handle_and_refuses_oversized_scratch():
+    path = os.path.join(FIXTURES, "small_reduceall_sqsum_f32_768x512.info")
+    kernel = driver.HipKernel.from_file(path)
+    inputs = harness.make_inputs(harness.load_desc(path), seed=harness.BASE_SEED)
+    ins, outs = _device_buffers(kernel, inputs)
+    ptrs = [t.data_ptr() for t in ins + outs]
+    with pytest.raises(driver.AkgHipError) as not_loaded:
+        kernel.launch_static_scratch_ptrs(ptrs)
+    assert not_loaded.value.code == -1 and "akg_hip_kernel_prepare" in str(not_loaded.value)
+    # 335 MB of grouped rows: beyond the 16 MiB array
+    big = driver.HipKernel.from_file(os.path.join(FIXTURES, "n7_segment_sum_f32_4954x4953_by_1x3_seg4954.info"))
+    assert big.workspace_bytes > (16 << 20)
+    fake = [ptrs[0]] * len(big.tensors)
+    with pytest.raises(driver.AkgHipError) as too_big:
+        big.launch_static_scratch_ptrs(fake)
+    assert too_big.value.code == -4 and "scratch" in str(too_big.value)
+
+
+def test_static_scratch_launch_serves_kernels_without_scratch():
+    import torch
+    path = os.path.join(FIXTURES, "small_softmax_f16_64x4096.info")
+    if not os.path.exists(path):
+        pytest.skip("fixture missing")
+    kernel = driver.HipKernel.from_file(path)
+    assert kernel.workspace_bytes == 0
+    kernel.prepare()
+    inputs = harness.make_inputs(harness.load_desc(path), seed=harness.BASE_SEED + 7)
+    want = _run(kernel, inputs, static=False)
+    got = _run(kernel, inputs, static=True)
+    for g, w in zip(got, want):
+        assert np.array_equal(g, w)
+    torch.cuda.synchronize()
