@@ -414,8 +414,20 @@ std::string elementwiseExpr(const OpGraph &g, const OpNode &op, const std::vecto
     case OpKind::Asin: return unaryMath("op_asin");
     case OpKind::Acos: return unaryMath("op_acos");
     case OpKind::Atan: return unaryMath("op_atan");
-    case OpKind::Asinh: return unaryMath("op_asinh");
-    case OpKind::Acosh: return unaryMath("op_acosh");
+    case OpKind::Asinh:
+    case OpKind::Acosh: {
+      // not the library functions: the reference spells them log(x + sqrt(1 + x*x)) and log(x + sqrt(x*x - 1)), one
+      // arith / math op of the result type per step (createAsinhOp / createAcoshOp, MindSporeToLinalg.cpp:156-180), so a
+      // large negative x cancels to log(0) and a float16 square overflows - results a caller of the reference sees
+      need(1);
+      floatOnly();
+      const std::string x = conv(0), one = literalFor(od, 1.0);
+      const std::string sq = rnd("akg::op_mul(" + x + ", " + x + ")");
+      const std::string inner = op.kind == OpKind::Asinh ? rnd("akg::op_add(" + one + ", " + sq + ")")
+                                                          : rnd("akg::op_sub(" + sq + ", " + one + ")");
+      const std::string root = rnd("akg::op_sqrt(" + inner + ")");
+      return rnd("akg::op_log(" + rnd("akg::op_add(" + x + ", " + root + ")") + ")");
+    }
     case OpKind::IsNan: return predicate("op_isnan");
     case OpKind::IsInf: return predicate("op_isinf");
     case OpKind::IsFinite: return predicate("op_isfinite");

@@ -9,8 +9,11 @@
  * [M,N] int32 / float32 intermediates never exist in memory.
  *
  * Float MatMul: the reference accumulates in the MatMul's declared result type, element by element in k order
- * (zero-filled accumulator of the output type, MindSporeToLinalg.cpp:1520-1540). The MFMA accumulates in float32
- * whatever the declared type; a float16 / bfloat16 result is rounded once, after the whole sum.
+ * (zero-filled accumulator of the output type, MindSporeToLinalg.cpp:1520-1540). The MFMA kernels serve a declared
+ * float32 result (their float32 sum differs from the reference's only in the order of the additions). A declared
+ * float16 / bfloat16 result means a product and a sum rounded to 16 bits at every k, which no matrix unit computes:
+ * such descriptions, and the shapes and element types the MFMA kernels do not take, go to the serial kernel of
+ * kernels/akg_gemm_serial.hpp, which keeps the reference's order and rounding exactly.
  *
  * Epilogue operands are classified by how they vary over the output tile:
  *   Full   [M,N]      4-element chunk per (row, 4 columns), loaded / computed per output chunk
@@ -51,7 +54,10 @@ class GemmEmitter {
     k.family = KernelFamily::GemmEpilogue;
     const int64_t tiles = ((m_ + 255) / 256) * ((n_ + 255) / 256);
     const int64_t gridTiles = ((tiles + 7) / 8) * 8;
-    if (skinny_) {
+    if (serial_) {
+      k.grid[0] = static_cast<unsigned>(((m_ + 63) / 64) * ((n_ + 16 * epiWidth() - 1) / (16 * epiWidth())));
+      k.block[0] = 256;
+    } else if (skinny_) {
       const int64_t strips = (n_ + 127) / 128;
       k.grid[0] = static_cast<unsigned>(strips * kSplit_);
       if (kSplit_ > 1) {
@@ -74,7 +80,10 @@ class GemmEmitter {
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
     note << "gemm_epilogue batch=" << batch_ << " M=" << m_ << " N=" << n_ << " K=" << k_ << " transpose_b=" << (transB_ ? 1 : 0);
-    if (skinny_) {
+    if (serial_) {
+      note << " serial: the reference's k-ordered sum in the declared type on the vector ALUs, tile=64x" << 16 * epiWidth()
+           << " grid=" << k.grid[0];
+    } else if (skinny_) {
       note << " skinny: strips of 128 columns, B straight into MFMA operands, mfma=" << mfmaName() << " waves=4 grid=" << k.grid[0];
     } else {
       note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
@@ -94,6 +103,8 @@ class GemmEmitter {
   int skinnyRows() const { return (opt_.variant & 16) ? 32 : 64; }   // (96 rows: no faster than the tile kernel; 128: slower)
   int skinnyWaves() const { return opt_.block == 512 ? 8 : 4; }
   int skinnyUnroll() const { return opt_.chunks > 0 ? opt_.chunks : 2; }
+  bool serial_ = false;  // no MFMA kernel takes the description: gemm_serial (akg_gemm_serial.hpp)
+  int epiWidth() const { return (serial_ && n_ % 4 != 0) ? 1 : 4; }   // adjacent result columns per epilogue call
   bool skinny_ = false;  // M <= 64: the kernel that streams B straight into MFMA operands (gemm_skinny)
   bool transB_ = false;
   int matmulOp_ = -1;
@@ -110,7 +121,7 @@ class GemmEmitter {
   const char *mfmaName() const {
     return elem_ == DType::I8 ? "i32_32x32x32_i8" : (elem_ == DType::BF16 ? "f32_32x32x16_bf16" : "f32_32x32x16_f16");
   }
-  const char *accType() const { return elem_ == DType::I8 ? "int" : "float"; }
+  std::string accType() const { return serial_ ? computeTypeName(g_.tensor(accId_).dtype) : (elem_ == DType::I8 ? "int" : "float"); }
   // The tuning variants exist for the 8-bit kernel only; 16-bit operands always use 4 x 2 wavefronts and 128-byte steps.
   // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_VARIANT=1.
   int wavesM() const { return (opt_.variant & 1) ? 2 : 4; }
@@ -123,6 +134,7 @@ class GemmEmitter {
   // enough workgroups to fill the chip, at least four K steps each.
   void pickSplit() {
     kSplit_ = 1;
+    if (serial_) return;
     // At most 64 rows of A (and K a multiple of 32 bytes): the time is that of streaming B, which gemm_skinny reads
     // straight into MFMA operands; 256 workgroups of four wavefronts (one per CU: 16 x 8192 x 8192 bf16 reaches 66 % of
     // the HBM peak with 4 splits of 64 strips, 59 % with 8, 48 % with 2; 8 wavefronts or more steps in flight change
@@ -179,14 +191,23 @@ class GemmEmitter {
     if (a.inputIndex < 0 || b.inputIndex < 0) {
       throw LoweringError("MatMul operands must be kernel inputs (prologue fusion is not supported yet)");
     }
-    if (a.dtype == DType::I8 && b.dtype == DType::I8 && c.dtype == DType::I32) {
+    if (a.dtype != b.dtype) throw LoweringError("MatMul: the operands must have one element type");
+    if (a.dtype == DType::I8 && c.dtype == DType::I32) {
       elem_ = DType::I8;
-    } else if ((a.dtype == DType::BF16 || a.dtype == DType::F16) && b.dtype == a.dtype &&
-               (c.dtype == DType::F32 || c.dtype == a.dtype)) {
+    } else if ((a.dtype == DType::BF16 || a.dtype == DType::F16) && c.dtype == DType::F32) {
       elem_ = a.dtype;
     } else {
-      throw LoweringError("MatMul: MFMA kernels exist for int8 x int8 -> int32 and for bfloat16 / float16 operands "
-                          "with a float32 or same-type result");
+      // linalg.matmul converts both operands to the accumulator's element type: the same type, a wider integer, or a
+      // wider float
+      auto isIntType = [](DType t) { return t == DType::I8 || t == DType::I16 || t == DType::I32 || t == DType::I64; };
+      const bool sameType = c.dtype == a.dtype && a.dtype != DType::Bool;
+      const bool widerInt = isIntType(a.dtype) && isIntType(c.dtype) && dtypeSize(c.dtype) > dtypeSize(a.dtype);
+      const bool widerFloat = isFloatType(a.dtype) && isFloatType(c.dtype) && dtypeSize(c.dtype) > dtypeSize(a.dtype);
+      if (!sameType && !widerInt && !widerFloat) {
+        throw LoweringError("MatMul: the result type must be the operands' type or a wider one of the same kind");
+      }
+      elem_ = a.dtype;
+      serial_ = true;
     }
     // [M,K] x [K,N], or one leading batch dimension on all three ([B,M,K] x [B,K,N] -> [B,M,N]: linalg.batch_matmul,
     // MindSporeToLinalg.cpp:1511-1530); every batch is one grid.y slice of the same tile kernel.
@@ -203,8 +224,11 @@ class GemmEmitter {
     n_ = transB_ ? b.shape[o] : b.shape[o + 1];
     const int64_t kb = transB_ ? b.shape[o + 1] : b.shape[o];
     if (kb != k_ || c.shape[o] != m_ || c.shape[o + 1] != n_) throw LoweringError("MatMul: inconsistent shapes");
-    if ((k_ * elemBytes()) % 16 != 0) throw LoweringError("MatMul: a row of K must be a multiple of 16 bytes");
-    if (n_ % 4 != 0) throw LoweringError("MatMul: N must be a multiple of 4");
+    // rows of K that are not whole 16-byte pieces, N not a multiple of 4: shapes the MFMA kernels' loads do not take
+    if ((k_ * elemBytes()) % 16 != 0 || n_ % 4 != 0) serial_ = true;
+    if (serial_ && (m_ * k_ >= (1LL << 31) || k_ * n_ >= (1LL << 31) || m_ * n_ >= (1LL << 31))) {
+      throw LoweringError("MatMul: operands of 2^31 elements and more need the MFMA kernels' shapes");
+    }
     for (const OpNode &op : g_.ops) {
       if (op.kind == OpKind::MatMul) continue;
       for (int in : op.inputs) {
@@ -253,6 +277,7 @@ class GemmEmitter {
     vals_.assign(g_.tensors.size(), EpiVal());
     relaxed_ = lowering::relaxedPrecisionTensors(g_);
     const bool nt = opt_.nonTemporal != 0;
+    const std::string W = std::to_string(epiWidth());   // result columns per epilogue call
 
     // accumulators
     EpiVal &acc = vals_[static_cast<size_t>(accId_)];
@@ -260,7 +285,7 @@ class GemmEmitter {
     acc.rank = EpiRank::Full;
     acc.ident = "acc";
     const DType accDt = g_.tensor(accId_).dtype;
-    if (accDt == DType::F16 || accDt == DType::BF16) {
+    if (!serial_ && (accDt == DType::F16 || accDt == DType::BF16)) {
       // a 16-bit MatMul result: the float32 sum is rounded to the declared type once
       acc.ident = "accr";
       apply_ << "    float accr[4];\n#pragma unroll\n    for (int e = 0; e < 4; ++e) accr[e] = " << dtypeTag(accDt)
@@ -294,8 +319,8 @@ class GemmEmitter {
           break;
         case EpiRank::Col:
           v.ident = "c_in" + std::to_string(i);
-          members_ << "  " << ct << " " << v.ident << "[4];\n";
-          prepare_ << "    akg::load_chunk<" << tag << ", 4, false>(in" << i << " + col, " << v.ident << ");\n";
+          members_ << "  " << ct << " " << v.ident << "[" << W << "];\n";
+          prepare_ << "    akg::load_chunk<" << tag << ", " << W << ", false>(in" << i << " + col, " << v.ident << ");\n";
           break;
         case EpiRank::Row:
           v.ident = "r_in" + std::to_string(i);
@@ -303,8 +328,8 @@ class GemmEmitter {
           break;
         case EpiRank::Full:
           v.ident = "t_in" + std::to_string(i);
-          apply_ << "    " << ct << " " << v.ident << "[4];\n";
-          apply_ << "    akg::load_chunk<" << tag << ", 4, " << (nt ? "true" : "false") << ">(in" << i << " + grow * " << n_
+          apply_ << "    " << ct << " " << v.ident << "[" << W << "];\n";
+          apply_ << "    akg::load_chunk<" << tag << ", " << W << ", " << (nt ? "true" : "false") << ">(in" << i << " + grow * " << n_
                  << "L + col, " << v.ident << ");\n";
           break;
         default:
@@ -348,13 +373,13 @@ class GemmEmitter {
       switch (rank) {
         case EpiRank::Full:
           v.ident = "t" + std::to_string(outId);
-          apply_ << "    " << ct << " " << v.ident << "[4];" << comment;
-          apply_ << "#pragma unroll\n    for (int e = 0; e < 4; ++e) " << v.ident << "[e] = " << expr << ";\n";
+          apply_ << "    " << ct << " " << v.ident << "[" << W << "];" << comment;
+          apply_ << "#pragma unroll\n    for (int e = 0; e < " << W << "; ++e) " << v.ident << "[e] = " << expr << ";\n";
           break;
         case EpiRank::Col:
           v.ident = "c" + std::to_string(outId);
-          members_ << "  " << ct << " " << v.ident << "[4];\n";
-          prepare_ << "#pragma unroll\n    for (int e = 0; e < 4; ++e) " << v.ident << "[e] = " << expr << ";" << comment;
+          members_ << "  " << ct << " " << v.ident << "[" << W << "];\n";
+          prepare_ << "#pragma unroll\n    for (int e = 0; e < " << W << "; ++e) " << v.ident << "[e] = " << expr << ";" << comment;
           break;
         case EpiRank::Row:
           v.ident = "r" + std::to_string(outId);
@@ -376,21 +401,21 @@ class GemmEmitter {
       if (t.numel() != batch_ * m_ * n_ || v.rank != EpiRank::Full) {
         throw LoweringError("output " + t.name + ": only [M,N] outputs of a MatMul fusion are supported");
       }
-      apply_ << "    akg::store_chunk<" << tagOf(id) << ", 4, " << (nt ? "true" : "false") << ">(out" << i << " + grow * "
+      apply_ << "    akg::store_chunk<" << tagOf(id) << ", " << W << ", " << (nt ? "true" : "false") << ">(out" << i << " + grow * "
              << n_ << "L + col, " << v.ident << ");\n";
     }
 
     const std::string kname = g_.name + "_kernel";
     src_ << "// Generated by the akg HIP lowering for gfx950. Op description: " << g_.name << "\n";
     src_ << "// family: gemm_epilogue, fusion class: " << operatorTemplateName(g_.operatorTemplate) << "\n";
-    src_ << "#include \"akg_rt.hpp\"\n#include \"akg_gemm_mfma.hpp\"\n\n";
+    src_ << "#include \"akg_rt.hpp\"\n#include \"" << (serial_ ? "akg_gemm_serial.hpp" : "akg_gemm_mfma.hpp") << "\"\n\n";
     src_ << "namespace {\nstruct Epilogue {\n" << members_.str();
     src_ << "  AKG_DEV void prepare(long col) {\n    (void)col;\n" << prepare_.str() << "  }\n";
     src_ << "  long row0;  // first row of this batch in the [batch * M, N] view of the result\n";
-    src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[4], long row, long col) {\n"
+    src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[" << W << "], long row, long col) {\n"
          << "    const long grow = row0 + row;\n    (void)grow;\n" << apply_.str() << "  }\n";
     src_ << "};\n}  // namespace\n\n";
-    src_ << "extern \"C\" __global__ __launch_bounds__(" << (skinny_ ? skinnyWaves() * 64 : wavesM() * 128) << ") void " << kname << "(";
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << (serial_ ? 256 : (skinny_ ? skinnyWaves() * 64 : wavesM() * 128)) << ") void " << kname << "(";
     size_t argc = 0;
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
@@ -407,6 +432,12 @@ class GemmEmitter {
       src_ << "  epi.in" << i << " = in" << i << ";\n";
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";
+    if (serial_) {
+      src_ << "  akg::gemm_serial<" << tagOf(aId_) << ", " << tagOf(accId_) << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, "
+           << (transB_ ? "true" : "false") << ", " << W << ", Epilogue>(in" << g_.tensor(aId_).inputIndex << " + akg_batch * "
+           << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex << " + akg_batch * " << k_ * n_ << "L, epi);\n}\n";
+      return;
+    }
     if (skinny_) {
       src_ << "  akg::gemm_skinny<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
            << ", Epilogue, " << kSplit_ << ", " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (opt_.nonTemporal != 0 ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in"

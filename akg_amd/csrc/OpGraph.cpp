@@ -458,7 +458,7 @@ class GraphBuilder {
   //                :1126-1135, MindSporeToLinalg.cpp:970-1040)
   //   Slice        attrs "begin", "size" (-1: to the end) (convertSliceOp :1089-1101)
   //   StridedSlice attrs or constant inputs begin / end / strides, negative end counted from the back; the
-  //                lowering uses these three only (MindSporeFinalizingLower.cpp:102-140), so non-zero masks are refused
+  //                lowering uses these three only (MindSporeFinalizingLower.cpp:102-140): the mask attributes are ignored, as there
   //   Pad          attr "padding" = (before, after) pairs listed from the LAST dimension backwards, "value",
   //                mode "constant" (MindSporeToTosa.cpp:305-376)
   //   Concat       two operands, attr "axis" (default 0) (convertConcatOp :1117-1124)
@@ -617,12 +617,11 @@ class GraphBuilder {
         needRank(node->begin, "begin");
         needRank(end, "end");
         needRank(node->strides, "strides");
-        for (const char *mask : {"beginMask", "endMask", "ellipsisMask", "newAxisMask", "shrinkAxisMask"}) {
-          const json::Value *m = findAttr(attrs, mask);
-          if (m != nullptr && m->asDouble() != 0.0) {
-            throw TranslateError("op " + nm + ": a non-zero " + mask + " is not supported");
-          }
-        }
+        // beginMask / endMask / ellipsisMask / newAxisMask / shrinkAxisMask are copied onto the op by the reference's
+        // translator (TranslateToMindsporeDialect.cpp:1034-1087) and never read again: its lowering builds the
+        // tensor.extract_slice from begin, end and strides alone (MindSporeFinalizingLower.cpp:117-124). They are
+        // ignored here the same way. (A declared result that drops unit dimensions, as a shrink mask implies, is
+        // refused below with every other shape that does not follow from begin / end / strides.)
         for (size_t d = 0; d < rank; ++d) {
           if (end[d] < 0) end[d] += inShape[d];
           if (node->strides[d] < 1) throw TranslateError("op " + nm + ": strides must be positive");

@@ -196,7 +196,11 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
   }
   int maxLevel = 0;
   for (int t : g.outputs) maxLevel = std::max(maxLevel, level[static_cast<size_t>(t)]);
-  if (maxLevel == 0) {   // (outputs of different shapes alone are no reason for several kernels)
+  std::set<std::vector<int64_t>> outputShapes;
+  for (int t : g.outputs) outputShapes.insert(g.tensor(t).shape);
+  // nothing to cut at: only outputs of different shapes are then a reason for several kernels (one per shape; the
+  // single-kernel families write outputs of one iteration space)
+  if (maxLevel == 0 && (!reductionsToo || outputShapes.size() < 2)) {
     *why = reductionsToo ? "it has no reduction, contraction or data-movement result to cut at"
                          : "it has no contraction or data-movement result to cut at";
     return false;

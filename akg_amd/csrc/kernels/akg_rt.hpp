@@ -452,10 +452,6 @@ AKG_DEV float op_acos(float a) { return acosf(a); }
 AKG_DEV double op_acos(double a) { return acos(a); }
 AKG_DEV float op_atan(float a) { return atanf(a); }
 AKG_DEV double op_atan(double a) { return atan(a); }
-AKG_DEV float op_asinh(float a) { return asinhf(a); }
-AKG_DEV double op_asinh(double a) { return asinh(a); }
-AKG_DEV float op_acosh(float a) { return acoshf(a); }
-AKG_DEV double op_acosh(double a) { return acosh(a); }
 AKG_DEV float op_pow(float a, float b) { return powf(a, b); }
 AKG_DEV double op_pow(double a, double b) { return pow(a, b); }
 AKG_DEV float op_atan2(float a, float b) { return atan2f(a, b); }

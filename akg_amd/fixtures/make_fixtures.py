@@ -51,6 +51,19 @@ FIXTURES = {
     "small_momentum_update_f32_37x130": lambda n: op_desc.momentum_update(37, 130, "float32", name=n),
     "small_momentum_update_bf16_64x256": lambda n: op_desc.momentum_update(64, 256, "bfloat16", name=n),
     "small_elemany_greater_f32_9x130": lambda n: op_desc.any_greater(9, 130, 2.5, "ElemAny", n),
+    # op-table rows outside the measured fusions, one kernel per group
+    "small_optable_unary_math_f32_37x130": lambda n: op_desc.optable_unary_math(37, 130, "float32", n),
+    "small_optable_unary_math_f16_16x256": lambda n: op_desc.optable_unary_math(16, 256, "float16", n),
+    "small_optable_predicates_logic_33x100": lambda n: op_desc.optable_predicates_logic(33, 100, n),
+    "small_optable_pow_atan2_addn_f32_19x264": lambda n: op_desc.optable_pow_atan2_addn(19, 264, "float32", n),
+    "small_optable_pow_atan2_addn_bf16_8x1024": lambda n: op_desc.optable_pow_atan2_addn(8, 1024, "bfloat16", n),
+    "small_optable_int_div_21x77": lambda n: op_desc.optable_int_div(21, 77, n),
+    # MatMul in the reference's own arithmetic: a 16-bit declared result (product and sum rounded to it at every k), and
+    # shapes / element types the MFMA kernels do not take
+    "small_gemm_f16_result_f16_bias_relu_70x200x36": lambda n: op_desc.gemm_bias_act(70, 200, 36, "float16", "relu", False, "float16", n),
+    "small_gemm_bf16_result_bf16_bias_none_33x129x5_tb": lambda n: op_desc.gemm_bias_act(33, 129, 5, "bfloat16", "none", True, "bfloat16", n),
+    "small_gemm_f32_bias_gelu_70x100x36": lambda n: op_desc.gemm_bias_act(70, 100, 36, "float32", "gelu", False, "float32", n),
+    "small_gemm_bf16_bias_gelu_65x30x10": lambda n: op_desc.gemm_bias_act(65, 30, 10, "bfloat16", "gelu", False, "float32", n),
     # streaming reductions: direction Y, direction ALL, long rows, multi-output
     "small_reducey_sqsum_f32_1x5100x3072": lambda n: op_desc.square_reduce([1, 5100, 3072], [1], "float32", True, "ReduceSum", n),
     "small_reducey_sqsum_f32_3x37x50": lambda n: op_desc.square_reduce([3, 37, 50], [1], "float32", False, "ReduceSum", n),

@@ -648,3 +648,63 @@ def momentum_update(rows, cols, dtype="float32", lr=0.01, mu=0.9, name=None):
     p_out = b.op("InplaceAssign", [p, back(p_new), back(v_new)], [rows, cols], dtype,
                  attrs=[{"data_type": "bool", "name": "fake_output", "value": True}])
     return b.dumps([v_out, p_out])
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Op-table rows outside the measured fusions, grouped so that each group is one small kernel.
+# ---------------------------------------------------------------------------------------------------------
+def optable_unary_math(rows, cols, dtype="float32", name=None):
+    """Log, Sin, Cos, ASin, ACos, Atan, Asinh, Acosh and Floor of one input, each on the part of its domain where an ulp
+    of the function is an ulp of the answer; nine outputs of the input's type (computed in float32 for 16-bit inputs)."""
+    b = DescBuilder(name or "Fused_optable_unary_math_%s_%dx%d" % (dtype, rows, cols))
+    x = b.input([rows, cols], dtype)
+    xf = b.cast(x, "float32") if dtype != "float32" else x
+    c = lambda v: b.const(float(v), "float32")  # noqa: E731
+    mag = b.unary("Abs", xf)
+    unit = b.minimum(b.maximum(xf, c(-0.9)), c(0.9))
+    outs = [b.unary("Log", b.add(mag, c(0.5))), b.unary("Sin", xf), b.unary("Cos", xf), b.unary("ASin", unit),
+            b.unary("ACos", unit), b.unary("Atan", xf), b.unary("Asinh", b.add(mag, c(0.5))),
+            b.unary("Acosh", b.add(mag, c(1.5))), b.unary("Floor", b.mul(xf, c(3.0)))]
+    return b.dumps([b.cast(t, dtype) if dtype != "float32" else t for t in outs])
+
+
+def optable_predicates_logic(rows, cols, name=None):
+    """IsNan / IsInf / IsFinite on values that are NaN (Sqrt of a negative) or -inf (Log of zero) for about half of the
+    elements, LogicalNot / And / Or over them, GreaterEqual and Less, and a Select steered by the result."""
+    b = DescBuilder(name or "Fused_optable_predicates_logic_%dx%d" % (rows, cols))
+    x = b.input([rows, cols], "float32")
+    y = b.input([rows, cols], "float32")
+    zero = b.const(0.0, "float32")
+    nan_ = b.unary("IsNan", b.unary("Sqrt", x), "bool")
+    inf_ = b.unary("IsInf", b.unary("Log", b.maximum(y, zero)), "bool")
+    fin_ = b.unary("IsFinite", b.unary("Log", b.maximum(x, zero)), "bool")
+    q = b.binary("LogicalAnd", b.unary("LogicalNot", nan_), b.binary("LogicalOr", inf_, fin_, "bool"), "bool")
+    ge = b.binary("GreaterEqual", x, y, "bool")
+    lt = b.binary("Less", x, y, "bool")
+    pick = b.op("Select", [b.binary("LogicalAnd", ge, q, "bool"), x, y], [rows, cols], "float32")
+    return b.dumps([q, lt, pick])
+
+
+def optable_pow_atan2_addn(rows, cols, dtype="float32", name=None):
+    """Pow with a positive base and with a whole exponent on a base of either sign, Atan2 over all four quadrants, AddN
+    of four operands."""
+    b = DescBuilder(name or "Fused_optable_pow_atan2_addn_%s_%dx%d" % (dtype, rows, cols))
+    ins = [b.input([rows, cols], dtype) for _ in range(3)]
+    x, y, z = [b.cast(t, "float32") if dtype != "float32" else t for t in ins]
+    c = lambda v: b.const(float(v), "float32")  # noqa: E731
+    clip2 = lambda t: b.minimum(b.maximum(t, c(-2.0)), c(2.0))  # noqa: E731
+    outs = [b.binary("Pow", b.add(b.minimum(b.unary("Abs", x), c(1.5)), c(0.5)), clip2(y)),
+            b.binary("Pow", clip2(x), c(3.0)),
+            b.binary("Atan2", x, y),
+            b.op("AddN", [x, y, z, x], [rows, cols], "float32")]
+    return b.dumps([b.cast(t, dtype) if dtype != "float32" else t for t in outs])
+
+
+def optable_int_div(rows, cols, name=None):
+    """Integer Div (truncating; zero divisors occur) and a comparison of an integer with a float tensor."""
+    b = DescBuilder(name or "Fused_optable_int_div_%dx%d" % (rows, cols))
+    n = b.input([rows, cols], "int32")
+    d = b.input([rows, cols], "int32")
+    f = b.input([rows, cols], "float32")
+    q = b.binary("Div", b.mul(n, b.const(37, "int32")), d, "int32")
+    return b.dumps([q, b.binary("Less", d, b.mul(f, b.const(50.0, "float32")), "bool")])

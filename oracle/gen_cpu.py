@@ -52,8 +52,12 @@ C_COMPUTE = {
 INT_RANGE = {"int8": (-128, 127), "int16": (-32768, 32767), "int32": (-2147483648, 2147483647),
              "int64": (-9223372036854775808, 9223372036854775807)}
 
+# Exp / Log / Tanh / Floor come through tosa (MindSporeToTosa.cpp:490-497) and end in libm (`convert-math-to-libm`), Sin / Cos /
+# Sqrt through math.sin / cos / sqrt (MindSporeToLinalg.cpp:182-193,248-259). ASin, ACos and Atan are in the op table but
+# have no lowering in the reference (createLinalgBodyCalculationForElementwiseOp, MindSporeToLinalg.cpp:341-375, returns
+# nothing for them and its conversion fails): they are restated as the functions their names say.
 UNARY_MATH = {"Exp": "exp", "Log": "log", "Tanh": "tanh", "Sqrt": "sqrt", "Floor": "floor", "Sin": "sin", "Cos": "cos",
-              "ASin": "asin", "ACos": "acos", "Atan": "atan", "Asinh": "asinh", "Acosh": "acosh"}
+              "ASin": "asin", "ACos": "acos", "Atan": "atan"}
 COMPARE = {"Equal": "==", "NotEqual": "!=", "Greater": ">", "GreaterEqual": ">=", "Less": "<", "LessEqual": "<="}
 MATMULS = ("MatMul", "BatchMatMul")
 # Assign / InplaceAssign: linalg.copy ins=input1 outs=input0 (MindSporeToLinalg.cpp:495-524): the value is written over
@@ -416,6 +420,16 @@ class Emitter:
             if od not in FLOATS:
                 raise OracleError("%s needs a float tensor" % n)
             return self.rnd(od, "%s%s(%s)" % (UNARY_MATH[n], suffix, conv[0]))
+        if n in ("Asinh", "Acosh"):
+            # not libm: log(x + sqrt(1 + x*x)) and log(x + sqrt(x*x - 1)), one arith / math op of the result type each
+            # (createAsinhOp / createAcoshOp, MindSporeToLinalg.cpp:156-180)
+            if od not in FLOATS:
+                raise OracleError("%s needs a float tensor" % n)
+            one = "1.0" if od == "float64" else "1.0f"
+            sq = self.rnd(od, "(%s * %s)" % (conv[0], conv[0]))
+            inner = self.rnd(od, "(%s + %s)" % (one, sq)) if n == "Asinh" else self.rnd(od, "(%s - %s)" % (sq, one))
+            root = self.rnd(od, "sqrt%s(%s)" % (suffix, inner))
+            return self.rnd(od, "log%s(%s)" % (suffix, self.rnd(od, "(%s + %s)" % (conv[0], root))))
         if n == "Rsqrt":
             one = "1.0" if od == "float64" else "1.0f"
             return self.rnd(od, "(%s / sqrt%s(%s))" % (one, suffix, conv[0]))
@@ -722,8 +736,6 @@ class Emitter:
         cidx = "(bt * %dL + i) * %dL + j" % (m, n)
         # zero-filled accumulator of the output type
         self.emit("memset(%s, 0, sizeof(%s) * %dL);" % (out.buffer, C_STORAGE[od], batch * m * n))
-        if od in FLOATS and od not in ("float32", "float64"):
-            raise OracleError("MatMul accumulating in %s is not restated" % od)
         self.emit("for (int64_t bt = 0; bt < %dL; ++bt) {" % batch)
         if self.openmp:
             self.emit("#pragma omp parallel for schedule(static)", 2)
@@ -737,6 +749,11 @@ class Emitter:
         if od in INTS:
             ut = "uint64_t" if od == "int64" else "uint32_t"
             self.emit("%s[%s] = (%s)((%s)%s[%s] + (%s)(%s));" % (out.buffer, cidx, C_STORAGE[od], ut, out.buffer, cidx, ut, prod), 5)
+        elif od in ("float16", "bfloat16"):
+            # linalg.matmul casts both operands to the accumulator's element type, multiplies and adds in it: a product
+            # rounded to the 16-bit type, then a sum rounded to it, every step (the accumulator lives in the result buffer)
+            step = self.rnd(od, "(%s + %s)" % (self.load_expr(out, cidx), self.rnd(od, "(%s)" % prod)))
+            self.emit("%s[%s] = %s;" % (out.buffer, cidx, self.store_expr(od, step)), 5)
         else:
             self.emit("%s[%s] = %s[%s] + %s;" % (out.buffer, cidx, out.buffer, cidx, prod), 5)
         self.emit("}", 4)

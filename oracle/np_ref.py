@@ -254,10 +254,17 @@ def evaluate(desc, inputs, updates=None):
                 res = x.dtype.type(1) / x
             elif name == "Floor":
                 res = np.floor(same(cv[0]))
-            elif name in ("Sin", "Cos", "ASin", "ACos", "Atan", "Asinh", "Acosh"):
-                f = {"Sin": np.sin, "Cos": np.cos, "ASin": np.arcsin, "ACos": np.arccos, "Atan": np.arctan,
-                     "Asinh": np.arcsinh, "Acosh": np.arccosh}[name]
+            elif name in ("Sin", "Cos", "ASin", "ACos", "Atan"):
+                f = {"Sin": np.sin, "Cos": np.cos, "ASin": np.arcsin, "ACos": np.arccos, "Atan": np.arctan}[name]
                 res = f(same(cv[0]))
+            elif name in ("Asinh", "Acosh"):
+                # createAsinhOp / createAcoshOp (MindSporeToLinalg.cpp:156-180): log(x + sqrt(1 + x*x)) and
+                # log(x + sqrt(x*x - 1)) spelled as single ops of the result type, not the libm functions
+                x = same(cv[0])
+                step = lambda v: compute_view(finish(v, odt), odt)
+                sq = step(x * x)
+                inner = step(x.dtype.type(1) + sq) if name == "Asinh" else step(sq - x.dtype.type(1))
+                res = np.log(step(x + step(np.sqrt(inner))))
             elif name == "Pow":
                 res = np.power(same(cv[0]), same(cv[1]))
             elif name == "Atan2":
@@ -397,6 +404,15 @@ def evaluate(desc, inputs, updates=None):
                         acc = np.zeros((a2.shape[0], b2.shape[1]), dtype=NP_DTYPE[odt])
                         for k in range(a2.shape[1]):
                             acc = acc + np.outer(a2[:, k].astype(acc.dtype), b2[k, :].astype(acc.dtype))
+                        slices.append(acc)
+                    elif odt in ("float16", "bfloat16") and in_dt[0] == odt and in_dt[1] == odt:
+                        # accumulator of the 16-bit result type (MindSporeToLinalg.cpp:1453-1546): the product and the
+                        # sum are each rounded to it, step by step in k order
+                        rnd = lambda v: compute_view(finish(v, odt), odt)
+                        acc = np.zeros((a2.shape[0], b2.shape[1]), dtype=np.float32)
+                        a32, b32 = compute_view(a2, odt), compute_view(b2, odt)
+                        for k in range(a2.shape[1]):
+                            acc = rnd(acc + rnd(np.outer(a32[:, k], b32[k, :])))
                         slices.append(acc)
                     else:
                         raise ValueError("MatMul %s x %s -> %s is not restated" % (in_dt[0], in_dt[1], odt))

@@ -236,3 +236,127 @@ def random_matmul_description(seed):
     else:
         outs.append(y)
     return b.dumps([b.cast(t, dtype) for t in outs]), notes
+
+
+def random_optable_description(seed):
+    """The rows of the op table that `random_description` does not draw: Log, Sin, Cos, ASin, ACos, Atan, Asinh, Acosh,
+    Floor, IsNan / IsInf / IsFinite, LogicalNot / And / Or, Pow, Atan2, AddN, GreaterEqual, Less, integer Div, a
+    comparison of an integer with a float tensor, ReduceAny / ReduceAll. Same discipline as above: discontinuous ops see
+    exactly computed operands only (the predicates excepted: whether Sqrt or Log of an exact value is NaN / infinite does
+    not depend on the last bit), transcendental ops see operands from the part of their domain where an ulp of their
+    result is an ulp of the answer. Returns (json_text, notes)."""
+    rng = np.random.default_rng(500000 + seed)
+    rank = int(rng.integers(1, 4))
+    base = [int(rng.choice([1, 2, 3, 5, 8, 9, 33])) for _ in range(rank)]
+    base[-1] = int(rng.choice([7, 16, 40, 64, 100, 257]))
+    dtype = str(rng.choice(FLOATS))
+    b = op_desc.DescBuilder("Fused_random_optable_%d" % seed)
+    c = lambda v: b.const(float(v), "float32")  # noqa: E731
+    ins = [b.input(base, dtype)] + [b.input(_variant_shape(rng, base), dtype) for _ in range(int(rng.integers(1, 3)))]
+    work = [Val(b.cast(t, "float32") if dtype != "float32" else t, True) for t in ins]
+    bools = []
+    notes = []
+
+    def pick(pred=lambda v: True):
+        cands = [v for v in work if pred(v)]
+        return cands[int(rng.integers(0, len(cands)))] if cands else None
+
+    def clip(t, lo, hi):
+        return b.minimum(b.maximum(t, c(lo)), c(hi))
+
+    for _ in range(int(rng.integers(3, 9))):
+        kind = str(rng.choice(["trig", "inverse", "hyper", "log", "pow", "atan2", "addn", "floor", "predicate", "logic",
+                               "compare", "intdiv", "mixed"]))
+        x = pick()
+        try:
+            if kind == "trig":
+                name = str(rng.choice(["Sin", "Cos", "Atan"]))
+                work.append(Val(b.unary(name, clip(x.t, -6.0, 6.0)), False))
+            elif kind == "inverse":
+                name = str(rng.choice(["ASin", "ACos"]))
+                work.append(Val(b.unary(name, clip(x.t, -0.9, 0.9)), False))
+            elif kind == "hyper":
+                name = str(rng.choice(["Asinh", "Acosh"]))
+                arg = b.add(clip(b.unary("Abs", x.t), 0.0, 40.0), c(0.5 if name == "Asinh" else 1.5))
+                work.append(Val(b.unary(name, arg), False, positive=True))
+            elif kind == "log":
+                name = "Log"
+                work.append(Val(b.unary("Log", b.add(clip(b.unary("Abs", x.t), 0.0, 40.0), c(0.5))), False))
+            elif kind == "pow":
+                name = "Pow"
+                if rng.random() < 0.5:     # any sign of the base, a whole exponent
+                    t = b.binary("Pow", clip(x.t, -2.0, 2.0), c(int(rng.choice([2, 3]))))
+                else:
+                    y = pick()
+                    t = b.binary("Pow", b.add(clip(b.unary("Abs", x.t), 0.0, 1.5), c(0.5)), clip(y.t, -2.0, 2.0))
+                work.append(Val(t, False))
+            elif kind == "atan2":
+                name = "Atan2"
+                xe, ye = pick(lambda v: v.exact), pick(lambda v: v.exact)
+                work.append(Val(b.binary("Atan2", ye.t, xe.t), False))
+            elif kind == "addn":
+                name = "AddN"
+                terms = [pick() for _ in range(int(rng.integers(3, 5)))]
+                shape = terms[0].t.shape
+                for t in terms[1:]:
+                    shape = b._broadcast(shape, t.t.shape)
+                if any(list(t.t.shape) != list(shape) for t in terms):
+                    continue     # linalg's AddN takes operands of one shape
+                work.append(Val(b.op("AddN", [t.t for t in terms], shape, "float32"), all(t.exact for t in terms), bounded=False))
+            elif kind == "floor":
+                name = "Floor"
+                xe = pick(lambda v: v.exact)
+                work.append(Val(b.unary("Floor", b.mul(xe.t, c(3.0))), True))
+            elif kind == "predicate":
+                name = str(rng.choice(["IsNan", "IsInf", "IsFinite"]))
+                xe = pick(lambda v: v.exact)
+                # Sqrt of a negative value is NaN, Log of zero is -inf: both whatever the last bit of the function says
+                src = b.unary("Sqrt", xe.t) if name == "IsNan" else b.unary("Log", b.maximum(xe.t, c(0.0)))
+                bools.append(b.unary(name, src, "bool"))
+            elif kind == "logic":
+                if len(bools) < 1:
+                    continue
+                name = str(rng.choice(["LogicalNot", "LogicalAnd", "LogicalOr"]))
+                p = bools[int(rng.integers(0, len(bools)))]
+                if name == "LogicalNot":
+                    bools.append(b.unary(name, p))
+                else:
+                    q = bools[int(rng.integers(0, len(bools)))]
+                    bools.append(b.binary(name, p, q, "bool"))
+            elif kind == "compare":
+                name = str(rng.choice(["GreaterEqual", "Less"]))
+                xe, ye = pick(lambda v: v.exact), pick(lambda v: v.exact)
+                bools.append(b.binary(name, xe.t, ye.t, "bool"))
+            elif kind == "intdiv":
+                name = "Div"
+                xe, ye = pick(lambda v: v.exact), pick(lambda v: v.exact)
+                num = b.cast(b.mul(xe.t, c(100.0)), "int32")
+                den = b.cast(b.mul(ye.t, c(3.0)), "int32")        # zero now and then: the agreed x / 0 = 0
+                work.append(Val(b.cast(b.binary("Div", num, den, "int32"), "float32"), True, bounded=False))
+            else:
+                name = "Less-mixed"
+                xe, ye = pick(lambda v: v.exact), pick(lambda v: v.exact)
+                bools.append(b.binary("Less", b.cast(b.mul(xe.t, c(2.0)), "int32"), ye.t, "bool"))
+        except ValueError:
+            continue
+        notes.append(name)
+    outs = []
+    if bools:
+        p = bools[-1]
+        a2, b2 = pick(), pick()
+        try:
+            shape = b._broadcast(b._broadcast(p.shape, a2.t.shape), b2.t.shape)
+            work.append(Val(b.op("Select", [p, a2.t, b2.t], shape, "float32"), a2.exact and b2.exact))
+            notes.append("Select")
+        except ValueError:
+            pass
+        if rng.random() < 0.6 and len(p.shape) >= 1:
+            name = str(rng.choice(["ReduceAny", "ElemAny", "ReduceAll"]))
+            axis = [len(p.shape) - 1] if rng.random() < 0.6 else list(range(len(p.shape)))
+            outs.append(b.reduce(name, p, axis, bool(rng.random() < 0.5)))
+            notes.append("%s%s" % (name, axis))
+        else:
+            outs.append(p)
+    y = work[-1].t
+    outs.append(b.cast(y, dtype) if dtype != "float32" and rng.random() < 0.7 else y)
+    return b.dumps(outs), notes

@@ -976,22 +976,40 @@ def test_full_size_bf16_gemm_bias_gelu_fusion():
     assert ok, msg
 
 
-def test_sixteen_bit_matmul_result_is_one_rounding_of_the_float32_sum():
-    """A MatMul whose declared result type is float16: the reference accumulates in float16 step by step, the MFMA
-    path sums in float32 and rounds once. Checked against torch float64 on a short K, where a float16 running sum
-    would still be inside the 1e-2 / 1e-3 bar (parity with the reference's own rounding sequence is not claimed)."""
-    from akg_amd import op_desc
-    text = op_desc.gemm_bias_act(128, 64, 96, "float16", "none", False, "float16", "Fused_MatMul_f16_result_128x64x96")
-    desc = json_loads(text)
-    kernel = driver.HipKernel(text)
-    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 7)
+SERIAL_GEMMS = ["small_gemm_f16_result_f16_bias_relu_70x200x36.info", "small_gemm_bf16_result_bf16_bias_none_33x129x5_tb.info",
+                "small_gemm_f32_bias_gelu_70x100x36.info", "small_gemm_bf16_bias_gelu_65x30x10.info"]
+
+
+@pytest.mark.parametrize("name", SERIAL_GEMMS)
+def test_matmul_in_the_reference_arithmetic_is_bit_identical_to_the_oracle(name):
+    """A MatMul whose declared result type is float16 / bfloat16 (the reference rounds the product and the sum to it at
+    every k), or whose shape or element type the MFMA kernels do not take, runs as one serial chain over k per result
+    element: the same additions in the same order as the oracle's loop nest, so the accumulators are identical. The
+    fixtures without a transcendental epilogue are compared bit for bit, the GELU ones to the 16-bit / float32 bars."""
+    path = os.path.join(FIXTURES, name)
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)
+    assert kernel.family == "gemm_epilogue" and "gemm_serial" in kernel.source
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 16)
     got = run_on_gpu(kernel, inputs)[0]
-    a, w, bias = [x.astype(np.float64) for x in inputs]
-    acc = (a @ w).astype(np.float16).astype(np.float64)
-    ref = (acc + bias).astype(np.float32).astype(np.float16)
-    ok, msg = harness.compare(got, ref, "float16")
-    print("  float16-result MatMul vs float64: %s" % msg, flush=True)
-    assert ok, msg
+    expect = cpu_ref.CpuKernel(path)(inputs)[0]
+    if "gelu" in name:
+        ok, msg = harness.compare(got, expect, kernel.outputs[0].dtype)
+        assert ok, msg
+    else:
+        assert np.array_equal(got.view(np.uint16), expect.view(np.uint16))
+
+
+def test_sixteen_bit_matmul_result_follows_the_declared_type_on_a_long_k():
+    """4096 products of 1 in float16: the running sum stalls at 2048 as the reference's does; an accumulator that is
+    silently float32 returns 4096."""
+    from akg_amd import op_desc
+    b = op_desc.DescBuilder("Fused_MatMul_f16_result_ones_8x4096x12")
+    a = b.input([8, 4096], "float16")
+    w = b.input([4096, 12], "float16")
+    kernel = driver.HipKernel(b.dumps([b.matmul(a, w, "float16")]))
+    got = run_on_gpu(kernel, [np.ones((8, 4096), np.float16), np.ones((4096, 12), np.float16)])[0]
+    assert np.all(got.astype(np.float32) == 2048.0)
 
 
 def json_loads(text):

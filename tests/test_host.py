@@ -10,6 +10,7 @@ import os
 import re
 import subprocess
 
+import numpy as np
 import pytest
 
 from akg_amd import driver, harness, op_desc
@@ -368,14 +369,26 @@ def test_data_movement_ops_translate_and_go_to_the_indexed_family():
     with pytest.raises(driver.AkgHipError) as e:   # declared shape does not follow from the attributes
         driver.HipKernel(broken(lambda d: d["op_desc"][0]["output_desc"][0].update(shape=[4, 6])), out_dir=None)
     assert e.value.code == -3 and "declared result shape" in str(e.value)
-    # a strided slice with a mask set is refused rather than silently read without it
+    # the mask attributes of a strided slice are ignored, as the reference's lowering ignores them
+    # (MindSporeFinalizingLower.cpp:117-124 reads begin / end / strides only): same kernel source with and without
     b = op_desc.DescBuilder("Fused_masked_slice")
     x = b.input([8, 8], "float32")
-    d = b.build([op_desc.strided_slice(b, x, [0, 0], [4, 8], [1, 1])])
-    d["op_desc"][0]["attr"].append({"data_type": "int", "name": "shrinkAxisMask", "value": 1})
+    d = b.build([op_desc.strided_slice(b, x, [1, 0], [4, 8], [1, 2])])
+    plain = driver.HipKernel(json.dumps(d), out_dir=None).source
+    for mask in ("beginMask", "endMask", "shrinkAxisMask"):
+        d["op_desc"][0]["attr"].append({"data_type": "int", "name": mask, "value": 1})
+    assert driver.HipKernel(json.dumps(d), out_dir=None).source == plain
+    from oracle import np_ref
+    grid = np.arange(64, dtype=np.float32).reshape(8, 8)
+    assert np.array_equal(np_ref.evaluate(d, [grid])[0], grid[1:4, 0:8:2])
+    # ... but a declared result that drops the unit dimension a shrink mask stands for is not what begin / end / strides
+    # give, and is refused
+    d["op_desc"][0]["attr"][1]["value"] = [2, 8]     # end: rows 1..2, one row
+    d["op_desc"][0]["output_desc"][0]["shape"] = [4]
+    d["output_desc"][0]["shape"] = [4]
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(json.dumps(d), out_dir=None)
-    assert e.value.code == -3
+    assert e.value.code == -3 and "declared result shape" in str(e.value)
     # a reduction or a MatMul next to a transpose has no single kernel: the transpose gets a kernel of its own and the
     # other reads its result from the handle's workspace
     b = op_desc.DescBuilder("Fused_Transpose_ReduceSum")

@@ -11,7 +11,7 @@ import pytest
 
 from akg_amd import driver, harness
 from oracle import cpu_ref, np_ref
-from random_graphs import random_description, random_matmul_description
+from random_graphs import random_description, random_matmul_description, random_optable_description
 
 # AKG_RANDOM_GRAPHS=N widens the sweep for a one-off soak on the CPU oracle / a GPU box
 SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_GRAPHS", "40"))))
@@ -52,17 +52,13 @@ def test_random_description_compiles_and_oracles_agree(seed, tmp_path):
         assert ok, "seed %d %s (%s): %s" % (seed, d["tensor_name"], " ".join(notes), msg)
 
 
-@pytest.mark.gpu
-@pytest.mark.parametrize("seed", SEEDS)
-def test_random_description_matches_oracle_on_gpu(seed, tmp_path):
-    from test_gpu_parity import run_on_gpu
-    text, notes = random_description(seed)
-    desc, path = _write(tmp_path, text)
-    print("seed %d: %s" % (seed, " ".join(notes)), flush=True)
-    kernel = driver.HipKernel(text, out_dir=None)
-    inputs = harness.make_inputs(desc, seed=seed)
-    got = run_on_gpu(kernel, inputs)
-    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+INEXACT = ("Exp", "Tanh", "Sqrt", "Rsqrt", "Reciprocal", "RealDiv", "Log", "Sin", "Cos", "ASin", "ACos", "Atan", "Asinh",
+           "Acosh", "Pow", "Atan2")
+
+
+def compare_with_oracle(kernel, desc, notes, inputs, got, expect, seed):
+    """Bars of the GPU half: bool / integer / 16-bit outputs by `harness.compare`; float32 outputs to rtol 1e-5 plus what
+    the conditioning of the description itself allows (see the comments inside)."""
     terms = _terms(desc)
     wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
     exact = np_ref.evaluate(harness.widen_to_float64(desc), wide)
@@ -75,20 +71,36 @@ def test_random_description_matches_oracle_on_gpu(seed, tmp_path):
             # after a subtraction of nearly equal tanh / exp values two correct float32 evaluations differ by that much
             e64 = np.asarray(x, dtype=np.float64).reshape(e.shape)
             slack = 16.0 * np.abs(e.astype(np.float64) - e64)
-            if any(n in ("Exp", "Tanh", "Sqrt", "Rsqrt", "Reciprocal", "RealDiv") for n in notes):
-                # the device's exp / tanh (and its hardware square roots and reciprocals where relaxed) are good to
-                # an ulp or two of their own results, which here are of the inputs' order of magnitude (operands are
-                # clipped to [-6, 6] in front of exp / tanh); a subtraction of two such values keeps that absolute
+            if any(n in INEXACT for n in notes):
+                # the device's transcendental functions (and its hardware square roots and reciprocals where relaxed)
+                # are good to an ulp or two of their own results, which here are of the inputs' order of magnitude
+                # (operands are clipped in front of them); a subtraction of two such values keeps that absolute
                 # error however small its result is, and the oracle may happen to be exact at that element
                 scale = max([1.0] + [float(np.max(np.abs(a.astype(np.float64)))) for a in inputs if a.dtype.kind == "f" and a.size])
                 slack = slack + 2.0 * float(np.finfo(np.float32).eps) * scale
-            bad = np.abs(g.astype(np.float64) - e.astype(np.float64)) > 1e-5 * np.abs(e) + 1e-8 + slack
+            with np.errstate(invalid="ignore"):
+                bad = np.abs(g.astype(np.float64) - e.astype(np.float64)) > 1e-5 * np.abs(e) + 1e-8 + slack
             bad &= ~(np.isnan(g) & np.isnan(e))
+            bad &= ~(np.isinf(g) & (g == e))
             ok, msg = not bad.any(), "%d of %d elements outside rtol 1e-5 + conditioning slack" % (bad.sum(), bad.size)
         else:
             ok, msg = harness.compare(g, e, d.dtype)
         print("  %s %s %s: %s" % (kernel.family, d.name, d.dtype, msg), flush=True)
         assert ok, "seed %d (%s) output %s: %s" % (seed, " ".join(notes), d.name, msg)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", SEEDS)
+def test_random_description_matches_oracle_on_gpu(seed, tmp_path):
+    from test_gpu_parity import run_on_gpu
+    text, notes = random_description(seed)
+    desc, path = _write(tmp_path, text)
+    print("seed %d: %s" % (seed, " ".join(notes)), flush=True)
+    kernel = driver.HipKernel(text, out_dir=None)
+    inputs = harness.make_inputs(desc, seed=seed)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    compare_with_oracle(kernel, desc, notes, inputs, got, expect, seed)
 
 
 MATMUL_SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_MATMULS", "40"))))
@@ -117,3 +129,41 @@ def test_random_matmul_description_matches_oracle_on_gpu(seed, tmp_path):
         ok, msg = harness.compare(g, e, d.dtype)
         print("  %s %s %s: %s" % (kernel.family, d.name, d.dtype, msg), flush=True)
         assert ok, "seed %d (%s) output %s: %s" % (seed, " ".join(notes), d.name, msg)
+
+
+OPTABLE_SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_OPTABLE", "40"))))
+
+
+@pytest.mark.parametrize("seed", OPTABLE_SEEDS[:16])
+def test_random_optable_description_compiles_and_oracles_agree(seed, tmp_path):
+    text, notes = random_optable_description(seed)
+    desc, path = _write(tmp_path, text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family in ("elementwise", "row_reduce", "stream_reduce", "staged"), notes
+    inputs = harness.make_inputs(desc, seed=seed)
+    c_out = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    n_out = np_ref.evaluate(desc, inputs)
+    for d, a, b in zip(desc["output_desc"], c_out, n_out):
+        if d["data_type"] == "float32":
+            # libm against numpy's vectorised float32 functions: an ulp or two of values of the operands' magnitude
+            with np.errstate(invalid="ignore"):
+                bad = np.abs(a.astype(np.float64) - b.astype(np.float64)) > 1e-5 * np.abs(b) + 4e-6
+            bad &= ~(np.isnan(a) & np.isnan(b)) & ~(np.isinf(a) & (a == b))
+            ok, msg = not bad.any(), "%d of %d elements apart" % (bad.sum(), bad.size)
+        else:
+            ok, msg = harness.compare(a, b, d["data_type"])
+        assert ok, "seed %d %s (%s): %s" % (seed, d["tensor_name"], " ".join(notes), msg)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", OPTABLE_SEEDS)
+def test_random_optable_description_matches_oracle_on_gpu(seed, tmp_path):
+    from test_gpu_parity import run_on_gpu
+    text, notes = random_optable_description(seed)
+    desc, path = _write(tmp_path, text)
+    print("seed %d: %s" % (seed, " ".join(notes)), flush=True)
+    kernel = driver.HipKernel(text, out_dir=None)
+    inputs = harness.make_inputs(desc, seed=seed)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    compare_with_oracle(kernel, desc, notes, inputs, got, expect, seed)
