@@ -71,7 +71,7 @@ class GemmEmitter {
         const int64_t partRows = std::min<int64_t>(m_, 256);
         k.workspaceBytes = static_cast<uint64_t>((gridTiles * 4 + 255) / 256 * 256 + tiles * kSplit_ * partRows * 256 * 4);
       }
-      k.block[0] = static_cast<unsigned>(wavesM() * 2 * 64);
+      k.block[0] = 512;
     }
     k.grid[1] = static_cast<unsigned>(batch_);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
@@ -86,8 +86,7 @@ class GemmEmitter {
     } else if (skinny_) {
       note << " skinny: strips of 128 columns, B straight into MFMA operands, mfma=" << mfmaName() << " waves=4 grid=" << k.grid[0];
     } else {
-      note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=" << wavesM() << "x2 grid="
-           << k.grid[0];
+      note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=4x2 grid=" << k.grid[0];
     }
     if (kSplit_ > 1) note << " k_splits=" << kSplit_;
     k.scheduleNote = note.str();
@@ -122,12 +121,7 @@ class GemmEmitter {
     return elem_ == DType::I8 ? "i32_32x32x32_i8" : (elem_ == DType::BF16 ? "f32_32x32x16_bf16" : "f32_32x32x16_f16");
   }
   std::string accType() const { return serial_ ? computeTypeName(g_.tensor(accId_).dtype) : (elem_ == DType::I8 ? "int" : "float"); }
-  // The tuning variants exist for the 8-bit kernel only; 16-bit operands always use 4 x 2 wavefronts and 128-byte steps.
-  // Wavefront grid of the workgroup: 4 x 2 (two wavefronts per SIMD) by default, 2 x 2 with AKG_HIP_VARIANT=1.
-  int wavesM() const { return (opt_.variant & 1) ? 2 : 4; }
-  // Bytes of K in one step: 128 by default, 64 with bit 1 of AKG_HIP_VARIANT set.
-  int stepK() const { return (elem_ == DType::I8 && (opt_.variant & 2)) ? 64 : 128; }
-  bool splitDuty() const { return (opt_.variant & 4) != 0 && wavesM() == 4; }
+  int stepK() const { return 128; }   // bytes of K in one step of the tile kernel
 
   // Few tiles and a long K (a skinny activation in front of a big weight matrix: M = 16 .. 1024 against 8192 x 8192
   // leaves 32 .. 128 of 256 CUs busy, and the time is that of streaming the weights through those few): split K over
@@ -415,7 +409,7 @@ class GemmEmitter {
     src_ << "  AKG_DEV void apply(const " << accType() << " (&acc)[" << W << "], long row, long col) {\n"
          << "    const long grow = row0 + row;\n    (void)grow;\n" << apply_.str() << "  }\n";
     src_ << "};\n}  // namespace\n\n";
-    src_ << "extern \"C\" __global__ __launch_bounds__(" << (serial_ ? 256 : (skinny_ ? skinnyWaves() * 64 : wavesM() * 128)) << ") void " << kname << "(";
+    src_ << "extern \"C\" __global__ __launch_bounds__(" << (serial_ ? 256 : (skinny_ ? skinnyWaves() * 64 : 512)) << ") void " << kname << "(";
     size_t argc = 0;
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
@@ -446,8 +440,7 @@ class GemmEmitter {
       return;
     }
     src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ", " << wavesM() << ", " << stepK() << ", " << (splitDuty() ? "true" : "false") << ", Epilogue, " << kSplit_
-         << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
+         << ", Epilogue, " << kSplit_ << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
          << " + akg_batch * " << k_ * n_ << "L, epi" << (kSplit_ > 1 ? ", akg_ws" : "") << ");\n}\n";
   }
 };

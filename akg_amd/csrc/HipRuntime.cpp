@@ -15,6 +15,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <fstream>
 #include <map>
 #include <memory>
@@ -50,8 +51,15 @@ struct akg_hip_kernel {
     hipFunction_t function = nullptr;
     std::vector<hipFunction_t> earlier;  // lowered.earlierPhases, in their order
     void *workspace = nullptr;  // lowered.workspaceBytes of zero-filled device memory, or NULL
+    // Launches of one handle share its workspace. They are ordered on the device by the library: a launch that goes to
+    // another stream than the last one first waits (through this event) for what that stream holds.
+    hipEvent_t lastUse = nullptr;
+    hipStream_t lastStream = nullptr;
+    bool used = false;
+    // a launch sequence that failed half way may have left arrival counters set: zero-fill before the next launch
+    bool dirty = false;
   };
-  std::vector<Loaded> loaded;
+  std::deque<Loaded> loaded;   // (a deque: launches keep pointers to their entry while other devices are added)
   // A description run as a sequence of kernels (Staging.h): each stage is a handle of its own; this handle owns
   // them and the temporaries between them (its workspace), and has no code object itself.
   struct Stage {
@@ -530,14 +538,14 @@ int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t 
 }
 
 // Code object and workspace of `k` on the current device, loaded / allocated on first use.
-int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
+int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded **out) {
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipGetDevice: " + hipErr(e));
   std::lock_guard<std::mutex> lock(k->mu);
-  for (const auto &l : k->loaded) {
+  for (auto &l : k->loaded) {
     if (l.device == device) {
-      *out = l;
+      *out = &l;
       return AKG_HIP_OK;
     }
   }
@@ -545,7 +553,7 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
   l.device = device;
   if (!k->stages.empty()) {
     for (auto &st : k->stages) {
-      akg_hip_kernel::Loaded ls;
+      akg_hip_kernel::Loaded *ls = nullptr;
       const int rc = ensureLoaded(st.kernel, &ls);
       if (rc != AKG_HIP_OK) return rc;
     }
@@ -575,6 +583,7 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
     // the fill runs on the null stream and may still be in flight when hipMemset returns; the first launch may go to
     // a stream that does not wait for the null stream
     if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&l.lastUse, hipEventDisableTiming);
     if (e != hipSuccess) {
       if (l.workspace) (void)hipFree(l.workspace);
       if (l.module) (void)hipModuleUnload(l.module);
@@ -582,7 +591,7 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded *out) {
     }
   }
   k->loaded.push_back(l);
-  *out = l;
+  *out = &k->loaded.back();
   return AKG_HIP_OK;
 }
 
@@ -590,6 +599,7 @@ void destroyKernel(akg_hip_kernel *kernel) {
   if (kernel == nullptr) return;
   for (auto &st : kernel->stages) destroyKernel(st.kernel);
   for (auto &l : kernel->loaded) {
+    if (l.lastUse) (void)hipEventDestroy(l.lastUse);
     if (l.workspace) (void)hipFree(l.workspace);
     if (l.module) (void)hipModuleUnload(l.module);
   }
@@ -615,32 +625,103 @@ uint64_t scratchBytesNeeded(const akg_hip_kernel *k) {
 }
 
 // Code object of `k` (and of its stages) on `device`, if it has been loaded there; loads nothing.
-bool findLoaded(akg_hip_kernel *k, int device, akg_hip_kernel::Loaded *out) {
+bool findLoaded(akg_hip_kernel *k, int device, akg_hip_kernel::Loaded **out) {
   for (auto &st : k->stages) {
-    akg_hip_kernel::Loaded ls;
+    akg_hip_kernel::Loaded *ls = nullptr;
     if (!findLoaded(st.kernel, device, &ls)) return false;
   }
   std::lock_guard<std::mutex> lock(k->mu);
-  for (const auto &l : k->loaded) {
+  for (auto &l : k->loaded) {
     if (l.device == device) {
-      *out = l;
+      *out = &l;
       return true;
     }
   }
   return false;
 }
 
+// Orders a launch that uses the handle's own workspace behind the handle's previous launch when that went to another
+// stream, and zero-fills the workspace first if an earlier launch sequence broke off. Nothing of this is recorded into a
+// stream capture (a captured launch is ordered by the graph it becomes part of).
+struct WorkspaceTurn {
+  akg_hip_kernel *k;
+  akg_hip_kernel::Loaded *l;
+  hipStream_t stream;
+  bool active = false;      // the launch uses the handle's workspace and the stream is not capturing
+  std::unique_lock<std::mutex> lock;
+  WorkspaceTurn(akg_hip_kernel *kernel, akg_hip_kernel::Loaded *loaded, hipStream_t s, bool usesOwnWorkspace)
+      : k(kernel), l(loaded), stream(s) {
+    if (!usesOwnWorkspace || l->workspace == nullptr) return;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) (void)hipGetLastError();
+    if (status != hipStreamCaptureStatusNone) return;
+    lock = std::unique_lock<std::mutex>(k->mu);
+    active = true;
+  }
+  int begin() {
+    if (!active) return AKG_HIP_OK;
+    if (l->used && l->lastStream != stream) {
+      // The event is recorded only now, at the switch of streams, behind everything enqueued on the previous stream so
+      // far (an event after every launch would put a marker between back-to-back launches of the common one-stream
+      // caller: 3 us on a 45 us reduction).
+      hipStreamCaptureStatus prev = hipStreamCaptureStatusNone;
+      hipError_t e = hipStreamIsCapturing(l->lastStream, &prev);
+      if (e == hipSuccess && prev != hipStreamCaptureStatusNone) {
+        return fail(AKG_HIP_ERR_RUNTIME, "kernel " + k->graph.name + ": its previous launch went to a stream that is being "
+                                         "captured now; launches of one handle share its workspace and cannot be ordered across that");
+      }
+      if (e == hipSuccess) e = hipEventRecord(l->lastUse, l->lastStream);
+      if (e == hipSuccess) {
+        e = hipStreamWaitEvent(stream, l->lastUse, 0);
+        if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipStreamWaitEvent: " + hipErr(e));
+      } else {
+        // the previous stream is gone (destroyed by the caller): wait for the device instead
+        (void)hipGetLastError();
+        e = hipDeviceSynchronize();
+        if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipDeviceSynchronize: " + hipErr(e));
+      }
+    }
+    if (l->dirty) {
+      const hipError_t e = hipMemsetAsync(l->workspace, 0, k->lowered.workspaceBytes, stream);
+      if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "clearing the workspace: " + hipErr(e));
+      l->dirty = false;
+    }
+    return AKG_HIP_OK;
+  }
+  int end(int rc) {
+    if (!active) return rc;
+    if (rc != AKG_HIP_OK) {
+      l->dirty = true;   // some launches of the sequence may have run: the counters cannot be trusted
+    }
+    // also after a failure: what did get enqueued still uses the workspace
+    l->lastStream = stream;
+    l->used = true;
+    return rc;
+  }
+};
+
 // Enqueues the kernel(s) of `k`. With `scratchBase` NULL the handle's own workspaces are used; otherwise the launch
 // takes its scratchBytesNeeded(k) bytes from `scratchBase` (laid out as that function says) and nothing is loaded or
 // allocated: every code object must be on the device already.
-int launchOn(akg_hip_kernel *k, const akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream,
+int launchSequence(akg_hip_kernel *k, akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream,
+                   char *scratchBase);
+
+int launchOn(akg_hip_kernel *k, akg_hip_kernel::Loaded *l, void *const *devicePtrs, hipStream_t stream,
              char *scratchBase = nullptr) {
+  WorkspaceTurn turn(k, l, stream, scratchBase == nullptr);
+  int rc = turn.begin();
+  if (rc == AKG_HIP_OK) rc = launchSequence(k, *l, devicePtrs, stream, scratchBase);
+  return turn.end(rc);
+}
+
+int launchSequence(akg_hip_kernel *k, akg_hip_kernel::Loaded &l, void *const *devicePtrs, hipStream_t stream,
+                   char *scratchBase) {
   void *const workspace = scratchBase != nullptr ? (k->lowered.workspaceBytes > 0 ? scratchBase : nullptr) : l.workspace;
   if (!k->stages.empty()) {
     const size_t nin = k->graph.inputs.size();
     char *stageScratch = scratchBase != nullptr ? scratchBase + alignScratch(k->lowered.workspaceBytes) : nullptr;
     for (auto &st : k->stages) {
-      akg_hip_kernel::Loaded ls;
+      akg_hip_kernel::Loaded *ls = nullptr;
       int rc = AKG_HIP_OK;
       if (scratchBase != nullptr) {
         if (!findLoaded(st.kernel, l.device, &ls)) return fail(AKG_HIP_ERR_INTERNAL, "stage not loaded");
@@ -784,7 +865,7 @@ int akg_hip_kernel_source(const akg_hip_kernel_t *kernel, const char **source) {
 int akg_hip_launch(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_ptrs, void *stream) {
   int rc = checkPtrs(kernel, device_ptrs, n_ptrs);
   if (rc != AKG_HIP_OK) return rc;
-  akg_hip_kernel::Loaded fn;
+  akg_hip_kernel::Loaded *fn = nullptr;
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   return launchOn(kernel, fn, device_ptrs, static_cast<hipStream_t>(stream));
@@ -802,7 +883,7 @@ int akg_hip_launch_static_scratch(akg_hip_kernel_t *kernel, void *const *device_
   int device = 0;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipGetDevice: " + hipErr(e));
-  akg_hip_kernel::Loaded fn;
+  akg_hip_kernel::Loaded *fn = nullptr;
   if (!findLoaded(kernel, device, &fn)) {
     return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel " + kernel->graph.name + " is not loaded on device " +
                                                 std::to_string(device) +
@@ -828,14 +909,14 @@ int akg_hip_launch_static_scratch(akg_hip_kernel_t *kernel, void *const *device_
 
 int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel) {
   if (kernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel is NULL");
-  akg_hip_kernel::Loaded l;
+  akg_hip_kernel::Loaded *l = nullptr;
   return ensureLoaded(kernel, &l);
 }
 
 int akg_hip_run_host(akg_hip_kernel_t *kernel, void *const *host_ptrs, int n_ptrs) {
   int rc = checkPtrs(kernel, host_ptrs, n_ptrs);
   if (rc != AKG_HIP_OK) return rc;
-  akg_hip_kernel::Loaded fn;
+  akg_hip_kernel::Loaded *fn = nullptr;
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   const int n = numTensors(kernel);
@@ -889,7 +970,7 @@ int akg_hip_profile(akg_hip_kernel_t *kernel, void *const *device_ptrs, int n_pt
   if (avg_ms == nullptr || number <= 0 || repeat <= 0) {
     return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "number and repeat must be positive and avg_ms non-NULL");
   }
-  akg_hip_kernel::Loaded fn;
+  akg_hip_kernel::Loaded *fn = nullptr;
   rc = ensureLoaded(kernel, &fn);
   if (rc != AKG_HIP_OK) return rc;
   hipStream_t stream = nullptr;

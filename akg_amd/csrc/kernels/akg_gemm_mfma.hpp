@@ -8,8 +8,8 @@
  *
  * Shape of the computation (all sizes are compile-time constants of the emitted kernel):
  *   C[M,N] = A[M,K] * B[K,N]            A row-major, B row-major ([N,K] when TRANSB)
- *   workgroup tile 256 x 256, K step 128 bytes (64 optional), 4 x 2 wavefronts (2 x 2 optional)
- *   wavefront tile 64 x 128 (128 x 128) = 2 x 4 (4 x 4) MFMA tiles of 32 x 32 (16 accumulator registers each)
+ *   workgroup tile 256 x 256, K step 128 bytes, 4 x 2 wavefronts
+ *   wavefront tile 64 x 128 = 2 x 4 MFMA tiles of 32 x 32 (16 accumulator registers each)
  *
  * Data movement:
  *   global -> registers -> LDS, double buffered in LDS (one barrier per K step); the global loads of step
@@ -18,8 +18,8 @@
  *   B (not transposed) is row-major along N but the MFMA wants, per lane, 16 consecutive k of one column.
  *   Each thread therefore loads a 16(k) x 4(n) byte block as 16 dwords, transposes it in registers with
  *   v_perm_b32 (8 permutes per 4 x 4 sub-block) and writes four 16-byte k-vectors to LDS.
- *   LDS rows are 64 data bytes + 16 pad bytes: with a row pitch of 80 bytes eight consecutive rows start in
- *   eight different 16-byte bank groups, so the ds_read_b128 fragment loads are conflict free.
+ *   LDS rows are 128 data bytes + 16 pad bytes: with a row pitch of 144 bytes consecutive rows start in
+ *   different 16-byte bank groups, and the ds_read_b128 fragment loads are conflict free (SQ_LDS_BANK_CONFLICT reads 0).
  *   LDS row r of the B tile holds global column 4 * (r % 64) + r / 64 of the tile. A wavefront's four column
  *   tiles are r / 64 = 0..3 with the same r % 64 range, so each lane ends up owning 4 ADJACENT output columns:
  *   the epilogue works on 4-element chunks and a wavefront stores 256 contiguous bytes per output row.
@@ -63,12 +63,6 @@ struct MmaF16 {
   }
 };
 
-#ifdef AKG_GEMM_STRICT_ORDER
-#define AKG_GEMM_PIN __builtin_amdgcn_sched_barrier(0)
-#else
-#define AKG_GEMM_PIN
-#endif
-
 constexpr int kGemmBM = 256;
 constexpr int kGemmBN = 256;
 constexpr int kGemmXcds = 8;
@@ -95,19 +89,13 @@ AKG_DEV void transpose4x4_bytes(const u32 (&r)[4], u32 (&t)[4]) {
 AKG_DEV u32 pack_lo16(u32 x, u32 y) { return __builtin_amdgcn_perm(y, x, 0x05040100u); }
 AKG_DEV u32 pack_hi16(u32 x, u32 y) { return __builtin_amdgcn_perm(y, x, 0x07060302u); }
 
-// WAVES_M x 2 wavefronts per workgroup: 2 x 2 (one wavefront per SIMD, 128 x 128 per wavefront, 256 accumulator
-// registers) or 4 x 2 (two wavefronts per SIMD, 64 x 128 per wavefront, 128 accumulator registers: the second
-// wavefront's MFMAs cover the first one's loads, transposes and barriers).
-// BK = BYTES of K in one step: 64 or 128. With 128 every row of A contributes one full 128-byte cache line per step
-// (with 64 each line is fetched from L2 twice), there are half as many barriers, and LDS holds 2 x 72 KiB.
 // KE is the K extent in elements; everything below counts K in bytes (K = KE * element size).
 // KSPLIT > 1 (few tiles, long K: a skinny A in front of a big weight matrix) gives every tile to KSPLIT workgroups,
 // each with a contiguous range of K steps; they leave their accumulators in the workspace `ws` (one arrival counter per
 // tile, then kPartRows x 256 accumulators per tile and split), and the last one to arrive adds the partials in split
 // order and runs the epilogue: deterministic, and the weight matrix is still read exactly once. The launch has
 // KSPLIT times the workgroups; the counters are left at zero.
-template <typename Mma, long M, long N, long KE, bool TRANSB, int WAVES_M, int BK, bool SPLIT, typename Epilogue,
-          int KSPLIT = 1>
+template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1>
 AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi,
                           unsigned *__restrict__ ws = nullptr) {
   constexpr int EB = Mma::kElemBytes;
@@ -115,15 +103,16 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   constexpr long NB = N * EB;    // bytes per k-row of a row-major B
   static_assert(K % 16 == 0, "K must be a multiple of 16 bytes");
   static_assert(TRANSB || (N % 4 == 0), "N must be a multiple of 4");
-  static_assert(WAVES_M == 2 || WAVES_M == 4, "2 x 2 or 4 x 2 wavefronts");
-  static_assert(BK == 64 || BK == 128, "K step of 64 or 128");
-  static_assert(!SPLIT || WAVES_M == 4, "split staging duty needs 8 wavefronts");
-  // Staging (global -> registers -> LDS) is done either by every thread for both operands (uniform control flow:
-  // the whole K step is one basic block, so loads, transposes and LDS writes interleave with the MFMAs), or, with
-  // SPLIT, by wavefronts 0..3 for B and 4..7 for A (fewer, longer bursts per wavefront).
-  constexpr bool kSplitDuty = SPLIT;
+  // 4 x 2 wavefronts (two per SIMD: one's MFMAs cover the other's loads, transposes and waits), 128 bytes of K per step
+  // (every row of A contributes one whole cache line, half as many barriers as with 64; LDS holds 2 x 72 KiB).
+  // Staging (global -> registers -> LDS) is done by every thread for both operands: uniform control flow, so the whole
+  // K step is one basic block and loads, transposes and LDS writes interleave with the MFMAs. (Measured and dropped:
+  // 2 x 2 wavefronts of 128 x 128 each, 64-byte steps, staging split between two groups of wavefronts, 256 x 128 tiles
+  // with two workgroups per CU.)
+  constexpr int WAVES_M = 4;
+  constexpr int BK = 128;
   constexpr int kThreads = WAVES_M * 128;
-  constexpr int kStageThreads = kSplitDuty ? 256 : kThreads;  // threads that share one operand tile
+  constexpr int kStageThreads = kThreads;             // threads that share one operand tile
   constexpr int kPitch = BK + 16;                     // LDS row: BK data bytes + 16 pad (odd multiple of 16)
   constexpr int kSub = BK / 32;                       // MFMA k-substeps per step (2 or 4)
   constexpr int kChunksPerRow = BK / 16;              // 16-byte chunks per row of a K-contiguous operand tile
@@ -181,16 +170,14 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 
   // ---- staging registers: the tile of step s+1 travels memory -> registers during step s-1.. s and is written to
   // LDS at the top of step s.
-  // Uniform duty: every thread stages its share of A (x) and of B (y).
-  // Split duty:   wavefronts 0..3 stage all of B, wavefronts 4..7 all of A, both in x.
+  // Every thread stages its share of A (x) and of B (y).
   struct Stage {
     v4i x[kRowChunks];
-    v4i y[kSplitDuty ? 1 : kRowChunks];
+    v4i y[kRowChunks];
   };
   Stage stage;
 
-  const int ltid = kSplitDuty ? (tid & 255) : tid;
-  const bool stageA = !kSplitDuty || tid >= 256;
+  const int ltid = tid;
   const int aRow = ltid / kChunksPerRow;   // + kRowStep * i
   const int aChunk = ltid % kChunksPerRow;
   const int bN4 = ltid & 63;
@@ -243,21 +230,11 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   };
   auto loadGlobal = [&](long step, Stage &st) {
     const long k0 = (stepBase + step) * BK;
-    if constexpr (kSplitDuty) {
-      if (stageA) {
-        loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
-      } else if constexpr (TRANSB) {
-        loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.x);
-      } else {
-        loadBlock(k0, st.x);
-      }
+    loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
+    if constexpr (TRANSB) {
+      loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.y);
     } else {
-      loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
-      if constexpr (TRANSB) {
-        loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.y);
-      } else {
-        loadBlock(k0, st.y);
-      }
+      loadBlock(k0, st.y);
     }
   };
 
@@ -277,9 +254,9 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   };
   auto storeBlockB16 = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
     // 16-bit elements: src[g] = k-rows 2g, 2g+1, each as (columns 0 1 | columns 2 3). A column's 8 consecutive k
-    // (16 bytes) are gathered two at a time with v_perm_b32; a thread holds 8 k-rows (4 x 2 wavefronts) or 16 (2 x 2).
-    static_assert(EB != 2 || kRowChunks == 4 || kRowChunks == 8, "16-bit staging is written for 8 or 16 k-rows per thread");
-    if constexpr (EB == 2 && (kRowChunks == 4 || kRowChunks == 8)) {
+    // (16 bytes) are gathered two at a time with v_perm_b32; a thread holds 8 k-rows.
+    static_assert(kRowChunks == 4, "the staging is written for four 16-byte chunks per thread and operand");
+    if constexpr (EB == 2) {
 #pragma unroll
       for (int h = 0; h < kRowChunks / 4; ++h) {
         v4i w[4];
@@ -308,14 +285,6 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
                            static_cast<u32>(src[g][3])};
       transpose4x4_bytes(rows, t[g]);
     }
-    if constexpr (kRowChunks == 2) {
-      typedef int v2i __attribute__((ext_vector_type(2)));
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const v2i w = {static_cast<int>(t[0][j]), static_cast<int>(t[1][j])};
-        *reinterpret_cast<v2i *>(lb + (j * 64 + bN4) * kPitch + bKq * kBlockRows) = w;
-      }
-    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -339,21 +308,11 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   auto storeLds = [&](int buf, const Stage &st) {
     u8 *la = lds[buf][0];
     u8 *lb = lds[buf][1];
-    if constexpr (kSplitDuty) {
-      if (stageA) {
-        storeRowsA(la, st.x);
-      } else if constexpr (TRANSB) {
-        storeRowsBt(lb, st.x);
-      } else {
-        storeBlockB(lb, st.x);
-      }
+    storeRowsA(la, st.x);
+    if constexpr (TRANSB) {
+      storeRowsBt(lb, st.y);
     } else {
-      storeRowsA(la, st.x);
-      if constexpr (TRANSB) {
-        storeRowsBt(lb, st.y);
-      } else {
-        storeBlockB(lb, st.y);
-      }
+      storeBlockB(lb, st.y);
     }
   };
 
@@ -377,7 +336,6 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   };
   auto mfmaAll = [&](const v4i (&af)[kTM], const v4i (&bf)[4]) {
     if (!kAllRowsReal && !waveHasRows) return;
-#ifndef AKG_DIAG_NO_MFMA
 #pragma unroll
     for (int i = 0; i < kTM; ++i) {
 #pragma unroll
@@ -385,7 +343,6 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
         acc[i][j] = Mma::mma(af[i], bf[j], acc[i][j]);
       }
     }
-#endif
   };
 
   // ---- main loop. Invariant at the top of step s: LDS buffer s&1 holds tile s (complete), the staging registers hold
@@ -407,12 +364,8 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     // The staged tile goes to the other LDS buffer at the very top of the step (its last readers finished before
     // the previous step's barrier), and the freed staging registers are refilled at once: the LDS writes complete
     // and the global loads travel while the step's MFMAs run, instead of piling up in front of the barrier.
-#ifndef AKG_DIAG_NO_LDS_STORE
     if constexpr (kStore) storeLds(buf ^ 1, stage);
-#endif
-#ifndef AKG_DIAG_NO_GLOBAL_LOAD
     if constexpr (kLoad) loadGlobal(step + 2, stage);
-#endif
 #pragma unroll
     for (int ks = 0; ks + 2 < kSub; ks += 2) {
       readFrags(buf, ks + 1, f1a, f1b);
@@ -423,9 +376,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     if constexpr (kSub > 2) __builtin_amdgcn_sched_barrier(0);  // keep the staging work in the early substeps
     readFrags(buf, kSub - 1, f1a, f1b);
     mfmaAll(f0a, f0b);
-#ifndef AKG_DIAG_NO_BARRIER
     __syncthreads();
-#endif
     // ---- after the barrier: MFMAs on the last fragments of this tile; meanwhile fetch the first fragments of the next
     if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
     mfmaAll(f1a, f1b);

@@ -522,6 +522,41 @@ def test_reference_repository_descriptions_match_oracle(name):
         assert ok, "%s output %s: %s" % (name, d.name, msg)
 
 
+@pytest.mark.parametrize("shape,axes,split", [([8192, 1024], [0], 64), ([2048, 4096], [0, 1], 128), ([64, 32, 4096], [0, 2], 32)])
+def test_workspace_launches_from_two_streams_are_ordered_and_repeat_bit_for_bit(shape, axes, split, monkeypatch):
+    """Many workgroups per output group (the split is forced up) leave partial results and arrival counters in the
+    handle's workspace; the last one to arrive finishes in slot order. 300 launches of ONE handle, alternating between
+    two streams with no host synchronisation in between, each into an output buffer of its own: the library orders
+    them on the device (they share the workspace), and every result must equal the first bit for bit - a lost
+    partial, a counter left set or two launches inside the workspace at once would show as a different sum."""
+    import torch
+    monkeypatch.setenv("AKG_HIP_SPLIT", str(split))
+    name = "ws_order_%s_%s" % ("x".join(map(str, shape)), "".join(map(str, axes)))
+    text = op_desc.square_reduce(shape, axes, "float32", False, "ReduceSum", name)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family == "stream_reduce" and kernel.workspace_bytes > 0
+    print("case %s grid %d workspace %d" % (name, kernel.grid[0], kernel.workspace_bytes), flush=True)
+    desc = json_loads(text)
+    x = harness.make_inputs(desc, seed=harness.BASE_SEED + 99)[0]
+    dev = torch.device("cuda:0")
+    xin = torch.from_numpy(x).to(dev)
+    launches = 300
+    nbytes = kernel.outputs[0].nbytes
+    outs = torch.full((launches, nbytes), 0xFF, dtype=torch.uint8, device=dev)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for i in range(launches):
+        kernel.launch_ptrs([xin.data_ptr(), outs[i].data_ptr()], streams[i % 2].cuda_stream)
+    torch.cuda.synchronize()
+    host = outs.cpu().numpy()
+    for i in range(1, launches):
+        assert np.array_equal(host[i], host[0]), "launch %d differs from launch 0" % i
+    got = host[0].view(np.float32).reshape(kernel.outputs[0].shape)
+    exact = np.sum(x.astype(np.float64) ** 2, axis=tuple(axes))
+    ok, msg = harness.compare_reassociated(got, exact, "float32", int(np.prod(shape)) // max(1, got.size))
+    assert ok, msg
+
+
 def check_segment_sum(path, seed, repeats=2):
     """UnsortedSegmentSum keeps the serial order of the additions per output element: bit-exact against the oracle,
     float types included, and on every launch (nothing may be left over from the one before)."""
