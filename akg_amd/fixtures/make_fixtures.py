@@ -22,6 +22,11 @@ FIXTURES = {
     "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": lambda n: op_desc.gemm_int8_dequant_bias_gelu(4096, 8192, 8192, "bfloat16", False, n),
     # plain streaming kernel of known size, used to calibrate the HBM traffic counters
     "calib_neg_f32_16384x4096": lambda n: _neg(16384, 4096, n),
+    # streaming kernels with next to no arithmetic, of exactly the tensor sizes of c1 (3 reads + 1 write) and c2 (1 + 1)
+    "calib_add3_f32_1024x4096": lambda n: _add3(1024, 4096, n),
+    "calib_neg_f16_8192x4096": lambda n: _neg(8192, 4096, n, "float16"),
+    # the sample of c5 the CPU baseline runs: 64 of the 4096 rows of A against the whole of B
+    "c5_mslice64_gemm_i8_dequant_bias_gelu_64x8192x8192": lambda n: op_desc.gemm_int8_dequant_bias_gelu(64, 8192, 8192, "bfloat16", False, n),
     # small parity cases
     "small_ew_tanh_add_mul_f32_8x128": lambda n: op_desc.elementwise_tanh_add_mul(8, 128, n),
     "small_ew_tanh_add_mul_f32_7x33": lambda n: op_desc.elementwise_tanh_add_mul(7, 33, n),
@@ -146,10 +151,16 @@ FIXTURES = {
 }
 
 
-def _neg(rows, cols, name):
+def _neg(rows, cols, name, dtype="float32"):
     b = op_desc.DescBuilder(name)
-    x = b.input([rows, cols], "float32")
+    x = b.input([rows, cols], dtype)
     return b.dumps([b.unary("Neg", x)])
+
+
+def _add3(rows, cols, name):
+    b = op_desc.DescBuilder(name)
+    x, y, z = [b.input([rows, cols], "float32") for _ in range(3)]
+    return b.dumps([b.add(b.add(x, y), z)])
 
 
 def main():

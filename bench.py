@@ -2,20 +2,32 @@
 """Benchmark of the fused-operator hot path on one MI355X.
 
 A "step" is one launch of the fused kernel of one op description through the C ABI (akg_hip_launch) on buffers that
-are already resident in HBM. The headline workload is the fused softmax fp16 [8192,4096]; the other measured
-configurations are reported in `per_config`. Inputs are synthetic (seeded); several distinct buffer sets are rotated so
-that a launch reads from HBM and not from the 256 MB last-level cache.
+are already resident in HBM. The headline workload is the fused softmax fp16 [8192,4096]; every measured configuration
+is reported under `per_config`. Inputs are synthetic (seeded); several distinct buffer sets are rotated so that a launch
+reads from HBM and not from the 256 MB last-level cache.
 
 Prints ONE JSON line:
   value / ms_per_step  host-clock throughput of K back-to-back steps (algorithmic bytes / wall time)
-  roofline             achieved = algorithmic bytes per launch / mean launch duration from HIP events recorded on the
-                       launch stream around the same K launches; peak = 8 TB/s HBM3E (or the dense int8 MFMA peak)
-  cpu_baseline         the CPU oracle (C restatement of the reference CPU pipeline, 1 thread, like the reference's
-                       default) timed on this host on the same workload
+  roofline             achieved = algorithmic bytes (or ops) per launch / mean launch duration from HIP events recorded
+                       on the launch stream around the same K launches; peak = 8 TB/s HBM3E (or the dense MFMA peak);
+                       traffic = HBM bytes per launch as the rocprofv3 summary under profiles/ holds them (null if the
+                       summary is missing)
+  cpu_baseline         the CPU oracle (C restatement of the reference CPU pipeline, 1 thread like the reference's
+                       default, and its OpenMP build on all host cores) timed on this host on a bounded sample
+  per_config           the same roofline object per workload, with kernel_ms (mean of the K launches), kernel_ms_median
+                       and kernel_ms_min (over groups of 10 launches), a cache-resident figure for the two configurations
+                       that fit the last-level cache, and a cpu_baseline for each of the five measured configurations
+  calibration          what the box itself allows, measured in the same run: streaming kernels of exactly the sizes of
+                       C1 and C2 (this backend's own minimal kernels and the vendor's device-to-device copy), register-only
+                       MFMA loops on zero and on random operands (the part is power limited), and the vendor library's
+                       GEMM on the shapes of C5 and N2
 """
 import argparse
+import ctypes
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
@@ -23,6 +35,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 FIXTURES = os.path.join(ROOT, "akg_amd", "fixtures")
+PROFILES = os.path.join(ROOT, "profiles")
+PROBE_LIB = os.path.join(ROOT, "akg_amd", "libakg_bench_probe.so")
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published (no sparsity)
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published (no sparsity)
@@ -50,35 +64,88 @@ WORKLOADS = {
 DEFAULT_WORKLOAD = "c2_softmax_f16_8192x4096"
 # plain streaming kernel of known size (out = -x, 256 MiB in + 256 MiB out): calibrates the HBM traffic counters
 CALIBRATION = "calib_neg_f32_16384x4096"
-
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; scaled by the same counters' reading
-# for a plain copy of known size: FETCH_SIZE reads half the bytes, scale 2.0; WRITE_SIZE scale 1.0). Values are the
-# ones of the summaries under profiles/; None = not measured yet.
-CLOCK_RAMP_MS = 120.0
-MEASURED_TRAFFIC_BYTES = {
-    "c1_ew_tanh_add_mul_f32_1024x4096": 67142582,
-    "c2_softmax_f16_8192x4096": 134243913,
-    "c3_layernorm_residual_bf16_16384x4096": 402797563,
-    "c4_quant_int8_residual_bf16_32768x8192": 1343173505,
-    "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": 470254548,
-    "n1_biasgrad_bf16_16384x4096": 270924759,
-    "n2_gemm_bf16_bias_gelu_4096x8192x8192": 872910920,
-    "n3_transpose_bias_add_bf16_32x2048x1024": 268462651,
-    "n4_softmax_f16_512x131072": 268593234,
-    "n5_bnstats_bf16_256x64x56x56": 102898801,
-    "n6_gemm_bf16_bias_gelu_16x8192x8192": 140865236,
-    "n7_segment_sum_f32_4954x4953_by_1x3_seg4954": 2127240577,
+# streaming kernels with next to no arithmetic, of exactly the tensor sizes of C1 (3 reads + 1 write of 16 MiB) and C2
+# (1 read + 1 write of 64 MiB): what a kernel of that size can reach on this box
+SIZE_MATCHED = {"calib_add3_f32_1024x4096": "c1_ew_tanh_add_mul_f32_1024x4096",
+                "calib_neg_f16_8192x4096": "c2_softmax_f16_8192x4096"}
+# bounded CPU samples: the description the CPU leg runs, and how it relates to the workload
+CPU_SAMPLES = {
+    "c1_ew_tanh_add_mul_f32_1024x4096": ("c1_ew_tanh_add_mul_f32_1024x4096", "the full workload", 1.0),
+    "c2_softmax_f16_8192x4096": ("c2_softmax_f16_8192x4096", "the full workload", 1.0),
+    "c3_layernorm_residual_bf16_16384x4096": ("c3_layernorm_residual_bf16_16384x4096", "the full workload", 1.0),
+    "c4_quant_int8_residual_bf16_32768x8192": ("c4_quant_int8_residual_bf16_32768x8192", "the full workload", 1.0),
+    "c5_gemm_i8_dequant_bias_gelu_4096x8192x8192": ("c5_mslice64_gemm_i8_dequant_bias_gelu_64x8192x8192",
+                                                    "an M-slice of 64 of the 4096 rows of A (1/64 of the ops, the whole of B)", 1.0 / 64),
 }
+CACHE_RESIDENT = ("c1_ew_tanh_add_mul_f32_1024x4096", "c2_softmax_f16_8192x4096")
+CLOCK_RAMP_MS = 120.0
+GROUP = 10   # launches per timed group of the median / min pass
 
 
-def gpu_measure(name, steps, warmup, torch, driver, harness, np):
+def traffic_from_profile(name):
+    """HBM bytes per launch from the rocprofv3 summary of this workload (profiles/<name>.md), or None."""
+    try:
+        with open(os.path.join(PROFILES, name + ".md"), "r", encoding="utf-8") as f:
+            m = re.search(r"Traffic per launch = (\d+) bytes", f.read())
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
+def ramp(launch, torch):
+    """An idle MI355X sits at a few hundred MHz and needs some tens of milliseconds of sustained work to reach its
+    steady clocks (the first ~15 ms of launches after idle run 10-25 % slower). The figures reported are steady-state
+    ones, so the device is kept busy for CLOCK_RAMP_MS before the warm-up steps."""
+    t_ramp = time.perf_counter()
+    i = 0
+    while (time.perf_counter() - t_ramp) * 1e3 < CLOCK_RAMP_MS:
+        for _ in range(16):
+            launch(i)
+            i += 1
+        torch.cuda.synchronize()
+
+
+def timed(launch, steps, warmup, torch, groups=True):
+    """(wall ms, mean event ms, median ms, min ms) per step of `launch(i)`. The K steps of the contract are one region
+    bracketed by two events on the launch stream; median and min come from a second pass in groups of GROUP launches."""
+    stream = torch.cuda.current_stream()
+    ramp(launch, torch)
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for i in range(steps):
+        launch(i)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    wall_ms = (t1 - t0) * 1e3 / steps
+    mean_ms = e0.elapsed_time(e1) / steps
+    if not groups:
+        return wall_ms, mean_ms, None, None
+    n_groups = max(3, steps // GROUP)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(n_groups + 1)]
+    marks[0].record(stream)
+    for g in range(n_groups):
+        for i in range(GROUP):
+            launch(g * GROUP + i)
+        marks[g + 1].record(stream)
+    torch.cuda.synchronize()
+    per = [marks[g].elapsed_time(marks[g + 1]) / GROUP for g in range(n_groups)]
+    return wall_ms, mean_ms, statistics.median(per), min(per)
+
+
+def gpu_measure(name, steps, warmup, torch, driver, harness, np, resident=False):
     path = os.path.join(FIXTURES, name + ".info")
     desc = harness.load_desc(path)
     kernel = driver.HipKernel.from_file(path)
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 1)
     dev = torch.device("cuda:0")
     per_set = sum(t.nbytes for t in kernel.tensors)
-    nsets = max(2, min(12, int(1.2e9 // per_set) + 1))
+    nsets = 1 if resident else max(2, min(12, int(1.2e9 // per_set) + 1))
     sets = []
     for _ in range(nsets):
         bufs = []
@@ -89,33 +156,9 @@ def gpu_measure(name, steps, warmup, torch, driver, harness, np):
             bufs.append(b)
         sets.append(bufs)
     ptrs = [[b.data_ptr() for b in bufs] for bufs in sets]
-    stream = torch.cuda.current_stream()
-    st = stream.cuda_stream
-    # Clock ramp: an idle MI355X sits at a few hundred MHz and needs some tens of milliseconds of sustained work
-    # to reach its steady clocks (the first ~15 ms of launches after idle run 10-25 % slower). The figures reported
-    # are steady-state ones, so the device is kept busy for CLOCK_RAMP_MS before the W warm-up steps.
-    t_ramp = time.perf_counter()
-    i = 0
-    while (time.perf_counter() - t_ramp) * 1e3 < CLOCK_RAMP_MS:
-        for _ in range(16):
-            kernel.launch_ptrs(ptrs[i % nsets], st)
-            i += 1
-        torch.cuda.synchronize()
-    for i in range(warmup):
-        kernel.launch_ptrs(ptrs[i % nsets], st)
-    torch.cuda.synchronize()
-    e0 = torch.cuda.Event(enable_timing=True)
-    e1 = torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for i in range(steps):
-        kernel.launch_ptrs(ptrs[i % nsets], st)
-    e1.record(stream)
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    wall_ms = (t1 - t0) * 1e3 / steps
-    kernel_ms = e0.elapsed_time(e1) / steps
-    return kernel, inputs, wall_ms, kernel_ms, nsets
+    st = torch.cuda.current_stream().cuda_stream
+    wall_ms, mean_ms, med_ms, min_ms = timed(lambda i: kernel.launch_ptrs(ptrs[i % nsets], st), steps, warmup, torch)
+    return kernel, inputs, wall_ms, mean_ms, med_ms, min_ms, nsets
 
 
 def roofline_of(kernel, kernel_ms, name):
@@ -127,28 +170,119 @@ def roofline_of(kernel, kernel_ms, name):
         achieved = kernel.algorithmic_ops / (kernel_ms * 1e-3) / 1e12
         peak = mfma_peak
         return {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TOP/s" if int8 else "TFLOP/s",
-                "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+                "frac": round(achieved / peak, 4), "traffic": traffic_from_profile(name)}
     achieved = kernel.algorithmic_bytes / (kernel_ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(name)}
+            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic_from_profile(name)}
 
 
-def cpu_baseline(name, inputs, kernel):
-    """Time the CPU oracle (checker code; used here only as the reported CPU baseline)."""
+def cpu_baseline(name, harness, driver):
+    """Time the CPU oracle (checker code; used here only as the reported CPU baseline) on the bounded sample of `name`."""
     from oracle import cpu_ref
-    path = os.path.join(FIXTURES, name + ".info")
+    sample, what, share = CPU_SAMPLES[name]
+    path = os.path.join(FIXTURES, sample + ".info")
+    desc = harness.load_desc(path)
+    kernel = driver.HipKernel.from_file(path)       # algorithmic work of the sample, from the same accounting
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 1)
+    is_gemm = kernel.algorithmic_ops > 0
+    work = kernel.algorithmic_ops / 1e12 if is_gemm else kernel.algorithmic_bytes / 1e9
+    unit = ("TOP/s" if WORKLOADS.get(name) == "int8" else "TFLOP/s") if is_gemm else "GB/s"
     serial = cpu_ref.CpuKernel(path, openmp=False)
-    # bounded sample: the full workload, called a few times (a call of the largest configuration takes seconds)
-    t = serial.time(inputs, warmup=1, iters=3)
-    out = {"value": round(kernel.algorithmic_bytes / t / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-           "sample": "full %s workload, 1 warm-up + 3 timed calls of the serial C restatement (%.3f s per call)" % (name, t)}
+    slow = is_gemm or kernel.algorithmic_bytes > 1e9
+    t = serial.time(inputs, warmup=0 if slow else 1, iters=1 if slow else 3)
+    out = {"value": round(work / t, 6 if is_gemm else 3), "unit": unit, "cores": 1, "kind": "port",
+           "sample": "%s: %s, serial C restatement, %.3f s per call%s" %
+                     (sample, what, t, "" if share == 1.0 else " (the rate is that of the slice; the full workload is %d slices)" % round(1 / share))}
     try:
         par = cpu_ref.CpuKernel(path, openmp=True)
-        tp = par.time(inputs, warmup=1, iters=3)
-        out["all_cores_value"] = round(kernel.algorithmic_bytes / tp / 1e9, 3)
+        tp = par.time(inputs, warmup=1, iters=2)
+        out["all_cores_value"] = round(work / tp, 6 if is_gemm else 3)
         out["all_cores"] = int(os.environ.get("OMP_NUM_THREADS", 0)) or (os.cpu_count() or 1)
     except Exception as e:  # the OpenMP build is optional
         out["all_cores_error"] = str(e)
+    return out
+
+
+def calibration(torch, driver, harness, np, steps, warmup):
+    """Ceilings of this box, measured in this run."""
+    out = {}
+    dev = torch.device("cuda:0")
+    # 1. streaming kernels of exactly C1's and C2's sizes: this backend's own minimal kernels ...
+    for calib, twin in SIZE_MATCHED.items():
+        try:
+            k, _, _, mean_ms, med_ms, min_ms, _ = gpu_measure(calib, steps, warmup, torch, driver, harness, np)
+            gbs = k.algorithmic_bytes / (mean_ms * 1e-3) / 1e9
+            out[calib] = {"size_of": twin, "bytes": k.algorithmic_bytes, "kernel_ms": round(mean_ms, 5),
+                          "kernel_ms_median": round(med_ms, 5), "kernel_ms_min": round(min_ms, 5),
+                          "achieved": round(gbs, 1), "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4)}
+        except Exception as e:
+            out[calib] = {"error": str(e)}
+    # ... and the vendor's device-to-device copy moving the same number of bytes (half read, half written)
+    for label, total in (("vendor_copy_64MiB_moved", 64 << 20), ("vendor_copy_128MiB_moved", 128 << 20)):
+        half = total // 2
+        nsets = max(2, int(1.2e9 // total) + 1)
+        src = [torch.randint(0, 255, (half,), dtype=torch.uint8, device=dev) for _ in range(nsets)]
+        dst = [torch.empty(half, dtype=torch.uint8, device=dev) for _ in range(nsets)]
+        _, mean_ms, med_ms, min_ms = timed(lambda i: dst[i % nsets].copy_(src[i % nsets]), steps, warmup, torch)
+        gbs = total / (mean_ms * 1e-3) / 1e9
+        out[label] = {"bytes": total, "kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5),
+                      "kernel_ms_min": round(min_ms, 5), "achieved": round(gbs, 1), "unit": "GB/s",
+                      "frac": round(gbs / HBM_PEAK_GBS, 4), "what": "torch Tensor.copy_ between two device buffers"}
+        del src, dst
+    # 2. register-only MFMA loops (no memory traffic in the loop) on zero and on random operands
+    try:
+        probe = ctypes.CDLL(PROBE_LIB)
+        vp, ci = ctypes.c_void_p, ctypes.c_int
+        for fn in (probe.akg_probe_mfma_i8, probe.akg_probe_mfma_bf16):
+            fn.argtypes = [vp, vp, ci, ci, vp]
+        rng = np.random.default_rng(7)
+        workgroups, iterations = 512, 500
+        sink = torch.empty(workgroups * 512, dtype=torch.int32, device=dev)
+        st = torch.cuda.current_stream().cuda_stream
+        operands = {
+            "mfma_i8_register_loop_zero_operands": (probe.akg_probe_mfma_i8, np.zeros(24 * 1024, np.uint8), INT8_MFMA_PEAK_TOPS, "TOP/s"),
+            "mfma_i8_register_loop_random_operands": (probe.akg_probe_mfma_i8,
+                                                      rng.integers(-127, 128, 24 * 1024, dtype=np.int8).view(np.uint8), INT8_MFMA_PEAK_TOPS, "TOP/s"),
+            "mfma_bf16_register_loop_zero_operands": (probe.akg_probe_mfma_bf16, np.zeros(24 * 1024, np.uint8), BF16_MFMA_PEAK_TFLOPS, "TFLOP/s"),
+            "mfma_bf16_register_loop_random_operands": (probe.akg_probe_mfma_bf16,
+                                                        harness.f32_to_bf16_bits((rng.standard_normal(12 * 1024) * 0.25).astype(np.float32)).view(np.uint8),
+                                                        BF16_MFMA_PEAK_TFLOPS, "TFLOP/s"),
+        }
+        ops = workgroups * 8 * iterations * 32 * 65536
+        for label, (fn, host, peak, unit) in operands.items():
+            buf = torch.from_numpy(np.ascontiguousarray(host)).to(dev)
+            _, mean_ms, med_ms, min_ms = timed(lambda i: fn(st, buf.data_ptr(), iterations, workgroups, sink.data_ptr()),
+                                               max(10, steps // 10), 2, torch)
+            rate = ops / (mean_ms * 1e-3) / 1e12
+            out[label] = {"ops": ops, "kernel_ms": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
+                          "kernel_ms_min": round(min_ms, 4), "achieved": round(rate, 1), "unit": unit, "peak": peak,
+                          "frac": round(rate / peak, 4),
+                          "what": "512 workgroups x 8 wavefronts, 2 x 4 accumulator tiles each, nothing but MFMAs on register operands"}
+    except OSError as e:
+        out["mfma_register_loops"] = {"error": str(e)}
+    # 3. the vendor library on the GEMM shapes (no epilogue: plain int32 / bf16 result)
+    try:
+        m, k, n = 4096, 8192, 8192
+        a8 = torch.randint(-127, 128, (m, k), dtype=torch.int8, device=dev)
+        b8 = torch.randint(-127, 128, (k, n), dtype=torch.int8, device=dev)
+        _, mean_ms, med_ms, min_ms = timed(lambda i: torch._int_mm(a8, b8), max(20, steps // 4), 3, torch)
+        rate = 2.0 * m * n * k / (mean_ms * 1e-3) / 1e12
+        out["vendor_int8_gemm_4096x8192x8192"] = {"kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5),
+                                                  "kernel_ms_min": round(min_ms, 5), "achieved": round(rate, 1), "unit": "TOP/s",
+                                                  "frac": round(rate / INT8_MFMA_PEAK_TOPS, 4),
+                                                  "what": "torch._int_mm, B row-major as in C5, int32 result, no epilogue, same buffers reused"}
+        del a8, b8
+        a16 = (torch.randn((m, k), device=dev) * 0.25).to(torch.bfloat16)
+        b16 = (torch.randn((k, n), device=dev) * 0.25).to(torch.bfloat16)
+        _, mean_ms, med_ms, min_ms = timed(lambda i: torch.matmul(a16, b16), max(20, steps // 4), 3, torch)
+        rate = 2.0 * m * n * k / (mean_ms * 1e-3) / 1e12
+        out["vendor_bf16_gemm_4096x8192x8192"] = {"kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5),
+                                                  "kernel_ms_min": round(min_ms, 5), "achieved": round(rate, 1), "unit": "TFLOP/s",
+                                                  "frac": round(rate / BF16_MFMA_PEAK_TFLOPS, 4),
+                                                  "what": "torch.matmul, B row-major as in N2, bf16 result, no epilogue, same buffers reused"}
+        del a16, b16
+    except Exception as e:  # a torch build without these routines
+        out["vendor_gemm"] = {"error": str(e)}
     return out
 
 
@@ -157,8 +291,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [CALIBRATION])
-    ap.add_argument("--only", action="store_true", help="measure only --workload (no per_config sweep)")
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [CALIBRATION] + sorted(SIZE_MATCHED))
+    ap.add_argument("--only", action="store_true", help="measure only --workload (no per_config sweep, no calibration)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -172,9 +306,9 @@ def main():
         sys.exit("bench.py needs a GPU")
 
     name = args.workload
-    kernel, inputs, wall_ms, kernel_ms, nsets = gpu_measure(name, args.steps, args.warmup, torch, driver, harness, np)
-    is_gemm = roofline_of(kernel, kernel_ms, name)["bound"] == "mfma"
-    if is_gemm:
+    kernel, _, wall_ms, kernel_ms, med_ms, min_ms, nsets = gpu_measure(name, args.steps, args.warmup, torch, driver, harness, np)
+    roof = roofline_of(kernel, kernel_ms, name)
+    if roof["bound"] == "mfma":
         value = kernel.algorithmic_ops / (wall_ms * 1e-3) / 1e12
         if WORKLOADS.get(name) == "int8":
             unit, metric = "TOP/s", "achieved int8 TOP/s of the fused GEMM (2*M*N*K ops per launch / time)"
@@ -190,24 +324,37 @@ def main():
         "config": {"workload": name, "family": kernel.family, "grid": kernel.grid[0], "block": kernel.block[0],
                    "algorithmic_bytes": kernel.algorithmic_bytes, "algorithmic_ops": kernel.algorithmic_ops,
                    "buffer_sets_rotated": nsets, "clock_ramp_ms": CLOCK_RAMP_MS},
-        "roofline": roofline_of(kernel, kernel_ms, name),
-        "kernel_ms": round(kernel_ms, 5),
+        "roofline": roof,
+        "kernel_ms": round(kernel_ms, 5), "kernel_ms_median": round(med_ms, 5), "kernel_ms_min": round(min_ms, 5),
     }
-    if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(name, inputs, kernel)
+    if not args.no_cpu_baseline and name in CPU_SAMPLES:
+        line["cpu_baseline"] = cpu_baseline(name, harness, driver)
     if not args.only:
         per = {}
         for other in sorted(WORKLOADS):
-            if other == name:
-                per[other] = dict(line["roofline"], kernel_ms=line["kernel_ms"])
-                continue
             try:
-                k2, _, _, kms, _ = gpu_measure(other, max(20, args.steps // 4), max(5, args.warmup // 2), torch, driver,
-                                               harness, np)
-                per[other] = dict(roofline_of(k2, kms, other), kernel_ms=round(kms, 5))
+                if other == name:
+                    k2, entry = kernel, dict(roof, kernel_ms=line["kernel_ms"], kernel_ms_median=line["kernel_ms_median"],
+                                             kernel_ms_min=line["kernel_ms_min"])
+                else:
+                    k2, _, _, kms, kmed, kmin, _ = gpu_measure(other, max(20, args.steps // 4), max(5, args.warmup // 2), torch,
+                                                               driver, harness, np)
+                    entry = dict(roofline_of(k2, kms, other), kernel_ms=round(kms, 5), kernel_ms_median=round(kmed, 5),
+                                 kernel_ms_min=round(kmin, 5))
+                if other in CACHE_RESIDENT:
+                    # the same buffers launch after launch: reads come from the 256 MB last-level cache
+                    _, _, _, rms, _, rmin, _ = gpu_measure(other, max(20, args.steps // 4), max(5, args.warmup // 2), torch,
+                                                           driver, harness, np, resident=True)
+                    r = roofline_of(k2, rms, other)
+                    entry["cache_resident"] = {"kernel_ms": round(rms, 5), "kernel_ms_min": round(rmin, 5),
+                                               "achieved": r["achieved"], "unit": r["unit"], "frac_of_hbm_peak": r["frac"]}
+                if other in CPU_SAMPLES and not args.no_cpu_baseline:
+                    entry["cpu_baseline"] = line["cpu_baseline"] if other == name else cpu_baseline(other, harness, driver)
+                per[other] = entry
             except driver.AkgHipError as e:
                 per[other] = {"error": str(e)}
         line["per_config"] = per
+        line["calibration"] = calibration(torch, driver, harness, np, max(20, args.steps // 4), max(5, args.warmup // 2))
     print(json.dumps(line))
 
 
