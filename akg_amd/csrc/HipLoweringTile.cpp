@@ -76,11 +76,13 @@ class TileEmitter {
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
     if (extentArg_) k.scalarArgs.push_back(extentIsCols_ ? cols_ : rows_);
+    if (colsArg_) k.scalarArgs.push_back(cols_);
     std::ostringstream note;
     note << kernelFamilyName(k.family) << " rows=" << rows_ << " cols=" << cols_ << " vec=" << vec_
          << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
          << " block=" << block_ << " grid=" << grid_;
     if (overlap_ > 0) note << " tail_overlap=" << overlap_;
+    if (colsArg_) note << " (row length is a kernel argument: one code object for rows of " << bucketLow_ << " .. " << bucketHigh_ << " elements)";
     if (multiPass_) note << " walks_of_groups=" << groups_ << (packedRow_ ? " (row packed in registers)" : "");
     k.scheduleNote = note.str();
     return k;
@@ -96,6 +98,13 @@ class TileEmitter {
   int64_t rows_ = 1, cols_ = 1, numel_ = 1;
   bool extentArg_ = false;     // the row count (or COLS when everything folded into one dim) is a kernel argument
   bool extentIsCols_ = false;
+  // Dynamic descriptions: the row length COLS is a second kernel argument. The schedule (threads per row, chunks per
+  // thread) is then chosen for the power-of-two bucket of chunk counts the row falls into, chunks are only
+  // element-aligned and the last one of a row starts at COLS - V (the overlap is a run-time value), so that every row
+  // length of the bucket shares the source and with it the code object.
+  bool colsArg_ = false;
+  bool allowColsArg_ = true;
+  int64_t bucketLow_ = 0, bucketHigh_ = 0;
   std::vector<InputAccess> access_;  // per graph input
   std::vector<ValInfo> vals_;        // per tensor
 
@@ -294,7 +303,20 @@ class TileEmitter {
     if ((v & (v - 1)) != 0) v = 1;
     bool inPlace = false;
     for (const OpNode &op : g_.ops) inPlace = inPlace || op.kind == OpKind::Assign;
-    if (rowMode_ && useBuffers_ && !inPlace && opt_.vec == 0 && (cols_ % v) != 0 && cols_ >= 2 * v) {
+    // the row length as an argument: row kernels whose rows hold at least two chunks (tried first, given up below if the
+    // bucket's longest row would not stay in registers), elementwise kernels with a row structure
+    colsArg_ = allowColsArg_ && extentArg_ && !extentIsCols_ && useBuffers_ && opt_.vec == 0 && opt_.threadsPerRow == 0 && opt_.chunks == 0 &&
+               (rowMode_ ? (!inPlace && cols_ >= 2 * v) : rows_ > 1);
+    int64_t schedCols = cols_;   // the row length the schedule is made for
+    if (colsArg_ && rowMode_) {
+      const int64_t bucketChunks = pow2AtLeast(static_cast<int>(std::min<int64_t>(ceilDiv(cols_, v), 1 << 20)));
+      bucketHigh_ = bucketChunks * v;
+      bucketLow_ = std::max<int64_t>(2 * v, bucketChunks / 2 * v + 1);
+      schedCols = bucketHigh_;
+    }
+    if (colsArg_ && rowMode_) {
+      // element-aligned chunks; the overlap of the last one is computed in the kernel
+    } else if (rowMode_ && useBuffers_ && !inPlace && opt_.vec == 0 && (cols_ % v) != 0 && cols_ >= 2 * v) {
       overlap_ = static_cast<int>(v - cols_ % v);
     } else {
       while (v > 1 && (cols_ % v) != 0) v >>= 1;
@@ -314,7 +336,7 @@ class TileEmitter {
       // 512 x 2 75.8; 4096-wide f32 rows 512 x 2 78.4, 1024 x 1 69.0; 768-wide bf16 LayerNorm 32 x 3 80.5, 128 x 1
       // (25 % idle) 60.3; 5120-wide 128 x 5 78.7, 1024 x 1 (37 % idle) 50.3; 11008-wide f32 softmax 1024 x 3 72.6,
       // 256 x 11 68.2.
-      const int64_t rowChunks = ceilDiv(cols_, vec_);
+      const int64_t rowChunks = ceilDiv(schedCols, vec_);
       int tpr = 0;
       if (opt_.threadsPerRow > 0) {
         tpr = pow2AtLeast(std::max(1, std::min(opt_.threadsPerRow, 1024)));
@@ -334,7 +356,7 @@ class TileEmitter {
         }
       }
       tpr_ = tpr;
-      int64_t perThread = ceilDiv(cols_, static_cast<int64_t>(tpr_) * vec_);
+      int64_t perThread = ceilDiv(schedCols, static_cast<int64_t>(tpr_) * vec_);
       // More than 64 values per thread of one row-sized input, or 96 over all of them, do not stay in registers: walk the row in groups of
       // `chunks` chunks per thread instead. The walks after the first re-read the row from HBM (rows in flight exceed
       // L2), so the register-resident row is kept as long as it fits. Measured, % of the HBM peak, resident / walks:
@@ -370,6 +392,14 @@ class TileEmitter {
           }
         }
       }
+      if (colsArg_ && (multiPass_ || packedRow_)) {
+        // rows of this bucket do not stay in registers: the walked kernels are made per row length
+        colsArg_ = allowColsArg_ = false;
+        multiPass_ = packedRow_ = false;
+        packedInput_.clear();
+        pickSchedule();
+        return;
+      }
       if (multiPass_) {
         const int64_t perGroup = opt_.chunks > 0 ? opt_.chunks : std::max<int64_t>(1, (packedRow_ ? 16 : 32) / vec_);
         chunks_ = static_cast<int>(std::min<int64_t>(perGroup, perThread));
@@ -387,7 +417,7 @@ class TileEmitter {
       if (block_ % tpr_ != 0 || block_ % 64 != 0) block_ = std::max(tpr_, 64);
       rowsPerBlock_ = block_ / tpr_;
       grid_ = ceilDiv(rows_, rowsPerBlock_);
-      raggedCols_ = (groups_ * chunks_ * tpr_ != rowChunks);
+      raggedCols_ = colsArg_ || (groups_ * chunks_ * tpr_ != rowChunks);
       raggedRows_ = (rows_ % rowsPerBlock_) != 0 || extentArg_;
     } else {
       block_ = opt_.block > 0 ? opt_.block : 256;
@@ -493,10 +523,13 @@ class TileEmitter {
       if (s[d] != 1) allOne = false;
     }
     if (r == 1 || allOne) return "0L";
-    if (allFull) return "(" + rowVar + " * " + std::to_string(s[r - 1]) + "L)";
+    // the innermost extent of the operand: a number, or the kernel argument when the row length is one
+    const bool symbolic = colsArg_ && s[r - 1] == cols_ && cols_ != 1;
+    const std::string inner = symbolic ? std::string("COLS") : std::to_string(s[r - 1]) + "L";
+    if (allFull) return "(" + rowVar + " * " + inner + ")";
     // general leading-dim broadcast: decompose the row index over the leading dims
     std::vector<int64_t> stride(r, 0);
-    int64_t acc = s[r - 1];
+    int64_t acc = symbolic ? 1 : s[r - 1];
     for (int d = static_cast<int>(r) - 2; d >= 0; --d) {
       stride[static_cast<size_t>(d)] = (s[static_cast<size_t>(d)] == 1) ? 0 : acc;
       acc *= s[static_cast<size_t>(d)];
@@ -515,6 +548,7 @@ class TileEmitter {
       div *= extent;
     }
     if (firstTerm) return "0L";
+    if (symbolic) return "((" + e.str() + ") * COLS)";
     return "(" + e.str() + ")";
   }
 
@@ -543,10 +577,14 @@ class TileEmitter {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
     if (extentArg_) src_ << ", const long akg_extent";
+    if (colsArg_) src_ << ", const long akg_cols_arg";
     line(") {");
     if (extentArg_ && extentIsCols_) {
       line("  constexpr long ROWS = 1L;");
       line("  const long COLS = akg_extent;   // everything folds into one dimension: the element count");
+    } else if (extentArg_ && colsArg_) {
+      line("  const long COLS = akg_cols_arg;   // the row length (innermost extent)");
+      line("  const long ROWS = akg_extent;   // product of the leading dimensions");
     } else if (extentArg_) {
       src_ << "  constexpr long COLS = " << cols_ << "L;\n";
       line("  const long ROWS = akg_extent;   // product of the leading dimensions");
@@ -594,6 +632,7 @@ class TileEmitter {
       if (multiPass_) {
         src_ << "  constexpr int GROUPS = " << groups_ << ";\n";
       } else {
+        if (colsArg_) line("  const int akg_overlap = static_cast<int>((V - COLS % V) % V);   // elements the last chunk of a row shares with its neighbour");
         emitColumnsOfGroup("0");
       }
     } else {
@@ -673,8 +712,10 @@ class TileEmitter {
       if (folded[d] != full_[d]) leadFull = false;
       if (folded[d] != 1) leadOne = false;
     }
-    if (leadOne && rows_ != 1) return number;
+    const bool symbolicCols = colsArg_ && folded.back() == cols_ && cols_ != 1;
+    if (leadOne && rows_ != 1) return symbolicCols ? "COLS * " + std::to_string(dtypeSize(t.dtype)) + "L" : number;
     if (!leadFull) return number;
+    if (symbolicCols) return "akg_extent * COLS * " + std::to_string(dtypeSize(t.dtype)) + "L";
     return "akg_extent * " + std::to_string(folded.back() * static_cast<int64_t>(dtypeSize(t.dtype))) + "L";
   }
 
@@ -685,6 +726,7 @@ class TileEmitter {
   bool streamsWholeLines(int tensorId) const {
     if (!nonTemporal_) return false;
     if (!rowMode_) return true;
+    if (colsArg_) return false;   // rows of any length: their first and last cache lines may be shared with neighbours
     const int64_t rowBytes = cols_ * static_cast<int64_t>(dtypeSize(g_.tensor(tensorId).dtype));
     return rowBytes % 64 == 0 || rowBytes >= 16384;  // two shared lines in 256 or more do not matter
   }
@@ -693,12 +735,13 @@ class TileEmitter {
   void emitColumnsOfGroup(const std::string &group) {
     line("  long akg_cols[NCHUNK];");
     line("  bool akg_ok[NCHUNK];");
-    if (overlap_ > 0) line("  bool akg_tail[NCHUNK];");
+    const bool tails = overlap_ > 0 || (colsArg_ && rowMode_);
+    if (tails) line("  bool akg_tail[NCHUNK];");
     line("#pragma unroll");
     line("  for (int j = 0; j < NCHUNK; ++j) {");
     line("    akg_cols[j] = ((static_cast<long>(" + group + ") * NCHUNK + j) * TPR + tcol) * V;");
     line(std::string("    akg_ok[j] = ") + (raggedCols_ ? "akg_cols[j] < COLS;" : "true;"));
-    if (overlap_ > 0) {
+    if (tails) {
       line("    akg_tail[j] = akg_cols[j] > COLS - V;");
       line("    if (akg_tail[j]) akg_cols[j] = COLS - V;");
     }
@@ -1060,7 +1103,9 @@ class TileEmitter {
     line("    for (int e = 0; e < V; ++e) {");
     std::string step = spec.combiner + "::apply(" + acc + ", " + in.ident + "[j][e])";
     if (spec.roundEachStep) step = tag + "::rnd(" + step + ")";
-    if (overlap_ > 0) {
+    if (colsArg_) {
+      src_ << "      if (akg_ok[j] && (!akg_tail[j] || e >= akg_overlap)) " << acc << " = " << step << ";\n";
+    } else if (overlap_ > 0) {
       src_ << "      if (akg_ok[j] && (!akg_tail[j] || e >= " << overlap_ << ")) " << acc << " = " << step << ";\n";
     } else if (raggedCols_) {
       src_ << "      if (akg_ok[j]) " << acc << " = " << step << ";\n";

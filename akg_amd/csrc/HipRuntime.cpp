@@ -12,6 +12,7 @@
 #include <sys/stat.h>
 
 #include <cerrno>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -43,6 +44,7 @@ struct akg_hip_kernel {
   std::vector<char> codeObject;
   std::string codeSha256;
   bool cacheHit = false;
+  double buildMs = 0.0;   // wall time of translation, lowering and (unless cached) device compilation of this handle
   std::mutex mu;
   // loaded lazily on first launch, per device
   struct Loaded {
@@ -83,6 +85,7 @@ struct akg_hip_dynamic {
   bool hasOutDir = false;
   int numInputs = 0;
   std::vector<int> inputRanks;
+  std::vector<int> outputRanks;   // declared ranks of the outputs (output_desc), for the packed launch form
   std::mutex mu;
   std::map<std::string, akg_hip_kernel_t *> specializations;
 };
@@ -430,8 +433,21 @@ int compileStaged(const std::string &jsonText, std::unique_ptr<akg_hip_kernel> k
   return AKG_HIP_OK;
 }
 
+int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
+                   const akg::ShapeBinding *binding, bool allowStages);
+
 int doCompile(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
               const akg::ShapeBinding *binding, bool allowStages) {
+  const auto t0 = std::chrono::steady_clock::now();
+  const int rc = doCompileTimed(jsonText, outDir, outKernel, binding, allowStages);
+  if (rc == AKG_HIP_OK && outKernel != nullptr && *outKernel != nullptr) {
+    (*outKernel)->buildMs = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  }
+  return rc;
+}
+
+int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kernel_t **outKernel,
+                   const akg::ShapeBinding *binding, bool allowStages) {
   if (outKernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "out_kernel is NULL");
   *outKernel = nullptr;
   std::unique_ptr<akg_hip_kernel> k(new akg_hip_kernel());
@@ -853,6 +869,7 @@ int akg_hip_kernel_get_info(const akg_hip_kernel_t *kernel, akg_hip_kernel_info 
   info->algorithmic_ops = kernel->lowered.algorithmicOps;
   info->cache_hit = kernel->cacheHit ? 1 : 0;
   info->workspace_bytes = kernel->lowered.workspaceBytes;
+  info->build_ms = kernel->buildMs;
   return AKG_HIP_OK;
 }
 
@@ -1052,6 +1069,10 @@ int akg_hip_dynamic_create(const char *json_text, size_t json_len, const char *o
       const akg::json::Value &desc = root.at("input_desc")[i][0];
       d->inputRanks.push_back(desc.contains("shape") ? static_cast<int>(desc.at("shape").size()) : 1);
     }
+    for (size_t i = 0; i < root.at("output_desc").size(); ++i) {
+      const akg::json::Value &desc = root.at("output_desc")[i];
+      d->outputRanks.push_back(desc.contains("shape") ? static_cast<int>(desc.at("shape").size()) : 1);
+    }
     *out = d.release();
     g_lastError.clear();
     return AKG_HIP_OK;
@@ -1106,6 +1127,59 @@ int akg_hip_dynamic_specialize(akg_hip_dynamic_t *dyn, const int64_t *const *inp
   dyn->specializations[key] = k;
   *out_kernel = k;
   return AKG_HIP_OK;
+}
+
+int akg_hip_dynamic_launch_packed(akg_hip_dynamic_t *dyn, void *const *tensor_ptrs, const int64_t *const *shape_lists,
+                                  int n_tensors, void *stream, akg_hip_kernel_t **used_kernel) {
+  if (dyn == nullptr || tensor_ptrs == nullptr || shape_lists == nullptr) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "NULL argument");
+  }
+  const int nin = dyn->numInputs, nout = static_cast<int>(dyn->outputRanks.size());
+  if (n_tensors != nin + nout) {
+    return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "the description has " + std::to_string(nin) + " inputs and " +
+                                                std::to_string(nout) + " outputs, " + std::to_string(n_tensors) + " tensors given");
+  }
+  // per tensor: [offset, sizes..., strides...] (the integer fields of its memref descriptor)
+  auto readDense = [&](int i, int rank, std::vector<int64_t> *shape) -> int {
+    const int64_t *list = shape_lists[i];
+    if (list == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "shape list " + std::to_string(i) + " is NULL");
+    if (list[0] != 0) return fail(AKG_HIP_ERR_UNSUPPORTED, "tensor " + std::to_string(i) + ": a non-zero offset is not supported");
+    shape->assign(list + 1, list + 1 + rank);
+    int64_t expect = 1;
+    for (int d = rank; d-- > 0;) {
+      const int64_t extent = (*shape)[static_cast<size_t>(d)];
+      if (extent < 0) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "tensor " + std::to_string(i) + ": negative extent");
+      if (extent != 1 && list[1 + rank + d] != expect) {
+        return fail(AKG_HIP_ERR_UNSUPPORTED, "tensor " + std::to_string(i) + ": only dense row-major tensors are supported");
+      }
+      expect *= extent;
+    }
+    return AKG_HIP_OK;
+  };
+  std::vector<std::vector<int64_t>> inShapes(static_cast<size_t>(nin));
+  std::vector<const int64_t *> shapePtrs(static_cast<size_t>(nin));
+  for (int i = 0; i < nin; ++i) {
+    const int rc = readDense(i, dyn->inputRanks[static_cast<size_t>(i)], &inShapes[static_cast<size_t>(i)]);
+    if (rc != AKG_HIP_OK) return rc;
+    shapePtrs[static_cast<size_t>(i)] = inShapes[static_cast<size_t>(i)].data();
+  }
+  std::vector<int32_t> ranks(dyn->inputRanks.begin(), dyn->inputRanks.end());
+  akg_hip_kernel_t *kernel = nullptr;
+  int rc = akg_hip_dynamic_specialize(dyn, shapePtrs.data(), ranks.data(), nin, &kernel);
+  if (rc != AKG_HIP_OK) return rc;
+  for (int j = 0; j < nout; ++j) {
+    std::vector<int64_t> given;
+    rc = readDense(nin + j, dyn->outputRanks[static_cast<size_t>(j)], &given);
+    if (rc != AKG_HIP_OK) return rc;
+    const akg::TensorValue &t = tensorAt(kernel, nin + j);
+    int64_t n = 1;
+    for (int64_t e : given) n *= e;
+    if (n != t.numel()) {
+      return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "output " + std::to_string(j) + ": the shape given does not follow from the input shapes");
+    }
+  }
+  if (used_kernel != nullptr) *used_kernel = kernel;
+  return akg_hip_launch(kernel, tensor_ptrs, n_tensors, stream);
 }
 
 void akg_hip_dynamic_destroy(akg_hip_dynamic_t *dyn) {

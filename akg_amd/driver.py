@@ -38,7 +38,7 @@ class _KernelInfo(ctypes.Structure):
     _fields_ = [("kernel_name", ctypes.c_char * 256), ("family", ctypes.c_char * 32),
                 ("operator_type", ctypes.c_char * 32), ("grid", ctypes.c_uint32 * 3), ("block", ctypes.c_uint32 * 3),
                 ("algorithmic_bytes", ctypes.c_uint64), ("algorithmic_ops", ctypes.c_uint64),
-                ("cache_hit", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64)]
+                ("cache_hit", ctypes.c_int32), ("workspace_bytes", ctypes.c_uint64), ("build_ms", ctypes.c_double)]
 
 
 _lib = None
@@ -81,6 +81,8 @@ def load_library():
     lib.akg_hip_dynamic_num_inputs.argtypes = [vp, ctypes.POINTER(ci)]
     lib.akg_hip_dynamic_specialize.argtypes = [vp, ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)),
                                                ctypes.POINTER(ctypes.c_int32), ci, ctypes.POINTER(vp)]
+    lib.akg_hip_dynamic_launch_packed.argtypes = [vp, ctypes.POINTER(vp), ctypes.POINTER(ctypes.POINTER(ctypes.c_int64)), ci, vp,
+                                                  ctypes.POINTER(vp)]
     lib.akg_hip_dynamic_destroy.argtypes = [vp]
     lib.akg_hip_dynamic_destroy.restype = None
     _lib = lib
@@ -114,6 +116,7 @@ class HipDynamicKernel:
         od = out_dir.encode("utf-8") if out_dir else None
         _check(self._lib.akg_hip_dynamic_create(raw, len(raw), od, ctypes.byref(self._handle)))
         self._kernels = {}
+        self._by_handle = {}
 
     def specialize(self, input_shapes):
         """HipKernel for exactly these input shapes (list of lists, input_desc order); cached per shape set."""
@@ -131,10 +134,36 @@ class HipDynamicKernel:
         self._kernels[key] = k
         return k
 
+    def launch_packed(self, device_ptrs, shapes, stream=None):
+        """The reference's dynamic calling form (LLVMParameterPacking.cpp:91-194): `device_ptrs` for inputs then outputs,
+        `shapes` their concrete shapes; packs [0, sizes, strides] per tensor like transform_data_to_ctypes
+        (mlir_driver.py:186-252) and returns the HipKernel that ran."""
+        n = len(device_ptrs)
+        width = 1 + 2 * max([len(s) for s in shapes] + [1])
+        lists = []
+        for s in shapes:
+            strides = [1] * len(s)
+            for d in range(len(s) - 2, -1, -1):
+                strides[d] = strides[d + 1] * s[d + 1]
+            row = [0] + list(s) + strides
+            lists.append((ctypes.c_int64 * width)(*(row + [0] * (width - len(row)))))
+        lptrs = (ctypes.POINTER(ctypes.c_int64) * n)(*[ctypes.cast(a, ctypes.POINTER(ctypes.c_int64)) for a in lists])
+        ptrs = (ctypes.c_void_p * n)(*device_ptrs)
+        used = ctypes.c_void_p()
+        _check(self._lib.akg_hip_dynamic_launch_packed(self._handle, ptrs, lptrs, n, ctypes.c_void_p(stream or 0),
+                                                       ctypes.byref(used)))
+        key = used.value
+        if key not in self._by_handle:
+            k = HipKernel(None, _borrowed=used)
+            k._keepalive = self
+            self._by_handle[key] = k
+        return self._by_handle[key]
+
     def __del__(self):
         h = getattr(self, "_handle", None)
         if h:
             self._kernels = {}
+            self._by_handle = {}
             self._lib.akg_hip_dynamic_destroy(h)
             self._handle = None
 
@@ -184,6 +213,7 @@ class HipKernel:
         self.algorithmic_ops = int(info.algorithmic_ops)
         self.cache_hit = bool(info.cache_hit)
         self.workspace_bytes = int(info.workspace_bytes)
+        self.build_ms = float(info.build_ms)
 
     @classmethod
     def from_file(cls, info_path, out_dir=DEFAULT_META_DIR):

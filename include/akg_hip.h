@@ -71,6 +71,9 @@ typedef struct akg_hip_kernel_info {
                                          artifact directory or from this process's memory (same source digest) */
   uint64_t workspace_bytes;           /* device scratch the handle owns per device (streaming reductions, GEMMs
                                          with K split over workgroups, grouped segment sums), else 0 */
+  double build_ms;                    /* wall time it took to make this handle: translation, lowering and, unless
+                                         cache_hit, device compilation (a new shape set of a dynamic description that
+                                         shares a code object costs about a millisecond, a device compilation ~0.5 s) */
 } akg_hip_kernel_info;
 
 typedef struct akg_hip_kernel akg_hip_kernel_t;
@@ -185,7 +188,8 @@ void akg_hip_free_string(char *text);
  * (dynamic_utils.py:269-526). Here a dynamic description is kept as text and specialised on demand:
  * akg_hip_dynamic_specialize binds the -1s to the given input shapes, derives every op's result shape, lowers the
  * kernel for these shapes and returns its handle. Elementwise and row-reduction kernels take the product of their
- * leading dimensions as a kernel argument, so shape sets that differ only there share one code object and the second
+ * leading dimensions and their row length as kernel arguments (the schedule is made for the power-of-two bucket of
+ * 16-byte chunks the row falls into), so shape sets that differ only there share one code object and the second
  * one needs no device compilation; anything else compiles once per shape set (or is found in the artifact directory). The handle is owned by the dynamic object (do not destroy it); it is
  * launched with akg_hip_launch like any other, and akg_hip_kernel_tensor reports the concrete output shapes.
  */
@@ -195,6 +199,17 @@ int akg_hip_dynamic_num_inputs(const akg_hip_dynamic_t *dyn, int *n_inputs);
 /** input_shapes[i] points at input_ranks[i] extents of kernel input i (input_desc order). */
 int akg_hip_dynamic_specialize(akg_hip_dynamic_t *dyn, const int64_t *const *input_shapes, const int32_t *input_ranks,
                                int n_inputs, akg_hip_kernel_t **out_kernel);
+/**
+ * The reference's calling form for dynamic-shape kernels (packParamsDynamicShape, LLVMParameterPacking.cpp:91-194, as
+ * filled by transform_data_to_ctypes, mlir_driver.py:186-252): one array with the data pointer of every tensor, inputs
+ * then outputs, and one array with, per tensor, a pointer to its int64 list [offset, sizes..., strides...] (the integer
+ * fields of its memref descriptor; trailing padding is ignored). Reads the input shapes from the lists, finds or makes
+ * the specialisation for them (akg_hip_dynamic_specialize), checks the output shapes given against the derived ones,
+ * and enqueues the launch on `stream` with the pointers as DEVICE pointers. Tensors must be dense row-major with offset
+ * 0 (anything else: AKG_HIP_ERR_UNSUPPORTED). `used_kernel`, if non-NULL, receives the handle that ran (owned by `dyn`).
+ */
+int akg_hip_dynamic_launch_packed(akg_hip_dynamic_t *dyn, void *const *tensor_ptrs, const int64_t *const *shape_lists,
+                                  int n_tensors, void *stream, akg_hip_kernel_t **used_kernel);
 void akg_hip_dynamic_destroy(akg_hip_dynamic_t *dyn);
 
 /** Library version string. */

@@ -653,15 +653,22 @@ def test_grouped_segment_sum_on_skewed_ids(pattern):
 
 # Shapes the dynamic descriptions of the reference's test tree are specialised to (input_desc order).
 REF_DYNAMIC_SHAPES = {
-    "Fused_Cast_Sub_Mul_split_14802837530264465372": [[[32, 1, 48, 48]], [[32, 1, 5, 1000]]],
-    "Fused_Mul_Add_ReduceMax_split_8454462579718005500": [[[32, 1, 40, 72], [32, 12, 40, 72]], [[1, 1, 16, 520], [32, 12, 16, 520]]],
-    "Fused_RealDiv_split_4177286244677596212": [[[32, 12, 24, 40], [32, 12, 24, 1]]],
-    "Fused_ReduceMax_fusion_2054638663855723468": [[[100, 768]], [[3, 768]]],
-    "Fused_ReduceMax_fusion_234578345729057892345": [[[4096, 33]], [[4096, 4096]]],
-    "Fused_Sub_Exp_ReduceSum_split_7283368012049929718": [[[32, 12, 24, 40], [32, 12, 24, 1]]],
-    "Fused_Sub_Mul_Cast_fusion_4217325526348104075": [[[32, 16, 20, 64], [32, 16, 20, 1], [32, 16, 20, 64]]],
-    "Fused_Sub_Mul_split_1454621004286351279": [[[32, 1, 48, 48]]],
-    "elem_dyn_fuse_broadcast": [[[4096, 96], [96], [1, 96]], [[4096, 7], [7], [1, 7]]],
+    "Fused_Cast_Sub_Mul_split_14802837530264465372": [[[32, 1, 48, 48]], [[32, 1, 5, 1000]], [[32, 1, 48, 40]]],
+    "Fused_Mul_Add_ReduceMax_split_8454462579718005500": [[[32, 1, 40, 72], [32, 12, 40, 72]], [[1, 1, 16, 520], [32, 12, 16, 520]],
+                                                          [[32, 1, 9, 72], [32, 12, 9, 72]]],
+    "Fused_RealDiv_split_4177286244677596212": [[[32, 12, 24, 40], [32, 12, 24, 1]], [[32, 12, 7, 40], [32, 12, 7, 1]],
+                                                [[32, 12, 24, 136], [32, 12, 24, 1]]],
+    "Fused_ReduceMax_fusion_2054638663855723468": [[[100, 768]], [[3, 768]], [[2048, 768]]],
+    "Fused_ReduceMax_fusion_234578345729057892345": [[[4096, 33]], [[4096, 4096]], [[4096, 40]]],
+    "Fused_Sub_Exp_ReduceSum_split_7283368012049929718": [[[32, 12, 24, 40], [32, 12, 24, 1]], [[32, 12, 5, 40], [32, 12, 5, 1]],
+                                                          [[32, 12, 24, 1000], [32, 12, 24, 1]]],
+    "Fused_Sub_Mul_Cast_fusion_4217325526348104075": [[[32, 16, 20, 64], [32, 16, 20, 1], [32, 16, 20, 64]],
+                                                      [[32, 16, 3, 64], [32, 16, 3, 1], [32, 16, 3, 64]],
+                                                      [[32, 16, 20, 72], [32, 16, 20, 1], [32, 16, 20, 72]]],
+    "Fused_Sub_Mul_split_1454621004286351279": [[[32, 1, 48, 48]], [[32, 1, 6, 48]], [[32, 1, 48, 520]]],
+    "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic": [[[32, 1, 48, 48], [32, 12, 48, 48]], [[1, 1, 40, 72], [32, 12, 40, 72]],
+                                                                          [[32, 1, 7, 1000], [32, 12, 7, 1000]]],
+    "elem_dyn_fuse_broadcast": [[[4096, 96], [96], [1, 96]], [[4096, 7], [7], [1, 7]], [[4096, 1000], [1000], [1, 1000]]],
 }
 
 
@@ -725,6 +732,121 @@ def test_reference_dynamic_descriptions_specialised(name):
                 ok, msg = harness.compare(g, e, d.dtype)
             print("  %s %s %s %s: %s" % (kernel.family, shapes, d.name, d.dtype, msg), flush=True)
             assert ok, "%s %s output %s: %s" % (name, shapes, d.name, msg)
+
+
+@pytest.mark.parametrize("name", REF_DYNAMIC)
+def test_reference_dynamic_descriptions_through_the_packed_calling_form(name):
+    """All ten dynamic-shape descriptions of the reference's test tree, three shape sets each, called the way the
+    reference calls a dynamic kernel: one array of data pointers and one of [offset, sizes, strides] lists
+    (LLVMParameterPacking.cpp:91-194); the library reads the shapes from the lists and finds or makes the
+    specialisation. The first set is launched again at the end: it must come from the cache (same handle)."""
+    import torch
+    from oracle import np_ref
+    path = os.path.join(REF_INFO, name)
+    desc = harness.load_desc(path)
+    dyn = driver.HipDynamicKernel(open(path, encoding="utf-8").read())
+    sets = REF_DYNAMIC_SHAPES[name.split(".info")[0]]
+    assert len(sets) >= 3
+    dev = torch.device("cuda:0")
+    seen = []
+    for shapes in sets + sets[:1]:
+        bound = _bind_description(desc, shapes)
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 651)
+        ins = [_torch_view(a).to(dev) for a in inputs]
+        out_shapes = [o["shape"] for o in bound["output_desc"]]
+        out_dtypes = [o["data_type"] for o in bound["output_desc"]]
+        outs = []
+        for shp, dt in zip(out_shapes, out_dtypes):
+            t = torch.empty(int(np.prod(shp)) * np.dtype(driver.NP_HOST_DTYPE[dt]).itemsize, dtype=torch.uint8, device=dev)
+            t.fill_(0xFF if dt in ("float16", "bfloat16", "float32", "float64") else 0x7B)
+            outs.append(t)
+        kernel = dyn.launch_packed([t.data_ptr() for t in ins + outs], list(shapes) + out_shapes,
+                                   torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        seen.append(kernel)
+        print("  %s %s: %s, made in %.1f ms%s" % (name[:40], shapes, kernel.family, kernel.build_ms,
+                                                 " (no device compilation)" if kernel.cache_hit else ""), flush=True)
+        got = [o.cpu().numpy().view(driver.NP_HOST_DTYPE[dt]).reshape(shp) for o, dt, shp in zip(outs, out_dtypes, out_shapes)]
+        expect = np_ref.evaluate(bound, inputs)
+        wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+        exact = np_ref.evaluate(harness.widen_to_float64(bound), wide)
+        full = max(int(np.prod(s)) for s in shapes)
+        for dt, g, e, x in zip(out_dtypes, got, expect, exact):
+            terms = max(1, full // max(1, g.size))
+            if dt == "float32" and terms > 1 and any(o["name"] == "ReduceSum" for o in desc["op_desc"]):
+                ok, msg = harness.compare_reassociated(g, x, dt, terms)
+            else:
+                ok, msg = harness.compare(g, e, dt)
+            assert ok, "%s %s: %s" % (name, shapes, msg)
+    assert seen[-1] is seen[0]
+    # a wrong output shape and a strided tensor are refused, not launched
+    shapes = sets[0]
+    bound = _bind_description(desc, shapes)
+    out_shapes = [o["shape"] for o in bound["output_desc"]]
+    bad = [list(s) for s in out_shapes]
+    bad[0][-1] += 1
+    with pytest.raises(driver.AkgHipError) as e:
+        dyn.launch_packed([ins[0].data_ptr()] * (len(shapes) + len(out_shapes)), list(shapes) + bad)
+    assert e.value.code == -1
+
+
+def _open_dims(text, rows, cols):
+    """Turns the extents `rows` and `cols` of a description built for those sentinel sizes into open (-1) dimensions."""
+    d = json_loads(text)
+
+    def walk(x):
+        if isinstance(x, dict):
+            if "shape" in x:
+                x["shape"] = [-1 if n in (rows, cols) else n for n in x["shape"]]
+            for v in x.values():
+                walk(v)
+        elif isinstance(x, list):
+            for v in x:
+                walk(v)
+    walk(d)
+    return d
+
+
+@pytest.mark.parametrize("pattern", ["softmax_f16", "layernorm_bf16", "quant_bf16", "bias_gelu_f32"])
+def test_row_lengths_of_one_bucket_share_a_code_object_and_stay_correct(pattern):
+    """Dynamic descriptions take the row length as a kernel argument: the schedule is made for a power-of-two bucket of
+    chunk counts, chunks are element-aligned and the last one overlaps its neighbour by a run-time amount. Row lengths
+    across a bucket (odd ones, the bucket's ends, one chunk short of it), with different row counts: the first makes the
+    code object, the others must reuse it (no device compilation) and all must match the oracle."""
+    from oracle import np_ref
+    R, C = 7777, 9999
+    if pattern == "softmax_f16":
+        text, v, lengths = op_desc.softmax_last_axis(R, C, "float16", "dyn_softmax_f16"), 8, [520, 1000, 1024, 513, 777]
+    elif pattern == "layernorm_bf16":
+        text, v, lengths = op_desc.layernorm_residual(R, C, "bfloat16", 1e-5, "dyn_layernorm_bf16"), 8, [4096, 2056, 3001, 4095]
+    elif pattern == "quant_bf16":
+        text, v, lengths = op_desc.quant_int8_residual(R, C, "bfloat16", "dyn_quant_bf16"), 8, [300, 264, 511, 512]
+    else:
+        b = op_desc.DescBuilder("dyn_bias_gelu_f32")
+        x, bias = b.input([R, C], "float32"), b.input([C], "float32")
+        y = b.add(x, bias)
+        text, v, lengths = b.dumps([b.mul(y, b.unary("Tanh", y))]), 4, [72, 100, 128, 68]
+    desc = _open_dims(text, R, C)
+    dyn = driver.HipDynamicKernel(__import__("json").dumps(desc), out_dir=None)
+    first = None
+    for n, cols in enumerate(lengths):
+        rows = [37, 5, 130, 64, 2][n % 5]
+        # the description's open dims are (rows, cols) for matrices and (cols) for vectors
+        shapes = [[cols] if len(e[0]["shape"]) == 1 else [rows, cols] for e in desc["input_desc"]]
+        kernel = dyn.specialize(shapes)
+        bound = _bind_description(desc, shapes)
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 41 + n)
+        got = run_on_gpu(kernel, inputs)
+        expect = np_ref.evaluate(bound, inputs)
+        for d, g, e in zip(kernel.outputs, got, expect):
+            ok, msg = harness.compare(g, e, d.dtype)
+            print("  %s rows %d cols %d %s: %s (made in %.1f ms, cache_hit %s)" % (pattern, rows, cols, d.name, msg, kernel.build_ms,
+                                                                                 kernel.cache_hit), flush=True)
+            assert ok, "%s cols %d output %s: %s" % (pattern, cols, d.name, msg)
+        if first is None:
+            first = kernel
+        elif pattern != "bias_gelu_f32" or cols % v == 0:
+            assert kernel.cache_hit, "%s: row length %d compiled anew" % (pattern, cols)
 
 
 def _bind_softmax_description(desc, shapes):
