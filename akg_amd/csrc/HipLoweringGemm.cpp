@@ -111,6 +111,7 @@ class GemmEmitter {
   std::vector<EpiVal> vals_;
   std::vector<bool> relaxed_;
   std::ostringstream members_, prepare_, apply_;
+  std::vector<int> assignOnly_;   // inputs that are only written (Assign destinations the description never reads)
 
   DType elem_ = DType::I8;  // operand element type: I8, BF16 or F16
   int elemBytes() const { return elem_ == DType::I8 ? 1 : 2; }
@@ -169,7 +170,7 @@ class GemmEmitter {
         matmulOp_ = static_cast<int>(i);
       } else if (op.kind == OpKind::Unknown) {
         throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
-      } else if (op.kind == OpKind::Unsupported || op.kind == OpKind::Assign || lowering::isReduceKind(op.kind)) {
+      } else if (op.kind == OpKind::Unsupported || lowering::isReduceKind(op.kind)) {
         throw LoweringError("op " + op.name + " cannot be fused into a MatMul epilogue yet");
       }
     }
@@ -338,6 +339,34 @@ class GemmEmitter {
       if (op.kind == OpKind::MatMul) continue;
       if (op.outputs.size() != 1) throw LoweringError("op " + op.name + ": multiple results are not supported");
       const int outId = op.outputs[0];
+      if (op.kind == OpKind::Assign) {
+        // the value is stored over the destination (a kernel input as large as the MatMul result) besides being the
+        // op's result: linalg.copy ins=value outs=destination (MindSporeToLinalg.cpp:495-524). Every thread writes
+        // exactly the chunk of the destination that it has read (if the description reads it at all) before.
+        const TensorValue &dst = g_.tensor(op.inputs[0]);
+        if (dst.inputIndex < 0 || op.inputs[0] == aId_ || op.inputs[0] == bId_ || dst.dtype != g_.tensor(outId).dtype ||
+            dst.numel() != batch_ * m_ * n_ || classifyInput(dst) != EpiRank::Full) {
+          throw LoweringError("op " + op.name + ": in a MatMul fusion the destination must be a kernel input of the result's shape and type (not a MatMul operand)");
+        }
+        const EpiVal &value = vals_[static_cast<size_t>(op.inputs[1])];
+        if (!value.defined) throw LoweringError("op " + op.name + ": value is undefined");
+        const std::string ct = ctOf(outId), tag = tagOf(outId);
+        EpiVal &v = vals_[static_cast<size_t>(outId)];
+        v.defined = true;
+        v.rank = EpiRank::Full;
+        v.ident = "t" + std::to_string(outId);
+        std::vector<std::string> operands = {"", operand(op.inputs[1])};
+        apply_ << "    " << ct << " " << v.ident << "[" << W << "];  // " << op.name << " -> " << dst.name << "\n";
+        apply_ << "#pragma unroll\n    for (int e = 0; e < " << W << "; ++e) " << v.ident << "[e] = "
+               << lowering::elementwiseExpr(g_, op, operands, false) << ";\n";
+        if (!g_.tensor(op.inputs[0]).used || !vals_[static_cast<size_t>(op.inputs[0])].defined) {
+          members_ << "  const " << tag << "::storage *__restrict__ in" << dst.inputIndex << ";\n";
+          assignOnly_.push_back(dst.inputIndex);
+        }
+        apply_ << "    akg::store_chunk<" << tag << ", " << W << ", false>(const_cast<" << tag << "::storage *>(in" << dst.inputIndex
+               << ") + grow * " << n_ << "L + col, " << v.ident << ");\n";
+        continue;
+      }
       bool hasRow = false, hasCol = false, hasFull = false, hasScalar = false;
       for (int in : op.inputs) {
         const EpiVal &vi = vals_[static_cast<size_t>(in)];
@@ -422,7 +451,8 @@ class GemmEmitter {
          << "  epi.row0 = akg_batch * " << m_ << "L;\n";
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       const int id = g_.inputs[i];
-      if (id == aId_ || id == bId_ || !g_.tensor(id).used) continue;
+      const bool written = std::find(assignOnly_.begin(), assignOnly_.end(), static_cast<int>(i)) != assignOnly_.end();
+      if (id == aId_ || id == bId_ || (!g_.tensor(id).used && !written)) continue;
       src_ << "  epi.in" << i << " = in" << i << ";\n";
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i) src_ << "  epi.out" << i << " = out" << i << ";\n";

@@ -114,6 +114,7 @@ class IndexedEmitter {
   std::vector<Staged> staged_;
   int tDim_ = -1;               // output dimension the staged inputs' innermost axis lands on
   Index canonical_;             // index of the current output element, by dimension
+  std::vector<bool> assignedInput_;   // per kernel input: overwritten by an Assign of this kernel (empty: none is)
   std::vector<bool> relaxed_;
   int nextTemp_ = 0;
   int indent_ = 2;
@@ -144,7 +145,19 @@ class IndexedEmitter {
         throw LoweringError("op " + op.name + " is not in the op table (mindspore.unknown cannot be legalized)");
       }
       if (op.kind == OpKind::Unsupported) throw LoweringError("op " + op.name + " has no kernel family yet");
-      if (op.kind == OpKind::Assign) throw LoweringError("op " + op.name + " has no lowering in the indexed family yet");
+      if (op.kind == OpKind::Assign) {
+        // The value is stored over the destination (a kernel input) besides being the op's result (linalg.copy
+        // ins=value outs=destination, MindSporeToLinalg.cpp:495-524). The thread that computes an element of the result
+        // stores it to the same position of the destination, so the result must be an output of the kernel, and no
+        // thread may read the destination anywhere but at its own position (checked where inputs are read).
+        const TensorValue &dst = g_.tensor(op.inputs[0]);
+        const TensorValue &res = g_.tensor(op.outputs[0]);
+        if (dst.inputIndex < 0 || res.outputIndex < 0 || dst.dtype != res.dtype) {
+          throw LoweringError("op " + op.name + ": next to data-movement ops the destination must be a kernel input and the result an output of the kernel");
+        }
+        if (assignedInput_.empty()) assignedInput_.assign(g_.inputs.size(), false);
+        assignedInput_[static_cast<size_t>(dst.inputIndex)] = true;
+      }
       if (op.kind == OpKind::MatMul || lowering::isReduceKind(op.kind)) {
         throw LoweringError("op " + op.name + " cannot be fused with data-movement ops (Transpose, Tile, Slice, Pad, "
                             "Concat) in one kernel yet");
@@ -180,7 +193,8 @@ class IndexedEmitter {
     // An innermost extent that V does not divide keeps the full chunk width: the last chunk of a row then starts
     // at extent - V and shares elements with its neighbour (both write the same values); such chunks are only
     // element-aligned in memory.
-    if (opt_.vec == 0 && (space_.back() % v) != 0 && space_.back() >= 2 * v) {
+    // (not with an Assign: a thread would read elements of the destination that its neighbour has already overwritten)
+    if (opt_.vec == 0 && (space_.back() % v) != 0 && space_.back() >= 2 * v && assignedInput_.empty()) {
       overlapTail_ = true;
     } else {
       while (v > 1 && (space_.back() % v) != 0) v >>= 1;
@@ -403,6 +417,16 @@ class IndexedEmitter {
     const std::string ct = ctOf(id);
     if (t.producer < 0) {
       if (t.inputIndex < 0) throw LoweringError("operand " + t.name + " is undefined");
+      if (!assignedInput_.empty() && assignedInput_[static_cast<size_t>(t.inputIndex)]) {
+        Index own = canonical_;
+        for (size_t d = 0; d < t.shape.size() && d < own.size(); ++d) {
+          if (t.shape[d] == 1) own[d] = Ix();
+        }
+        if (own.size() != idx.size() || idx != own) {
+          throw LoweringError("input " + t.name + " is overwritten by an Assign of this kernel and read through an index map: "
+                              "a thread would read positions that another thread writes");
+        }
+      }
       const std::string chunkLoad = inLoop_ ? tryChunkLoad(id, idx) : std::string();
       if (!chunkLoad.empty()) {
         scopes_.back()[key] = chunkLoad;
@@ -601,6 +625,12 @@ class IndexedEmitter {
         stmt("}");
         break;
       }
+      case OpKind::Assign: {
+        const std::vector<std::string> operands = {
+            "", valueAt(op.inputs[1], broadcastIndex(idx, outShape, inShapeOf(1), "op " + op.name))};
+        stmt("const " + ct + " " + var + " = " + lowering::elementwiseExpr(g_, op, operands, false) + ";" + note);
+        break;
+      }
       default: {
         if (!lowering::isElementwiseKind(op.kind)) throw LoweringError("op " + op.name + " has no indexed lowering");
         std::vector<std::string> operands;
@@ -797,12 +827,16 @@ class IndexedEmitter {
     src_ << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << kname << "(";
     size_t argc = 0;
     for (size_t i = 0; i < g_.inputs.size(); ++i, ++argc) {
-      src_ << (argc ? ", " : "") << "const " << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
+      const bool written = !assignedInput_.empty() && assignedInput_[i];
+      src_ << (argc ? ", " : "") << (written ? "" : "const ") << tagOf(g_.inputs[i]) << "::storage *__restrict__ in" << i;
     }
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
     src_ << ") {\n";
+    if (!staged_.empty() && !assignedInput_.empty()) {
+      throw LoweringError("an Assign next to a transpose that is staged through LDS tiles has no kernel yet");
+    }
     if (!staged_.empty()) {
       emitTiledBody();
       src_ << "}\n";
@@ -835,6 +869,7 @@ class IndexedEmitter {
            (overlapTail_ ? "" : "  // a multiple of V: V divides the innermost extent"));
       idx.back() = affine("inner0", !overlapTail_, true);
     }
+    canonical_ = idx;
     openElementLoop(indent_);
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       const std::string v = valueAt(g_.outputs[i], idx);
@@ -848,6 +883,13 @@ class IndexedEmitter {
       stmt(std::string("akg::store_chunk") + (overlapTail_ ? "_unaligned<" : "<") + tagOf(g_.outputs[i]) + ", V" +
            (overlapTail_ ? "" : (ntOut ? ", true" : ", false")) + ">(out" + std::to_string(i) + " + base, o" +
            std::to_string(i) + ");");
+      // an output that is the result of an Assign: the same chunk goes over the destination
+      const int producer = g_.tensor(g_.outputs[i]).producer;
+      if (producer >= 0 && g_.ops[static_cast<size_t>(producer)].kind == OpKind::Assign) {
+        const OpNode &as = g_.ops[static_cast<size_t>(producer)];
+        stmt("akg::store_chunk<" + tagOf(g_.outputs[i]) + ", V, false>(in" + std::to_string(g_.tensor(as.inputs[0]).inputIndex) +
+             " + base, o" + std::to_string(i) + ");  // " + as.name + " -> " + g_.tensor(as.inputs[0]).name);
+      }
     }
     src_ << "}\n";
   }

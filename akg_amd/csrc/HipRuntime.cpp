@@ -471,6 +471,23 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
   } catch (const akg::TranslateError &e) {
     return fail(AKG_HIP_ERR_TRANSLATE, e.what());
   }
+  if (binding == nullptr) {
+    // ArgMax over an axis that is not the innermost one: respelled as Transpose + ArgMax over the last axis (+ Reshape)
+    bool outerArgMax = false;
+    for (const akg::OpNode &op : k->graph.ops) {
+      if (op.kind != akg::OpKind::ArgMax || op.axes.size() != 1) continue;
+      const std::vector<int64_t> &shape = k->graph.tensor(op.inputs[0]).shape;
+      for (size_t d = static_cast<size_t>(op.axes[0]) + 1; d < shape.size(); ++d) outerArgMax = outerArgMax || shape[d] != 1;
+    }
+    std::string respelled;
+    try {
+      if (outerArgMax && akg::moveArgMaxToInnermostAxis(jsonText, &respelled)) {
+        return doCompileTimed(respelled, outDir, outKernel, binding, allowStages);
+      }
+    } catch (const std::exception &) {
+      // leave the description as it is: the lowering below says what it cannot do
+    }
+  }
   try {
     akg::LoweringOptions options = akg::LoweringOptions::fromEnvironment();
     options.extentAsArgument = binding != nullptr;

@@ -378,4 +378,99 @@ bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsTo
   return true;
 }
 
+bool moveArgMaxToInnermostAxis(const std::string &jsonText, std::string *rewritten) {
+  const json::Value doc = json::Value::parse(jsonText);
+  if (!doc.isObject() || !doc.contains("op_desc")) return false;
+  auto shapeText = [](const std::vector<int64_t> &shape) {
+    std::string o = "[";
+    for (size_t i = 0; i < shape.size(); ++i) o += (i ? ", " : "") + std::to_string(shape[i]);
+    return o + "]";
+  };
+  auto tensorText = [&](const std::string &name, const std::vector<int64_t> &shape, const std::string &dtype) {
+    return "{\"data_type\": " + quote(dtype) + ", \"format\": \"DefaultFormat\", \"shape\": " + shapeText(shape) +
+           ", \"tensor_name\": " + quote(name) + "}";
+  };
+  bool changed = false;
+  std::string ops = "[";
+  const json::Value &opDesc = doc.at("op_desc");
+  for (size_t k = 0; k < opDesc.size(); ++k) {
+    const json::Value &entry = opDesc[k];
+    std::string text = dump(entry);
+    do {
+      if (!entry.contains("name") || entry.at("name").asString() != "ArgMax") break;
+      const json::Value &in = entry.at("input_desc")[0][0];
+      const json::Value &out = entry.at("output_desc")[0];
+      if (!in.contains("shape") || !out.contains("shape")) break;
+      const std::vector<int64_t> shape = in.at("shape").asIntVector();
+      const std::vector<int64_t> outShape = out.at("shape").asIntVector();
+      bool open = false;
+      for (int64_t d : shape) open = open || d < 0;
+      if (open || shape.size() < 2) break;
+      // the axis: value of the second input, else the attribute
+      std::vector<int64_t> axes;
+      bool keep = false;
+      if (entry.at("input_desc").size() > 1 && entry.at("input_desc")[1][0].contains("value")) {
+        const json::Value &v = entry.at("input_desc")[1][0].at("value");
+        axes = v.isArray() ? v.asIntVector() : std::vector<int64_t>{v.asInt()};
+      }
+      const json::Value &attrs = entry.contains("attr") ? entry.at("attr") : json::Value();
+      for (size_t a = 0; a < attrs.size(); ++a) {
+        const std::string an = attrs[a].at("name").asString();
+        if (an == "axis" && axes.empty()) {
+          const json::Value &v = attrs[a].at("value");
+          axes = v.isArray() ? v.asIntVector() : std::vector<int64_t>{v.asInt()};
+        } else if (an == "keep_dims") {
+          keep = attrs[a].at("value").asBool();
+        }
+      }
+      if (axes.size() != 1) break;
+      const int64_t rank = static_cast<int64_t>(shape.size());
+      const int64_t axis = axes[0] < 0 ? axes[0] + rank : axes[0];
+      if (axis < 0 || axis >= rank) break;
+      // innermost already (extent-1 dimensions behind it do not count)
+      bool innermost = true;
+      for (int64_t d = axis + 1; d < rank; ++d) innermost = innermost && shape[static_cast<size_t>(d)] == 1;
+      if (innermost) break;
+      std::vector<int64_t> perm, moved, without;
+      for (int64_t d = 0; d < rank; ++d) {
+        if (d == axis) continue;
+        perm.push_back(d);
+        moved.push_back(shape[static_cast<size_t>(d)]);
+        without.push_back(shape[static_cast<size_t>(d)]);
+      }
+      perm.push_back(axis);
+      moved.push_back(shape[static_cast<size_t>(axis)]);
+      const std::string inName = in.at("tensor_name").asString(), outName = out.at("tensor_name").asString();
+      const std::string inType = in.at("data_type").asString(), outType = out.at("data_type").asString();
+      const std::string tName = outName + "_akg_moved", iName = outName + "_akg_index";
+      const bool reshape = keep || without != outShape;
+      std::string t = "{\"attr\": [{\"data_type\": \"listInt\", \"name\": \"perm\", \"value\": " + shapeText(perm) +
+                      "}], \"impl_path\": \"\", \"input_desc\": [[" + dump(in) + "]], \"name\": \"Transpose\", \"output_desc\": [" +
+                      tensorText(tName, moved, inType) + "]}";
+      std::string a = "{\"attr\": [{\"data_type\": \"listInt\", \"name\": \"axis\", \"value\": [" + std::to_string(rank - 1) +
+                      "]}, {\"data_type\": \"bool\", \"name\": \"keep_dims\", \"value\": false}], \"impl_path\": \"\", \"input_desc\": [[" +
+                      tensorText(tName, moved, inType) + "]], \"name\": \"ArgMax\", \"output_desc\": [" +
+                      (reshape ? tensorText(iName, without, outType) : dump(out)) + "]}";
+      text = t + ", " + a;
+      if (reshape) {
+        text += ", {\"attr\": [{\"data_type\": \"listInt\", \"name\": \"shape\", \"value\": " + shapeText(outShape) +
+                "}], \"impl_path\": \"\", \"input_desc\": [[" + tensorText(iName, without, outType) +
+                "]], \"name\": \"Reshape\", \"output_desc\": [" + dump(out) + "]}";
+      }
+      changed = true;
+    } while (false);
+    ops += (k ? ", " : "") + text;
+  }
+  ops += "]";
+  if (!changed) return false;
+  std::string o = "{";
+  bool first = true;
+  for (const auto &m : doc.members()) {
+    o += (first ? "" : ", ") + quote(m.first) + ": " + (m.first == "op_desc" ? ops : dump(m.second));
+    first = false;
+  }
+  *rewritten = o + "}";
+  return true;
+}
+
 }  // namespace akg

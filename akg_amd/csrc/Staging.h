@@ -53,6 +53,13 @@ struct StagingPlan {
 // one kernel: a softmax behind a MatMul); true: at reduction results as well.
 bool planStages(const std::string &jsonText, const OpGraph &g, bool reductionsToo, StagingPlan *plan, std::string *why);
 
+// ArgMax over an axis that is not the innermost one. The row family finds the position of the greatest element along
+// the innermost axis only, so such an op is respelled in the description itself: Transpose (the reduced axis moved to
+// the back), ArgMax over the last axis, and a Reshape where keep_dims put a 1 in the middle of the result shape. The
+// respelled description then runs as two kernels (the transpose gets one of its own). Returns true and the new text
+// when something was respelled; descriptions with open (-1) extents are left alone.
+bool moveArgMaxToInnermostAxis(const std::string &jsonText, std::string *rewritten);
+
 }  // namespace akg
 
 #endif  // AKG_HIP_STAGING_H_

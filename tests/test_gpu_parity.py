@@ -557,6 +557,121 @@ def test_workspace_launches_from_two_streams_are_ordered_and_repeat_bit_for_bit(
     assert ok, msg
 
 
+def _run_with_inputs_back(kernel, inputs):
+    """Like run_on_gpu, but also returns the device copies of the inputs after the launch (Assign writes over them)."""
+    import torch
+    dev = torch.device("cuda:0")
+    ins = [_torch_view(a).to(dev) for a in inputs]
+    outs = []
+    for d in kernel.outputs:
+        t = torch.empty(d.nbytes, dtype=torch.uint8, device=dev)
+        t.fill_(0xFF if d.dtype in ("float16", "bfloat16", "float32", "float64") else 0x7B)
+        outs.append(t)
+    kernel.launch(ins + outs)
+    torch.cuda.synchronize()
+    got = [o.cpu().numpy().view(driver.NP_HOST_DTYPE[d.dtype]).reshape(d.shape) for d, o in zip(kernel.outputs, outs)]
+    back = [t.cpu().numpy().view(a.dtype).reshape(a.shape) for t, a in zip(ins, inputs)]
+    return got, back
+
+
+def _gemm_assign(m, k, n, dtype, name):
+    """Accumulator update behind a MatMul: acc <- 0.9 acc + 0.1 (A @ B), the product also returned in 16 bits."""
+    b = op_desc.DescBuilder(name)
+    a, w, acc = b.input([m, k], dtype), b.input([k, n], dtype), b.input([m, n], "float32")
+    y = b.matmul(a, w, "float32")
+    upd = b.add(b.mul(acc, b.const(0.9, "float32")), b.mul(y, b.const(0.1, "float32")))
+    return b.dumps([b.op("Assign", [acc, upd], [m, n], "float32"), b.cast(y, dtype if dtype != "float32" else "float32")])
+
+
+def _slice_assign(name):
+    """momentum <- 0.9 momentum + grad[:, 8:72]: an in-place update whose value comes through a Slice."""
+    b = op_desc.DescBuilder(name)
+    mom, grad = b.input([37, 64], "float32"), b.input([37, 100], "float32")
+    upd = b.add(b.mul(mom, b.const(0.9, "float32")), op_desc.slice_(b, grad, [0, 8], [37, 64]))
+    return b.dumps([b.op("Assign", [mom, upd], [37, 64], "float32")])
+
+
+def _transposed_self_assign(name):
+    """p <- p + p^T: the destination is read through a Transpose, so the transposed copy must be made before the update."""
+    b = op_desc.DescBuilder(name)
+    p = b.input([48, 48], "float32")
+    return b.dumps([b.op("Assign", [p, b.add(p, op_desc.transpose(b, p, [1, 0]))], [48, 48], "float32")])
+
+
+@pytest.mark.parametrize("case", ["gemm_bf16_256x512x256", "gemm_f16_100x264x136", "gemm_f32_70x100x36", "slice", "transposed_self"])
+def test_assign_next_to_a_matmul_or_a_data_movement_op(case, tmp_path):
+    """Assign in the GEMM epilogue (the destination is a kernel input of the result's shape; also on the split-K and the
+    serial kernels) and in the indexed family (the thread that computes an element stores it over the destination too);
+    a destination that is read through an index map makes the description run as two kernels. The destination's device
+    copy must hold the oracle's updated values afterwards, the other inputs must be untouched."""
+    from oracle import np_ref
+    if case.startswith("gemm"):
+        _, dt, dims = case.split("_")
+        m, k, n = [int(x) for x in dims.split("x")]
+        text = _gemm_assign(m, k, n, {"bf16": "bfloat16", "f16": "float16", "f32": "float32"}[dt], "assign_" + case)
+    elif case == "slice":
+        text = _slice_assign("assign_slice")
+    else:
+        text = _transposed_self_assign("assign_transposed_self")
+    desc = json_loads(text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    print("case %s: %s grid %d" % (case, kernel.family, kernel.grid[0]), flush=True)
+    if case == "transposed_self":
+        assert kernel.family == "staged"
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 77)
+    updates = {}
+    expect = np_ref.evaluate(desc, inputs, updates=updates)
+    got, back = _run_with_inputs_back(kernel, [a.copy() for a in inputs])
+    # float32 results of the matrix units add the same products in another order than the oracle's k loop
+    # and are held against the float64 evaluation of the same description instead
+    mfma_terms = k if case.startswith("gemm") and "gemm_serial" not in kernel.source else 0
+    exact, exact_updates = expect, updates
+    if mfma_terms:
+        exact_updates = {}
+        wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+        exact = np_ref.evaluate(harness.widen_to_float64(desc), wide, updates=exact_updates)
+
+    def check(g, e, x, dt, what):
+        if dt == "float32" and mfma_terms:
+            ok, msg = harness.compare_reassociated(g, np.asarray(x, dtype=np.float64), dt, mfma_terms)
+        else:
+            ok, msg = harness.compare(g, e, dt)
+        assert ok, "%s %s: %s" % (case, what, msg)
+
+    for d, g, e, x in zip(kernel.outputs, got, expect, exact):
+        check(g, e, x, d.dtype, "output " + d.name)
+    assert updates, "the description overwrites no input"
+    for pos, a in enumerate(inputs):
+        check(back[pos], updates.get(pos, a), exact_updates.get(pos, a), desc["input_desc"][pos][0]["data_type"],
+              "input %d after the launch" % pos)
+        if pos not in updates:
+            assert np.array_equal(back[pos].view(np.uint8), a.view(np.uint8)), "%s: input %d was modified" % (case, pos)
+
+
+@pytest.mark.parametrize("shape,axis,keep,dtype", [([5, 7, 9], 1, False, "float32"), ([5, 7, 9], 0, True, "float16"),
+                                                   ([40, 300], 0, False, "bfloat16"), ([3, 4, 5, 6], 2, True, "float32"),
+                                                   ([64, 1000, 2], 1, False, "float32")])
+def test_argmax_over_an_axis_that_is_not_the_innermost(shape, axis, keep, dtype):
+    """ArgMax over an outer axis is respelled as Transpose + ArgMax over the last axis (+ Reshape for keep_dims) and runs
+    as two kernels; positions must equal the oracle's (first of equal maxima: the inputs are rounded to a coarse grid so
+    that ties occur)."""
+    from oracle import np_ref
+    b = op_desc.DescBuilder("argmax_axis%d_%s_%s" % (axis, dtype, "x".join(map(str, shape))))
+    x = b.input(shape, dtype)
+    text = b.dumps([op_desc.argmax(b, x, axis, keep, "int32")])
+    desc = json_loads(text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family == "staged" and kernel.source.count('extern "C" __global__') == 2
+    x_in = harness.make_inputs(desc, seed=harness.BASE_SEED + 5)[0]
+    as_f32 = harness.bf16_bits_to_f32(x_in) if dtype == "bfloat16" else x_in.astype(np.float32)
+    coarse = (np.round(as_f32 * 4) / 4).astype(np.float32)          # ties
+    x_in = harness.f32_to_bf16_bits(coarse) if dtype == "bfloat16" else coarse.astype(x_in.dtype)
+    got = run_on_gpu(kernel, [x_in])[0]
+    expect = np_ref.evaluate(desc, [x_in])[0]
+    assert np.array_equal(got, expect)
+    assert np.array_equal(got.reshape(-1), np.argmax(coarse, axis=axis).reshape(-1))
+
+
 def check_segment_sum(path, seed, repeats=2):
     """UnsortedSegmentSum keeps the serial order of the additions per output element: bit-exact against the oracle,
     float types included, and on every launch (nothing may be left over from the one before)."""

@@ -334,10 +334,13 @@ def test_argmax_becomes_a_max_and_a_least_position_in_the_row_family():
     # a row too long for registers: the position pass is one more walk over the (packed) row
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_argmax_bf16_scaled_4x70000.info"))
     assert k.source.count("for (int akg_g = 0; akg_g < GROUPS") == 3 and "RawChunk" in k.source
+    # an outer axis: respelled as Transpose + ArgMax over the last axis, two kernels
     b = op_desc.DescBuilder("Fused_ArgMax_axis0")
-    with pytest.raises(driver.AkgHipError) as e:
-        driver.HipKernel(b.dumps([op_desc.argmax(b, b.input([8, 16], "float32"), 0)]), out_dir=None)
-    assert e.value.code == -4 and "innermost axis" in str(e.value)
+    k = driver.HipKernel(b.dumps([op_desc.argmax(b, b.input([8, 16], "float32"), 0)]), out_dir=None)
+    assert k.family == "staged" and k.source.count('extern "C" __global__') == 2 and [t.shape for t in k.outputs] == [[16]]
+    b = op_desc.DescBuilder("Fused_ArgMax_axis1_keep")
+    k = driver.HipKernel(b.dumps([op_desc.argmax(b, b.input([4, 8, 16], "float32"), 1, True)]), out_dir=None)
+    assert k.family == "staged" and [t.shape for t in k.outputs] == [[4, 1, 16]]
     b = op_desc.DescBuilder("Fused_ArgMax_float_result")
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(b.dumps([op_desc.argmax(b, b.input([8, 16], "float32"), 1, dtype="float32")]), out_dir=None)
