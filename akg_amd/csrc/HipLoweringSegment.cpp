@@ -60,6 +60,106 @@ SegmentShapes checkSegmentSum(const OpGraph &g) {
   return sh;
 }
 
+// The three counting launches both grouped schedules share. The generated source must define POSITIONS, KEYS (counters
+// per run), RUNS, RUN, W_HIST, W_TOTAL, W_START, as_segment() and key_of(segment):
+//   <op>_count    workgroup b counts the keys of its run of positions (LDS counters) -> hist[b][key]
+//   <op>_offsets  per key, the exclusive prefix of hist over b (in place) and the key's total
+//   <op>_starts   exclusive prefix of the totals: where each key's list starts (and, at [KEYS], where the last one ends)
+// Workgroups of the <op>_offsets launch for `keys` counters per run (see emitCountingLaunches).
+int64_t offsetsGrid(int64_t keys) {
+  const int64_t perWg = keys >= 4096 ? 16 : 4, groups = (keys + perWg - 1) / perWg;
+  return (groups + 7) / 8 * 8;
+}
+
+void emitCountingLaunches(std::ostringstream &s, const std::string &name, const std::string &paramList, const std::string &idTag,
+                          const std::string &idsName, int64_t runs, int64_t keys) {
+  const int perStart = static_cast<int>((keys + 1023) / 1024);
+  // ---- count ----
+  s << "extern \"C\" __global__ __launch_bounds__(256) void " << name << "_count(" << paramList << ") {\n";
+  s << "  __shared__ unsigned akg_cnt[KEYS];\n";
+  s << "  const int tid = static_cast<int>(threadIdx.x), run = static_cast<int>(blockIdx.x);\n";
+  s << "  for (int k = tid; k < KEYS; k += 256) akg_cnt[k] = 0u;\n";
+  s << "  __syncthreads();\n";
+  s << "  const int p0 = run * RUN, p1 = p0 + RUN < POSITIONS ? p0 + RUN : POSITIONS;\n";
+  s << "#pragma unroll 4\n";
+  s << "  for (int p = p0 + tid; p < p1; p += 256) {\n";
+  s << "    const int id = as_segment(" << idTag << "::load(" << idsName << "[p]));\n";
+  s << "    if (id >= 0) atomicAdd(&akg_cnt[key_of(id)], 1u);\n";
+  s << "  }\n";
+  s << "  __syncthreads();\n";
+  s << "  for (int k = tid; k < KEYS; k += 256) akg_ws[W_HIST + static_cast<long>(run) * KEYS + k] = akg_cnt[k];\n";
+  s << "}\n\n";
+
+  // ---- offsets ----
+  // A workgroup takes a few keys and splits the runs among its threads: KPW keys x (256 / KPW) slabs of runs. Few keys
+  // (the bucketed schedule) take 4 a workgroup, so that the launch still fills the chip.
+  const int keysPerWg = keys >= 4096 ? 16 : 4, slabs = 256 / keysPerWg;
+  const int64_t runsPer = (runs + slabs - 1) / slabs;
+  s << "extern \"C\" __global__ __launch_bounds__(256) void " << name << "_offsets(" << paramList << ") {\n";
+  s << "  constexpr int PER = " << runsPer << ", KPW = " << keysPerWg << ", SLABS = " << slabs << ";   // runs per thread, keys per workgroup, threads a key\n";
+  s << "  __shared__ unsigned akg_part[SLABS][KPW + 1];\n";
+  s << "  const int tid = static_cast<int>(threadIdx.x), sl = tid % KPW, bl = tid / KPW;\n";
+  s << "  // (workgroups of one XCD - launch order: workgroup b runs on XCD b mod 8 - take neighbouring keys, which share lines)\n";
+  s << "  constexpr int GROUPS = (KEYS + KPW - 1) / KPW, PER_XCD = (GROUPS + 7) / 8;\n";
+  s << "  const int group = static_cast<int>(blockIdx.x & 7u) * PER_XCD + static_cast<int>(blockIdx.x >> 3);\n";
+  s << "  if (group >= GROUPS) return;   // (uniform)\n";
+  s << "  const int seg = group * KPW + sl;\n";
+  s << "  const int b0 = bl * PER < RUNS ? bl * PER : RUNS, b1 = b0 + PER < RUNS ? b0 + PER : RUNS;\n";
+  s << "  unsigned *__restrict__ col = akg_ws + W_HIST + seg;\n";
+  s << "  unsigned sum = 0u;\n";
+  s << "  if (seg < KEYS) {\n";
+  s << "#pragma unroll 8\n";
+  s << "    for (int b = b0; b < b1; ++b) sum += col[static_cast<long>(b) * KEYS];\n";
+  s << "  }\n";
+  s << "  akg_part[bl][sl] = sum;\n";
+  s << "  __syncthreads();\n";
+  s << "  unsigned before = 0u;\n";
+  s << "  for (int j = 0; j < bl; ++j) before += akg_part[j][sl];\n";
+  s << "  if (seg >= KEYS) return;\n";
+  s << "  if (bl == SLABS - 1) akg_ws[W_TOTAL + seg] = before + sum;\n";
+  s << "  for (int b = b0; b < b1; b += 8) {\n";
+  s << "    unsigned v[8];\n";
+  s << "#pragma unroll\n";
+  s << "    for (int j = 0; j < 8; ++j) v[j] = b + j < b1 ? col[static_cast<long>(b + j) * KEYS] : 0u;\n";
+  s << "#pragma unroll\n";
+  s << "    for (int j = 0; j < 8; ++j) {\n";
+  s << "      if (b + j < b1) col[static_cast<long>(b + j) * KEYS] = before;\n";
+  s << "      before += v[j];\n";
+  s << "    }\n  }\n";
+  s << "}\n\n";
+
+  // ---- starts ----
+  s << "extern \"C\" __global__ __launch_bounds__(1024) void " << name << "_starts(" << paramList << ") {\n";
+  s << "  constexpr int PER = " << perStart << ";\n";
+  s << "  __shared__ unsigned akg_scan[1024];\n";
+  s << "  const int tid = static_cast<int>(threadIdx.x);\n";
+  s << "  unsigned v[PER], sum = 0u;\n";
+  s << "#pragma unroll\n";
+  s << "  for (int j = 0; j < PER; ++j) {\n";
+  s << "    const int seg = tid * PER + j;\n";
+  s << "    v[j] = seg < KEYS ? akg_ws[W_TOTAL + seg] : 0u;\n";
+  s << "    sum += v[j];\n";
+  s << "  }\n";
+  s << "  akg_scan[tid] = sum;\n";
+  s << "  __syncthreads();\n";
+  s << "  for (int d = 1; d < 1024; d <<= 1) {\n";
+  s << "    const unsigned add = tid >= d ? akg_scan[tid - d] : 0u;\n";
+  s << "    __syncthreads();\n";
+  s << "    akg_scan[tid] += add;\n";
+  s << "    __syncthreads();\n";
+  s << "  }\n";
+  s << "  unsigned run = akg_scan[tid] - sum;\n";
+  s << "#pragma unroll\n";
+  s << "  for (int j = 0; j < PER; ++j) {\n";
+  s << "    const int seg = tid * PER + j;\n";
+  s << "    if (seg < KEYS) akg_ws[W_START + seg] = run;\n";
+  s << "    run += v[j];\n";
+  s << "  }\n";
+  s << "  if (tid == 1023) akg_ws[W_START + KEYS] = akg_scan[1023];\n";
+  s << "}\n\n";
+
+}
+
 /**
  * Many positions: the scan above costs (workgroups x positions) id reads, which dominates from a few hundred thousand
  * positions on. Here the positions are first grouped by segment, in position order within a segment (a counting sort
@@ -102,15 +202,12 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
   const int64_t wHist = 0, wTotal = wHist + runs * segments, wStart = wTotal + segments,
                 wSorted = (wStart + segments + 1 + 3) / 4 * 4;   // 16-byte aligned
   const int64_t words = wSorted + (staged ? (positions * slice * elemBytes + 3) / 4 : positions);
-  const int perStart = static_cast<int>((segments + 1023) / 1024);
-  const int64_t runsPer = (runs + 15) / 16;
-
   std::ostringstream s;
   s << "// Generated by the akg HIP lowering for gfx950. Op description: " << g.name << "\n";
   s << "// family: segment_sum (positions grouped by segment first), fusion class: " << operatorTemplateName(g.operatorTemplate) << "\n";
   s << "#include \"akg_rt.hpp\"\n\n";
   s << "namespace {\n";
-  s << "constexpr int POSITIONS = " << positions << ", SEGMENTS = " << segments << ", RUNS = " << runs << ", RUN = " << runLength
+  s << "constexpr int POSITIONS = " << positions << ", SEGMENTS = " << segments << ", KEYS = SEGMENTS, RUNS = " << runs << ", RUN = " << runLength
     << ", ID_BITS = " << idBits << ";\n";
   s << "constexpr long SLICE = " << slice << ", CHAINS = " << chains << ";\n";
   s << "constexpr long W_HIST = " << wHist << ", W_TOTAL = " << wTotal << ", W_START = " << wStart << ", W_SORTED = " << wSorted << ";\n";
@@ -121,6 +218,7 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
   } else {
     s << "__device__ inline int as_segment(int v) { return v < 0 || v >= SEGMENTS ? -1 : v; }\n";
   }
+  s << "__device__ inline int key_of(int segment) { return segment; }\n";
   s << "}  // namespace\n\n";
   std::ostringstream params;
   for (size_t i = 0; i < g.inputs.size(); ++i) {
@@ -129,81 +227,7 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
   params << ", " << tag << "::storage *__restrict__ out0, unsigned *__restrict__ akg_ws";
   const std::string idsName = "in" + std::to_string(ids.inputIndex), dataName = "in" + std::to_string(data.inputIndex);
 
-  // ---- count ----
-  s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.name << "_count(" << params.str() << ") {\n";
-  s << "  __shared__ unsigned akg_cnt[SEGMENTS];\n";
-  s << "  const int tid = static_cast<int>(threadIdx.x), run = static_cast<int>(blockIdx.x);\n";
-  s << "  for (int k = tid; k < SEGMENTS; k += 256) akg_cnt[k] = 0u;\n";
-  s << "  __syncthreads();\n";
-  s << "  const int p0 = run * RUN, p1 = p0 + RUN < POSITIONS ? p0 + RUN : POSITIONS;\n";
-  s << "#pragma unroll 4\n";
-  s << "  for (int p = p0 + tid; p < p1; p += 256) {\n";
-  s << "    const int id = as_segment(" << idTag << "::load(" << idsName << "[p]));\n";
-  s << "    if (id >= 0) atomicAdd(&akg_cnt[id], 1u);\n";
-  s << "  }\n";
-  s << "  __syncthreads();\n";
-  s << "  for (int k = tid; k < SEGMENTS; k += 256) akg_ws[W_HIST + static_cast<long>(run) * SEGMENTS + k] = akg_cnt[k];\n";
-  s << "}\n\n";
-
-  // ---- offsets ----
-  s << "extern \"C\" __global__ __launch_bounds__(256) void " << g.name << "_offsets(" << params.str() << ") {\n";
-  s << "  constexpr int PER = " << runsPer << ";   // runs per thread; 16 threads share a segment, 16 segments a workgroup\n";
-  s << "  __shared__ unsigned akg_part[16][17];\n";
-  s << "  const int tid = static_cast<int>(threadIdx.x), sl = tid & 15, bl = tid >> 4;\n";
-  s << "  const int seg = static_cast<int>(blockIdx.x) * 16 + sl;\n";
-  s << "  const int b0 = bl * PER, b1 = b0 + PER < RUNS ? b0 + PER : RUNS;\n";
-  s << "  unsigned *__restrict__ col = akg_ws + W_HIST + seg;\n";
-  s << "  unsigned sum = 0u;\n";
-  s << "  if (seg < SEGMENTS) {\n";
-  s << "#pragma unroll 8\n";
-  s << "    for (int b = b0; b < b1; ++b) sum += col[static_cast<long>(b) * SEGMENTS];\n";
-  s << "  }\n";
-  s << "  akg_part[bl][sl] = sum;\n";
-  s << "  __syncthreads();\n";
-  s << "  unsigned before = 0u;\n";
-  s << "  for (int j = 0; j < bl; ++j) before += akg_part[j][sl];\n";
-  s << "  if (seg >= SEGMENTS) return;\n";
-  s << "  if (bl == 15) akg_ws[W_TOTAL + seg] = before + sum;\n";
-  s << "  for (int b = b0; b < b1; b += 8) {\n";
-  s << "    unsigned v[8];\n";
-  s << "#pragma unroll\n";
-  s << "    for (int j = 0; j < 8; ++j) v[j] = b + j < b1 ? col[static_cast<long>(b + j) * SEGMENTS] : 0u;\n";
-  s << "#pragma unroll\n";
-  s << "    for (int j = 0; j < 8; ++j) {\n";
-  s << "      if (b + j < b1) col[static_cast<long>(b + j) * SEGMENTS] = before;\n";
-  s << "      before += v[j];\n";
-  s << "    }\n  }\n";
-  s << "}\n\n";
-
-  // ---- starts ----
-  s << "extern \"C\" __global__ __launch_bounds__(1024) void " << g.name << "_starts(" << params.str() << ") {\n";
-  s << "  constexpr int PER = " << perStart << ";\n";
-  s << "  __shared__ unsigned akg_scan[1024];\n";
-  s << "  const int tid = static_cast<int>(threadIdx.x);\n";
-  s << "  unsigned v[PER], sum = 0u;\n";
-  s << "#pragma unroll\n";
-  s << "  for (int j = 0; j < PER; ++j) {\n";
-  s << "    const int seg = tid * PER + j;\n";
-  s << "    v[j] = seg < SEGMENTS ? akg_ws[W_TOTAL + seg] : 0u;\n";
-  s << "    sum += v[j];\n";
-  s << "  }\n";
-  s << "  akg_scan[tid] = sum;\n";
-  s << "  __syncthreads();\n";
-  s << "  for (int d = 1; d < 1024; d <<= 1) {\n";
-  s << "    const unsigned add = tid >= d ? akg_scan[tid - d] : 0u;\n";
-  s << "    __syncthreads();\n";
-  s << "    akg_scan[tid] += add;\n";
-  s << "    __syncthreads();\n";
-  s << "  }\n";
-  s << "  unsigned run = akg_scan[tid] - sum;\n";
-  s << "#pragma unroll\n";
-  s << "  for (int j = 0; j < PER; ++j) {\n";
-  s << "    const int seg = tid * PER + j;\n";
-  s << "    if (seg < SEGMENTS) akg_ws[W_START + seg] = run;\n";
-  s << "    run += v[j];\n";
-  s << "  }\n";
-  s << "  if (tid == 1023) akg_ws[W_START + SEGMENTS] = akg_scan[1023];\n";
-  s << "}\n\n";
+  emitCountingLaunches(s, g.name, params.str(), idTag, idsName, runs, segments);
 
   // ---- place ----
   s << "extern \"C\" __global__ __launch_bounds__(64) void " << g.name << "_place(" << params.str() << ") {\n";
@@ -378,7 +402,7 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
     k.earlierPhases.push_back(ph);
   };
   phase("_count", runs, 256);
-  phase("_offsets", (segments + 15) / 16, 256);
+  phase("_offsets", offsetsGrid(segments), 256);
   phase("_starts", 1, 1024);
   phase("_place", runs, 64);
   k.workspaceBytes = static_cast<uint64_t>(words) * 4;
@@ -387,6 +411,299 @@ LoweredKernel lowerSegmentSorted(const OpGraph &g, const LoweringOptions &option
   std::ostringstream note;
   note << "segment_sum positions=" << positions << " segments=" << segments << " slice=" << slice << " grouped by segment: runs="
        << runs << " of " << runLength << " positions, 5 launches";
+  k.scheduleNote = note.str();
+  return k;
+}
+
+// Device code both launches of the bucketed schedule share: a stable counting sort of a chunk by key inside a workgroup.
+const char *const kChunkSort = R"AKG(
+// Stable counting sort of a chunk of NW x TILES x 64 items by key, inside a workgroup of NW wavefronts. Item (w, u, lane)
+// - wavefront, tile, lane, in this order of significance - has key[u] (negative: the item takes no part); the function
+// returns its place among the sorted items in slot[u]. First every wavefront ranks its own items: lanes of a tile with
+// the same key find each other with one ballot per key bit and stand behind the wavefront's running counter of that
+// key (its LDS accesses complete in program order, so the counters need no barrier between the tiles). Then the
+// counters are summed over the wavefronts and the keys (each key's run starts at a multiple of ALIGN), and every item
+// adds where the run of its key and wavefront starts. On return start[k] is where key k's run starts, len[k] its
+// length; a barrier has been passed since they were written. cnt: NW * KEYS counters, scan: NW words.
+template <int NW, int KEYS, int KEY_BITS, int TILES, int ALIGN>
+__device__ inline void chunk_sort(const int (&key)[TILES], unsigned (&slot)[TILES], unsigned short *cnt, unsigned *start,
+                                  unsigned *len, unsigned *scan) {
+  constexpr int THREADS = NW * 64, PER = (KEYS + THREADS - 1) / THREADS;
+  const int tid = static_cast<int>(threadIdx.x), lane = tid & 63, w = tid >> 6;
+  for (int k = tid; k < NW * KEYS; k += THREADS) cnt[k] = 0;
+  __syncthreads();
+  const unsigned long long below = (1ull << lane) - 1ull;
+  unsigned short *mine = cnt + w * KEYS;
+#pragma unroll
+  for (int u = 0; u < TILES; ++u) {
+    const int k = key[u] >= 0 ? key[u] : 0;
+    unsigned long long same = __ballot(key[u] >= 0);
+#pragma unroll
+    for (int bit = 0; bit < KEY_BITS; ++bit) {
+      const int mine_bit = __builtin_amdgcn_sbfe(k, bit, 1);   // 0 or all ones
+      const unsigned long long with = __ballot(mine_bit != 0);
+      const unsigned lo = ~(static_cast<unsigned>(with) ^ static_cast<unsigned>(mine_bit));
+      const unsigned hi = ~(static_cast<unsigned>(with >> 32) ^ static_cast<unsigned>(mine_bit));
+      same &= (static_cast<unsigned long long>(hi) << 32) | lo;   // lanes whose bit equals mine
+    }
+    slot[u] = 0u;
+    if (key[u] >= 0) {
+      const unsigned at = mine[k] + static_cast<unsigned>(__popcll(same & below));
+      slot[u] = at;
+      if ((same >> lane) >> 1 == 0ull) mine[k] = static_cast<unsigned short>(at + 1u);   // the group's highest lane
+    }
+  }
+  __syncthreads();
+  unsigned total[PER], sum = 0u;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int k = tid * PER + j;
+    unsigned before = 0u;
+    if (k < KEYS) {
+#pragma unroll
+      for (int h = 0; h < NW; ++h) {
+        const unsigned c = cnt[h * KEYS + k];
+        cnt[h * KEYS + k] = static_cast<unsigned short>(before);
+        before += c;
+      }
+      len[k] = before;
+    }
+    total[j] = (before + ALIGN - 1) / ALIGN * ALIGN;
+    sum += total[j];
+  }
+  unsigned incl = sum;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned o = __shfl_up(incl, d);
+    if (lane >= d) incl += o;
+  }
+  if (lane == 63) scan[w] = incl;
+  __syncthreads();
+  unsigned at = incl - sum;
+#pragma unroll
+  for (int j = 0; j < NW; ++j) at += j < w ? scan[j] : 0u;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int k = tid * PER + j;
+    if (k < KEYS) {
+      start[k] = at;
+#pragma unroll
+      for (int h = 0; h < NW; ++h) cnt[h * KEYS + k] += static_cast<unsigned short>(at);
+    }
+    at += total[j];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < TILES; ++u) {
+    if (key[u] >= 0) slot[u] += mine[key[u]];
+  }
+}
+)AKG";
+
+/**
+ * Very many positions of short rows (at most 12 bytes): grouping by segment in one step writes every row to a place of
+ * its own, a partial cache line each time (24.5 million 12-byte rows: 1.07 GB written for 0.29 GB of rows). Here the
+ * positions are first grouped by BUCKET, a few neighbouring segments, and the last step to the segment happens in LDS:
+ *
+ *   <op>_count / _offsets / _starts   as above, with the bucket as the key and chunks of 4096 positions as the runs
+ *   <op>_place    a workgroup sorts its chunk by bucket in LDS (chunk_sort above) and copies the sorted chunk out, one
+ *                 16-byte entry per position {row, segment}: a bucket's entries of one chunk are contiguous, so the
+ *                 stores fill whole sectors
+ *   <op>_kernel   a workgroup per bucket walks the bucket's entries, 4096 per round: the same sort, by segment now,
+ *                 puts the rows' columns into LDS lists per segment, and one lane per output element adds its list
+ *
+ * Both sorts are stable, so the order per output element is the position order and the result is the serial loop's,
+ * bit for bit.
+ */
+LoweredKernel lowerSegmentBucketed(const OpGraph &g, const LoweringOptions &options, const SegmentShapes &sh, int bucketBits) {
+  using lowering::computeTypeName;
+  using lowering::dtypeTag;
+  const TensorValue &data = *sh.data, &ids = *sh.ids, &out = *sh.out;
+  const int64_t positions = sh.positions, segments = sh.segments, slice = sh.slice;
+  const std::string ct = computeTypeName(out.dtype), tag = dtypeTag(out.dtype), idTag = dtypeTag(ids.dtype);
+  const bool narrow = out.dtype == DType::F16 || out.dtype == DType::BF16 || out.dtype == DType::I8 || out.dtype == DType::I16;
+  const std::string rndOpen = narrow ? tag + "::rnd(" : std::string("(");
+  const int elemBytes = static_cast<int>(dtypeSize(out.dtype));
+  const int64_t rowWords = slice * elemBytes / 4;
+  const int64_t perBucket = 1LL << bucketBits, buckets = (segments + perBucket - 1) / perBucket;
+  const int64_t chunk = 4096, chunks = (positions + chunk - 1) / chunk;
+  int keyBits = 1;
+  while ((1LL << keyBits) < buckets) ++keyBits;
+  // workspace, in 4-byte words
+  const int64_t wHist = 0, wTotal = wHist + chunks * buckets, wStart = wTotal + buckets,
+                wSorted = (wStart + buckets + 1 + 3) / 4 * 4;   // 16-byte aligned
+  const int64_t words = wSorted + positions * 4;
+
+  std::ostringstream s;
+  s << "// Generated by the akg HIP lowering for gfx950. Op description: " << g.name << "\n";
+  s << "// family: segment_sum (positions grouped by bucket of segments first), fusion class: " << operatorTemplateName(g.operatorTemplate) << "\n";
+  s << "#include \"akg_rt.hpp\"\n\n";
+  s << "namespace {\n";
+  s << "constexpr int POSITIONS = " << positions << ", SEGMENTS = " << segments << ", BUCKET_BITS = " << bucketBits << ", KEYS = " << buckets
+    << ", KEY_BITS = " << keyBits << ", RUNS = " << chunks << ", RUN = " << chunk << ";\n";
+  s << "constexpr int ROW = " << slice << ", ROW_WORDS = " << rowWords << ", NW = 8, TILES = RUN / (64 * NW);\n";
+  s << "constexpr long W_HIST = " << wHist << ", W_TOTAL = " << wTotal << ", W_START = " << wStart << ", W_SORTED = " << wSorted << ";\n";
+  s << "using id_t = " << idTag << "::storage;\n";
+  if (ids.dtype == DType::I64) {
+    s << "__device__ inline int as_segment(long v) { return v < 0 || v >= SEGMENTS ? -1 : static_cast<int>(v); }\n";
+  } else {
+    s << "__device__ inline int as_segment(int v) { return v < 0 || v >= SEGMENTS ? -1 : v; }\n";
+  }
+  s << "__device__ inline int key_of(int segment) { return segment >> BUCKET_BITS; }\n";
+  s << "typedef unsigned entry_t __attribute__((ext_vector_type(4)));   // x, y, z: the row's words, zero filled; w: segment\n";
+  s << kChunkSort;
+  s << "}  // namespace\n\n";
+  std::ostringstream params;
+  for (size_t i = 0; i < g.inputs.size(); ++i) {
+    params << (i ? ", " : "") << "const " << dtypeTag(g.tensor(g.inputs[i]).dtype) << "::storage *__restrict__ in" << i;
+  }
+  params << ", " << tag << "::storage *__restrict__ out0, unsigned *__restrict__ akg_ws";
+  const std::string idsName = "in" + std::to_string(ids.inputIndex), dataName = "in" + std::to_string(data.inputIndex);
+
+  emitCountingLaunches(s, g.name, params.str(), idTag, idsName, chunks, buckets);
+
+  // ---- place ----
+  // Workgroups that run at the same time on one XCD (launch order: workgroup b runs on XCD b mod 8) take neighbouring
+  // chunks, whose entries are neighbours in every bucket: the line two chunks share is completed in that XCD's L2.
+  const int64_t perXcd = (chunks + 7) / 8;
+  s << "extern \"C\" __global__ __launch_bounds__(512) void " << g.name << "_place(" << params.str() << ") {\n";
+  s << "  __shared__ entry_t akg_stage[RUN];\n";
+  s << "  __shared__ unsigned short akg_cnt[NW * KEYS];\n";
+  s << "  __shared__ unsigned akg_start[KEYS], akg_len[KEYS], akg_scan[NW];\n";
+  s << "  const int tid = static_cast<int>(threadIdx.x), lane = tid & 63, w = tid >> 6;\n";
+  if (options.variant == 4) {
+    s << "  const int run = static_cast<int>(blockIdx.x);\n";
+  } else {
+    s << "  const int run = static_cast<int>(blockIdx.x & 7u) * " << perXcd << " + static_cast<int>(blockIdx.x >> 3);\n";
+    s << "  if (run >= RUNS) return;   // (uniform)\n";
+  }
+  s << "  const int p0 = run * RUN + w * (64 * TILES);\n";
+  s << "  const unsigned *__restrict__ rows = reinterpret_cast<const unsigned *>(" << dataName << ");\n";
+  s << "  int id[TILES], key[TILES];\n  unsigned row[TILES][ROW_WORDS], slot[TILES];\n";
+  s << "#pragma unroll\n";
+  s << "  for (int u = 0; u < TILES; ++u) {\n";
+  s << "    const int p = p0 + u * 64 + lane;\n";
+  s << "    id[u] = p < POSITIONS ? as_segment(" << idTag << "::load(" << idsName << "[p])) : -1;\n";
+  s << "    key[u] = id[u] >= 0 ? key_of(id[u]) : -1;\n";
+  s << "#pragma unroll\n";
+  s << "    for (int c = 0; c < ROW_WORDS; ++c) row[u][c] = p < POSITIONS ? rows[static_cast<long>(p) * ROW_WORDS + c] : 0u;\n";
+  s << "  }\n";
+  s << "  chunk_sort<NW, KEYS, KEY_BITS, TILES, 1>(key, slot, akg_cnt, akg_start, akg_len, akg_scan);\n";
+  s << "#pragma unroll\n";
+  s << "  for (int u = 0; u < TILES; ++u) {\n";
+  s << "    if (id[u] >= 0) {\n";
+  s << "      entry_t e = {0u, 0u, 0u, static_cast<unsigned>(id[u])};\n";
+  s << "      e.x = row[u][0];\n";
+  if (rowWords > 1) s << "      e.y = row[u][1];\n";
+  if (rowWords > 2) s << "      e.z = row[u][2];\n";
+  s << "      akg_stage[slot[u]] = e;\n";
+  s << "    }\n";
+  s << "  }\n";
+  s << "  // where the bucket's entries of this chunk go, less where they are in the sorted chunk\n";
+  s << "  unsigned valid = 0u;\n";
+  s << "  for (int k = tid; k < KEYS; k += 64 * NW) {\n";
+  s << "    if (k == KEYS - 1) akg_scan[0] = akg_start[k] + akg_len[k];\n";
+  s << "    akg_start[k] = akg_ws[W_START + k] + akg_ws[W_HIST + static_cast<long>(run) * KEYS + k] - akg_start[k];\n";
+  s << "  }\n";
+  s << "  __syncthreads();\n";
+  s << "  valid = akg_scan[0];\n";
+  s << "  entry_t *__restrict__ placed = reinterpret_cast<entry_t *>(akg_ws + W_SORTED);\n";
+  s << "  for (unsigned i = tid; i < valid; i += 64 * NW) {\n";
+  s << "    const entry_t e = akg_stage[i];\n";
+  s << "    placed[akg_start[key_of(static_cast<int>(e.w))] + i] = e;\n";
+  s << "  }\n";
+  s << "}\n\n";
+
+  // ---- chains ----
+  const int64_t chains = perBucket * slice, chainsPerWave = (chains + 7) / 8;
+  s << "extern \"C\" __global__ __launch_bounds__(512) void " << g.name << "_kernel(" << params.str() << ") {\n";
+  s << "  constexpr int S = 1 << BUCKET_BITS, PLANE = RUN + 4 * S + 8, CHAINS = " << chains << ", PER_WAVE = " << chainsPerWave << ";\n";
+  s << "  __shared__ __attribute__((aligned(16))) " << ct << " akg_plane[ROW][PLANE];   // column c of the rows, lists per segment\n";
+  s << "  __shared__ unsigned short akg_cnt[NW * S];\n";
+  s << "  __shared__ unsigned akg_start[S], akg_len[S], akg_scan[NW];\n";
+  s << "  const int tid = static_cast<int>(threadIdx.x), lane = tid & 63, w = tid >> 6, bucket = static_cast<int>(blockIdx.x);\n";
+  s << "  const entry_t *__restrict__ placed = reinterpret_cast<const entry_t *>(akg_ws + W_SORTED);\n";
+  s << "  const unsigned from = akg_ws[W_START + bucket], upto = akg_ws[W_START + bucket + 1];\n";
+  s << "  constexpr unsigned LAST = POSITIONS - 1;\n";
+  s << "  // the output element of this lane, if it has one: wavefront w adds chains w * PER_WAVE ...\n";
+  s << "  const int chain = w * PER_WAVE + lane;\n";
+  s << "  const bool has = lane < PER_WAVE && chain < CHAINS;\n";
+  s << "  const int cs = has ? chain / ROW : 0, cc = has ? chain - cs * ROW : 0;\n";
+  s << "  union cell_t { entry_t q; " << tag << "::storage v[16 / sizeof(" << tag << "::storage)]; };\n";
+  s << "  typedef " << ct << " quad_t __attribute__((ext_vector_type(4)));\n";
+  s << "  " << ct << " acc = " << lowering::literalFor(out.dtype, 0.0) << ";\n";
+  s << "  for (unsigned r = from; r < upto; r += RUN) {\n";
+  s << "    cell_t cur[TILES];\n";
+  s << "    int key[TILES];\n";
+  s << "    unsigned slot[TILES];\n";
+  s << "    // (every load is issued, the address clamped to the workspace's last entry: no branch between the loads)\n";
+  s << "#pragma unroll\n";
+  s << "    for (int u = 0; u < TILES; ++u) {\n";
+  s << "      const unsigned k = r + (w * TILES + u) * 64 + lane;\n";
+  s << "      cur[u].q = __builtin_nontemporal_load(placed + (k < LAST ? k : LAST));\n";
+  s << "    }\n";
+  s << "#pragma unroll\n";
+  s << "    for (int u = 0; u < TILES; ++u) {\n";
+  s << "      const unsigned k = r + (w * TILES + u) * 64 + lane;\n";
+  s << "      key[u] = k < upto ? static_cast<int>(cur[u].q.w) & (S - 1) : -1;\n";
+  s << "    }\n";
+  s << "    chunk_sort<NW, S, BUCKET_BITS, TILES, 4>(key, slot, akg_cnt, akg_start, akg_len, akg_scan);\n";
+  s << "#pragma unroll\n";
+  s << "    for (int u = 0; u < TILES; ++u) {\n";
+  s << "      if (key[u] >= 0) {\n";
+  s << "#pragma unroll\n";
+  s << "        for (int c = 0; c < ROW; ++c) akg_plane[c][slot[u]] = " << tag << "::load(cur[u].v[c]);\n";
+  s << "      }\n";
+  s << "    }\n";
+  s << "    __syncthreads();\n";
+  s << "    if (has) {\n";
+  s << "      const int n = static_cast<int>(akg_len[cs]);\n";
+  s << "      const quad_t *__restrict__ list = reinterpret_cast<const quad_t *>(&akg_plane[cc][akg_start[cs]]);   // (a multiple of 4)\n";
+  s << "      int j = 0;\n";
+  s << "      for (; j + 8 <= n; j += 8) {\n";
+  s << "        const quad_t a = list[j / 4], b = list[j / 4 + 1];\n";
+  s << "#pragma unroll\n";
+  s << "        for (int u = 0; u < 4; ++u) acc = " << rndOpen << "akg::op_add(a[u], acc));\n";
+  s << "#pragma unroll\n";
+  s << "        for (int u = 0; u < 4; ++u) acc = " << rndOpen << "akg::op_add(b[u], acc));\n";
+  s << "      }\n";
+  s << "      if (j < n) {   // (what lies behind the list's end is read, inside the plane, and not added)\n";
+  s << "        const quad_t a = list[j / 4], b = list[j / 4 + 1];\n";
+  s << "#pragma unroll\n";
+  s << "        for (int u = 0; u < 8; ++u) {\n";
+  s << "          const " << ct << " sum = " << rndOpen << "akg::op_add(u < 4 ? a[u & 3] : b[u & 3], acc));\n";
+  s << "          acc = j + u < n ? sum : acc;\n";
+  s << "        }\n";
+  s << "      }\n";
+  s << "    }\n";
+  s << "    __syncthreads();\n";
+  s << "  }\n";
+  s << "  if (has && bucket * S + cs < SEGMENTS) out0[static_cast<long>(bucket * S + cs) * ROW + cc] = " << tag << "::store(acc);\n";
+  s << "}\n";
+
+  LoweredKernel k;
+  k.kernelName = g.name + "_kernel";
+  k.source = s.str();
+  k.family = KernelFamily::SegmentSum;
+  k.grid[0] = static_cast<unsigned>(buckets);
+  k.block[0] = 512;
+  const auto phase = [&](const char *suffix, int64_t grid, unsigned block) {
+    KernelPhase ph;
+    ph.kernelName = g.name + suffix;
+    ph.grid[0] = static_cast<unsigned>(grid);
+    ph.block[0] = block;
+    k.earlierPhases.push_back(ph);
+  };
+  phase("_count", chunks, 256);
+  phase("_offsets", offsetsGrid(buckets), 256);
+  phase("_starts", 1, 1024);
+  phase("_place", options.variant == 4 ? chunks : perXcd * 8, 512);
+  k.workspaceBytes = static_cast<uint64_t>(words) * 4;
+  k.algorithmicBytes = lowering::countAlgorithmicBytes(g);
+  k.shapeArgs = lowering::buildShapeArgs(g);
+  std::ostringstream note;
+  note << "segment_sum positions=" << positions << " segments=" << segments << " slice=" << slice << " grouped by bucket of " << perBucket
+       << " segments: " << buckets << " buckets, chunks=" << chunks << " of " << chunk << " positions, 5 launches";
   k.scheduleNote = note.str();
   return k;
 }
@@ -573,7 +890,21 @@ LoweredKernel lowerSegmentSumToHip(const OpGraph &g, const LoweringOptions &opti
   // (69 thousand positions into 4954 segments: 0.050 ms grouped, 0.069 ms scanned). Its LDS counters
   // hold one word per segment.
   const bool canGroup = sh.segments <= 16384 && sh.segments * sh.slice + 256 < (1LL << 31);
-  const bool group = options.variant == 2 ? canGroup : options.variant == 1 ? false : canGroup && sh.positions >= (1 << 16);
+  const bool group = options.variant >= 2 ? canGroup : options.variant == 1 ? false : canGroup && sh.positions >= (1 << 16);
+  // Short rows (4, 8 or 12 bytes, 4-byte arithmetic) into many segments: by bucket first. The bucket is the largest power
+  // of two of segments whose output elements number at most 32; there are at most 640 buckets (the counters of a chunk
+  // must leave room for two workgroups per CU) and, unless asked for, at least 96 (the last launch has one workgroup
+  // per bucket: 1 to 4 million positions into 300 segments run 1.3 to 1.9 times slower than grouped by segment; 0.3 to
+  // 4 million into 5000 segments 1.7 to 2.2 times faster, 24.5 million 1.9 times).
+  const int64_t rowBytes = sh.slice * static_cast<int64_t>(dtypeSize(sh.out->dtype));
+  const bool wide = sh.out->dtype == DType::I64 || sh.out->dtype == DType::F64;
+  int bucketBits = 4;
+  while (bucketBits > 0 && (sh.slice << bucketBits) > 32) --bucketBits;
+  const int64_t buckets = (sh.segments + (1LL << bucketBits) - 1) >> bucketBits;
+  const bool canBucket = group && !wide && rowBytes <= 12 && rowBytes % 4 == 0 && bucketBits >= 2 && buckets <= 640 && buckets >= 2;
+  if (canBucket && (options.variant == 3 || options.variant == 4 || (options.variant == 0 && buckets >= 96))) {
+    return lowerSegmentBucketed(g, options, sh, bucketBits);
+  }
   return group ? lowerSegmentSorted(g, options, sh) : lowerSegmentScan(g, options, sh);
 }
 

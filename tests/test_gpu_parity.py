@@ -702,14 +702,16 @@ def test_segment_sum_is_bit_exact(name):
     check_segment_sum(os.path.join(FIXTURES, name), seed=harness.BASE_SEED + 301)
 
 
-@pytest.mark.parametrize("schedule", ["scan", "grouped"])
+@pytest.mark.parametrize("schedule", ["scan", "grouped", "bucketed"])
 def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero(schedule, monkeypatch, tmp_path):
-    """Both schedules (every workgroup scanning all ids; positions grouped by segment first) on the same small case."""
-    monkeypatch.setenv("AKG_HIP_VARIANT", "1" if schedule == "scan" else "2")
+    """The three schedules (every workgroup scanning all ids; positions grouped by segment first; grouped by bucket of
+    eight segments first and by segment in LDS) on the same small case."""
+    monkeypatch.setenv("AKG_HIP_VARIANT", {"scan": "1", "grouped": "2", "bucketed": "3"}[schedule])
     path = os.path.join(FIXTURES, "small_segment_sum_f32_700x3_by_1x3_seg50.info")
     desc = harness.load_desc(path)
     kernel = driver.HipKernel.from_file(path, out_dir=str(tmp_path))
     assert ("grouped by segment" in kernel.source) == (schedule == "grouped")
+    assert ("grouped by bucket" in kernel.source) == (schedule == "bucketed")
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 302)
     ids = inputs[1]
     ids[ids == 17] = 50          # nobody names row 17; 50 and -3 are outside [0, 50)
@@ -739,15 +741,18 @@ def test_segment_sum_with_neighbours_runs_as_stages_and_stays_bit_exact(tmp_path
         assert np.array_equal(got[0].view(np.uint8), expect[0].view(np.uint8)), "launch %d" % launch
 
 
-@pytest.mark.parametrize("pattern", ["one_segment", "sorted", "runs_of_64", "mostly_outside"])
-def test_grouped_segment_sum_on_skewed_ids(pattern):
-    """The grouped schedule where the ids are far from uniform: every position in one segment (every lane of a tile
+@pytest.mark.parametrize("schedule", ["by_segment", "by_bucket"])
+@pytest.mark.parametrize("pattern", ["one_segment", "sorted", "runs_of_64", "mostly_outside", "one_bucket"])
+def test_grouped_segment_sum_on_skewed_ids(pattern, schedule, monkeypatch, tmp_path):
+    """The grouped schedules where the ids are far from uniform: every position in one segment (every lane of a tile
     ranks behind its neighbours, one chain of 300000 additions), ids already sorted (a run touches few segments), whole
-    tiles of equal ids, and nine ids in ten outside [0, segments). Bit-exact against the serial loop."""
+    tiles of equal ids, nine ids in ten outside [0, segments), and every id within one bucket of eight segments.
+    Bit-exact against the serial loop."""
+    monkeypatch.setenv("AKG_HIP_VARIANT", "2" if schedule == "by_segment" else "3")
     path = os.path.join(FIXTURES, "small_segment_sum_f32_300000_by_3_seg5000.info")
     desc = harness.load_desc(path)
-    kernel = driver.HipKernel.from_file(path)
-    assert "grouped by segment" in kernel.source
+    kernel = driver.HipKernel.from_file(path, out_dir=str(tmp_path))
+    assert ("grouped by segment" if schedule == "by_segment" else "grouped by bucket") in kernel.source
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 760)
     ids = inputs[1]
     rng = np.random.default_rng(harness.BASE_SEED + 761)
@@ -757,6 +762,8 @@ def test_grouped_segment_sum_on_skewed_ids(pattern):
         ids[...] = np.sort(ids.reshape(-1)).reshape(ids.shape)
     elif pattern == "runs_of_64":
         ids[...] = np.repeat(rng.integers(0, 5000, size=(ids.size + 63) // 64), 64)[:ids.size].reshape(ids.shape)
+    elif pattern == "one_bucket":
+        ids[...] = rng.integers(4992, 5000, size=ids.shape)
     else:
         outside = rng.random(ids.shape) < 0.9
         ids[outside] = rng.choice(np.array([-1, -70000, 5000, 2 ** 31 - 1], dtype=ids.dtype), size=int(outside.sum()))

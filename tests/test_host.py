@@ -296,10 +296,11 @@ def test_unsorted_segment_sum_translates_and_gets_its_own_family():
     assert k.family == "staged" and "_stage0_kernel" in k.source and "_stage1_kernel" in k.source
 
 
-def test_segment_sum_over_many_positions_is_grouped_by_segment_first(tmp_path):
+def test_segment_sum_over_many_positions_is_grouped_by_segment_first(tmp_path, monkeypatch):
     """From 65536 positions on: four launches that sort the positions by segment (integer counters only) precede the
     kernel proper; they are listed in the artifact's JSON in launch order, and the handle owns the workspace they
     share. Short rows are moved into segment order, wide ones stay where they are."""
+    monkeypatch.setenv("AKG_HIP_VARIANT", "2")
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_300000_by_3_seg5000.info"), out_dir=str(tmp_path))
     meta = json.load(open(os.path.join(str(tmp_path), k.kernel_name[:-len("_kernel")] + ".json")))
     assert k.family == "segment_sum" and "grouped by segment" in meta["schedule"]
@@ -312,17 +313,41 @@ def test_segment_sum_over_many_positions_is_grouped_by_segment_first(tmp_path):
     names = [p["kernelName"] for p in meta["earlier_phases"]]
     stem = k.kernel_name[:-len("_kernel")]
     assert names == [stem + "_count", stem + "_offsets", stem + "_starts", stem + "_place"]
-    assert [p["blockIdx.x"] for p in meta["earlier_phases"]] == [runs, -(-5000 // 16), 1, runs]
+    assert [p["blockIdx.x"] for p in meta["earlier_phases"]] == [runs, -(-(-(-5000 // 16)) // 8) * 8, 1, runs]
     assert meta["kernelName"] == k.kernel_name and meta["workspace_bytes"] == k.workspace_bytes
     for n in names + [k.kernel_name]:
         assert 'void %s(' % n in k.source
     assert "placed[static_cast<long>(at + rank) * UNITS + c] = row[u][c]" in k.source
     # no float atomics anywhere: the only atomic is the integer count in LDS
-    assert k.source.count("atomicAdd(&akg_cnt[id], 1u)") == 1 and k.source.count("atomic") == 1
+    assert k.source.count("atomicAdd(&akg_cnt[key_of(id)], 1u)") == 1 and k.source.count("atomic") == 1
+    monkeypatch.delenv("AKG_HIP_VARIANT")
     wide = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_140000_by_40_seg129.info"), out_dir=None)
     assert "akg_ws[W_SORTED + at + rank] = " in wide.source and "placed" not in wide.source
     small = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_700x3_by_1x3_seg50.info"), out_dir=None)
     assert small.workspace_bytes == 0 and "grouped" not in small.source
+
+
+def test_short_rows_into_many_segments_are_grouped_by_bucket_first(tmp_path):
+    """Rows of 4, 8 or 12 bytes into enough segments for 96 buckets: the positions are sorted by bucket of eight
+    segments, chunk by chunk in LDS, into 16-byte entries {row, segment}; the last launch has one workgroup per bucket
+    and sorts by segment in LDS. Same launch names, integer counters only."""
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_segment_sum_f32_300000_by_3_seg5000.info"), out_dir=str(tmp_path))
+    meta = json.load(open(os.path.join(str(tmp_path), k.kernel_name[:-len("_kernel")] + ".json")))
+    assert k.family == "segment_sum" and "grouped by bucket of 8 segments: 625 buckets" in meta["schedule"]
+    chunks = -(-300000 // 4096)
+    words = chunks * 625 + 625 + 625 + 1
+    words = -(-words // 4) * 4 + 300000 * 4
+    assert k.workspace_bytes == 4 * words
+    stem = k.kernel_name[:-len("_kernel")]
+    assert [p["kernelName"] for p in meta["earlier_phases"]] == [stem + "_count", stem + "_offsets", stem + "_starts", stem + "_place"]
+    assert [p["blockIdx.x"] for p in meta["earlier_phases"]] == [chunks, -(-(-(-625 // 4)) // 8) * 8, 1, -(-chunks // 8) * 8]
+    assert meta["blockIdx.x"] == 625 and meta["threadIdx.x"] == 512
+    assert k.source.count("chunk_sort<NW, KEYS, KEY_BITS, TILES, 1>") == 1 and k.source.count("chunk_sort<NW, S, BUCKET_BITS, TILES, 4>") == 1
+    assert k.source.count("atomic") == 1
+    # few segments, 16-byte rows, 8-byte arithmetic: grouped by segment as before
+    for name in ("small_segment_sum_f16_150001_by_4_seg300.info",):
+        other = driver.HipKernel.from_file(os.path.join(FIXTURES, name), out_dir=None)
+        assert "grouped by segment" in other.source
 
 
 def test_argmax_becomes_a_max_and_a_least_position_in_the_row_family():
