@@ -15,6 +15,7 @@ const char *kernelFamilyName(KernelFamily f) {
     case KernelFamily::RowReduce: return "row_reduce";
     case KernelFamily::GemmEpilogue: return "gemm_epilogue";
     case KernelFamily::StreamReduce: return "stream_reduce";
+    case KernelFamily::ColumnReduce: return "column_reduce";
     case KernelFamily::Indexed: return "indexed";
     case KernelFamily::SegmentSum: return "segment_sum";
     case KernelFamily::Staged: return "staged";
@@ -520,7 +521,20 @@ LoweredKernel lowerToHip(const OpGraph &described, const LoweringOptions &option
   }
   if (wantsIndexedKernel(graph)) return lowerIndexedToHip(graph, options);
   if (hasMatMul) return lowerGemmToHip(graph, options);
-  if (wantsStreamReduce(graph)) return lowerStreamReduceToHip(graph, options);
+  if (wantsStreamReduce(graph)) {
+    // A reduction result that meets the unreduced tensor again is not for the streaming kernels, which keep nothing of
+    // what they read: the column kernel keeps the run in registers, if it fits. Failing both, the first reason stands.
+    try {
+      return lowerStreamReduceToHip(graph, options);
+    } catch (const LoweringError &streaming) {
+      if (options.variant == 7) throw;
+      try {
+        return lowerColumnToHip(graph, options);
+      } catch (const LoweringError &) {
+        throw streaming;
+      }
+    }
+  }
   return lowerTileToHip(graph, options);
 }
 

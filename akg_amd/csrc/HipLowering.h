@@ -31,7 +31,7 @@ class LoweringError : public std::runtime_error {
   explicit LoweringError(const std::string &msg) : std::runtime_error(msg) {}
 };
 
-enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce, Indexed, SegmentSum, Staged };
+enum class KernelFamily { Elementwise, RowReduce, GemmEpilogue, StreamReduce, Indexed, SegmentSum, Staged, ColumnReduce };
 const char *kernelFamilyName(KernelFamily f);
 
 // Tuning knobs; 0 means "let the heuristic decide". They can be set through the environment
@@ -45,7 +45,7 @@ struct LoweringOptions {
   // Experiment switch (AKG_HIP_VARIANT), read by whichever family lowers the kernel; 0 = the measured default.
   //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows
   //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
-  //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs
+  //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs, 7: no column kernel (several kernels instead)
   //   segment_sum    1: every workgroup scans all ids, 2: positions grouped by segment first (whatever the size),
   //                  3: grouped by bucket of segments first (whatever the number of buckets), 4: as 3, chunks in launch order
   //   indexed        1: no LDS-tiled transposes, 2: no chunk-wide loads, 3: launch order of tiles, 5: no non-temporal hints
@@ -91,6 +91,8 @@ LoweredKernel lowerToHip(const OpGraph &graph, const LoweringOptions &options);
 // Family-specific entries used by lowerToHip (HipLoweringGemm.cpp, HipLoweringReduce.cpp, HipLoweringIndexed.cpp).
 LoweredKernel lowerGemmToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerStreamReduceToHip(const OpGraph &graph, const LoweringOptions &options);
+// One reduced axis that is not the innermost one, reduction results used against the unreduced tensor (HipLoweringColumn.cpp).
+LoweredKernel lowerColumnToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerTileToHip(const OpGraph &graph, const LoweringOptions &options);      // elementwise, row_reduce
 LoweredKernel lowerIndexedToHip(const OpGraph &graph, const LoweringOptions &options);
 LoweredKernel lowerSegmentSumToHip(const OpGraph &graph, const LoweringOptions &options);

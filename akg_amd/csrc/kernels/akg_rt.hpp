@@ -769,6 +769,110 @@ AKG_DEV T group_reduce(T v, T *scratch, int tid) {
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Column kernels: a chunk of V columns kept as it came from memory, and reductions whose V lanes are V different runs.
+// ---------------------------------------------------------------------------------------------------------
+template <typename DT, int V>
+struct PackedChunk {
+  static constexpr int kBytes = static_cast<int>(sizeof(typename DT::storage)) * V;
+  static_assert(kBytes <= 16, "a packed chunk is one memory access");
+  typename Raw<kBytes>::type raw;
+};
+
+template <typename DT, int V, bool NT = false>
+AKG_DEV void load_packed(const typename DT::storage *__restrict__ p, PackedChunk<DT, V> &dst) {
+  typedef typename Raw<PackedChunk<DT, V>::kBytes>::type R;
+  const R *rp = reinterpret_cast<const R *>(p);
+  dst.raw = NT ? __builtin_nontemporal_load(rp) : *rp;
+}
+
+template <typename DT, int V>
+AKG_DEV void zero_packed(PackedChunk<DT, V> &dst) {
+  dst.raw = {};
+}
+
+// The first n elements of a chunk that is only element-aligned (n = V: one unaligned access); the rest is zero.
+template <typename DT, int V>
+AKG_DEV void load_packed_partial(const typename DT::storage *__restrict__ p, int n, PackedChunk<DT, V> &dst) {
+  typename DT::storage tmp[V];
+  if (n == V) {
+    __builtin_memcpy(tmp, p, sizeof(tmp));
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) tmp[e] = e < n ? p[e] : typename DT::storage();
+  }
+  __builtin_memcpy(&dst.raw, tmp, sizeof(tmp));
+}
+
+template <typename DT, int V>
+AKG_DEV void unpack_packed(const PackedChunk<DT, V> &src, typename DT::compute (&dst)[V]) {
+  typename DT::storage tmp[V];
+  __builtin_memcpy(tmp, &src.raw, sizeof(tmp));
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(tmp[e]);
+}
+
+// The first n elements of a chunk to an address that is only element-aligned.
+template <typename DT, int V>
+AKG_DEV void store_chunk_partial(typename DT::storage *__restrict__ p, int n, const typename DT::compute (&src)[V]) {
+  if (n == V) {
+    store_chunk_unaligned<DT, V>(p, src);
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      if (e < n) p[e] = DT::store(src[e]);
+    }
+  }
+}
+
+// Thread tid = ly * LX + lx of a workgroup of BLOCK threads holds V partial results for the columns of lx; on return
+// every thread holds the results over all ly. Partners inside a wavefront first (lanes LX, 2 LX, ... apart hold the
+// same columns), then the wavefronts through `scratch` ((BLOCK / 64) * LX * V values; the caller alternates between
+// two such arrays from one reduction to the next, so one barrier per reduction suffices). ROUND: DT::rnd after every
+// step, which keeps a narrow result type's rounding (sums and products; a maximum is one of its operands).
+template <typename Red, typename DT, bool ROUND, typename T>
+AKG_DEV T column_step(T a, T b) {
+  if constexpr (ROUND) {
+    return DT::rnd(Red::apply(a, b));
+  } else {
+    return Red::apply(a, b);
+  }
+}
+
+template <typename Red, typename DT, bool ROUND, int LX, int BLOCK, int V>
+AKG_DEV void column_reduce(typename DT::compute (&acc)[V], typename DT::compute *scratch, int tid) {
+  static_assert(LX <= kWaveSize && (LX & (LX - 1)) == 0 && BLOCK % kWaveSize == 0, "column groups are powers of two within a wavefront");
+  typedef typename DT::compute T;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    T v = acc[e];
+    if constexpr (LX <= 1) v = column_step<Red, DT, ROUND>(v, lane_partner<1>(v));
+    if constexpr (LX <= 2) v = column_step<Red, DT, ROUND>(v, lane_partner<2>(v));
+    // (lane_partner<4> and <8> mirror their groups, which is no good here: the partner must hold the same columns)
+    if constexpr (LX <= 4) v = column_step<Red, DT, ROUND>(v, static_cast<T>(__shfl_xor(v, 4)));
+    if constexpr (LX <= 8) v = column_step<Red, DT, ROUND>(v, static_cast<T>(__shfl_xor(v, 8)));
+    if constexpr (LX <= 16) v = column_step<Red, DT, ROUND>(v, lane_partner<16>(v));
+    if constexpr (LX <= 32) v = column_step<Red, DT, ROUND>(v, lane_partner<32>(v));
+    acc[e] = v;
+  }
+  if constexpr (BLOCK > kWaveSize) {
+    constexpr int kWaves = BLOCK / kWaveSize;
+    const int wave = tid / kWaveSize, lane = tid % kWaveSize, lx = tid % LX;
+    if (lane < LX) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) scratch[(wave * LX + lx) * V + e] = acc[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      T r = scratch[lx * V + e];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) r = column_step<Red, DT, ROUND>(r, scratch[(w * LX + lx) * V + e]);
+      acc[e] = r;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // Workspace protocol of the streaming reductions. Several workgroups share one group of outputs; each leaves
 // its partial result in device memory and counts its arrival; the workgroup that arrives last reads all the
 // partials back (in slot order, so the result does not depend on the arrival order) and finishes the job.

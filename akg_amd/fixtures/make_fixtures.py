@@ -148,6 +148,10 @@ FIXTURES = {
     "n1_biasgrad_bf16_16384x4096": lambda n: op_desc.bias_grad(16384, 4096, "bfloat16", n),
     # the shape of the reference's largest UnsortedSegmentSum description: 24.5 million positions of 3 floats into 4954 rows
     "n7_segment_sum_f32_4954x4953_by_1x3_seg4954": lambda n: op_desc.unsorted_segment_sum([4954, 4953], [1, 3], 4954, "float32", "int32", n),
+    # reductions over an axis that is not the innermost one, whose results meet the tensor again (column kernel, or one
+    # kernel per reduction level): a softmax over the 21 classes of a segmentation map, a channels-first LayerNorm
+    "n8_softmax_axis1_f16_32x21x512x512": lambda n: op_desc.softmax_over_axis([32, 21, 512, 512], 1, "float16", n),
+    "n9_layernorm_axis1_bf16_64x768x1024": lambda n: op_desc.layernorm_over_axis1(64, 768, 1024, "bfloat16", 1e-5, n),
 }
 
 

@@ -60,7 +60,14 @@ WORKLOADS = {
     "n6_gemm_bf16_bias_gelu_16x8192x8192": "bf16",
     # 24.5 million index positions of 3 floats added into 4954 rows in the serial order (five launches per step)
     "n7_segment_sum_f32_4954x4953_by_1x3_seg4954": "f32",
+    # reductions over an axis that is not the innermost one whose results meet the tensor again: the column kernel keeps
+    # the reduced run in registers (one read, one write); per_config also times the same description as one kernel per
+    # reduction level (three reads)
+    "n8_softmax_axis1_f16_32x21x512x512": "f32",
+    "n9_layernorm_axis1_bf16_64x768x1024": "f32",
 }
+# workloads also measured on the schedule of several kernels (AKG_HIP_VARIANT=7 while the handle is built)
+SEVERAL_KERNELS = ("n8_softmax_axis1_f16_32x21x512x512", "n9_layernorm_axis1_bf16_64x768x1024")
 DEFAULT_WORKLOAD = "c2_softmax_f16_8192x4096"
 # plain streaming kernel of known size (out = -x, 256 MiB in + 256 MiB out): calibrates the HBM traffic counters
 CALIBRATION = "calib_neg_f32_16384x4096"
@@ -138,10 +145,22 @@ def timed(launch, steps, warmup, torch, groups=True):
     return wall_ms, mean_ms, statistics.median(per), min(per)
 
 
-def gpu_measure(name, steps, warmup, torch, driver, harness, np, resident=False):
+def gpu_measure(name, steps, warmup, torch, driver, harness, np, resident=False, variant=None):
     path = os.path.join(FIXTURES, name + ".info")
     desc = harness.load_desc(path)
-    kernel = driver.HipKernel.from_file(path)
+    if variant is None:
+        kernel = driver.HipKernel.from_file(path)
+    else:
+        # another schedule of the same description: built without artifacts, so that the cached default stays
+        before = os.environ.get("AKG_HIP_VARIANT")
+        os.environ["AKG_HIP_VARIANT"] = str(variant)
+        try:
+            kernel = driver.HipKernel.from_file(path, out_dir=None)
+        finally:
+            if before is None:
+                del os.environ["AKG_HIP_VARIANT"]
+            else:
+                os.environ["AKG_HIP_VARIANT"] = before
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 1)
     dev = torch.device("cuda:0")
     per_set = sum(t.nbytes for t in kernel.tensors)
@@ -348,6 +367,13 @@ def main():
                     r = roofline_of(k2, rms, other)
                     entry["cache_resident"] = {"kernel_ms": round(rms, 5), "kernel_ms_min": round(rmin, 5),
                                                "achieved": r["achieved"], "unit": r["unit"], "frac_of_hbm_peak": r["frac"]}
+                if other in SEVERAL_KERNELS:
+                    k3, _, _, sms, smed, smin, _ = gpu_measure(other, max(20, args.steps // 4), max(5, args.warmup // 2), torch,
+                                                               driver, harness, np, variant=7)
+                    r = roofline_of(k3, sms, other)
+                    entry["several_kernels"] = {"family": k3.family, "kernel_ms": round(sms, 5), "kernel_ms_median": round(smed, 5),
+                                                "kernel_ms_min": round(smin, 5), "achieved": r["achieved"], "unit": r["unit"],
+                                                "frac": r["frac"]}
                 if other in CPU_SAMPLES and not args.no_cpu_baseline:
                     entry["cpu_baseline"] = line["cpu_baseline"] if other == name else cpu_baseline(other, harness, driver)
                 per[other] = entry

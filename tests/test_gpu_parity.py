@@ -99,17 +99,28 @@ def check_stream_reduction(path, seed, repeats=1, family="stream_reduce"):
             assert ok, "%s output %s: %s" % (os.path.basename(path), d.name, msg)
 
 
-@pytest.mark.parametrize("name", STAGED)
-def test_descriptions_cut_into_several_kernels_match_the_oracle(name):
-    """A softmax or a normalisation over an outer axis, batch-norm statistics and their use in one description: no
-    single kernel serves them, so the handle runs one kernel per reduction level (temporaries in its workspace).
-    float32 results against the float64 evaluation (the sums are reassociated), 16-bit ones against the serial
-    oracle; three launches of one handle."""
+# a softmax / LayerNorm over ONE outer axis: the column kernel keeps the reduced run in registers (one kernel, one read)
+COLUMN = [n for n in STAGED if "softmax" in n or "layernorm" in n]
+
+
+@pytest.mark.parametrize("name,schedule", [(n, "default") for n in STAGED] + [(n, "several_kernels") for n in COLUMN])
+def test_descriptions_cut_into_several_kernels_match_the_oracle(name, schedule, monkeypatch, tmp_path):
+    """A softmax or a normalisation over an outer axis, batch-norm statistics and their use in one description: the
+    streaming reductions cannot serve them. One reduced axis whose run fits a workgroup's registers goes to the column
+    kernel (one kernel); otherwise, or when asked for, the handle runs one kernel per reduction level (temporaries in
+    its workspace). float32 results against the float64 evaluation (the sums are reassociated), 16-bit ones against the
+    serial oracle; three launches of one handle."""
     from oracle import np_ref
     path = os.path.join(FIXTURES, name)
     desc = harness.load_desc(path)
-    kernel = driver.HipKernel.from_file(path)
-    assert kernel.family == "staged" and kernel.source.count("extern \"C\" __global__") >= 2
+    if schedule == "several_kernels":
+        monkeypatch.setenv("AKG_HIP_VARIANT", "7")
+    kernel = driver.HipKernel.from_file(path, out_dir=str(tmp_path))
+    print("case %s %s: %s grid %d block %d" % (name, schedule, kernel.family, kernel.grid[0], kernel.block[0]), flush=True)
+    if name in COLUMN and schedule == "default":
+        assert kernel.family == "column_reduce" and kernel.source.count("extern \"C\" __global__") == 1 and kernel.workspace_bytes == 0
+    else:
+        assert kernel.family == "staged" and kernel.source.count("extern \"C\" __global__") >= 2
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 730)
     serial = cpu_ref.CpuKernel(path)(inputs)
     wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
@@ -132,10 +143,98 @@ def test_descriptions_cut_into_several_kernels_match_the_oracle(name):
         assert np.array_equal(np.ascontiguousarray(g).view(np.uint8), h.view(np.uint8))
 
 
-def test_dynamic_description_that_needs_several_kernels(tmp_path):
-    """A softmax over axis 1 with an open leading dimension: every shape set is specialised into its own sequence of
-    kernels (stage artifacts carry the shape digest); results against the oracle of the same description written with
-    the bound shape."""
+def _column_cases():
+    """name -> (builder function, family expected)"""
+    def l2_normalise_no_keep(b):
+        # x / sqrt(sum(x * x) over axis 1): the reduction drops its axis and a Reshape puts it back
+        x = b.input([6, 37, 50], "float32")
+        ss = b.reduce("ReduceSum", b.mul(x, x), [1], False)
+        return [b.div(x, b.unary("Sqrt", b.reshape(ss, [6, 1, 50])))]
+
+    def centred_with_statistics(b):
+        # three outputs: the centred tensor, the mean [4,1,9,8] and the greatest centred value per column
+        x = b.input([4, 23, 9, 8], "float16")
+        xf = b.cast(x, "float32")
+        mean = b.mul(b.reduce("ReduceSum", xf, [1], True), b.const(1.0 / 23, "float32"))
+        xc = b.sub(xf, mean)
+        return [b.cast(xc, "float16"), mean, b.reduce("ReduceMax", xc, [1], True)]
+
+    def scaled_by_a_shared_plane(b):
+        # an operand [1, 19, 6] that every outer index shares, one value per outer index [7,1,1], an inner axis of 6
+        x = b.input([7, 19, 6], "float32")
+        w = b.input([1, 19, 6], "float32")
+        g = b.input([7, 1, 1], "float32")
+        y = b.mul(b.mul(x, w), g)
+        return [b.sub(y, b.reduce("ReduceMin", y, [1], True))]
+
+    def integer_range(b):
+        x = b.input([3, 130, 20], "int32")
+        lo, hi = b.reduce("ReduceMin", x, [1], True), b.reduce("ReduceMax", x, [1], True)
+        return [b.sub(x, lo), b.sub(hi, lo)]
+
+    def narrow_columns(b):
+        # two columns only: the threads of a wavefront that share a column are 2, 4, ... 32 lanes apart
+        x = b.input([5, 300, 2], "float32")
+        return [b.div(x, b.reduce("ReduceSum", b.unary("Abs", x), [1], True))]
+
+    def half_sums(b):
+        # the sum is declared float16: rounded after every addition, in the kernel's order
+        x = b.input([2, 40, 24], "float16")
+        return [b.sub(x, b.reduce("ReduceMax", x, [1], True)), b.reduce("ReduceSum", x, [1], True)]
+
+    def run_too_long_for_registers(b):
+        x = b.input([2, 20000, 64], "float32")
+        return [b.sub(x, b.reduce("ReduceMax", x, [1], True))]
+
+    return {"l2_normalise_no_keep": (l2_normalise_no_keep, "column_reduce"), "centred_with_statistics": (centred_with_statistics, "column_reduce"),
+            "scaled_by_a_shared_plane": (scaled_by_a_shared_plane, "column_reduce"), "integer_range": (integer_range, "column_reduce"),
+            "narrow_columns": (narrow_columns, "column_reduce"), "half_sums": (half_sums, "column_reduce"),
+            "run_too_long_for_registers": (run_too_long_for_registers, "staged")}
+
+
+@pytest.mark.parametrize("case", sorted(_column_cases()))
+def test_reductions_over_a_middle_axis_whose_results_meet_the_tensor_again(case):
+    """The column kernel on shapes that stress its layout: a reduction without keep_dims and the Reshape that follows,
+    outputs of the reduced shape next to full ones, operands that broadcast over the outer or the inner axes, integer
+    data, two columns only, a 16-bit sum, and a run too long for a workgroup's registers (several kernels instead).
+    float32 sums against the float64 evaluation, everything else against the oracle bit for bit or to its tolerance."""
+    from oracle import np_ref
+    build, family = _column_cases()[case]
+    b = op_desc.DescBuilder("column_" + case)
+    text = b.dumps(build(b))
+    desc = json_loads(text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    print("case %s: %s grid %d block %d" % (case, kernel.family, kernel.grid[0], kernel.block[0]), flush=True)
+    assert kernel.family == family
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 790)
+    expect = np_ref.evaluate(desc, inputs)
+    wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+    exact = np_ref.evaluate(harness.widen_to_float64(desc), wide)
+    run = max(e[0]["shape"][1] for e in desc["input_desc"])
+    sums = any(o["name"] == "ReduceSum" for o in desc["op_desc"])
+    for launch in range(2):
+        got = run_on_gpu(kernel, inputs)
+        for d, g, e, x in zip(kernel.outputs, got, expect, exact):
+            if d.dtype == "float32" and sums:
+                ok, msg = harness.compare_reassociated(g, x, d.dtype, run)
+            elif case == "half_sums" and d.name == kernel.outputs[1].name:
+                # 40 float16 additions in another order than the serial loop's: each within half an ulp of its partial sum
+                err = np.abs(g.astype(np.float64) - np.asarray(x, dtype=np.float64))
+                bound = 40 * 2.0 ** -11 * np.abs(inputs[0].astype(np.float64)).sum(axis=1, keepdims=True)
+                ok, msg = bool((err <= bound).all()), "max error %.3g (bound %.3g)" % (err.max(), bound.min())
+            else:
+                ok, msg = harness.compare(g, e, d.dtype)
+            print("  launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
+            assert ok, "%s output %s: %s" % (case, d.name, msg)
+
+
+@pytest.mark.parametrize("schedule", ["column_reduce", "staged"])
+def test_dynamic_description_that_needs_several_kernels(schedule, tmp_path, monkeypatch):
+    """A softmax over axis 1 with an open leading dimension: every shape set is specialised into its own column kernel
+    or, with that kernel switched off, its own sequence of kernels (stage artifacts carry the shape digest); results
+    against the oracle of the same description written with the bound shape."""
+    if schedule == "staged":
+        monkeypatch.setenv("AKG_HIP_VARIANT", "7")
     text = op_desc.softmax_over_axis([32, 12, 24, 40], 1, "float32", "dyn_softmax_axis1")
     d = json_loads(text)
 
@@ -152,7 +251,7 @@ def test_dynamic_description_that_needs_several_kernels(tmp_path):
     dyn = driver.HipDynamicKernel(__import__("json").dumps(d), out_dir=str(tmp_path))
     for lead in (32, 7, 32):
         kernel = dyn.specialize([[lead, 12, 24, 40]])
-        assert kernel.family == "staged" and [t.shape for t in kernel.tensors] == [[lead, 12, 24, 40]] * 2
+        assert kernel.family == schedule and [t.shape for t in kernel.tensors] == [[lead, 12, 24, 40]] * 2
         static = op_desc.softmax_over_axis([lead, 12, 24, 40], 1, "float32", "static_softmax_axis1_%d" % lead)
         path = os.path.join(str(tmp_path), "static_%d.info" % lead)
         open(path, "w").write(static)
@@ -161,7 +260,8 @@ def test_dynamic_description_that_needs_several_kernels(tmp_path):
         expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
         ok, msg = harness.compare(got[0], expect[0], "float32")
         assert ok, "leading dimension %d: %s" % (lead, msg)
-    assert len([f for f in os.listdir(str(tmp_path)) if f.startswith("dyn_softmax_axis1_stage0_s") and f.endswith(".hsaco")]) == 2
+    stem = "dyn_softmax_axis1_stage0_s" if schedule == "staged" else "dyn_softmax_axis1_s"
+    assert len([f for f in os.listdir(str(tmp_path)) if f.startswith(stem) and f.endswith(".hsaco")]) == 2
 
 
 @pytest.mark.parametrize("name", STREAM)

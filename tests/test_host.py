@@ -148,12 +148,16 @@ def test_error_conventions():
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(_desc(lambda d: d["op_desc"][0]["input_desc"][0][0].update(tensor_name="nowhere")), out_dir=None)
     assert e.value.code == -3 and "nowhere" in str(e.value)
-    # a reduced value that meets an unreduced one along an outer axis needs a second pass: such a description runs as
-    # several kernels, unless it also holds an op that is not cut (an Assign), and then both reasons are given
+    # a reduced value that meets an unreduced one along an outer axis: the column kernel keeps the reduced run in
+    # registers; what it does not take (a run too long, an Assign) needs a second pass and runs as several kernels,
+    # unless it also holds an op that is not cut, and then both reasons are given
     b = op_desc.DescBuilder("Fused_ReduceMax_Sub_axis0")
     x = b.input([64, 128], "float32")
     text = b.dumps([b.sub(x, b.reduce("ReduceMax", x, [0], True))])
-    assert driver.HipKernel(text, out_dir=None).family == "staged"
+    assert driver.HipKernel(text, out_dir=None).family == "column_reduce"
+    b = op_desc.DescBuilder("Fused_ReduceMax_Sub_axis0_long")
+    x = b.input([40000, 128], "float32")
+    assert driver.HipKernel(b.dumps([b.sub(x, b.reduce("ReduceMax", x, [0], True))]), out_dir=None).family == "staged"
     b = op_desc.DescBuilder("Fused_ReduceMax_Sub_Assign_axis0")
     x = b.input([64, 128], "float32")
     a = b.op("Assign", [x, b.sub(x, b.reduce("ReduceMax", x, [0], True))], [64, 128], "float32")
@@ -650,15 +654,20 @@ def test_description_no_single_kernel_serves_is_cut_at_its_reduction_results(tmp
     assert one.family == "row_reduce"
 
 
-def test_descriptions_that_cannot_be_cut_say_both_reasons():
+def test_descriptions_that_cannot_be_cut_say_both_reasons(monkeypatch):
     """Staging refuses what it cannot order or name: an output listed twice (two kernels would write one buffer) keeps the
-    single-kernel refusal and adds its own reason; nothing crashes."""
+    single-kernel refusal and adds its own reason; nothing crashes. (The column kernel serves this description - it
+    stores the value to both buffers - so it is switched off here.)"""
     b = op_desc.DescBuilder("twice_listed_outer_softmax")
     x = b.input([64, 128], "float32")
     y = b.sub(x, b.reduce("ReduceMax", x, [0], True))
+    k = driver.HipKernel(b.dumps([y, y]), out_dir=None)
+    assert k.family == "column_reduce" and "out0 + " in k.source and "out1 + " in k.source
+    monkeypatch.setenv("AKG_HIP_VARIANT", "7")
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(b.dumps([y, y]), out_dir=None)
     assert e.value.code == -4 and "second pass" in str(e.value) and "listed twice" in str(e.value)
+    monkeypatch.delenv("AKG_HIP_VARIANT")
     # an op outside the op table is refused before any cut is tried
     d = json.loads(op_desc.softmax_over_axis([8, 16], 0, "float32", "unknown_op_outer"))
     d["op_desc"][1]["name"] = "Frobnicate"
@@ -667,7 +676,7 @@ def test_descriptions_that_cannot_be_cut_say_both_reasons():
     assert e.value.code in (-3, -4) and "Frobnicate" in str(e.value)
 
 
-def test_matmul_next_to_a_softmax_is_cut_behind_the_contraction(tmp_path):
+def test_matmul_next_to_a_softmax_is_cut_behind_the_contraction(tmp_path, monkeypatch):
     """Attention probabilities in one description: the contraction (with nothing fused behind it) leaves the float32
     scores in the workspace, and everything behind it, scale, mask and softmax, is ONE row kernel: the cut is made
     behind contractions and data-movement ops first, and at reductions only where a piece still needs it."""
@@ -684,11 +693,46 @@ def test_matmul_next_to_a_softmax_is_cut_behind_the_contraction(tmp_path):
     x = b.input([64, 96], "float32")
     t = op_desc.transpose(b, x, [1, 0])
     e = b.unary("Exp", b.sub(t, b.reduce("ReduceMax", t, [0], True)))
-    k = driver.HipKernel(b.dumps([b.div(e, b.reduce("ReduceSum", e, [0], True))]), out_dir=str(tmp_path))
+    text = b.dumps([b.div(e, b.reduce("ReduceSum", e, [0], True))])
+    k = driver.HipKernel(text, out_dir=str(tmp_path))
     meta = json.load(open(os.path.join(str(tmp_path), "transpose_then_softmax_axis0.json")))
+    # the softmax over axis 0 of the transposed tensor is one column kernel ...
+    assert [s["kernelName"] for s in meta["stages"]] == ["transpose_then_softmax_axis0_stage%d_kernel" % i for i in range(2)]
+    assert json.load(open(os.path.join(str(tmp_path), "transpose_then_softmax_axis0_stage1.json")))["family"] == "column_reduce"
+    assert k.workspace_bytes == 96 * 64 * 4
+    # ... and three kernels without it
+    monkeypatch.setenv("AKG_HIP_VARIANT", "7")
+    other = os.path.join(str(tmp_path), "several")
+    os.makedirs(other)
+    k = driver.HipKernel(text, out_dir=other)
+    meta = json.load(open(os.path.join(other, "transpose_then_softmax_axis0.json")))
     assert [s["kernelName"] for s in meta["stages"]] == ["transpose_then_softmax_axis0_stage0_kernel"] + [
         "transpose_then_softmax_axis0_stage1_stage%d_kernel" % i for i in range(3)]
     assert k.workspace_bytes == 96 * 64 * 4 + 256 + 256
+
+
+def test_column_kernel_schedule():
+    """One reduced axis that is not the innermost one, results used against the tensor: [O, R, I] with a workgroup per
+    strip of columns; the chunks of a thread's rows stay in registers as loaded (the workgroup grows until they fit), one
+    walk per reduction level, no workspace."""
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n9_layernorm_axis1_bf16_64x768x1024.info"), out_dir=None)
+    assert k.family == "column_reduce" and k.workspace_bytes == 0 and (k.grid[0], k.block[0]) == (64 * 16, 512)
+    assert "constexpr int V = 8, LX = 8, LY = 64, CH = 12, BLOCK = 512;" in k.source and "// ---- walk 2 ----" in k.source
+    assert k.source.count("akg::column_reduce<akg::RedSum, akg::f32, false, LX, BLOCK, V>") == 2
+    assert "akg::PackedChunk<akg::bf16, V> p_in0[CH];" in k.source and k.source.count("global__") == 1
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n8_softmax_axis1_f16_32x21x512x512.info"), out_dir=None)
+    assert (k.grid[0], k.block[0]) == (32 * 512, 256) and "LX = 64, LY = 4, CH = 6" in k.source
+    # rows that are not a multiple of the chunk: element-aligned accesses, the last chunk partly outside
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_staged_layernorm_axis1_bf16_8x64x49.info"), out_dir=None)
+    assert "load_packed_partial<akg::bf16, V>(akg_p, akg_row_ok[j] ? akg_cols : 0" in k.source and "store_chunk_partial" in k.source
+    # a 16-bit sum keeps its rounding per step, a maximum needs none
+    b = op_desc.DescBuilder("column_half")
+    x = b.input([2, 40, 24], "float16")
+    k = driver.HipKernel(b.dumps([b.sub(x, b.reduce("ReduceMax", x, [1], True)), b.reduce("ReduceSum", x, [1], True)]), out_dir=None)
+    assert "column_reduce<akg::RedSum, akg::f16, true," in k.source and "column_reduce<akg::RedMax, akg::f16, false," in k.source
+    # two reduced axes around a kept one (batch-norm statistics and their use) are not for this kernel
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_staged_bn_train_forward_f32_16x8x14x14.info"), out_dir=None)
+    assert k.family == "staged"
 
 
 def test_skinny_matmul_gets_the_streaming_kernel():

@@ -23,7 +23,7 @@ SEQUENCES = [
     ("small_biasgrad_bf16_2048x1024.info", "small_reducey_max_f16_130x66.info"),
     ("small_reducey_sqsum_f32_1x5100x3072.info", "small_reduceall_sqsum_f32_768x512.info"),
     ("small_gemm_i8_dequant_bias_gelu_300x2064x520_tb.info", "small_gemm_bf16_bias_gelu_256x512x256.info"),
-    ("small_staged_softmax_f32_32x12x24x40_axis1.info", "small_staged_layernorm_axis1_bf16_8x64x49.info"),
+    ("small_staged_bn_train_forward_f32_16x8x14x14.info", "small_staged_bn_train_forward_bf16_8x6x7x12.info"),
     ("small_segment_sum_f16_150001_by_4_seg300.info", "small_bnstats_f32_32x16x28x28.info"),
 ]
 
