@@ -11,7 +11,7 @@
  * Entry points (plain C, asynchronous on the given stream; the caller times them with events):
  *   akg_probe_mfma_i8 / akg_probe_mfma_bf16 (stream, operands, iterations, workgroups, sink)
  *     operands: device buffer of at least 24 KiB (24 fragments of 64 lanes x 16 bytes), sink: workgroups * 512 ints
- *     work done = workgroups * 8 wavefronts * iterations * 32 MFMAs * 65536 ops
+ *     work done = workgroups * 8 wavefronts * iterations * 32 MFMAs * 65536 ops (int8, 32 x 32 x 32) or 32768 (bf16, 32 x 32 x 16)
  */
 #include <hip/hip_runtime.h>
 

@@ -267,8 +267,9 @@ def calibration(torch, driver, harness, np, steps, warmup):
                                                         harness.f32_to_bf16_bits((rng.standard_normal(12 * 1024) * 0.25).astype(np.float32)).view(np.uint8),
                                                         BF16_MFMA_PEAK_TFLOPS, "TFLOP/s"),
         }
-        ops = workgroups * 8 * iterations * 32 * 65536
         for label, (fn, host, peak, unit) in operands.items():
+            # 32 MFMAs per wavefront and iteration: 32 x 32 x 32 int8 (65536 ops each) or 32 x 32 x 16 bf16 (32768)
+            ops = workgroups * 8 * iterations * 32 * (65536 if "i8" in label else 32768)
             buf = torch.from_numpy(np.ascontiguousarray(host)).to(dev)
             _, mean_ms, med_ms, min_ms = timed(lambda i: fn(st, buf.data_ptr(), iterations, workgroups, sink.data_ptr()),
                                                max(10, steps // 10), 2, torch)
