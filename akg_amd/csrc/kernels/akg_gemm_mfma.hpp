@@ -15,8 +15,13 @@
  *   global -> registers -> LDS, double buffered in LDS (one barrier per K step); the global loads of step
  *   i+1 are issued before the MFMAs of step i.
  *   A: each thread moves 4 x 16 bytes (16 consecutive k of one row) straight into LDS.
- *   B (not transposed) is row-major along N but the MFMA wants, per lane, 16 consecutive k of one column.
- *   Each thread therefore loads a 16(k) x 4(n) byte block as 16 dwords, transposes it in registers with
+ *   B (not transposed) is row-major along N but the MFMA wants, per lane, 16 consecutive k of one column. By default
+ *   (TRB) its tile goes to LDS as it lies in memory, 16-byte chunks of a k-row, and the fragments are read with the
+ *   transposing LDS reads of gfx950 (ds_read_b64_tr_b8 / _b16: sixteen lanes hand in 8 bytes of a k-row each and get
+ *   back, per column, 8 or 4 consecutive k); the staging of both operands is then a plain copy, spread over the
+ *   substeps, and the order of MFMAs, LDS accesses and loads inside a substep is fixed with scheduling groups
+ *   (int8 4096 x 8192 x 8192: 0.428 -> 0.463 of the MFMA peak, bfloat16: 0.465 -> 0.516; MFMA units busy 58 -> 68 %).
+ *   Without TRB each thread loads a 16(k) x 4(n) byte block as 16 dwords, transposes it in registers with
  *   v_perm_b32 (8 permutes per 4 x 4 sub-block) and writes four 16-byte k-vectors to LDS.
  *   LDS rows are 128 data bytes + 16 pad bytes: with a row pitch of 144 bytes consecutive rows start in
  *   different 16-byte bank groups, and the ds_read_b128 fragment loads are conflict free (SQ_LDS_BANK_CONFLICT reads 0).
@@ -95,7 +100,27 @@ AKG_DEV u32 pack_hi16(u32 x, u32 y) { return __builtin_amdgcn_perm(y, x, 0x07060
 // tile, then kPartRows x 256 accumulators per tile and split), and the last one to arrive adds the partials in split
 // order and runs the epilogue: deterministic, and the weight matrix is still read exactly once. The launch has
 // KSPLIT times the workgroups; the counters are left at zero.
-template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1>
+// Instruction order of a substep of 8 MFMAs with R LDS reads, W LDS writes and L memory loads beside them: after every
+// MFMA its share of the others, reads first. (Scheduling-group barriers: the compiler orders the instructions of the
+// region to match the sequence of groups, as far as their dependences allow.)
+template <int R, int W, int L, int M = 0>
+struct SubstepOrder {
+  static constexpr int kAll = R + W + L;
+  static constexpr int kFrom = M * kAll / 8, kUpto = (M + 1) * kAll / 8;
+  static constexpr int within(int lo, int hi) {
+    const int a = kFrom > lo ? kFrom : lo, b = kUpto < hi ? kUpto : hi;
+    return b > a ? b - a : 0;
+  }
+  static AKG_DEV void emit() {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (within(0, R) > 0) __builtin_amdgcn_sched_group_barrier(0x100, within(0, R), 0);
+    if constexpr (within(R, R + W) > 0) __builtin_amdgcn_sched_group_barrier(0x200, within(R, R + W), 0);
+    if constexpr (within(R + W, kAll) > 0) __builtin_amdgcn_sched_group_barrier(0x020, within(R + W, kAll), 0);
+    if constexpr (M < 7) SubstepOrder<R, W, L, M + 1>::emit();
+  }
+};
+
+template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1, bool TRB = false>
 AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi,
                           unsigned *__restrict__ ws = nullptr) {
   constexpr int EB = Mma::kElemBytes;
@@ -128,6 +153,18 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   constexpr long kSteps = (K + BK - 1) / BK;
   constexpr bool kFull = (M % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
   constexpr int kTileBytes = kGemmBM * kPitch;        // one operand tile in LDS
+  // TRB: a row-major B goes to LDS as it lies in memory, k-rows of 256 columns, and the fragments are read with the
+  // transposing LDS reads (ds_read_b64_tr_b8 / _b16): no transposes in registers.
+  static_assert(!(TRB && TRANSB), "the transposing reads are for a row-major B");
+  constexpr int kRowBytesB = kGemmBN * EB;            // bytes of one k-row of the B tile
+  // Row pitch: the 16 lanes of a transposing read hand in 8 rows x 16 bytes (8-bit) or 4 rows x 32 bytes (16-bit), and the
+  // neighbouring 16 lanes the 16 or 32 bytes beside them; with rows 32 (64) bytes apart modulo the 256 bytes of the
+  // banks, the two groups of a half wavefront interleave without sharing a bank.
+  constexpr int kPitchB = kRowBytesB + (EB == 1 ? 32 : 64);
+  constexpr int kRowsB = BK / EB;                     // k-rows per step
+  constexpr int kChunksPerRowB = kRowBytesB / 16;
+  constexpr int kRowStepB = kStageThreads / kChunksPerRowB;
+  static_assert(!TRB || kRowsB * kPitchB <= kTileBytes, "the row-major B tile must fit the operand's LDS space");
 
   __shared__ __attribute__((aligned(16))) u8 lds[2][2][kTileBytes];  // [buffer][A|B]
 
@@ -195,6 +232,9 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
                            : static_cast<int>((bKq * kBlockRows) * NB + (n0 + 4 * bN4) * EB);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  const int bRowT = ltid / kChunksPerRowB;     // + kRowStepB * i
+  const int bChunkT = ltid % kChunksPerRowB;
+  const int bVoffT = static_cast<int>(bRowT * NB + n0 * EB + bChunkT * 16);
 
   auto loadRows = [&](__amdgpu_buffer_rsrc_t rsrc, int voff, long rowBase, long rowLimit, long k0,
                       v4i (&dst)[kRowChunks]) {
@@ -233,6 +273,18 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
     if constexpr (TRANSB) {
       loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.y);
+    } else if constexpr (TRB) {
+      // kRowChunks chunks of 16 bytes along n: k-rows bRowT + kRowStepB * i of the step
+#pragma unroll
+      for (int i = 0; i < kRowChunks; ++i) {
+        const long krow = k0 / EB + bRowT + kRowStepB * i;
+        if (kFull || (krow < KE && n0 * EB + bChunkT * 16 < NB)) {
+          const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoffT, static_cast<int>((k0 / EB + kRowStepB * i) * NB), 0);
+          st.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
+        } else {
+          st.y[i] = v4i{0, 0, 0, 0};
+        }
+      }
     } else {
       loadBlock(k0, st.y);
     }
@@ -311,6 +363,11 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     storeRowsA(la, st.x);
     if constexpr (TRANSB) {
       storeRowsBt(lb, st.y);
+    } else if constexpr (TRB) {
+#pragma unroll
+      for (int i = 0; i < kRowChunks; ++i) {
+        *reinterpret_cast<v4i *>(lb + (bRowT + kRowStepB * i) * kPitchB + bChunkT * 16) = st.y[i];
+      }
     } else {
       storeBlockB(lb, st.y);
     }
@@ -320,6 +377,12 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const int fragHalf = (lane >> 5) * 16;
   const int aFragOff = (wm * kWaveRows + fragRow) * kPitch + fragHalf;
   const int bFragOff = (wn * 32 + fragRow) * kPitch + fragHalf;
+  // TRB: lane = 16 g + s. Group g reads the columns 16 (g & 1) .. of the fragment's 32 for the k-half g >> 1; inside
+  // the group, 8-bit: lane s hands in k-row s >> 1, column octet s & 1; 16-bit: k-row s >> 2, column quad s & 3.
+  const int trS = lane & 15, trG = lane >> 4;
+  const int bFragOffT = EB == 1
+      ? ((trG >> 1) * 16 + (trS >> 1)) * kPitchB + (wn * 128 + (trG & 1) * 16 + (trS & 1) * 8)
+      : ((trG >> 1) * 8 + (trS >> 2)) * kPitchB + (wn * 128 + (trG & 1) * 16 + (trS & 3) * 4) * 2;
 
   // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
   // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
@@ -331,8 +394,31 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     const u8 *lb = lds[buf][1] + bFragOff + ks * 32;
 #pragma unroll
     for (int i = 0; i < kTM; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 32 * kPitch);
+    if constexpr (TRB) {
+      // Sixteen lanes share a transposing read: each hands in 8 bytes of one k-row and gets back, for one column,
+      // the elements of 8 (8-bit) or 4 (16-bit) consecutive k-rows. Two reads make the 16 bytes of K of a fragment.
+      typedef int v2i __attribute__((ext_vector_type(2)));
+      typedef short v4s __attribute__((ext_vector_type(4)));
+      const u8 *lt = lds[buf][1] + bFragOffT + ks * (32 / EB) * kPitchB;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 64 * kPitch);
+      for (int j = 0; j < 4; ++j) {
+        const u8 *p0 = lt + j * 32 * EB;
+        const u8 *p1 = p0 + (8 / EB) * kPitchB;
+        if constexpr (EB == 1) {
+          const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(p0));
+          const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(p1));
+          bf[j] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(p0));
+          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(p1));
+          const v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
+          bf[j] = v4i{l2[0], l2[1], h2[0], h2[1]};
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 64 * kPitch);
+    }
   };
   auto mfmaAll = [&](const v4i (&af)[kTM], const v4i (&bf)[4]) {
     if (!kAllRowsReal && !waveHasRows) return;
@@ -381,21 +467,133 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
     mfmaAll(f1a, f1b);
   };
+  // ---- the same step with the staging spread over the substeps (operands whose staging is a plain copy of 16-byte
+  // chunks: B transposed in memory, or read with the transposing LDS reads): substep ks writes chunk ks of both operands
+  // to LDS and refills its registers from the tile after next, so that every group of 8 MFMAs has about the same
+  // number of LDS and memory instructions to cover; the order inside a substep is then fixed instruction by
+  // instruction (one MFMA, then a few of the others) instead of left to the scheduler, which clusters them.
+  constexpr bool kSpread = (TRB || TRANSB) && kSub == 4 && kRowChunks == 4;
+  auto storeChunk = [&](int buf, int i) {
+    u8 *la = lds[buf][0];
+    u8 *lb = lds[buf][1];
+    *reinterpret_cast<v4i *>(la + (aRow + kRowStep * i) * kPitch + aChunk * 16) = stage.x[i];
+    if constexpr (TRANSB) {
+      const int col = aRow + kRowStep * i;
+      const int r = (col & 3) * 64 + (col >> 2);
+      *reinterpret_cast<v4i *>(lb + r * kPitch + aChunk * 16) = stage.y[i];
+    } else {
+      *reinterpret_cast<v4i *>(lb + (bRowT + kRowStepB * i) * kPitchB + bChunkT * 16) = stage.y[i];
+    }
+  };
+  auto loadChunk = [&](long step, int i) {
+    const long k0 = (stepBase + step) * BK;
+    if (kFull || (m0 + aRow + kRowStep * i < M && k0 + aChunk * 16 < K)) {
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(aRsrc, aVoff, static_cast<int>((kRowStep * i) * K + k0), 0);
+      stage.x[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
+    } else {
+      stage.x[i] = v4i{0, 0, 0, 0};
+    }
+    if constexpr (TRANSB) {
+      if (kFull || (n0 + aRow + kRowStep * i < N && k0 + aChunk * 16 < K)) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoff, static_cast<int>((kRowStep * i) * K + k0), 0);
+        stage.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
+      } else {
+        stage.y[i] = v4i{0, 0, 0, 0};
+      }
+    } else {
+      const long krow = k0 / EB + bRowT + kRowStepB * i;
+      if (kFull || (krow < KE && n0 * EB + bChunkT * 16 < NB)) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoffT, static_cast<int>((k0 / EB + kRowStepB * i) * NB), 0);
+        stage.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
+      } else {
+        stage.y[i] = v4i{0, 0, 0, 0};
+      }
+    }
+  };
+  auto stepSpread = [&](long step, auto storeTag, auto loadTag) {
+    constexpr bool kStore = decltype(storeTag)::value;
+    constexpr bool kLoad = decltype(loadTag)::value;
+    constexpr int kFragReads = kTM + (TRB ? 8 : 4);
+    const int buf = static_cast<int>(step & 1);
+    // substep 0: fragments of substep 1; chunks 0 and 1 of tile s+1 to LDS
+    readFrags(buf, 1, f1a, f1b);
+    if constexpr (kStore) {
+      storeChunk(buf ^ 1, 0);
+      storeChunk(buf ^ 1, 1);
+    }
+    mfmaAll(f0a, f0b);
+    SubstepOrder<kFragReads, kStore ? 4 : 0, 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    // substep 1: fragments of substep 2; chunk 2 to LDS; chunks 0 and 1 of tile s+2 on their way
+    readFrags(buf, 2, f0a, f0b);
+    if constexpr (kStore) storeChunk(buf ^ 1, 2);
+    if constexpr (kLoad) {
+      loadChunk(step + 2, 0);
+      loadChunk(step + 2, 1);
+    }
+    mfmaAll(f1a, f1b);
+    SubstepOrder<kFragReads, kStore ? 2 : 0, kLoad ? 4 : 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    // substep 2: fragments of substep 3; chunk 3 to LDS; chunk 2 on its way
+    readFrags(buf, 3, f1a, f1b);
+    if constexpr (kStore) storeChunk(buf ^ 1, 3);
+    if constexpr (kLoad) loadChunk(step + 2, 2);
+    mfmaAll(f0a, f0b);
+    SubstepOrder<kFragReads, kStore ? 2 : 0, kLoad ? 2 : 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();   // everybody has read tile s completely and has written tile s+1
+    // substep 3: first fragments of tile s+1; chunk 3 on its way
+    if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
+    if constexpr (kLoad) loadChunk(step + 2, 3);
+    mfmaAll(f1a, f1b);
+    SubstepOrder<kStore ? kFragReads : 0, 0, kLoad ? 2 : 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+  };
   loadGlobal(0, stage);
   storeLds(0, stage);
   if (mySteps > 1) loadGlobal(1, stage);
   __syncthreads();
   readFrags(0, 0, f0a, f0b);
   long step = 0;
-  for (; step + 2 < mySteps; ++step) stepBody(step, BoolTag<true>(), BoolTag<true>());
-  if (step + 1 < mySteps) {
-    stepBody(step, BoolTag<true>(), BoolTag<false>());
-    ++step;
+  if constexpr (kSpread) {
+    for (; step + 2 < mySteps; ++step) stepSpread(step, BoolTag<true>(), BoolTag<true>());
+    if (step + 1 < mySteps) {
+      stepSpread(step, BoolTag<true>(), BoolTag<false>());
+      ++step;
+    }
+    stepSpread(step, BoolTag<false>(), BoolTag<false>());
+  } else {
+    for (; step + 2 < mySteps; ++step) stepBody(step, BoolTag<true>(), BoolTag<true>());
+    if (step + 1 < mySteps) {
+      stepBody(step, BoolTag<true>(), BoolTag<false>());
+      ++step;
+    }
+    stepBody(step, BoolTag<false>(), BoolTag<false>());
   }
-  stepBody(step, BoolTag<false>(), BoolTag<false>());
 
   // ---- epilogue: lane owns columns col4 .. col4+3 of 16 * kTM rows
-  const long col4 = n0 + 4 * (wn * 32 + fragRow);
+  // With the transposing reads column tile j holds the columns 32 j .. 32 j + 31 of the wavefront's 128, lane by lane,
+  // so the four lanes of a quad hold four neighbouring columns of each of the four tiles: a 4 x 4 transpose between
+  // the lanes of the quad and the tiles (two exchanges with quad permutations) gives lane c the four columns of tile c.
+  if constexpr (TRB) {
+    const bool odd = (lane & 1) != 0, upper = (lane & 2) != 0;
+#pragma unroll
+    for (int i = 0; i < kTM; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        typename Mma::acc_t a0 = acc[i][0][v], a1 = acc[i][1][v], a2 = acc[i][2][v], a3 = acc[i][3][v];
+        const typename Mma::acc_t r01 = lane_partner<1>(odd ? a0 : a1), r23 = lane_partner<1>(odd ? a2 : a3);
+        if (odd) { a0 = r01; a2 = r23; } else { a1 = r01; a3 = r23; }
+        const typename Mma::acc_t r02 = lane_partner<2>(upper ? a0 : a2), r13 = lane_partner<2>(upper ? a1 : a3);
+        if (upper) { a0 = r02; a1 = r13; } else { a2 = r02; a3 = r13; }
+        acc[i][0][v] = a0;
+        acc[i][1][v] = a1;
+        acc[i][2][v] = a2;
+        acc[i][3][v] = a3;
+      }
+    }
+  }
+  const long col4 = TRB ? n0 + wn * 128 + 32 * (lane & 3) + (fragRow & ~3) : n0 + 4 * (wn * 32 + fragRow);
   if constexpr (KSPLIT > 1) {
     constexpr long kPartRows = M < kGemmBM ? M : kGemmBM;            // rows of a tile that can hold results
     constexpr long kCounterBytes = (kGridTiles * 4 + 255) / 256 * 256;
