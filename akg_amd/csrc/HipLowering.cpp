@@ -315,6 +315,20 @@ std::vector<bool> relaxedPrecisionTensors(const OpGraph &g) {
       case OpKind::MatMul:
         inDemand = 2;
         break;
+      case OpKind::Mul:
+      case OpKind::Div: {
+        // A constant factor of 1024 and more (a divisor of 1/1024 and less) would carry the absolute error of an
+        // approximation (1.2e-7 for the hardware tanh form) into the 16-bit tolerance: exact operands from here on.
+        if (!isFloatType(od)) inDemand = 2;
+        for (size_t i = 0; i < op.inputs.size(); ++i) {
+          const TensorValue &t = g.tensor(op.inputs[i]);
+          if (!t.isConst) continue;
+          const double c = std::fabs(t.constValue);
+          const bool divisor = op.kind == OpKind::Div && i == 1;
+          if (divisor ? (c <= 1.0 / 1024.0) : (c >= 1024.0)) inDemand = 2;
+        }
+        break;
+      }
       default:
         if (!isFloatType(od)) inDemand = 2;
         break;

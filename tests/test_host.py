@@ -547,6 +547,13 @@ def test_math_selection_follows_the_precision_demand():
     # float32 elementwise chain: device-library tanh
     src = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_ew_tanh_add_mul_f32_8x128.info")).source
     assert "akg::op_tanh(" in src and "fast_" not in src
+    # a constant factor of 1024 and more between an approximation and the 16-bit cast would carry its absolute error
+    # (1.2e-7 for the hardware tanh form) towards the tolerance: the operands behind such a factor are exact
+    for factor, fast in ((4.0, True), (4096.0, False)):
+        b = op_desc.DescBuilder("scaled_tanh_f16_%d" % int(factor))
+        x = b.input([64, 128], "float32")
+        src = driver.HipKernel(b.dumps([b.cast(b.mul(b.unary("Tanh", x), b.const(factor, "float32")), "float16")]), out_dir=None).source
+        assert ("akg::fast_tanh(" in src) == fast and ("akg::op_tanh(" in src) != fast
     # AKG_HIP_PRECISE=1 switches every relaxation off
     os.environ["AKG_HIP_PRECISE"] = "1"
     try:
