@@ -802,6 +802,24 @@ def test_segment_sum_is_bit_exact(name):
     check_segment_sum(os.path.join(FIXTURES, name), seed=harness.BASE_SEED + 301)
 
 
+@pytest.mark.parametrize("dtype,slice_,segments,positions,ids", [
+    ("float16", 2, 2000, 200000, "int32"),      # 4-byte rows, 16 segments a bucket, 16-bit additions rounded per step
+    ("int32", 3, 1600, 150000, "int64"),        # 12-byte integer rows, 64-bit ids
+    ("bfloat16", 6, 800, 131077, "int32"),      # 12-byte rows of six elements, 4 segments a bucket, a ragged last chunk
+    ("float32", 1, 4000, 100000, "int32"),      # one column
+])
+def test_bucketed_segment_sum_in_other_types(dtype, slice_, segments, positions, ids, tmp_path):
+    """The schedule by bucket of segments for rows of 4, 8 and 12 bytes in 16-bit, integer and float32 data: bit-exact
+    against the serial loop (16-bit sums included: every addition is rounded, in position order)."""
+    name = "bucketed_%s_x%d_seg%d_%d" % (dtype, slice_, segments, positions)
+    text = op_desc.unsorted_segment_sum([positions], [slice_], segments, dtype, ids, name)
+    path = os.path.join(str(tmp_path), name + ".info")
+    open(path, "w").write(text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert "grouped by bucket" in kernel.source, kernel.source[:200]
+    check_segment_sum(path, seed=harness.BASE_SEED + 770)
+
+
 @pytest.mark.parametrize("schedule", ["scan", "grouped", "bucketed"])
 def test_segment_sum_drops_ids_outside_the_range_and_leaves_unnamed_rows_zero(schedule, monkeypatch, tmp_path):
     """The three schedules (every workgroup scanning all ids; positions grouped by segment first; grouped by bucket of
