@@ -350,8 +350,6 @@ class ColumnEmitter {
     src_ << ") {\n";
     src_ << "  constexpr int V = " << vec_ << ", LX = " << lx_ << ", LY = " << ly_ << ", CH = " << chunks_ << ", BLOCK = " << block_ << ";\n";
     src_ << "  constexpr long RUN = " << run_ << ", INNER = " << inner_ << ", STRIPS = " << strips_ << ";\n";
-    int reductions = 0;
-    for (const OpNode &op : g_.ops) reductions += lowering::isReduceKind(op.kind) ? 1 : 0;
     if (block_ > 64) line("  __shared__ __attribute__((aligned(16))) unsigned char akg_scratch[2][(BLOCK / 64) * LX * V * 8];");
     line("  const int tid = static_cast<int>(threadIdx.x), lx = tid % LX, ly = tid / LX;");
     line("  const long akg_o = static_cast<long>(blockIdx.x) / STRIPS;");
@@ -526,7 +524,6 @@ class ColumnEmitter {
       src_ << "  if (ly == 0) akg::store_chunk_partial<" << tag << ", V>(out" << i << " + " << offsetExpr(f, "0", "akg_col") << ", akg_cols, " << src << ");\n";
     }
     line("}");
-    (void)reductions;
   }
 };
 
