@@ -171,6 +171,19 @@ class ColumnEmitter {
         if (!(flags_[static_cast<size_t>(out)] == flags_[static_cast<size_t>(op.inputs[0])])) {
           throw LoweringError("op Reshape: more than adding or dropping unit dimensions");
         }
+      } else if (axis_ > 0) {
+        // A reduction result without keep_dims has lost the reduced axis: against a tensor of the full rank, broadcasting
+        // would align it on the right, not where it came from. Only a Reshape may put the axis back.
+        bool droppedAxis = false, fullRank = false;
+        for (int in : op.inputs) {
+          const TensorValue &t = g_.tensor(in);
+          if (t.isConst || t.numel() == 1) continue;
+          droppedAxis = droppedAxis || (t.shape.size() + 1 == full_.size() && flags_[static_cast<size_t>(in)].rank() == Rank::Col);
+          fullRank = fullRank || t.shape.size() == full_.size();
+        }
+        if (droppedAxis && fullRank) {
+          throw LoweringError("op " + op.name + ": a reduce result without keep_dims cannot be broadcast against the reduced tensor; reshape it first");
+        }
       }
       level_[static_cast<size_t>(out)] = lv;
       maxLevel_ = std::max(maxLevel_, lv);

@@ -182,6 +182,12 @@ def _column_cases():
         x = b.input([2, 40, 24], "float16")
         return [b.sub(x, b.reduce("ReduceMax", x, [1], True)), b.reduce("ReduceSum", x, [1], True)]
 
+    def no_keep_meets_the_tensor_unreshaped(b):
+        # the [5,5] result of a reduction over the middle axis used directly against [5,5,5]: broadcasting aligns it on
+        # the right (as rows and columns of every outer index), which is not the column kernel's business
+        x = b.input([5, 5, 5], "float32")
+        return [b.sub(x, b.reduce("ReduceMax", x, [1], False))]
+
     def run_too_long_for_registers(b):
         x = b.input([2, 20000, 64], "float32")
         return [b.sub(x, b.reduce("ReduceMax", x, [1], True))]
@@ -189,6 +195,7 @@ def _column_cases():
     return {"l2_normalise_no_keep": (l2_normalise_no_keep, "column_reduce"), "centred_with_statistics": (centred_with_statistics, "column_reduce"),
             "scaled_by_a_shared_plane": (scaled_by_a_shared_plane, "column_reduce"), "integer_range": (integer_range, "column_reduce"),
             "narrow_columns": (narrow_columns, "column_reduce"), "half_sums": (half_sums, "column_reduce"),
+            "no_keep_meets_the_tensor_unreshaped": (no_keep_meets_the_tensor_unreshaped, "staged"),
             "run_too_long_for_registers": (run_too_long_for_registers, "staged")}
 
 
