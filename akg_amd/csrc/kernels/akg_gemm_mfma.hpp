@@ -132,7 +132,8 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // (every row of A contributes one whole cache line, half as many barriers as with 64; LDS holds 2 x 72 KiB).
   // Staging (global -> registers -> LDS) is done by every thread for both operands: uniform control flow, so the whole
   // K step is one basic block and loads, transposes and LDS writes interleave with the MFMAs. (Measured and dropped:
-  // 2 x 2 wavefronts of 128 x 128 each, 64-byte steps, staging split between two groups of wavefronts, 256 x 128 tiles
+  // 2 x 2 wavefronts of 128 x 128 each (a third less LDS traffic, one wavefront per SIMD: 2 to 4 % slower, also with the
+  // fixed instruction order below), 64-byte steps, staging split between two groups of wavefronts, 256 x 128 tiles
   // with two workgroups per CU; tiles fetched memory -> LDS directly (buffer_load_dwordx4 ... lds into rows without
   // padding, chunks permuted against bank conflicts): correct, 2 % slower than the staging through registers; the K
   // steps of different tiles in rotated order: 8 to 25 % slower, the workgroups of an XCD share their panels in L2
