@@ -43,8 +43,7 @@ struct LoweringOptions {
   int block = 0;        // threads per workgroup
   int split = 0;        // streaming reductions: workgroups sharing one group of outputs (AKG_HIP_SPLIT)
   // Experiment switch (AKG_HIP_VARIANT), read by whichever family lowers the kernel; 0 = the measured default.
-  //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows,
-  //                  bit 5: a row-major B is transposed in registers on its way to LDS (no transposing LDS reads)
+  //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows
   //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
   //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs, 7: no column kernel (several kernels instead)
   //   segment_sum    1: every workgroup scans all ids, 2: positions grouped by segment first (whatever the size),

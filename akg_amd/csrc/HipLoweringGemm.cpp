@@ -470,7 +470,7 @@ class GemmEmitter {
       return;
     }
     src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-         << ", Epilogue, " << kSplit_ << (!(opt_.variant & 32) && !transB_ ? ", true" : "") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
+         << ", Epilogue, " << kSplit_ << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in" << g_.tensor(bId_).inputIndex
          << " + akg_batch * " << k_ * n_ << "L, epi" << (kSplit_ > 1 ? ", akg_ws" : "") << ");\n}\n";
   }
 };

@@ -1,33 +1,31 @@
 /**
  * MFMA GEMM tile kernel for gfx950 (CDNA4) with a caller-supplied epilogue applied to the accumulators while they
  * are still in registers (dequantise / bias / activation / cast fusions). The element type is a template
- * parameter (`Mma`): int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), bfloat16 or float16 -> float32
- * (v_mfma_f32_32x32x16_bf16 / _f16). Both instruction shapes consume 32 BYTES of K per row and MFMA (a lane holds 16
- * consecutive bytes), so the kernel is written in bytes along K and the LDS layout, the fragment reads and the A
- * staging are the same for every element type; only the in-register transpose of a row-major B differs.
+ * parameter (`Mma`): int8 x int8 -> int32 (v_mfma_i32_16x16x64_i8), bfloat16 or float16 -> float32
+ * (v_mfma_f32_16x16x32_bf16 / _f16). Both instruction shapes consume 64 BYTES of K per row and MFMA (a lane holds 16
+ * consecutive bytes), so the kernel is written in bytes along K and the LDS layout, the fragment reads and the
+ * staging are the same for every element type.
+ * Why 16 x 16 tiles and not 32 x 32 (half the MFMAs for the same work): the part is power limited, and a loop of
+ * nothing but MFMAs on random operands sustains 0.85 of the nominal peak in the 16 x 16 shapes against 0.72 (int8) and
+ * 0.75 (bfloat16) in the 32 x 32 ones; the same kernel on 32 x 32 MFMAs was 5 % (int8) and 3 % (bfloat16) slower.
  *
  * Shape of the computation (all sizes are compile-time constants of the emitted kernel):
  *   C[M,N] = A[M,K] * B[K,N]            A row-major, B row-major ([N,K] when TRANSB)
  *   workgroup tile 256 x 256, K step 128 bytes, 4 x 2 wavefronts
- *   wavefront tile 64 x 128 = 2 x 4 MFMA tiles of 32 x 32 (16 accumulator registers each)
+ *   wavefront tile 64 x 128 = 4 x 8 MFMA tiles of 16 x 16 (4 accumulator registers each)
  *
  * Data movement:
  *   global -> registers -> LDS, double buffered in LDS (one barrier per K step); the global loads of step
- *   i+1 are issued before the MFMAs of step i.
- *   A: each thread moves 4 x 16 bytes (16 consecutive k of one row) straight into LDS.
- *   B (not transposed) is row-major along N but the MFMA wants, per lane, 16 consecutive k of one column. By default
- *   (TRB) its tile goes to LDS as it lies in memory, 16-byte chunks of a k-row, and the fragments are read with the
+ *   i+2 are issued during step i. Both operands travel as 16-byte chunks, a plain copy.
+ *   A (and a B given as [N,K]): rows of 128 data bytes + 16 pad bytes; with a row pitch of 144 bytes consecutive rows
+ *   start in different 16-byte bank groups. Fragments are read with ds_read_b128.
+ *   B row-major: its tile goes to LDS as it lies in memory, k-rows of 256 columns, and the fragments are read with the
  *   transposing LDS reads of gfx950 (ds_read_b64_tr_b8 / _b16: sixteen lanes hand in 8 bytes of a k-row each and get
- *   back, per column, 8 or 4 consecutive k); the staging of both operands is then a plain copy, spread over the
- *   substeps, and the order of MFMAs, LDS accesses and loads inside a substep is fixed with scheduling groups
- *   (int8 4096 x 8192 x 8192: 0.428 -> 0.463 of the MFMA peak, bfloat16: 0.465 -> 0.516; MFMA units busy 58 -> 68 %).
- *   Without TRB each thread loads a 16(k) x 4(n) byte block as 16 dwords, transposes it in registers with
- *   v_perm_b32 (8 permutes per 4 x 4 sub-block) and writes four 16-byte k-vectors to LDS.
- *   LDS rows are 128 data bytes + 16 pad bytes: with a row pitch of 144 bytes consecutive rows start in
- *   different 16-byte bank groups, and the ds_read_b128 fragment loads are conflict free (SQ_LDS_BANK_CONFLICT reads 0).
- *   LDS row r of the B tile holds global column 4 * (r % 64) + r / 64 of the tile. A wavefront's four column
- *   tiles are r / 64 = 0..3 with the same r % 64 range, so each lane ends up owning 4 ADJACENT output columns:
- *   the epilogue works on 4-element chunks and a wavefront stores 256 contiguous bytes per output row.
+ *   back, per column, 8 or 4 consecutive k): no transposes in registers.
+ *   SQ_LDS_BANK_CONFLICT reads 0 for both layouts (how the chunks are placed for that is said where they are written).
+ *   Every lane ends up owning 4 ADJACENT output columns (by the order of the LDS rows of an [N,K] B; by a 4 x 4
+ *   exchange inside each lane quad for a row-major B): the epilogue works on 4-element chunks and sixteen lanes store
+ *   one aligned piece of 64 columns per output row.
  *
  * Workgroup -> tile mapping: consecutive workgroup ids go round-robin to the 8 XCDs (each with its own L2), so
  * ids are first regrouped per XCD and then walked in column-major groups of 8 tile-rows, which keeps the A and B
@@ -40,14 +38,18 @@ namespace akg {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 
 // Element-type traits of the contraction: bytes per element, accumulator type, and the MFMA on one 16-byte
-// fragment per operand (32 x 32 outputs, 32 bytes of K).
+// fragment per operand: `mma16` 16 x 16 outputs and 64 bytes of K (the tile kernel), `mma` 32 x 32 outputs and 32 bytes
+// of K (the skinny kernel, whose time is that of streaming B).
 struct MmaI8 {
   static constexpr int kElemBytes = 1;
   typedef int acc_t;
   typedef v16i acc_v;
+  typedef v4i acc4_v;
   static AKG_DEV acc_v mma(v4i a, v4i b, acc_v c) { return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0); }
+  static AKG_DEV acc4_v mma16(v4i a, v4i b, acc4_v c) { return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0); }
 };
 struct MmaBF16 {
   static constexpr int kElemBytes = 2;
@@ -57,6 +59,10 @@ struct MmaBF16 {
   static AKG_DEV acc_v mma(v4i a, v4i b, acc_v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(frag, a), __builtin_bit_cast(frag, b), c, 0, 0, 0);
   }
+  typedef v4f acc4_v;
+  static AKG_DEV acc4_v mma16(v4i a, v4i b, acc4_v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(frag, a), __builtin_bit_cast(frag, b), c, 0, 0, 0);
+  }
 };
 struct MmaF16 {
   static constexpr int kElemBytes = 2;
@@ -65,6 +71,10 @@ struct MmaF16 {
   typedef _Float16 frag __attribute__((ext_vector_type(8)));
   static AKG_DEV acc_v mma(v4i a, v4i b, acc_v c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(frag, a), __builtin_bit_cast(frag, b), c, 0, 0, 0);
+  }
+  typedef v4f acc4_v;
+  static AKG_DEV acc4_v mma16(v4i a, v4i b, acc4_v c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(frag, a), __builtin_bit_cast(frag, b), c, 0, 0, 0);
   }
 };
 
@@ -120,7 +130,26 @@ struct SubstepOrder {
   }
 };
 
-template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1, bool TRB = false>
+// The same for the substeps of the 16 x 16 kernel, whose MFMAs are half as long: the others go in front, two after each
+// of the first MFMAs, reads first (their results are wanted by the very next substep), then writes, then loads.
+template <int R, int W, int L, int M = 0>
+struct SubstepFront {
+  static constexpr int kAll = R + W + L;
+  static constexpr int kFrom = 2 * M < kAll ? 2 * M : kAll, kUpto = 2 * M + 2 < kAll ? 2 * M + 2 : kAll;
+  static constexpr int within(int lo, int hi) {
+    const int a = kFrom > lo ? kFrom : lo, b = kUpto < hi ? kUpto : hi;
+    return b > a ? b - a : 0;
+  }
+  static AKG_DEV void emit() {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (within(0, R) > 0) __builtin_amdgcn_sched_group_barrier(0x100, within(0, R), 0);
+    if constexpr (within(R, R + W) > 0) __builtin_amdgcn_sched_group_barrier(0x200, within(R, R + W), 0);
+    if constexpr (within(R + W, kAll) > 0) __builtin_amdgcn_sched_group_barrier(0x020, within(R + W, kAll), 0);
+    if constexpr (M < 7) SubstepFront<R, W, L, M + 1>::emit();
+  }
+};
+
+template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1>
 AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi,
                           unsigned *__restrict__ ws = nullptr) {
   constexpr int EB = Mma::kElemBytes;
@@ -128,29 +157,26 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   constexpr long NB = N * EB;    // bytes per k-row of a row-major B
   static_assert(K % 16 == 0, "K must be a multiple of 16 bytes");
   static_assert(TRANSB || (N % 4 == 0), "N must be a multiple of 4");
-  // 4 x 2 wavefronts (two per SIMD: one's MFMAs cover the other's loads, transposes and waits), 128 bytes of K per step
-  // (every row of A contributes one whole cache line, half as many barriers as with 64; LDS holds 2 x 72 KiB).
-  // Staging (global -> registers -> LDS) is done by every thread for both operands: uniform control flow, so the whole
-  // K step is one basic block and loads, transposes and LDS writes interleave with the MFMAs. (Measured and dropped:
-  // 2 x 2 wavefronts of 128 x 128 each (a third less LDS traffic, one wavefront per SIMD: 2 to 4 % slower, also with the
-  // fixed instruction order below), 64-byte steps, staging split between two groups of wavefronts, 256 x 128 tiles
-  // with two workgroups per CU; tiles fetched memory -> LDS directly (buffer_load_dwordx4 ... lds into rows without
-  // padding, chunks permuted against bank conflicts): correct, 2 % slower than the staging through registers; the K
-  // steps of different tiles in rotated order: 8 to 25 % slower, the workgroups of an XCD share their panels in L2
-  // only while they walk K together. With the staging switched off altogether the loop runs 17 % faster, whichever
-  // way the tiles travel: what is left is the price of moving 64 KB per step and CU on a power-limited part.)
+  // 4 x 2 wavefronts (two per SIMD: one's MFMAs cover the other's LDS accesses and waits), 128 bytes of K per step
+  // (every row of A contributes one whole cache line; LDS holds 2 x 72 KiB). Every thread stages its share of both
+  // operands: uniform control flow, so a K step is one basic block.
+  // (Measured and dropped: 2 x 2 wavefronts of 128 x 128 each (a third less LDS traffic, one wavefront per SIMD: 2 to 4 %
+  // slower), 64-byte steps, staging split between two groups of wavefronts, 256 x 128 tiles with two workgroups per
+  // CU; tiles fetched memory -> LDS directly (buffer_load_dwordx4 ... lds into rows without padding, chunks permuted
+  // against bank conflicts): correct, 2 % slower than the staging through registers; the K steps of different tiles in
+  // rotated order: 8 to 25 % slower, the workgroups of an XCD share their panels in L2 only while they walk K
+  // together. With the staging switched off altogether the loop runs 17 % faster, whichever way the tiles travel: what
+  // is left is the price of moving 64 KB per step and CU on a power-limited part.)
   constexpr int WAVES_M = 4;
   constexpr int BK = 128;
   constexpr int kThreads = WAVES_M * 128;
-  constexpr int kStageThreads = kThreads;             // threads that share one operand tile
-  constexpr int kPitch = BK + 16;                     // LDS row: BK data bytes + 16 pad (odd multiple of 16)
-  constexpr int kSub = BK / 32;                       // MFMA k-substeps per step (2 or 4)
+  constexpr int kPitch = BK + 16;                     // LDS row of a K-contiguous tile: BK data bytes + 16 pad
   constexpr int kChunksPerRow = BK / 16;              // 16-byte chunks per row of a K-contiguous operand tile
-  constexpr int kRowChunks = 256 * kChunksPerRow / kStageThreads;  // 16-byte chunks per staging thread and operand
-  constexpr int kRowStep = kStageThreads / kChunksPerRow;          // rows between two chunks of one thread
-  constexpr int kBlockRows = 4 * kRowChunks / EB;     // k-rows of B per staging thread, 4 columns each (16 k-bytes per chunk)
-  constexpr int kTM = kGemmBM / (32 * WAVES_M);       // MFMA row tiles per wavefront
-  constexpr int kWaveRows = kGemmBM / WAVES_M;
+  constexpr int kRowChunks = 256 * kChunksPerRow / kThreads;  // 16-byte chunks per thread and operand (4)
+  constexpr int kRowStep = kThreads / kChunksPerRow;  // rows between two chunks of one thread
+  constexpr int kTM = 4;                              // MFMA row tiles (16 rows) per wavefront
+  constexpr int kTN = 8;                              // MFMA column tiles (16 columns) per wavefront
+  constexpr int kWaveRows = kGemmBM / WAVES_M;        // 64
   constexpr long kTilesM = (M + kGemmBM - 1) / kGemmBM;
   constexpr long kTilesN = (N + kGemmBN - 1) / kGemmBN;
   constexpr long kTiles = kTilesM * kTilesN;
@@ -158,18 +184,21 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   constexpr long kSteps = (K + BK - 1) / BK;
   constexpr bool kFull = (M % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
   constexpr int kTileBytes = kGemmBM * kPitch;        // one operand tile in LDS
-  // TRB: a row-major B goes to LDS as it lies in memory, k-rows of 256 columns, and the fragments are read with the
-  // transposing LDS reads (ds_read_b64_tr_b8 / _b16): no transposes in registers.
-  static_assert(!(TRB && TRANSB), "the transposing reads are for a row-major B");
+  static_assert(kRowChunks == 4, "the staging schedule is written for four 16-byte chunks per thread and operand");
+  // A row-major B goes to LDS as it lies in memory, k-rows of 256 columns. Sixteen lanes share a transposing read:
+  // each hands in 8 bytes of one k-row (8-bit: 8 k-rows x 16 bytes, 16-bit: 4 k-rows x 32 bytes) and gets back, for one
+  // column, 8 or 4 consecutive k. The four 16-lane groups of a wavefront read the same 16 columns, each its own
+  // sixteen (8-bit) or eight (16-bit) k-rows; the rows of neighbouring groups are a multiple of 256 bytes apart whatever
+  // the pitch, so odd groups find their columns in the neighbouring 16-column unit of the row (units swapped in pairs
+  // when the row is written), and with rows 32 (64) bytes apart modulo the 256 bytes of the banks the two groups of a
+  // half wavefront interleave without sharing a bank.
   constexpr int kRowBytesB = kGemmBN * EB;            // bytes of one k-row of the B tile
-  // Row pitch: the 16 lanes of a transposing read hand in 8 rows x 16 bytes (8-bit) or 4 rows x 32 bytes (16-bit), and the
-  // neighbouring 16 lanes the 16 or 32 bytes beside them; with rows 32 (64) bytes apart modulo the 256 bytes of the
-  // banks, the two groups of a half wavefront interleave without sharing a bank.
   constexpr int kPitchB = kRowBytesB + (EB == 1 ? 32 : 64);
   constexpr int kRowsB = BK / EB;                     // k-rows per step
   constexpr int kChunksPerRowB = kRowBytesB / 16;
-  constexpr int kRowStepB = kStageThreads / kChunksPerRowB;
-  static_assert(!TRB || kRowsB * kPitchB <= kTileBytes, "the row-major B tile must fit the operand's LDS space");
+  constexpr int kRowStepB = kThreads / kChunksPerRowB;
+  constexpr int kGroupRowsB = 16 / EB;                // k-rows one 16-lane group owns per MFMA
+  static_assert(TRANSB || kRowsB * kPitchB <= kTileBytes, "the row-major B tile must fit the operand's LDS space");
 
   __shared__ __attribute__((aligned(16))) u8 lds[2][2][kTileBytes];  // [buffer][A|B]
 
@@ -200,31 +229,25 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const int wm = wave >> 1;
   const int wn = wave & 1;
 
-  typename Mma::acc_v acc[kTM][4];
+  typename Mma::acc4_v acc[kTM][kTN];
 #pragma unroll
   for (int i = 0; i < kTM; ++i) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < kTN; ++j) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0;
+      for (int v = 0; v < 4; ++v) acc[i][j][v] = 0;
     }
   }
 
-  // ---- staging registers: the tile of step s+1 travels memory -> registers during step s-1.. s and is written to
-  // LDS at the top of step s.
-  // Every thread stages its share of A (x) and of B (y).
+  // ---- staging registers: chunk i of tile s+1 waits here from its load (during step s-1) to its LDS write (step s).
   struct Stage {
-    v4i x[kRowChunks];
-    v4i y[kRowChunks];
+    v4i x[kRowChunks];   // A
+    v4i y[kRowChunks];   // B
   };
   Stage stage;
 
-  const int ltid = tid;
-  const int aRow = ltid / kChunksPerRow;   // + kRowStep * i
-  const int aChunk = ltid % kChunksPerRow;
-  const int bN4 = ltid & 63;
-  const int bKq = ltid >> 6;
-
+  const int aRow = tid / kChunksPerRow;   // + kRowStep * i
+  const int aChunk = tid % kChunksPerRow;
   // Global loads are buffer loads: the per-lane offset is computed once, everything that changes from load to load
   // (row block, k-row, K step) is a scalar offset, so the loop spends no vector instructions on addresses (vector
   // instructions and MFMAs compete for issue cycles). Out-of-range lanes read zero through the descriptor's size.
@@ -233,263 +256,34 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
       const_cast<void *>(A), 0, static_cast<int>(M * K), 0x00020000);
   const __amdgpu_buffer_rsrc_t bRsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<void *>(B), 0, static_cast<int>(N * K), 0x00020000);
-  const int aVoff = static_cast<int>((m0 + aRow) * K + aChunk * 16);
-  const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
-                           : static_cast<int>((bKq * kBlockRows) * NB + (n0 + 4 * bN4) * EB);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-  const int bRowT = ltid / kChunksPerRowB;     // + kRowStepB * i
-  const int bChunkT = ltid % kChunksPerRowB;
-  const int bVoffT = static_cast<int>(bRowT * NB + n0 * EB + bChunkT * 16);
-
-  auto loadRows = [&](__amdgpu_buffer_rsrc_t rsrc, int voff, long rowBase, long rowLimit, long k0,
-                      v4i (&dst)[kRowChunks]) {
-    // kRowChunks chunks of 16 consecutive k, rows rowBase + kRowStep * i of a K-contiguous operand
+  const int aVoff = static_cast<int>((m0 + aRow) * K + aChunk * 16);
+  const int bRowT = tid / kChunksPerRowB;     // + kRowStepB * i
+  const int bChunkT = tid % kChunksPerRowB;
+  const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
+                           : static_cast<int>(bRowT * NB + n0 * EB + bChunkT * 16);
+  // LDS write offsets. [N,K] B: the LDS row of a column is chosen so that the 16 lanes of a fragment read find, in the
+  // four column tiles 4 q .. 4 q + 3, four ADJACENT columns (row 64 q + 16 t + c holds column 64 q + 4 c + t).
+  // Row-major B: the 16-column units of a k-row are swapped in pairs for the k-rows of odd 16-lane groups.
+  // K-contiguous tiles: a 128-bit LDS read is served sixteen lanes at a time, and not sixteen neighbours: the lane
+  // quads 0, 3, 5, 6 of a half wavefront go together, then 1, 2, 4, 7 (measured). The 16 rows x 2 quarters of K such a
+  // group reads fall into 16 different bank groups when rows 4 .. 11 of every 16 keep their 16-byte chunks swapped in pairs.
+  auto pairSwap = [](int row) { return ((row >> 2) ^ (row >> 3)) & 1; };
+  const int aStoreOff = aRow * kPitch + (aChunk ^ pairSwap(aRow)) * 16;
+  int bStoreOff[kRowChunks];
 #pragma unroll
-    for (int i = 0; i < kRowChunks; ++i) {
-      if (kFull || (rowBase + kRowStep * i < rowLimit && k0 + aChunk * 16 < K)) {
-        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff, static_cast<int>((kRowStep * i) * K + k0), 0);
-        dst[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
-      } else {
-        dst[i] = v4i{0, 0, 0, 0};
-      }
-    }
-  };
-  auto loadBlock = [&](long k0, v4i (&dst)[kRowChunks]) {
-    // kBlockRows k-rows x 4 columns of row-major B: one dword (8-bit elements) or two (16-bit) per k-row.
-    // k0 is in bytes of K: the first k-row of the step is k0 / EB.
-#pragma unroll
-    for (int i = 0; i < kBlockRows; ++i) {
-      const bool ok = kFull || (n0 + 4 * bN4 < N && k0 / EB + bKq * kBlockRows + i < KE);
-      if constexpr (EB == 1) {
-        u32 v = 0u;
-        if (ok) v = __builtin_amdgcn_raw_buffer_load_b32(bRsrc, bVoff, static_cast<int>((k0 + i) * NB), 0);
-        dst[i >> 2][i & 3] = static_cast<int>(v);
-      } else {
-        typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-        u32x2 v = {0u, 0u};
-        if (ok) v = __builtin_amdgcn_raw_buffer_load_b64(bRsrc, bVoff, static_cast<int>((k0 / EB + i) * NB), 0);
-        dst[i >> 1][(i & 1) * 2] = static_cast<int>(v[0]);
-        dst[i >> 1][(i & 1) * 2 + 1] = static_cast<int>(v[1]);
-      }
-    }
-  };
-  auto loadGlobal = [&](long step, Stage &st) {
-    const long k0 = (stepBase + step) * BK;
-    loadRows(aRsrc, aVoff, m0 + aRow, M, k0, st.x);
-    if constexpr (TRANSB) {
-      loadRows(bRsrc, bVoff, n0 + aRow, N, k0, st.y);
-    } else if constexpr (TRB) {
-      // kRowChunks chunks of 16 bytes along n: k-rows bRowT + kRowStepB * i of the step
-#pragma unroll
-      for (int i = 0; i < kRowChunks; ++i) {
-        const long krow = k0 / EB + bRowT + kRowStepB * i;
-        if (kFull || (krow < KE && n0 * EB + bChunkT * 16 < NB)) {
-          const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoffT, static_cast<int>((k0 / EB + kRowStepB * i) * NB), 0);
-          st.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
-        } else {
-          st.y[i] = v4i{0, 0, 0, 0};
-        }
-      }
-    } else {
-      loadBlock(k0, st.y);
-    }
-  };
-
-  auto storeRowsA = [&](u8 *la, const v4i (&src)[kRowChunks]) {
-#pragma unroll
-    for (int i = 0; i < kRowChunks; ++i) {
-      *reinterpret_cast<v4i *>(la + (aRow + kRowStep * i) * kPitch + aChunk * 16) = src[i];
-    }
-  };
-  auto storeRowsBt = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
-#pragma unroll
-    for (int i = 0; i < kRowChunks; ++i) {
-      const int col = aRow + kRowStep * i;           // column of the tile
-      const int r = (col & 3) * 64 + (col >> 2);     // its LDS row
-      *reinterpret_cast<v4i *>(lb + r * kPitch + aChunk * 16) = src[i];
-    }
-  };
-  auto storeBlockB16 = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
-    // 16-bit elements: src[g] = k-rows 2g, 2g+1, each as (columns 0 1 | columns 2 3). A column's 8 consecutive k
-    // (16 bytes) are gathered two at a time with v_perm_b32; a thread holds 8 k-rows.
-    static_assert(kRowChunks == 4, "the staging is written for four 16-byte chunks per thread and operand");
-    if constexpr (EB == 2) {
-#pragma unroll
-      for (int h = 0; h < kRowChunks / 4; ++h) {
-        v4i w[4];
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const u32 c01a = static_cast<u32>(src[4 * h + g][0]), c23a = static_cast<u32>(src[4 * h + g][1]);  // k-row 2g
-          const u32 c01b = static_cast<u32>(src[4 * h + g][2]), c23b = static_cast<u32>(src[4 * h + g][3]);  // k-row 2g + 1
-          w[0][g] = static_cast<int>(pack_lo16(c01a, c01b));
-          w[1][g] = static_cast<int>(pack_hi16(c01a, c01b));
-          w[2][g] = static_cast<int>(pack_lo16(c23a, c23b));
-          w[3][g] = static_cast<int>(pack_hi16(c23a, c23b));
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * (kRowChunks * 4) + h * 16) = w[j];
-        }
-      }
-    }
-  };
-  auto storeBlockB8 = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
-    // src[g] = 4 k-rows x 4 columns; after the byte transpose t[g][j] = 4 consecutive k of column j
-    u32 t[kRowChunks][4];
-#pragma unroll
-    for (int g = 0; g < kRowChunks; ++g) {
-      const u32 rows[4] = {static_cast<u32>(src[g][0]), static_cast<u32>(src[g][1]), static_cast<u32>(src[g][2]),
-                           static_cast<u32>(src[g][3])};
-      transpose4x4_bytes(rows, t[g]);
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int h = 0; h < kRowChunks / 4; ++h) {
-        v4i w;
-        w[0] = static_cast<int>(t[4 * h + 0][j]);
-        w[1] = static_cast<int>(t[4 * h + 1][j]);
-        w[2] = static_cast<int>(t[4 * h + 2][j]);
-        w[3] = static_cast<int>(t[4 * h + 3][j]);
-        *reinterpret_cast<v4i *>(lb + (j * 64 + bN4) * kPitch + bKq * kBlockRows + h * 16) = w;
-      }
-    }
-  };
-  auto storeBlockB = [&](u8 *lb, const v4i (&src)[kRowChunks]) {
-    if constexpr (EB == 1) {
-      storeBlockB8(lb, src);
-    } else {
-      storeBlockB16(lb, src);
-    }
-  };
-  auto storeLds = [&](int buf, const Stage &st) {
-    u8 *la = lds[buf][0];
-    u8 *lb = lds[buf][1];
-    storeRowsA(la, st.x);
-    if constexpr (TRANSB) {
-      storeRowsBt(lb, st.y);
-    } else if constexpr (TRB) {
-#pragma unroll
-      for (int i = 0; i < kRowChunks; ++i) {
-        *reinterpret_cast<v4i *>(lb + (bRowT + kRowStepB * i) * kPitchB + bChunkT * 16) = st.y[i];
-      }
-    } else {
-      storeBlockB(lb, st.y);
-    }
-  };
-
-  const int fragRow = lane & 31;
-  const int fragHalf = (lane >> 5) * 16;
-  const int aFragOff = (wm * kWaveRows + fragRow) * kPitch + fragHalf;
-  const int bFragOff = (wn * 32 + fragRow) * kPitch + fragHalf;
-  // TRB: lane = 16 g + s. Group g reads the columns 16 (g & 1) .. of the fragment's 32 for the k-half g >> 1; inside
-  // the group, 8-bit: lane s hands in k-row s >> 1, column octet s & 1; 16-bit: k-row s >> 2, column quad s & 3.
-  const int trS = lane & 15, trG = lane >> 4;
-  const int bFragOffT = EB == 1
-      ? ((trG >> 1) * 16 + (trS >> 1)) * kPitchB + (wn * 128 + (trG & 1) * 16 + (trS & 1) * 8)
-      : ((trG >> 1) * 8 + (trS >> 2)) * kPitchB + (wn * 128 + (trG & 1) * 16 + (trS & 3) * 4) * 2;
-
-  // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
-  // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
-  constexpr bool kAllRowsReal = (M % kGemmBM == 0);
-  const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
-  auto readFrags = [&](int buf, int ks, v4i (&af)[kTM], v4i (&bf)[4]) {
-    if (!kAllRowsReal && !waveHasRows) return;
-    const u8 *la = lds[buf][0] + aFragOff + ks * 32;
-    const u8 *lb = lds[buf][1] + bFragOff + ks * 32;
-#pragma unroll
-    for (int i = 0; i < kTM; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 32 * kPitch);
-    if constexpr (TRB) {
-      // Sixteen lanes share a transposing read: each hands in 8 bytes of one k-row and gets back, for one column,
-      // the elements of 8 (8-bit) or 4 (16-bit) consecutive k-rows. Two reads make the 16 bytes of K of a fragment.
-      typedef int v2i __attribute__((ext_vector_type(2)));
-      typedef short v4s __attribute__((ext_vector_type(4)));
-      const u8 *lt = lds[buf][1] + bFragOffT + ks * (32 / EB) * kPitchB;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const u8 *p0 = lt + j * 32 * EB;
-        const u8 *p1 = p0 + (8 / EB) * kPitchB;
-        if constexpr (EB == 1) {
-          const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(p0));
-          const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(p1));
-          bf[j] = v4i{lo[0], lo[1], hi[0], hi[1]};
-        } else {
-          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(p0));
-          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(p1));
-          const v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
-          bf[j] = v4i{l2[0], l2[1], h2[0], h2[1]};
-        }
-      }
-    } else {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 64 * kPitch);
-    }
-  };
-  auto mfmaAll = [&](const v4i (&af)[kTM], const v4i (&bf)[4]) {
-    if (!kAllRowsReal && !waveHasRows) return;
-#pragma unroll
-    for (int i = 0; i < kTM; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        acc[i][j] = Mma::mma(af[i], bf[j], acc[i][j]);
-      }
-    }
-  };
-
-  // ---- main loop. Invariant at the top of step s: LDS buffer s&1 holds tile s (complete), the staging registers hold
-  // tile s+1 (possibly still in flight), and f0 holds the fragments of the first 32 k of tile s.
-  //   a. staged tile s+1 -> LDS buffer (s+1)&1      (its last readers finished before the previous barrier)
-  //   b. issue the global loads of tile s+2 into the staging registers (they have a whole step to arrive)
-  //   c. for every k-substep but the last: read the next substep's fragments, MFMAs on the current ones
-  //      (a and b interleave with the MFMAs of the early substeps)
-  //   d. barrier: everybody has read tile s completely and has written tile s+1
-  //   e. read the first fragments of tile s+1         (their latency hides behind the MFMAs of f)
-  //   f. MFMAs on the last substep's fragments
-  v4i f0a[kTM], f0b[4], f1a[kTM], f1b[4];
-  // One K step. kStore / kLoad are compile-time so that the steady-state loop body is a single basic block (the
-  // last two steps, which have nothing left to store or load, are peeled off below).
-  auto stepBody = [&](long step, auto storeTag, auto loadTag) {
-    constexpr bool kStore = decltype(storeTag)::value;
-    constexpr bool kLoad = decltype(loadTag)::value;
-    const int buf = static_cast<int>(step & 1);
-    // The staged tile goes to the other LDS buffer at the very top of the step (its last readers finished before
-    // the previous step's barrier), and the freed staging registers are refilled at once: the LDS writes complete
-    // and the global loads travel while the step's MFMAs run, instead of piling up in front of the barrier.
-    if constexpr (kStore) storeLds(buf ^ 1, stage);
-    if constexpr (kLoad) loadGlobal(step + 2, stage);
-#pragma unroll
-    for (int ks = 0; ks + 2 < kSub; ks += 2) {
-      readFrags(buf, ks + 1, f1a, f1b);
-      mfmaAll(f0a, f0b);
-      readFrags(buf, ks + 2, f0a, f0b);
-      mfmaAll(f1a, f1b);
-    }
-    if constexpr (kSub > 2) __builtin_amdgcn_sched_barrier(0);  // keep the staging work in the early substeps
-    readFrags(buf, kSub - 1, f1a, f1b);
-    mfmaAll(f0a, f0b);
-    __syncthreads();
-    // ---- after the barrier: MFMAs on the last fragments of this tile; meanwhile fetch the first fragments of the next
-    if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
-    mfmaAll(f1a, f1b);
-  };
-  // ---- the same step with the staging spread over the substeps (operands whose staging is a plain copy of 16-byte
-  // chunks: B transposed in memory, or read with the transposing LDS reads): substep ks writes chunk ks of both operands
-  // to LDS and refills its registers from the tile after next, so that every group of 8 MFMAs has about the same
-  // number of LDS and memory instructions to cover; the order inside a substep is then fixed instruction by
-  // instruction (one MFMA, then a few of the others) instead of left to the scheduler, which clusters them.
-  constexpr bool kSpread = (TRB || TRANSB) && kSub == 4 && kRowChunks == 4;
-  auto storeChunk = [&](int buf, int i) {
-    u8 *la = lds[buf][0];
-    u8 *lb = lds[buf][1];
-    *reinterpret_cast<v4i *>(la + (aRow + kRowStep * i) * kPitch + aChunk * 16) = stage.x[i];
+  for (int i = 0; i < kRowChunks; ++i) {
     if constexpr (TRANSB) {
       const int col = aRow + kRowStep * i;
-      const int r = (col & 3) * 64 + (col >> 2);
-      *reinterpret_cast<v4i *>(lb + r * kPitch + aChunk * 16) = stage.y[i];
+      const int r = (col & ~63) + (col & 3) * 16 + ((col >> 2) & 15);
+      bStoreOff[i] = r * kPitch + (aChunk ^ pairSwap(r)) * 16;
     } else {
-      *reinterpret_cast<v4i *>(lb + (bRowT + kRowStepB * i) * kPitchB + bChunkT * 16) = stage.y[i];
+      const int krow = bRowT + kRowStepB * i;
+      const int odd = (krow / kGroupRowsB) & 1;
+      bStoreOff[i] = krow * kPitchB + (bChunkT ^ (odd * EB)) * 16;
     }
-  };
+  }
+
   auto loadChunk = [&](long step, int i) {
     const long k0 = (stepBase + step) * BK;
     if (kFull || (m0 + aRow + kRowStep * i < M && k0 + aChunk * 16 < K)) {
@@ -508,97 +302,226 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     } else {
       const long krow = k0 / EB + bRowT + kRowStepB * i;
       if (kFull || (krow < KE && n0 * EB + bChunkT * 16 < NB)) {
-        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoffT, static_cast<int>((k0 / EB + kRowStepB * i) * NB), 0);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoff, static_cast<int>((k0 / EB + kRowStepB * i) * NB), 0);
         stage.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
       } else {
         stage.y[i] = v4i{0, 0, 0, 0};
       }
     }
   };
+  auto storeChunk = [&](int buf, int i) {
+    *reinterpret_cast<v4i *>(lds[buf][0] + aStoreOff + (kRowStep * i) * kPitch) = stage.x[i];
+    *reinterpret_cast<v4i *>(lds[buf][1] + bStoreOff[i]) = stage.y[i];
+  };
+
+  // ---- fragments. Every MFMA takes 64 bytes of K per row: lane (c = lane % 16, g = lane / 16) holds the 16 bytes
+  // [16 g, +16) of row c of its A tile and of column c of its B tile (the same bytes of K in both, which is all the
+  // instruction needs), and receives rows 4 g .. 4 g + 3 of column c of the 16 x 16 result.
+  const int fragC = lane & 15, fragG = lane >> 4;
+  const int aFragOff = (wm * kWaveRows + fragC) * kPitch + (fragG ^ pairSwap(fragC)) * 16;
+  const int bFragOff = (wn * 128 + fragC) * kPitch + (fragG ^ pairSwap(fragC)) * 16;
+  // Row-major B: group g reads k-rows kGroupRowsB * g .. of the 64 bytes of K; inside the group, 8-bit: lane s hands in
+  // k-row s >> 1, column octet s & 1; 16-bit: k-row s >> 2, column quad s & 3. Even and odd column tiles have their own
+  // base because of the swap of units in the rows of odd groups.
+  const int trRow = fragG * kGroupRowsB + (EB == 1 ? (fragC >> 1) : (fragC >> 2));
+  const int trCol = EB == 1 ? (fragC & 1) * 8 : (fragC & 3) * 8;
+  const int trSwap = (fragG & 1) * 16 * EB;
+  const int bFragOffEven = trRow * kPitchB + wn * 128 * EB + trSwap + trCol;
+  const int bFragOffOdd = trRow * kPitchB + wn * 128 * EB - trSwap + trCol;
+
+  // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
+  // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
+  constexpr bool kAllRowsReal = (M % kGemmBM == 0);
+  const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
+  // A fragments of row half rh (2 tiles of 16 rows), K half kh (64 bytes)
+  auto readA = [&](int buf, int kh, int rh, v4i (&af)[2]) {
+    if (!kAllRowsReal && !waveHasRows) return;
+    const u8 *la = lds[buf][0] + aFragOff + kh * 64 + rh * 32 * kPitch;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 16 * kPitch);
+  };
+  // B fragments of column half ch (4 tiles of 16 columns), K half kh
+  auto readB = [&](int buf, int kh, int ch, v4i (&bf)[4]) {
+    if (!kAllRowsReal && !waveHasRows) return;
+    if constexpr (TRANSB) {
+      const u8 *lb = lds[buf][1] + bFragOff + kh * 64 + ch * 64 * kPitch;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 16 * kPitch);
+    } else {
+      typedef int v2i __attribute__((ext_vector_type(2)));
+      typedef short v4s __attribute__((ext_vector_type(4)));
+      const u8 *lt = lds[buf][1] + kh * (64 / EB) * kPitchB + ch * 64 * EB;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const u8 *p0 = lt + ((j & 1) ? bFragOffOdd : bFragOffEven) + j * 16 * EB;
+        const u8 *p1 = p0 + (8 / EB) * kPitchB;
+        if constexpr (EB == 1) {
+          const v2i lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(p0));
+          const v2i hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i *)(p1));
+          bf[j] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+          const v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(p0));
+          const v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(p1));
+          const v2i l2 = __builtin_bit_cast(v2i, lo), h2 = __builtin_bit_cast(v2i, hi);
+          bf[j] = v4i{l2[0], l2[1], h2[0], h2[1]};
+        }
+      }
+    }
+  };
+  // bFresh: the B fragments are the ones that have just been read: walk them one after the other (both row tiles on
+  // each) so that the last to arrive is wanted last; else the A fragments one after the other.
+  auto mfma8 = [&](int rh, int ch, const v4i (&af)[2], const v4i (&bf)[4], auto bFresh) {
+    if (!kAllRowsReal && !waveHasRows) return;
+    if constexpr (decltype(bFresh)::value) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          acc[rh * 2 + i][ch * 4 + j] = Mma::mma16(af[i], bf[j], acc[rh * 2 + i][ch * 4 + j]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[rh * 2 + i][ch * 4 + j] = Mma::mma16(af[i], bf[j], acc[rh * 2 + i][ch * 4 + j]);
+        }
+      }
+    }
+  };
+
+  // ---- main loop. A step is 8 substeps of 8 MFMAs: the wavefront's 64 x 128 tile in quarters (row half rh, column half
+  // ch), for each of the two 64-byte halves of K, walked so that consecutive substeps share one operand half and only the
+  // other is read anew: (0,0) (0,1) (1,1) (1,0) | (0,1) (0,0) (1,0) (1,1). Two register sets per operand: while one
+  // half feeds the MFMAs, the half needed next arrives in the other. Invariant at the top of step s: LDS buffer s & 1
+  // holds tile s, the staging registers hold tile s + 1 (possibly still in flight), fa[0] and fb[0] hold the fragments
+  // (rh 0, ch 0) of the first K half of tile s. The eight chunks of tile s + 1 go to the other LDS buffer in the
+  // substeps that read only A fragments (1, 2 and 5: an LDS write of 1 KiB occupies the LDS twice as long as a read, and
+  // eight wavefronts in step writing at once cost more cycles than the same writes one per MFMA), and their registers
+  // are refilled from tile s + 2 in substeps 3, 4 and 6; all fragment reads of tile s are issued by substep 5, the
+  // barrier follows it, and substeps 6 and 7 fetch the first fragments of tile s + 1. The order of MFMAs, LDS accesses
+  // and loads inside a substep is fixed instruction by instruction with scheduling groups instead of left to the
+  // scheduler, which clusters them: fragment reads two after each of the first MFMAs (their results are wanted by the
+  // next substep), writes one per MFMA.
+  v4i fa[2][2], fb[2][4];
   auto stepSpread = [&](long step, auto storeTag, auto loadTag) {
     constexpr bool kStore = decltype(storeTag)::value;
     constexpr bool kLoad = decltype(loadTag)::value;
-    constexpr int kFragReads = kTM + (TRB ? 8 : 4);
+    constexpr int kReadsA = 2, kReadsB = TRANSB ? 4 : 8;
     const int buf = static_cast<int>(step & 1);
-    // substep 0: fragments of substep 1; chunks 0 and 1 of tile s+1 to LDS
-    readFrags(buf, 1, f1a, f1b);
-    if constexpr (kStore) {
-      storeChunk(buf ^ 1, 0);
-      storeChunk(buf ^ 1, 1);
-    }
-    mfmaAll(f0a, f0b);
-    SubstepOrder<kFragReads, kStore ? 4 : 0, 0>::emit();
+    auto storeX = [&](int i) { *reinterpret_cast<v4i *>(lds[buf ^ 1][0] + aStoreOff + (kRowStep * i) * kPitch) = stage.x[i]; };
+    auto storeY = [&](int i) { *reinterpret_cast<v4i *>(lds[buf ^ 1][1] + bStoreOff[i]) = stage.y[i]; };
+    // substep 0: (0,0) of K half 0; B (ch 1) arrives
+    readB(buf, 0, 1, fb[1]);
+    mfma8(0, 0, fa[0], fb[0], BoolTag<true>());
+    SubstepFront<kReadsB, 0, 0>::emit();
     __builtin_amdgcn_sched_barrier(0);
-    // substep 1: fragments of substep 2; chunk 2 to LDS; chunks 0 and 1 of tile s+2 on their way
-    readFrags(buf, 2, f0a, f0b);
-    if constexpr (kStore) storeChunk(buf ^ 1, 2);
+    // substep 1: (0,1); A (rh 1) arrives; three chunks of tile s+1 to LDS
+    readA(buf, 0, 1, fa[1]);
+    if constexpr (kStore) {
+      storeX(0);
+      storeY(0);
+      storeX(1);
+    }
+    mfma8(0, 1, fa[0], fb[1], BoolTag<true>());
+    SubstepOrder<kReadsA, kStore ? 3 : 0, 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    // substep 2: (1,1); A (rh 0) of K half 1 arrives; three more chunks to LDS
+    readA(buf, 1, 0, fa[0]);
+    if constexpr (kStore) {
+      storeY(1);
+      storeX(2);
+      storeY(2);
+    }
+    mfma8(1, 1, fa[1], fb[1], BoolTag<false>());
+    SubstepOrder<kReadsA, kStore ? 3 : 0, 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    // substep 3: (1,0); B (ch 1) of K half 1 arrives; chunks 0 and 1 of tile s+2 on their way
+    readB(buf, 1, 1, fb[1]);
     if constexpr (kLoad) {
       loadChunk(step + 2, 0);
       loadChunk(step + 2, 1);
     }
-    mfmaAll(f1a, f1b);
-    SubstepOrder<kFragReads, kStore ? 2 : 0, kLoad ? 4 : 0>::emit();
+    mfma8(1, 0, fa[1], fb[0], BoolTag<false>());
+    SubstepFront<kReadsB, 0, kLoad ? 4 : 0>::emit();
     __builtin_amdgcn_sched_barrier(0);
-    // substep 2: fragments of substep 3; chunk 3 to LDS; chunk 2 on its way
-    readFrags(buf, 3, f1a, f1b);
-    if constexpr (kStore) storeChunk(buf ^ 1, 3);
+    // substep 4: K half 1, (0,1); B (ch 0) arrives; chunk 2 on its way
+    readB(buf, 1, 0, fb[0]);
     if constexpr (kLoad) loadChunk(step + 2, 2);
-    mfmaAll(f0a, f0b);
-    SubstepOrder<kFragReads, kStore ? 2 : 0, kLoad ? 2 : 0>::emit();
+    mfma8(0, 1, fa[0], fb[1], BoolTag<true>());
+    SubstepFront<kReadsB, 0, kLoad ? 2 : 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    // substep 5: (0,0); A (rh 1) arrives: the last read of tile s; the last two chunks to LDS
+    readA(buf, 1, 1, fa[1]);
+    if constexpr (kStore) {
+      storeX(3);
+      storeY(3);
+    }
+    mfma8(0, 0, fa[0], fb[0], BoolTag<true>());
+    SubstepOrder<kReadsA, kStore ? 2 : 0, 0>::emit();
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();   // everybody has read tile s completely and has written tile s+1
-    // substep 3: first fragments of tile s+1; chunk 3 on its way
-    if constexpr (kStore) readFrags(buf ^ 1, 0, f0a, f0b);
+    // substep 6: (1,0); first A fragments of tile s+1; chunk 3 of tile s+2 on its way
+    if constexpr (kStore) readA(buf ^ 1, 0, 0, fa[0]);
     if constexpr (kLoad) loadChunk(step + 2, 3);
-    mfmaAll(f1a, f1b);
-    SubstepOrder<kStore ? kFragReads : 0, 0, kLoad ? 2 : 0>::emit();
+    mfma8(1, 0, fa[1], fb[0], BoolTag<false>());
+    SubstepFront<kStore ? kReadsA : 0, 0, kLoad ? 2 : 0>::emit();
+    __builtin_amdgcn_sched_barrier(0);
+    // substep 7: (1,1); first B fragments of tile s+1
+    if constexpr (kStore) readB(buf ^ 1, 0, 0, fb[0]);
+    mfma8(1, 1, fa[1], fb[1], BoolTag<false>());
+    SubstepFront<kStore ? kReadsB : 0, 0, 0>::emit();
     __builtin_amdgcn_sched_barrier(0);
   };
-  loadGlobal(0, stage);
-  storeLds(0, stage);
-  if (mySteps > 1) loadGlobal(1, stage);
-  __syncthreads();
-  readFrags(0, 0, f0a, f0b);
-  long step = 0;
-  if constexpr (kSpread) {
-    for (; step + 2 < mySteps; ++step) stepSpread(step, BoolTag<true>(), BoolTag<true>());
-    if (step + 1 < mySteps) {
-      stepSpread(step, BoolTag<true>(), BoolTag<false>());
-      ++step;
-    }
-    stepSpread(step, BoolTag<false>(), BoolTag<false>());
-  } else {
-    for (; step + 2 < mySteps; ++step) stepBody(step, BoolTag<true>(), BoolTag<true>());
-    if (step + 1 < mySteps) {
-      stepBody(step, BoolTag<true>(), BoolTag<false>());
-      ++step;
-    }
-    stepBody(step, BoolTag<false>(), BoolTag<false>());
+#pragma unroll
+  for (int i = 0; i < kRowChunks; ++i) loadChunk(0, i);
+#pragma unroll
+  for (int i = 0; i < kRowChunks; ++i) storeChunk(0, i);
+  if (mySteps > 1) {
+#pragma unroll
+    for (int i = 0; i < kRowChunks; ++i) loadChunk(1, i);
   }
+  __syncthreads();
+  readA(0, 0, 0, fa[0]);
+  readB(0, 0, 0, fb[0]);
+  long step = 0;
+  for (; step + 2 < mySteps; ++step) stepSpread(step, BoolTag<true>(), BoolTag<true>());
+  if (step + 1 < mySteps) {
+    stepSpread(step, BoolTag<true>(), BoolTag<false>());
+    ++step;
+  }
+  stepSpread(step, BoolTag<false>(), BoolTag<false>());
 
-  // ---- epilogue: lane owns columns col4 .. col4+3 of 16 * kTM rows
-  // With the transposing reads column tile j holds the columns 32 j .. 32 j + 31 of the wavefront's 128, lane by lane,
-  // so the four lanes of a quad hold four neighbouring columns of each of the four tiles: a 4 x 4 transpose between
-  // the lanes of the quad and the tiles (two exchanges with quad permutations) gives lane c the four columns of tile c.
-  if constexpr (TRB) {
+  // ---- epilogue: a lane owns, per group of four column tiles (q = 0, 1), four ADJACENT columns of 16 rows.
+  // [N,K] B: the LDS row order gave tile 4 q + t of lane c column 64 q + 4 c + t. Row-major B: tile j holds the columns
+  // 16 j .. 16 j + 15 lane by lane, so the four lanes of a quad hold four neighbouring columns of each of four tiles:
+  // a 4 x 4 transpose between the lanes of the quad and the tiles (two exchanges with quad permutations) gives lane s
+  // of the quad the four columns of tile 4 q + s.
+  if constexpr (!TRANSB) {
     const bool odd = (lane & 1) != 0, upper = (lane & 2) != 0;
 #pragma unroll
     for (int i = 0; i < kTM; ++i) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        typename Mma::acc_t a0 = acc[i][0][v], a1 = acc[i][1][v], a2 = acc[i][2][v], a3 = acc[i][3][v];
-        const typename Mma::acc_t r01 = lane_partner<1>(odd ? a0 : a1), r23 = lane_partner<1>(odd ? a2 : a3);
-        if (odd) { a0 = r01; a2 = r23; } else { a1 = r01; a3 = r23; }
-        const typename Mma::acc_t r02 = lane_partner<2>(upper ? a0 : a2), r13 = lane_partner<2>(upper ? a1 : a3);
-        if (upper) { a0 = r02; a1 = r13; } else { a2 = r02; a3 = r13; }
-        acc[i][0][v] = a0;
-        acc[i][1][v] = a1;
-        acc[i][2][v] = a2;
-        acc[i][3][v] = a3;
+      for (int q = 0; q < 2; ++q) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          typename Mma::acc_t a0 = acc[i][4 * q][v], a1 = acc[i][4 * q + 1][v], a2 = acc[i][4 * q + 2][v], a3 = acc[i][4 * q + 3][v];
+          const typename Mma::acc_t r01 = lane_partner<1>(odd ? a0 : a1), r23 = lane_partner<1>(odd ? a2 : a3);
+          if (odd) { a0 = r01; a2 = r23; } else { a1 = r01; a3 = r23; }
+          const typename Mma::acc_t r02 = lane_partner<2>(upper ? a0 : a2), r13 = lane_partner<2>(upper ? a1 : a3);
+          if (upper) { a0 = r02; a1 = r13; } else { a2 = r02; a3 = r13; }
+          acc[i][4 * q][v] = a0;
+          acc[i][4 * q + 1][v] = a1;
+          acc[i][4 * q + 2][v] = a2;
+          acc[i][4 * q + 3][v] = a3;
+        }
       }
     }
   }
-  const long col4 = TRB ? n0 + wn * 128 + 32 * (lane & 3) + (fragRow & ~3) : n0 + 4 * (wn * 32 + fragRow);
+  // first of the lane's four columns in column group q, and the row of accumulator v of row tile i inside the tile
+  const long colBase = n0 + wn * 128 + (TRANSB ? 4 * fragC : 16 * (fragC & 3) + (fragC & ~3));
+  auto rowInTileOf = [&](int i, int v) { return static_cast<long>(wm * kWaveRows + i * 16 + fragG * 4 + v); };
   if constexpr (KSPLIT > 1) {
     constexpr long kPartRows = M < kGemmBM ? M : kGemmBM;            // rows of a tile that can hold results
     constexpr long kCounterBytes = (kGridTiles * 4 + 255) / 256 * 256;
@@ -607,56 +530,61 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     static_assert(kWsBytes < (1L << 31), "split-K workspace too large");
     const Buffer wsBuf = make_buffer(ws, kWsBytes);
     const u32 tileBase = static_cast<u32>(kCounterBytes + linear * KSPLIT * kPartBytes);
-    const bool colOk = kFull || col4 < N;
-    auto partOffset = [&](int i, int v) {
-      const long rowInTile = wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-      return static_cast<long>((rowInTile * kGemmBN + (col4 - n0)) * static_cast<long>(sizeof(typename Mma::acc_t)));
+    auto partOffset = [&](int i, int q, int v) {
+      return static_cast<long>((rowInTileOf(i, v) * kGemmBN + (colBase + 64 * q - n0)) * static_cast<long>(sizeof(typename Mma::acc_t)));
     };
-    auto rowOk = [&](int i, int v) {
-      const long rowInTile = wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-      return rowInTile < kPartRows && m0 + rowInTile < M;
-    };
+    auto rowOk = [&](int i, int v) { return rowInTileOf(i, v) < kPartRows && m0 + rowInTileOf(i, v) < M; };
 #pragma unroll
-    for (int i = 0; i < kTM; ++i) {
+    for (int q = 0; q < 2; ++q) {
+      if (!(kFull || colBase + 64 * q < N)) continue;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        if (colOk && rowOk(i, v)) {
-          const typename Mma::acc_t a4[4] = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
-          ws_store_chunk<4>(wsBuf, tileBase + static_cast<u32>(ksplit * kPartBytes + partOffset(i, v)), a4);
+      for (int i = 0; i < kTM; ++i) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          if (rowOk(i, v)) {
+            const typename Mma::acc_t a4[4] = {acc[i][4 * q][v], acc[i][4 * q + 1][v], acc[i][4 * q + 2][v], acc[i][4 * q + 3][v]};
+            ws_store_chunk<4>(wsBuf, tileBase + static_cast<u32>(ksplit * kPartBytes + partOffset(i, q, v)), a4);
+          }
         }
       }
     }
     __shared__ unsigned akg_gemm_flag;
     if (!last_workgroup(ws, linear, KSPLIT, tid, &akg_gemm_flag)) return;
-    if (!colOk) return;
-    epi.prepare(col4);
 #pragma unroll
-    for (int i = 0; i < kTM; ++i) {
+    for (int q = 0; q < 2; ++q) {
+      const long col4 = colBase + 64 * q;
+      if (!(kFull || col4 < N)) continue;
+      epi.prepare(col4);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        if (!rowOk(i, v)) continue;
-        typename Mma::acc_t sum[4] = {0, 0, 0, 0};
-        for (int p = 0; p < KSPLIT; ++p) {
-          typename Mma::acc_t part[4];
-          ws_load_chunk<4>(wsBuf, tileBase + static_cast<u32>(p * kPartBytes + partOffset(i, v)), part);
+      for (int i = 0; i < kTM; ++i) {
 #pragma unroll
-          for (int c = 0; c < 4; ++c) sum[c] += part[c];
+        for (int v = 0; v < 4; ++v) {
+          if (!rowOk(i, v)) continue;
+          typename Mma::acc_t sum[4] = {0, 0, 0, 0};
+          for (int p = 0; p < KSPLIT; ++p) {
+            typename Mma::acc_t part[4];
+            ws_load_chunk<4>(wsBuf, tileBase + static_cast<u32>(p * kPartBytes + partOffset(i, q, v)), part);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) sum[c] += part[c];
+          }
+          epi.apply(sum, m0 + rowInTileOf(i, v), col4);
         }
-        const long row = m0 + wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-        epi.apply(sum, row, col4);
       }
     }
     return;
   }
-  if (kFull || col4 < N) {
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const long col4 = colBase + 64 * q;
+    if (!(kFull || col4 < N)) continue;
     epi.prepare(col4);
 #pragma unroll
     for (int i = 0; i < kTM; ++i) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const long row = m0 + wm * kWaveRows + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+      for (int v = 0; v < 4; ++v) {
+        const long row = m0 + rowInTileOf(i, v);
         if (kFull || row < M) {
-          const typename Mma::acc_t a4[4] = {acc[i][0][v], acc[i][1][v], acc[i][2][v], acc[i][3][v]};
+          const typename Mma::acc_t a4[4] = {acc[i][4 * q][v], acc[i][4 * q + 1][v], acc[i][4 * q + 2][v], acc[i][4 * q + 3][v]};
           epi.apply(a4, row, col4);
         }
       }

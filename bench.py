@@ -222,6 +222,26 @@ def cpu_baseline(name, harness, driver):
     return out
 
 
+def vendor_gemm(kind, torch, steps):
+    """The vendor library's GEMM on the shape and layout of C5 (int8) / N2 (bf16): no epilogue, same buffers reused."""
+    dev = torch.device("cuda:0")
+    m, k, n = 4096, 8192, 8192
+    if kind == "int8":
+        a = torch.randint(-127, 128, (m, k), dtype=torch.int8, device=dev)
+        b = torch.randint(-127, 128, (k, n), dtype=torch.int8, device=dev)
+        call, peak, unit = (lambda i: torch._int_mm(a, b)), INT8_MFMA_PEAK_TOPS, "TOP/s"
+        what = "torch._int_mm, B row-major as in C5, int32 result, no epilogue, same buffers reused"
+    else:
+        a = (torch.randn((m, k), device=dev) * 0.25).to(torch.bfloat16)
+        b = (torch.randn((k, n), device=dev) * 0.25).to(torch.bfloat16)
+        call, peak, unit = (lambda i: torch.matmul(a, b)), BF16_MFMA_PEAK_TFLOPS, "TFLOP/s"
+        what = "torch.matmul, B row-major as in N2, bf16 result, no epilogue, same buffers reused"
+    _, mean_ms, med_ms, min_ms = timed(call, steps, 3, torch)
+    rate = 2.0 * m * n * k / (mean_ms * 1e-3) / 1e12
+    return {"kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5), "kernel_ms_min": round(min_ms, 5),
+            "achieved": round(rate, 1), "unit": unit, "frac": round(rate / peak, 4), "what": what}
+
+
 def calibration(torch, driver, harness, np, steps, warmup):
     """Ceilings of this box, measured in this run."""
     out = {}
@@ -282,25 +302,8 @@ def calibration(torch, driver, harness, np, steps, warmup):
         out["mfma_register_loops"] = {"error": str(e)}
     # 3. the vendor library on the GEMM shapes (no epilogue: plain int32 / bf16 result)
     try:
-        m, k, n = 4096, 8192, 8192
-        a8 = torch.randint(-127, 128, (m, k), dtype=torch.int8, device=dev)
-        b8 = torch.randint(-127, 128, (k, n), dtype=torch.int8, device=dev)
-        _, mean_ms, med_ms, min_ms = timed(lambda i: torch._int_mm(a8, b8), max(20, steps // 4), 3, torch)
-        rate = 2.0 * m * n * k / (mean_ms * 1e-3) / 1e12
-        out["vendor_int8_gemm_4096x8192x8192"] = {"kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5),
-                                                  "kernel_ms_min": round(min_ms, 5), "achieved": round(rate, 1), "unit": "TOP/s",
-                                                  "frac": round(rate / INT8_MFMA_PEAK_TOPS, 4),
-                                                  "what": "torch._int_mm, B row-major as in C5, int32 result, no epilogue, same buffers reused"}
-        del a8, b8
-        a16 = (torch.randn((m, k), device=dev) * 0.25).to(torch.bfloat16)
-        b16 = (torch.randn((k, n), device=dev) * 0.25).to(torch.bfloat16)
-        _, mean_ms, med_ms, min_ms = timed(lambda i: torch.matmul(a16, b16), max(20, steps // 4), 3, torch)
-        rate = 2.0 * m * n * k / (mean_ms * 1e-3) / 1e12
-        out["vendor_bf16_gemm_4096x8192x8192"] = {"kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5),
-                                                  "kernel_ms_min": round(min_ms, 5), "achieved": round(rate, 1), "unit": "TFLOP/s",
-                                                  "frac": round(rate / BF16_MFMA_PEAK_TFLOPS, 4),
-                                                  "what": "torch.matmul, B row-major as in N2, bf16 result, no epilogue, same buffers reused"}
-        del a16, b16
+        for kind in ("int8", "bf16"):
+            out["vendor_%s_gemm_4096x8192x8192" % kind] = vendor_gemm(kind, torch, max(20, steps // 4))
     except Exception as e:  # a torch build without these routines
         out["vendor_gemm"] = {"error": str(e)}
     return out
@@ -314,6 +317,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS) + [CALIBRATION] + sorted(SIZE_MATCHED))
     ap.add_argument("--only", action="store_true", help="measure only --workload (no per_config sweep, no calibration)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--vendor-gemm", choices=("int8", "bf16"),
+                    help="run only the vendor library's GEMM of the calibration (for a profiler) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every fused operator here is a single-device kernel (rows shard with no "
@@ -325,6 +330,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
 
+    if args.vendor_gemm:
+        print(json.dumps({"vendor_%s_gemm_4096x8192x8192" % args.vendor_gemm: vendor_gemm(args.vendor_gemm, torch, args.steps)}))
+        return
     name = args.workload
     kernel, _, wall_ms, kernel_ms, med_ms, min_ms, nsets = gpu_measure(name, args.steps, args.warmup, torch, driver, harness, np)
     roof = roofline_of(kernel, kernel_ms, name)
