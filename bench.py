@@ -272,32 +272,31 @@ def calibration(torch, driver, harness, np, steps, warmup):
     try:
         probe = ctypes.CDLL(PROBE_LIB)
         vp, ci = ctypes.c_void_p, ctypes.c_int
-        for fn in (probe.akg_probe_mfma_i8, probe.akg_probe_mfma_bf16):
+        fns = {"i8": probe.akg_probe_mfma_i8, "bf16": probe.akg_probe_mfma_bf16,
+               "i8_32x32": probe.akg_probe_mfma_i8_32x32, "bf16_32x32": probe.akg_probe_mfma_bf16_32x32}
+        for fn in fns.values():
             fn.argtypes = [vp, vp, ci, ci, vp]
         rng = np.random.default_rng(7)
         workgroups, iterations = 512, 500
         sink = torch.empty(workgroups * 512, dtype=torch.int32, device=dev)
         st = torch.cuda.current_stream().cuda_stream
-        operands = {
-            "mfma_i8_register_loop_zero_operands": (probe.akg_probe_mfma_i8, np.zeros(24 * 1024, np.uint8), INT8_MFMA_PEAK_TOPS, "TOP/s"),
-            "mfma_i8_register_loop_random_operands": (probe.akg_probe_mfma_i8,
-                                                      rng.integers(-127, 128, 24 * 1024, dtype=np.int8).view(np.uint8), INT8_MFMA_PEAK_TOPS, "TOP/s"),
-            "mfma_bf16_register_loop_zero_operands": (probe.akg_probe_mfma_bf16, np.zeros(24 * 1024, np.uint8), BF16_MFMA_PEAK_TFLOPS, "TFLOP/s"),
-            "mfma_bf16_register_loop_random_operands": (probe.akg_probe_mfma_bf16,
-                                                        harness.f32_to_bf16_bits((rng.standard_normal(12 * 1024) * 0.25).astype(np.float32)).view(np.uint8),
-                                                        BF16_MFMA_PEAK_TFLOPS, "TFLOP/s"),
-        }
-        for label, (fn, host, peak, unit) in operands.items():
-            # 32 MFMAs per wavefront and iteration: 32 x 32 x 32 int8 (65536 ops each) or 32 x 32 x 16 bf16 (32768)
-            ops = workgroups * 8 * iterations * 32 * (65536 if "i8" in label else 32768)
-            buf = torch.from_numpy(np.ascontiguousarray(host)).to(dev)
-            _, mean_ms, med_ms, min_ms = timed(lambda i: fn(st, buf.data_ptr(), iterations, workgroups, sink.data_ptr()),
-                                               max(10, steps // 10), 2, torch)
-            rate = ops / (mean_ms * 1e-3) / 1e12
-            out[label] = {"ops": ops, "kernel_ms": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
-                          "kernel_ms_min": round(min_ms, 4), "achieved": round(rate, 1), "unit": unit, "peak": peak,
-                          "frac": round(rate / peak, 4),
-                          "what": "512 workgroups x 8 wavefronts, 2 x 4 accumulator tiles each, nothing but MFMAs on register operands"}
+        zeros = np.zeros(32 * 1024, np.uint8)
+        random_i8 = rng.integers(-127, 128, 32 * 1024, dtype=np.int8).view(np.uint8)
+        random_bf16 = harness.f32_to_bf16_bits((rng.standard_normal(16 * 1024) * 0.25).astype(np.float32)).view(np.uint8)
+        for kind, peak, unit, per_iteration in (("i8", INT8_MFMA_PEAK_TOPS, "TOP/s", 2097152), ("bf16", BF16_MFMA_PEAK_TFLOPS, "TFLOP/s", 1048576)):
+            for shape, suffix in (("16x16 tiles, 64 bytes of K per MFMA (the GEMM kernel's shape)", ""), ("32x32 tiles, 32 bytes of K per MFMA", "_32x32")):
+                for operands, host in (("zero", zeros), ("random", random_i8 if kind == "i8" else random_bf16)):
+                    label = "mfma_%s%s_register_loop_%s_operands" % (kind, suffix, operands)
+                    fn = fns[kind + suffix]
+                    ops = workgroups * 8 * iterations * per_iteration
+                    buf = torch.from_numpy(np.ascontiguousarray(host)).to(dev)
+                    _, mean_ms, med_ms, min_ms = timed(lambda i: fn(st, buf.data_ptr(), iterations, workgroups, sink.data_ptr()),
+                                                       max(10, steps // 10), 2, torch)
+                    rate = ops / (mean_ms * 1e-3) / 1e12
+                    out[label] = {"ops": ops, "kernel_ms": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
+                                  "kernel_ms_min": round(min_ms, 4), "achieved": round(rate, 1), "unit": unit, "peak": peak,
+                                  "frac": round(rate / peak, 4),
+                                  "what": "512 workgroups x 8 wavefronts, nothing but MFMAs on register operands, " + shape}
     except OSError as e:
         out["mfma_register_loops"] = {"error": str(e)}
     # 3. the vendor library on the GEMM shapes (no epilogue: plain int32 / bf16 result)
