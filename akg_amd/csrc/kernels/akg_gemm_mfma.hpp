@@ -163,7 +163,8 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // (Measured and dropped: 2 x 2 wavefronts of 128 x 128 each (a third less LDS traffic, one wavefront per SIMD: 2 to 4 %
   // slower), 64-byte steps, staging split between two groups of wavefronts, 256 x 128 tiles with two workgroups per
   // CU; tiles fetched memory -> LDS directly (buffer_load_dwordx4 ... lds into rows without padding, chunks permuted
-  // against bank conflicts): correct, 2 % slower than the staging through registers; the K steps of different tiles in
+  // against bank conflicts; tried with both MFMA shapes): correct, the LDS pipe a third less busy, and 2 % slower (int8) or
+  // equal (bfloat16): the cycles saved on LDS writes are spent waiting for the tile to land before the barrier; the K steps of different tiles in
   // rotated order: 8 to 25 % slower, the workgroups of an XCD share their panels in L2 only while they walk K
   // together. With the staging switched off altogether the loop runs 17 % faster, whichever way the tiles travel: what
   // is left is the price of moving 64 KB per step and CU on a power-limited part.)
