@@ -46,6 +46,7 @@ struct LoweringOptions {
   //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows
   //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
   //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs, 7: no column kernel (several kernels instead)
+  //   column_reduce  5: one strip per workgroup (no second set of resident registers)
   //   segment_sum    1: every workgroup scans all ids, 2: positions grouped by segment first (whatever the size),
   //                  3: grouped by bucket of segments first (whatever the number of buckets), 4: as 3, chunks in launch order
   //   indexed        1: no LDS-tiled transposes, 2: no chunk-wide loads, 3: launch order of tiles, 5: no non-temporal hints

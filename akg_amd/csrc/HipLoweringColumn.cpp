@@ -55,13 +55,13 @@ class ColumnEmitter {
     k.kernelName = g_.name + "_kernel";
     k.source = src_.str();
     k.family = KernelFamily::ColumnReduce;
-    k.grid[0] = static_cast<unsigned>(outer_ * strips_);
+    k.grid[0] = static_cast<unsigned>(launched_);
     k.block[0] = static_cast<unsigned>(block_);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
     std::ostringstream note;
     note << "column_reduce outer=" << outer_ << " run=" << run_ << " inner=" << inner_ << " vec=" << vec_ << " threads=" << ly_ << "x" << lx_
-         << " rows/thread=" << chunks_ << " walks=" << (maxLevel_ + 1);
+         << " rows/thread=" << chunks_ << " walks=" << (maxLevel_ + 1) << (pipelined_ ? " strips pipelined" : "");
     k.scheduleNote = note.str();
     return k;
   }
@@ -80,6 +80,8 @@ class ColumnEmitter {
   int maxLevel_ = 0;
   int vec_ = 4, lx_ = 8, ly_ = 32, chunks_ = 1, block_ = 256;
   int64_t strips_ = 1;
+  bool pipelined_ = false;         // workgroups stay and walk several strips, the next strip's loads issued before the work on this one
+  int64_t launched_ = 0;           // workgroups launched
   bool aligned_ = true;            // every chunk starts at a multiple of its size and lies inside its row
   int reduceCount_ = 0;
 
@@ -224,14 +226,18 @@ class ColumnEmitter {
     // About four rows per thread keep enough loads in flight; the registers of the resident chunks bound the rest:
     // a chunk of every full-sized input per row of the thread, at most 64 registers in all, else a larger workgroup
     // (bf16 [64,768,1024] over the middle axis: 24 rows a thread in 256 threads 50.7 us, 12 in 512 48.6, 6 in 1024 49.4).
-    for (block_ = opt_.block > 0 ? opt_.block : 256; ; block_ *= 2) {
-      int64_t ly = std::min<int64_t>(std::max<int64_t>(1, pow2floor(run_ / 4)), block_ / 8);
-      int64_t lx = std::min<int64_t>(block_ / ly, lxMax);
-      ly = block_ / lx;
+    const auto shapeFor = [&](int block) {
+      int64_t ly = std::min<int64_t>(std::max<int64_t>(1, pow2floor(run_ / 4)), block / 8);
+      int64_t lx = std::min<int64_t>(block / ly, lxMax);
+      ly = block / lx;
+      block_ = block;
       lx_ = static_cast<int>(lx);
       ly_ = static_cast<int>(ly);
       chunks_ = static_cast<int>((run_ + ly - 1) / ly);
-      const int64_t regs = static_cast<int64_t>(chunks_) * ((fullBytes * vec_ + 3) / 4);
+      return static_cast<int64_t>(chunks_) * ((fullBytes * vec_ + 3) / 4);   // registers of a thread's resident chunks
+    };
+    for (int block = opt_.block > 0 ? opt_.block : 256; ; block *= 2) {
+      const int64_t regs = shapeFor(block);
       if (regs <= 64 || (regs <= 96 && block_ >= 1024)) break;
       if (block_ >= 1024 || opt_.block > 0) throw LoweringError("column kernel: the run does not fit the registers of a workgroup");
     }
@@ -242,6 +248,18 @@ class ColumnEmitter {
     }
     strips_ = (inner_ + static_cast<int64_t>(lx_) * vec_ - 1) / (static_cast<int64_t>(lx_) * vec_);
     if (outer_ * strips_ >= (1LL << 31)) throw LoweringError("column kernel: too many workgroups");
+    // A workgroup that keeps tens of KB resident loads, reduces, then stores, and its neighbours on the CU do the same in
+    // step: memory idles while they compute. With several strips per workgroup the loads of the next strip are issued
+    // before the work on this one (a second set of resident registers, one workgroup per CU). Worth it for large
+    // footprints only: many small workgroups per CU drift apart by themselves.
+    // (Measured on bf16 [64,768,1024] over the middle axis, LayerNorm: 48.0 us as 1024 workgroups of one strip, 45.0 us as
+    // 256 workgroups of four strips each. A 1024-thread workgroup with half the rows per thread, which would fit four
+    // wavefronts per SIMD beside the second set, spills under the 128-register limit and takes 87 us; softmax over 21
+    // classes of f16 [32,21,512,512], 24 resident registers in 256 threads: 114 us as it is, 150 us pipelined.)
+    const int64_t regs = static_cast<int64_t>(chunks_) * ((fullBytes * vec_ + 3) / 4);
+    constexpr int64_t kCUs = 256;
+    pipelined_ = opt_.variant != 5 && regs >= 40 && regs <= 64 && block_ == 512 && outer_ * strips_ >= 2 * kCUs;
+    launched_ = pipelined_ ? kCUs : outer_ * strips_;
   }
 
   void line(const std::string &s) { src_ << s << "\n"; }
@@ -363,14 +381,52 @@ class ColumnEmitter {
     src_ << ") {\n";
     src_ << "  constexpr int V = " << vec_ << ", LX = " << lx_ << ", LY = " << ly_ << ", CH = " << chunks_ << ", BLOCK = " << block_ << ";\n";
     src_ << "  constexpr long RUN = " << run_ << ", INNER = " << inner_ << ", STRIPS = " << strips_ << ";\n";
+    src_ << "  constexpr long TOTAL = " << outer_ * strips_ << ";   // strips in all\n";
     if (block_ > 64) line("  __shared__ __attribute__((aligned(16))) unsigned char akg_scratch[2][(BLOCK / 64) * LX * V * 8];");
     line("  const int tid = static_cast<int>(threadIdx.x), lx = tid % LX, ly = tid / LX;");
-    line("  const long akg_o = static_cast<long>(blockIdx.x) / STRIPS;");
-    line("  const long akg_col = (static_cast<long>(blockIdx.x) % STRIPS) * (LX * V) + lx * V;   // first column of this thread's chunks");
-    line("  const int akg_cols = akg_col >= INNER ? 0 : (INNER - akg_col < V ? static_cast<int>(INNER - akg_col) : V);   // columns inside the tensor");
-    line("  bool akg_row_ok[CH];");
-    line("#pragma unroll");
-    line("  for (int j = 0; j < CH; ++j) akg_row_ok[j] = ly + j * LY < RUN;");
+    // the resident chunks of one strip: every full-sized input as it came from memory
+    std::string packedParams, packedArgsA, packedArgsB;
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      const TensorValue &tv = g_.tensor(g_.inputs[i]);
+      if (!tv.used || flags_[static_cast<size_t>(g_.inputs[i])].rank() != Rank::Full) continue;
+      const std::string tag = dtypeTag(tv.dtype);
+      packedParams += ", akg::PackedChunk<" + tag + ", V> (&p_in" + std::to_string(i) + ")[CH]";
+      packedArgsA += ", akg_a" + std::to_string(i);
+      packedArgsB += ", akg_b_set" + std::to_string(i);
+      src_ << "  akg::PackedChunk<" << tag << ", V> akg_a" << i << "[CH];  // " << tv.name << "\n";
+      if (pipelined_) src_ << "  akg::PackedChunk<" << tag << ", V> akg_b_set" << i << "[CH];\n";
+    }
+    const char *kStripIndex =
+        "    const long akg_o = akg_strip / STRIPS;\n"
+        "    const long akg_col = (akg_strip % STRIPS) * (LX * V) + lx * V;   // first column of this thread's chunks\n"
+        "    const int akg_cols = akg_col >= INNER ? 0 : (INNER - akg_col < V ? static_cast<int>(INNER - akg_col) : V);   // columns inside the tensor\n"
+        "    bool akg_row_ok[CH];\n"
+        "#pragma unroll\n"
+        "    for (int j = 0; j < CH; ++j) akg_row_ok[j] = ly + j * LY < RUN;\n";
+    // ---- loads of a strip's resident chunks ----
+    src_ << "  auto akg_load = [&](long akg_strip" << packedParams << ") {\n" << kStripIndex;
+    for (size_t i = 0; i < g_.inputs.size(); ++i) {
+      const int t = g_.inputs[i];
+      const TensorValue &tv = g_.tensor(t);
+      const Flags f = flags_[static_cast<size_t>(t)];
+      if (!tv.used || f.rank() != Rank::Full) continue;
+      const std::string tag = dtypeTag(tv.dtype), in = "in" + std::to_string(i);
+      line("#pragma unroll");
+      line("    for (int j = 0; j < CH; ++j) {");
+      src_ << "      const " << tag << "::storage *akg_p = " << in << " + " << offsetExpr(f, "ly + j * LY", "akg_col") << ";\n";
+      if (aligned_) {
+        src_ << "      if (akg_row_ok[j] && akg_cols == V) akg::load_packed<" << tag << ", V, true>(akg_p, p_in" << i << "[j]);\n";
+        src_ << "      else akg::zero_packed(p_in" << i << "[j]);\n";
+      } else {
+        src_ << "      akg::load_packed_partial<" << tag << ", V>(akg_p, akg_row_ok[j] ? akg_cols : 0, p_in" << i << "[j]);\n";
+      }
+      line("    }");
+    }
+    line("  };");
+    // ---- the work on one strip ----
+    // (akg_between runs behind the loads of the strip's small inputs: the place to issue the next strip's resident loads,
+    // which then return after them)
+    src_ << "  auto akg_work = [&](long akg_strip" << packedParams << ", auto akg_between) {\n" << kStripIndex;
 
     // ---- inputs ----
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
@@ -384,18 +440,7 @@ class ColumnEmitter {
       v.level = 0;
       switch (v.rank) {
         case Rank::Full: {
-          // kept as it came from memory; unpacked at the top of every walk
-          src_ << "  akg::PackedChunk<" << tag << ", V> p_in" << i << "[CH];  // " << tv.name << "\n";
-          line("#pragma unroll");
-          line("  for (int j = 0; j < CH; ++j) {");
-          src_ << "    const " << tag << "::storage *akg_p = " << in << " + " << offsetExpr(f, "ly + j * LY", "akg_col") << ";\n";
-          if (aligned_) {
-            src_ << "    if (akg_row_ok[j] && akg_cols == V) akg::load_packed<" << tag << ", V, true>(akg_p, p_in" << i << "[j]);\n";
-            src_ << "    else akg::zero_packed(p_in" << i << "[j]);\n";
-          } else {
-            src_ << "    akg::load_packed_partial<" << tag << ", V>(akg_p, akg_row_ok[j] ? akg_cols : 0, p_in" << i << "[j]);\n";
-          }
-          line("  }");
+          // kept as it came from memory (akg_load); unpacked at the top of every walk
           v.defined = false;   // defined inside the walks
           v.ident = id("x", static_cast<int>(i));
           break;
@@ -428,6 +473,8 @@ class ColumnEmitter {
       }
     }
 
+    line("    akg_between();");
+
     // ---- one walk per level ----
     for (int walk = 0; walk <= maxLevel_; ++walk) {
       std::vector<const OpNode *> reduces;
@@ -458,6 +505,8 @@ class ColumnEmitter {
         const TensorValue &tv = g_.tensor(t);
         Val &v = vals_[static_cast<size_t>(t)];
         if (!tv.used || v.rank != Rank::Full) continue;
+        // (two sets of resident chunks leave no registers for what a walk could hand to the next one)
+        if (pipelined_ && walk > 0) src_ << "    akg::forget_derived(p_in" << i << "[j]);\n";
         src_ << "    " << computeTypeName(tv.dtype) << " " << v.ident << "[V];\n";
         src_ << "    akg::unpack_packed(p_in" << i << "[j], " << v.ident << ");\n";
         v.defined = true;
@@ -535,6 +584,26 @@ class ColumnEmitter {
         src_ << "  for (int e = 0; e < V; ++e) " << src << "[e] = " << v.ident << ";\n";
       }
       src_ << "  if (ly == 0) akg::store_chunk_partial<" << tag << ", V>(out" << i << " + " << offsetExpr(f, "0", "akg_col") << ", akg_cols, " << src << ");\n";
+    }
+    if (pipelined_ && block_ > 64) line("  __syncthreads();   // the scratch of the reductions is free for the next strip");
+    line("  };");
+    if (!pipelined_) {
+      src_ << "  akg_load(static_cast<long>(blockIdx.x)" << packedArgsA << ");\n";
+      src_ << "  akg_work(static_cast<long>(blockIdx.x)" << packedArgsA << ", [] {});\n";
+    } else {
+      line("  long akg_at = static_cast<long>(blockIdx.x);");
+      line("  if (akg_at >= TOTAL) return;");
+      src_ << "  akg_load(akg_at" << packedArgsA << ");\n";
+      line("  for (;;) {");
+      line("    long akg_next = akg_at + static_cast<long>(gridDim.x);");
+      src_ << "    akg_work(akg_at" << packedArgsA << ", [&] { if (akg_next < TOTAL) akg_load(akg_next" << packedArgsB << "); });\n";
+      line("    if (akg_next >= TOTAL) break;");
+      line("    akg_at = akg_next;");
+      line("    akg_next = akg_at + static_cast<long>(gridDim.x);");
+      src_ << "    akg_work(akg_at" << packedArgsB << ", [&] { if (akg_next < TOTAL) akg_load(akg_next" << packedArgsA << "); });\n";
+      line("    if (akg_next >= TOTAL) break;");
+      line("    akg_at = akg_next;");
+      line("  }");
     }
     line("}");
   }

@@ -803,6 +803,13 @@ AKG_DEV void load_packed_partial(const typename DT::storage *__restrict__ p, int
   __builtin_memcpy(&dst.raw, tmp, sizeof(tmp));
 }
 
+// Makes the compiler forget what it derived from a resident chunk: the next walk unpacks it again instead of keeping
+// every unpacked (or further computed) element of the previous walk alive in registers of its own.
+template <typename DT, int V>
+AKG_DEV void forget_derived(PackedChunk<DT, V> &p) {
+  if constexpr (PackedChunk<DT, V>::kBytes >= 4) asm volatile("" : "+v"(p.raw));
+}
+
 template <typename DT, int V>
 AKG_DEV void unpack_packed(const PackedChunk<DT, V> &src, typename DT::compute (&dst)[V]) {
   typename DT::storage tmp[V];

@@ -192,7 +192,17 @@ def _column_cases():
         x = b.input([2, 20000, 64], "float32")
         return [b.sub(x, b.reduce("ReduceMax", x, [1], True))]
 
+    def several_strips_per_workgroup(b):
+        # 16 x 35 strips of 44 resident registers a thread: 256 workgroups stay and take two or three strips each, the
+        # next one's chunks on their way while this one is worked on; 1101 columns end inside a chunk, 700 rows inside
+        # the last round of a thread's rows. Softmax over the middle axis, a weight per row of the run beside it.
+        x = b.input([16, 700, 1101], "float32")
+        w = b.input([700, 1], "float32")
+        e = b.unary("Exp", b.sub(x, b.reduce("ReduceMax", x, [1], True)))
+        return [b.mul(b.div(e, b.reduce("ReduceSum", e, [1], True)), w)]
+
     return {"l2_normalise_no_keep": (l2_normalise_no_keep, "column_reduce"), "centred_with_statistics": (centred_with_statistics, "column_reduce"),
+            "several_strips_per_workgroup": (several_strips_per_workgroup, "column_reduce"),
             "scaled_by_a_shared_plane": (scaled_by_a_shared_plane, "column_reduce"), "integer_range": (integer_range, "column_reduce"),
             "narrow_columns": (narrow_columns, "column_reduce"), "half_sums": (half_sums, "column_reduce"),
             "no_keep_meets_the_tensor_unreshaped": (no_keep_meets_the_tensor_unreshaped, "staged"),
@@ -213,6 +223,8 @@ def test_reductions_over_a_middle_axis_whose_results_meet_the_tensor_again(case)
     kernel = driver.HipKernel(text, out_dir=None)
     print("case %s: %s grid %d block %d" % (case, kernel.family, kernel.grid[0], kernel.block[0]), flush=True)
     assert kernel.family == family
+    if case == "several_strips_per_workgroup":
+        assert kernel.grid[0] == 256 and "constexpr long TOTAL = 560;" in kernel.source and "load_packed_partial" in kernel.source
     inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 790)
     expect = np_ref.evaluate(desc, inputs)
     wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]

@@ -721,14 +721,24 @@ def test_matmul_next_to_a_softmax_is_cut_behind_the_contraction(tmp_path, monkey
 def test_column_kernel_schedule():
     """One reduced axis that is not the innermost one, results used against the tensor: [O, R, I] with a workgroup per
     strip of columns; the chunks of a thread's rows stay in registers as loaded (the workgroup grows until they fit), one
-    walk per reduction level, no workspace."""
+    walk per reduction level, no workspace. Strips with a large footprint: one workgroup per CU walks several of them, the
+    next strip's chunks on their way into a second set of registers while this one is worked on."""
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n9_layernorm_axis1_bf16_64x768x1024.info"), out_dir=None)
-    assert k.family == "column_reduce" and k.workspace_bytes == 0 and (k.grid[0], k.block[0]) == (64 * 16, 512)
+    assert k.family == "column_reduce" and k.workspace_bytes == 0 and (k.grid[0], k.block[0]) == (256, 512)
     assert "constexpr int V = 8, LX = 8, LY = 64, CH = 12, BLOCK = 512;" in k.source and "// ---- walk 2 ----" in k.source
+    assert "constexpr long TOTAL = 1024;" in k.source
     assert k.source.count("akg::column_reduce<akg::RedSum, akg::f32, false, LX, BLOCK, V>") == 2
-    assert "akg::PackedChunk<akg::bf16, V> p_in0[CH];" in k.source and k.source.count("global__") == 1
+    assert "akg::PackedChunk<akg::bf16, V> akg_a0[CH];" in k.source and "akg::PackedChunk<akg::bf16, V> akg_b_set0[CH];" in k.source
+    assert k.source.count("global__") == 1 and k.source.count("akg::forget_derived(p_in0[j]);") == 2
+    assert "[&] { if (akg_next < TOTAL) akg_load(akg_next, akg_b_set0); }" in k.source
+    os.environ["AKG_HIP_VARIANT"] = "5"   # one strip per workgroup
+    try:
+        k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n9_layernorm_axis1_bf16_64x768x1024.info"), out_dir=None)
+    finally:
+        del os.environ["AKG_HIP_VARIANT"]
+    assert (k.grid[0], k.block[0]) == (64 * 16, 512) and "akg_b_set0" not in k.source and "forget_derived" not in k.source
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n8_softmax_axis1_f16_32x21x512x512.info"), out_dir=None)
-    assert (k.grid[0], k.block[0]) == (32 * 512, 256) and "LX = 64, LY = 4, CH = 6" in k.source
+    assert (k.grid[0], k.block[0]) == (32 * 512, 256) and "LX = 64, LY = 4, CH = 6" in k.source and "akg_b_set0" not in k.source
     # rows that are not a multiple of the chunk: element-aligned accesses, the last chunk partly outside
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_staged_layernorm_axis1_bf16_8x64x49.info"), out_dir=None)
     assert "load_packed_partial<akg::bf16, V>(akg_p, akg_row_ok[j] ? akg_cols : 0" in k.source and "store_chunk_partial" in k.source
