@@ -84,9 +84,9 @@ class GemmEmitter {
       note << " serial: the reference's k-ordered sum in the declared type on the vector ALUs, tile=64x" << 16 * epiWidth()
            << " grid=" << k.grid[0];
     } else if (skinny_) {
-      note << " skinny: strips of 128 columns, B straight into MFMA operands, mfma=" << mfmaName() << " waves=4 grid=" << k.grid[0];
+      note << " skinny: strips of 128 columns, B straight into MFMA operands, mfma=" << mfmaName(false) << " waves=4 grid=" << k.grid[0];
     } else {
-      note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName() << " waves=4x2 grid=" << k.grid[0];
+      note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName(true) << " waves=4x2 grid=" << k.grid[0];
     }
     if (kSplit_ > 1) note << " k_splits=" << kSplit_;
     k.scheduleNote = note.str();
@@ -118,7 +118,9 @@ class GemmEmitter {
   const char *mmaTraits() const {
     return elem_ == DType::I8 ? "akg::MmaI8" : (elem_ == DType::BF16 ? "akg::MmaBF16" : "akg::MmaF16");
   }
-  const char *mfmaName() const {
+  // the skinny kernel issues 32 x 32 MFMAs (32 bytes of K), the tile kernel 16 x 16 ones (64 bytes of K)
+  const char *mfmaName(bool tileKernel) const {
+    if (tileKernel) return elem_ == DType::I8 ? "i32_16x16x64_i8" : (elem_ == DType::BF16 ? "f32_16x16x32_bf16" : "f32_16x16x32_f16");
     return elem_ == DType::I8 ? "i32_32x32x32_i8" : (elem_ == DType::BF16 ? "f32_32x32x16_bf16" : "f32_32x32x16_f16");
   }
   std::string accType() const { return serial_ ? computeTypeName(g_.tensor(accId_).dtype) : (elem_ == DType::I8 ? "int" : "float"); }
