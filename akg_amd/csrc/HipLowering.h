@@ -43,7 +43,8 @@ struct LoweringOptions {
   int block = 0;        // threads per workgroup
   int split = 0;        // streaming reductions: workgroups sharing one group of outputs (AKG_HIP_SPLIT)
   // Experiment switch (AKG_HIP_VARIANT), read by whichever family lowers the kernel; 0 = the measured default.
-  //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows
+  //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows,
+  //                  bit 5: the other arrangement of the tile kernel's wavefronts (2 x 4 for 4 x 2 and back)
   //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
   //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs, 7: no column kernel (several kernels instead)
   //   column_reduce  5: one strip per workgroup (no second set of resident registers)

@@ -11,8 +11,8 @@
  *
  * Shape of the computation (all sizes are compile-time constants of the emitted kernel):
  *   C[M,N] = A[M,K] * B[K,N]            A row-major, B row-major ([N,K] when TRANSB)
- *   workgroup tile 256 x 256, K step 128 bytes, 4 x 2 wavefronts
- *   wavefront tile 64 x 128 = 4 x 8 MFMA tiles of 16 x 16 (4 accumulator registers each)
+ *   workgroup tile 256 x 256, K step 128 bytes, 4 x 2 wavefronts (WM = 4) or 2 x 4 (WM = 2)
+ *   wavefront tile 64 x 128 = 4 x 8 MFMA tiles of 16 x 16 (4 accumulator registers each), or 128 x 64 = 8 x 4
  *
  * Data movement:
  *   global -> registers -> LDS, double buffered in LDS (one barrier per K step); the global loads of step
@@ -149,7 +149,7 @@ struct SubstepFront {
   }
 };
 
-template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1>
+template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1, int WM = 4>
 AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi,
                           unsigned *__restrict__ ws = nullptr) {
   constexpr int EB = Mma::kElemBytes;
@@ -168,16 +168,20 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // rotated order: 8 to 25 % slower, the workgroups of an XCD share their panels in L2 only while they walk K
   // together. With the staging switched off altogether the loop runs 17 % faster, whichever way the tiles travel: what
   // is left is the price of moving 64 KB per step and CU on a power-limited part.)
-  constexpr int WAVES_M = 4;
+  constexpr int WAVES_M = WM;            // 4 x 2 wavefronts of 64 x 128, or 2 x 4 of 128 x 64
+  constexpr int WAVES_N = 8 / WM;
   constexpr int BK = 128;
-  constexpr int kThreads = WAVES_M * 128;
+  constexpr int kThreads = 512;
   constexpr int kPitch = BK + 16;                     // LDS row of a K-contiguous tile: BK data bytes + 16 pad
   constexpr int kChunksPerRow = BK / 16;              // 16-byte chunks per row of a K-contiguous operand tile
   constexpr int kRowChunks = 256 * kChunksPerRow / kThreads;  // 16-byte chunks per thread and operand (4)
   constexpr int kRowStep = kThreads / kChunksPerRow;  // rows between two chunks of one thread
-  constexpr int kTM = 4;                              // MFMA row tiles (16 rows) per wavefront
-  constexpr int kTN = 8;                              // MFMA column tiles (16 columns) per wavefront
-  constexpr int kWaveRows = kGemmBM / WAVES_M;        // 64
+  constexpr int kWaveRows = kGemmBM / WAVES_M;        // 64 (128)
+  constexpr int kWaveCols = kGemmBN / WAVES_N;        // 128 (64)
+  constexpr int kTM = kWaveRows / 16;                 // MFMA row tiles (16 rows) per wavefront
+  constexpr int kTN = kWaveCols / 16;                 // MFMA column tiles (16 columns) per wavefront
+  constexpr int kHM = kTM / 2, kHN = kTN / 2;         // tiles per half: a quarter of the wavefront tile is kHM x kHN = 8 MFMAs
+  static_assert(kHM * kHN == 8, "a substep is 8 MFMAs");
   constexpr long kTilesM = (M + kGemmBM - 1) / kGemmBM;
   constexpr long kTilesN = (N + kGemmBN - 1) / kGemmBN;
   constexpr long kTiles = kTilesM * kTilesN;
@@ -227,8 +231,8 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const int tid = static_cast<int>(threadIdx.x);
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1;
-  const int wn = wave & 1;
+  const int wm = wave / WAVES_N;
+  const int wn = wave % WAVES_N;
 
   typename Mma::acc4_v acc[kTM][kTN];
 #pragma unroll
@@ -320,40 +324,40 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // instruction needs), and receives rows 4 g .. 4 g + 3 of column c of the 16 x 16 result.
   const int fragC = lane & 15, fragG = lane >> 4;
   const int aFragOff = (wm * kWaveRows + fragC) * kPitch + (fragG ^ pairSwap(fragC)) * 16;
-  const int bFragOff = (wn * 128 + fragC) * kPitch + (fragG ^ pairSwap(fragC)) * 16;
+  const int bFragOff = (wn * kWaveCols + fragC) * kPitch + (fragG ^ pairSwap(fragC)) * 16;
   // Row-major B: group g reads k-rows kGroupRowsB * g .. of the 64 bytes of K; inside the group, 8-bit: lane s hands in
   // k-row s >> 1, column octet s & 1; 16-bit: k-row s >> 2, column quad s & 3. Even and odd column tiles have their own
   // base because of the swap of units in the rows of odd groups.
   const int trRow = fragG * kGroupRowsB + (EB == 1 ? (fragC >> 1) : (fragC >> 2));
   const int trCol = EB == 1 ? (fragC & 1) * 8 : (fragC & 3) * 8;
   const int trSwap = (fragG & 1) * 16 * EB;
-  const int bFragOffEven = trRow * kPitchB + wn * 128 * EB + trSwap + trCol;
-  const int bFragOffOdd = trRow * kPitchB + wn * 128 * EB - trSwap + trCol;
+  const int bFragOffEven = trRow * kPitchB + wn * kWaveCols * EB + trSwap + trCol;
+  const int bFragOffOdd = trRow * kPitchB + wn * kWaveCols * EB - trSwap + trCol;
 
   // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
   // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
   constexpr bool kAllRowsReal = (M % kGemmBM == 0);
   const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
   // A fragments of row half rh (2 tiles of 16 rows), K half kh (64 bytes)
-  auto readA = [&](int buf, int kh, int rh, v4i (&af)[2]) {
+  auto readA = [&](int buf, int kh, int rh, v4i (&af)[kHM]) {
     if (!kAllRowsReal && !waveHasRows) return;
-    const u8 *la = lds[buf][0] + aFragOff + kh * 64 + rh * 32 * kPitch;
+    const u8 *la = lds[buf][0] + aFragOff + kh * 64 + rh * (kHM * 16) * kPitch;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 16 * kPitch);
+    for (int i = 0; i < kHM; ++i) af[i] = *reinterpret_cast<const v4i *>(la + i * 16 * kPitch);
   };
   // B fragments of column half ch (4 tiles of 16 columns), K half kh
-  auto readB = [&](int buf, int kh, int ch, v4i (&bf)[4]) {
+  auto readB = [&](int buf, int kh, int ch, v4i (&bf)[kHN]) {
     if (!kAllRowsReal && !waveHasRows) return;
     if constexpr (TRANSB) {
-      const u8 *lb = lds[buf][1] + bFragOff + kh * 64 + ch * 64 * kPitch;
+      const u8 *lb = lds[buf][1] + bFragOff + kh * 64 + ch * (kHN * 16) * kPitch;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 16 * kPitch);
+      for (int j = 0; j < kHN; ++j) bf[j] = *reinterpret_cast<const v4i *>(lb + j * 16 * kPitch);
     } else {
       typedef int v2i __attribute__((ext_vector_type(2)));
       typedef short v4s __attribute__((ext_vector_type(4)));
-      const u8 *lt = lds[buf][1] + kh * (64 / EB) * kPitchB + ch * 64 * EB;
+      const u8 *lt = lds[buf][1] + kh * (64 / EB) * kPitchB + ch * (kHN * 16) * EB;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < kHN; ++j) {
         const u8 *p0 = lt + ((j & 1) ? bFragOffOdd : bFragOffEven) + j * 16 * EB;
         const u8 *p1 = p0 + (8 / EB) * kPitchB;
         if constexpr (EB == 1) {
@@ -371,22 +375,22 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   };
   // bFresh: the B fragments are the ones that have just been read: walk them one after the other (both row tiles on
   // each) so that the last to arrive is wanted last; else the A fragments one after the other.
-  auto mfma8 = [&](int rh, int ch, const v4i (&af)[2], const v4i (&bf)[4], auto bFresh) {
+  auto mfma8 = [&](int rh, int ch, const v4i (&af)[kHM], const v4i (&bf)[kHN], auto bFresh) {
     if (!kAllRowsReal && !waveHasRows) return;
     if constexpr (decltype(bFresh)::value) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < kHN; ++j) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-          acc[rh * 2 + i][ch * 4 + j] = Mma::mma16(af[i], bf[j], acc[rh * 2 + i][ch * 4 + j]);
+        for (int i = 0; i < kHM; ++i) {
+          acc[rh * kHM + i][ch * kHN + j] = Mma::mma16(af[i], bf[j], acc[rh * kHM + i][ch * kHN + j]);
         }
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < kHM; ++i) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          acc[rh * 2 + i][ch * 4 + j] = Mma::mma16(af[i], bf[j], acc[rh * 2 + i][ch * 4 + j]);
+        for (int j = 0; j < kHN; ++j) {
+          acc[rh * kHM + i][ch * kHN + j] = Mma::mma16(af[i], bf[j], acc[rh * kHM + i][ch * kHN + j]);
         }
       }
     }
@@ -405,11 +409,11 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // and loads inside a substep is fixed instruction by instruction with scheduling groups instead of left to the
   // scheduler, which clusters them: fragment reads two after each of the first MFMAs (their results are wanted by the
   // next substep), writes one per MFMA.
-  v4i fa[2][2], fb[2][4];
+  v4i fa[2][kHM], fb[2][kHN];
   auto stepSpread = [&](long step, auto storeTag, auto loadTag) {
     constexpr bool kStore = decltype(storeTag)::value;
     constexpr bool kLoad = decltype(loadTag)::value;
-    constexpr int kReadsA = 2, kReadsB = TRANSB ? 4 : 8;
+    constexpr int kReadsA = kHM, kReadsB = TRANSB ? kHN : 2 * kHN;
     const int buf = static_cast<int>(step & 1);
     auto storeX = [&](int i) { *reinterpret_cast<v4i *>(lds[buf ^ 1][0] + aStoreOff + (kRowStep * i) * kPitch) = stage.x[i]; };
     auto storeY = [&](int i) { *reinterpret_cast<v4i *>(lds[buf ^ 1][1] + bStoreOff[i]) = stage.y[i]; };
@@ -504,7 +508,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 #pragma unroll
     for (int i = 0; i < kTM; ++i) {
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
+      for (int q = 0; q < kTN / 4; ++q) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
           typename Mma::acc_t a0 = acc[i][4 * q][v], a1 = acc[i][4 * q + 1][v], a2 = acc[i][4 * q + 2][v], a3 = acc[i][4 * q + 3][v];
@@ -521,7 +525,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     }
   }
   // first of the lane's four columns in column group q, and the row of accumulator v of row tile i inside the tile
-  const long colBase = n0 + wn * 128 + (TRANSB ? 4 * fragC : 16 * (fragC & 3) + (fragC & ~3));
+  const long colBase = n0 + wn * kWaveCols + (TRANSB ? 4 * fragC : 16 * (fragC & 3) + (fragC & ~3));
   auto rowInTileOf = [&](int i, int v) { return static_cast<long>(wm * kWaveRows + i * 16 + fragG * 4 + v); };
   if constexpr (KSPLIT > 1) {
     constexpr long kPartRows = M < kGemmBM ? M : kGemmBM;            // rows of a tile that can hold results
@@ -536,7 +540,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     };
     auto rowOk = [&](int i, int v) { return rowInTileOf(i, v) < kPartRows && m0 + rowInTileOf(i, v) < M; };
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < kTN / 4; ++q) {
       if (!(kFull || colBase + 64 * q < N)) continue;
 #pragma unroll
       for (int i = 0; i < kTM; ++i) {
@@ -552,7 +556,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     __shared__ unsigned akg_gemm_flag;
     if (!last_workgroup(ws, linear, KSPLIT, tid, &akg_gemm_flag)) return;
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
+    for (int q = 0; q < kTN / 4; ++q) {
       const long col4 = colBase + 64 * q;
       if (!(kFull || col4 < N)) continue;
       epi.prepare(col4);
@@ -575,7 +579,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
     return;
   }
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
+  for (int q = 0; q < kTN / 4; ++q) {
     const long col4 = colBase + 64 * q;
     if (!(kFull || col4 < N)) continue;
     epi.prepare(col4);
