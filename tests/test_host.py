@@ -767,6 +767,26 @@ def test_skinny_matmul_gets_the_streaming_kernel():
     assert "gemm_skinny" not in k.source                    # 6000 bytes of K: not a multiple of 32
 
 
+def test_tile_kernel_arranges_its_wavefronts_by_operand_type():
+    """The 256 x 256 tile kernel: int8 with a row-major B runs 2 x 4 wavefronts of 128 x 64 (half the transposing reads of
+    B), the 16-bit types and a B given as [N,K] keep 4 x 2 wavefronts of 64 x 128; AKG_HIP_VARIANT bit 5 swaps the two."""
+    tall = "akg::gemm_256x256<akg::MmaI8, 512L, 768L, 1024L, false, Epilogue, 1, 2>("
+    k = driver.HipKernel(op_desc.gemm_int8_dequant_bias_gelu(512, 1024, 768, "bfloat16", False, "tall_tiles"), out_dir=None)
+    assert tall in k.source
+    k = driver.HipKernel(op_desc.gemm_int8_dequant_bias_gelu(512, 1024, 768, "bfloat16", True, "wide_tiles_tb"), out_dir=None)
+    assert "akg::gemm_256x256<akg::MmaI8, 512L, 768L, 1024L, true, Epilogue, 1>(" in k.source
+    k = driver.HipKernel(op_desc.gemm_bias_act(512, 1024, 768, "bfloat16", "gelu", False, "float32", "wide_tiles_bf16"), out_dir=None)
+    assert "akg::gemm_256x256<akg::MmaBF16, 512L, 768L, 1024L, false, Epilogue, 3>(" in k.source
+    os.environ["AKG_HIP_VARIANT"] = "32"
+    try:
+        k = driver.HipKernel(op_desc.gemm_int8_dequant_bias_gelu(512, 1024, 768, "bfloat16", False, "tall_tiles"), out_dir=None)
+        assert tall not in k.source
+        k = driver.HipKernel(op_desc.gemm_bias_act(512, 1024, 768, "bfloat16", "gelu", False, "float32", "wide_tiles_bf16"), out_dir=None)
+        assert "akg::gemm_256x256<akg::MmaBF16, 512L, 768L, 1024L, false, Epilogue, 3, 2>(" in k.source
+    finally:
+        del os.environ["AKG_HIP_VARIANT"]
+
+
 def test_compiling_from_several_threads_gives_the_serial_results(tmp_path, monkeypatch):
     """The reference compiles one kernel per process (its schedule tools are process-wide singletons,
     GlobalVars.hpp:129-132) and forks workers over a directory (benchmark.py:304-317). This library is called from
