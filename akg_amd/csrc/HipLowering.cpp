@@ -219,11 +219,13 @@ ReduceSpec reduceSpec(const OpNode &op, DType od) {
       if (od == DType::Bool) throw LoweringError("ReduceSum on bool is not supported");
       r.combiner = "akg::RedSum";
       r.init = literalFor(od, 0.0);
+      r.ordered = od == DType::F16 || od == DType::BF16;
       break;
     case OpKind::ReduceProd:
       if (od == DType::Bool) throw LoweringError("ReducePrd on bool is not supported");
       r.combiner = "akg::RedProd";
       r.init = literalFor(od, 1.0);
+      r.ordered = od == DType::F16 || od == DType::BF16;
       break;
     case OpKind::ReduceMax:
       if (od == DType::Bool) throw LoweringError("ReduceMax on bool is not supported");

@@ -128,6 +128,10 @@ struct ReduceSpec {
   std::string combiner;        // "akg::RedSum", ...
   std::string init;            // literal of the compute type
   bool roundEachStep = false;  // narrow result types accumulate in that type: round after every step
+  // A float16 / bfloat16 sum or product: rounding after every step makes the order of the steps part of the result, and
+  // the reference's is one serial loop per result element in index order. (Integer sums and products wrap around and
+  // are the same in any order; a maximum is one of its operands.)
+  bool ordered = false;
 };
 ReduceSpec reduceSpec(const OpNode &op, DType od);
 }  // namespace lowering

@@ -13,8 +13,10 @@
  * the elementwise ops in front of it; the last walk computes the outputs. The tensor is read once and written once.
  *
  * Reductions follow createInitValueForReduce / createCombinerForReduce of the reference (MindSporeToLinalg.cpp:791-901):
- * same initial values and combiners, narrow result types rounded after every step; the order of a run's additions is the
- * kernel's own (rows of one thread in increasing order, then the threads), as in the other reducing families.
+ * same initial values and combiners, narrow result types rounded after every step. A float16 / bfloat16 sum or product
+ * keeps the reference's order, one serial chain per column over the rows of the run (akg::column_chain_step); every
+ * other combiner gives the same result in any order (integers wrap, a maximum is one of its operands) or is a float32 /
+ * float64 sum, whose order is the kernel's own (rows of one thread in increasing order, then the threads).
  */
 #include <algorithm>
 #include <sstream>
@@ -84,6 +86,7 @@ class ColumnEmitter {
   int64_t launched_ = 0;           // workgroups launched
   bool aligned_ = true;            // every chunk starts at a multiple of its size and lies inside its row
   int reduceCount_ = 0;
+  bool ordered_ = false;           // some reduction is a float16 / bfloat16 sum or product: steps in index order
 
   static std::string id(const char *prefix, int t) { return std::string(prefix) + std::to_string(t); }
 
@@ -166,6 +169,7 @@ class ColumnEmitter {
         if (flags_[static_cast<size_t>(out)].r || !flags_[static_cast<size_t>(out)].i) {
           throw LoweringError("op " + op.name + ": result shape does not match");
         }
+        ordered_ = ordered_ || lowering::reduceSpec(op, g_.tensor(out).dtype).ordered;
         lv += 1;
       } else if (!lowering::isElementwiseKind(op.kind) || op.kind == OpKind::Assign || op.kind == OpKind::Iota) {
         throw LoweringError("op " + op.name + ": not an elementwise op or a reduction");
@@ -258,7 +262,7 @@ class ColumnEmitter {
     // classes of f16 [32,21,512,512], 24 resident registers in 256 threads: 114 us as it is, 150 us pipelined.)
     const int64_t regs = static_cast<int64_t>(chunks_) * ((fullBytes * vec_ + 3) / 4);
     constexpr int64_t kCUs = 256;
-    pipelined_ = opt_.variant != 5 && regs >= 40 && regs <= 64 && block_ == 512 && outer_ * strips_ >= 2 * kCUs;
+    pipelined_ = !ordered_ && opt_.variant != 5 && regs >= 40 && regs <= 64 && block_ == 512 && outer_ * strips_ >= 2 * kCUs;
     launched_ = pipelined_ ? kCUs : outer_ * strips_;
   }
 
@@ -383,6 +387,12 @@ class ColumnEmitter {
     src_ << "  constexpr long RUN = " << run_ << ", INNER = " << inner_ << ", STRIPS = " << strips_ << ";\n";
     src_ << "  constexpr long TOTAL = " << outer_ * strips_ << ";   // strips in all\n";
     if (block_ > 64) line("  __shared__ __attribute__((aligned(16))) unsigned char akg_scratch[2][(BLOCK / 64) * LX * V * 8];");
+    if (ordered_) {
+      // the rows of one step of an ordered reduction, in their 16-bit type, and the folded results per column
+      line("  constexpr int NOWN = (LX * V + BLOCK - 1) / BLOCK;   // columns a thread folds");
+      line("  __shared__ __attribute__((aligned(16))) unsigned short akg_chain[LY * LX * V];");
+      line("  __shared__ float akg_chain_res[LX * V];");
+    }
     line("  const int tid = static_cast<int>(threadIdx.x), lx = tid % LX, ly = tid / LX;");
     // the resident chunks of one strip: every full-sized input as it came from memory
     std::string packedParams, packedArgsA, packedArgsB;
@@ -497,6 +507,11 @@ class ColumnEmitter {
         src_ << "  " << computeTypeName(od) << " acc" << out << "[V];  // " << op->name << " -> " << g_.tensor(out).name << "\n";
         line("#pragma unroll");
         src_ << "  for (int e = 0; e < V; ++e) acc" << out << "[e] = " << spec.init << ";\n";
+        if (spec.ordered) {
+          src_ << "  " << computeTypeName(od) << " own" << out << "[NOWN];\n";
+          line("#pragma unroll");
+          src_ << "  for (int k = 0; k < NOWN; ++k) own" << out << "[k] = " << spec.init << ";\n";
+        }
       }
       line("#pragma unroll");
       line("  for (int j = 0; j < CH; ++j) {");
@@ -518,6 +533,12 @@ class ColumnEmitter {
         const lowering::ReduceSpec spec = lowering::reduceSpec(*op, od);
         const Val &in = vals_[static_cast<size_t>(op->inputs[0])];
         if (!in.defined || in.rank != Rank::Full) throw LoweringError("op " + op->name + ": operand is not computed in its walk");
+        if (spec.ordered) {
+          // rows j * LY .. j * LY + LY - 1 of the run are this step's: through LDS, folded in order by the columns' owners
+          src_ << "    akg::column_chain_step<" << spec.combiner << ", " << dtypeTag(od) << ", LX, BLOCK, V, NOWN>(own" << out << ", " << in.ident
+               << ", reinterpret_cast<" << dtypeTag(od) << "::storage *>(akg_chain), tid, static_cast<int>(RUN - j * LY < LY ? RUN - j * LY : LY));\n";
+          continue;
+        }
         std::string step = spec.combiner + "::apply(acc" + std::to_string(out) + "[e], " + in.ident + "[e])";
         if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
         line("#pragma unroll");
@@ -556,6 +577,15 @@ class ColumnEmitter {
         const DType od = g_.tensor(out).dtype;
         const lowering::ReduceSpec spec = lowering::reduceSpec(*op, od);
         const std::string ct = computeTypeName(od);
+        if (spec.ordered) {
+          src_ << "  akg::column_chain_finish<" << dtypeTag(od) << ", LX, BLOCK, V, NOWN>(own" << out << ", acc" << out << ", akg_chain_res, tid);\n";
+          Val &v = vals_[static_cast<size_t>(out)];
+          v.defined = true;
+          v.rank = Rank::Col;
+          v.ident = "acc" + std::to_string(out);
+          v.level = walk + 1;
+          continue;
+        }
         const std::string scratch = block_ > 64 ? "reinterpret_cast<" + ct + " *>(akg_scratch[" + std::to_string(reduceCount_ & 1) + "])"
                                                 : "static_cast<" + ct + " *>(nullptr)";
         src_ << "  akg::column_reduce<" << spec.combiner << ", " << dtypeTag(od) << ", " << (spec.roundEachStep ? "true" : "false")

@@ -109,6 +109,10 @@ class StreamReduceEmitter {
   uint64_t workspaceBytes_ = 0;
   std::vector<uint64_t> partialOffset_;  // per reduction, bytes from the workspace base
   bool useBuffers_ = true;
+  // Some reduction is a float16 / bfloat16 sum or product, whose steps the reference takes in index order: no split
+  // over workgroups or thread-rows. Direction Y: one thread per V columns walks the whole reduced extent. Direction
+  // X: the workgroup streams tiles of BLOCK * V elements through LDS and its first thread folds them in order.
+  bool ordered_ = false;
   std::vector<bool> relaxed_;
   std::vector<std::string> ident_;  // per tensor: array / scalar name once defined
 
@@ -198,6 +202,7 @@ class StreamReduceEmitter {
       if (std::string(computeTypeName(in.dtype)) != computeTypeName(od)) {
         throw LoweringError("op " + op->name + ": operand and result element types differ");
       }
+      ordered_ = ordered_ || lowering::reduceSpec(*op, od).ordered;
     }
     // Fold: neighbouring dims that are both reduced or both kept, and that every input spans or broadcasts together,
     // become one dim ([N,C,H,W] over N, H, W is [N,C,H*W]: chunks may then run across H). Unit dims join their
@@ -410,7 +415,7 @@ class StreamReduceEmitter {
     for (int id : g_.outputs) allBuffers = allBuffers && !tooLargeForBuffer(id);
     if (dirY_ && allBuffers && opt_.vec == 0 && fastExtent == I_ && (I_ % v) != 0 && I_ >= 2 * v) {
       overlapTail_ = true;
-    } else if (!dirY_ && allBuffers && opt_.vec == 0 && (fastExtent % v) != 0 && fastExtent >= 2 * v && R_ < (1LL << 30)) {
+    } else if (!dirY_ && !ordered_ && allBuffers && opt_.vec == 0 && (fastExtent % v) != 0 && fastExtent >= 2 * v && R_ < (1LL << 30)) {
       overlapRun_ = true;
       runLength_ = fastExtent;
       runChunks_ = ceilDivL(fastExtent, v);
@@ -445,7 +450,21 @@ class StreamReduceEmitter {
     unroll_ = opt_.chunks > 0 ? std::min(opt_.chunks, 16)
                               : std::max(1, (dirY_ ? 2 : (scatteredR ? 4 : 8)) / streamedInputs);
     if (opt_.block >= 64 && opt_.block <= 1024 && (opt_.block & (opt_.block - 1)) == 0) kBlock = opt_.block;
-    if (dirY_) {
+    if (ordered_ && dirY_) {
+      // one wavefront per strip of 64 * V columns, every thread the whole reduced extent of its columns, in order
+      kBlock = 64;
+      lanes_ = 64;
+      strips_ = ceilDivL(I_, static_cast<int64_t>(lanes_) * vec_);
+      groups_ = O_ * strips_;
+      rps_ = R_;
+      split_ = 1;
+    } else if (ordered_) {
+      lanes_ = kBlock;
+      strips_ = 1;
+      groups_ = O_;
+      rps_ = R_;
+      split_ = 1;
+    } else if (dirY_) {
       // A workgroup is TR thread-rows of LANES lanes; a lane owns V adjacent columns. Narrow strips (16 lanes = one
       // 256-byte run per row) give many groups, so few workgroups share a group and the partials stay small.
       int lanes = opt_.threadsPerRow > 0 ? opt_.threadsPerRow : 16;
@@ -778,7 +797,8 @@ class StreamReduceEmitter {
       }
     }
     // ---- streaming loop
-    line("#pragma unroll " + std::to_string(unroll_));
+    if (ordered_ && !dirY_) line("  __shared__ __attribute__((aligned(16))) unsigned short akg_chain[BLOCK * V];");
+    line("#pragma unroll " + std::to_string(ordered_ && !dirY_ ? 1 : unroll_));
     if (dirY_) {
       line("  for (long r = r_begin + tr; r < r_end; r += TR) {");
     } else if (overlapRun_) {
@@ -788,6 +808,10 @@ class StreamReduceEmitter {
       line("    const bool akg_tail = akg_start > RUN - V;");
       line("    if (akg_tail) akg_start = RUN - V;");
       line("    const long r = static_cast<long>(akg_run) * RUN + akg_start;");
+    } else if (ordered_) {
+      line("  for (long akg_tile = r_begin; akg_tile < r_end; akg_tile += static_cast<long>(BLOCK) * V) {");
+      line("    const bool akg_in = akg_tile + static_cast<long>(tid) * V < r_end;");
+      line("    const long r = akg_in ? akg_tile + static_cast<long>(tid) * V : r_begin;");
     } else {
       line("  for (long r = r_begin + static_cast<long>(tid) * V; r < r_end; r += static_cast<long>(BLOCK) * V) {");
     }
@@ -804,8 +828,19 @@ class StreamReduceEmitter {
         const std::string accName = "acc" + std::to_string(k) + (dirY_ ? "[e]" : "");
         std::string step = spec.combiner + "::apply(" + accName + ", " + val + ")";
         if (spec.roundEachStep) step = std::string(dtypeTag(od)) + "::rnd(" + step + ")";
+        if (spec.ordered && !dirY_) {
+          // the tile's elements in their 16-bit type into LDS; the first thread folds them in index order
+          const std::string tag = dtypeTag(od);
+          src_ << in4 << "if (akg_in) akg::chain_put<" << tag << ", V>(reinterpret_cast<" << tag << "::storage *>(akg_chain), tid * V, "
+               << ident_[static_cast<size_t>(op.inputs[0])] << ", 0);\n";
+          src_ << in4 << "__syncthreads();\n";
+          src_ << in4 << "if (tid == 0) acc" << k << " = akg::chain_fold<" << spec.combiner << ", " << tag << ">(acc" << k
+               << ", reinterpret_cast<const " << tag << "::storage *>(akg_chain), static_cast<int>(r_end - akg_tile < BLOCK * V ? r_end - akg_tile : BLOCK * V));\n";
+          src_ << in4 << "__syncthreads();\n";
+          continue;
+        }
         src_ << in4 << "#pragma unroll\n";
-        src_ << in4 << "for (int e = 0; e < V; ++e) " << (overlapRun_ ? "if (!akg_tail || e >= OVERLAP) " : "") << accName
+        src_ << in4 << "for (int e = 0; e < V; ++e) " << (overlapRun_ ? "if (!akg_tail || e >= OVERLAP) " : (ordered_ && !dirY_ ? "if (akg_in) " : "")) << accName
              << " = " << step << ";\n";
         continue;
       }
@@ -816,7 +851,7 @@ class StreamReduceEmitter {
       const int id = g_.outputs[i];
       if (phase_[static_cast<size_t>(id)] != Phase::Pre) continue;
       const std::string off = offsetExpr(g_.tensor(id), "akg_o", "r", dirY_ ? "akg_i" : "");
-      src_ << in4 << (dirY_ ? "if (col_ok) " : "") << "akg::store_chunk<" << tagOf(id) << ", V, "
+      src_ << in4 << (dirY_ ? "if (col_ok) " : (ordered_ ? "if (akg_in) " : "")) << "akg::store_chunk<" << tagOf(id) << ", V, "
            << (opt_.nonTemporal != 0 ? "true" : "false") << ">(" << memRef("out" + std::to_string(i), off) << ", "
            << ident_[static_cast<size_t>(id)] << ");\n";
     }
@@ -912,7 +947,11 @@ class StreamReduceEmitter {
            << " *>(akg_scratch[" << (scratchUse & 1) << "]), tid)" << (spec.roundEachStep ? ")" : "") << ";\n";
       ++scratchUse;
     };
-    for (size_t k = 0; k < reduces_.size(); ++k) blockReduce(k, "acc" + std::to_string(k));
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      // (an ordered reduction is complete in the first thread, which is the one that stores)
+      if (lowering::reduceSpec(*reduces_[k], g_.tensor(reduces_[k]->outputs[0]).dtype).ordered) continue;
+      blockReduce(k, "acc" + std::to_string(k));
+    }
     if (split_ > 1) {
       line("  // ---- partial of this workgroup -> workspace; the last workgroup of the group to arrive finishes the job");
       line("  unsigned char *akg_wsb = reinterpret_cast<unsigned char *>(akg_ws);");

@@ -112,6 +112,9 @@ class TileEmitter {
   int64_t grid_ = 1;
   bool raggedCols_ = false, raggedRows_ = false, raggedFlat_ = false;
   int reduceCount_ = 0;
+  // Some reduction is a float16 / bfloat16 sum or product: its steps run in index order, one thread per row folding
+  // the row's LDS image (akg::chain_fold), so rows get few threads each and a workgroup many rows.
+  bool ordered_ = false;
   // Rows too long to stay in registers: the row is walked in `groups_` groups of NCHUNK chunks per thread, once per
   // reduction of the fusion and once more for the outputs; every walk recomputes the element values it needs from
   // the kernel inputs (re-read from L2 / the last-level cache after the first walk).
@@ -148,7 +151,10 @@ class TileEmitter {
         throw LoweringError("op " + op.name + " has no gfx950 kernel family yet");
       }
       if (op.kind == OpKind::MatMul) throw LoweringError("internal: MatMul reached the tile emitter");
-      if (lowering::isReduceKind(op.kind)) rowMode_ = true;
+      if (lowering::isReduceKind(op.kind)) {
+        rowMode_ = true;
+        ordered_ = ordered_ || lowering::reduceSpec(op, g_.tensor(op.outputs[0]).dtype).ordered;
+      }
     }
     if (rowMode_) {
       analyseRowSpace();
@@ -353,6 +359,13 @@ class TileEmitter {
             tpr = t;
             best = slots;
           }
+        }
+      }
+      if (ordered_ && opt_.threadsPerRow == 0) {
+        // one thread folds a row while the row's other threads wait: as few threads per row as keep it in registers
+        for (int t = 1; t <= 1024; t <<= 1) {
+          tpr = t;
+          if (ceilDiv(rowChunks, t) <= 8) break;
         }
       }
       tpr_ = tpr;
@@ -625,6 +638,12 @@ class TileEmitter {
       }
       if (tpr_ > 64) {
         line("  __shared__ double akg_scratch[2][BLOCK / 64];");
+      }
+      if (ordered_) {
+        // the part of every row of the workgroup that is being folded, in its 16-bit type (rows 16 bytes apart in the banks)
+        line("  constexpr int CHAIN_PITCH = NCHUNK * TPR * V + 8;");
+        line("  __shared__ __attribute__((aligned(16))) unsigned short akg_chain[RPB][CHAIN_PITCH];");
+        line("  __shared__ float akg_chain_res[RPB];");
       }
       line("  long akg_rows[NCHUNK];");
       line("#pragma unroll");
@@ -1097,6 +1116,31 @@ class TileEmitter {
     const std::string tag = dtypeTag(od);
     const lowering::ReduceSpec spec = lowering::reduceSpec(op, od);
     const std::string acc = "acc" + std::to_string(outId);
+    if (spec.ordered) {
+      // this group of the row into LDS, then the row's first thread folds it onto its accumulator in index order
+      const std::string base = multiPass_ ? "static_cast<long>(akg_g) * (NCHUNK * TPR * V)" : "0L";
+      src_ << "  {\n";
+      src_ << "    " << tag << "::storage *akg_run = reinterpret_cast<" << tag << "::storage *>(akg_chain[tid / TPR]);\n";
+      src_ << "    const long akg_base = " << base << ";\n";
+      line("#pragma unroll");
+      line("    for (int j = 0; j < NCHUNK; ++j) {");
+      std::string from = "0";
+      if (colsArg_) {
+        from = "akg_tail[j] ? akg_overlap : 0";
+      } else if (overlap_ > 0) {
+        from = "akg_tail[j] ? " + std::to_string(overlap_) + " : 0";
+      }
+      src_ << "      " << (raggedCols_ || colsArg_ || overlap_ > 0 ? "if (akg_ok[j]) " : "") << "akg::chain_put<" << tag
+           << ", V>(akg_run, static_cast<int>(akg_cols[j] - akg_base), " << in.ident << "[j], " << from << ");\n";
+      line("    }");
+      line("    __syncthreads();");
+      line("    const long akg_left = COLS - akg_base;");
+      src_ << "    if (tcol == 0) " << acc << " = akg::chain_fold<" << spec.combiner << ", " << tag << ">(" << acc
+           << ", akg_run, static_cast<int>(akg_left < NCHUNK * TPR * V ? akg_left : NCHUNK * TPR * V));\n";
+      line("    __syncthreads();");
+      src_ << "  }\n";
+      return;
+    }
     line("#pragma unroll");
     line("  for (int j = 0; j < NCHUNK; ++j) {");
     line("#pragma unroll");
@@ -1128,6 +1172,17 @@ class TileEmitter {
     ValInfo &v = vals_[static_cast<size_t>(outId)];
     std::ostringstream nm;
     nm << "u" << outId;
+    if (spec.ordered) {
+      src_ << "  if (tcol == 0) akg_chain_res[tid / TPR] = " << acc << ";\n";
+      line("  __syncthreads();");
+      src_ << "  const " << ct << " " << nm.str() << " = akg_chain_res[tid / TPR];\n";
+      v.defined = true;
+      v.rank = ValRank::Uniform;
+      v.ident = nm.str();
+      const TensorValue &outT = g_.tensor(outId);
+      v.rowvecNoKeep = outT.numel() != 1 && !outT.shape.empty() && outT.shape.back() != 1;
+      return;
+    }
     std::string scratch = tpr_ > 64 ? "reinterpret_cast<" + ct + " *>(akg_scratch[" + std::to_string(reduceCount_ & 1) + "])"
                                     : "static_cast<" + ct + " *>(nullptr)";
     src_ << "  const " << ct << " " << nm.str() << " = " << (roundEachStep ? tag + "::rnd(" : "")

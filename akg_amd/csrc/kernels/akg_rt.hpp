@@ -880,6 +880,90 @@ AKG_DEV void column_reduce(typename DT::compute (&acc)[V], typename DT::compute 
 }
 
 // ---------------------------------------------------------------------------------------------------------
+// Ordered reductions. A sum or a product whose declared result is float16 / bfloat16 is rounded to that type after
+// every step, so the order of the steps is part of the result: the reference runs ONE serial loop per result
+// element, in index order (linalg.reduce lowered to loops, MindSporeToLinalg.cpp:845-901,1333-1451). 4096 float16
+// ones sum to 2048 that way, and to 4096 in a tree. The kernels keep that order: the elements of a run go through
+// LDS in their declared 16-bit type (what they hold is already rounded to it), and one thread per run folds them one
+// after the other; many runs fold side by side on the lanes of a wavefront.
+// ---------------------------------------------------------------------------------------------------------
+// Elements e >= from of a thread's chunk to positions at + e of a run's LDS image.
+template <typename DT, int V>
+AKG_DEV void chain_put(typename DT::storage *run, int at, const typename DT::compute (&v)[V], int from) {
+  static_assert(sizeof(typename DT::storage) == 2, "ordered reductions are those of the 16-bit float types");
+  if constexpr (V * 2 >= 4 && V * 2 <= 16) {
+    if (from == 0 && (at % V) == 0) {
+      typename DT::storage tmp[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) tmp[e] = DT::store(v[e]);
+      typedef typename Raw<V * 2>::type R;
+      R raw;
+      __builtin_memcpy(&raw, tmp, sizeof(tmp));
+      *reinterpret_cast<R *>(run + at) = raw;
+      return;
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    if (e >= from) run[at + e] = DT::store(v[e]);
+  }
+}
+
+// acc folded with run[0 .. n) in index order, rounded to the declared type after every step.
+// `run` is 16-byte aligned.
+template <typename Red, typename DT>
+AKG_DEV typename DT::compute chain_fold(typename DT::compute acc, const typename DT::storage *run, int n) {
+  int i = 0;
+  for (; i + 8 <= n; i += 8) {
+    typename DT::storage tmp[8];
+    const typename Raw<16>::type raw = *reinterpret_cast<const typename Raw<16>::type *>(run + i);
+    __builtin_memcpy(tmp, &raw, sizeof(tmp));
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc = DT::rnd(Red::apply(acc, DT::load(tmp[e])));
+  }
+  for (; i < n; ++i) acc = DT::rnd(Red::apply(acc, DT::load(run[i])));
+  return acc;
+}
+
+// Column kernels: thread (ly, lx) of LY x LX holds V values of row `first + ly` of the run, columns lx * V + e. The
+// rows of one step are neighbours in the run, so a step puts them into LDS ([LY][LX * V]) and the thread that owns
+// column c = tid, tid + BLOCK, ... folds rows 0 .. nrows - 1 of it onto its accumulator, in order.
+template <typename Red, typename DT, int LX, int BLOCK, int V, int NOWN>
+AKG_DEV void column_chain_step(typename DT::compute (&own)[NOWN], const typename DT::compute (&v)[V],
+                               typename DT::storage *lds, int tid, int nrows) {
+  constexpr int kCols = LX * V;
+  const int lx = tid % LX, ly = tid / LX;
+  chain_put<DT, V>(lds + ly * kCols, lx * V, v, 0);
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < NOWN; ++k) {
+    const int c = tid + k * BLOCK;
+    if (c < kCols) {
+      typename DT::compute a = own[k];
+      for (int r = 0; r < nrows; ++r) a = DT::rnd(Red::apply(a, DT::load(lds[r * kCols + c])));
+      own[k] = a;
+    }
+  }
+  __syncthreads();
+}
+
+// The owners' results to every thread of the column (`res`: LX * V values of the compute type).
+template <typename DT, int LX, int BLOCK, int V, int NOWN>
+AKG_DEV void column_chain_finish(const typename DT::compute (&own)[NOWN], typename DT::compute (&acc)[V],
+                                 typename DT::compute *res, int tid) {
+  constexpr int kCols = LX * V;
+#pragma unroll
+  for (int k = 0; k < NOWN; ++k) {
+    const int c = tid + k * BLOCK;
+    if (c < kCols) res[c] = own[k];
+  }
+  __syncthreads();
+  const int lx = tid % LX;
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = res[lx * V + e];
+}
+
+// ---------------------------------------------------------------------------------------------------------
 // Workspace protocol of the streaming reductions. Several workgroups share one group of outputs; each leaves
 // its partial result in device memory and counts its arrival; the workgroup that arrives last reads all the
 // partials back (in slot order, so the result does not depend on the arrival order) and finishes the job.

@@ -162,6 +162,24 @@ def compare(actual, expected, dtype):
     return True, "max abs err %.3g, max rel err %.3g" % (float(np.nanmax(err)) if a.size else 0.0, float(rel))
 
 
+def compare_bits(actual, expected, dtype):
+    """Returns (ok, message): the two tensors must hold the same bit patterns, whatever the element type (the bar for
+    results the workload states as bit-exact, e.g. the float32 scales of the per-token quantisation)."""
+    a, e = np.ascontiguousarray(actual), np.ascontiguousarray(expected)
+    if a.shape != e.shape:
+        return False, "shape %s != %s" % (a.shape, e.shape)
+    if a.dtype.itemsize != e.dtype.itemsize:
+        return False, "element size %d != %d" % (a.dtype.itemsize, e.dtype.itemsize)
+    raw = np.dtype("u%d" % a.dtype.itemsize)
+    ab, eb = a.view(raw), e.view(raw)
+    bad = int(np.count_nonzero(ab != eb))
+    if bad:
+        idx = tuple(np.argwhere(ab != eb)[0])
+        return False, "%d of %d %s elements differ in their bits; first at %s: %r vs %r" % (
+            bad, ab.size, dtype, idx, a[idx], e[idx])
+    return True, "bit-exact"
+
+
 def widen_to_float64(desc):
     """The same description with every float32 tensor, cast target and constant declared float64: evaluated by the
     oracle it gives the fused expression with (nearly) exact accumulation, whatever the order of a summation."""

@@ -168,6 +168,12 @@ def random_description(seed, allow_views=True, allow_reduce=True):
             axis = sorted(int(a) for a in rng.choice(r, size=int(rng.integers(2, r + 1)), replace=False))
         name = str(rng.choice(["ReduceSum", "ReduceMax", "ReduceMin"]))
         notes.append("%s%s" % (name, axis))
+        # A sum declared in the 16-bit type of the description: rounded after every step, so its steps must come in the
+        # reference's serial order. Only of exactly computed values (an ulp of difference in one term would round the
+        # chain differently); drawn from a generator of its own so that the other descriptions stay what they were.
+        if name == "ReduceSum" and dtype != "float32" and out.exact and np.random.default_rng(seed + 7_000_000).random() < 0.6:
+            out = Val(b.cast(out.t, dtype), True, out.positive, out.bounded)
+            notes.append("declared-" + dtype)
         if rng.random() < 0.4 and (axis == [len(out.t.shape) - 1] or name != "ReduceSum"):
             # use the reduced value again on the elements it came from (softmax-like): the row kernel serves the last
             # axis, other axes need a kernel per pass (max / min only there: they do not depend on the order)

@@ -742,11 +742,17 @@ def test_column_kernel_schedule():
     # rows that are not a multiple of the chunk: element-aligned accesses, the last chunk partly outside
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_staged_layernorm_axis1_bf16_8x64x49.info"), out_dir=None)
     assert "load_packed_partial<akg::bf16, V>(akg_p, akg_row_ok[j] ? akg_cols : 0" in k.source and "store_chunk_partial" in k.source
-    # a 16-bit sum keeps its rounding per step, a maximum needs none
+    # a 16-bit sum keeps its rounding per step and the serial order of the steps (one chain per column through LDS), a
+    # maximum needs neither; a 16-bit integer sum wraps around and is the same in any order
     b = op_desc.DescBuilder("column_half")
     x = b.input([2, 40, 24], "float16")
     k = driver.HipKernel(b.dumps([b.sub(x, b.reduce("ReduceMax", x, [1], True)), b.reduce("ReduceSum", x, [1], True)]), out_dir=None)
-    assert "column_reduce<akg::RedSum, akg::f16, true," in k.source and "column_reduce<akg::RedMax, akg::f16, false," in k.source
+    assert "column_chain_step<akg::RedSum, akg::f16, LX, BLOCK, V, NOWN>" in k.source and "column_chain_finish<akg::f16," in k.source
+    assert "column_reduce<akg::RedMax, akg::f16, false," in k.source and "column_reduce<akg::RedSum" not in k.source
+    b = op_desc.DescBuilder("column_short")
+    x = b.input([2, 40, 24], "int16")
+    k = driver.HipKernel(b.dumps([b.sub(x, b.reduce("ReduceSum", x, [1], True))]), out_dir=None)
+    assert "column_reduce<akg::RedSum, akg::i16, true," in k.source and "column_chain" not in k.source
     # two reduced axes around a kept one (batch-norm statistics and their use) are not for this kernel
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_staged_bn_train_forward_f32_16x8x14x14.info"), out_dir=None)
     assert k.family == "staged"
