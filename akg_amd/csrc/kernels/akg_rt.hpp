@@ -417,7 +417,8 @@ AKG_DEV double op_exp(double a) { return exp(a); }
 AKG_DEV float op_log(float a) { return logf(a); }
 AKG_DEV double op_log(double a) { return log(a); }
 // float32 tanh, maximum relative error about 1e-6 (the bar for float32 results is 1e-5 against libm):
-//   |a| <  0.25 : a + a^3 * Q(a^2), the odd Taylor series through a^9 (truncation below 1e-8 relative)
+//   |a| <  0.25 : a * (1 + a^2 * Q(a^2)), the odd Taylor series through a^9 (truncation below 1e-8 relative); the
+//                 product form keeps the sign of a zero argument, as libm's tanhf does
 //   |a| >= 0.25 : 1 - 2 / (exp(2|a|) + 1) with the hardware exp2 and reciprocal (1 ulp each); the subtraction
 //                 loses at most log2(1 / tanh(0.25)) = 2 bits there
 // A third of the instructions of the device library's tanhf, which a 64 MiB elementwise kernel cannot hide.
@@ -427,7 +428,7 @@ AKG_DEV float op_tanh(float a) {
   float q = __builtin_fmaf(0x1.664f48p-6f, z, -0x1.ba1ba2p-5f);  // 62/2835, -17/315
   q = __builtin_fmaf(q, z, 0x1.111112p-3f);                       // 2/15
   q = __builtin_fmaf(q, z, -0x1.555556p-2f);                      // -1/3
-  const float small = __builtin_fmaf(a * z, q, a);
+  const float small = a * __builtin_fmaf(z, q, 1.0f);
   const float t = __builtin_amdgcn_exp2f(ax * 0x1.715476p+1f);    // exp(2|a|); +inf beyond |a| = 44.4
   const float big = __builtin_fmaf(-2.0f, __builtin_amdgcn_rcpf(t + 1.0f), 1.0f);
   return (ax < 0.25f) ? small : __builtin_copysignf(big, a);      // NaN takes the second branch and stays NaN

@@ -117,11 +117,21 @@ def cast(x, src, dst):
 
 
 def maximum_nan(a, b):
-    return np.maximum(a, b)   # numpy's maximum propagates NaN, like arith.maximumf
+    """arith.maximumf: NaN propagates (numpy's maximum does that too) and -0 is less than +0 (numpy returns either)."""
+    r = np.maximum(a, b)
+    if np.asarray(r).dtype.kind != "f":
+        return r
+    zeros = (np.asarray(a) == 0) & (np.asarray(b) == 0)
+    return np.where(zeros, np.where(np.signbit(a) & np.signbit(b), -0.0, 0.0).astype(r.dtype), r)
 
 
 def minimum_nan(a, b):
-    return np.minimum(a, b)
+    """arith.minimumf: NaN propagates, -0 is less than +0."""
+    r = np.minimum(a, b)
+    if np.asarray(r).dtype.kind != "f":
+        return r
+    zeros = (np.asarray(a) == 0) & (np.asarray(b) == 0)
+    return np.where(zeros, np.where(np.signbit(a) | np.signbit(b), -0.0, 0.0).astype(r.dtype), r)
 
 
 def serial_reduce(x, axes, combine, init, dtype, keep_dims):

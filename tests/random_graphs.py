@@ -244,6 +244,45 @@ def random_matmul_description(seed):
     return b.dumps([b.cast(t, dtype) for t in outs]), notes
 
 
+def random_int8_matmul_description(seed):
+    """An int8 x int8 -> int32 MatMul (the quantised contraction): the bare int32 accumulators as an output (held to their
+    bits), and / or a dequantising epilogue (per-row and per-column float32 scales, bias, activation) cast to a float
+    type. Shapes cover whole and ragged MFMA tiles, skinny A, K that is not a whole number of 16-byte pieces (the
+    serial kernel) and both layouts of B. Returns (json_text, notes)."""
+    rng = np.random.default_rng(300000 + seed)
+    m = int(rng.choice([1, 7, 40, 64, 130, 300]))
+    k = int(rng.choice([32, 64, 256, 100, 1040]))
+    n = int(rng.choice([8, 36, 136, 256, 520]))
+    tb = bool(rng.integers(0, 2))
+    b = op_desc.DescBuilder("Fused_random_int8_matmul_%d" % seed)
+    notes = ["%dx%dx%d" % (m, k, n), "tb" if tb else "nt"]
+    a = b.input([m, k], "int8")
+    w = b.input([n, k] if tb else [k, n], "int8")
+    acc = b.matmul(a, w, "int32", transpose_b=tb)
+    outs = []
+    shape = str(rng.choice(["bare", "dequant", "both"]))
+    notes.append(shape)
+    if shape in ("bare", "both"):
+        outs.append(acc)
+    if shape in ("dequant", "both"):
+        y = b.cast(acc, "float32")
+        y = b.mul(y, b.input([m, 1], "float32"))
+        y = b.mul(y, b.input([n], "float32"))
+        if rng.random() < 0.6:
+            y = b.add(y, b.cast(b.input([n], "bfloat16"), "float32"))
+            notes.append("bias")
+        act = str(rng.choice(["none", "relu", "tanh"]))
+        if act == "relu":
+            y = b.maximum(y, b.const(0.0, "float32"))
+        elif act == "tanh":
+            y = b.unary("Tanh", y)
+        notes.append(act)
+        out_dtype = str(rng.choice(["bfloat16", "float16", "float32"]))
+        notes.append(out_dtype)
+        outs.append(b.cast(y, out_dtype) if out_dtype != "float32" else y)
+    return b.dumps(outs), notes
+
+
 def random_optable_description(seed):
     """The rows of the op table that `random_description` does not draw: Log, Sin, Cos, ASin, ACos, Atan, Asinh, Acosh,
     Floor, IsNan / IsInf / IsFinite, LogicalNot / And / Or, Pow, Atan2, AddN, GreaterEqual, Less, integer Div, a

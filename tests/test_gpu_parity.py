@@ -1423,6 +1423,44 @@ def test_profile_entry_point_returns_a_plausible_time():
     assert 0.0 < ms < 50.0
 
 
+@pytest.mark.parametrize("m,k,n,tb", [(512, 8192, 512, False), (4096, 8192, 8192, False), (4096, 8192, 8192, True),
+                                      (1000, 4112, 1032, False), (48, 8192, 4096, False)])
+def test_bare_int8_matmul_accumulators_are_exact(m, k, n, tb):
+    """MatMul int8 x int8 -> int32 with the accumulators themselves as the output (no epilogue to hide a dropped or doubled
+    product behind a 16-bit tolerance), at the shape of the measured fusion and on ragged, split-K and skinny ones:
+    every element equal to torch._int_mm's exact integer product, and sampled rows (spread over every row tile) equal
+    to the oracle's exact accumulation."""
+    import torch
+    from oracle import np_ref
+    b = op_desc.DescBuilder("bare_mm_i8_%dx%dx%d%s" % (m, k, n, "_tb" if tb else ""))
+    a_t = b.input([m, k], "int8")
+    w_t = b.input([n, k] if tb else [k, n], "int8")
+    text = b.dumps([b.matmul(a_t, w_t, "int32", transpose_b=tb)])
+    kernel = driver.HipKernel(text, out_dir=None)
+    print("case %s: %s grid %d block %d" % (kernel.kernel_name, kernel.family, kernel.grid[0], kernel.block[0]), flush=True)
+    assert kernel.family == "gemm_epilogue" and "mfma" in kernel.source
+    rng = np.random.default_rng(harness.BASE_SEED + 55)
+    a = rng.integers(-127, 128, size=(m, k), dtype=np.int8)
+    w = rng.integers(-127, 128, size=(n, k) if tb else (k, n), dtype=np.int8)
+    got = run_on_gpu(kernel, [a, w])[0]
+    assert got.dtype == np.int32 and got.shape == (m, n)
+    wk = np.ascontiguousarray(w.T) if tb else w
+    rows = np.unique(np.concatenate([np.arange(0, m, max(1, m // 16)), rng.integers(0, m, 16), [m - 1]]))
+    expect_rows = np_ref.matmul_exact_i32(a[rows], wk)
+    bad = int(np.count_nonzero(got[rows] != expect_rows))
+    print("  %d sampled rows vs exact accumulation: %d elements differ" % (len(rows), bad), flush=True)
+    assert bad == 0
+    dev = torch.device("cuda:0")
+    # torch._int_mm wants at least 17 rows and extents that are multiples of 8: pad A with zero rows, compare the real ones
+    pad_m = max(32, (m + 7) // 8 * 8)
+    a_pad = np.zeros((pad_m, k), dtype=np.int8)
+    a_pad[:m] = a
+    ref = torch._int_mm(torch.from_numpy(a_pad).to(dev), torch.from_numpy(wk).to(dev))[:m].cpu().numpy()
+    bad = int(np.count_nonzero(got != ref))
+    print("  all %d accumulators vs torch._int_mm: %d differ" % (got.size, bad), flush=True)
+    assert bad == 0
+
+
 def test_c5_full_size_gemm_fusion():
     """Full configuration: 4096 x 8192 x 8192. The CPU oracle cannot run 2.7e11 MACs in a test, so:
     (1) 96 sampled rows (all 8192 columns each, rows spread over every 256-row tile) against the oracle evaluated on

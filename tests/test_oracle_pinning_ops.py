@@ -349,3 +349,21 @@ def test_sixteen_bit_matmul_rounds_product_and_sum_every_step(dtype, transpose_b
     for out in run_both(matmul_desc(m, k, n, dtype, transpose_b), [a, w_in], tmp_path):
         got = out[0].astype(np.float64) if dtype == "float16" else np_ref.bf16_bits_to_f32(out[0]).astype(np.float64)
         assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------------------------------------------------
+# the shared known-answer table (tests/known_answers.py): both restatements against it; the GPU suite pushes the same
+# vectors through the HIP kernels
+# ---------------------------------------------------------------------------------------------------------
+import known_answers  # noqa: E402
+
+_KAT = {c["name"]: c for c in known_answers.cases()}
+
+
+@pytest.mark.parametrize("name", sorted(_KAT))
+def test_known_answer_table_holds_for_both_restatements(name, tmp_path):
+    case = _KAT[name]
+    c_out, n_out = run_both(case["text"], case["inputs"], tmp_path)
+    for which, outs in (("C restatement", c_out), ("numpy restatement", n_out)):
+        ok, msg = known_answers.check(case, outs)
+        assert ok, "%s, %s: %s" % (name, which, msg)

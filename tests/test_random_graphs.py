@@ -11,7 +11,7 @@ import pytest
 
 from akg_amd import driver, harness
 from oracle import cpu_ref, np_ref
-from random_graphs import random_description, random_matmul_description, random_optable_description
+from random_graphs import random_description, random_int8_matmul_description, random_matmul_description, random_optable_description
 
 # AKG_RANDOM_GRAPHS=N widens the sweep for a one-off soak on the CPU oracle / a GPU box
 SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_GRAPHS", "40"))))
@@ -119,6 +119,49 @@ def test_random_matmul_description_compiles(seed):
 def test_random_matmul_description_matches_oracle_on_gpu(seed, tmp_path):
     from test_gpu_parity import run_on_gpu
     text, notes = random_matmul_description(seed)
+    desc, path = _write(tmp_path, text)
+    print("seed %d: %s" % (seed, " ".join(notes)), flush=True)
+    kernel = driver.HipKernel(text, out_dir=None)
+    inputs = harness.make_inputs(desc, seed=seed)
+    got = run_on_gpu(kernel, inputs)
+    expect = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    for d, g, e in zip(kernel.outputs, got, expect):
+        ok, msg = harness.compare(g, e, d.dtype)
+        print("  %s %s %s: %s" % (kernel.family, d.name, d.dtype, msg), flush=True)
+        assert ok, "seed %d (%s) output %s: %s" % (seed, " ".join(notes), d.name, msg)
+
+
+INT8_MATMUL_SEEDS = list(range(1, 1 + int(os.environ.get("AKG_RANDOM_INT8_MATMULS", "30"))))
+
+
+@pytest.mark.parametrize("seed", INT8_MATMUL_SEEDS[:12])
+def test_random_int8_matmul_description_compiles_and_oracles_agree(seed, tmp_path):
+    text, notes = random_int8_matmul_description(seed)
+    desc, path = _write(tmp_path, text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family in ("gemm_epilogue", "staged"), notes
+    inputs = harness.make_inputs(desc, seed=seed)
+    c_out = cpu_ref.CpuKernel(path, rebuild=True)(inputs)
+    n_out = np_ref.evaluate(desc, inputs)
+    for d, a, b in zip(desc["output_desc"], c_out, n_out):
+        ok, msg = harness.compare(a, b, d["data_type"])
+        assert ok, "seed %d (%s) output %s: the two oracles disagree: %s" % (seed, " ".join(notes), d["tensor_name"], msg)
+    if notes[2] in ("bare", "both"):
+        # the accumulators against Python integers on a few elements: exact, whatever the machine arithmetic
+        a, w = inputs[0].astype(object), inputs[1].astype(object)
+        if notes[1] == "tb":
+            w = w.T
+        for (i, j) in [(0, 0), (a.shape[0] - 1, w.shape[1] - 1), (a.shape[0] // 2, w.shape[1] // 3)]:
+            assert int(c_out[0][i, j]) == int(sum(a[i, :] * w[:, j]))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", INT8_MATMUL_SEEDS)
+def test_random_int8_matmul_description_matches_oracle_on_gpu(seed, tmp_path):
+    """int32 accumulators bit for bit (harness.compare holds integer outputs to equality), the dequantised results to the
+    bar of their type."""
+    from test_gpu_parity import run_on_gpu
+    text, notes = random_int8_matmul_description(seed)
     desc, path = _write(tmp_path, text)
     print("seed %d: %s" % (seed, " ".join(notes)), flush=True)
     kernel = driver.HipKernel(text, out_dir=None)
