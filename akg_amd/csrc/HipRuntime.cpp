@@ -941,10 +941,24 @@ int akg_hip_launch_static_scratch(akg_hip_kernel_t *kernel, void *const *device_
   return launchOn(kernel, fn, device_ptrs, static_cast<hipStream_t>(stream), base);
 }
 
+static_assert(AKG_HIP_STATIC_SCRATCH_MAX == AKG_HIP_STATIC_SCRATCH_BYTES,
+              "the limit the header states and the size of the array are one number");
+
 int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel) {
   if (kernel == nullptr) return fail(AKG_HIP_ERR_INVALID_ARGUMENT, "kernel is NULL");
   akg_hip_kernel::Loaded *l = nullptr;
-  return ensureLoaded(kernel, &l);
+  const int rc = ensureLoaded(kernel, &l);
+  if (rc != AKG_HIP_OK) return rc;
+  // A handle that akg_hip_launch_static_scratch can serve: look the array's address up now. The first look-up on a
+  // device makes the runtime load the library's own code object there and materialise the array, which a launch that
+  // must not allocate (or that is being captured into a graph) cannot afford; afterwards it is a table read.
+  const uint64_t need = scratchBytesNeeded(kernel);
+  if (need > 0 && need <= AKG_HIP_STATIC_SCRATCH_BYTES) {
+    void *p = nullptr;
+    const hipError_t e = akg::staticScratchOnCurrentDevice(&p);
+    if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "address of the static scratch array: " + hipErr(e));
+  }
+  return AKG_HIP_OK;
 }
 
 int akg_hip_run_host(akg_hip_kernel_t *kernel, void *const *host_ptrs, int n_ptrs) {

@@ -235,6 +235,30 @@ def layernorm_residual(rows, cols, dtype="bfloat16", eps=1e-5, name=None):
     return b.dumps([out])
 
 
+def rmsnorm(rows, cols, dtype="bfloat16", eps=1e-6, residual=False, name=None):
+    """out = x * rsqrt(mean(x * x) + eps) * gamma over the last axis, float32 internals. With `residual` the normalised
+    tensor is h = x + r (rounded to the storage type, as the next layer reads it) and h is the first output."""
+    tag = {"float16": "f16", "bfloat16": "bf16", "float32": "f32"}[dtype]
+    b = DescBuilder(name or "Fused_%sRMSNorm_%s_%dx%d" % ("Add_" if residual else "", tag, rows, cols))
+    x = b.input([rows, cols], dtype)
+    gamma = b.input([cols], dtype)
+    f = (lambda t: b.cast(t, "float32")) if dtype != "float32" else (lambda t: t)
+    outs = []
+    if residual:
+        r = b.input([rows, cols], dtype)
+        h = b.add(f(x), f(r))
+        h = b.cast(h, dtype) if dtype != "float32" else h
+        outs.append(h)
+        xf = f(h)
+    else:
+        xf = f(x)
+    ms = b.mul(b.reduce("ReduceSum", b.mul(xf, xf), [1], True), b.const(1.0 / cols, "float32"))
+    rstd = b.unary("Rsqrt", b.add(ms, b.const(eps, "float32")))
+    y = b.mul(b.mul(xf, rstd), f(gamma))
+    outs.append(b.cast(y, dtype) if dtype != "float32" else y)
+    return b.dumps(outs)
+
+
 def quant_int8_residual(rows, cols, dtype="bfloat16", name=None):
     """Per-token symmetric int8 quantisation of s = x + r: scale = absmax(s) / 127 per row,
     q = cast_int8(clamp(s / scale, -127, 127)) with the cast rounding half to even. Outputs: q, scale."""

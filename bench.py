@@ -6,7 +6,8 @@ are already resident in HBM. The headline workload is the fused softmax fp16 [81
 is reported under `per_config`. Inputs are synthetic (seeded); several distinct buffer sets are rotated so that a launch
 reads from HBM and not from the 256 MB last-level cache.
 
-Prints ONE JSON line:
+Prints ONE JSON line on stdout (kept short, so that a stored tail holds all of it); the long per-workload and
+calibration records go to stderr as one line that starts with "detail: ":
   value / ms_per_step  host-clock throughput of K back-to-back steps (algorithmic bytes / wall time)
   roofline             achieved = algorithmic bytes (or ops) per launch / mean launch duration from HIP events recorded
                        on the launch stream around the same K launches; peak = 8 TB/s HBM3E (or the dense MFMA peak);
@@ -14,10 +15,15 @@ Prints ONE JSON line:
                        summary is missing)
   cpu_baseline         the CPU oracle (C restatement of the reference CPU pipeline, 1 thread like the reference's
                        default, and its OpenMP build on all host cores) timed on this host on a bounded sample
-  per_config           the same roofline object per workload, with kernel_ms (mean of the K launches), kernel_ms_median
+  roofline.by_config   {short name: {bound, frac, kernel_ms}} for every measured workload (c1 .. c5 are the five of
+                       BASELINE.json), from the same run
+  cpu_by_config        the CPU baseline of the other BASELINE configurations, in short
+  calibration          {name: fraction of the peak} of what the box itself allows (below), and socket power / shader clock
+                       sampled while C5 and the register-only MFMA loop run (outside any timed region)
+  per_config (detail)  the same roofline object per workload, with kernel_ms (mean of the K launches), kernel_ms_median
                        and kernel_ms_min (over groups of 10 launches), a cache-resident figure for the two configurations
                        that fit the last-level cache, and a cpu_baseline for each of the five measured configurations
-  calibration          what the box itself allows, measured in the same run: streaming kernels of exactly the sizes of
+  calibration (detail) what the box itself allows, measured in the same run: streaming kernels of exactly the sizes of
                        C1 and C2 (this backend's own minimal kernels and the vendor's device-to-device copy), register-only
                        MFMA loops on zero and on random operands (the part is power limited), and the vendor library's
                        GEMM on the shapes of C5 and N2
@@ -36,7 +42,7 @@ sys.path.insert(0, ROOT)
 
 FIXTURES = os.path.join(ROOT, "akg_amd", "fixtures")
 PROFILES = os.path.join(ROOT, "profiles")
-PROBE_LIB = os.path.join(ROOT, "akg_amd", "libakg_bench_probe.so")
+PROBE_LIB = os.path.join(ROOT, "bench_probe", "libakg_bench_probe.so")
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published (no sparsity)
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published (no sparsity)
@@ -65,6 +71,9 @@ WORKLOADS = {
     # reduction level (three reads)
     "n8_softmax_axis1_f16_32x21x512x512": "f32",
     "n9_layernorm_axis1_bf16_64x768x1024": "f32",
+    # RMSNorm over the last axis (row family), alone and with the residual add in front (two outputs)
+    "n10_rmsnorm_bf16_16384x4096": "f32",
+    "n11_rmsnorm_add_bf16_16384x4096": "f32",
 }
 # workloads also measured on the schedule of several kernels (AKG_HIP_VARIANT=7 while the handle is built)
 SEVERAL_KERNELS = ("n8_softmax_axis1_f16_32x21x512x512", "n9_layernorm_axis1_bf16_64x768x1024")
@@ -222,6 +231,65 @@ def cpu_baseline(name, harness, driver):
     return out
 
 
+class PowerSampler:
+    """Socket power (W) and shader clock (MHz) of GPU 0 read through amdsmi while a callable keeps the device busy; never
+    inside a timed region. Every field is None where the library or the permission to read is missing."""
+
+    def __init__(self):
+        self.smi = None
+        self.handle = None
+        try:
+            import amdsmi
+            amdsmi.amdsmi_init()
+            self.smi = amdsmi
+            self.handle = amdsmi.amdsmi_get_processor_handles()[0]
+        except Exception:  # no library, no device node, no permission
+            self.smi = None
+
+    def read(self):
+        if self.smi is None:
+            return None, None
+        power = clock = None
+        try:
+            info = self.smi.amdsmi_get_power_info(self.handle)
+            for key in ("current_socket_power", "average_socket_power", "socket_power"):
+                v = info.get(key)
+                if isinstance(v, (int, float)) and v > 0:
+                    power = float(v)
+                    break
+        except Exception:
+            pass
+        try:
+            info = self.smi.amdsmi_get_clock_info(self.handle, self.smi.AmdSmiClkType.GFX)
+            v = info.get("clk", info.get("cur_clk"))
+            if isinstance(v, (int, float)) and v > 0:
+                clock = float(v)
+        except Exception:
+            pass
+        return power, clock
+
+    def during(self, launch, torch, busy_ms=400.0):
+        """Keeps the device busy with `launch(i)` for busy_ms and samples between batches of launches."""
+        if self.smi is None:
+            return {"socket_power_w": None, "shader_clock_mhz": None, "samples": 0}
+        powers, clocks = [], []
+        t0 = time.perf_counter()
+        i = 0
+        while (time.perf_counter() - t0) * 1e3 < busy_ms:
+            for _ in range(8):
+                launch(i)
+                i += 1
+            if (time.perf_counter() - t0) * 1e3 > busy_ms / 4:   # past the clock ramp
+                p, c = self.read()
+                if p is not None:
+                    powers.append(p)
+                if c is not None:
+                    clocks.append(c)
+            torch.cuda.synchronize()
+        return {"socket_power_w": round(statistics.median(powers), 1) if powers else None,
+                "shader_clock_mhz": round(statistics.median(clocks), 0) if clocks else None, "samples": max(len(powers), len(clocks))}
+
+
 def vendor_gemm(kind, torch, steps):
     """The vendor library's GEMM on the shape and layout of C5 (int8) / N2 (bf16): no epilogue, same buffers reused."""
     dev = torch.device("cuda:0")
@@ -242,9 +310,10 @@ def vendor_gemm(kind, torch, steps):
             "achieved": round(rate, 1), "unit": unit, "frac": round(rate / peak, 4), "what": what}
 
 
-def calibration(torch, driver, harness, np, steps, warmup):
+def calibration(torch, driver, harness, np, steps, warmup, sampler=None, power=None):
     """Ceilings of this box, measured in this run."""
     out = {}
+    power = {} if power is None else power
     dev = torch.device("cuda:0")
     # 1. streaming kernels of exactly C1's and C2's sizes: this backend's own minimal kernels ...
     for calib, twin in SIZE_MATCHED.items():
@@ -293,6 +362,8 @@ def calibration(torch, driver, harness, np, steps, warmup):
                     _, mean_ms, med_ms, min_ms = timed(lambda i: fn(st, buf.data_ptr(), iterations, workgroups, sink.data_ptr()),
                                                        max(10, steps // 10), 2, torch)
                     rate = ops / (mean_ms * 1e-3) / 1e12
+                    if sampler is not None and kind == "i8" and suffix == "":
+                        power[label] = sampler.during(lambda i: fn(st, buf.data_ptr(), iterations, workgroups, sink.data_ptr()), torch)
                     out[label] = {"ops": ops, "kernel_ms": round(mean_ms, 4), "kernel_ms_median": round(med_ms, 4),
                                   "kernel_ms_min": round(min_ms, 4), "achieved": round(rate, 1), "unit": unit, "peak": peak,
                                   "frac": round(rate / peak, 4),
@@ -356,8 +427,15 @@ def main():
     }
     if not args.no_cpu_baseline and name in CPU_SAMPLES:
         line["cpu_baseline"] = cpu_baseline(name, harness, driver)
+    short = lambda w: w.split("_", 1)[0]   # noqa: E731  "c5_gemm_..." -> "c5"
+    line["config"]["why_this_workload"] = ("configs[1] of BASELINE.json, the configuration the contract names for N=1; all five "
+                                           "configurations are under roofline.by_config" if name == DEFAULT_WORKLOAD else "--workload")
     if not args.only:
         per = {}
+        by_config = {}
+        cpu_by_config = {}
+        power = {}
+        sampler = PowerSampler()
         for other in sorted(WORKLOADS):
             try:
                 if other == name:
@@ -368,6 +446,7 @@ def main():
                                                                driver, harness, np)
                     entry = dict(roofline_of(k2, kms, other), kernel_ms=round(kms, 5), kernel_ms_median=round(kmed, 5),
                                  kernel_ms_min=round(kmin, 5))
+                by_config[short(other)] = {"bound": entry["bound"], "frac": entry["frac"], "kernel_ms": entry["kernel_ms"]}
                 if other in CACHE_RESIDENT:
                     # the same buffers launch after launch: reads come from the 256 MB last-level cache
                     _, _, _, rms, _, rmin, _ = gpu_measure(other, max(20, args.steps // 4), max(5, args.warmup // 2), torch,
@@ -384,11 +463,33 @@ def main():
                                                 "frac": r["frac"]}
                 if other in CPU_SAMPLES and not args.no_cpu_baseline:
                     entry["cpu_baseline"] = line["cpu_baseline"] if other == name else cpu_baseline(other, harness, driver)
+                    c = entry["cpu_baseline"]
+                    cpu_by_config[short(other)] = {"value": c["value"], "unit": c["unit"], "cores": c["cores"],
+                                                   "all_cores_value": c.get("all_cores_value"), "all_cores": c.get("all_cores")}
+                if other.startswith("c5_") and sampler.smi is not None:
+                    # power and clock while the int8 GEMM runs (its own buffers, outside any timed region)
+                    dev = torch.device("cuda:0")
+                    bufs = [torch.zeros(t.nbytes, dtype=torch.uint8, device=dev) for t in k2.tensors]
+                    for b, a in zip(bufs, harness.make_inputs(harness.load_desc(os.path.join(FIXTURES, other + ".info")), seed=harness.BASE_SEED + 1)):
+                        b.copy_(torch.from_numpy(a.view(np.uint8).reshape(-1)))
+                    ptrs = [b.data_ptr() for b in bufs]
+                    st = torch.cuda.current_stream().cuda_stream
+                    power[short(other)] = sampler.during(lambda i: k2.launch_ptrs(ptrs, st), torch)
+                    del bufs
                 per[other] = entry
             except driver.AkgHipError as e:
                 per[other] = {"error": str(e)}
-        line["per_config"] = per
-        line["calibration"] = calibration(torch, driver, harness, np, max(20, args.steps // 4), max(5, args.warmup // 2))
+                by_config[short(other)] = {"error": str(e)[:80]}
+        detail = {"per_config": per,
+                  "calibration": calibration(torch, driver, harness, np, max(20, args.steps // 4), max(5, args.warmup // 2), sampler, power)}
+        detail["power"] = power
+        line["roofline"]["by_config"] = by_config
+        if cpu_by_config:
+            line["cpu_by_config"] = cpu_by_config
+        line["calibration"] = dict({k: v.get("frac") for k, v in detail["calibration"].items() if isinstance(v, dict) and "frac" in v},
+                                   power=power)
+        sys.stderr.write("detail: " + json.dumps(detail) + "\n")
+        sys.stderr.flush()
     print(json.dumps(line))
 
 

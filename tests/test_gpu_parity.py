@@ -24,7 +24,8 @@ SMALL = [n for n in ALL_SMALL if not any(m in n for m in STREAM_MARKS) and "segm
          and "sgdclip" not in n]
 STREAM = [n for n in ALL_SMALL if any(m in n for m in STREAM_MARKS) and "bnstats_update" not in n and n not in STAGED]
 FULL = ["c1_ew_tanh_add_mul_f32_1024x4096.info", "c2_softmax_f16_8192x4096.info",
-        "c3_layernorm_residual_bf16_16384x4096.info", "c4_quant_int8_residual_bf16_32768x8192.info"]
+        "c3_layernorm_residual_bf16_16384x4096.info", "c4_quant_int8_residual_bf16_32768x8192.info",
+        "n10_rmsnorm_bf16_16384x4096.info", "n11_rmsnorm_add_bf16_16384x4096.info"]
 
 
 def _torch_view(a):

@@ -199,6 +199,46 @@ def test_layernorm_float32_against_float64_tight(tmp_path):
     assert not np.allclose(unbiased, want, rtol=1e-4, atol=1e-4)
 
 
+def test_rmsnorm_matches_float64_closed_form(tmp_path):
+    # x * rsqrt(mean(x^2) + eps) * gamma in float32 end to end against float64: a mean subtracted by mistake (LayerNorm), a
+    # sum in place of the mean, or epsilon outside the root all show at 1e-4 on small-variance rows
+    text = op_desc.rmsnorm(6, 64, "float32", eps=1e-6, name="rms_f32_6x64")
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal((6, 64)) * 1e-3 + 2e-3).astype(np.float32)      # small, not centred: epsilon and the mean matter
+    g = rng.uniform(0.5, 1.5, 64).astype(np.float32)
+    _, c_out, n_out = build_and_run(text, [x, g], tmp_path)
+    xd, gd = x.astype(np.float64), g.astype(np.float64)
+    want = xd / np.sqrt((xd * xd).mean(axis=1, keepdims=True) + 1e-6) * gd
+    assert np.allclose(c_out[0], want, rtol=3e-6, atol=1e-9)
+    assert np.allclose(n_out[0], want, rtol=3e-6, atol=1e-9)
+    centred = (xd - xd.mean(1, keepdims=True)) / np.sqrt(xd.var(1, keepdims=True) + 1e-6) * gd
+    no_eps = xd / np.sqrt((xd * xd).mean(axis=1, keepdims=True)) * gd
+    summed = xd / np.sqrt((xd * xd).sum(axis=1, keepdims=True) + 1e-6) * gd
+    for wrong in (centred, no_eps, summed):
+        assert not np.allclose(wrong, want, rtol=1e-4, atol=1e-9)
+
+
+def test_rmsnorm_fixtures_match_torch_float64_and_invariants():
+    import torch
+    desc, (x, g), c_out, n_out = run_fixture_both("small_rmsnorm_bf16_19x520", 15)
+    xf, gf = (torch.from_numpy(harness.bf16_bits_to_f32(t)).double() for t in (x, g))
+    want = torch.nn.functional.rms_norm(xf, (520,), gf, eps=1e-6).numpy()
+    for got in (c_out[0], n_out[0]):
+        gotf = harness.bf16_bits_to_f32(got).astype(np.float64)
+        assert np.allclose(gotf, want, rtol=8e-3, atol=1e-6)              # bfloat16 output: 2^-8 relative
+        z = gotf / gf.numpy()
+        assert np.abs((z * z).mean(axis=1) - 1.0).max() < 2e-2           # rows have unit mean square
+    # with the residual add in front: h = bf16(x + r) is an output and is what gets normalised
+    desc, (x, g, r), c_out, n_out = run_fixture_both("small_rmsnorm_add_bf16_64x4096", 16)
+    xf, gf, rf = (harness.bf16_bits_to_f32(t) for t in (x, g, r))
+    h_bits = harness.f32_to_bf16_bits(xf + rf)
+    hd = torch.from_numpy(harness.bf16_bits_to_f32(h_bits)).double()
+    want = torch.nn.functional.rms_norm(hd, (4096,), torch.from_numpy(gf).double(), eps=1e-6).numpy()
+    for outs in (c_out, n_out):
+        assert np.array_equal(outs[0], h_bits)
+        assert np.allclose(harness.bf16_bits_to_f32(outs[1]).astype(np.float64), want, rtol=8e-3, atol=1e-6)
+
+
 def correctly_rounded_f32(fr):
     """Nearest float32 (ties to even) of an exact Fraction, by comparing against the neighbours' midpoints."""
     approx = np.float32(float(fr))

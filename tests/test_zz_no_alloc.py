@@ -54,6 +54,49 @@ def _run(kernel, inputs, static):
     return [t.cpu().numpy().view(np.uint8).copy() for t in outs + ins]
 
 
+def test_first_static_scratch_launch_is_captured_into_a_graph_and_allocates_nothing():
+    """The callers this entry point is for: the FIRST launch through it in the process (when this file runs alone) is
+    recorded into a HIP graph - `prepare` has looked the array's address up, so nothing is loaded or materialised under
+    capture -, the graph is replayed three times on fresh inputs with the program's own eager launches and
+    synchronisations in between, every replay equal to akg_hip_launch bit for bit; and an eager call leaves the
+    device's free memory exactly as it found it."""
+    import torch
+    dev = torch.device("cuda:0")
+    path = os.path.join(FIXTURES, "small_biasgrad_bf16_2048x1024.info")
+    kernel = driver.HipKernel.from_file(path)
+    assert kernel.workspace_bytes > 0
+    desc = harness.load_desc(path)
+    kernel.prepare()
+    static = [torch.zeros(t.nbytes, dtype=torch.uint8, device=dev) for t in kernel.tensors]
+    eager = [torch.zeros(t.nbytes, dtype=torch.uint8, device=dev) for t in kernel.tensors]
+    n_in = len(kernel.tensors) - len(kernel.outputs)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        kernel.launch_static_scratch_ptrs([b.data_ptr() for b in static], torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        print("replay %d" % replay, flush=True)
+        inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 77 + replay)
+        for bufs in (static, eager):
+            for b, a in zip(bufs, inputs):
+                b.copy_(torch.from_numpy(a.view(np.uint8).reshape(-1)))
+            for b in bufs[n_in:]:
+                b.fill_(0x7B)
+        graph.replay()
+        torch.cuda.synchronize()
+        kernel.launch(eager)                      # the allocating entry point, eagerly, between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(static[n_in:], eager[n_in:]):
+            assert torch.equal(a, b), "replay %d differs from akg_hip_launch" % replay
+    free_before = torch.cuda.mem_get_info()[0]
+    kernel.launch_static_scratch_ptrs([b.data_ptr() for b in static], torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free_after = torch.cuda.mem_get_info()[0]
+    assert free_after == free_before, "an eager static-scratch launch changed the free device memory by %d bytes" % (free_before - free_after)
+    for a, b in zip(static[n_in:], eager[n_in:]):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("first,second", SEQUENCES)
 def test_static_scratch_launch_equals_the_allocating_launch(first, second):
     cases = []
