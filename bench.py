@@ -154,10 +154,12 @@ def timed(launch, steps, warmup, torch, groups=True):
     return wall_ms, mean_ms, statistics.median(per), min(per)
 
 
-def gpu_measure(name, steps, warmup, torch, driver, harness, np, resident=False, variant=None):
+def gpu_measure(name, steps, warmup, torch, driver, harness, np, resident=False, variant=None, text=None):
     path = os.path.join(FIXTURES, name + ".info")
-    desc = harness.load_desc(path)
-    if variant is None:
+    desc = json.loads(text) if text is not None else harness.load_desc(path)
+    if text is not None:
+        kernel = driver.HipKernel(text, out_dir=None)      # a description made for this run (the size sweep)
+    elif variant is None:
         kernel = driver.HipKernel.from_file(path)
     else:
         # another schedule of the same description: built without artifacts, so that the cached default stays
@@ -232,8 +234,8 @@ def cpu_baseline(name, harness, driver):
 
 
 class PowerSampler:
-    """Socket power (W) and shader clock (MHz) of GPU 0 read through amdsmi while a callable keeps the device busy; never
-    inside a timed region. Every field is None where the library or the permission to read is missing."""
+    """Socket power (W) and shader clock (MHz) of GPU 0 read through amdsmi while a callable keeps the device busy (2.6 s, the
+    readings of the last second: they refresh about once a second); never inside a timed region. Every field is None where the library or the permission to read is missing."""
 
     def __init__(self):
         self.smi = None
@@ -268,7 +270,7 @@ class PowerSampler:
             pass
         return power, clock
 
-    def during(self, launch, torch, busy_ms=400.0):
+    def during(self, launch, torch, busy_ms=2600.0):
         """Keeps the device busy with `launch(i)` for busy_ms and samples between batches of launches."""
         if self.smi is None:
             return {"socket_power_w": None, "shader_clock_mhz": None, "samples": 0}
@@ -279,14 +281,19 @@ class PowerSampler:
             for _ in range(8):
                 launch(i)
                 i += 1
-            if (time.perf_counter() - t0) * 1e3 > busy_ms / 4:   # past the clock ramp
+            if (time.perf_counter() - t0) * 1e3 > busy_ms * 0.6:   # the library's readings refresh about once a second
                 p, c = self.read()
                 if p is not None:
                     powers.append(p)
                 if c is not None:
                     clocks.append(c)
             torch.cuda.synchronize()
-        return {"socket_power_w": round(statistics.median(powers), 1) if powers else None,
+        cap = None
+        try:
+            cap = round(float(self.smi.amdsmi_get_power_cap_info(self.handle).get("power_cap", 0)) / 1e6, 0) or None
+        except Exception:
+            pass
+        return {"socket_power_w": round(statistics.median(powers), 1) if powers else None, "power_cap_w": cap,
                 "shader_clock_mhz": round(statistics.median(clocks), 0) if clocks else None, "samples": max(len(powers), len(clocks))}
 
 
@@ -308,6 +315,35 @@ def vendor_gemm(kind, torch, steps):
     rate = 2.0 * m * n * k / (mean_ms * 1e-3) / 1e12
     return {"kernel_ms": round(mean_ms, 5), "kernel_ms_median": round(med_ms, 5), "kernel_ms_min": round(min_ms, 5),
             "achieved": round(rate, 1), "unit": unit, "frac": round(rate / peak, 4), "what": what}
+
+
+def size_sweep(torch, driver, harness, np, steps, warmup):
+    """C1's and C2's kernels at half to eight times their rows: kernel time = fixed + bytes / rate fitted by least
+    squares. `fixed_us` is what a launch of this kind costs whatever its size (ramp of the first loads, drain of the
+    last stores), `asymptote_frac` the fraction of the HBM peak the same kernel streams at once that cost is amortised;
+    `frac_at_size` is what the fit gives at the configuration's own size."""
+    from akg_amd import op_desc
+    out = {}
+    patterns = {
+        "c1": (lambda r: op_desc.elementwise_tanh_add_mul(r, 4096, name="sweep_c1_%d" % r), 1024),
+        "c2": (lambda r: op_desc.softmax_last_axis(r, 4096, "float16", name="sweep_c2_%d" % r), 8192),
+    }
+    for key, (make, base_rows) in patterns.items():
+        xs, ys, points = [], [], {}
+        for factor in (0.5, 1, 2, 4, 8):
+            rows = int(base_rows * factor)
+            k, _, _, mean_ms, _, _, _ = gpu_measure("sweep", steps, warmup, torch, driver, harness, np, text=make(rows))
+            xs.append(float(k.algorithmic_bytes))
+            ys.append(mean_ms * 1e-3)
+            points["%dx4096" % rows] = round(mean_ms * 1e3, 2)
+            del k
+        a = np.vstack([np.ones(len(xs)), np.array(xs)]).T
+        (fixed_s, per_byte), *_ = np.linalg.lstsq(a, np.array(ys), rcond=None)
+        base_bytes = xs[1]
+        out[key] = {"kernel_us_by_shape": points, "fixed_us": round(fixed_s * 1e6, 2),
+                    "asymptote_frac": round(1.0 / per_byte / 1e9 / HBM_PEAK_GBS, 4),
+                    "frac_at_size": round(base_bytes / (fixed_s + per_byte * base_bytes) / 1e9 / HBM_PEAK_GBS, 4)}
+    return out
 
 
 def calibration(torch, driver, harness, np, steps, warmup, sampler=None, power=None):
@@ -483,11 +519,16 @@ def main():
         detail = {"per_config": per,
                   "calibration": calibration(torch, driver, harness, np, max(20, args.steps // 4), max(5, args.warmup // 2), sampler, power)}
         detail["power"] = power
+        try:
+            detail["size_sweep"] = size_sweep(torch, driver, harness, np, max(20, args.steps // 4), max(5, args.warmup // 2))
+        except driver.AkgHipError as e:
+            detail["size_sweep"] = {"error": str(e)}
         line["roofline"]["by_config"] = by_config
         if cpu_by_config:
             line["cpu_by_config"] = cpu_by_config
         line["calibration"] = dict({k: v.get("frac") for k, v in detail["calibration"].items() if isinstance(v, dict) and "frac" in v},
-                                   power=power)
+                                   power=power, size_sweep={k: {x: v[x] for x in ("fixed_us", "asymptote_frac", "frac_at_size")}
+                                                            for k, v in detail["size_sweep"].items() if isinstance(v, dict) and "fixed_us" in v})
         sys.stderr.write("detail: " + json.dumps(detail) + "\n")
         sys.stderr.flush()
     print(json.dumps(line))
