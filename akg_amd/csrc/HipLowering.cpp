@@ -35,7 +35,7 @@ LoweringOptions LoweringOptions::fromEnvironment() {
   o.block = readInt("AKG_HIP_BLOCK");
   o.split = readInt("AKG_HIP_SPLIT");
   o.variant = readInt("AKG_HIP_VARIANT");
-  if (o.variant == 0) o.variant = readInt("AKG_HIP_GEMM_VARIANT");   // the switch's earlier name
+  if (const int cus = readInt("AKG_HIP_CUS"); cus >= 1 && cus <= 4096) o.computeUnits = cus;
   if (const char *nt = std::getenv("AKG_HIP_NT")) o.nonTemporal = (nt[0] != '0') ? 1 : 0;
   return o;
 }

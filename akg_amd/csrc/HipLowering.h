@@ -43,16 +43,19 @@ struct LoweringOptions {
   int block = 0;        // threads per workgroup
   int split = 0;        // streaming reductions: workgroups sharing one group of outputs (AKG_HIP_SPLIT)
   // Experiment switch (AKG_HIP_VARIANT), read by whichever family lowers the kernel; 0 = the measured default.
-  //   gemm_epilogue  bit 3: no skinny kernel for M <= 64, bit 4: skinny kernel only up to 32 rows,
+  //   gemm_epilogue  bit 3: no skinny kernel for M <= 64 (the tile kernel with K split instead),
   //                  bit 5: the other arrangement of the tile kernel's wavefronts (2 x 4 for 4 x 2 and back)
   //   row_reduce     1: keep the row in registers, 2: walk the row (no packing), 4: walk it, packed if possible
-  //   stream_reduce  1: split-major workgroup order, 3: launch order for short runs, 7: no column kernel (several kernels instead)
+  //   stream_reduce  7: no column kernel (several kernels instead)
   //   column_reduce  5: one strip per workgroup (no second set of resident registers)
   //   segment_sum    1: every workgroup scans all ids, 2: positions grouped by segment first (whatever the size),
-  //                  3: grouped by bucket of segments first (whatever the number of buckets), 4: as 3, chunks in launch order
-  //   indexed        1: no LDS-tiled transposes, 2: no chunk-wide loads, 3: launch order of tiles, 5: no non-temporal hints
+  //                  3: grouped by bucket of segments first (whatever the number of buckets)
+  //   indexed        1: no LDS-tiled transposes, 2: no chunk-wide loads
   int variant = 0;
   int nonTemporal = 1;  // stream once-touched tensors with non-temporal accesses (AKG_HIP_NT=0 turns it off)
+  // Compute units of the part the kernels are made for (MI355X / MI350X: 256; AKG_HIP_CUS for another gfx950 part):
+  // what persistent grids are sized by. The lowering runs without a device, so this is not asked of one.
+  int computeUnits = 256;
   // Dynamic-shape descriptions: the elementwise / row-reduction kernels take their row count (or, when everything
   // folds into one dimension, their element count) as a kernel argument instead of a constant, so that shape sets
   // that differ only there share one code object (the source no longer depends on them).

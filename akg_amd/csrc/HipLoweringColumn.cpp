@@ -261,7 +261,7 @@ class ColumnEmitter {
     // wavefronts per SIMD beside the second set, spills under the 128-register limit and takes 87 us; softmax over 21
     // classes of f16 [32,21,512,512], 24 resident registers in 256 threads: 114 us as it is, 150 us pipelined.)
     const int64_t regs = static_cast<int64_t>(chunks_) * ((fullBytes * vec_ + 3) / 4);
-    constexpr int64_t kCUs = 256;
+    const int64_t kCUs = opt_.computeUnits;
     pipelined_ = !ordered_ && opt_.variant != 5 && regs >= 40 && regs <= 64 && block_ == 512 && outer_ * strips_ >= 2 * kCUs;
     launched_ = pipelined_ ? kCUs : outer_ * strips_;
   }

@@ -99,7 +99,7 @@ class GemmEmitter {
   std::ostringstream src_;
   int64_t m_ = 0, n_ = 0, k_ = 0, batch_ = 1;
   int kSplit_ = 1;  // workgroups per tile, each with a range of K steps (see pickSplit)
-  int skinnyRows() const { return (opt_.variant & 16) ? 32 : 64; }   // (96 rows: no faster than the tile kernel; 128: slower)
+  int skinnyRows() const { return 64; }   // (96 rows: no faster than the tile kernel; 128: slower)
   int skinnyWaves() const { return opt_.block == 512 ? 8 : 4; }
   int skinnyUnroll() const { return opt_.chunks > 0 ? opt_.chunks : 2; }
   bool serial_ = false;  // no MFMA kernel takes the description: gemm_serial (akg_gemm_serial.hpp)

@@ -227,7 +227,7 @@ class IndexedEmitter {
   // broadcast, a Gather's data operand or a second consumer mean re-use, and such inputs keep ordinary loads.
   void findStreamedInputs() {
     streamedInput_.assign(g_.inputs.size(), false);
-    if (opt_.nonTemporal == 0 || opt_.variant == 5) return;
+    if (opt_.nonTemporal == 0) return;
     std::vector<int> uses(g_.tensors.size(), 0);
     for (const OpNode &op : g_.ops) {
       for (int in : op.inputs) ++uses[static_cast<size_t>(in)];
@@ -726,7 +726,7 @@ class IndexedEmitter {
     // output rows that are not whole cache lines: tiles that write parts of one line next to each other on one XCD
     // (64 x 1000 x 1024 -> 64 x 1024 x 1000 bf16: 33.5 % of the HBM peak in launch order)
     const int64_t outRowBytes = space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[0]).dtype));
-    if (outRowBytes % 64 != 0 && opt_.variant != 3 && grid_ >= 64) {
+    if (outRowBytes % 64 != 0 && grid_ >= 64) {
       src_ << "  int akg_w = akg::xcd_contiguous_id(static_cast<int>(blockIdx.x), " << grid_ << ");\n";
     } else {
       src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
@@ -878,7 +878,7 @@ class IndexedEmitter {
     closeElementLoop();
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       // results are written once and never read by this kernel: non-temporal where whole 64-byte pieces are stored
-      const bool ntOut = opt_.nonTemporal != 0 && opt_.variant != 5 &&
+      const bool ntOut = opt_.nonTemporal != 0 &&
                          (space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[i]).dtype))) % 64 == 0;
       stmt(std::string("akg::store_chunk") + (overlapTail_ ? "_unaligned<" : "<") + tagOf(g_.outputs[i]) + ", V" +
            (overlapTail_ ? "" : (ntOut ? ", true" : ", false")) + ">(out" + std::to_string(i) + " + base, o" +

@@ -496,7 +496,7 @@ class StreamReduceEmitter {
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
     // Runs shorter than a few cache lines that do not end on line boundaries ([N,C,7,7]: 98 bytes per channel and
     // image): the lines are shared with the neighbouring outputs' runs.
-    xcdContiguous_ = !dirY_ && scatteredR && grid_ >= 64 && opt_.variant != 3 &&
+    xcdContiguous_ = !dirY_ && scatteredR && grid_ >= 64 &&
                      (fastExtent * static_cast<int64_t>(widest)) % 128 != 0 && fastExtent * static_cast<int64_t>(widest) < 2048;
     // workspace: one arrival counter per group, then the partials of every reduction
     workspaceBytes_ = 0;
@@ -744,7 +744,7 @@ class StreamReduceEmitter {
     } else {
       line("  const long akg_wg = static_cast<long>(blockIdx.x);");
     }
-    if (dirY_ && opt_.variant != 1) {
+    if (dirY_) {
       // neighbouring workgroups take neighbouring column strips of the same rows: what is in flight at any time
       // covers whole rows of the tensor rather than 256-byte pieces 8 KiB apart
       src_ << "  constexpr long GROUPS = " << groups_ << "L;\n";

@@ -515,7 +515,7 @@ __device__ inline void chunk_sort(const int (&key)[TILES], unsigned (&slot)[TILE
  * Both sorts are stable, so the order per output element is the position order and the result is the serial loop's,
  * bit for bit.
  */
-LoweredKernel lowerSegmentBucketed(const OpGraph &g, const LoweringOptions &options, const SegmentShapes &sh, int bucketBits) {
+LoweredKernel lowerSegmentBucketed(const OpGraph &g, const LoweringOptions &, const SegmentShapes &sh, int bucketBits) {
   using lowering::computeTypeName;
   using lowering::dtypeTag;
   const TensorValue &data = *sh.data, &ids = *sh.ids, &out = *sh.out;
@@ -571,12 +571,8 @@ LoweredKernel lowerSegmentBucketed(const OpGraph &g, const LoweringOptions &opti
   s << "  __shared__ unsigned short akg_cnt[NW * KEYS];\n";
   s << "  __shared__ unsigned akg_start[KEYS], akg_len[KEYS], akg_scan[NW];\n";
   s << "  const int tid = static_cast<int>(threadIdx.x), lane = tid & 63, w = tid >> 6;\n";
-  if (options.variant == 4) {
-    s << "  const int run = static_cast<int>(blockIdx.x);\n";
-  } else {
-    s << "  const int run = static_cast<int>(blockIdx.x & 7u) * " << perXcd << " + static_cast<int>(blockIdx.x >> 3);\n";
-    s << "  if (run >= RUNS) return;   // (uniform)\n";
-  }
+  s << "  const int run = static_cast<int>(blockIdx.x & 7u) * " << perXcd << " + static_cast<int>(blockIdx.x >> 3);\n";
+  s << "  if (run >= RUNS) return;   // (uniform)\n";
   s << "  const int p0 = run * RUN + w * (64 * TILES);\n";
   s << "  const unsigned *__restrict__ rows = reinterpret_cast<const unsigned *>(" << dataName << ");\n";
   s << "  int id[TILES], key[TILES];\n  unsigned row[TILES][ROW_WORDS], slot[TILES];\n";
@@ -697,7 +693,7 @@ LoweredKernel lowerSegmentBucketed(const OpGraph &g, const LoweringOptions &opti
   phase("_count", chunks, 256);
   phase("_offsets", offsetsGrid(buckets), 256);
   phase("_starts", 1, 1024);
-  phase("_place", options.variant == 4 ? chunks : perXcd * 8, 512);
+  phase("_place", perXcd * 8, 512);
   k.workspaceBytes = static_cast<uint64_t>(words) * 4;
   k.algorithmicBytes = lowering::countAlgorithmicBytes(g);
   k.shapeArgs = lowering::buildShapeArgs(g);
@@ -902,7 +898,7 @@ LoweredKernel lowerSegmentSumToHip(const OpGraph &g, const LoweringOptions &opti
   while (bucketBits > 0 && (sh.slice << bucketBits) > 32) --bucketBits;
   const int64_t buckets = (sh.segments + (1LL << bucketBits) - 1) >> bucketBits;
   const bool canBucket = group && !wide && rowBytes <= 12 && rowBytes % 4 == 0 && bucketBits >= 2 && buckets <= 640 && buckets >= 2;
-  if (canBucket && (options.variant == 3 || options.variant == 4 || (options.variant == 0 && buckets >= 96))) {
+  if (canBucket && (options.variant == 3 || (options.variant == 0 && buckets >= 96))) {
     return lowerSegmentBucketed(g, options, sh, bucketBits);
   }
   return group ? lowerSegmentSorted(g, options, sh) : lowerSegmentScan(g, options, sh);

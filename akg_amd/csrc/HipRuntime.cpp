@@ -543,6 +543,15 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
     int rc = fromMemory ? AKG_HIP_OK : compileToCodeObject(k->lowered, &k->codeObject, &log);
     if (rc != AKG_HIP_OK) {
       if (!base.empty()) (void)writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size());
+      if (k->lowered.family == akg::KernelFamily::ColumnReduce && allowStages) {
+        // The column kernel is an optimisation over one kernel per reduction level (registers of two resident sets,
+        // LDS of the widest strips): if its source does not compile, the description still runs the other way.
+        if (!artifactSuffix.empty() && k->graph.name.size() > artifactSuffix.size()) {
+          k->graph.name.erase(k->graph.name.size() - artifactSuffix.size());
+        }
+        return compileStaged(jsonText, std::move(k), outDir, outKernel,
+                             "device compilation of the column kernel failed (" + log.substr(0, 200) + ")", binding != nullptr, artifactSuffix);
+      }
       return fail(rc, "device compilation of " + k->lowered.kernelName + " failed:\n" + log);
     }
     akg::Sha256 h;
