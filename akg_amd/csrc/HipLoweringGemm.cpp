@@ -73,6 +73,13 @@ class GemmEmitter {
       }
       k.block[0] = 512;
     }
+    if (dyn_) {
+      // the row count and the number of K splits travel as kernel arguments, and the workspace pointer is part of the
+      // signature whether this shape set splits K or not
+      k.scalarArgs.push_back(m_);
+      k.scalarArgs.push_back(kSplit_);
+      k.workspaceBytes = std::max<uint64_t>(k.workspaceBytes, 256);
+    }
     k.grid[1] = static_cast<unsigned>(batch_);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.algorithmicOps = 2ull * static_cast<uint64_t>(batch_) * static_cast<uint64_t>(m_) * static_cast<uint64_t>(n_) *
@@ -89,6 +96,7 @@ class GemmEmitter {
       note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName(true) << " waves=" << (tallWavefrontTiles() ? "2x4" : "4x2") << " grid=" << k.grid[0];
     }
     if (kSplit_ > 1) note << " k_splits=" << kSplit_;
+    if (dyn_) note << " (rows of A and K splits are kernel arguments: one code object for " << (skinny_ ? "up to " + std::to_string(skinnyBucket()) + " rows" : "more than 64 rows") << ")";
     k.scheduleNote = note.str();
     return k;
   }
@@ -105,6 +113,10 @@ class GemmEmitter {
   bool serial_ = false;  // no MFMA kernel takes the description: gemm_serial (akg_gemm_serial.hpp)
   int epiWidth() const { return (serial_ && n_ % 4 != 0) ? 1 : 4; }   // adjacent result columns per epilogue call
   bool skinny_ = false;  // M <= 64: the kernel that streams B straight into MFMA operands (gemm_skinny)
+  // A dynamic description (extents bound per call): M and the K split are kernel arguments, so the source - and with it
+  // the code object - is the same for every token count; the skinny kernel comes in three sizes (16, 32, 64 rows).
+  bool dyn_ = false;
+  int skinnyBucket() const { return m_ <= 16 ? 16 : (m_ <= 32 ? 32 : 64); }
   bool transB_ = false;
   int matmulOp_ = -1;
   int aId_ = -1, bId_ = -1, accId_ = -1;
@@ -136,6 +148,7 @@ class GemmEmitter {
   void pickSplit() {
     kSplit_ = 1;
     if (serial_) return;
+    dyn_ = opt_.extentAsArgument && batch_ == 1 && m_ * k_ * elemBytes() < (1LL << 31);
     // At most 64 rows of A (and K a multiple of 32 bytes): the time is that of streaming B, which gemm_skinny reads
     // straight into MFMA operands; 256 workgroups of four wavefronts (one per CU: 16 x 8192 x 8192 bf16 reaches 66 % of
     // the HBM peak with 4 splits of 64 strips, 59 % with 8, 48 % with 2; 8 wavefronts or more steps in flight change
@@ -452,9 +465,14 @@ class GemmEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
-    if (kSplit_ > 1) src_ << ", unsigned *__restrict__ akg_ws";
-    src_ << ") {\n  Epilogue epi;\n  const long akg_batch = static_cast<long>(blockIdx.y);\n"
-         << "  epi.row0 = akg_batch * " << m_ << "L;\n";
+    if (dyn_) src_ << ", const long akg_m, const long akg_ksplit";
+    if (kSplit_ > 1 || dyn_) src_ << ", unsigned *__restrict__ akg_ws";
+    src_ << ") {\n  Epilogue epi;\n  const long akg_batch = static_cast<long>(blockIdx.y);\n";
+    if (dyn_) {
+      src_ << "  epi.row0 = 0L;   // (one batch)\n";
+    } else {
+      src_ << "  epi.row0 = akg_batch * " << m_ << "L;\n";
+    }
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       const int id = g_.inputs[i];
       const bool written = std::find(assignOnly_.begin(), assignOnly_.end(), static_cast<int>(i)) != assignOnly_.end();
@@ -469,10 +487,22 @@ class GemmEmitter {
       return;
     }
     if (skinny_) {
+      if (dyn_) {
+        src_ << "  akg::gemm_skinny<" << mmaTraits() << ", " << skinnyBucket() << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
+             << ", Epilogue, 1, " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (opt_.nonTemporal != 0 ? "true" : "false") << ", true>(in"
+             << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi, akg_ws, 0L, akg_m, static_cast<int>(akg_ksplit));\n}\n";
+        return;
+      }
       src_ << "  akg::gemm_skinny<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
            << ", Epilogue, " << kSplit_ << ", " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (opt_.nonTemporal != 0 ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in"
            << g_.tensor(bId_).inputIndex << " + akg_batch * " << k_ * n_ << "L, epi, " << (kSplit_ > 1 ? "akg_ws" : "nullptr")
            << ", akg_batch * " << (n_ + 127) / 128 << "L);\n}\n";
+      return;
+    }
+    if (dyn_) {
+      src_ << "  akg::gemm_256x256<" << mmaTraits() << ", 0L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
+           << ", Epilogue, 1, " << (tallWavefrontTiles() ? 2 : 4) << ", true>(in" << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex
+           << ", epi, akg_ws, akg_m, static_cast<int>(akg_ksplit));\n}\n";
       return;
     }
     src_ << "  akg::gemm_256x256<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")

@@ -149,9 +149,15 @@ struct SubstepFront {
   }
 };
 
-template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1, int WM = 4>
+// DYN: the row count of A and the number of K splits are kernel arguments (`mDyn`, `ksDyn`; the template's M and KSPLIT
+// are then ignored): one code object serves every M of a description whose leading extents are open, and the host
+// chooses the split for each call. Rows are bounds-checked at run time; `ws` is always a valid pointer.
+template <typename Mma, long MS, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT = 1, int WM = 4, bool DYN = false>
 AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B, Epilogue &epi,
-                          unsigned *__restrict__ ws = nullptr) {
+                          unsigned *__restrict__ ws = nullptr, long mDyn = 0, int ksDyn = 1) {
+  const long M = DYN ? mDyn : MS;                 // (a constant after inlining unless DYN)
+  const int kSplits = DYN ? ksDyn : KSPLIT;
+  constexpr bool kSplitPossible = DYN || KSPLIT > 1;
   constexpr int EB = Mma::kElemBytes;
   constexpr long K = KE * EB;    // bytes of K per row of A (and per column of B)
   constexpr long NB = N * EB;    // bytes per k-row of a row-major B
@@ -182,12 +188,12 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   constexpr int kTN = kWaveCols / 16;                 // MFMA column tiles (16 columns) per wavefront
   constexpr int kHM = kTM / 2, kHN = kTN / 2;         // tiles per half: a quarter of the wavefront tile is kHM x kHN = 8 MFMAs
   static_assert(kHM * kHN == 8, "a substep is 8 MFMAs");
-  constexpr long kTilesM = (M + kGemmBM - 1) / kGemmBM;
+  const long kTilesM = (M + kGemmBM - 1) / kGemmBM;
   constexpr long kTilesN = (N + kGemmBN - 1) / kGemmBN;
-  constexpr long kTiles = kTilesM * kTilesN;
-  constexpr long kPerXcd = (kTiles + kGemmXcds - 1) / kGemmXcds;
+  const long kTiles = kTilesM * kTilesN;
+  const long kPerXcd = (kTiles + kGemmXcds - 1) / kGemmXcds;
   constexpr long kSteps = (K + BK - 1) / BK;
-  constexpr bool kFull = (M % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
+  constexpr bool kFull = !DYN && (MS % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
   constexpr int kTileBytes = kGemmBM * kPitch;        // one operand tile in LDS
   static_assert(kRowChunks == 4, "the staging schedule is written for four 16-byte chunks per thread and operand");
   // A row-major B goes to LDS as it lies in memory, k-rows of 256 columns. Sixteen lanes share a transposing read:
@@ -208,16 +214,16 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   __shared__ __attribute__((aligned(16))) u8 lds[2][2][kTileBytes];  // [buffer][A|B]
 
   // ---- workgroup -> tile
-  constexpr long kGridTiles = kPerXcd * kGemmXcds;   // workgroups per K split (a multiple of the XCD count)
+  const long kGridTiles = kPerXcd * kGemmXcds;   // workgroups per K split (a multiple of the XCD count)
   const long wgAll = static_cast<long>(blockIdx.x);
-  const long ksplit = KSPLIT > 1 ? wgAll / kGridTiles : 0;
-  const long wg = KSPLIT > 1 ? wgAll % kGridTiles : wgAll;
+  const long ksplit = kSplitPossible ? wgAll / kGridTiles : 0;
+  const long wg = kSplitPossible ? wgAll % kGridTiles : wgAll;
   const long linear = (wg % kGemmXcds) * kPerXcd + wg / kGemmXcds;
   if (linear >= kTiles) return;
-  constexpr long kStepsPer = (kSteps + KSPLIT - 1) / KSPLIT;
-  static_assert((KSPLIT - 1) * kStepsPer < kSteps, "every K split needs at least one step");
+  const long kStepsPer = (kSteps + kSplits - 1) / kSplits;
+  static_assert(DYN || (KSPLIT - 1) * ((kSteps + KSPLIT - 1) / KSPLIT) < kSteps, "every K split needs at least one step");
   const long stepBase = ksplit * kStepsPer;
-  const long mySteps = KSPLIT == 1 ? kSteps : ((kSteps - stepBase) < kStepsPer ? (kSteps - stepBase) : kStepsPer);
+  const long mySteps = !kSplitPossible ? kSteps : ((kSteps - stepBase) < kStepsPer ? (kSteps - stepBase) : kStepsPer);
   constexpr long kGroupSize = kGemmGroupRows * kTilesN;
   const long group = linear / kGroupSize;
   const long firstRow = group * kGemmGroupRows;
@@ -256,7 +262,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // Global loads are buffer loads: the per-lane offset is computed once, everything that changes from load to load
   // (row block, k-row, K step) is a scalar offset, so the loop spends no vector instructions on addresses (vector
   // instructions and MFMAs compete for issue cycles). Out-of-range lanes read zero through the descriptor's size.
-  static_assert(M * K < (1L << 31) && N * K < (1L << 31), "operand too large for 32-bit buffer offsets");
+  static_assert((DYN || MS * K < (1L << 31)) && N * K < (1L << 31), "operand too large for 32-bit buffer offsets");
   const __amdgpu_buffer_rsrc_t aRsrc = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<void *>(A), 0, static_cast<int>(M * K), 0x00020000);
   const __amdgpu_buffer_rsrc_t bRsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -336,7 +342,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 
   // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
   // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
-  constexpr bool kAllRowsReal = (M % kGemmBM == 0);
+  constexpr bool kAllRowsReal = !DYN && (MS % kGemmBM == 0);
   const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
   // A fragments of row half rh (2 tiles of 16 rows), K half kh (64 bytes)
   auto readA = [&](int buf, int kh, int rh, v4i (&af)[kHM]) {
@@ -527,14 +533,13 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // first of the lane's four columns in column group q, and the row of accumulator v of row tile i inside the tile
   const long colBase = n0 + wn * kWaveCols + (TRANSB ? 4 * fragC : 16 * (fragC & 3) + (fragC & ~3));
   auto rowInTileOf = [&](int i, int v) { return static_cast<long>(wm * kWaveRows + i * 16 + fragG * 4 + v); };
-  if constexpr (KSPLIT > 1) {
-    constexpr long kPartRows = M < kGemmBM ? M : kGemmBM;            // rows of a tile that can hold results
-    constexpr long kCounterBytes = (kGridTiles * 4 + 255) / 256 * 256;
-    constexpr long kPartBytes = kPartRows * kGemmBN * static_cast<long>(sizeof(typename Mma::acc_t));
-    constexpr long kWsBytes = kCounterBytes + kTiles * KSPLIT * kPartBytes;
-    static_assert(kWsBytes < (1L << 31), "split-K workspace too large");
+  if (kSplitPossible && kSplits > 1) {
+    const long kPartRows = M < kGemmBM ? M : kGemmBM;            // rows of a tile that can hold results
+    const long kCounterBytes = (kGridTiles * 4 + 255) / 256 * 256;
+    const long kPartBytes = kPartRows * kGemmBN * static_cast<long>(sizeof(typename Mma::acc_t));
+    const long kWsBytes = kCounterBytes + kTiles * kSplits * kPartBytes;   // (below 2 GiB: checked by the host)
     const Buffer wsBuf = make_buffer(ws, kWsBytes);
-    const u32 tileBase = static_cast<u32>(kCounterBytes + linear * KSPLIT * kPartBytes);
+    const u32 tileBase = static_cast<u32>(kCounterBytes + linear * kSplits * kPartBytes);
     auto partOffset = [&](int i, int q, int v) {
       return static_cast<long>((rowInTileOf(i, v) * kGemmBN + (colBase + 64 * q - n0)) * static_cast<long>(sizeof(typename Mma::acc_t)));
     };
@@ -554,7 +559,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
       }
     }
     __shared__ unsigned akg_gemm_flag;
-    if (!last_workgroup(ws, linear, KSPLIT, tid, &akg_gemm_flag)) return;
+    if (!last_workgroup(ws, linear, kSplits, tid, &akg_gemm_flag)) return;
 #pragma unroll
     for (int q = 0; q < kTN / 4; ++q) {
       const long col4 = colBase + 64 * q;
@@ -566,7 +571,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
         for (int v = 0; v < 4; ++v) {
           if (!rowOk(i, v)) continue;
           typename Mma::acc_t sum[4] = {0, 0, 0, 0};
-          for (int p = 0; p < KSPLIT; ++p) {
+          for (int p = 0; p < kSplits; ++p) {
             typename Mma::acc_t part[4];
             ws_load_chunk<4>(wsBuf, tileBase + static_cast<u32>(p * kPartBytes + partOffset(i, q, v)), part);
 #pragma unroll
@@ -609,14 +614,19 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 // The four wavefronts add their accumulators through LDS (only the M real rows), the KSPLIT workgroups of a strip
 // through the workspace in split order (counter per strip, then M x 128 partials per strip and split), and the thread
 // that owns (row, 4 columns) runs the epilogue on the sums. Deterministic; B is read exactly once.
-template <typename Mma, long M, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT, int WAVES = 4, int UNROLL = 2, bool NT = false>
+// DYN: MS is the most rows the code object takes (16, 32 or 64), the actual row count and the number of K splits are
+// kernel arguments (`mDyn` <= MS, `ksDyn`); `ws` is always a valid pointer.
+template <typename Mma, long MS, long N, long KE, bool TRANSB, typename Epilogue, int KSPLIT, int WAVES = 4, int UNROLL = 2, bool NT = false, bool DYN = false>
 AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ Bv, Epilogue &epi,
-                         unsigned *__restrict__ ws, long group0) {
+                         unsigned *__restrict__ ws, long group0, long mDyn = 0, int ksDyn = 1) {
+  const long M = DYN ? mDyn : MS;
+  const int kSplits = DYN ? ksDyn : KSPLIT;
+  constexpr bool kSplitPossible = DYN || KSPLIT > 1;
   constexpr int EB = Mma::kElemBytes;
   constexpr long K = KE * EB;   // bytes of K per row of A
   constexpr long NB = N * EB;   // bytes per k-row of a row-major B
-  static_assert(M >= 1 && M <= 128, "at most 128 rows");
-  constexpr int kRowTiles = static_cast<int>((M + 31) / 32);   // MFMA tiles of 32 rows
+  static_assert(MS >= 1 && MS <= 128, "at most 128 rows");
+  constexpr int kRowTiles = static_cast<int>((MS + 31) / 32);   // MFMA tiles of 32 rows
   static_assert(K % 32 == 0, "K must be a multiple of 32 bytes");
   static_assert(TRANSB || N % 4 == 0, "N must be a multiple of 4");
   constexpr long kSteps = K / 32;
@@ -629,7 +639,7 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
   const int tid = static_cast<int>(threadIdx.x), lane = tid & 63, wave = tid >> 6;
   const long strip = static_cast<long>(blockIdx.x) % kStrips;   // neighbours in launch order read neighbouring columns
   const int ksplit = static_cast<int>(static_cast<long>(blockIdx.x) / kStrips);
-  const long t0 = kSteps * ksplit / KSPLIT, t1 = kSteps * (ksplit + 1) / KSPLIT;
+  const long t0 = kSteps * ksplit / kSplits, t1 = kSteps * (ksplit + 1) / kSplits;
   const int n32 = lane & 31, kg = lane >> 5;
   const long myCol = strip * 128 + 4 * n32;
   const long ldCol = myCol + 3 < N ? myCol : 0;   // columns beyond N: load something valid, the results are dropped
@@ -732,15 +742,15 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
 
   // ---- the four wavefronts' sums, rows below M only, 16 rows at a time: accumulator v of a lane is row
   // 8 (v / 4) + 4 g + v % 4; thread (c4, r0) then owns 4 columns of the strip and the rows r0, r0 + 8, ...
-  constexpr int kHalfRows = M < 16 ? static_cast<int>(M) : 16;
+  constexpr int kHalfRows = MS < 16 ? static_cast<int>(MS) : 16;
   __shared__ acc_t akg_skinny_sum[kWaves][kHalfRows][128];
   const int c4 = tid & 31, r0 = (tid >> 5) & 7;
   const long col = strip * 128 + 4 * c4;
   const bool colOk = col < N && tid < 256;   // (of 8 wavefronts the first four finish the sums)
-  constexpr int kRowsPerThread = (M + 7) / 8;
+  constexpr int kRowsPerThread = (MS + 7) / 8;
   acc_t sum[kRowsPerThread][4];
 #pragma unroll
-  for (int h = 0; h < (M + 15) / 16; ++h) {
+  for (int h = 0; h < (MS + 15) / 16; ++h) {
     if (h > 0) __syncthreads();
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
@@ -765,14 +775,14 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
       }
     }
   }
-  if constexpr (KSPLIT > 1) {
-    constexpr long kPartBytes = M * 128 * static_cast<long>(sizeof(acc_t));
+  if (kSplitPossible && kSplits > 1) {
+    const long kPartBytes = M * 128 * static_cast<long>(sizeof(acc_t));
     const long group = group0 + strip;
     // layout: [groups x 4 bytes of counters, rounded up to 256][group][split][M][128]
     const long groups = static_cast<long>(gridDim.y) * kStrips;
     const long counterBytes = (groups * 4 + 255) / 256 * 256;
-    const Buffer wsBuf = make_buffer(ws, counterBytes + groups * KSPLIT * kPartBytes);
-    const u32 base = static_cast<u32>(counterBytes + group * KSPLIT * kPartBytes);
+    const Buffer wsBuf = make_buffer(ws, counterBytes + groups * kSplits * kPartBytes);
+    const u32 base = static_cast<u32>(counterBytes + group * kSplits * kPartBytes);
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
       const int row = r0 + 8 * i;
@@ -781,7 +791,7 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
       }
     }
     __shared__ unsigned akg_skinny_flag;
-    if (!last_workgroup(ws, group, KSPLIT, tid, &akg_skinny_flag)) return;
+    if (!last_workgroup(ws, group, kSplits, tid, &akg_skinny_flag)) return;
     if (!colOk) return;
     epi.prepare(col);
 #pragma unroll
@@ -789,7 +799,7 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
       const int row = r0 + 8 * i;
       if (row >= M) continue;
       acc_t total[4] = {0, 0, 0, 0};
-      for (int p = 0; p < KSPLIT; ++p) {
+      for (int p = 0; p < kSplits; ++p) {
         acc_t part[4];
         ws_load_chunk<4>(wsBuf, base + static_cast<u32>(p * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))), part);
 #pragma unroll

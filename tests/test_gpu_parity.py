@@ -1424,6 +1424,55 @@ def test_profile_entry_point_returns_a_plausible_time():
     assert 0.0 < ms < 50.0
 
 
+@pytest.mark.parametrize("kind", ["int8_dequant_bias_gelu", "bf16_bias_gelu_tb"])
+def test_dynamic_matmul_shares_code_objects_across_token_counts(kind):
+    """A MatMul fusion whose row count (the token count) is open: the reference compiles such a kernel once and passes
+    sizes at call time (LLVMParameterPacking.cpp:91-194). Here M and the K split are kernel arguments of the tile kernel
+    (every M above 64: one code object, the split chosen per call) and of the skinny kernel (three sizes: up to 16, 32
+    and 64 rows), so a new token count costs a lowering and no device compilation. Results against the oracle of the
+    same description written with the bound M: int8 fusions to the bf16 bar with exact accumulators behind them, bf16 to
+    its bar."""
+    from oracle import np_ref
+    sentinel = 777
+    if kind == "int8_dequant_bias_gelu":
+        make = lambda m, name: op_desc.gemm_int8_dequant_bias_gelu(m, 2048, 1024, "bfloat16", False, name)   # noqa: E731
+    else:
+        make = lambda m, name: op_desc.gemm_bias_act(m, 2048, 1024, "bfloat16", "gelu", True, "float32", name)  # noqa: E731
+    open_desc = json_loads(make(sentinel, "dyn_" + kind))
+
+    def walk(x):
+        if isinstance(x, dict):
+            if "shape" in x:
+                x["shape"] = [-1 if n == sentinel else n for n in x["shape"]]
+            for v in x.values():
+                walk(v)
+        elif isinstance(x, list):
+            for v in x:
+                walk(v)
+    walk(open_desc)
+    dyn = driver.HipDynamicKernel(__import__("json").dumps(open_desc), out_dir=None)
+    compiled = {}
+    for m in (1000, 300, 2304, 65, 64, 48, 33, 32, 20, 16, 7, 2):
+        bound = json_loads(make(m, "dyn_" + kind))
+        shapes = [e[0]["shape"] for e in bound["input_desc"]]
+        kernel = dyn.specialize(shapes)
+        bucket = "tile" if m > 64 else ("skinny%d" % (16 if m <= 16 else 32 if m <= 32 else 64))
+        print("  M=%d: %s grid %d block %d, made in %.1f ms%s" % (m, bucket, kernel.grid[0], kernel.block[0], kernel.build_ms,
+                                                                " (no device compilation)" if kernel.cache_hit else ""), flush=True)
+        if bucket in compiled:
+            assert kernel.cache_hit and kernel.build_ms < 20.0, "M=%d compiled again (%s was built for M=%d)" % (m, bucket, compiled[bucket])
+        else:
+            compiled[bucket] = m
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 31 + m)
+        got = run_on_gpu(kernel, inputs)
+        expect = np_ref.evaluate(bound, inputs)
+        for d, g, e in zip(kernel.outputs, got, expect):
+            ok, msg = harness.compare(g, e, d.dtype)
+            print("    %s %s: %s" % (d.name, d.dtype, msg), flush=True)
+            assert ok, "M=%d output %s: %s" % (m, d.name, msg)
+    assert sorted(compiled) == ["skinny16", "skinny32", "skinny64", "tile"]
+
+
 @pytest.mark.parametrize("m,k,n,tb", [(512, 8192, 512, False), (4096, 8192, 8192, False), (4096, 8192, 8192, True),
                                       (1000, 4112, 1032, False), (48, 8192, 4096, False)])
 def test_bare_int8_matmul_accumulators_are_exact(m, k, n, tb):
