@@ -77,6 +77,9 @@ class TileEmitter {
     k.shapeArgs = lowering::buildShapeArgs(g_);
     if (extentArg_) k.scalarArgs.push_back(extentIsCols_ ? cols_ : rows_);
     if (colsArg_) k.scalarArgs.push_back(cols_);
+    if (dimsArg_) {
+      for (size_t d = 0; d + 1 < full_.size(); ++d) k.scalarArgs.push_back(full_[d]);
+    }
     std::ostringstream note;
     note << kernelFamilyName(k.family) << " rows=" << rows_ << " cols=" << cols_ << " vec=" << vec_
          << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
@@ -104,6 +107,10 @@ class TileEmitter {
   // length of the bucket shares the source and with it the code object.
   bool colsArg_ = false;
   bool allowColsArg_ = true;
+  // Dynamic descriptions with an operand that spans only some of the leading dimensions (an attention mask shared by
+  // the heads): the leading extents of the folded iteration space are kernel arguments too, and the operand's row
+  // offset is computed from them, so the source does not carry them as numbers.
+  bool dimsArg_ = false;
   int64_t bucketLow_ = 0, bucketHigh_ = 0;
   std::vector<InputAccess> access_;  // per graph input
   std::vector<ValInfo> vals_;        // per tensor
@@ -281,6 +288,18 @@ class TileEmitter {
   void pickSchedule() {
     extentArg_ = opt_.extentAsArgument;
     extentIsCols_ = extentArg_ && !rowMode_ && rows_ == 1;
+    dimsArg_ = false;
+    if (extentArg_ && !extentIsCols_ && full_.size() >= 3 && rows_ < (1LL << 31)) {
+      for (const InputAccess &a : access_) {
+        if (a.foldedShape.size() != full_.size()) continue;
+        bool allFull = true, allOne = true;
+        for (size_t d = 0; d + 1 < full_.size(); ++d) {
+          allFull = allFull && a.foldedShape[d] == full_[d];
+          allOne = allOne && a.foldedShape[d] == 1;
+        }
+        dimsArg_ = dimsArg_ || (!allFull && !allOne);
+      }
+    }
     useBuffers_ = true;
     for (int id : g_.inputs) {
       if (g_.tensor(id).numel() * static_cast<int64_t>(dtypeSize(g_.tensor(id).dtype)) >= (1LL << 31)) useBuffers_ = false;
@@ -437,7 +456,12 @@ class TileEmitter {
       if (block_ % 64 != 0 || block_ > 1024) block_ = 256;
       int chunks = opt_.chunks > 0 ? opt_.chunks : std::max(1, 16 / vec_);
       // Small problems: fewer chunks per thread so the grid still covers the chip.
-      while (chunks > 1 && ceilDiv(numel_, static_cast<int64_t>(block_) * vec_ * chunks) < 1024) chunks >>= 1;
+      if (extentArg_ && opt_.chunks == 0) {
+        // a dynamic description: two sizes only (the source must not follow every element count)
+        if (ceilDiv(numel_, static_cast<int64_t>(block_) * vec_ * chunks) < 1024) chunks = 1;
+      } else {
+        while (chunks > 1 && ceilDiv(numel_, static_cast<int64_t>(block_) * vec_ * chunks) < 1024) chunks >>= 1;
+      }
       chunks_ = std::max(1, chunks);
       tpr_ = block_;
       rowsPerBlock_ = 1;
@@ -540,6 +564,27 @@ class TileEmitter {
     const bool symbolic = colsArg_ && s[r - 1] == cols_ && cols_ != 1;
     const std::string inner = symbolic ? std::string("COLS") : std::to_string(s[r - 1]) + "L";
     if (allFull) return "(" + rowVar + " * " + inner + ")";
+    if (dimsArg_) {
+      // the same decomposition with the leading extents as kernel arguments (32-bit arithmetic: ROWS is below 2^31)
+      std::ostringstream e;
+      std::string div;          // product of the extents inside dim d, as an expression ("" = 1)
+      std::string own;          // product of the operand's own extents inside dim d
+      bool firstTerm = true;
+      for (int d = static_cast<int>(r) - 2; d >= 0; --d) {
+        const std::string dim = "akg_dim" + std::to_string(d);
+        if (s[static_cast<size_t>(d)] != 1) {
+          if (!firstTerm) e << " + ";
+          std::string idx = div.empty() ? "static_cast<unsigned>(" + rowVar + ")" : "(static_cast<unsigned>(" + rowVar + ") / (" + div + "))";
+          if (d > 0) idx = "(" + idx + " % " + dim + ")";
+          e << "static_cast<long>(" << idx << ")" << (own.empty() ? "" : " * static_cast<long>(" + own + ")");
+          firstTerm = false;
+          own = own.empty() ? dim : own + " * " + dim;
+        }
+        div = div.empty() ? dim : div + " * " + dim;
+      }
+      if (firstTerm) return "0L";
+      return "((" + e.str() + ") * " + inner + ")";
+    }
     // general leading-dim broadcast: decompose the row index over the leading dims
     std::vector<int64_t> stride(r, 0);
     int64_t acc = symbolic ? 1 : s[r - 1];
@@ -591,7 +636,15 @@ class TileEmitter {
     }
     if (extentArg_) src_ << ", const long akg_extent";
     if (colsArg_) src_ << ", const long akg_cols_arg";
+    if (dimsArg_) {
+      for (size_t d = 0; d + 1 < full_.size(); ++d) src_ << ", const long akg_dim_arg" << d;
+    }
     line(") {");
+    if (dimsArg_) {
+      for (size_t d = 0; d + 1 < full_.size(); ++d) {
+        src_ << "  const unsigned akg_dim" << d << " = static_cast<unsigned>(akg_dim_arg" << d << ");   // leading extent " << d << " of the iteration space\n";
+      }
+    }
     if (extentArg_ && extentIsCols_) {
       line("  constexpr long ROWS = 1L;");
       line("  const long COLS = akg_extent;   // everything folds into one dimension: the element count");
@@ -733,6 +786,13 @@ class TileEmitter {
     }
     const bool symbolicCols = colsArg_ && folded.back() == cols_ && cols_ != 1;
     if (leadOne && rows_ != 1) return symbolicCols ? "COLS * " + std::to_string(dtypeSize(t.dtype)) + "L" : number;
+    if (!leadFull && dimsArg_) {
+      std::string e = symbolicCols ? std::string("COLS") : std::to_string(folded.back()) + "L";
+      for (size_t d = 0; d + 1 < folded.size(); ++d) {
+        if (folded[d] != 1) e += " * static_cast<long>(akg_dim" + std::to_string(d) + ")";
+      }
+      return e + " * " + std::to_string(dtypeSize(t.dtype)) + "L";
+    }
     if (!leadFull) return number;
     if (symbolicCols) return "akg_extent * COLS * " + std::to_string(dtypeSize(t.dtype)) + "L";
     return "akg_extent * " + std::to_string(folded.back() * static_cast<int64_t>(dtypeSize(t.dtype))) + "L";

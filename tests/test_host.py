@@ -847,3 +847,40 @@ def test_cli_tool():
     r = subprocess.run([tool, "emit", os.path.join(
         REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")], capture_output=True, text=True)
     assert r.returncode == 1 and "error -3" in r.stderr
+
+
+def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
+    """What a new shape set of a dynamic description costs: a device compilation only when the source changes. The leading
+    extents (also of operands that span only some of them: a mask shared by the heads), the row count, the row length
+    inside its power-of-two bucket of chunk counts, the rows of A of a MatMul and its K split are kernel arguments; what
+    still makes a new source is a row length in another bucket and a chunk width that stops dividing the rows. Counted
+    on the shape sets the GPU tests use for the reference's ten dynamic descriptions (three each)."""
+    monkeypatch.setenv("AKG_HIP_NO_CACHE", "0")
+    shape_sets = {
+        "Fused_Cast_Sub_Mul_split_14802837530264465372": ([[[32, 1, 48, 48]], [[32, 1, 5, 1000]], [[32, 1, 48, 40]]], 1),
+        "Fused_RealDiv_split_4177286244677596212": ([[[32, 12, 24, 40], [32, 12, 24, 1]], [[32, 12, 7, 40], [32, 12, 7, 1]],
+                                                    [[32, 12, 24, 136], [32, 12, 24, 1]]], 1),
+        "Fused_ReduceMax_fusion_2054638663855723468": ([[[100, 768]], [[3, 768]], [[2048, 768]]], 1),
+        "Fused_ReduceMax_fusion_234578345729057892345": ([[[4096, 33]], [[4096, 4096]], [[4096, 40]]], 2),       # 33 / 40 and 4096: two buckets
+        "Fused_Sub_Mul_Cast_fusion_4217325526348104075": ([[[32, 16, 20, 64], [32, 16, 20, 1], [32, 16, 20, 64]],
+                                                          [[32, 16, 3, 64], [32, 16, 3, 1], [32, 16, 3, 64]],
+                                                          [[32, 16, 20, 72], [32, 16, 20, 1], [32, 16, 20, 72]]], 1),
+        "Fused_Sub_Mul_split_1454621004286351279": ([[[32, 1, 48, 48]], [[32, 1, 6, 48]], [[32, 1, 48, 520]]], 1),
+    }
+    for f in sorted(os.listdir(REF_INFO)):
+        stem = f.split(".info")[0]
+        if stem not in shape_sets:
+            continue
+        sets, allowed = shape_sets[stem]
+        dyn = driver.HipDynamicKernel(open(os.path.join(REF_INFO, f), encoding="utf-8").read(), out_dir=None)
+        compiled = sum(0 if dyn.specialize(shapes).cache_hit else 1 for shapes in sets)
+        assert compiled <= allowed, "%s: %d device compilations for three shape sets (%d allowed)" % (stem, compiled, allowed)
+    # an attention mask [32,1,S,T] against scores [32,12,S,T] with S and T open: one code object
+    # as long as the rows stay in one bucket (40 and 48 columns: 5 and 6 chunks of 8)
+    path = os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")
+    dyn = driver.HipDynamicKernel(open(path, encoding="utf-8").read(), out_dir=None)
+    first = dyn.specialize([[32, 1, 48, 48], [32, 12, 48, 48]])
+    assert "akg_dim_arg0" in first.source and "akg_dim_arg2" in first.source
+    for shapes in ([[32, 1, 40, 40], [32, 12, 40, 40]], [[32, 1, 9, 48], [32, 12, 9, 48]]):
+        k = dyn.specialize(shapes)
+        assert k.cache_hit and k.source == first.source, shapes
