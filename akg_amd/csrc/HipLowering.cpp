@@ -345,6 +345,76 @@ std::vector<bool> relaxedPrecisionTensors(const OpGraph &g) {
     const DType dt = g.tensors[t].dtype;
     relaxed[t] = demand[t] == 1 && (dt == DType::F32 || dt == DType::F16 || dt == DType::BF16);
   }
+  // The hardware tanh form 1 - 2 / (e^2x + 1) is the one approximation whose error is ABSOLUTE (1.2e-7 near zero, where
+  // the relative error is unbounded). Sums carry that error on; a product with a computed factor turns it into whatever
+  // the factor's magnitude makes of it. Harmless where the factor is tied to the tanh's own argument (GELU:
+  // x * (1 + tanh(f(x))) - a large x saturates the tanh, whose form is then exact); anywhere else the Tanh keeps the
+  // series-near-zero implementation, whose error is relative. Forward pass over the ops:
+  std::vector<std::vector<bool>> ancestors(n);       // per tensor: the tensors it is computed from (itself included)
+  std::vector<int> taint(n, -1);                     // per tensor: the relaxed Tanh op whose absolute error it carries
+  auto base = [&](int t) {
+    // the tensor behind constant factors, casts, sign flips and reshapes
+    for (;;) {
+      const TensorValue &tv = g.tensor(t);
+      if (tv.producer < 0) return t;
+      const OpNode &p = g.ops[static_cast<size_t>(tv.producer)];
+      int next = -1;
+      if (p.kind == OpKind::Cast || p.kind == OpKind::Neg || p.kind == OpKind::Reshape || p.kind == OpKind::BroadcastTo) {
+        next = p.inputs[0];
+      } else if ((p.kind == OpKind::Mul || p.kind == OpKind::Div) && p.inputs.size() == 2) {
+        if (g.tensor(p.inputs[1]).isConst) next = p.inputs[0];
+        else if (p.kind == OpKind::Mul && g.tensor(p.inputs[0]).isConst) next = p.inputs[1];
+      }
+      if (next < 0) return t;
+      t = next;
+    }
+  };
+  for (size_t t = 0; t < n; ++t) {
+    ancestors[t].assign(n, false);
+    ancestors[t][t] = true;
+  }
+  for (size_t k = 0; k < g.ops.size(); ++k) {
+    const OpNode &op = g.ops[k];
+    const size_t out = static_cast<size_t>(op.outputs[0]);
+    for (int in : op.inputs) {
+      for (size_t a = 0; a < n; ++a) ancestors[out][a] = ancestors[out][a] || ancestors[static_cast<size_t>(in)][a];
+    }
+    auto precise = [&](int tanhOp) { relaxed[static_cast<size_t>(g.ops[static_cast<size_t>(tanhOp)].outputs[0])] = false; };
+    switch (op.kind) {
+      case OpKind::Tanh:
+        if (relaxed[out]) taint[out] = static_cast<int>(k);
+        break;
+      case OpKind::Add: case OpKind::Sub: case OpKind::AddN: case OpKind::Neg: case OpKind::Reshape:
+      case OpKind::BroadcastTo: case OpKind::Cast: case OpKind::Select: case OpKind::Maximum: case OpKind::Minimum:
+      case OpKind::Abs:
+        for (int in : op.inputs) {
+          if (taint[static_cast<size_t>(in)] >= 0) taint[out] = taint[static_cast<size_t>(in)];
+        }
+        break;
+      case OpKind::Mul:
+      case OpKind::Div:
+        for (size_t i = 0; i < op.inputs.size() && op.inputs.size() == 2; ++i) {
+          const int tk = taint[static_cast<size_t>(op.inputs[i])];
+          if (tk < 0) continue;
+          const int other = op.inputs[1 - i];
+          const int arg = g.ops[static_cast<size_t>(tk)].inputs[0];
+          if (g.tensor(other).isConst && !(op.kind == OpKind::Div && i == 1)) {
+            taint[out] = tk;   // (constants of 1024 and more were answered above)
+          } else if (op.kind == OpKind::Mul && ancestors[static_cast<size_t>(arg)][static_cast<size_t>(base(other))]) {
+            // the factor is what the tanh's argument is made of: the product's error is relative from here on
+          } else {
+            precise(tk);
+          }
+        }
+        break;
+      default:
+        // anything else (Exp, Pow, Sqrt, a reduction ...) may amplify an absolute error near zero: keep the tanh relative
+        for (int in : op.inputs) {
+          if (taint[static_cast<size_t>(in)] >= 0) precise(taint[static_cast<size_t>(in)]);
+        }
+        break;
+    }
+  }
   return relaxed;
 }
 

@@ -884,3 +884,25 @@ def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
     for shapes in ([[32, 1, 40, 40], [32, 12, 40, 40]], [[32, 1, 9, 48], [32, 12, 9, 48]]):
         k = dyn.specialize(shapes)
         assert k.cache_hit and k.source == first.source, shapes
+
+
+def test_hardware_tanh_form_only_where_its_absolute_error_cannot_grow():
+    """Values that only reach 16-bit outputs may use hardware approximations. The tanh form 1 - 2 / (e^2x + 1) is the one
+    whose error is absolute (1.2e-7 near zero): it stays only where nothing can blow that up - GELU, whose factor x is what
+    the tanh's own argument is made of (a large x saturates the tanh exactly) - and gives way to the series-near-zero
+    implementation (relative error) behind a constant of 1024 and more or an unrelated computed factor."""
+    gelu = driver.HipKernel(op_desc.gemm_bias_act(64, 64, 64, "bfloat16", "gelu", False, "float32", "tanh_gelu"), out_dir=None)
+    assert "akg::fast_tanh(" in gelu.source and "akg::op_tanh(" not in gelu.source
+
+    def scaled(factor_is_input, constant):
+        b = op_desc.DescBuilder("tanh_scaled_%d_%d" % (int(factor_is_input), int(constant)))
+        x = b.cast(b.input([64, 256], "bfloat16"), "float32")
+        t = b.unary("Tanh", x)
+        f = b.cast(b.input([64, 256], "bfloat16"), "float32") if factor_is_input else b.const(constant, "float32")
+        return driver.HipKernel(b.dumps([b.cast(b.mul(t, f), "bfloat16")]), out_dir=None).source
+    assert "akg::fast_tanh(" in scaled(False, 8.0)
+    assert "akg::op_tanh(" in scaled(False, 4096.0) and "akg::fast_tanh(" not in scaled(False, 4096.0)
+    assert "akg::op_tanh(" in scaled(True, 0.0) and "akg::fast_tanh(" not in scaled(True, 0.0)
+    # a float32 output never sees an approximation
+    b = op_desc.DescBuilder("tanh_f32")
+    assert "akg::fast_tanh(" not in driver.HipKernel(b.dumps([b.unary("Tanh", b.input([64, 256], "float32"))]), out_dir=None).source
