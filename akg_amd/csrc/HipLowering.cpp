@@ -36,6 +36,7 @@ LoweringOptions LoweringOptions::fromEnvironment() {
   o.split = readInt("AKG_HIP_SPLIT");
   o.variant = readInt("AKG_HIP_VARIANT");
   if (const int cus = readInt("AKG_HIP_CUS"); cus >= 1 && cus <= 4096) o.computeUnits = cus;
+  o.matmulF32Acc = readInt("AKG_HIP_MATMUL_F32_ACC") == 1;
   if (const char *nt = std::getenv("AKG_HIP_NT")) o.nonTemporal = (nt[0] != '0') ? 1 : 0;
   return o;
 }

@@ -56,6 +56,11 @@ struct LoweringOptions {
   // Compute units of the part the kernels are made for (MI355X / MI350X: 256; AKG_HIP_CUS for another gfx950 part):
   // what persistent grids are sized by. The lowering runs without a device, so this is not asked of one.
   int computeUnits = 256;
+  // A MatMul whose declared result is float16 / bfloat16 accumulates in that type in the reference (product and sum
+  // rounded at every k), which only the serial kernel on the vector ALUs reproduces. AKG_HIP_MATMUL_F32_ACC=1 is the
+  // caller's explicit consent to the matrix units instead: float32 accumulation, ONE rounding to the declared type - more
+  // accurate than the reference's value and different from it (outside rtol 1e-2 from K = 64 on for N(0,1) data).
+  bool matmulF32Acc = false;
   // Dynamic-shape descriptions: the elementwise / row-reduction kernels take their row count (or, when everything
   // folds into one dimension, their element count) as a kernel argument instead of a constant, so that shape sets
   // that differ only there share one code object (the source no longer depends on them).

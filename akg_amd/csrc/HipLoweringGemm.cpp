@@ -96,6 +96,7 @@ class GemmEmitter {
       note << " tile=256x256x" << stepK() / elemBytes() << " mfma=" << mfmaName(true) << " waves=" << (tallWavefrontTiles() ? "2x4" : "4x2") << " grid=" << k.grid[0];
     }
     if (kSplit_ > 1) note << " k_splits=" << kSplit_;
+    if (roundedOnce_) note << " (AKG_HIP_MATMUL_F32_ACC: float32 accumulation rounded once to the declared 16-bit type, not the reference's per-step rounding)";
     if (dyn_) note << " (rows of A and K splits are kernel arguments: one code object for " << (skinny_ ? "up to " + std::to_string(skinnyBucket()) + " rows" : "more than 64 rows") << ")";
     k.scheduleNote = note.str();
     return k;
@@ -118,6 +119,7 @@ class GemmEmitter {
   bool dyn_ = false;
   int skinnyBucket() const { return m_ <= 16 ? 16 : (m_ <= 32 ? 32 : 64); }
   bool transB_ = false;
+  bool roundedOnce_ = false;   // a 16-bit declared MatMul result on the matrix units by the caller's switch
   int matmulOp_ = -1;
   int aId_ = -1, bId_ = -1, accId_ = -1;
   std::vector<EpiVal> vals_;
@@ -210,6 +212,9 @@ class GemmEmitter {
       elem_ = DType::I8;
     } else if ((a.dtype == DType::BF16 || a.dtype == DType::F16) && c.dtype == DType::F32) {
       elem_ = a.dtype;
+    } else if ((a.dtype == DType::BF16 || a.dtype == DType::F16) && c.dtype == a.dtype && opt_.matmulF32Acc) {
+      elem_ = a.dtype;   // the caller asked for the matrix units: float32 sum, rounded once (see LoweringOptions)
+      roundedOnce_ = true;
     } else {
       // linalg.matmul converts both operands to the accumulator's element type: the same type, a wider integer, or a
       // wider float

@@ -74,6 +74,9 @@ WORKLOADS = {
     # RMSNorm over the last axis (row family), alone and with the residual add in front (two outputs)
     "n10_rmsnorm_bf16_16384x4096": "f32",
     "n11_rmsnorm_add_bf16_16384x4096": "f32",
+    # a MatMul DECLARED bfloat16: the reference rounds product and sum to 16 bits at every k, which only a serial chain
+    # per result on the vector ALUs reproduces (bit-exact); this row shows what that rule costs against n2's float32 spelling
+    "n12_gemm_serial_bf16_declared_bf16_1024x1024x1024": "bf16",
 }
 # workloads also measured on the schedule of several kernels (AKG_HIP_VARIANT=7 while the handle is built)
 SEVERAL_KERNELS = ("n8_softmax_axis1_f16_32x21x512x512", "n9_layernorm_axis1_bf16_64x768x1024")

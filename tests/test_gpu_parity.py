@@ -1424,6 +1424,27 @@ def test_profile_entry_point_returns_a_plausible_time():
     assert 0.0 < ms < 50.0
 
 
+def test_sixteen_bit_matmul_on_the_matrix_units_by_switch(monkeypatch):
+    """AKG_HIP_MATMUL_F32_ACC=1: a MatMul declared bfloat16 runs on the MFMA kernel with a float32 sum rounded once. That is
+    not the reference's value (16-bit accumulation, which the default serial kernel reproduces bit for bit), so it is held
+    to the float64 product of the same bfloat16 operands within the bfloat16 bar."""
+    import torch
+    monkeypatch.setenv("AKG_HIP_MATMUL_F32_ACC", "1")
+    b = op_desc.DescBuilder("mm_bf16_f32acc")
+    a_t = b.input([300, 1024], "bfloat16")
+    w_t = b.input([1024, 520], "bfloat16")
+    kernel = driver.HipKernel(b.dumps([b.matmul(a_t, w_t, "bfloat16")]), out_dir=None)
+    assert "gemm_256x256" in kernel.source
+    rng = np.random.default_rng(5)
+    a = harness.f32_to_bf16_bits((rng.standard_normal((300, 1024)) * 0.25).astype(np.float32))
+    w = harness.f32_to_bf16_bits((rng.standard_normal((1024, 520)) * 0.25).astype(np.float32))
+    got = run_on_gpu(kernel, [a, w])[0]
+    want = torch.from_numpy(harness.bf16_bits_to_f32(a)).double() @ torch.from_numpy(harness.bf16_bits_to_f32(w)).double()
+    ok, msg = harness.compare(got, harness.f32_to_bf16_bits(want.float().numpy()), "bfloat16")
+    print("  float32 accumulation rounded once vs float64: %s" % msg, flush=True)
+    assert ok, msg
+
+
 @pytest.mark.parametrize("kind", ["int8_dequant_bias_gelu", "bf16_bias_gelu_tb"])
 def test_dynamic_matmul_shares_code_objects_across_token_counts(kind):
     """A MatMul fusion whose row count (the token count) is open: the reference compiles such a kernel once and passes

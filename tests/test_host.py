@@ -906,3 +906,18 @@ def test_hardware_tanh_form_only_where_its_absolute_error_cannot_grow():
     # a float32 output never sees an approximation
     b = op_desc.DescBuilder("tanh_f32")
     assert "akg::fast_tanh(" not in driver.HipKernel(b.dumps([b.unary("Tanh", b.input([64, 256], "float32"))]), out_dir=None).source
+
+
+def test_sixteen_bit_matmul_runs_on_the_matrix_units_only_by_explicit_switch(monkeypatch, tmp_path):
+    """A MatMul declared float16 / bfloat16 means 16-bit accumulation in the reference: the serial kernel by default (bit
+    for bit, slow). AKG_HIP_MATMUL_F32_ACC=1 is the caller's consent to float32 accumulation rounded once; the `schedule`
+    entry of `<k>.json` says which one runs."""
+    text = op_desc.gemm_bias_act(256, 512, 256, "bfloat16", "gelu", False, "bfloat16", "mm_declared_bf16")
+    k = driver.HipKernel(text, out_dir=str(tmp_path / "serial"))
+    meta = json.load(open(tmp_path / "serial" / "mm_declared_bf16.json"))
+    assert "akg::gemm_serial<" in k.source and "serial" in meta["schedule"]
+    monkeypatch.setenv("AKG_HIP_MATMUL_F32_ACC", "1")
+    k = driver.HipKernel(text, out_dir=str(tmp_path / "mfma"))
+    meta = json.load(open(tmp_path / "mfma" / "mm_declared_bf16.json"))
+    assert "akg::gemm_256x256<akg::MmaBF16" in k.source and "accr[e] = akg::bf16::rnd(acc[e])" in k.source
+    assert "AKG_HIP_MATMUL_F32_ACC" in meta["schedule"]
