@@ -58,6 +58,7 @@ struct akg_hip_kernel {
     hipEvent_t lastUse = nullptr;
     hipStream_t lastStream = nullptr;
     bool used = false;
+    bool recorded = false;   // lastUse was recorded behind the previous launch already (AKG_HIP_SAFE_STREAMS=1)
     // a launch sequence that failed half way may have left arrival counters set: zero-fill before the next launch
     bool dirty = false;
   };
@@ -702,7 +703,11 @@ struct WorkspaceTurn {
   }
   int begin() {
     if (!active) return AKG_HIP_OK;
-    if (l->used && l->lastStream != stream) {
+    if (l->used && l->lastStream != stream && l->recorded) {
+      // the previous launch left its event behind itself: the stream it went to is not touched again
+      const hipError_t e = hipStreamWaitEvent(stream, l->lastUse, 0);
+      if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipStreamWaitEvent: " + hipErr(e));
+    } else if (l->used && l->lastStream != stream) {
       // The event is recorded only now, at the switch of streams, behind everything enqueued on the previous stream so
       // far (an event after every launch would put a marker between back-to-back launches of the common one-stream
       // caller: 3 us on a 45 us reduction).
@@ -738,6 +743,13 @@ struct WorkspaceTurn {
     // also after a failure: what did get enqueued still uses the workspace
     l->lastStream = stream;
     l->used = true;
+    // AKG_HIP_SAFE_STREAMS=1: for callers that destroy streams between launches of one handle. The event goes behind
+    // every launch (≈3 us between back-to-back launches), and the next launch on another stream waits for it without
+    // ever touching this stream's handle again (which may be gone by then, or be another stream at the same address).
+    const char *safe = std::getenv("AKG_HIP_SAFE_STREAMS");
+    const bool safeStreams = safe != nullptr && safe[0] == '1';
+    l->recorded = false;
+    if (safeStreams && hipEventRecord(l->lastUse, stream) == hipSuccess) l->recorded = true;
     return rc;
   }
 };

@@ -126,8 +126,10 @@ int akg_hip_kernel_prepare(akg_hip_kernel_t *kernel);
  * pointer per argument, inputs then outputs. Asynchronous; after the first call on a device (or
  * akg_hip_kernel_prepare) it allocates nothing. Launches of one handle whose workspace_bytes is non-zero share
  * that workspace: the library keeps them apart on the device (a launch that goes to another stream than the handle's
- * previous one first waits, through an event, for what that stream holds), and zero-fills the workspace again in front
- * of the next launch if a launch sequence broke off half way. Launches recorded into a stream capture are ordered by
+ * previous one first waits, through an event recorded on that previous stream at the switch, for what it holds - so a
+ * stream must outlive the handle's next launch on another stream, or AKG_HIP_SAFE_STREAMS=1 must be set, which records
+ * the event behind every launch instead and never touches a stream after its launch), and zero-fills the workspace again
+ * in front of the next launch if a launch sequence broke off half way. Launches recorded into a stream capture are ordered by
  * the graph they become part of; two graphs replaying one handle at the same time are the caller's to keep apart.
  * Replaces the cuLaunchKernel
  * step of the generated shim (code_template.py:204) without its per-call context creation, module load,

@@ -778,6 +778,36 @@ def test_workspace_launches_from_two_streams_are_ordered_and_repeat_bit_for_bit(
     assert ok, msg
 
 
+def test_a_stream_destroyed_between_launches_of_one_handle(monkeypatch):
+    """AKG_HIP_SAFE_STREAMS=1: the event that orders launches of a handle with a workspace is recorded behind every
+    launch, so the library never touches a stream again after launching on it - the caller may destroy it. Launch on a
+    stream, destroy it while the work may still be running, launch on a second one: both results equal the first launch
+    of all (made on the default stream)."""
+    import ctypes
+    import torch
+    monkeypatch.setenv("AKG_HIP_SAFE_STREAMS", "1")
+    monkeypatch.setenv("AKG_HIP_SPLIT", "64")
+    hip = ctypes.CDLL("libamdhip64.so")
+    text = op_desc.square_reduce([8192, 1024], [0], "float32", False, "ReduceSum", "ws_stream_gone")
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.workspace_bytes > 0
+    x = harness.make_inputs(json_loads(text), seed=harness.BASE_SEED + 98)[0]
+    dev = torch.device("cuda:0")
+    xin = torch.from_numpy(x).to(dev)
+    outs = torch.full((5, kernel.outputs[0].nbytes), 0xFF, dtype=torch.uint8, device=dev)
+    kernel.launch_ptrs([xin.data_ptr(), outs[0].data_ptr()], torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    for i in range(1, 5):
+        stream = ctypes.c_void_p()
+        assert hip.hipStreamCreate(ctypes.byref(stream)) == 0
+        kernel.launch_ptrs([xin.data_ptr(), outs[i].data_ptr()], stream.value)
+        assert hip.hipStreamDestroy(stream) == 0      # asynchronous: the stream goes once its work has drained
+    torch.cuda.synchronize()
+    host = outs.cpu().numpy()
+    for i in range(1, 5):
+        assert np.array_equal(host[i], host[0]), "launch %d differs" % i
+
+
 def _run_with_inputs_back(kernel, inputs):
     """Like run_on_gpu, but also returns the device copies of the inputs after the launch (Assign writes over them)."""
     import torch
