@@ -724,7 +724,7 @@ def test_column_kernel_schedule():
     walk per reduction level, no workspace. Strips with a large footprint: one workgroup per CU walks several of them, the
     next strip's chunks on their way into a second set of registers while this one is worked on."""
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n9_layernorm_axis1_bf16_64x768x1024.info"), out_dir=None)
-    assert k.family == "column_reduce" and k.workspace_bytes == 0 and (k.grid[0], k.block[0]) == (256, 512)
+    assert k.family == "column_reduce" and k.workspace_bytes == 0 and (k.grid[0], k.block[0]) == (512, 512)   # 1024 strips: two workgroups a CU, two strips each
     assert "constexpr int V = 8, LX = 8, LY = 64, CH = 12, BLOCK = 512;" in k.source and "// ---- walk 2 ----" in k.source
     assert "constexpr long TOTAL = 1024;" in k.source
     assert k.source.count("akg::column_reduce<akg::RedSum, akg::f32, false, LX, BLOCK, V>") == 2
