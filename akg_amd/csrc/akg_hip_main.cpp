@@ -7,10 +7,19 @@
  *   akg-hip emit X.info                 print the emitted HIP source
  *   akg-hip compile X.info -o DIR       write <op>.hsaco, <op>.json, <op>_shape_arg.txt, <op>.hip to DIR
  *   akg-hip info X.info                 print signature, family, launch shape, algorithmic bytes
- *   akg-hip run X.info [-n N] [-r R]    what `akg_benchmark -e gpu -f X.info -p` does without the numeric compare
- *                                       (benchmark.py:94-130): seeded inputs, NaN-prefilled outputs, one call on host
- *                                       buffers, then R x N timed launches on device buffers; prints the time, the
- *                                       achieved bandwidth, the outputs' checksums and how many NaNs they hold
+ *   akg-hip run X.info [-n N] [-r R] [--inputs DIR] [--dump DIR] [--expect DIR]
+ *                                       what `akg_benchmark -e gpu -f X.info -p` does (benchmark.py:94-130): seeded
+ *                                       inputs, NaN-prefilled outputs, one call on host buffers, then R x N timed
+ *                                       launches on device buffers; prints the time, the achieved bandwidth, the
+ *                                       outputs' checksums and how many NaNs they hold.
+ *                                       The numeric compare of the reference's tool is split from the expectation's
+ *                                       maker, so that this binary links no CPU implementation of the operators:
+ *                                       --dump writes every argument as DIR/arg<i>.bin (raw little-endian elements,
+ *                                       inputs as given, outputs as computed), --inputs reads the inputs from such
+ *                                       files, --expect compares each output with DIR/arg<i>.bin (integers and bool
+ *                                       bit for bit; float32 within rtol 1e-5, float16 / bfloat16 within rtol 1e-2 and
+ *                                       atol 1e-3, float64 within rtol 1e-12; a NaN matches a NaN) and exits 1 on a
+ *                                       mismatch.
  */
 #include <hip/hip_runtime_api.h>
 
@@ -33,7 +42,8 @@ int usage() {
                "       akg-hip emit X.info\n"
                "       akg-hip compile X.info -o DIR\n"
                "       akg-hip info X.info\n"
-               "       akg-hip run X.info [-n launches per measurement] [-r measurements]\n");
+               "       akg-hip run X.info [-n launches per measurement] [-r measurements]\n"
+               "                          [--inputs DIR] [--dump DIR] [--expect DIR]\n");
   return 2;
 }
 
@@ -153,7 +163,88 @@ long long countNans(const akg_hip_tensor_desc &d, const std::vector<unsigned cha
   return nans;
 }
 
-int runKernel(akg_hip_kernel_t *k, int number, int repeat) {
+std::string argPath(const char *dir, int i) { return std::string(dir) + "/arg" + std::to_string(i) + ".bin"; }
+
+bool writeAll(const std::string &path, const std::vector<unsigned char> &bytes) {
+  std::ofstream f(path, std::ios::binary);
+  f.write(reinterpret_cast<const char *>(bytes.data()), static_cast<std::streamsize>(bytes.size()));
+  return static_cast<bool>(f);
+}
+
+float halfValue(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+  const int exp = (h >> 10) & 0x1F;
+  const uint32_t man = h & 0x3FFu;
+  float f;
+  if (exp == 0) {
+    f = static_cast<float>(man) * 0x1p-24f;   // subnormal or zero
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    u |= sign;
+    std::memcpy(&f, &u, 4);
+    return f;
+  }
+  const uint32_t u = sign | (exp == 31 ? 0x7F800000u : static_cast<uint32_t>(exp - 15 + 127) << 23) | (man << 13);
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+// Element `i` of a float tensor as a double (float16 / bfloat16 / float32 / float64).
+double floatAt(const char *t, const unsigned char *base, size_t i) {
+  if (std::strcmp(t, "float64") == 0) {
+    double v;
+    std::memcpy(&v, base + i * 8, 8);
+    return v;
+  }
+  if (std::strcmp(t, "float32") == 0) {
+    float v;
+    std::memcpy(&v, base + i * 4, 4);
+    return v;
+  }
+  uint16_t h;
+  std::memcpy(&h, base + i * 2, 2);
+  if (std::strcmp(t, "float16") == 0) return halfValue(h);
+  const uint32_t u = static_cast<uint32_t>(h) << 16;
+  float v;
+  std::memcpy(&v, &u, 4);
+  return v;
+}
+
+// How many elements of output `d` differ from the expectation by more than the type's tolerance; the
+// first one is described in *first. Integers and bool compare bit for bit.
+long long countMismatches(const akg_hip_tensor_desc &d, const std::vector<unsigned char> &got,
+                          const std::vector<unsigned char> &want, std::string *first) {
+  const char *t = dtypeName(d.dtype);
+  const bool isFloat = std::strncmp(t, "float", 5) == 0 || std::strcmp(t, "bfloat16") == 0;
+  const size_t esize = std::strstr(t, "64") ? 8 : std::strstr(t, "32") ? 4 : std::strstr(t, "16") ? 2 : 1;
+  const size_t n = got.size() / esize;
+  long long bad = 0;
+  for (size_t i = 0; i < n; ++i) {
+    bool same;
+    char what[160];
+    if (isFloat) {
+      const double a = floatAt(t, got.data(), i), b = floatAt(t, want.data(), i);
+      const double rtol = esize == 2 ? 1e-2 : esize == 4 ? 1e-5 : 1e-12, atol = esize == 2 ? 1e-3 : 0.0;
+      const double mag = b < 0 ? -b : b, diff = a > b ? a - b : b - a;
+      same = (a != a && b != b) || a == b || diff <= atol + rtol * mag;
+      if (!same) std::snprintf(what, sizeof what, "element %zu: got %.9g, expected %.9g", i, a, b);
+    } else {
+      same = std::memcmp(got.data() + i * esize, want.data() + i * esize, esize) == 0;
+      if (!same) {
+        int64_t a = 0, b = 0;
+        std::memcpy(&a, got.data() + i * esize, esize);
+        std::memcpy(&b, want.data() + i * esize, esize);
+        std::snprintf(what, sizeof what, "element %zu: got 0x%llx, expected 0x%llx", i,
+                      static_cast<unsigned long long>(a), static_cast<unsigned long long>(b));
+      }
+    }
+    if (!same && bad++ == 0) *first = what;
+  }
+  return bad;
+}
+
+int runKernel(akg_hip_kernel_t *k, int number, int repeat, const char *inputsDir, const char *dumpDir,
+              const char *expectDir) {
   akg_hip_kernel_info info;
   int n = 0;
   if (akg_hip_kernel_get_info(k, &info) != AKG_HIP_OK || akg_hip_kernel_num_tensors(k, &n) != AKG_HIP_OK) return 1;
@@ -165,6 +256,14 @@ int runKernel(akg_hip_kernel_t *k, int number, int repeat) {
     const akg_hip_tensor_desc &d = descs[static_cast<size_t>(i)];
     if (d.is_output) {
       host[static_cast<size_t>(i)].assign(static_cast<size_t>(d.bytes), 0xFF);   // all-ones is a NaN in every float type
+    } else if (inputsDir != nullptr) {
+      std::string raw;
+      if (!readAll(argPath(inputsDir, i).c_str(), &raw) || static_cast<int64_t>(raw.size()) != d.bytes) {
+        std::fprintf(stderr, "akg-hip: %s must hold the %lld bytes of input %s\n", argPath(inputsDir, i).c_str(),
+                     static_cast<long long>(d.bytes), d.name);
+        return 1;
+      }
+      host[static_cast<size_t>(i)].assign(raw.begin(), raw.end());
     } else {
       fillInput(d, 20260000ull + static_cast<uint64_t>(i), &host[static_cast<size_t>(i)]);
     }
@@ -206,7 +305,36 @@ int runKernel(akg_hip_kernel_t *k, int number, int repeat) {
     std::printf("output %-12s %-9s fnv1a %016llx  nans %lld\n", d.name, dtypeName(d.dtype),
                 static_cast<unsigned long long>(h), countNans(d, host[static_cast<size_t>(i)]));
   }
-  return 0;
+  if (dumpDir != nullptr) {
+    for (int i = 0; i < n; ++i) {
+      if (!writeAll(argPath(dumpDir, i), host[static_cast<size_t>(i)])) {
+        std::fprintf(stderr, "akg-hip: cannot write %s\n", argPath(dumpDir, i).c_str());
+        return 1;
+      }
+    }
+  }
+  int status = 0;
+  if (expectDir != nullptr) {
+    for (int i = 0; i < n; ++i) {
+      const akg_hip_tensor_desc &d = descs[static_cast<size_t>(i)];
+      if (!d.is_output) continue;
+      std::string raw, first;
+      if (!readAll(argPath(expectDir, i).c_str(), &raw) || static_cast<int64_t>(raw.size()) != d.bytes) {
+        std::fprintf(stderr, "akg-hip: %s must hold the %lld bytes expected of output %s\n",
+                     argPath(expectDir, i).c_str(), static_cast<long long>(d.bytes), d.name);
+        return 1;
+      }
+      const std::vector<unsigned char> want(raw.begin(), raw.end());
+      const long long bad = countMismatches(d, host[static_cast<size_t>(i)], want, &first);
+      if (bad == 0) {
+        std::printf("compare %-12s ok\n", d.name);
+      } else {
+        std::printf("compare %-12s MISMATCH in %lld elements, first %s\n", d.name, bad, first.c_str());
+        status = 1;
+      }
+    }
+  }
+  return status;
 }
 
 }  // namespace
@@ -215,9 +343,12 @@ int main(int argc, char **argv) {
   if (argc < 3) return usage();
   const std::string cmd = argv[1];
   const char *path = argv[2];
-  const char *outDir = nullptr;
+  const char *outDir = nullptr, *inputsDir = nullptr, *dumpDir = nullptr, *expectDir = nullptr;
   int number = 10, repeat = 5;
   for (int i = 3; i + 1 < argc; ++i) {
+    if (std::strcmp(argv[i], "--inputs") == 0) inputsDir = argv[i + 1];
+    if (std::strcmp(argv[i], "--dump") == 0) dumpDir = argv[i + 1];
+    if (std::strcmp(argv[i], "--expect") == 0) expectDir = argv[i + 1];
     if (std::strcmp(argv[i], "-o") == 0) outDir = argv[i + 1];
     if (std::strcmp(argv[i], "-n") == 0) number = std::atoi(argv[i + 1]);
     if (std::strcmp(argv[i], "-r") == 0) repeat = std::atoi(argv[i + 1]);
@@ -246,7 +377,7 @@ int main(int argc, char **argv) {
     return 1;
   }
   if (cmd == "run") {
-    rc = runKernel(k, number, repeat);
+    rc = runKernel(k, number, repeat, inputsDir, dumpDir, expectDir);
     akg_hip_kernel_destroy(k);
     return rc;
   }

@@ -695,6 +695,46 @@ def test_cli_runs_a_description_on_the_gpu():
     assert p.returncode == 1 and "cannot read" in p.stderr
 
 
+def test_cli_compares_against_expectations_made_elsewhere(tmp_path):
+    """`akg-hip run --dump / --inputs / --expect`: the numeric compare of the reference's akg_benchmark
+    (benchmark.py:94-130) with the expectation computed outside the tool. The tool's own seeded inputs are dumped,
+    the oracle evaluates the description on them, and the tool, given those inputs again, accepts the oracle's
+    outputs and rejects them once one element is changed."""
+    import subprocess
+    tool = os.path.join(ROOT, "akg_amd", "akg-hip")
+    for fixture in ("small_softmax_f16_64x4096.info", "small_quant_int8_residual_bf16_37x1544.info",
+                    "small_ew_tanh_add_mul_f32_7x33.info"):
+        path = os.path.join(FIXTURES, fixture)
+        dump, want = tmp_path / (fixture + ".dump"), tmp_path / (fixture + ".want")
+        dump.mkdir()
+        want.mkdir()
+        p = subprocess.run([tool, "run", path, "-n", "1", "-r", "1", "--dump", str(dump)], capture_output=True, text=True,
+                           timeout=120)
+        assert p.returncode == 0, p.stderr
+        kernel = driver.HipKernel.from_file(path)
+        n_in = len(kernel.inputs)
+        inputs = [np.fromfile(str(dump / ("arg%d.bin" % i)), dtype=driver.NP_HOST_DTYPE[d.dtype]).reshape(d.shape)
+                  for i, d in enumerate(kernel.inputs)]
+        expect = cpu_ref.CpuKernel(path, openmp=False)(inputs)
+        for j, e in enumerate(expect):
+            np.ascontiguousarray(e).tofile(str(want / ("arg%d.bin" % (n_in + j))))
+        cmd = [tool, "run", path, "-n", "1", "-r", "1", "--inputs", str(dump), "--expect", str(want)]
+        p = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+        assert p.returncode == 0, p.stdout + p.stderr
+        assert p.stdout.count("compare ") == len(expect) and "MISMATCH" not in p.stdout, p.stdout
+        # one element off by far more than any bar (the top exponent bit of a float, bit 6 of an int8): the tool
+        # counts it and exits 1
+        raw = bytearray((want / ("arg%d.bin" % n_in)).read_bytes())
+        esize = np.dtype(driver.NP_HOST_DTYPE[kernel.outputs[0].dtype]).itemsize
+        raw[(len(raw) // esize // 2) * esize + esize - 1] ^= 0x40
+        (want / ("arg%d.bin" % n_in)).write_bytes(bytes(raw))
+        p = subprocess.run(cmd, capture_output=True, text=True, timeout=120)
+        assert p.returncode == 1 and "MISMATCH in 1 elements" in p.stdout, p.stdout + p.stderr
+    p = subprocess.run([tool, "run", os.path.join(FIXTURES, "small_softmax_f16_64x4096.info"), "--inputs",
+                        str(tmp_path / "nowhere")], capture_output=True, text=True, timeout=60)
+    assert p.returncode == 1 and "must hold" in p.stderr
+
+
 @pytest.mark.parametrize("name", FULL)
 def test_full_size_config_matches_oracle(name):
     # the full sizes of the measured configurations; the oracle runs its OpenMP build (same per-row arithmetic, rows in parallel)
