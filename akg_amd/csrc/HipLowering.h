@@ -63,7 +63,8 @@ struct LoweringOptions {
   bool matmulF32Acc = false;
   // Dynamic-shape descriptions: the elementwise / row-reduction kernels take their row count (or, when everything
   // folds into one dimension, their element count) as a kernel argument instead of a constant, so that shape sets
-  // that differ only there share one code object (the source no longer depends on them).
+  // that differ only there share one code object (the source no longer depends on them). Likewise the rows of A of
+  // a MatMul, the outermost reduced extent of a streaming reduction and the batch of the column kernel.
   bool extentAsArgument = false;
   static LoweringOptions fromEnvironment();
 };

@@ -61,9 +61,11 @@ class ColumnEmitter {
     k.block[0] = static_cast<unsigned>(block_);
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
+    if (dynOuter_) k.scalarArgs.push_back(outer_);
     std::ostringstream note;
     note << "column_reduce outer=" << outer_ << " run=" << run_ << " inner=" << inner_ << " vec=" << vec_ << " threads=" << ly_ << "x" << lx_
          << " rows/thread=" << chunks_ << " walks=" << (maxLevel_ + 1) << (pipelined_ ? " strips pipelined" : "");
+    if (dynOuter_) note << " (the outer extent is a kernel argument)";
     k.scheduleNote = note.str();
     return k;
   }
@@ -84,6 +86,9 @@ class ColumnEmitter {
   int64_t strips_ = 1;
   bool pipelined_ = false;         // workgroups stay and walk several strips, the next strip's loads issued before the work on this one
   int64_t launched_ = 0;           // workgroups launched
+  // A description with open extents: the extent in front of the reduced axis (the batch) is a kernel argument. Nothing
+  // else in the source depends on it but the choice between one strip per workgroup and persistent workgroups.
+  bool dynOuter_ = false;
   bool aligned_ = true;            // every chunk starts at a multiple of its size and lies inside its row
   int reduceCount_ = 0;
   bool ordered_ = false;           // some reduction is a float16 / bfloat16 sum or product: steps in index order
@@ -265,6 +270,7 @@ class ColumnEmitter {
     pipelined_ = !ordered_ && opt_.variant != 5 && regs >= 40 && regs <= 64 && block_ == 512 && outer_ * strips_ >= 2 * kCUs;
     // (two such workgroups per CU where every one still gets two strips and more: 45.0 -> 43.5 us on the shape above)
     launched_ = pipelined_ ? (outer_ * strips_ >= 4 * kCUs ? 2 * kCUs : kCUs) : outer_ * strips_;
+    dynOuter_ = opt_.extentAsArgument && outer_ > 1;
   }
 
   void line(const std::string &s) { src_ << s << "\n"; }
@@ -383,10 +389,16 @@ class ColumnEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i) {
       src_ << ", " << dtypeTag(g_.tensor(g_.outputs[i]).dtype) << "::storage *__restrict__ out" << i;
     }
+    if (dynOuter_) src_ << ", const long akg_outer_arg";
     src_ << ") {\n";
     src_ << "  constexpr int V = " << vec_ << ", LX = " << lx_ << ", LY = " << ly_ << ", CH = " << chunks_ << ", BLOCK = " << block_ << ";\n";
     src_ << "  constexpr long RUN = " << run_ << ", INNER = " << inner_ << ", STRIPS = " << strips_ << ";\n";
-    src_ << "  constexpr long TOTAL = " << outer_ * strips_ << ";   // strips in all\n";
+    if (dynOuter_) {
+      line("  const long TOTAL = akg_outer_arg * STRIPS;   // strips in all");
+      line("  (void)TOTAL;");
+    } else {
+      src_ << "  constexpr long TOTAL = " << outer_ * strips_ << ";   // strips in all\n";
+    }
     if (block_ > 64) line("  __shared__ __attribute__((aligned(16))) unsigned char akg_scratch[2][(BLOCK / 64) * LX * V * 8];");
     if (ordered_) {
       // the rows of one step of an ordered reduction, in their 16-bit type, and the folded results per column

@@ -68,10 +68,12 @@ class StreamReduceEmitter {
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
     k.workspaceBytes = workspaceBytes_;
+    if (dynR_) k.scalarArgs = {R_, rps_, static_cast<int64_t>(split_)};
     std::ostringstream note;
     note << "stream_reduce direction=" << (dirY_ ? "Y" : "X") << " outer=" << O_ << " reduced=" << R_ << " inner=" << I_
          << " vec=" << vec_ << ((overlapTail_ || overlapRun_) ? " (overlapping last chunk)" : "") << " lanes=" << lanes_ << " split=" << split_ << " rows_per_split=" << rps_
          << " block=" << kBlock << " grid=" << grid_ << " workspace=" << workspaceBytes_;
+    if (dynR_) note << " (reduced extent, rows per split and split are kernel arguments)";
     k.scheduleNote = note.str();
     return k;
   }
@@ -113,6 +115,12 @@ class StreamReduceEmitter {
   // over workgroups or thread-rows. Direction Y: one thread per V columns walks the whole reduced extent. Direction
   // X: the workgroup streams tiles of BLOCK * V elements through LDS and its first thread folds them in order.
   bool ordered_ = false;
+  // A description with open extents whose reduced extent is the outermost one of the iteration space ([tokens, hidden]
+  // summed over the tokens, a whole tensor folded into one number): that extent, the share of it a workgroup walks
+  // and the number of workgroups sharing a result are kernel arguments, so the source does not depend on them and
+  // every such extent runs on one code object. The workspace is then always passed (its layout follows the split).
+  bool dynR_ = false;
+  int dynDim_ = -1;   // the dim of space_ that is the reduced extent
   std::vector<bool> relaxed_;
   std::vector<std::string> ident_;  // per tensor: array / scalar name once defined
 
@@ -273,6 +281,16 @@ class StreamReduceEmitter {
       if (kind_[d] == 2) I_ *= space_[d];
     }
     dirY_ = I_ > 1;
+    if (opt_.extentAsArgument && O_ == 1) {
+      int reducedDims = 0;
+      for (size_t d = 0; d < n; ++d) {
+        if (kind_[d] == 1) {
+          ++reducedDims;
+          dynDim_ = static_cast<int>(d);
+        }
+      }
+      dynR_ = reducedDims == 1 && R_ < (1LL << 31);
+    }
 
     // phases by data flow: Post = depends on a reduction result. Values computed only from constants and from kernel
     // inputs that do not vary along the reduced axes (running statistics, per-channel scales) belong to neither: they
@@ -413,9 +431,10 @@ class StreamReduceEmitter {
     };
     for (int id : g_.inputs) allBuffers = allBuffers && !tooLargeForBuffer(id);
     for (int id : g_.outputs) allBuffers = allBuffers && !tooLargeForBuffer(id);
+    if (!allBuffers) dynR_ = false;   // (tensors beyond 2 GiB are addressed without descriptors, by constants)
     if (dirY_ && allBuffers && opt_.vec == 0 && fastExtent == I_ && (I_ % v) != 0 && I_ >= 2 * v) {
       overlapTail_ = true;
-    } else if (!dirY_ && !ordered_ && allBuffers && opt_.vec == 0 && (fastExtent % v) != 0 && fastExtent >= 2 * v && R_ < (1LL << 30)) {
+    } else if (!dirY_ && !ordered_ && !dynR_ && allBuffers && opt_.vec == 0 && (fastExtent % v) != 0 && fastExtent >= 2 * v && R_ < (1LL << 30)) {
       overlapRun_ = true;
       runLength_ = fastExtent;
       runChunks_ = ceilDivL(fastExtent, v);
@@ -496,7 +515,7 @@ class StreamReduceEmitter {
     if (grid_ > 2147483647LL) throw LoweringError("grid too large");
     // Runs shorter than a few cache lines that do not end on line boundaries ([N,C,7,7]: 98 bytes per channel and
     // image): the lines are shared with the neighbouring outputs' runs.
-    xcdContiguous_ = !dirY_ && scatteredR && grid_ >= 64 &&
+    xcdContiguous_ = !dirY_ && !dynR_ && scatteredR && grid_ >= 64 &&
                      (fastExtent * static_cast<int64_t>(widest)) % 128 != 0 && fastExtent * static_cast<int64_t>(widest) < 2048;
     // workspace: one arrival counter per group, then the partials of every reduction
     workspaceBytes_ = 0;
@@ -513,6 +532,7 @@ class StreamReduceEmitter {
       workspaceBytes_ = off;
       if (workspaceBytes_ >= (1ULL << 31)) throw LoweringError("workspace of the streaming reduction exceeds 2 GiB");
     }
+    if (dynR_) workspaceBytes_ = std::max<uint64_t>(workspaceBytes_, 256);   // the kernel always takes the pointer
   }
 
   // ------------------------------------------------------------------ addressing
@@ -709,7 +729,8 @@ class StreamReduceEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
-    if (split_ > 1) src_ << (argc ? ", " : "") << "unsigned *__restrict__ akg_ws";
+    if (dynR_) src_ << (argc ? ", " : "") << "const long akg_r_arg, const long akg_rps_arg, const long akg_split_arg";
+    if (split_ > 1 || dynR_) src_ << (argc ? ", " : "") << "unsigned *__restrict__ akg_ws";
     line(") {");
     useBuffers_ = true;
     auto tooLarge = [&](int id) {
@@ -717,25 +738,36 @@ class StreamReduceEmitter {
     };
     for (int id : g_.inputs) useBuffers_ = useBuffers_ && !tooLarge(id);
     for (int id : g_.outputs) useBuffers_ = useBuffers_ && !tooLarge(id);
+    // bytes of a tensor: a constant, or (the reduced extent being an argument) that extent times the bytes per index
+    auto bytesOf = [&](const TensorValue &t) {
+      const int64_t bytes = t.numel() * static_cast<int64_t>(dtypeSize(t.dtype));
+      if (dynR_ && t.used && padTo(t.shape, "tensor " + t.name)[static_cast<size_t>(dynDim_)] != 1) {
+        return "akg_r_arg * " + std::to_string(bytes / R_) + "L";
+      }
+      return std::to_string(bytes) + "L";
+    };
     if (useBuffers_) {
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
-        const TensorValue &t = g_.tensor(g_.inputs[i]);
-        src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", "
-             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+        src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", " << bytesOf(g_.tensor(g_.inputs[i])) << ");\n";
       }
       for (size_t i = 0; i < g_.outputs.size(); ++i) {
-        const TensorValue &t = g_.tensor(g_.outputs[i]);
-        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", "
-             << t.numel() * static_cast<int64_t>(dtypeSize(t.dtype)) << "L);\n";
+        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", " << bytesOf(g_.tensor(g_.outputs[i])) << ");\n";
       }
     }
     src_ << "  constexpr int V = " << vec_ << ";\n";
     src_ << "  constexpr int BLOCK = " << kBlock << ";\n";
     src_ << "  constexpr int LANES = " << lanes_ << ";\n";
-    src_ << "  constexpr long O = " << O_ << "L, R = " << R_ << "L, I = " << I_ << "L;\n";
-    src_ << "  constexpr long STRIPS = " << strips_ << "L;\n";
-    src_ << "  constexpr int SPLIT = " << split_ << ";\n";
-    src_ << "  constexpr long RPS = " << rps_ << "L;\n";
+    if (dynR_) {
+      src_ << "  constexpr long O = " << O_ << "L, I = " << I_ << "L;\n";
+      src_ << "  constexpr long STRIPS = " << strips_ << "L;\n";
+      line("  const long R = akg_r_arg, RPS = akg_rps_arg;");
+      line("  const int SPLIT = static_cast<int>(akg_split_arg);");
+    } else {
+      src_ << "  constexpr long O = " << O_ << "L, R = " << R_ << "L, I = " << I_ << "L;\n";
+      src_ << "  constexpr long STRIPS = " << strips_ << "L;\n";
+      src_ << "  constexpr int SPLIT = " << split_ << ";\n";
+      src_ << "  constexpr long RPS = " << rps_ << "L;\n";
+    }
     line("  (void)O; (void)I; (void)STRIPS;");
     line("  const int tid = static_cast<int>(threadIdx.x);");
     if (!dirY_ && xcdContiguous_) {
@@ -865,6 +897,23 @@ class StreamReduceEmitter {
     line("}");
   }
 
+  // Where the partials of reduction k start in the workspace: a constant, or (the split being an argument) computed
+  // from it the way pickSchedule lays the workspace out. `partialOffsetExpr(reduces_.size())` is the workspace's size.
+  void emitPartialOffsets(const std::string &indent) {
+    if (!dynR_) return;
+    const uint64_t width = dirY_ ? static_cast<uint64_t>(lanes_) * vec_ : 1;
+    src_ << indent << "const unsigned akg_po0 = " << (static_cast<uint64_t>(groups_) * 4 + 255) / 256 * 256 << "u;\n";
+    for (size_t k = 0; k < reduces_.size(); ++k) {
+      const uint64_t ctSize = std::max<size_t>(4, dtypeSize(g_.tensor(reduces_[k]->outputs[0]).dtype));
+      src_ << indent << "const unsigned akg_po" << k + 1 << " = (akg_po" << k << " + " << static_cast<uint64_t>(groups_) * width * ctSize
+           << "u * static_cast<unsigned>(SPLIT) + 255u) / 256u * 256u;\n";
+    }
+  }
+  std::string partialOffsetExpr(size_t k) const {
+    if (dynR_) return "akg_po" + std::to_string(k);
+    return std::to_string(partialOffset_[k]) + (dirY_ ? "u" : "UL");
+  }
+
   // Sum of the TR thread-rows of the workgroup into thread-row 0 (fixed order), through LDS.
   void emitRowCombineY(const std::string &ldsPrefix) {
     line("  if (TR > 1) {");
@@ -896,14 +945,20 @@ class StreamReduceEmitter {
       src_ << "  __shared__ " << computeTypeName(od) << " akg_lds" << k << "[TR > 1 ? TR : 1][LANES * V];\n";
     }
     emitRowCombineY("akg_lds");
-    if (split_ > 1) {
+    if (split_ > 1 || dynR_) {
       line("  // ---- partials of this workgroup -> workspace; the last workgroup of the group to arrive finishes the job");
-      src_ << "  const akg::Buffer b_ws = akg::make_buffer(akg_ws, " << workspaceBytes_ << "L);\n";
+      if (dynR_) line("  if (SPLIT > 1) {");
+      emitPartialOffsets("  ");
+      if (dynR_) {
+        src_ << "  const akg::Buffer b_ws = akg::make_buffer(akg_ws, static_cast<long>(" << partialOffsetExpr(reduces_.size()) << "));\n";
+      } else {
+        src_ << "  const akg::Buffer b_ws = akg::make_buffer(akg_ws, " << workspaceBytes_ << "L);\n";
+      }
       for (size_t k = 0; k < reduces_.size(); ++k) {
         const DType od = g_.tensor(reduces_[k]->outputs[0]).dtype;
         const uint64_t ctSize = std::max<size_t>(4, dtypeSize(od));
         // byte offset of partial slot 0 of this lane; slot p is p * LANES * V elements further
-        src_ << "  const unsigned part" << k << " = " << partialOffset_[k] << "u + static_cast<unsigned>((akg_group * "
+        src_ << "  const unsigned part" << k << " = " << partialOffsetExpr(k) << " + static_cast<unsigned>((akg_group * "
              << "(static_cast<long>(SPLIT) * LANES * V) + li * V) * " << ctSize << "L);\n";
         src_ << "  if (tr == 0) akg::ws_store_chunk<V>(b_ws, part" << k << " + static_cast<unsigned>(akg_s) * (LANES * V * "
              << ctSize << "u), acc" << k << ");\n";
@@ -929,6 +984,7 @@ class StreamReduceEmitter {
         line("  }");
       }
       emitRowCombineY("akg_lds");
+      if (dynR_) line("  }");
     }
     // ---- post phase: thread-row 0 holds the reduced values of its V columns
     line("  if (tr != 0 || !col_ok) return;");
@@ -952,13 +1008,15 @@ class StreamReduceEmitter {
       if (lowering::reduceSpec(*reduces_[k], g_.tensor(reduces_[k]->outputs[0]).dtype).ordered) continue;
       blockReduce(k, "acc" + std::to_string(k));
     }
-    if (split_ > 1) {
+    if (split_ > 1 || dynR_) {
       line("  // ---- partial of this workgroup -> workspace; the last workgroup of the group to arrive finishes the job");
+      if (dynR_) line("  if (SPLIT > 1) {");
+      emitPartialOffsets("  ");
       line("  unsigned char *akg_wsb = reinterpret_cast<unsigned char *>(akg_ws);");
       for (size_t k = 0; k < reduces_.size(); ++k) {
         const std::string ct = computeTypeName(g_.tensor(reduces_[k]->outputs[0]).dtype);
-        src_ << "  " << ct << " *part" << k << " = reinterpret_cast<" << ct << " *>(akg_wsb + " << partialOffset_[k]
-             << "UL) + akg_group * SPLIT;\n";
+        src_ << "  " << ct << " *part" << k << " = reinterpret_cast<" << ct << " *>(akg_wsb + " << partialOffsetExpr(k)
+             << ") + akg_group * SPLIT;\n";
         src_ << "  if (tid == 0) akg::ws_store(part" << k << " + akg_s, acc" << k << ");\n";
       }
       line("  __shared__ unsigned akg_flag;");
@@ -969,6 +1027,7 @@ class StreamReduceEmitter {
         src_ << "  acc" << k << " = (tid < SPLIT) ? akg::ws_load(part" << k << " + tid) : " << spec.init << ";\n";
         blockReduce(k, "acc" + std::to_string(k));
       }
+      if (dynR_) line("  }");
     }
     emitPost(true);
   }

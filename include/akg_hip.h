@@ -191,8 +191,10 @@ void akg_hip_free_string(char *text);
  * akg_hip_dynamic_specialize binds the -1s to the given input shapes, derives every op's result shape, lowers the
  * kernel for these shapes and returns its handle. Elementwise and row-reduction kernels take the product of their
  * leading dimensions and their row length as kernel arguments (the schedule is made for the power-of-two bucket of
- * 16-byte chunks the row falls into), so shape sets that differ only there share one code object and the second
- * one needs no device compilation; anything else compiles once per shape set (or is found in the artifact directory). The handle is owned by the dynamic object (do not destroy it); it is
+ * 16-byte chunks the row falls into), MatMul fusions the rows of A and their K split, streaming reductions over the
+ * outermost extent that extent and their split, the column kernel the batch in front of its reduced axis: shape sets
+ * that differ only there share one code object and the second one needs no device compilation; anything else compiles
+ * once per shape set (or is found in the artifact directory). The handle is owned by the dynamic object (do not destroy it); it is
  * launched with akg_hip_launch like any other, and akg_hip_kernel_tensor reports the concrete output shapes.
  */
 typedef struct akg_hip_dynamic akg_hip_dynamic_t;

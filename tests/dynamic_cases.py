@@ -1,0 +1,64 @@
+"""Descriptions with one open extent (spelled -1) for the tests of kernels that take extents as arguments: made from a
+static builder called with a sentinel extent, which is then opened everywhere it occurs."""
+import json
+
+from akg_amd import op_desc
+
+
+def open_extent(text, sentinel):
+    """The description `text` with every extent equal to `sentinel` spelled -1 (an open extent)."""
+    d = json.loads(text)
+
+    def walk(x):
+        if isinstance(x, dict):
+            if "shape" in x:
+                x["shape"] = [-1 if n == sentinel else n for n in x["shape"]]
+            for v in x.values():
+                walk(v)
+        elif isinstance(x, list):
+            for v in x:
+                walk(v)
+    walk(d)
+    return json.dumps(d)
+
+
+DYNAMIC_STREAMS = {
+    # two float32 column sums of one pass over two bf16 operands (the gradient of a scale and a bias over the tokens)
+    "biasgrad_bf16": lambda t, name: op_desc.bias_grad(t, 1024, "bfloat16", name),
+    # a column maximum over rows the 16-byte chunks do not divide (the last chunk of a row overlaps its neighbour)
+    "colmax_f16": lambda t, name: op_desc.square_reduce([t, 1001], [0], "float16", False, "ReduceMax", name),
+    # a whole tensor into one number: sum of squares (float32)
+    "sqsum_all_f32": lambda t, name: op_desc.square_reduce([t, 512], [0, 1], "float32", False, "ReduceSum", name),
+}
+
+
+def _norm_absmax_all(t, name):
+    # two reductions of a whole tensor with an op behind one of them: its Euclidean norm and its absolute maximum
+    b = op_desc.DescBuilder(name)
+    x = b.input([t, 384], "float32")
+    norm = b.unary("Sqrt", b.reduce("ReduceSum", b.mul(x, x), [0, 1], False))
+    return b.dumps([norm, b.reduce("ReduceMax", b.unary("Abs", x), [0, 1], False)])
+
+
+DYNAMIC_STREAMS["norm_absmax_all_f32"] = _norm_absmax_all
+
+
+def _declared_half_colsum(t, name):
+    b = op_desc.DescBuilder(name)
+    return b.dumps([b.reduce("ReduceSum", b.input([t, 192], "float16"), [0], False)])
+
+
+def _declared_bf16_sum_all(t, name):
+    b = op_desc.DescBuilder(name)
+    return b.dumps([b.reduce("ReduceSum", b.input([t, 64], "bfloat16"), [0, 1], False)])
+
+
+# sums declared in a 16-bit type: one serial chain per result in index order, whatever the extent
+DYNAMIC_STREAMS["declared_f16_colsum"] = _declared_half_colsum
+DYNAMIC_STREAMS["declared_bf16_sum_all"] = _declared_bf16_sum_all
+
+
+DYNAMIC_COLUMNS = {
+    "softmax_classes_f16": lambda n, name: op_desc.softmax_over_axis([n, 21, 32, 48], 1, "float16", name),
+    "layernorm_channels_bf16": lambda n, name: op_desc.layernorm_over_axis1(n, 96, 520, "bfloat16", name=name),
+}

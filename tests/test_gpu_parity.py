@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 
 from akg_amd import driver, harness, op_desc
+from dynamic_cases import DYNAMIC_COLUMNS, DYNAMIC_STREAMS, open_extent
 from oracle import cpu_ref
 
 pytestmark = pytest.mark.gpu
@@ -1492,6 +1493,81 @@ def test_profile_entry_point_returns_a_plausible_time():
     bufs = [torch.zeros(t.nbytes, dtype=torch.uint8, device="cuda:0") for t in kernel.tensors]
     ms = kernel.profile_ptrs([b.data_ptr() for b in bufs], number=5, repeat=3)
     assert 0.0 < ms < 50.0
+
+
+@pytest.mark.parametrize("kind", sorted(DYNAMIC_STREAMS))
+def test_dynamic_streaming_reductions_share_one_code_object_across_reduced_extents(kind):
+    """A reduction over the outermost extent of its operand (column sums over the tokens, a whole tensor into one number)
+    with that extent open: the reference compiles such a kernel once and passes sizes at call time
+    (LLVMParameterPacking.cpp:91-194). Here the reduced extent, the share of it a workgroup walks and the number of
+    workgroups that share a result are kernel arguments: one code object for every extent, the split chosen per call
+    (one workgroup per result for the short extents, several hundred for the long ones). Float32 sums against
+    the float64 evaluation (they are reassociated), everything else against the oracle; 16-bit declared sums bit for
+    bit. Every handle is launched twice (the arrival counters must be left at zero)."""
+    from oracle import np_ref
+    make = DYNAMIC_STREAMS[kind]
+    sentinel = 7777
+    dyn = driver.HipDynamicKernel(open_extent(make(sentinel, "dyn_" + kind), sentinel), out_dir=None)
+    first = None
+    for t in (6000, 40, 16384, 7, 1000, 2):
+        bound = json_loads(make(t, "dyn_" + kind))
+        shapes = [e[0]["shape"] for e in bound["input_desc"]]
+        kernel = dyn.specialize(shapes)
+        print("  %s T=%d: %s grid %d block %d, made in %.1f ms%s" % (kind, t, kernel.family, kernel.grid[0], kernel.block[0], kernel.build_ms,
+                                                                      " (no device compilation)" if kernel.cache_hit else ""), flush=True)
+        assert kernel.family == "stream_reduce" and "akg_r_arg" in kernel.source
+        if first is None:
+            first = kernel.source
+        else:
+            assert kernel.cache_hit and kernel.source == first, "T=%d made a new source" % t
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 77 + t)
+        expect = np_ref.evaluate(bound, inputs)
+        wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+        exact = np_ref.evaluate(harness.widen_to_float64(bound), wide)
+        in_numel = max(int(np.prod(s)) for s in shapes)
+        for launch in range(2):
+            got = run_on_gpu(kernel, inputs)
+            for j, (d, g, e, x) in enumerate(zip(kernel.outputs, got, expect, exact)):
+                float_sum = kind in ("biasgrad_bf16", "sqsum_all_f32") or (kind == "norm_absmax_all_f32" and j == 0)
+                if kind.startswith("declared"):
+                    ok, msg = harness.compare_bits(g, e, d.dtype)
+                elif float_sum:
+                    ok, msg = harness.compare_reassociated(g, x, d.dtype, max(1, in_numel // max(1, g.size)))
+                else:
+                    ok, msg = harness.compare(g, e, d.dtype)
+                print("    launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
+                assert ok, "%s T=%d output %s: %s" % (kind, t, d.name, msg)
+
+
+@pytest.mark.parametrize("kind", sorted(DYNAMIC_COLUMNS))
+def test_dynamic_column_kernels_share_one_code_object_across_batch_sizes(kind):
+    """A softmax over the classes of [N,21,H,W] and a LayerNorm over the channels of [N,C,HW] with the batch open: the
+    extent in front of the reduced axis is a kernel argument of the column kernel, so every batch size above one runs
+    on one code object (LLVMParameterPacking.cpp:91-194: the reference passes sizes at call time). 16-bit results
+    against the oracle."""
+    from oracle import np_ref
+    make = DYNAMIC_COLUMNS[kind]
+    sentinel = 7777
+    dyn = driver.HipDynamicKernel(open_extent(make(sentinel, "dyn_" + kind), sentinel), out_dir=None)
+    first = None
+    for n in (6, 2, 40, 3):
+        bound = json_loads(make(n, "dyn_" + kind))
+        shapes = [e[0]["shape"] for e in bound["input_desc"]]
+        kernel = dyn.specialize(shapes)
+        print("  %s N=%d: %s grid %d block %d, made in %.1f ms%s" % (kind, n, kernel.family, kernel.grid[0], kernel.block[0], kernel.build_ms,
+                                                                      " (no device compilation)" if kernel.cache_hit else ""), flush=True)
+        assert kernel.family == "column_reduce" and "akg_outer_arg" in kernel.source
+        if first is None:
+            first = kernel.source
+        else:
+            assert kernel.cache_hit and kernel.source == first, "N=%d made a new source" % n
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 88 + n)
+        expect = np_ref.evaluate(bound, inputs)
+        got = run_on_gpu(kernel, inputs)
+        for d, g, e in zip(kernel.outputs, got, expect):
+            ok, msg = harness.compare(g, e, d.dtype)
+            print("    %s %s: %s" % (d.name, d.dtype, msg), flush=True)
+            assert ok, "%s N=%d output %s: %s" % (kind, n, d.name, msg)
 
 
 def test_sixteen_bit_matmul_on_the_matrix_units_by_switch(monkeypatch):

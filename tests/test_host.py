@@ -886,6 +886,34 @@ def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
         assert k.cache_hit and k.source == first.source, shapes
 
 
+def test_streaming_and_column_kernels_take_their_open_extent_as_an_argument(monkeypatch):
+    """Reductions over the outermost extent of their operand (column sums over the tokens, a whole tensor into one number)
+    and reductions over one inner axis with the batch in front of it: that extent is a kernel argument (with the split
+    of the streaming kernel, which the host chooses per call), so a new extent costs a lowering and no device
+    compilation. The grid and the workspace still follow the extent."""
+    import json
+    from dynamic_cases import DYNAMIC_COLUMNS, DYNAMIC_STREAMS, open_extent
+    monkeypatch.setenv("AKG_HIP_NO_CACHE", "0")
+    for cases, family, arg, extents in ((DYNAMIC_STREAMS, "stream_reduce", "akg_r_arg", (6000, 40, 16384, 7)),
+                                        (DYNAMIC_COLUMNS, "column_reduce", "akg_outer_arg", (6, 2, 40))):
+        for kind, make in sorted(cases.items()):
+            dyn = driver.HipDynamicKernel(open_extent(make(7777, "dynhost_" + kind), 7777), out_dir=None)
+            seen = []
+            for t in extents:
+                bound = json.loads(make(t, "dynhost_" + kind))
+                k = dyn.specialize([e[0]["shape"] for e in bound["input_desc"]])
+                assert k.family == family and arg in k.source, (kind, t, k.family)
+                seen.append(k)
+            assert all(k.source == seen[0].source for k in seen), kind
+            assert all(k.cache_hit for k in seen[1:]), kind
+            if family == "stream_reduce" and not kind.startswith("declared"):
+                # one workgroup per strip of columns for the short extent, hundreds for the long one
+                assert seen[2].grid[0] > seen[1].grid[0], (kind, seen[1].grid, seen[2].grid)
+                assert seen[2].workspace_bytes > seen[1].workspace_bytes >= 256
+            if family == "column_reduce":
+                assert seen[2].grid[0] == 20 * seen[1].grid[0]
+
+
 def test_hardware_tanh_form_only_where_its_absolute_error_cannot_grow():
     """Values that only reach 16-bit outputs may use hardware approximations. The tanh form 1 - 2 / (e^2x + 1) is the one
     whose error is absolute (1.2e-7 near zero): it stays only where nothing can blow that up - GELU, whose factor x is what
