@@ -110,6 +110,10 @@ const std::vector<std::string> &compileFlags() {
     std::vector<std::string> f = {
       "--offload-arch=gfx950", "-O3",      "-std=c++17",     "-ffp-contract=off",
       "-Xclang",               "-target-feature", "-Xclang", "-packed-fp32-ops",
+      // No SLP vectorisation: with packed float32 operations switched off, a two-lane float32 subtraction it forms
+      // next to 16-bit conversions has ended instruction selection with a fatal error (which ends the calling
+      // process), and the measured kernels run the same without it (every figure within its run-to-run spread).
+      "-fno-slp-vectorize",
     };
     // AKG_HIP_EXTRA_FLAGS: space-separated extra device-compiler flags (experiments; part of the cache key)
     if (const char *extra = std::getenv("AKG_HIP_EXTRA_FLAGS")) {
@@ -176,6 +180,11 @@ int compileToCodeObject(const akg::LoweredKernel &k, std::vector<char> *code, st
     headerNames.push_back(akg::kernel_lib::kHeaderNames[i]);
   }
   std::string progName = k.kernelName + ".hip";
+  // AKG_HIP_DUMP_SOURCE=DIR: every source goes to DIR/<kernel>.hip before the device compiler sees it (the compiler
+  // ends the process on an internal error; the source that did it is then on disk)
+  if (const char *dumpDir = std::getenv("AKG_HIP_DUMP_SOURCE")) {
+    if (dumpDir[0] != 0 && makeDirs(dumpDir)) writeFile(std::string(dumpDir) + "/" + progName, k.source.data(), k.source.size());
+  }
   hiprtcResult r = hiprtcCreateProgram(&prog, k.source.c_str(), progName.c_str(), static_cast<int>(headerTexts.size()),
                                        headerTexts.data(), headerNames.data());
   if (r != HIPRTC_SUCCESS) {

@@ -6,13 +6,14 @@ from akg_amd import op_desc
 
 
 def open_extent(text, sentinel):
-    """The description `text` with every extent equal to `sentinel` spelled -1 (an open extent)."""
+    """The description `text` with every extent equal to `sentinel` (one number or several) spelled -1 (an open extent)."""
     d = json.loads(text)
+    sentinels = tuple(sentinel) if isinstance(sentinel, (tuple, list)) else (sentinel,)
 
     def walk(x):
         if isinstance(x, dict):
             if "shape" in x:
-                x["shape"] = [-1 if n == sentinel else n for n in x["shape"]]
+                x["shape"] = [-1 if n in sentinels else n for n in x["shape"]]
             for v in x.values():
                 walk(v)
         elif isinstance(x, list):
@@ -61,4 +62,33 @@ DYNAMIC_STREAMS["declared_bf16_sum_all"] = _declared_bf16_sum_all
 DYNAMIC_COLUMNS = {
     "softmax_classes_f16": lambda n, name: op_desc.softmax_over_axis([n, 21, 32, 48], 1, "float16", name),
     "layernorm_channels_bf16": lambda n, name: op_desc.layernorm_over_axis1(n, 96, 520, "bfloat16", name=name),
+}
+
+
+def _pool_over_tokens(b_, t, name):
+    # [batch, tokens, hidden] float16 summed over the tokens in float32, batch and tokens both open
+    b = op_desc.DescBuilder(name)
+    x = b.cast(b.input([b_, t, 136], "float16"), "float32")
+    return b.dumps([b.reduce("ReduceSum", x, [1], False), b.reduce("ReduceMax", x, [1], False)])
+
+
+def _scaled_pool_over_tokens(b_, t, name):
+    # the same with operands that span only some of the extents: a weight per token and a bias per batch entry
+    b = op_desc.DescBuilder(name)
+    x = b.input([b_, t, 64], "float32")
+    w = b.input([1, t, 1], "float32")
+    c = b.input([b_, 1, 64], "float32")
+    return b.dumps([b.add(b.reduce("ReduceSum", b.mul(x, w), [1], True), c)])
+
+
+# (outer extent, reduced extent) both open: [O, R, I] reduced over R
+DYNAMIC_POOLS = {
+    "pool_f16": _pool_over_tokens,
+    "scaled_pool_f32": _scaled_pool_over_tokens,
+}
+
+# the batch of [N,C,H,W] statistics open: the reduced extent N * H * W is an argument, the channel extent lies between
+DYNAMIC_STATS = {
+    "bnstats_bf16_16x16": lambda n, name: op_desc.batchnorm_stats(n, 24, 16, 16, "bfloat16", name),
+    "bnstats_f32_7x7": lambda n, name: op_desc.batchnorm_stats(n, 40, 7, 7, "float32", name),
 }

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 from akg_amd import driver, harness, op_desc
-from dynamic_cases import DYNAMIC_COLUMNS, DYNAMIC_STREAMS, open_extent
+from dynamic_cases import DYNAMIC_COLUMNS, DYNAMIC_POOLS, DYNAMIC_STATS, DYNAMIC_STREAMS, open_extent
 from oracle import cpu_ref
 
 pytestmark = pytest.mark.gpu
@@ -1537,6 +1537,54 @@ def test_dynamic_streaming_reductions_share_one_code_object_across_reduced_exten
                     ok, msg = harness.compare(g, e, d.dtype)
                 print("    launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
                 assert ok, "%s T=%d output %s: %s" % (kind, t, d.name, msg)
+
+
+@pytest.mark.parametrize("kind", sorted(DYNAMIC_POOLS) + sorted(DYNAMIC_STATS))
+def test_dynamic_streaming_reductions_behind_an_open_batch(kind):
+    """[batch, tokens, hidden] reduced over the tokens with batch and tokens both open (what a batch index advances by is
+    then computed from the token count in the kernel), also with operands that span only some of the extents; and the
+    per-channel statistics of [N,C,H,W] with the batch open (the reduced extent N * H * W is the argument, the channels
+    lie between the reduced extents; 7 x 7 images keep their overlapping chunks). One code object per description, up to
+    the choice of the workgroup numbering for small grids. Float32 sums against the float64 evaluation, the maxima
+    against the oracle; two launches per handle."""
+    from oracle import np_ref
+    sources = set()
+    if kind in DYNAMIC_POOLS:
+        make = DYNAMIC_POOLS[kind]
+        dyn = driver.HipDynamicKernel(open_extent(make(7777, 5555, "dyn_" + kind), (7777, 5555)), out_dir=None)
+        bounds = [json_loads(make(b, t, "dyn_" + kind)) for b, t in ((4, 300), (32, 64), (2, 5000), (7, 9), (1, 700))]
+        arg = "akg_o_arg"
+    else:
+        make = DYNAMIC_STATS[kind]
+        dyn = driver.HipDynamicKernel(open_extent(make(7777, "dyn_" + kind), 7777), out_dir=None)
+        bounds = [json_loads(make(n, "dyn_" + kind)) for n in (8, 256, 3, 64)]
+        arg = "akg_r_arg"
+    for bound in bounds:
+        shapes = [e[0]["shape"] for e in bound["input_desc"]]
+        kernel = dyn.specialize(shapes)
+        print("  %s %s: %s grid %d block %d, made in %.1f ms%s" % (kind, shapes[0], kernel.family, kernel.grid[0], kernel.block[0], kernel.build_ms,
+                                                                    " (no device compilation)" if kernel.cache_hit else ""), flush=True)
+        assert kernel.family == "stream_reduce"
+        if shapes[0][0] > 1:
+            assert arg in kernel.source
+            sources.add(kernel.source)
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 99 + shapes[0][0])
+        expect = np_ref.evaluate(bound, inputs)
+        wide = [a.astype(np.float64) if a.dtype == np.float32 else a for a in inputs]
+        exact = np_ref.evaluate(harness.widen_to_float64(bound), wide)
+        in_numel = max(int(np.prod(sh)) for sh in shapes)
+        is_max = [o["name"] == "ReduceMax" for o in bound["op_desc"] if o["output_desc"][0]["tensor_name"] in
+                  [x["tensor_name"] for x in bound["output_desc"]]]
+        for launch in range(2):
+            got = run_on_gpu(kernel, inputs)
+            for j, (d, g, e, x) in enumerate(zip(kernel.outputs, got, expect, exact)):
+                if j < len(is_max) and is_max[j]:
+                    ok, msg = harness.compare(g, e, d.dtype)
+                else:
+                    ok, msg = harness.compare_reassociated(g, x, d.dtype, max(1, in_numel // max(1, g.size)))
+                print("    launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
+                assert ok, "%s %s output %s: %s" % (kind, shapes[0], d.name, msg)
+    assert len(sources) <= (2 if kind in DYNAMIC_STATS else 1), "%d sources" % len(sources)
 
 
 @pytest.mark.parametrize("kind", sorted(DYNAMIC_COLUMNS))

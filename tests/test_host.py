@@ -912,6 +912,21 @@ def test_streaming_and_column_kernels_take_their_open_extent_as_an_argument(monk
                 assert seen[2].workspace_bytes > seen[1].workspace_bytes >= 256
             if family == "column_reduce":
                 assert seen[2].grid[0] == 20 * seen[1].grid[0]
+    # batch and tokens of [batch, tokens, hidden] both open: the batch is a fourth argument and the stride of a batch
+    # index is computed from the token count
+    from dynamic_cases import DYNAMIC_POOLS, DYNAMIC_STATS
+    for kind, make in sorted(DYNAMIC_POOLS.items()):
+        dyn = driver.HipDynamicKernel(open_extent(make(7777, 5555, "dynhost_" + kind), (7777, 5555)), out_dir=None)
+        seen = [dyn.specialize([e[0]["shape"] for e in json.loads(make(b, t, "dynhost_" + kind))["input_desc"]])
+                for b, t in ((4, 300), (32, 64), (2, 5000))]
+        assert all(k.family == "stream_reduce" and "akg_o_arg" in k.source and "akg_o * (R * " in k.source for k in seen), kind
+        assert all(k.source == seen[0].source for k in seen) and all(k.cache_hit for k in seen[1:]), kind
+    # the batch of [N,C,H,W] statistics: N * H * W is the argument, the buffer sizes follow N
+    for kind, make in sorted(DYNAMIC_STATS.items()):
+        dyn = driver.HipDynamicKernel(open_extent(make(7777, "dynhost_" + kind), 7777), out_dir=None)
+        seen = [dyn.specialize([e[0]["shape"] for e in json.loads(make(n, "dynhost_" + kind))["input_desc"]]) for n in (8, 3, 32)]
+        assert all(k.family == "stream_reduce" and "akg_r_arg" in k.source for k in seen), kind
+        assert all(k.source == seen[0].source for k in seen) and all(k.cache_hit for k in seen[1:]), kind
 
 
 def test_hardware_tanh_form_only_where_its_absolute_error_cannot_grow():
