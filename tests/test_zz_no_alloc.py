@@ -117,6 +117,30 @@ def test_static_scratch_launch_equals_the_allocating_launch(first, second):
                 assert np.array_equal(g, w), "%s round %d: buffer %d differs from akg_hip_launch's" % (name, round_no, idx)
 
 
+def test_static_scratch_launch_of_kernels_that_take_their_extents_as_arguments():
+    """Specialisations of a dynamic description: the streaming reduction's kernel takes its reduced extent and its split
+    as arguments behind the tensor pointers and always takes the scratch pointer, also when one workgroup per result
+    needs no exchange (the second, smaller shape set). Same outputs through both entry points, two rounds."""
+    import json
+    from dynamic_cases import DYNAMIC_STREAMS, open_extent
+    make = DYNAMIC_STREAMS["biasgrad_bf16"]
+    dyn = driver.HipDynamicKernel(open_extent(make(7777, "dyn_noalloc"), 7777), out_dir=None)
+    cases = []
+    for t in (6000, 40):
+        bound = json.loads(make(t, "dyn_noalloc"))
+        kernel = dyn.specialize([e[0]["shape"] for e in bound["input_desc"]])
+        assert kernel.workspace_bytes > 0 and "akg_r_arg" in kernel.source
+        kernel.prepare()
+        cases.append((t, kernel, harness.make_inputs(bound, seed=harness.BASE_SEED + 4300 + t)))
+    expected = [_run(k, i, static=False) for _, k, i in cases]
+    for round_no in range(2):
+        for (t, kernel, inputs), want in zip(cases, expected):
+            print("case T=%d round %d" % (t, round_no), flush=True)
+            got = _run(kernel, inputs, static=True)
+            for idx, (g, w) in enumerate(zip(got, want)):
+                assert np.array_equal(g, w), "T=%d round %d: buffer %d differs from akg_hip_launch's" % (t, round_no, idx)
+
+
 def test_static_scratch_launch_needs_a_prepared_handle_and_refuses_oversized_scratch():
     path = os.path.join(FIXTURES, "small_reduceall_sqsum_f32_768x512.info")
     kernel = driver.HipKernel.from_file(path)
