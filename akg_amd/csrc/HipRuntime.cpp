@@ -41,7 +41,8 @@
 struct akg_hip_kernel {
   akg::OpGraph graph;
   akg::LoweredKernel lowered;
-  std::vector<char> codeObject;
+  // (shared between the handles that were made from one source: the specialisations of a dynamic description)
+  std::shared_ptr<const std::vector<char>> codeObject;
   std::string codeSha256;
   bool cacheHit = false;
   double buildMs = 0.0;   // wall time of translation, lowering and (unless cached) device compilation of this handle
@@ -77,7 +78,16 @@ struct akg_hip_kernel {
 // description is specialised to shape sets that its kernel takes as an argument, and when one description is compiled
 // twice).
 std::mutex g_codeCacheMutex;
-std::map<std::string, std::vector<char>> g_codeCache;
+std::map<std::string, std::shared_ptr<const std::vector<char>>> g_codeCache;
+
+// Code objects loaded on a device, by the digest of the code object: handles made from one source (every token count
+// of a dynamic MatMul is a handle of its own) share one module instead of loading a copy each.
+struct SharedModule {
+  hipModule_t module = nullptr;
+  long refs = 0;
+};
+std::mutex g_moduleMutex;
+std::map<std::pair<std::string, int>, SharedModule> g_modules;
 
 // A dynamic-shape description and the kernels specialised from it so far, keyed by the bound input shapes.
 struct akg_hip_dynamic {
@@ -526,7 +536,7 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
         akg::json::Value mv = akg::json::Value::parse(meta);
         if (mv.contains("source_sha256") && mv.at("source_sha256").asString() == srcDigest &&
             mv.contains("sha256") && mv.at("sha256").asString() == akg::Sha256::of(code)) {
-          k->codeObject.assign(code.begin(), code.end());
+          k->codeObject = std::make_shared<const std::vector<char>>(code.begin(), code.end());
           k->codeSha256 = mv.at("sha256").asString();
           k->cacheHit = true;
         }
@@ -542,7 +552,7 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
     if (it != g_codeCache.end()) {
       k->codeObject = it->second;
       akg::Sha256 h;
-      h.update(k->codeObject.data(), k->codeObject.size());
+      h.update(k->codeObject->data(), k->codeObject->size());
       k->codeSha256 = h.hexDigest();
       k->cacheHit = true;
       fromMemory = true;
@@ -550,7 +560,12 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
   }
   if (!k->cacheHit || (fromMemory && !base.empty())) {
     std::string log;
-    int rc = fromMemory ? AKG_HIP_OK : compileToCodeObject(k->lowered, &k->codeObject, &log);
+    int rc = AKG_HIP_OK;
+    if (!fromMemory) {
+      std::vector<char> fresh;
+      rc = compileToCodeObject(k->lowered, &fresh, &log);
+      if (rc == AKG_HIP_OK) k->codeObject = std::make_shared<const std::vector<char>>(std::move(fresh));
+    }
     if (rc != AKG_HIP_OK) {
       if (!base.empty()) (void)writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size());
       if (k->lowered.family == akg::KernelFamily::ColumnReduce && allowStages) {
@@ -565,7 +580,7 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
       return fail(rc, "device compilation of " + k->lowered.kernelName + " failed:\n" + log);
     }
     akg::Sha256 h;
-    h.update(k->codeObject.data(), k->codeObject.size());
+    h.update(k->codeObject->data(), k->codeObject->size());
     k->codeSha256 = h.hexDigest();
     if (!fromMemory) {
       std::lock_guard<std::mutex> lock(g_codeCacheMutex);
@@ -577,7 +592,7 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
       std::string shapeInfo = shapeInfoJson(k->graph);
       if (!writeFile(base + "_shape_info.json", shapeInfo.data(), shapeInfo.size()) ||
           !writeFile(base + ".hip", k->lowered.source.data(), k->lowered.source.size()) ||
-          !writeFile(base + ".hsaco", k->codeObject.data(), k->codeObject.size()) ||
+          !writeFile(base + ".hsaco", k->codeObject->data(), k->codeObject->size()) ||
           !writeFile(base + "_shape_arg.txt", shapeArg.data(), shapeArg.size()) ||
           !writeFile(base + ".json", meta.data(), meta.size())) {
         return fail(AKG_HIP_ERR_IO, "cannot write artifacts under " + dir);
@@ -587,6 +602,32 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
   *outKernel = k.release();
   g_lastError.clear();
   return AKG_HIP_OK;
+}
+
+// The module of `k`'s code object on `device` (the current one): loaded once per process and device, counted per user.
+hipError_t acquireModule(const akg_hip_kernel &k, int device, hipModule_t *out) {
+  std::lock_guard<std::mutex> lock(g_moduleMutex);
+  SharedModule &m = g_modules[std::make_pair(k.codeSha256, device)];
+  if (m.module == nullptr) {
+    const hipError_t e = hipModuleLoadData(&m.module, k.codeObject->data());
+    if (e != hipSuccess) {
+      g_modules.erase(std::make_pair(k.codeSha256, device));
+      return e;
+    }
+  }
+  ++m.refs;
+  *out = m.module;
+  return hipSuccess;
+}
+
+void releaseModule(const std::string &codeSha256, int device) {
+  std::lock_guard<std::mutex> lock(g_moduleMutex);
+  auto it = g_modules.find(std::make_pair(codeSha256, device));
+  if (it == g_modules.end()) return;
+  if (--it->second.refs <= 0) {
+    (void)hipModuleUnload(it->second.module);
+    g_modules.erase(it);
+  }
 }
 
 // Code object and workspace of `k` on the current device, loaded / allocated on first use.
@@ -610,11 +651,11 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded **out) {
       if (rc != AKG_HIP_OK) return rc;
     }
   } else {
-    e = hipModuleLoadData(&l.module, k->codeObject.data());
+    e = acquireModule(*k, device, &l.module);
     if (e != hipSuccess) return fail(AKG_HIP_ERR_RUNTIME, "hipModuleLoadData: " + hipErr(e));
     e = hipModuleGetFunction(&l.function, l.module, k->lowered.kernelName.c_str());
     if (e != hipSuccess) {
-      (void)hipModuleUnload(l.module);
+      releaseModule(k->codeSha256, device);
       return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + k->lowered.kernelName + "): " + hipErr(e));
     }
   }
@@ -622,7 +663,7 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded **out) {
     hipFunction_t f = nullptr;
     e = hipModuleGetFunction(&f, l.module, ph.kernelName.c_str());
     if (e != hipSuccess) {
-      (void)hipModuleUnload(l.module);
+      releaseModule(k->codeSha256, device);
       return fail(AKG_HIP_ERR_RUNTIME, "hipModuleGetFunction(" + ph.kernelName + "): " + hipErr(e));
     }
     l.earlier.push_back(f);
@@ -638,7 +679,7 @@ int ensureLoaded(akg_hip_kernel *k, akg_hip_kernel::Loaded **out) {
     if (e == hipSuccess) e = hipEventCreateWithFlags(&l.lastUse, hipEventDisableTiming);
     if (e != hipSuccess) {
       if (l.workspace) (void)hipFree(l.workspace);
-      if (l.module) (void)hipModuleUnload(l.module);
+      if (l.module) releaseModule(k->codeSha256, device);
       return fail(AKG_HIP_ERR_RUNTIME, "workspace of " + std::to_string(k->lowered.workspaceBytes) + " bytes: " + hipErr(e));
     }
   }
@@ -653,7 +694,7 @@ void destroyKernel(akg_hip_kernel *kernel) {
   for (auto &l : kernel->loaded) {
     if (l.lastUse) (void)hipEventDestroy(l.lastUse);
     if (l.workspace) (void)hipFree(l.workspace);
-    if (l.module) (void)hipModuleUnload(l.module);
+    if (l.module) releaseModule(kernel->codeSha256, l.device);
   }
   delete kernel;
 }

@@ -219,11 +219,15 @@ class HipKernel:
     def from_file(cls, info_path, out_dir=DEFAULT_META_DIR):
         return cls(None, out_dir=out_dir, _path=info_path)
 
-    def __del__(self):
+    def close(self):
+        """Destroy the handle now (akg_hip_kernel_destroy) instead of when the object is collected."""
         h = getattr(self, "_handle", None)
         if h and getattr(self, "_owned", True):
             self._lib.akg_hip_kernel_destroy(h)
         self._handle = None
+
+    def __del__(self):
+        self.close()
 
     @property
     def inputs(self):

@@ -673,6 +673,24 @@ def test_handles_launched_from_several_threads_on_their_own_streams():
             assert np.array_equal(got.view(np.uint8), np.ascontiguousarray(a).view(np.uint8)), k.kernel_name
 
 
+def test_handles_of_one_source_share_their_module_and_outlive_each_other():
+    """Handles made from one source (two compilations of one description; the specialisations of a dynamic description)
+    share the loaded code object. Destroying one of them must leave the others launchable, and the last one to go
+    unloads it: a third handle made afterwards loads it afresh."""
+    path = os.path.join(FIXTURES, "small_softmax_f16_64x4096.info")
+    desc = harness.load_desc(path)
+    inputs = harness.make_inputs(desc, seed=harness.BASE_SEED + 5)
+    a, b = driver.HipKernel.from_file(path, out_dir=None), driver.HipKernel.from_file(path, out_dir=None)
+    want = run_on_gpu(a, inputs)
+    assert np.array_equal(run_on_gpu(b, inputs)[0].view(np.uint8), want[0].view(np.uint8))
+    a.close()
+    for _ in range(2):
+        assert np.array_equal(run_on_gpu(b, inputs)[0].view(np.uint8), want[0].view(np.uint8))
+    b.close()
+    c = driver.HipKernel.from_file(path, out_dir=None)
+    assert np.array_equal(run_on_gpu(c, inputs)[0].view(np.uint8), want[0].view(np.uint8))
+
+
 def test_cli_runs_a_description_on_the_gpu():
     """`akg-hip run X.info`: seeded inputs, NaN-prefilled outputs, a call on host buffers and timed launches. Two runs
     give the same checksums (one kernel, a sequence of kernels, and a kernel that must leave unnamed rows zero) and no NaN
