@@ -58,6 +58,7 @@ class IndexedEmitter {
     k.block[0] = kBlock;
     k.algorithmicBytes = lowering::countAlgorithmicBytes(g_);
     k.shapeArgs = lowering::buildShapeArgs(g_);
+    if (chunksArg_) k.scalarArgs.push_back(chunksTotal_);
     std::ostringstream note;
     note << "indexed vec=" << vec_ << " block=" << kBlock << " grid=" << grid_ << " rank=" << space_.size();
     if (!staged_.empty()) note << " lds_tiles=" << staged_.size() << " tile=" << kTile << "x" << kTile << " axis=" << tDim_;
@@ -67,6 +68,12 @@ class IndexedEmitter {
 
  private:
   static constexpr int kBlock = 256;
+  // A description with open extents: nothing in an index map depends on the outermost extent of the outputs unless an
+  // op works on that axis (every stride is a product of the extents to its right), so the number of chunks is a kernel
+  // argument instead of a constant and the workgroup numbering of the tiled transposes does not name it: batches of
+  // any size then share one code object wherever the ops leave the batch axis alone.
+  bool chunksArg_ = false;
+  int64_t chunksTotal_ = 0;
   // One component of a tensor index at the element a thread is working on.
   struct Ix {
     std::string s;         // C expression for the current element
@@ -727,17 +734,29 @@ class IndexedEmitter {
     // (64 x 1000 x 1024 -> 64 x 1024 x 1000 bf16: 33.5 % of the HBM peak in launch order)
     const int64_t outRowBytes = space_.back() * static_cast<int64_t>(dtypeSize(g_.tensor(g_.outputs[0]).dtype));
     if (outRowBytes % 64 != 0 && grid_ >= 64) {
-      src_ << "  int akg_w = akg::xcd_contiguous_id(static_cast<int>(blockIdx.x), " << grid_ << ");\n";
+      src_ << "  int akg_w = akg::xcd_contiguous_id(static_cast<int>(blockIdx.x), "
+           << (opt_.extentAsArgument ? std::string("static_cast<int>(gridDim.x)") : std::to_string(grid_)) << ");\n";
     } else {
       src_ << "  int akg_w = static_cast<int>(blockIdx.x);\n";
     }
     src_ << "  const int i0 = (akg_w % " << tilesI << ") * TILE;\n  akg_w /= " << tilesI << ";\n";
     src_ << "  const int t0 = (akg_w % " << tilesT << ") * TILE;\n  akg_w /= " << tilesT << ";\n";
     canonical_.assign(rank, Ix());
+    size_t lastSplit = rank;   // the outermost dim of the numbering: what is left of the workgroup id is its index
+    for (size_t d = 0; d + 1 < rank; ++d) {
+      if (d != td && space_[d] != 1) {
+        lastSplit = d;
+        break;
+      }
+    }
     for (size_t d = rank - 1; d-- > 0;) {
       if (d == td) continue;
       if (space_[d] == 1) continue;
-      src_ << "  const int g" << d << " = akg_w % " << space_[d] << ";\n  akg_w /= " << space_[d] << ";\n";
+      if (opt_.extentAsArgument && d == lastSplit) {
+        src_ << "  const int g" << d << " = akg_w;\n";
+      } else {
+        src_ << "  const int g" << d << " = akg_w % " << space_[d] << ";\n  akg_w /= " << space_[d] << ";\n";
+      }
       canonical_[d] = Ix("g" + std::to_string(d));
     }
     canonical_[td] = Ix("gt");
@@ -833,6 +852,8 @@ class IndexedEmitter {
     for (size_t i = 0; i < g_.outputs.size(); ++i, ++argc) {
       src_ << (argc ? ", " : "") << tagOf(g_.outputs[i]) << "::storage *__restrict__ out" << i;
     }
+    chunksArg_ = opt_.extentAsArgument && staged_.empty();
+    if (chunksArg_) src_ << ", const long akg_chunks_arg";
     src_ << ") {\n";
     if (!staged_.empty() && !assignedInput_.empty()) {
       throw LoweringError("an Assign next to a transpose that is staged through LDS tiles has no kernel yet");
@@ -846,7 +867,12 @@ class IndexedEmitter {
     for (int64_t d : space_) numel *= d;
     src_ << "  constexpr int V = " << vec_ << ";\n";
     src_ << "  const int chunk = static_cast<int>(blockIdx.x) * " << kBlock << " + static_cast<int>(threadIdx.x);\n";
-    src_ << "  if (chunk >= " << numel / space_.back() * chunksPerRow_ << ") return;\n";
+    chunksTotal_ = numel / space_.back() * chunksPerRow_;
+    if (chunksArg_) {
+      src_ << "  if (chunk >= static_cast<int>(akg_chunks_arg)) return;\n";
+    } else {
+      src_ << "  if (chunk >= " << chunksTotal_ << ") return;\n";
+    }
     if (overlapTail_) {
       src_ << "  int akg_inner = (chunk % " << chunksPerRow_ << ") * V;\n";
       src_ << "  if (akg_inner > " << space_.back() - vec_ << ") akg_inner = " << space_.back() - vec_ << ";\n";

@@ -92,3 +92,27 @@ DYNAMIC_STATS = {
     "bnstats_bf16_16x16": lambda n, name: op_desc.batchnorm_stats(n, 24, 16, 16, "bfloat16", name),
     "bnstats_f32_7x7": lambda n, name: op_desc.batchnorm_stats(n, 40, 7, 7, "float32", name),
 }
+
+
+def _concat_along_the_batch(n, name):
+    # an op that works ON the open axis: the two halves of the result come from different operands
+    b = op_desc.DescBuilder(name)
+    x = b.input([n, 24, 40], "float32")
+    y = b.input([n, 24, 40], "float32")
+    return b.dumps([b.unary("Neg", op_desc.concat(b, x, y, 0))])
+
+
+def _tile_along_the_batch(n, name):
+    b = op_desc.DescBuilder(name)
+    x = b.input([n, 8, 72], "float16")
+    return b.dumps([op_desc.tile(b, b.unary("Abs", x), [2, 1, 1])])
+
+
+# data-movement descriptions with the batch open: (maker, extents opened when the maker is called with 7777, whether the
+# source is expected to be the same for every batch size)
+DYNAMIC_VIEWS = {
+    "transpose_0213_f16": (lambda n, name: op_desc.transpose_0213_neg([n, 128, 12, 64], "float16", name), (7777,), True),
+    "transpose_bias_add_bf16": (lambda n, name: op_desc.transpose_bias_add(n, 256, 128, "bfloat16", name), (7777,), True),
+    "concat_along_the_batch_f32": (_concat_along_the_batch, (7777, 15554), False),
+    "tile_along_the_batch_f16": (_tile_along_the_batch, (7777, 15554), False),
+}

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 from akg_amd import driver, harness, op_desc
-from dynamic_cases import DYNAMIC_COLUMNS, DYNAMIC_POOLS, DYNAMIC_STATS, DYNAMIC_STREAMS, open_extent
+from dynamic_cases import DYNAMIC_COLUMNS, DYNAMIC_POOLS, DYNAMIC_STATS, DYNAMIC_STREAMS, DYNAMIC_VIEWS, open_extent
 from oracle import cpu_ref
 
 pytestmark = pytest.mark.gpu
@@ -1603,6 +1603,35 @@ def test_dynamic_streaming_reductions_behind_an_open_batch(kind):
                 print("    launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
                 assert ok, "%s %s output %s: %s" % (kind, shapes[0], d.name, msg)
     assert len(sources) <= (2 if kind in DYNAMIC_STATS else 1), "%d sources" % len(sources)
+
+
+@pytest.mark.parametrize("kind", sorted(DYNAMIC_VIEWS))
+def test_dynamic_data_movement_with_an_open_batch(kind):
+    """Transposes (through index maps and through LDS tiles) with the batch open share one code object: the number of
+    chunks is a kernel argument and the workgroup numbering does not name the outermost extent. Ops that work on the
+    open axis itself (a Concat or a Tile along the batch) keep its extent in their index maps: every batch size is its
+    own source there, and every result is still right. Data movement is exact: bit for bit against the oracle."""
+    from oracle import np_ref
+    make, sentinels, shared = DYNAMIC_VIEWS[kind]
+    dyn = driver.HipDynamicKernel(open_extent(make(7777, "dyn_" + kind), sentinels), out_dir=None)
+    sources = set()
+    for n in (4, 32, 3):
+        bound = json_loads(make(n, "dyn_" + kind))
+        shapes = [e[0]["shape"] for e in bound["input_desc"]]
+        kernel = dyn.specialize(shapes)
+        print("  %s N=%d: %s grid %d, made in %.1f ms%s" % (kind, n, kernel.family, kernel.grid[0], kernel.build_ms,
+                                                          " (no device compilation)" if kernel.cache_hit else ""), flush=True)
+        assert kernel.family == "indexed"
+        assert [t.shape for t in kernel.outputs] == [o["shape"] for o in bound["output_desc"]]
+        sources.add(kernel.source)
+        inputs = harness.make_inputs(bound, seed=harness.BASE_SEED + 111 + n)
+        expect = np_ref.evaluate(bound, inputs)
+        got = run_on_gpu(kernel, inputs)
+        for d, g, e in zip(kernel.outputs, got, expect):
+            ok, msg = harness.compare_bits(g, e, d.dtype)
+            print("    %s %s: %s" % (d.name, d.dtype, msg), flush=True)
+            assert ok, "%s N=%d output %s: %s" % (kind, n, d.name, msg)
+    assert (len(sources) == 1) == shared, "%d sources" % len(sources)
 
 
 @pytest.mark.parametrize("kind", sorted(DYNAMIC_COLUMNS))

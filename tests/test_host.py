@@ -921,6 +921,14 @@ def test_streaming_and_column_kernels_take_their_open_extent_as_an_argument(monk
                 for b, t in ((4, 300), (32, 64), (2, 5000))]
         assert all(k.family == "stream_reduce" and "akg_o_arg" in k.source and "akg_o * (R * " in k.source for k in seen), kind
         assert all(k.source == seen[0].source for k in seen) and all(k.cache_hit for k in seen[1:]), kind
+    # data movement with the batch open: the number of chunks is an argument; ops on the batch axis keep its extent
+    from dynamic_cases import DYNAMIC_VIEWS
+    for kind, (make, sentinels, shared) in sorted(DYNAMIC_VIEWS.items()):
+        dyn = driver.HipDynamicKernel(open_extent(make(7777, "dynhost_" + kind), sentinels), out_dir=None)
+        seen = [dyn.specialize([e[0]["shape"] for e in json.loads(make(n, "dynhost_" + kind))["input_desc"]]) for n in (4, 32, 3)]
+        assert all(k.family == "indexed" for k in seen), kind
+        assert (len({k.source for k in seen}) == 1) == shared, kind
+        assert all(k.cache_hit for k in seen[1:]) == shared, kind
     # the batch of [N,C,H,W] statistics: N * H * W is the argument, the buffer sizes follow N
     for kind, make in sorted(DYNAMIC_STATS.items()):
         dyn = driver.HipDynamicKernel(open_extent(make(7777, "dynhost_" + kind), 7777), out_dir=None)
