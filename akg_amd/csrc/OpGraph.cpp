@@ -186,7 +186,8 @@ class GraphBuilder {
   int addTensor(const std::string &name, DType dtype, const std::vector<int64_t> &shape) {
     for (int64_t d : shape) {
       if (d < 0) {
-        throw TranslateError("tensor " + name + ": dynamic dimensions (-1) are not supported by the HIP backend");
+        throw TranslateError("tensor " + name + ": dynamic dimensions (-1) need the shapes of a call: a dynamic description "
+                             "goes through akg_hip_dynamic_create / akg_hip_dynamic_specialize (akg-hip --shapes)");
       }
     }
     TensorValue t;

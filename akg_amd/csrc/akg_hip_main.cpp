@@ -7,6 +7,9 @@
  *   akg-hip emit X.info                 print the emitted HIP source
  *   akg-hip compile X.info -o DIR       write <op>.hsaco, <op>.json, <op>_shape_arg.txt, <op>.hip to DIR
  *   akg-hip info X.info                 print signature, family, launch shape, algorithmic bytes
+ *   ... --shapes "32,1,48,48;32,12,48,48"   with emit / compile / info / run: X.info is a dynamic-shape description (-1
+ *                                       extents); it is specialised to these input shapes (one per input, in
+ *                                       input_desc order) through akg_hip_dynamic_specialize first
  *   akg-hip run X.info [-n N] [-r R] [--inputs DIR] [--dump DIR] [--expect DIR]
  *                                       what `akg_benchmark -e gpu -f X.info -p` does (benchmark.py:94-130): seeded
  *                                       inputs, NaN-prefilled outputs, one call on host buffers, then R x N timed
@@ -43,7 +46,8 @@ int usage() {
                "       akg-hip compile X.info -o DIR\n"
                "       akg-hip info X.info\n"
                "       akg-hip run X.info [-n launches per measurement] [-r measurements]\n"
-               "                          [--inputs DIR] [--dump DIR] [--expect DIR]\n");
+               "                          [--inputs DIR] [--dump DIR] [--expect DIR]\n"
+               "       emit / compile / info / run take --shapes \"d,d,..;d,d,..\" for a dynamic-shape description\n");
   return 2;
 }
 
@@ -343,12 +347,13 @@ int main(int argc, char **argv) {
   if (argc < 3) return usage();
   const std::string cmd = argv[1];
   const char *path = argv[2];
-  const char *outDir = nullptr, *inputsDir = nullptr, *dumpDir = nullptr, *expectDir = nullptr;
+  const char *outDir = nullptr, *inputsDir = nullptr, *dumpDir = nullptr, *expectDir = nullptr, *shapesText = nullptr;
   int number = 10, repeat = 5;
   for (int i = 3; i + 1 < argc; ++i) {
     if (std::strcmp(argv[i], "--inputs") == 0) inputsDir = argv[i + 1];
     if (std::strcmp(argv[i], "--dump") == 0) dumpDir = argv[i + 1];
     if (std::strcmp(argv[i], "--expect") == 0) expectDir = argv[i + 1];
+    if (std::strcmp(argv[i], "--shapes") == 0) shapesText = argv[i + 1];
     if (std::strcmp(argv[i], "-o") == 0) outDir = argv[i + 1];
     if (std::strcmp(argv[i], "-n") == 0) number = std::atoi(argv[i + 1]);
     if (std::strcmp(argv[i], "-r") == 0) repeat = std::atoi(argv[i + 1]);
@@ -371,23 +376,57 @@ int main(int argc, char **argv) {
   if (cmd != "emit" && cmd != "compile" && cmd != "info" && cmd != "run") return usage();
   if (cmd == "compile" && outDir == nullptr) return usage();
   akg_hip_kernel_t *k = nullptr;
-  int rc = akg_hip_compile_file(path, cmd == "compile" ? outDir : nullptr, &k);
+  akg_hip_dynamic_t *dyn = nullptr;   // owns k when the description is a dynamic one
+  int rc;
+  if (shapesText != nullptr) {
+    std::string text;
+    if (!readAll(path, &text)) {
+      std::fprintf(stderr, "akg-hip: cannot read %s\n", path);
+      return 1;
+    }
+    std::vector<std::vector<int64_t>> shapes(1);
+    for (const char *p = shapesText; *p != 0; ++p) {
+      if (*p == ';') {
+        shapes.emplace_back();
+      } else if (*p >= '0' && *p <= '9') {
+        char *end = nullptr;
+        shapes.back().push_back(std::strtoll(p, &end, 10));
+        p = end - 1;
+      } else if (*p != ',' && *p != ' ') {
+        std::fprintf(stderr, "akg-hip: --shapes takes extents separated by ',' and shapes separated by ';'\n");
+        return 2;
+      }
+    }
+    std::vector<const int64_t *> shapePtrs;
+    std::vector<int32_t> ranks;
+    for (const auto &sh : shapes) {
+      shapePtrs.push_back(sh.data());
+      ranks.push_back(static_cast<int32_t>(sh.size()));
+    }
+    rc = akg_hip_dynamic_create(text.data(), text.size(), cmd == "compile" ? outDir : nullptr, &dyn);
+    if (rc == AKG_HIP_OK) rc = akg_hip_dynamic_specialize(dyn, shapePtrs.data(), ranks.data(), static_cast<int>(shapes.size()), &k);
+  } else {
+    rc = akg_hip_compile_file(path, cmd == "compile" ? outDir : nullptr, &k);
+  }
   if (rc != AKG_HIP_OK) {
     std::fprintf(stderr, "akg-hip: error %d: %s\n", rc, akg_hip_last_error());
+    if (dyn) akg_hip_dynamic_destroy(dyn);
     return 1;
   }
+  int status = 0;
   if (cmd == "run") {
-    rc = runKernel(k, number, repeat, inputsDir, dumpDir, expectDir);
-    akg_hip_kernel_destroy(k);
-    return rc;
-  }
-  if (cmd == "emit") {
+    status = runKernel(k, number, repeat, inputsDir, dumpDir, expectDir);
+  } else if (cmd == "emit") {
     const char *src = nullptr;
     akg_hip_kernel_source(k, &src);
     std::fputs(src, stdout);
   } else {
     printInfo(k);
   }
-  akg_hip_kernel_destroy(k);
-  return 0;
+  if (dyn) {
+    akg_hip_dynamic_destroy(dyn);
+  } else {
+    akg_hip_kernel_destroy(k);
+  }
+  return status;
 }

@@ -846,7 +846,15 @@ def test_cli_tool():
     # a dynamic-shape description is an error with a non-zero exit, never a crash
     r = subprocess.run([tool, "emit", os.path.join(
         REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")], capture_output=True, text=True)
-    assert r.returncode == 1 and "error -3" in r.stderr
+    assert r.returncode == 1 and "error -3" in r.stderr and "--shapes" in r.stderr
+    # ... unless the shapes of a call come with it: then it is specialised to them first
+    dynamic = os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")
+    r = subprocess.run([tool, "info", dynamic, "--shapes", "32,1,48,48;32,12,48,48"], capture_output=True, text=True)
+    assert r.returncode == 0 and "row_reduce" in r.stdout and "[32,12,48,48]" in r.stdout, r.stderr
+    r = subprocess.run([tool, "emit", dynamic, "--shapes", "32,1,40,40;32,12,40,40"], capture_output=True, text=True)
+    assert r.returncode == 0 and "akg_dim_arg0" in r.stdout
+    r = subprocess.run([tool, "emit", dynamic, "--shapes", "32,1,40,40"], capture_output=True, text=True)
+    assert r.returncode == 1 and "2 inputs" in r.stderr
 
 
 def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
