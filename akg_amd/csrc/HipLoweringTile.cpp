@@ -85,7 +85,7 @@ class TileEmitter {
          << " threads_per_row=" << tpr_ << " chunks=" << chunks_ << " rows_per_block=" << rowsPerBlock_
          << " block=" << block_ << " grid=" << grid_;
     if (overlap_ > 0) note << " tail_overlap=" << overlap_;
-    if (colsArg_) note << " (row length is a kernel argument: one code object for rows of " << bucketLow_ << " .. " << bucketHigh_ << " elements)";
+    if (colsArg_) note << " (row length is a kernel argument: one code object for rows of " << bucketLow_ << " .. " << bucketHigh_ << " elements" << (colsWhole_ ? " that are whole 64-byte pieces" : "") << ")";
     if (multiPass_) note << " walks_of_groups=" << groups_ << (packedRow_ ? " (row packed in registers)" : "");
     k.scheduleNote = note.str();
     return k;
@@ -107,6 +107,10 @@ class TileEmitter {
   // length of the bucket shares the source and with it the code object.
   bool colsArg_ = false;
   bool allowColsArg_ = true;
+  // ... and every row of every tensor that spans the row is a whole number of 64-byte pieces (hidden sizes usually are):
+  // such row lengths have a source of their own, in which chunks never overlap, nothing is skipped in the reductions
+  // and whole lines are streamed with the non-temporal hint, like in the kernel of a static description.
+  bool colsWhole_ = false;
   // Dynamic descriptions with an operand that spans only some of the leading dimensions (an attention mask shared by
   // the heads): the leading extents of the folded iteration space are kernel arguments too, and the operand's row
   // offset is computed from them, so the source does not carry them as numbers.
@@ -310,16 +314,18 @@ class TileEmitter {
     // Chunk width: 16 bytes of the widest element type that is moved chunk-wise, so no tensor needs more than one
     // 128-bit access per chunk (narrower tensors use 64- or 32-bit accesses, which still coalesce fully). Measured
     // on MI355X: many small contiguous accesses per wave beat fewer, wider ones.
-    size_t minSize = 1;
+    size_t minSize = 1, narrowest = 16;
     bool any = false;
     for (size_t i = 0; i < g_.inputs.size(); ++i) {
       if (!access_[i].lastDimFull) continue;
       minSize = std::max(minSize, dtypeSize(g_.tensor(g_.inputs[i]).dtype));
+      narrowest = std::min(narrowest, dtypeSize(g_.tensor(g_.inputs[i]).dtype));
       any = true;
     }
     for (int id : g_.outputs) {
       if (rowMode_ && g_.tensor(id).numel() != numel_) continue;
       minSize = std::max(minSize, dtypeSize(g_.tensor(id).dtype));
+      narrowest = std::min(narrowest, dtypeSize(g_.tensor(id).dtype));
       any = true;
     }
     if (!any) minSize = 4;
@@ -339,8 +345,9 @@ class TileEmitter {
       bucketLow_ = std::max<int64_t>(2 * v, bucketChunks / 2 * v + 1);
       schedCols = bucketHigh_;
     }
+    colsWhole_ = colsArg_ && rowMode_ && any && (cols_ * static_cast<int64_t>(narrowest)) % 64 == 0;
     if (colsArg_ && rowMode_) {
-      // element-aligned chunks; the overlap of the last one is computed in the kernel
+      // element-aligned chunks; the overlap of the last one is computed in the kernel (none when rows are whole lines)
     } else if (rowMode_ && useBuffers_ && !inPlace && opt_.vec == 0 && (cols_ % v) != 0 && cols_ >= 2 * v) {
       overlap_ = static_cast<int>(v - cols_ % v);
     } else {
@@ -549,6 +556,9 @@ class TileEmitter {
     if (useBuffers_) return "b_" + arg + ", " + offset;
     return arg + " + " + offset;
   }
+  // The chunks' conditions are run-time values (ragged rows or tails, extents that are arguments) and the tensors are
+  // addressed through descriptors: accesses take their condition as an operand instead of standing behind a branch.
+  bool conditionalAccesses() const { return useBuffers_ && (rowMode_ ? raggedCols_ : raggedFlat_); }
 
   // Offset of the first element of `row` for an input, as an expression in `rowVar`.
   std::string rowOffsetExpr(const InputAccess &a, const std::string &rowVar) const {
@@ -704,7 +714,7 @@ class TileEmitter {
       if (multiPass_) {
         src_ << "  constexpr int GROUPS = " << groups_ << ";\n";
       } else {
-        if (colsArg_) line("  const int akg_overlap = static_cast<int>((V - COLS % V) % V);   // elements the last chunk of a row shares with its neighbour");
+        if (colsArg_ && !colsWhole_) line("  const int akg_overlap = static_cast<int>((V - COLS % V) % V);   // elements the last chunk of a row shares with its neighbour");
         emitColumnsOfGroup("0");
       }
     } else {
@@ -805,7 +815,7 @@ class TileEmitter {
   bool streamsWholeLines(int tensorId) const {
     if (!nonTemporal_) return false;
     if (!rowMode_) return true;
-    if (colsArg_) return false;   // rows of any length: their first and last cache lines may be shared with neighbours
+    if (colsArg_ && !colsWhole_) return false;   // rows of any length: their first and last cache lines may be shared with neighbours
     const int64_t rowBytes = cols_ * static_cast<int64_t>(dtypeSize(g_.tensor(tensorId).dtype));
     return rowBytes % 64 == 0 || rowBytes >= 16384;  // two shared lines in 256 or more do not matter
   }
@@ -814,7 +824,7 @@ class TileEmitter {
   void emitColumnsOfGroup(const std::string &group) {
     line("  long akg_cols[NCHUNK];");
     line("  bool akg_ok[NCHUNK];");
-    const bool tails = overlap_ > 0 || (colsArg_ && rowMode_);
+    const bool tails = overlap_ > 0 || (colsArg_ && rowMode_ && !colsWhole_);
     if (tails) line("  bool akg_tail[NCHUNK];");
     line("#pragma unroll");
     line("  for (int j = 0; j < NCHUNK; ++j) {");
@@ -933,6 +943,12 @@ class TileEmitter {
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
         if (!packedInput_[i]) continue;
         const std::string tag = tagOf(g_.inputs[i]);
+        if (conditionalAccesses()) {
+          src_ << "    akg::load_raw_chunk_if<" << tag << ", V, " << (streamsWholeLines(g_.inputs[i]) ? "true" : "false") << ">(b_in"
+               << i << ", akg_ok[j], " << rowOffsetExpr(access_[i], "akg_rows[j]") << " + akg_cols[j], r_in" << i
+               << "[akg_g * NCHUNK + j]);\n";
+          continue;
+        }
         src_ << "    if (akg_ok[j]) {\n";
         src_ << "      akg::load_raw_chunk<" << tag << ", V, " << (streamsWholeLines(g_.inputs[i]) ? "true" : "false") << ">(b_in"
              << i << ", " << rowOffsetExpr(access_[i], "akg_rows[j]") << " + akg_cols[j], r_in" << i
@@ -1015,17 +1031,22 @@ class TileEmitter {
       src_ << "  " << ct << " " << v.ident << "[NCHUNK][V];\n";
       line("#pragma unroll");
       line("  for (int j = 0; j < NCHUNK; ++j) {");
-      src_ << "    if (akg_ok[j]) {\n";
       // a tensor as large as the iteration space is read exactly once: stream it
       const bool streamed = streamsWholeLines(id) && (t.numel() == numel_) &&
                             (!multiPass_ || lastPassOfInput_[i] == pass_);
-      src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">("
-           << memRef("in" + std::to_string(i), rowOffsetExpr(a, "akg_rows[j]") + " + akg_cols[j]") << ", " << v.ident
-           << "[j]);\n";
-      src_ << "    } else {\n";
-      src_ << "      akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(" << tag
-           << "::storage()));\n";
-      src_ << "    }\n";
+      if (conditionalAccesses()) {
+        src_ << "    akg::load_chunk_if<" << tag << ", V, " << (streamed ? "true" : "false") << ">(b_in" << i << ", akg_ok[j], "
+             << rowOffsetExpr(a, "akg_rows[j]") << " + akg_cols[j], " << v.ident << "[j]);\n";
+      } else {
+        src_ << "    if (akg_ok[j]) {\n";
+        src_ << "      akg::load_chunk<" << tag << ", V, " << (streamed ? "true" : "false") << ">("
+             << memRef("in" + std::to_string(i), rowOffsetExpr(a, "akg_rows[j]") + " + akg_cols[j]") << ", " << v.ident
+             << "[j]);\n";
+        src_ << "    } else {\n";
+        src_ << "      akg::fill_chunk<" << tag << ", V>(" << v.ident << "[j], " << tag << "::load(" << tag
+             << "::storage()));\n";
+        src_ << "    }\n";
+      }
       line("  }");
     } else if (rowMode_) {
       // one element per row (or a single element for the whole kernel)
@@ -1185,7 +1206,7 @@ class TileEmitter {
       line("#pragma unroll");
       line("    for (int j = 0; j < NCHUNK; ++j) {");
       std::string from = "0";
-      if (colsArg_) {
+      if (colsArg_ && !colsWhole_) {
         from = "akg_tail[j] ? akg_overlap : 0";
       } else if (overlap_ > 0) {
         from = "akg_tail[j] ? " + std::to_string(overlap_) + " : 0";
@@ -1207,7 +1228,7 @@ class TileEmitter {
     line("    for (int e = 0; e < V; ++e) {");
     std::string step = spec.combiner + "::apply(" + acc + ", " + in.ident + "[j][e])";
     if (spec.roundEachStep) step = tag + "::rnd(" + step + ")";
-    if (colsArg_) {
+    if (colsArg_ && !colsWhole_) {
       src_ << "      if (akg_ok[j] && (!akg_tail[j] || e >= akg_overlap)) " << acc << " = " << step << ";\n";
     } else if (overlap_ > 0) {
       src_ << "      if (akg_ok[j] && (!akg_tail[j] || e >= " << overlap_ << ")) " << acc << " = " << step << ";\n";
@@ -1270,9 +1291,15 @@ class TileEmitter {
     std::string guard = "akg_ok[j]";
     if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
     const std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
-    src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (streamsWholeLines(op.inputs[0]) ? "true" : "false") << ">("
-         << memRef("in" + std::to_string(dst.inputIndex), offset) << ", " << v.ident << "[j]);  // " << op.name << " -> "
-         << dst.name << "\n";
+    if (conditionalAccesses() || (useBuffers_ && guard != "akg_ok[j]")) {
+      src_ << "    akg::store_chunk_if<" << tag << ", V, " << (streamsWholeLines(op.inputs[0]) ? "true" : "false") << ">(b_in"
+           << dst.inputIndex << ", " << guard << ", " << offset << ", " << v.ident << "[j]);  // " << op.name << " -> "
+           << dst.name << "\n";
+    } else {
+      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (streamsWholeLines(op.inputs[0]) ? "true" : "false") << ">("
+           << memRef("in" + std::to_string(dst.inputIndex), offset) << ", " << v.ident << "[j]);  // " << op.name << " -> "
+           << dst.name << "\n";
+    }
     line("  }");
   }
 
@@ -1300,9 +1327,14 @@ class TileEmitter {
       std::string guard = "akg_ok[j]";
       if (rowMode_ && raggedRows_) guard += " && akg_row_ok";
       std::string offset = rowMode_ ? "akg_rows[j] * COLS + akg_cols[j]" : "akg_flat[j]";
-      src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (streamsWholeLines(id) ? "true" : "false") << ">("
-           << memRef("out" + std::to_string(i), offset) << ", " << src
-           << "[j]);\n";
+      if (conditionalAccesses() || (useBuffers_ && guard != "akg_ok[j]")) {
+        src_ << "    akg::store_chunk_if<" << tag << ", V, " << (streamsWholeLines(id) ? "true" : "false") << ">(b_out" << i << ", "
+             << guard << ", " << offset << ", " << src << "[j]);\n";
+      } else {
+        src_ << "    if (" << guard << ") akg::store_chunk<" << tag << ", V, " << (streamsWholeLines(id) ? "true" : "false") << ">("
+             << memRef("out" + std::to_string(i), offset) << ", " << src
+             << "[j]);\n";
+      }
       line("  }");
     } else {
       if (t.numel() != rows_) {

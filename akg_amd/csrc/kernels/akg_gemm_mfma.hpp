@@ -194,6 +194,13 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const long kPerXcd = (kTiles + kGemmXcds - 1) / kGemmXcds;
   constexpr long kSteps = (K + BK - 1) / BK;
   constexpr bool kFull = !DYN && (MS % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
+  // DYN with whole tiles along N and K: the loads need no checks either. Every thread clamps the rows of A it stages to
+  // the last row once, in front of the loop (the scalar offset of a buffer load takes no part in the descriptor's range
+  // check, so the descriptor alone would not keep the rows of a ragged last tile inside A); rows beyond M then hold
+  // copies of row M - 1 and their accumulators are dropped by the epilogue's row check. The main loop is the one of a
+  // static shape: no compares, one basic block per K step.
+  constexpr bool kLoadsInRange = kFull || (DYN && (N % kGemmBN == 0) && (K % BK == 0));
+  constexpr bool kClampRows = DYN && kLoadsInRange;
   constexpr int kTileBytes = kGemmBM * kPitch;        // one operand tile in LDS
   static_assert(kRowChunks == 4, "the staging schedule is written for four 16-byte chunks per thread and operand");
   // A row-major B goes to LDS as it lies in memory, k-rows of 256 columns. Sixteen lanes share a transposing read:
@@ -269,6 +276,12 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
       const_cast<void *>(B), 0, static_cast<int>(N * K), 0x00020000);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
   const int aVoff = static_cast<int>((m0 + aRow) * K + aChunk * 16);
+  int aVoffClamped[kRowChunks];   // kClampRows: one vector offset per staged chunk, its row clamped to M - 1
+#pragma unroll
+  for (int i = 0; i < kRowChunks; ++i) {
+    const long row = m0 + aRow + kRowStep * i;
+    aVoffClamped[i] = static_cast<int>((row < M ? row : M - 1) * K + aChunk * 16);
+  }
   const int bRowT = tid / kChunksPerRowB;     // + kRowStepB * i
   const int bChunkT = tid % kChunksPerRowB;
   const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
@@ -297,14 +310,15 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 
   auto loadChunk = [&](long step, int i) {
     const long k0 = (stepBase + step) * BK;
-    if (kFull || (m0 + aRow + kRowStep * i < M && k0 + aChunk * 16 < K)) {
-      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(aRsrc, aVoff, static_cast<int>((kRowStep * i) * K + k0), 0);
+    if (kLoadsInRange || (m0 + aRow + kRowStep * i < M && k0 + aChunk * 16 < K)) {
+      const u32x4 v = kClampRows ? __builtin_amdgcn_raw_buffer_load_b128(aRsrc, aVoffClamped[i], static_cast<int>(k0), 0)
+                                 : __builtin_amdgcn_raw_buffer_load_b128(aRsrc, aVoff, static_cast<int>((kRowStep * i) * K + k0), 0);
       stage.x[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
     } else {
       stage.x[i] = v4i{0, 0, 0, 0};
     }
     if constexpr (TRANSB) {
-      if (kFull || (n0 + aRow + kRowStep * i < N && k0 + aChunk * 16 < K)) {
+      if (kLoadsInRange || (n0 + aRow + kRowStep * i < N && k0 + aChunk * 16 < K)) {
         const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoff, static_cast<int>((kRowStep * i) * K + k0), 0);
         stage.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
       } else {
@@ -312,7 +326,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
       }
     } else {
       const long krow = k0 / EB + bRowT + kRowStepB * i;
-      if (kFull || (krow < KE && n0 * EB + bChunkT * 16 < NB)) {
+      if (kLoadsInRange || (krow < KE && n0 * EB + bChunkT * 16 < NB)) {
         const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(bRsrc, bVoff, static_cast<int>((k0 / EB + kRowStepB * i) * NB), 0);
         stage.y[i] = v4i{static_cast<int>(v[0]), static_cast<int>(v[1]), static_cast<int>(v[2]), static_cast<int>(v[3])};
       } else {
@@ -342,7 +356,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 
   // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
   // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
-  constexpr bool kAllRowsReal = !DYN && (MS % kGemmBM == 0);
+  constexpr bool kAllRowsReal = DYN ? kLoadsInRange : (MS % kGemmBM == 0);   // (DYN: every wavefront computes; M > 64 there)
   const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
   // A fragments of row half rh (2 tiles of 16 rows), K half kh (64 bytes)
   auto readA = [&](int buf, int kh, int rh, v4i (&af)[kHM]) {

@@ -289,6 +289,46 @@ AKG_DEV void store_chunk(Buffer buf, long index, const typename DT::compute (&sr
   for (int k = 0; k < kPieces; ++k) Io::store(raw[k], buf, off + k * kPiece);
 }
 
+// The same under a condition that is a value, not a branch: where `ok` is false the access goes to byte 2^31, beyond
+// the end of every tensor addressed through a descriptor (they are below 2 GiB), and the range check of the hardware
+// answers a load with zeros and drops a store. The accesses of a thread's chunks then issue back to back whatever
+// their conditions are, where a branch per chunk would put each behind the test of its own condition.
+constexpr u32 kBeyondEveryBuffer = 0x80000000u;
+
+template <typename DT, int V, bool STREAM = false>
+AKG_DEV void load_chunk_if(Buffer buf, bool ok, long index, typename DT::compute (&dst)[V]) {
+  typedef typename DT::storage S;
+  constexpr int kBytes = static_cast<int>(sizeof(S)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef BufferIo<kPiece, STREAM ? kAuxStreamLoad : kAuxDefault> Io;
+  typename Io::type raw[kPieces];
+  const u32 off = ok ? static_cast<u32>(index) * static_cast<u32>(sizeof(S)) : kBeyondEveryBuffer;
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) raw[k] = Io::load(buf, off + k * kPiece);
+  S tmp[V];
+  __builtin_memcpy(tmp, raw, kBytes);
+#pragma unroll
+  for (int e = 0; e < V; ++e) dst[e] = DT::load(tmp[e]);
+}
+
+template <typename DT, int V, bool STREAM = false>
+AKG_DEV void store_chunk_if(Buffer buf, bool ok, long index, const typename DT::compute (&src)[V]) {
+  typedef typename DT::storage S;
+  constexpr int kBytes = static_cast<int>(sizeof(S)) * V;
+  constexpr int kPiece = kBytes > 16 ? 16 : kBytes;
+  constexpr int kPieces = kBytes / kPiece;
+  typedef BufferIo<kPiece, STREAM ? kAuxStreamStore : kAuxDefault> Io;
+  S tmp[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) tmp[e] = DT::store(src[e]);
+  typename Io::type raw[kPieces];
+  __builtin_memcpy(raw, tmp, kBytes);
+  const u32 off = ok ? static_cast<u32>(index) * static_cast<u32>(sizeof(S)) : kBeyondEveryBuffer;
+#pragma unroll
+  for (int k = 0; k < kPieces; ++k) Io::store(raw[k], buf, off + k * kPiece);
+}
+
 // A chunk kept as it came from memory (a 16-bit row held in registers takes half the space of its float image);
 // unpack_chunk converts it whenever the values are needed.
 template <typename DT, int V>
@@ -304,6 +344,15 @@ AKG_DEV void load_raw_chunk(Buffer buf, long index, RawChunk<DT, V> &dst) {
   typedef RawChunk<DT, V> R;
   typedef BufferIo<R::kPiece, STREAM ? kAuxStreamLoad : kAuxDefault> Io;
   const u32 off = static_cast<u32>(index) * static_cast<u32>(sizeof(typename DT::storage));
+#pragma unroll
+  for (int k = 0; k < R::kPieces; ++k) dst.raw[k] = Io::load(buf, off + k * R::kPiece);
+}
+
+template <typename DT, int V, bool STREAM = false>
+AKG_DEV void load_raw_chunk_if(Buffer buf, bool ok, long index, RawChunk<DT, V> &dst) {
+  typedef RawChunk<DT, V> R;
+  typedef BufferIo<R::kPiece, STREAM ? kAuxStreamLoad : kAuxDefault> Io;
+  const u32 off = ok ? static_cast<u32>(index) * static_cast<u32>(sizeof(typename DT::storage)) : kBeyondEveryBuffer;
 #pragma unroll
   for (int k = 0; k < R::kPieces; ++k) dst.raw[k] = Io::load(buf, off + k * R::kPiece);
 }

@@ -1260,17 +1260,19 @@ def _open_dims(text, rows, cols):
 @pytest.mark.parametrize("pattern", ["softmax_f16", "layernorm_bf16", "quant_bf16", "bias_gelu_f32"])
 def test_row_lengths_of_one_bucket_share_a_code_object_and_stay_correct(pattern):
     """Dynamic descriptions take the row length as a kernel argument: the schedule is made for a power-of-two bucket of
-    chunk counts, chunks are element-aligned and the last one overlaps its neighbour by a run-time amount. Row lengths
-    across a bucket (odd ones, the bucket's ends, one chunk short of it), with different row counts: the first makes the
-    code object, the others must reuse it (no device compilation) and all must match the oracle."""
+    chunk counts, chunks are element-aligned and the last one overlaps its neighbour by a run-time amount; rows that are
+    whole 64-byte pieces in every tensor have a source of their own (no overlap, whole lines streamed). Row lengths
+    across a bucket (odd ones, the bucket's ends, one chunk short of it, two whole-line ones), with different row counts:
+    the first of its kind makes the code object, the others must reuse it (no device compilation) and all must match
+    the oracle."""
     from oracle import np_ref
     R, C = 7777, 9999
     if pattern == "softmax_f16":
-        text, v, lengths = op_desc.softmax_last_axis(R, C, "float16", "dyn_softmax_f16"), 8, [520, 1000, 1024, 513, 777]
+        text, v, lengths = op_desc.softmax_last_axis(R, C, "float16", "dyn_softmax_f16"), 8, [520, 1000, 1024, 513, 777, 768]
     elif pattern == "layernorm_bf16":
-        text, v, lengths = op_desc.layernorm_residual(R, C, "bfloat16", 1e-5, "dyn_layernorm_bf16"), 8, [4096, 2056, 3001, 4095]
+        text, v, lengths = op_desc.layernorm_residual(R, C, "bfloat16", 1e-5, "dyn_layernorm_bf16"), 8, [4096, 2056, 3001, 4095, 3072]
     elif pattern == "quant_bf16":
-        text, v, lengths = op_desc.quant_int8_residual(R, C, "bfloat16", "dyn_quant_bf16"), 8, [300, 264, 511, 512]
+        text, v, lengths = op_desc.quant_int8_residual(R, C, "bfloat16", "dyn_quant_bf16"), 8, [300, 264, 511, 512, 320]
     else:
         b = op_desc.DescBuilder("dyn_bias_gelu_f32")
         x, bias = b.input([R, C], "float32"), b.input([C], "float32")
@@ -1278,7 +1280,8 @@ def test_row_lengths_of_one_bucket_share_a_code_object_and_stay_correct(pattern)
         text, v, lengths = b.dumps([b.mul(y, b.unary("Tanh", y))]), 4, [72, 100, 128, 68]
     desc = _open_dims(text, R, C)
     dyn = driver.HipDynamicKernel(__import__("json").dumps(desc), out_dir=None)
-    first = None
+    narrowest = min(np.dtype(driver.NP_HOST_DTYPE[e[0]["data_type"]]).itemsize for e in desc["input_desc"] + [desc["output_desc"][:1]])
+    first = {}
     for n, cols in enumerate(lengths):
         rows = [37, 5, 130, 64, 2][n % 5]
         # the description's open dims are (rows, cols) for matrices and (cols) for vectors
@@ -1293,8 +1296,11 @@ def test_row_lengths_of_one_bucket_share_a_code_object_and_stay_correct(pattern)
             print("  %s rows %d cols %d %s: %s (made in %.1f ms, cache_hit %s)" % (pattern, rows, cols, d.name, msg, kernel.build_ms,
                                                                                  kernel.cache_hit), flush=True)
             assert ok, "%s cols %d output %s: %s" % (pattern, cols, d.name, msg)
-        if first is None:
-            first = kernel
+        # rows of the row kernels that are whole 64-byte pieces in every tensor have a source of their own in the bucket
+        whole = pattern != "bias_gelu_f32" and (cols * narrowest) % 64 == 0
+        assert ("akg_overlap" not in kernel.source) == (whole or pattern == "bias_gelu_f32")
+        if whole not in first:
+            first[whole] = kernel
         elif pattern != "bias_gelu_f32" or cols % v == 0:
             assert kernel.cache_hit, "%s: row length %d compiled anew" % (pattern, cols)
 

@@ -602,14 +602,15 @@ def test_row_schedules_for_odd_and_long_rows():
     # 16-bit inputs that fits 64 registers per thread in its memory image is loaded once and kept packed ...
     c, src = consts("small_softmax_f16_3x70000")
     assert (c["TPR"], c["NCHUNK"], c["GROUPS"]) == (1024, 2, 5) and src.count("for (int akg_g = 0; akg_g < GROUPS") == 4
-    assert src.count("load_raw_chunk<akg::f16, V, true>(b_in0") == 1 and src.count("unpack_chunk<akg::f16, V>(r_in0") == 3
+    # (the last group of the row is ragged: the chunks' conditions are operands of the accesses, not branches around them)
+    assert src.count("load_raw_chunk_if<akg::f16, V, true>(b_in0, akg_ok[j], ") == 1 and src.count("unpack_chunk<akg::f16, V>(r_in0") == 3
     assert "load_chunk<akg::f16" not in src and src.count("forget_unpacked") == 2
     c, src = consts("small_layernorm_residual_bf16_2x57000")
     assert c["GROUPS"] == 4 and "r_in0[GROUPS * NCHUNK]" in src and "r_in3[GROUPS * NCHUNK]" in src and "r_in1" not in src
     # ... a longer one is re-read by every walk, with the non-temporal hint only in the last walk that reads it
     c, src = consts("small_layernorm_residual_bf16_2x66000")
     assert c["GROUPS"] == 3 and src.count("for (int akg_g = 0; akg_g < GROUPS") == 3 and "RawChunk" not in src
-    assert re.findall(r"load_chunk<akg::bf16, V, (true|false)>\(b_in0", src) == ["false", "false", "true"]
+    assert re.findall(r"load_chunk_if<akg::bf16, V, (true|false)>\(b_in0", src) == ["false", "false", "true"]
 
 
 def test_elementwise_dimension_folding():
@@ -861,7 +862,8 @@ def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
     """What a new shape set of a dynamic description costs: a device compilation only when the source changes. The leading
     extents (also of operands that span only some of them: a mask shared by the heads), the row count, the row length
     inside its power-of-two bucket of chunk counts, the rows of A of a MatMul and its K split are kernel arguments; what
-    still makes a new source is a row length in another bucket and a chunk width that stops dividing the rows. Counted
+    still makes a new source is a row length in another bucket, rows that are whole 64-byte pieces against rows that are
+    not, and a chunk width that stops dividing the rows. Counted
     on the shape sets the GPU tests use for the reference's ten dynamic descriptions (three each)."""
     monkeypatch.setenv("AKG_HIP_NO_CACHE", "0")
     shape_sets = {
@@ -889,9 +891,16 @@ def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
     dyn = driver.HipDynamicKernel(open(path, encoding="utf-8").read(), out_dir=None)
     first = dyn.specialize([[32, 1, 48, 48], [32, 12, 48, 48]])
     assert "akg_dim_arg0" in first.source and "akg_dim_arg2" in first.source
-    for shapes in ([[32, 1, 40, 40], [32, 12, 40, 40]], [[32, 1, 9, 48], [32, 12, 9, 48]]):
+    # rows that are whole 64-byte pieces (48 and 64 float32) have a source of their own inside the bucket: no chunk
+    # overlaps its neighbour there and whole lines are streamed
+    assert "akg_overlap" not in first.source
+    for shapes in ([[32, 1, 64, 64], [32, 12, 64, 64]], [[32, 1, 9, 48], [32, 12, 9, 48]]):
         k = dyn.specialize(shapes)
         assert k.cache_hit and k.source == first.source, shapes
+    ragged = dyn.specialize([[32, 1, 40, 40], [32, 12, 40, 40]])
+    assert not ragged.cache_hit and "akg_overlap" in ragged.source
+    k = dyn.specialize([[32, 1, 44, 44], [32, 12, 44, 44]])
+    assert k.cache_hit and k.source == ragged.source
 
 
 def test_streaming_and_column_kernels_take_their_open_extent_as_an_argument(monkeypatch):
