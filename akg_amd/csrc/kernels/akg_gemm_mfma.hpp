@@ -194,13 +194,14 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   const long kPerXcd = (kTiles + kGemmXcds - 1) / kGemmXcds;
   constexpr long kSteps = (K + BK - 1) / BK;
   constexpr bool kFull = !DYN && (MS % kGemmBM == 0) && (N % kGemmBN == 0) && (K % BK == 0);
-  // DYN with whole tiles along N and K: the loads need no checks either. Every thread clamps the rows of A it stages to
-  // the last row once, in front of the loop (the scalar offset of a buffer load takes no part in the descriptor's range
-  // check, so the descriptor alone would not keep the rows of a ragged last tile inside A); rows beyond M then hold
-  // copies of row M - 1 and their accumulators are dropped by the epilogue's row check. The main loop is the one of a
-  // static shape: no compares, one basic block per K step.
-  constexpr bool kLoadsInRange = kFull || (DYN && (N % kGemmBN == 0) && (K % BK == 0));
-  constexpr bool kClampRows = DYN && kLoadsInRange;
+  // Whole tiles along N and K, and an M that is an argument or leaves a ragged last tile behind full ones: the loads need
+  // no checks either. Every thread clamps the rows of A it stages to the last row once, in front of the loop (the scalar
+  // offset of a buffer load takes no part in the descriptor's range check, so the descriptor alone would not keep the
+  // rows of a ragged last tile inside A); rows beyond M then hold copies of row M - 1 and their accumulators are
+  // dropped by the epilogue's row check. The main loop is the one of a whole shape: no compares, one basic block per K
+  // step. (A single ragged tile, M < 256, keeps the checks: there the wavefronts without rows skip their MFMAs.)
+  constexpr bool kClampRows = !kFull && (DYN || MS > kGemmBM) && (N % kGemmBN == 0) && (K % BK == 0);
+  constexpr bool kLoadsInRange = kFull || kClampRows;
   constexpr int kTileBytes = kGemmBM * kPitch;        // one operand tile in LDS
   static_assert(kRowChunks == 4, "the staging schedule is written for four 16-byte chunks per thread and operand");
   // A row-major B goes to LDS as it lies in memory, k-rows of 256 columns. Sixteen lanes share a transposing read:
@@ -356,7 +357,7 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
 
   // Wavefronts whose rows all lie below the last row of A (a skinny A: M = 16 leaves three of the four wavefront rows
   // without a single real row) take part in the staging and the barriers but skip fragment reads and MFMAs.
-  constexpr bool kAllRowsReal = DYN ? kLoadsInRange : (MS % kGemmBM == 0);   // (DYN: every wavefront computes; M > 64 there)
+  constexpr bool kAllRowsReal = kClampRows || (!DYN && MS % kGemmBM == 0);   // (clamped rows: every wavefront computes)
   const bool waveHasRows = kAllRowsReal || (m0 + wm * kWaveRows < M);
   // A fragments of row half rh (2 tiles of 16 rows), K half kh (64 bytes)
   auto readA = [&](int buf, int kh, int rh, v4i (&af)[kHM]) {
