@@ -566,37 +566,70 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
       for (int i = 0; i < kTM; ++i) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          if (rowOk(i, v)) {
-            const typename Mma::acc_t a4[4] = {acc[i][4 * q][v], acc[i][4 * q + 1][v], acc[i][4 * q + 2][v], acc[i][4 * q + 3][v]};
-            ws_store_chunk<4>(wsBuf, tileBase + static_cast<u32>(ksplit * kPartBytes + partOffset(i, q, v)), a4);
-          }
+          // (a row beyond M stores to beyond the workspace, which drops it)
+          const typename Mma::acc_t a4[4] = {acc[i][4 * q][v], acc[i][4 * q + 1][v], acc[i][4 * q + 2][v], acc[i][4 * q + 3][v]};
+          ws_store_chunk<4>(wsBuf, rowOk(i, v) ? tileBase + static_cast<u32>(ksplit * kPartBytes + partOffset(i, q, v)) : kBeyondEveryBuffer, a4);
         }
       }
     }
     __shared__ unsigned akg_gemm_flag;
     if (!last_workgroup(ws, linear, kSplits, tid, &akg_gemm_flag)) return;
+    if constexpr (!DYN) {
+      // The number of splits is a constant: sum and epilogue per group of four accumulators, the loads of all splits of
+      // the group in flight together (the compiler unrolls the splits and overlaps the groups).
 #pragma unroll
-    for (int q = 0; q < kTN / 4; ++q) {
-      const long col4 = colBase + 64 * q;
-      if (!(kFull || col4 < N)) continue;
-      epi.prepare(col4);
+      for (int q = 0; q < kTN / 4; ++q) {
+        const long col4 = colBase + 64 * q;
+        if (!(kFull || col4 < N)) continue;
+        epi.prepare(col4);
+#pragma unroll
+        for (int i = 0; i < kTM; ++i) {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            if (!rowOk(i, v)) continue;
+            typename Mma::acc_t sum[4] = {0, 0, 0, 0};
+            for (int p = 0; p < kSplits; ++p) {
+              typename Mma::acc_t part[4];
+              ws_load_chunk<4>(wsBuf, tileBase + static_cast<u32>(p * kPartBytes + partOffset(i, q, v)), part);
+#pragma unroll
+              for (int c = 0; c < 4; ++c) sum[c] += part[c];
+            }
+            epi.apply(sum, m0 + rowInTileOf(i, v), col4);
+          }
+        }
+      }
+      return;
+    } else {
+      // The last workgroup of the tile: the sums of the partials, in split order, into the accumulators (this workgroup's
+      // own partial is among them). One round per split with every load of the round issued before the first addition
+      // (the number of splits may be an argument: a loop over the splits inside the loops over the accumulators would
+      // wait for every load by itself); a row beyond M loads from beyond the workspace, which reads zero.
 #pragma unroll
       for (int i = 0; i < kTM; ++i) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          if (!rowOk(i, v)) continue;
-          typename Mma::acc_t sum[4] = {0, 0, 0, 0};
-          for (int p = 0; p < kSplits; ++p) {
-            typename Mma::acc_t part[4];
-            ws_load_chunk<4>(wsBuf, tileBase + static_cast<u32>(p * kPartBytes + partOffset(i, q, v)), part);
+        for (int j = 0; j < kTN; ++j) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) sum[c] += part[c];
+          for (int v = 0; v < 4; ++v) acc[i][j][v] = 0;
+        }
+      }
+      for (int p = 0; p < kSplits; ++p) {
+        const u32 splitBase = tileBase + static_cast<u32>(p * kPartBytes);
+#pragma unroll
+        for (int q = 0; q < kTN / 4; ++q) {
+          if (!(kFull || colBase + 64 * q < N)) continue;
+#pragma unroll
+          for (int i = 0; i < kTM; ++i) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              typename Mma::acc_t part[4];
+              ws_load_chunk<4>(wsBuf, rowOk(i, v) ? splitBase + static_cast<u32>(partOffset(i, q, v)) : kBeyondEveryBuffer, part);
+#pragma unroll
+              for (int c = 0; c < 4; ++c) acc[i][4 * q + c][v] += part[c];
+            }
           }
-          epi.apply(sum, m0 + rowInTileOf(i, v), col4);
         }
       }
     }
-    return;
   }
 #pragma unroll
   for (int q = 0; q < kTN / 4; ++q) {
@@ -809,6 +842,42 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
     if (!last_workgroup(ws, group, kSplits, tid, &akg_skinny_flag)) return;
     if (!colOk) return;
     epi.prepare(col);
+    if constexpr (DYN) {
+      // the number of splits is an argument: rounds of two or four splits, the loads of all rows of a round issued
+      // together (a row beyond M loads from beyond the workspace, which reads zero); sums in split order, as below
+#pragma unroll
+      for (int i = 0; i < kRowsPerThread; ++i) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) sum[i][c] = 0;
+      }
+      constexpr int kRound = kRowsPerThread <= 4 ? 4 : 2;   // splits per round: at most 16 loads of 16 bytes in flight
+      for (int p0 = 0; p0 < kSplits; p0 += kRound) {
+        acc_t part[kRound][kRowsPerThread][4];
+#pragma unroll
+        for (int u = 0; u < kRound; ++u) {
+#pragma unroll
+          for (int i = 0; i < kRowsPerThread; ++i) {
+            const int row = r0 + 8 * i;
+            const bool there = row < M && p0 + u < kSplits;   // (a split beyond the last reads zero as well)
+            ws_load_chunk<4>(wsBuf, there ? base + static_cast<u32>((p0 + u) * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))) : kBeyondEveryBuffer, part[u][i]);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kRound; ++u) {
+#pragma unroll
+          for (int i = 0; i < kRowsPerThread; ++i) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) sum[i][c] += part[u][i][c];
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < kRowsPerThread; ++i) {
+        const int row = r0 + 8 * i;
+        if (row < M) epi.apply(sum[i], row, col);
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
       const int row = r0 + 8 * i;
