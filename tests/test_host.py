@@ -954,6 +954,23 @@ def test_streaming_and_column_kernels_take_their_open_extent_as_an_argument(monk
         assert all(k.source == seen[0].source for k in seen) and all(k.cache_hit for k in seen[1:]), kind
 
 
+def test_description_that_ended_the_device_compiler_with_slp_vectorisation(tmp_path, monkeypatch):
+    """A random description (bf16 operands, a Sub, casts through float16, a column sum with its reduced extent open) whose
+    kernel ended instruction selection with a fatal error - and the process with it - while the SLP vectoriser was on: it
+    formed a two-lane float32 subtraction that the backend cannot select with packed float32 operations switched off.
+    Device compiles run without that vectoriser; here the description must compile, and AKG_HIP_DUMP_SOURCE must leave
+    the source of what was compiled on disk (what names the culprit when a compiler does end the process)."""
+    import json
+    monkeypatch.setenv("AKG_HIP_DUMP_SOURCE", str(tmp_path))
+    monkeypatch.setenv("AKG_HIP_NO_CACHE", "1")
+    path = os.path.join(os.path.dirname(REF_INFO), "regress", "two_lane_float_sub_next_to_half_casts.dynamic.info")
+    dyn = driver.HipDynamicKernel(open(path, encoding="utf-8").read(), out_dir=None)
+    k = dyn.specialize([[8, 16, 33, 7], [1, 16, 33, 7]])
+    assert k.family == "stream_reduce" and not k.cache_hit
+    dumped = os.path.join(str(tmp_path), k.kernel_name + ".hip")
+    assert os.path.exists(dumped) and open(dumped, encoding="utf-8").read() == k.source
+
+
 def test_hardware_tanh_form_only_where_its_absolute_error_cannot_grow():
     """Values that only reach 16-bit outputs may use hardware approximations. The tanh form 1 - 2 / (e^2x + 1) is the one
     whose error is absolute (1.2e-7 near zero): it stays only where nothing can blow that up - GELU, whose factor x is what
