@@ -1222,6 +1222,20 @@ class TileEmitter {
       src_ << "  }\n";
       return;
     }
+    const bool anyOrder = spec.combiner == "akg::RedMax" || spec.combiner == "akg::RedMin";
+    if (anyOrder && (raggedCols_ || overlap_ > 0)) {
+      // A maximum or minimum does not depend on the order of its steps nor on an element taken twice (the elements a
+      // tail chunk shares with its neighbour): the chunk is folded by itself and joins the accumulator under the one
+      // condition of the chunk, instead of every element under its own.
+      line("#pragma unroll");
+      line("  for (int j = 0; j < NCHUNK; ++j) {");
+      src_ << "    " << computeTypeName(od) << " akg_part = " << in.ident << "[j][0];\n";
+      line("#pragma unroll");
+      src_ << "    for (int e = 1; e < V; ++e) akg_part = " << spec.combiner << "::apply(akg_part, " << in.ident << "[j][e]);\n";
+      src_ << "    if (akg_ok[j]) " << acc << " = " << spec.combiner << "::apply(" << acc << ", akg_part);\n";
+      line("  }");
+      return;
+    }
     line("#pragma unroll");
     line("  for (int j = 0; j < NCHUNK; ++j) {");
     line("#pragma unroll");
