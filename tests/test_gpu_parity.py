@@ -433,6 +433,16 @@ def test_tensors_of_two_gib_and_more_are_addressed_with_64_bit_offsets(tmp_path)
     got = run_on_gpu(kernel, [xs, vs])[0]
     expect = cpu_ref.CpuKernel(path, openmp=True, rebuild=True)([xs, vs])[0]
     assert np.array_equal(got, expect)
+    del got
+    # the same description with its row count open: the row count is a kernel argument, the addressing stays 64-bit
+    print("case big bias add, rows open", flush=True)
+    b = op_desc.DescBuilder("big_bias_add_rows_open_f32")
+    x, v = b.input([7777, cols], "float32"), b.input([cols], "float32")
+    dyn = driver.HipDynamicKernel(open_extent(b.dumps([b.add(x, v)]), 7777), out_dir=None)
+    kernel = dyn.specialize([[rows, cols], [cols]])
+    assert "make_buffer" not in kernel.source and "akg_extent" in kernel.source
+    got = run_on_gpu(kernel, [xs, vs])[0]
+    assert np.array_equal(got, expect)
     del got, expect
     print("case big column sum", flush=True)
     text = op_desc.square_reduce([rows, cols], [0], "float32", False, "ReduceSum", name="big_colsum_f32_%dx%d" % (rows, cols))
