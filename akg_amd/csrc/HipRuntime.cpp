@@ -558,6 +558,19 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
       fromMemory = true;
     }
   }
+  if (!k->cacheHit && !dir.empty() && !(std::getenv("AKG_HIP_NO_CACHE") && std::getenv("AKG_HIP_NO_CACHE")[0] == '1')) {
+    // code objects compiled by any process that used this artifact directory, by source digest: a shape set this
+    // process meets for the first time may share its source with one another process has compiled
+    std::string code;
+    if (readFile(dir + "/by_source/" + srcDigest + ".hsaco", &code) && !code.empty()) {
+      k->codeObject = std::make_shared<const std::vector<char>>(code.begin(), code.end());
+      k->codeSha256 = akg::Sha256::of(code);
+      k->cacheHit = true;
+      fromMemory = true;
+      std::lock_guard<std::mutex> lock(g_codeCacheMutex);
+      if (g_codeCache.size() < 1024) g_codeCache[srcDigest] = k->codeObject;
+    }
+  }
   if (!k->cacheHit || (fromMemory && !base.empty())) {
     std::string log;
     int rc = AKG_HIP_OK;
@@ -583,8 +596,13 @@ int doCompileTimed(const std::string &jsonText, const char *outDir, akg_hip_kern
     h.update(k->codeObject->data(), k->codeObject->size());
     k->codeSha256 = h.hexDigest();
     if (!fromMemory) {
-      std::lock_guard<std::mutex> lock(g_codeCacheMutex);
-      if (g_codeCache.size() < 1024) g_codeCache[srcDigest] = k->codeObject;   // bounded: some tens of MB at most
+      {
+        std::lock_guard<std::mutex> lock(g_codeCacheMutex);
+        if (g_codeCache.size() < 1024) g_codeCache[srcDigest] = k->codeObject;   // bounded: some tens of MB at most
+      }
+      if (!dir.empty() && makeDirs(dir + "/by_source")) {
+        (void)writeFile(dir + "/by_source/" + srcDigest + ".hsaco", k->codeObject->data(), k->codeObject->size());
+      }
     }
     if (!base.empty()) {
       std::string meta = metaJson(*k, srcDigest);

@@ -858,6 +858,26 @@ def test_cli_tool():
     assert r.returncode == 1 and "2 inputs" in r.stderr
 
 
+def test_code_objects_are_found_by_source_digest_across_processes(tmp_path):
+    """The artifact directory also keeps every code object under the digest of its source (by_source/): a process that
+    meets a shape set for the first time finds the code another process compiled for a different shape set with the
+    same source, and compiles nothing. Two runs of the command line tool; AKG_HIP_NO_CACHE=1 still compiles."""
+    tool = os.path.join(ROOT, "akg_amd", "akg-hip")
+    dynamic = os.path.join(REF_INFO, "Fused_Sub_Mul_Mul_Add_Softmax_fusion_13911402818667958957.dynamic.info")
+    env = {k: v for k, v in os.environ.items() if k != "AKG_HIP_NO_CACHE"}
+    out = str(tmp_path / "meta")
+
+    def hit(shapes, extra_env=None):
+        r = subprocess.run([tool, "compile", dynamic, "--shapes", shapes, "-o", out], capture_output=True, text=True,
+                           env=dict(env, **(extra_env or {})))
+        assert r.returncode == 0, r.stderr
+        return [l for l in r.stdout.splitlines() if l.startswith("cache hit")][0].split()[-1]
+    assert hit("32,1,48,48;32,12,48,48") == "0"
+    assert hit("32,1,9,48;32,12,9,48") == "1"           # another shape set, another process, the same source
+    assert len(os.listdir(os.path.join(out, "by_source"))) == 1
+    assert hit("32,1,7,48;32,12,7,48", {"AKG_HIP_NO_CACHE": "1"}) == "0"
+
+
 def test_dynamic_descriptions_share_code_objects_across_shape_sets(monkeypatch):
     """What a new shape set of a dynamic description costs: a device compilation only when the source changes. The leading
     extents (also of operands that span only some of them: a mask shared by the heads), the row count, the row length
