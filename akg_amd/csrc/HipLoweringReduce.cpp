@@ -766,10 +766,24 @@ class StreamReduceEmitter {
     for (int id : g_.inputs) useBuffers_ = useBuffers_ && !tooLarge(id);
     for (int id : g_.outputs) useBuffers_ = useBuffers_ && !tooLarge(id);
     // bytes of a tensor: a constant, or (the reduced extent being an argument) that extent times the bytes per index
-    auto bytesOf = [&](const TensorValue &t) {
+    // (an output has the shape of the reduced value - the kept extents, whatever its own extents happen to equal - or
+    // the shape of the reduced operand; inputs are placed in the iteration space as their offsets place them)
+    auto bytesOf = [&](int id, bool isOutput) {
+      const TensorValue &t = g_.tensor(id);
       int64_t bytes = t.numel() * static_cast<int64_t>(dtypeSize(t.dtype));
-      if (!dynR_ || !t.used) return std::to_string(bytes) + "L";
-      const std::vector<int64_t> s = padTo(t.shape, "tensor " + t.name);
+      if (!dynR_ || (!t.used && !isOutput)) return std::to_string(bytes) + "L";
+      std::vector<int64_t> s;
+      bool assignedTo = false;   // the destination of an Assign has the shape of the reduced value as well
+      for (const OpNode &op : g_.ops) assignedTo = assignedTo || (op.kind == OpKind::Assign && op.inputs[0] == id);
+      if (isOutput || assignedTo) {
+        s.assign(space_.size(), 1);
+        const bool full = isOutput && phase_[static_cast<size_t>(id)] == Phase::Pre;
+        for (size_t d = 0; d < space_.size(); ++d) {
+          if (kind_[d] >= 0 && (full || kind_[d] != 1)) s[d] = space_[d];
+        }
+      } else {
+        s = padTo(t.shape, "tensor " + t.name);
+      }
       std::string e;
       if (s[static_cast<size_t>(dynDim_)] != 1) {
         // the open extent itself: the reduced extent over what the other reduced dims contribute to it
@@ -785,10 +799,10 @@ class StreamReduceEmitter {
     };
     if (useBuffers_) {
       for (size_t i = 0; i < g_.inputs.size(); ++i) {
-        src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", " << bytesOf(g_.tensor(g_.inputs[i])) << ");\n";
+        src_ << "  const akg::Buffer b_in" << i << " = akg::make_buffer(in" << i << ", " << bytesOf(g_.inputs[i], false) << ");\n";
       }
       for (size_t i = 0; i < g_.outputs.size(); ++i) {
-        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", " << bytesOf(g_.tensor(g_.outputs[i])) << ");\n";
+        src_ << "  const akg::Buffer b_out" << i << " = akg::make_buffer(out" << i << ", " << bytesOf(g_.outputs[i], true) << ");\n";
       }
     }
     src_ << "  constexpr int V = " << vec_ << ";\n";

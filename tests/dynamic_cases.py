@@ -81,10 +81,19 @@ def _scaled_pool_over_tokens(b_, t, name):
     return b.dumps([b.add(b.reduce("ReduceSum", b.mul(x, w), [1], True), c)])
 
 
+def _rowmax_with_equal_outer_and_inner_extents(b_, t, name):
+    # [b, t, b] reduced over its two trailing axes without keep_dims: the result [b] has the extent of the innermost,
+    # reduced axis as well as that of the kept one (its size in bytes must follow the kept one)
+    b = op_desc.DescBuilder(name)
+    x = b.cast(b.input([b_, t, b_], "bfloat16"), "float32")
+    return b.dumps([b.cast(b.reduce("ReduceMax", b.mul(x, x), [1, 2], False), "bfloat16")])
+
+
 # (outer extent, reduced extent) both open: [O, R, I] reduced over R
 DYNAMIC_POOLS = {
     "pool_f16": _pool_over_tokens,
     "scaled_pool_f32": _scaled_pool_over_tokens,
+    "rowmax_equal_extents_bf16": _rowmax_with_equal_outer_and_inner_extents,
 }
 
 # the batch of [N,C,H,W] statistics open: the reduced extent N * H * W is an argument, the channel extent lies between

