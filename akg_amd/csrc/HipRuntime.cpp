@@ -10,7 +10,9 @@
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 #include <sys/stat.h>
+#include <unistd.h>
 
+#include <atomic>
 #include <cerrno>
 #include <chrono>
 #include <cstdio>
@@ -157,14 +159,19 @@ bool readFile(const std::string &path, std::string *out) {
 }
 
 bool writeFile(const std::string &path, const void *data, size_t len) {
-  std::string tmp = path + ".tmp";
+  // (a temporary name of this process and call: several processes may fill one artifact directory at once, and two
+  // writers of one temporary file could publish it half written)
+  static std::atomic<unsigned long> serial{0};
+  std::string tmp = path + ".tmp." + std::to_string(static_cast<long>(getpid())) + "." + std::to_string(serial.fetch_add(1));
   {
     std::ofstream f(tmp, std::ios::binary | std::ios::trunc);
     if (!f) return false;
     f.write(static_cast<const char *>(data), static_cast<std::streamsize>(len));
     if (!f) return false;
   }
-  return std::rename(tmp.c_str(), path.c_str()) == 0;
+  if (std::rename(tmp.c_str(), path.c_str()) == 0) return true;
+  (void)std::remove(tmp.c_str());
+  return false;
 }
 
 bool makeDirs(const std::string &dir) {
