@@ -272,6 +272,13 @@ std::string metaJson(const akg_hip_kernel &k, const std::string &srcDigest) {
   os << "\"algorithmic_bytes\": " << k.lowered.algorithmicBytes << ", ";
   os << "\"algorithmic_ops\": " << k.lowered.algorithmicOps << ", ";
   os << "\"workspace_bytes\": " << k.lowered.workspaceBytes << ", ";
+  if (!k.lowered.scalarArgs.empty()) {
+    // a specialisation of a dynamic description whose kernel takes extents as arguments: these 64-bit values follow
+    // the tensor pointers in the kernel's argument list (the workspace pointer, if any, comes last)
+    os << "\"scalar_args\": [";
+    for (size_t i = 0; i < k.lowered.scalarArgs.size(); ++i) os << (i ? ", " : "") << k.lowered.scalarArgs[i];
+    os << "], ";
+  }
   if (!k.stages.empty()) {
     // the description runs as these kernels, in this order, each with artifacts of its own under its name; "args" says
     // where each tensor of a stage's signature lives: input i / output j of this description, or temporary t at a byte

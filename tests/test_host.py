@@ -873,6 +873,9 @@ def test_code_objects_are_found_by_source_digest_across_processes(tmp_path):
         assert r.returncode == 0, r.stderr
         return [l for l in r.stdout.splitlines() if l.startswith("cache hit")][0].split()[-1]
     assert hit("32,1,48,48;32,12,48,48") == "0"
+    # the artifacts of a specialisation say which extents its kernel takes as arguments behind the tensor pointers
+    metas = [json.load(open(os.path.join(out, f))) for f in os.listdir(out) if f.endswith(".json") and "shape_info" not in f]
+    assert len(metas) == 1 and metas[0]["scalar_args"] == [32 * 12 * 48, 48, 32, 12, 48]
     assert hit("32,1,9,48;32,12,9,48") == "1"           # another shape set, another process, the same source
     assert len(os.listdir(os.path.join(out, "by_source"))) == 1
     assert hit("32,1,7,48;32,12,7,48", {"AKG_HIP_NO_CACHE": "1"}) == "0"
