@@ -422,6 +422,9 @@ class TileEmitter {
           }
         }
       }
+      if (opt_.threadsPerRow == 0 && !ordered_ && rowChunks > 2048 && rowChunks <= 4096 && normalisationLike()) {
+        tpr = 512;   // (32768-wide bf16 LayerNorm + residual: 74.9 -> 71.0 us; 65536-wide stays on 1024 threads)
+      }
       if (ordered_ && opt_.threadsPerRow == 0) {
         // one thread folds a row while the row's other threads wait: as few threads per row as keep it in registers
         for (int t = 1; t <= 1024; t <<= 1) {
@@ -447,7 +450,10 @@ class TileEmitter {
       // 32768-wide f16 softmax 67.8 / 70.0, 65536-wide 62.1 / 66.4, 32768-wide LayerNorm 69.6 / 67.4; at 16384 and
       // below the same within a point or two. So rows of 16-bit inputs on 1024 threads go packed from 64 values per
       // thread on.
-      const bool preferPacked = rowPasses == 0 && tpr_ == 1024 && perThread * vec_ * rowInputs >= 64;
+      // (a single row-sized input goes packed from 32 values per thread on: 32768-wide f16 softmax 49.1 -> 47.9 us,
+      // bf16 RMSNorm 49.1 -> 46.4 us; at 16 values the float row is ahead or level)
+      const bool preferPacked = rowPasses == 0 && tpr_ == 1024 &&
+                                (perThread * vec_ * rowInputs >= 64 || (rowInputs == 1 && perThread * vec_ >= 32));
       if ((multiPass_ || preferPacked) && useBuffers_ && rowPasses != 2) {
         // registers (32-bit) per thread for the packed row; 64 leave room for one group's float values
         int64_t packedRegs = 0;
