@@ -503,6 +503,15 @@ class TileEmitter {
       block_ = opt_.block > 0 ? opt_.block : 256;
       if (block_ % 64 != 0 || block_ > 1024) block_ = 256;
       int chunks = opt_.chunks > 0 ? opt_.chunks : std::max(1, 16 / vec_);
+      // An operand that is broadcast over the iteration space (a bias per column, a scale per row) is loaded again
+      // for every chunk of a thread, and those chunks lie a whole workgroup's width apart: one chunk per thread then
+      // (bias + activation on 64 M bf16 elements 43.6 -> 41.9 us, on 16 M float32 elements 23.6 -> 22.2 us).
+      if (opt_.chunks == 0) {
+        for (size_t i = 0; i < g_.inputs.size(); ++i) {
+          const TensorValue &t = g_.tensor(g_.inputs[i]);
+          if (t.used && t.numel() > 1 && t.numel() != numel_) chunks = 1;
+        }
+      }
       // Small problems: fewer chunks per thread so the grid still covers the chip.
       if (extentArg_ && opt_.chunks == 0) {
         // a dynamic description: two sizes only (the source must not follow every element count)
