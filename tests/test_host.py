@@ -248,6 +248,12 @@ def test_streaming_reduction_family_and_schedule():
     # the same reduction along the innermost axis with rows that fit in registers stays in the row family
     k = driver.HipKernel.from_file(os.path.join(FIXTURES, "small_softmax_f32_5x77.info"))
     assert k.family == "row_reduce" and k.workspace_bytes == 0
+    # The streaming loop issues a trip's loads together, conditions as operands, before the work on any of them; the
+    # depth of a trip is picked so that the last one is full (49 chunks per thread: 7 trips of 7, not 13 of 4).
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n5_bnstats_bf16_256x64x56x56.info"))
+    assert "constexpr int U = 7;" in k.source and "t_in0[U][V]" in k.source
+    loads, work = k.source.index("load_chunk_if<akg::bf16, V, true>(b_in0, akg_in"), k.source.index("if (akg_in) acc0 =")
+    assert loads < work and k.source.count("for (int u = 0; u < U; ++u)") == 2
 
 
 def test_assign_after_a_streaming_reduction_stores_over_its_input():
