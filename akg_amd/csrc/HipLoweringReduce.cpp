@@ -511,8 +511,12 @@ class StreamReduceEmitter {
       split_ = 1;
     } else if (dirY_) {
       // A workgroup is TR thread-rows of LANES lanes; a lane owns V adjacent columns. Narrow strips (16 lanes = one
-      // 256-byte run per row) give many groups, so few workgroups share a group and the partials stay small.
-      int lanes = opt_.threadsPerRow > 0 ? opt_.threadsPerRow : 16;
+      // 256-byte run per row) give many groups, so few workgroups share a group and the partials stay small. Where
+      // that makes more groups than half the workgroups aimed at (the grid then overshoots), strips of 32 lanes are
+      // faster (bf16 [64,2048,1024] over axis 1: 43.6 -> 41.4 us, [256,512,1024]: 45.5 -> 40.2, f16 [48,1024,4096]:
+      // 65.4 -> 57.2, float32 [256,128,4096]: 84.2 -> 82.7); where it does not, they are not (float32 [4,16384,768]:
+      // 33.1 -> 36.2, f16 [8,8192,4096]: 79.0 -> 80.3).
+      int lanes = opt_.threadsPerRow > 0 ? opt_.threadsPerRow : (O_ * ceilDivL(I_, 16 * static_cast<int64_t>(vec_)) > targetGroups / 2 ? 32 : 16);
       lanes = std::max(1, std::min(lanes, 64));
       if ((lanes & (lanes - 1)) != 0) lanes = 16;
       lanes_ = static_cast<int>(std::min<int64_t>(lanes, pow2AtLeastL(ceilDivL(I_, vec_))));
