@@ -565,7 +565,7 @@ class StreamReduceEmitter {
       // The loop takes `unroll_` chunks per trip and the last trip's empty slots still issue: between the depth above
       // and twice that, the one that leaves the fewest empty (49 chunks per thread: seven trips of 7, 69.6 % of the
       // HBM peak on bf16 [256,64,56,56]; thirteen of 4: 68.0 %).
-      if (opt_.chunks == 0 && !dynR_ && !overlapRun_ && unroll_ > 1) {
+      if (opt_.chunks == 0 && !dynR_ && unroll_ > 1) {
         const int64_t perThread = rps_ / chunk;
         int best = unroll_;
         int64_t bestIdle = ceilDivL(perThread, best) * best - perThread;
@@ -958,26 +958,41 @@ class StreamReduceEmitter {
     }
     // ---- streaming loop
     if (ordered_ && !dirY_) line("  __shared__ __attribute__((aligned(16))) unsigned short akg_chain[BLOCK * V];");
-    batched_ = useBuffers_ && !ordered_ && !overlapRun_ && unroll_ > 1;
+    // (short runs, 7 x 7 or 14 x 14 images, spend their time on the index split and gain nothing: 2 to 4 % slower)
+    batched_ = useBuffers_ && !ordered_ && unroll_ > 1 && (!overlapRun_ || runChunks_ >= 64);
     if (batched_) {
       src_ << "  constexpr int U = " << unroll_ << ";\n";
-      const std::string stepExpr = dirY_ ? "static_cast<long>(TR)" : "static_cast<long>(BLOCK) * V";
+      // where chunk u of the trip lies and whether it is inside the workgroup's slice
+      auto place = [&](const std::string &in) {
+        if (overlapRun_) {
+          src_ << in << "const long akg_slot = r0 + u * static_cast<long>(BLOCK);\n";
+          src_ << in << "const bool akg_in = akg_slot < r_end;\n";
+          src_ << in << "const int akg_run = static_cast<int>(akg_slot) / RUN_CHUNKS;\n";
+          src_ << in << "int akg_start = (static_cast<int>(akg_slot) % RUN_CHUNKS) * V;\n";
+          src_ << in << "const bool akg_tail = akg_start > RUN - V;\n";
+          src_ << in << "if (akg_tail) akg_start = RUN - V;\n";
+          src_ << in << "const long r = static_cast<long>(akg_run) * RUN + akg_start;\n";
+        } else {
+          src_ << in << "const long r = r0 + u * " << (dirY_ ? "static_cast<long>(TR)" : "static_cast<long>(BLOCK) * V") << ";\n";
+          src_ << in << "const bool akg_in = r < r_end;\n";
+        }
+      };
       if (dirY_) {
         line("  for (long r0 = r_begin + tr; r0 < r_end; r0 += static_cast<long>(TR) * U) {");
+      } else if (overlapRun_) {
+        line("  for (long r0 = r_begin + tid; r0 < r_end; r0 += static_cast<long>(BLOCK) * U) {   // in chunk slots");
       } else {
         line("  for (long r0 = r_begin + static_cast<long>(tid) * V; r0 < r_end; r0 += static_cast<long>(BLOCK) * V * U) {");
       }
       for (size_t i : inputsUsedIn(Phase::Pre)) src_ << "    " << ctOf(g_.inputs[i]) << " t_in" << i << "[U][V];\n";
       line("#pragma unroll");
       line("    for (int u = 0; u < U; ++u) {");
-      src_ << "      const long r = r0 + u * " << stepExpr << ";\n";
-      line("      const bool akg_in = r < r_end;");
+      place("      ");
       for (size_t i : inputsUsedIn(Phase::Pre)) emitInputLoad(i, "akg_o", "r", dirY_ ? "akg_i" : "", "", false, "      ", true);
       line("    }");
       line("#pragma unroll");
       line("    for (int u = 0; u < U; ++u) {");
-      src_ << "    const long r = r0 + u * " << stepExpr << ";\n";
-      line("    const bool akg_in = r < r_end;");
+      place("    ");
     } else {
       line("#pragma unroll " + std::to_string(ordered_ && !dirY_ ? 1 : unroll_));
     }
@@ -1026,7 +1041,8 @@ class StreamReduceEmitter {
           continue;
         }
         src_ << in4 << "#pragma unroll\n";
-        src_ << in4 << "for (int e = 0; e < V; ++e) " << (overlapRun_ ? "if (!akg_tail || e >= OVERLAP) " : ((ordered_ && !dirY_) || batched_ ? "if (akg_in) " : "")) << accName
+        src_ << in4 << "for (int e = 0; e < V; ++e) " << (overlapRun_ ? (batched_ ? "if (akg_in && (!akg_tail || e >= OVERLAP)) " : "if (!akg_tail || e >= OVERLAP) ")
+                                       : ((ordered_ && !dirY_) || batched_ ? "if (akg_in) " : "")) << accName
              << " = " << step << ";\n";
         continue;
       }

@@ -76,6 +76,9 @@ FIXTURES = {
     "small_reduceall_sqsum_f32_768x512": lambda n: op_desc.square_reduce([768, 512], [0, 1], "float32", False, "ReduceSum", n),
     "small_reduceall_min_f32_7x333": lambda n: op_desc.square_reduce([7, 333], [0, 1], "float32", False, "ReduceMin", n),
     "small_reducex_long_sqsum_f32_3x300000": lambda n: op_desc.square_reduce([3, 300000], [1], "float32", False, "ReduceSum", n),
+    # rows and runs that are long and no multiple of the chunk: walked in chunk slots, the last one of a run overlapping
+    "small_reducex_long_sqsum_f16_5x40001": lambda n: op_desc.square_reduce([5, 40001], [1], "float16", False, "ReduceSum", n),
+    "small_bnstats_bf16_4x6x35x35": lambda n: op_desc.batchnorm_stats(4, 6, 35, 35, "bfloat16", n),
     # kept axes between reduced ones: batch-norm statistics (contiguous runs of H*W), and a [4,5,6,16] sum over axes 0, 2
     "small_bnstats_bf16_8x6x7x12": lambda n: op_desc.batchnorm_stats(8, 6, 7, 12, "bfloat16", n),
     "small_bnstats_update_bf16_8x6x7x12": lambda n: op_desc.batchnorm_stats_update(8, 6, 7, 12, "bfloat16", 0.9, n),
