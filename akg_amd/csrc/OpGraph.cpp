@@ -189,6 +189,14 @@ class GraphBuilder {
         throw TranslateError("tensor " + name + ": dynamic dimensions (-1) need the shapes of a call: a dynamic description "
                              "goes through akg_hip_dynamic_create / akg_hip_dynamic_specialize (akg-hip --shapes)");
       }
+      // No schedule is made for nothing: the graphs the reference cuts its fused operators from hold no empty tensor.
+      if (d == 0) throw TranslateError("tensor " + name + ": an extent of 0 (empty tensors have no kernel)");
+    }
+    // Beyond what any device holds the schedules' 64-bit products would wrap: 2^40 elements is the limit.
+    int64_t count = 1;
+    for (int64_t d : shape) {
+      if (d > (1LL << 40) / count) throw TranslateError("tensor " + name + ": more than 2^40 elements");
+      count *= d;
     }
     TensorValue t;
     t.name = name;
@@ -312,6 +320,23 @@ class GraphBuilder {
           if (node.kind == OpKind::SegmentSum && j > 1) continue;    // the segment count carried as a constant
           if (node.kind == OpKind::Assign && j > 1) continue;        // convertInplaceAssignOp keeps two operands (:1104-1115)
           node.inputs.push_back(operandFor(inputDesc[j][0], node.name));
+        }
+      }
+
+      if (node.kind != OpKind::Unknown && node.kind != OpKind::Unsupported) {
+        // how many operands the op's kind reads; everything behind the translator indexes them without looking
+        const int k = static_cast<int>(node.kind);
+        size_t least = 1, most = 1;
+        if (k >= static_cast<int>(OpKind::Add) && k <= static_cast<int>(OpKind::LogicalOr)) least = most = 2;
+        if (node.kind == OpKind::Select) least = most = 3;
+        if (node.kind == OpKind::MatMul || node.kind == OpKind::Gather || node.kind == OpKind::SegmentSum ||
+            node.kind == OpKind::Assign) {
+          least = most = 2;
+        }
+        if (node.kind == OpKind::Concat || node.kind == OpKind::AddN) most = static_cast<size_t>(-1);
+        if (node.inputs.size() < least || node.inputs.size() > most) {
+          throw TranslateError("op " + node.name + ": " + std::to_string(node.inputs.size()) + " operands where " +
+                               (most == least ? std::to_string(least) : "at least " + std::to_string(least)) + " are read");
         }
       }
 

@@ -129,6 +129,36 @@ def test_error_conventions():
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(_desc(lambda d: d.pop("process")), out_dir=None)
     assert "process" in str(e.value)
+    # an empty tensor -> translate error, for every family (no schedule divides by an extent of 0)
+    for make in (lambda: op_desc.elementwise_tanh_add_mul(7, 128, "z_ew"), lambda: op_desc.softmax_last_axis(7, 128, "float16", "z_sm"),
+                 lambda: op_desc.square_reduce([7, 128], [0], "float32", False, "ReduceSum", "z_red"),
+                 lambda: op_desc.transpose_bias_add(2, 7, 128, "bfloat16", "z_tr"),
+                 lambda: op_desc.gemm_bias_act(7, 128, 64, "bfloat16", "gelu", False, "float32", "z_gemm"),
+                 lambda: op_desc.gemm_bias_act(8, 7, 64, "bfloat16", "gelu", False, "float32", "z_gemm_k")):
+        desc = json.loads(make())
+
+        def empty(node):
+            if isinstance(node, dict):
+                if isinstance(node.get("shape"), list):
+                    node["shape"] = [0 if d == 7 else d for d in node["shape"]]
+                for v in node.values():
+                    empty(v)
+            elif isinstance(node, list):
+                for v in node:
+                    empty(v)
+        empty(desc)
+        text = json.dumps(desc)
+        assert any(0 in e[0]["shape"] for e in desc["input_desc"])
+        with pytest.raises(driver.AkgHipError) as e:
+            driver.HipKernel(text, out_dir=None)
+        assert e.value.code == -3 and "extent of 0" in str(e.value)
+    # an op with fewer operands than its kind reads, and a tensor no device holds -> translate errors
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(_desc(lambda d: d["op_desc"][0].update(name="MatMul", input_desc=d["op_desc"][0]["input_desc"][:1])), out_dir=None)
+    assert e.value.code == -3 and "operands" in str(e.value)
+    with pytest.raises(driver.AkgHipError) as e:
+        driver.HipKernel(_desc(lambda d: d["input_desc"][0][0].update(shape=[2 ** 31, 2 ** 31])), out_dir=None)
+    assert e.value.code == -3 and "2^40" in str(e.value)
     # dtype outside the type table -> translate error
     with pytest.raises(driver.AkgHipError) as e:
         driver.HipKernel(_desc(lambda d: d["input_desc"][0][0].update(data_type="complex64")), out_dir=None)
