@@ -1061,6 +1061,13 @@ AKG_DEV void ws_load_chunk(Buffer ws, u32 off, T (&v)[V]) {
   __builtin_memcpy(v, raw, kBytes);
 }
 
+// ... or, where `ok` is false, nothing: the load is issued beyond the buffer and leaves zeros (no branch around it, so
+// that the loads of a trip go out together).
+template <int V, typename T>
+AKG_DEV void ws_load_chunk_if(Buffer ws, bool ok, u32 off, T (&v)[V]) {
+  ws_load_chunk<V>(ws, ok ? off : kBeyondEveryBuffer, v);
+}
+
 // True in every thread of exactly one workgroup out of the `split` that share counter `group`: the last to arrive.
 // Must be reached by all threads of the workgroup, after their ws_store / ws_store_chunk calls.
 AKG_DEV bool last_workgroup(unsigned *counters, long group, int split, int tid, unsigned *flag) {
