@@ -111,6 +111,9 @@ class GemmEmitter {
   int skinnyRows() const { return 64; }   // (96 rows: no faster than the tile kernel; 128: slower)
   int skinnyWaves() const { return opt_.block == 512 ? 8 : 4; }
   int skinnyUnroll() const { return opt_.chunks > 0 ? opt_.chunks : 2; }
+  // A [N,K] weight is read in 32-byte pieces, four per cache line, by instructions that follow each other: with the
+  // non-temporal hint the line is not kept for the next piece (bf16 16 x 8192 x 8192: 71 us with the hint, 37 without).
+  bool skinnyNonTemporal() const { return opt_.nonTemporal != 0 && !transB_; }
   bool serial_ = false;  // no MFMA kernel takes the description: gemm_serial (akg_gemm_serial.hpp)
   int epiWidth() const { return (serial_ && n_ % 4 != 0) ? 1 : 4; }   // adjacent result columns per epilogue call
   bool skinny_ = false;  // M <= 64: the kernel that streams B straight into MFMA operands (gemm_skinny)
@@ -494,12 +497,12 @@ class GemmEmitter {
     if (skinny_) {
       if (dyn_) {
         src_ << "  akg::gemm_skinny<" << mmaTraits() << ", " << skinnyBucket() << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-             << ", Epilogue, 1, " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (opt_.nonTemporal != 0 ? "true" : "false") << ", true>(in"
+             << ", Epilogue, 1, " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (skinnyNonTemporal() ? "true" : "false") << ", true>(in"
              << g_.tensor(aId_).inputIndex << ", in" << g_.tensor(bId_).inputIndex << ", epi, akg_ws, 0L, akg_m, static_cast<int>(akg_ksplit));\n}\n";
         return;
       }
       src_ << "  akg::gemm_skinny<" << mmaTraits() << ", " << m_ << "L, " << n_ << "L, " << k_ << "L, " << (transB_ ? "true" : "false")
-           << ", Epilogue, " << kSplit_ << ", " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (opt_.nonTemporal != 0 ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in"
+           << ", Epilogue, " << kSplit_ << ", " << skinnyWaves() << ", " << skinnyUnroll() << ", " << (skinnyNonTemporal() ? "true" : "false") << ">(in" << g_.tensor(aId_).inputIndex << " + akg_batch * " << m_ * k_ << "L, in"
            << g_.tensor(bId_).inputIndex << " + akg_batch * " << k_ * n_ << "L, epi, " << (kSplit_ > 1 ? "akg_ws" : "nullptr")
            << ", akg_batch * " << (n_ + 127) / 128 << "L);\n}\n";
       return;

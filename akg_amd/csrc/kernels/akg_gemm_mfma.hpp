@@ -776,6 +776,8 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
       for (int c = 0; c < 4; ++c) acc[rt][c] = Mma::mma(r.a[rt], b[c], acc[rt][c]);
     }
   };
+  // (For a [N,K] weight, whose columns are contiguous along K, giving a wavefront a run of adjacent steps instead of
+  // every fourth changes nothing: 36.9 us either way on bf16 16 x 8192 x 8192; the L1 merges the pieces of a line.)
   for (long t = t0 + wave; t < t1; t += kWaves * U) {   // (uniform per wavefront)
     Raw r[U];
 #pragma unroll
@@ -842,54 +844,39 @@ AKG_DEV void gemm_skinny(const void *__restrict__ Av, const void *__restrict__ B
     if (!last_workgroup(ws, group, kSplits, tid, &akg_skinny_flag)) return;
     if (!colOk) return;
     epi.prepare(col);
-    if constexpr (DYN) {
-      // the number of splits is an argument: rounds of two or four splits, the loads of all rows of a round issued
-      // together (a row beyond M loads from beyond the workspace, which reads zero); sums in split order, as below
+    // Rounds of two or four splits, the loads of all rows of a round issued together (a row beyond M or a split beyond
+    // the last loads from beyond the workspace, which reads zero); sums in split order, whether the number of splits
+    // is an argument or a constant.
 #pragma unroll
-      for (int i = 0; i < kRowsPerThread; ++i) {
+    for (int i = 0; i < kRowsPerThread; ++i) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) sum[i][c] = 0;
-      }
-      constexpr int kRound = kRowsPerThread <= 4 ? 4 : 2;   // splits per round: at most 16 loads of 16 bytes in flight
-      for (int p0 = 0; p0 < kSplits; p0 += kRound) {
-        acc_t part[kRound][kRowsPerThread][4];
+      for (int c = 0; c < 4; ++c) sum[i][c] = 0;
+    }
+    constexpr int kRound = kRowsPerThread <= 4 ? 4 : 2;   // splits per round: at most 16 loads of 16 bytes in flight
+    for (int p0 = 0; p0 < kSplits; p0 += kRound) {
+      acc_t part[kRound][kRowsPerThread][4];
 #pragma unroll
-        for (int u = 0; u < kRound; ++u) {
+      for (int u = 0; u < kRound; ++u) {
 #pragma unroll
-          for (int i = 0; i < kRowsPerThread; ++i) {
-            const int row = r0 + 8 * i;
-            const bool there = row < M && p0 + u < kSplits;   // (a split beyond the last reads zero as well)
-            ws_load_chunk<4>(wsBuf, there ? base + static_cast<u32>((p0 + u) * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))) : kBeyondEveryBuffer, part[u][i]);
-          }
-        }
-#pragma unroll
-        for (int u = 0; u < kRound; ++u) {
-#pragma unroll
-          for (int i = 0; i < kRowsPerThread; ++i) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) sum[i][c] += part[u][i][c];
-          }
+        for (int i = 0; i < kRowsPerThread; ++i) {
+          const int row = r0 + 8 * i;
+          const bool there = row < M && p0 + u < kSplits;
+          ws_load_chunk<4>(wsBuf, there ? base + static_cast<u32>((p0 + u) * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))) : kBeyondEveryBuffer, part[u][i]);
         }
       }
 #pragma unroll
-      for (int i = 0; i < kRowsPerThread; ++i) {
-        const int row = r0 + 8 * i;
-        if (row < M) epi.apply(sum[i], row, col);
+      for (int u = 0; u < kRound; ++u) {
+#pragma unroll
+        for (int i = 0; i < kRowsPerThread; ++i) {
+#pragma unroll
+          for (int c = 0; c < 4; ++c) sum[i][c] += part[u][i][c];
+        }
       }
-      return;
     }
 #pragma unroll
     for (int i = 0; i < kRowsPerThread; ++i) {
       const int row = r0 + 8 * i;
-      if (row >= M) continue;
-      acc_t total[4] = {0, 0, 0, 0};
-      for (int p = 0; p < kSplits; ++p) {
-        acc_t part[4];
-        ws_load_chunk<4>(wsBuf, base + static_cast<u32>(p * kPartBytes + (row * 128 + 4 * c4) * static_cast<long>(sizeof(acc_t))), part);
-#pragma unroll
-        for (int c = 0; c < 4; ++c) total[c] += part[c];
-      }
-      epi.apply(total, row, col);
+      if (row < M) epi.apply(sum[i], row, col);
     }
     return;
   }
