@@ -164,7 +164,9 @@ class GemmEmitter {
       const int64_t strips = (n_ + 127) / 128, steps = k_ * elemBytes() / 32;
       int64_t want = opt_.split > 0 ? opt_.split : std::max<int64_t>(1, 256 / (strips * batch_));
       want = std::min<int64_t>(want, std::max<int64_t>(1, opt_.split > 0 ? steps : steps / 16));
-      want = std::min<int64_t>(want, 64);
+      // (the last workgroup of a strip adds the partials of all its splits: 16 x 8192 x 1024 takes 10.1 us with 16
+      // splits, 12.9 with the 32 that would fill the chip)
+      want = std::min<int64_t>(want, 16);
       while (want > 1 && strips * batch_ * want * m_ * 128 * 4 >= (1LL << 30)) --want;
       kSplit_ = static_cast<int>(want);
       return;
@@ -181,6 +183,11 @@ class GemmEmitter {
       // splits moved 134 MB of partials for 8 MB of operands and lost 12 %; bf16 with twice the operands gained 26 %)
       const int64_t operandBytes = (m_ * k_ + k_ * n_) * elemBytes();
       while (want > 1 && 2 * tiles * want * partRows * 256 * 4 > 4 * operandBytes) --want;
+    }
+    if (opt_.split <= 0) {
+      // ... and the one workgroup that finishes a tile reads the partials of all its splits by itself: at most 1 MiB
+      // of them (256 x 8192 x 8192: four splits 68.0 us bf16 / 47.3 us int8, eight 75.5 / 60.7; 128 rows: eight are best)
+      want = std::min<int64_t>(want, std::max<int64_t>(1, (1LL << 20) / (partRows * 256 * 4)));
     }
     while (want > 1 && (want - 1) * ((steps + want - 1) / want) >= steps) --want;   // no empty split
     kSplit_ = static_cast<int>(std::max<int64_t>(1, want));
