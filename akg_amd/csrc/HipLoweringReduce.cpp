@@ -1309,12 +1309,14 @@ class StreamReduceEmitter {
       }
       line("  __shared__ unsigned akg_flag;");
       line("  if (!akg::last_workgroup(akg_ws, akg_group, SPLIT, tid, &akg_flag)) return;");
+      // (the partials of every reduction first: they come from other XCDs, and a load behind the previous reduction's
+      // barriers would be a memory round trip of its own)
       for (size_t k = 0; k < reduces_.size(); ++k) {
         const OpNode &op = *reduces_[k];
         const lowering::ReduceSpec spec = lowering::reduceSpec(op, g_.tensor(op.outputs[0]).dtype);
         src_ << "  acc" << k << " = (tid < SPLIT) ? akg::ws_load(part" << k << " + tid) : " << spec.init << ";\n";
-        blockReduce(k, "acc" + std::to_string(k));
       }
+      for (size_t k = 0; k < reduces_.size(); ++k) blockReduce(k, "acc" + std::to_string(k));
       if (dynR_) line("  }");
     }
     emitPost(true);
