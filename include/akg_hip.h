@@ -23,7 +23,8 @@ typedef enum akg_hip_status {
   AKG_HIP_OK = 0,
   AKG_HIP_ERR_INVALID_ARGUMENT = -1,
   AKG_HIP_ERR_JSON = -2,          /* malformed JSON text */
-  AKG_HIP_ERR_TRANSLATE = -3,     /* well-formed JSON that is not a valid op description */
+  AKG_HIP_ERR_TRANSLATE = -3,     /* well-formed JSON that is not a valid op description (also: a tensor with an extent
+                                     of 0 or more than 2^40 elements, an op with the wrong number of operands) */
   AKG_HIP_ERR_UNSUPPORTED = -4,   /* valid description with no gfx950 kernel family (or an unknown op) */
   AKG_HIP_ERR_COMPILE = -5,       /* device compilation failed */
   AKG_HIP_ERR_IO = -6,            /* artifact directory / file access */
