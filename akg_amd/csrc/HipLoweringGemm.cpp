@@ -153,7 +153,7 @@ class GemmEmitter {
   void pickSplit() {
     kSplit_ = 1;
     if (serial_) return;
-    dyn_ = opt_.extentAsArgument && batch_ == 1 && m_ * k_ * elemBytes() < (1LL << 31);
+    dyn_ = opt_.extentAsArgument && batch_ == 1;
     // At most 64 rows of A (and K a multiple of 32 bytes): the time is that of streaming B, which gemm_skinny reads
     // straight into MFMA operands; 256 workgroups of four wavefronts (one per CU: 16 x 8192 x 8192 bf16 reaches 66 % of
     // the HBM peak with 4 splits of 64 strips, 59 % with 8, 48 % with 2; 8 wavefronts or more steps in flight change

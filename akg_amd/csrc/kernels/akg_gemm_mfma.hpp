@@ -270,22 +270,25 @@ AKG_DEV void gemm_256x256(const void *__restrict__ A, const void *__restrict__ B
   // Global loads are buffer loads: the per-lane offset is computed once, everything that changes from load to load
   // (row block, k-row, K step) is a scalar offset, so the loop spends no vector instructions on addresses (vector
   // instructions and MFMAs compete for issue cycles). Out-of-range lanes read zero through the descriptor's size.
-  static_assert((DYN || MS * K < (1L << 31)) && N * K < (1L << 31), "operand too large for 32-bit buffer offsets");
+  // The descriptor of A (and of a [N,K] B) starts at the tile's first row, so the 32-bit offsets only have to span a
+  // tile and A may be of any size (131072 tokens x 8192 bf16 are 2 GiB); a row-major B is addressed from its start.
+  static_assert(kGemmBM * K < (1L << 31) && (TRANSB ? kGemmBN * K : N * K) < (1L << 31), "operand too large for 32-bit buffer offsets");
+  auto bytesLeft = [](long bytes) { return static_cast<int>(bytes < 0 ? 0 : (bytes < 0x7fffffffL ? bytes : 0x7fffffffL)); };
   const __amdgpu_buffer_rsrc_t aRsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<void *>(A), 0, static_cast<int>(M * K), 0x00020000);
+      const_cast<char *>(static_cast<const char *>(A)) + m0 * K, 0, bytesLeft((M - m0) * K), 0x00020000);
   const __amdgpu_buffer_rsrc_t bRsrc = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<void *>(B), 0, static_cast<int>(N * K), 0x00020000);
+      const_cast<char *>(static_cast<const char *>(B)) + (TRANSB ? n0 * K : 0L), 0, bytesLeft(TRANSB ? (N - n0) * K : N * K), 0x00020000);
   typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-  const int aVoff = static_cast<int>((m0 + aRow) * K + aChunk * 16);
+  const int aVoff = static_cast<int>(aRow * K + aChunk * 16);
   int aVoffClamped[kRowChunks];   // kClampRows: one vector offset per staged chunk, its row clamped to M - 1
 #pragma unroll
   for (int i = 0; i < kRowChunks; ++i) {
     const long row = m0 + aRow + kRowStep * i;
-    aVoffClamped[i] = static_cast<int>((row < M ? row : M - 1) * K + aChunk * 16);
+    aVoffClamped[i] = static_cast<int>(((row < M ? row : M - 1) - m0) * K + aChunk * 16);
   }
   const int bRowT = tid / kChunksPerRowB;     // + kRowStepB * i
   const int bChunkT = tid % kChunksPerRowB;
-  const int bVoff = TRANSB ? static_cast<int>((n0 + aRow) * K + aChunk * 16)
+  const int bVoff = TRANSB ? static_cast<int>(aRow * K + aChunk * 16)
                            : static_cast<int>(bRowT * NB + n0 * EB + bChunkT * 16);
   // LDS write offsets. [N,K] B: the LDS row of a column is chosen so that the 16 lanes of a fragment read find, in the
   // four column tiles 4 q .. 4 q + 3, four ADJACENT columns (row 64 q + 16 t + c holds column 64 q + 4 c + t).

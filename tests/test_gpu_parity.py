@@ -1869,6 +1869,40 @@ def test_full_size_bf16_gemm_bias_gelu_fusion():
     assert ok, msg
 
 
+@pytest.mark.parametrize("m,transpose_b", [(147456, True), (139264, False)])
+def test_matmul_whose_first_operand_is_larger_than_two_gib(m, transpose_b):
+    """A of [147456, 8192] bfloat16 is 2.25 GiB: the rows beyond 131072 lie at byte offsets no 32-bit buffer offset
+    reaches from the start of A, so the descriptor of A starts at each tile's first row. 64 sampled rows (every
+    region of A, the last tile and the rows either side of the 2 GiB line among them) against the oracle evaluated on
+    those rows, and the rest of the result must hold no NaN prefill."""
+    from oracle import np_ref
+    from akg_amd import op_desc
+    k, n = 8192, 256
+    name = "big_a_gemm_%dx%dx%d%s" % (m, k, n, "_tb" if transpose_b else "")
+    print("case %s" % name, flush=True)
+    text = op_desc.gemm_bias_act(m, k, n, "bfloat16", "gelu", transpose_b, "float32", name)
+    desc = json_loads(text)
+    kernel = driver.HipKernel(text, out_dir=None)
+    assert kernel.family == "gemm_epilogue"
+    rng = np.random.default_rng(4)
+    small = harness.make_inputs(json_loads(op_desc.gemm_bias_act(4096, k, n, "bfloat16", "gelu", transpose_b, "float32", "p")), seed=harness.BASE_SEED + 8)
+    a = np.tile(small[0], (m // 4096, 1))
+    # every row its own: the row index into a few elements, so that a wrong row cannot pass for the right one
+    a[:, 0] = harness.f32_to_bf16_bits((np.arange(m) % 251).astype(np.float32) / 64.0 - 2.0)
+    a[:, 4097] = harness.f32_to_bf16_bits((np.arange(m) // 251 % 241).astype(np.float32) / 64.0 - 2.0)
+    inputs = [a, small[1], small[2]]
+    got = run_on_gpu(kernel, inputs)[0]
+    line = (1 << 31) // (k * 2)   # first row beyond 2 GiB
+    rows = np.unique(np.concatenate([[0, 255, 256, line - 2, line - 1, line, line + 1, line + 255, line + 256, m - 257, m - 256, m - 1],
+                                     rng.integers(0, m, 52)]))
+    sub = json_loads(op_desc.gemm_bias_act(len(rows), k, n, "bfloat16", "gelu", transpose_b, "float32", "rows"))
+    expect_rows = np_ref.evaluate(sub, [a[rows], inputs[1], inputs[2]])[0]
+    ok, msg = harness.compare(got[rows], expect_rows, "bfloat16")
+    print("  sampled rows vs oracle: %s" % msg, flush=True)
+    assert ok, msg
+    assert not np.isnan(harness.bf16_bits_to_f32(got)).any()
+
+
 SERIAL_GEMMS = ["small_gemm_f16_result_f16_bias_relu_70x200x36.info", "small_gemm_bf16_result_bf16_bias_none_33x129x5_tb.info",
                 "small_gemm_f32_bias_gelu_70x100x36.info", "small_gemm_bf16_bias_gelu_65x30x10.info"]
 
