@@ -20,7 +20,7 @@ FIXTURES = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__
 # (larger first, smaller second) - streaming reductions, a GEMM with K split over workgroups, descriptions that run as
 # several kernels, a grouped segment sum (several launches of one code object sharing the scratch)
 SEQUENCES = [
-    ("small_biasgrad_bf16_2048x1024.info", "small_reducey_max_f16_130x66.info"),
+    ("small_biasgrad_bf16_1000x4095.info", "small_biasgrad_bf16_2048x1024.info"),
     ("small_reducey_sqsum_f32_1x5100x3072.info", "small_reduceall_sqsum_f32_768x512.info"),
     ("small_gemm_i8_dequant_bias_gelu_300x2064x520_tb.info", "small_gemm_bf16_bias_gelu_256x512x256.info"),
     ("small_staged_bn_train_forward_f32_16x8x14x14.info", "small_staged_bn_train_forward_bf16_8x6x7x12.info"),
