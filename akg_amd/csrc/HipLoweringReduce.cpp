@@ -605,6 +605,9 @@ class StreamReduceEmitter {
             streamedBytes / (groups_ * within512) >= 65536) {
           split = within512;
         }
+        // Small inputs with 64 channels or more: a channel is left whole, which needs no partials and no arrival count
+        // (bf16 [32,64,28,28]: 4.7 -> 3.7 us, [32,128,28,28]: 4.9 -> 3.9, [16,64,56,56]: 5.4 -> 4.8).
+        if (streamedBytes <= (16LL << 20) && groups_ >= 64) split = 1;
       }
       const int64_t maxSplit = std::max<int64_t>(1, extent / (chunk * 2));
       split = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(split, maxSplit), kBlock));
