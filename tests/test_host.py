@@ -801,6 +801,42 @@ def test_column_kernel_schedule():
     assert k.family == "staged"
 
 
+def test_streaming_schedules_follow_what_was_measured():
+    """The grid and the loads in flight of streaming reductions, and the K splits of MatMuls with few tiles: one
+    workgroup per CU with eight loads in flight per thread in both directions, fewer workgroups and whole groups for
+    small inputs, the loads divided by the workgroups a CU holds where the grid is larger, partials of at most 1 MiB
+    per tile."""
+    def red(shape, axes, dtype, name, op="ReduceSum"):
+        return driver.HipKernel(op_desc.square_reduce(shape, axes, dtype, False, op, name), out_dir=None)
+    k = driver.HipKernel.from_file(os.path.join(FIXTURES, "n1_biasgrad_bf16_16384x4096.info"))
+    assert k.grid[0] == 256 and "constexpr int U = 4;" in k.source and "RSTEP" in k.source     # two operands x four chunks
+    k = red([1, 65536, 1024], [1], "float32", "sched_tall")
+    assert k.grid[0] == 256 and "constexpr int U = 8;" in k.source
+    k = red([16, 4096, 1536], [1], "bfloat16", "sched_192_groups")        # 192 groups: 768 workgroups, two loads each
+    assert k.grid[0] == 768 and "constexpr int U = 2;" in k.source
+    k = red([4, 16384, 768], [1], "float32", "sched_48_groups")           # 48 groups: 240 workgroups, not 288
+    assert k.grid[0] == 240
+    k = red([1, 1024, 1024], [1], "float32", "sched_small_y")             # 4 MiB: 128 workgroups
+    assert k.grid[0] == 128 and k.workspace_bytes > 0
+    k = red([16, 256, 256], [1], "float32", "sched_small_whole_groups")   # 64 groups: each left whole, no partials
+    assert k.grid[0] == 64 and k.workspace_bytes == 0
+    k = driver.HipKernel(op_desc.batchnorm_stats(32, 64, 28, 28, "bfloat16", "sched_small_bn"), out_dir=None)
+    assert k.grid[0] == 64 and k.workspace_bytes == 0
+    k = red([1024, 4096], [0, 1], "float32", "sched_small_all")           # 16 MiB into one number: 128 workgroups
+    assert k.grid[0] == 128
+    k = red([64, 262143], [1], "float16", "sched_long_odd_rows")          # chunk slots with an overlapping last one, batched
+    assert "RUN_CHUNKS" in k.source and "constexpr int U = 8;" in k.source and "load_chunk_if" in k.source
+    k = driver.HipKernel(op_desc.gemm_bias_act(256, 8192, 8192, "bfloat16", "gelu", False, "float32", "sched_split_256"))
+    assert "k_splits=4" in _meta_schedule(k)
+    k = driver.HipKernel(op_desc.gemm_bias_act(128, 8192, 8192, "bfloat16", "gelu", False, "float32", "sched_split_128"))
+    assert "k_splits=8" in _meta_schedule(k)
+    k = driver.HipKernel(op_desc.gemm_bias_act(16, 8192, 1024, "bfloat16", "gelu", False, "float32", "sched_split_skinny"))
+    assert "k_splits=16" in _meta_schedule(k)
+    # a [N,K] weight is loaded without the non-temporal hint, a row-major one with it
+    k = driver.HipKernel(op_desc.gemm_bias_act(16, 8192, 8192, "bfloat16", "gelu", True, "float32", "sched_skinny_nk"), out_dir=None)
+    assert "true, Epilogue, 4, 4, 2, false>" in k.source
+
+
 def test_skinny_matmul_gets_the_streaming_kernel():
     """At most 64 rows of A and K a multiple of 32 bytes: B goes straight into MFMA operands (no 256 x 256 tile), strips
     of 128 columns times K splits make about 256 workgroups, and the workspace holds a counter per strip plus M x 128
